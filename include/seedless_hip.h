@@ -1,0 +1,220 @@
+/*
+ * seedless_hip.h — C ABI of libseedless_hip.so, an MI355X (gfx950) implementation of the
+ * Seedless fused decode engine of penta2himajin/qwisp.
+ *
+ * Every entry point below replaces one public member of the reference's
+ * `SeedlessFusedVerify.SeedlessFusedForward` (swift/Sources/QwispCore/SeedlessFusedVerify.swift,
+ * abbreviated SFV) — the object that `Tell.SpecBackend` (TellRuntime.swift:83-111) is populated
+ * from — or one of the static per-block functions its tests call.  Plain pointers and sizes only.
+ *
+ * Conventions
+ *  - fp16 data crosses the boundary as uint16_t bit patterns.
+ *  - All functions returning int return SL_OK (0) or a negative sl_status.  The first failure
+ *    of an engine is sticky: sl_fault() returns its message and every later call on that engine
+ *    returns SL_ERR_POISONED without touching its outputs (SFV:388-401, TellRuntime.swift:193).
+ *  - One thread inside one engine at a time (the reference serialises callers with a semaphore,
+ *    LLMBackend.swift:129).
+ *  - Weights are MLX-affine 4-bit, group 64 along K: w = scale*q + bias, q packed 8 per
+ *    little-endian uint32, nibble j of a word is (word >> 4*j) & 15 (SeedlessMetalForward.swift
+ *    :171-174); scales/biases are fp16 [N, K/64].
+ */
+#ifndef SEEDLESS_HIP_H
+#define SEEDLESS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- fixed per-layer geometry (SeedlessEngine.swift:13-16, QwispModel.swift:108-118) ---- */
+#define SL_H            2048   /* hidden size */
+#define SL_MOE_I        512    /* routed and shared expert intermediate size */
+#define SL_TOPK         8
+#define SL_MAX_EXPERTS  256
+#define SL_ATT_HEADS    16
+#define SL_ATT_KV       2
+#define SL_ATT_D        256
+#define SL_ROPE_DIM     64
+#define SL_GDN_HK       16
+#define SL_GDN_HV       32
+#define SL_GDN_D        128    /* d_k = d_v */
+#define SL_CONV_K       4
+#define SL_CONV_DIM     8192   /* 2*HK*D + HV*D */
+#define SL_GDN_IN_N     12352  /* qkv 8192 + z 4096 + b 32 + a 32 */
+#define SL_ATT_QKV_N    9216   /* q(+gate) 16*512 + k 512 + v 512 */
+
+typedef enum {
+  SL_OK = 0,
+  SL_ERR_ARG = -1,        /* bad argument (M > maxM, sequence overflow, null pointer, bad shape) */
+  SL_ERR_POISONED = -2,   /* engine has a sticky fault */
+  SL_ERR_DEVICE = -3,     /* a HIP call failed; message in sl_fault() */
+  SL_ERR_UNSUPPORTED = -4,
+  SL_ERR_FORMAT = -5      /* persisted-state blob does not match this engine */
+} sl_status;
+
+/* Where the tensors named by a model description live. */
+#define SL_LOC_HOST   0
+#define SL_LOC_DEVICE 1
+
+/* One quantized matrix [n, k] in the checkpoint layout. */
+typedef struct {
+  const uint32_t* w;        /* [n, k/8]  */
+  const uint16_t* scales;   /* [n, k/64] fp16 */
+  const uint16_t* biases;   /* [n, k/64] fp16 */
+  int32_t n, k;
+} sl_q4;
+
+/* Gated-DeltaNet mixer weights; tensor names as in SeedlessEngine.swift:47-66. */
+typedef struct {
+  sl_q4 in_proj_qkv;        /* [8192, 2048] */
+  sl_q4 in_proj_z;          /* [4096, 2048] */
+  sl_q4 in_proj_b;          /* [32, 2048]   */
+  sl_q4 in_proj_a;          /* [32, 2048]   */
+  sl_q4 out_proj;           /* [2048, 4096] */
+  const float*    conv1d_w; /* [8192, 4] fp32, tap 3 multiplies the newest sample */
+  const uint16_t* norm_w;   /* [128] fp16 */
+  const float*    a_log;    /* [32] */
+  const float*    dt_bias;  /* [32] */
+} sl_gdn_w;
+
+/* Full-attention mixer weights; names as in SeedlessEngine.swift:69-84. */
+typedef struct {
+  sl_q4 q_proj;             /* [16*512, 2048], per head [q 256 | gate 256] */
+  sl_q4 k_proj;             /* [512, 2048] */
+  sl_q4 v_proj;             /* [512, 2048] */
+  sl_q4 o_proj;             /* [2048, 4096] */
+  const uint16_t* q_norm;   /* [256] fp16 */
+  const uint16_t* k_norm;   /* [256] fp16 */
+} sl_attn_w;
+
+/* Sparse MoE block weights; names as in SeedlessEngine.swift:97-121. */
+typedef struct {
+  const uint16_t* router_w;      /* [E, 2048] fp16 gate */
+  const uint16_t* shared_gate_w; /* [2048] fp16 shared_expert_gate row */
+  sl_q4 sw_gate;                 /* [E*512, 2048]  switch_mlp.gate_proj, expert-major */
+  sl_q4 sw_up;                   /* [E*512, 2048]  */
+  sl_q4 sw_down;                 /* [E*2048, 512]  */
+  sl_q4 sh_gate;                 /* [512, 2048] shared expert */
+  sl_q4 sh_up;                   /* [512, 2048] */
+  sl_q4 sh_down;                 /* [2048, 512] */
+} sl_moe_w;
+
+typedef struct {
+  int32_t is_linear;             /* 1 = Gated-DeltaNet mixer, 0 = full attention (SeedlessEngine.swift:29) */
+  const uint16_t* input_ln;      /* [2048] fp16 */
+  const uint16_t* post_ln;       /* [2048] fp16 */
+  sl_gdn_w  gdn;                 /* valid when is_linear */
+  sl_attn_w attn;                /* valid when !is_linear */
+  sl_moe_w  moe;
+} sl_layer_desc;
+
+typedef struct {
+  int32_t n_layers;
+  int32_t n_experts;             /* multiple of 8, 8..256 */
+  int32_t vocab;                 /* multiple of 16 */
+  int32_t location;              /* SL_LOC_HOST or SL_LOC_DEVICE, applies to every pointer below */
+  const sl_layer_desc* layers;   /* [n_layers], host memory */
+  sl_q4 embed;                   /* [vocab, 2048]; all-null = engine without a head */
+  sl_q4 lm_head;                 /* [vocab, 2048] */
+  const uint16_t* final_norm;    /* [2048] fp16 */
+} sl_model_desc;
+
+typedef struct sl_engine sl_engine;
+typedef struct sl_full_snap sl_full_snap;
+
+/* Per-layer KV lengths captured before one forward (SFV:4039 `Snapshot`). */
+typedef struct { int32_t kv_len; int32_t gdn_parity; } sl_snap;
+
+/* SeedlessFusedForward.init (SFV:3368) + attachHead (SFV:3799).  Copies every tensor into
+ * device memory in the engine's own layout; the caller may free its tensors afterwards.
+ * Caches start cold: conv history zero, recurrent state zero, KV length 0
+ * (SeedlessEngine.swift:149-161). */
+int sl_create(const sl_model_desc* desc, int max_m, int max_seq_len, sl_engine** out);
+void sl_destroy(sl_engine* e);
+
+/* gpuFault.fault (SFV:388-401): NULL while healthy. */
+const char* sl_fault(const sl_engine* e);
+/* injectCBFailure (SFV:404): makes the next device submission report failure (test hook; no
+ * kernel is made to fault). */
+void sl_inject_failure(sl_engine* e);
+
+/* stepArgmax (SFV:3832): M <= max_m token ids in, M greedy next-token ids out; row m attends
+ * to the KV prefix base+m+1; all caches advance by M. */
+int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out);
+/* chainedStepArgmax (SFV:4413): equals K successive sl_step_argmax of one token each, the
+ * output of step k feeding step k+1 on the device. */
+int sl_chained_step_argmax(sl_engine* e, int32_t first_token, int k, int32_t* out);
+/* forwardRows (SFV:3641): hidden rows in, hidden rows (final_norm=0) or final-normed rows out. */
+int sl_forward_rows(sl_engine* e, const uint16_t* x_f16, int m, int final_norm, uint16_t* out_f16);
+/* Tell.SpecBackend.forward (TellRuntime.swift:84): embed + forwardRows with final norm. */
+int sl_forward_tokens(sl_engine* e, const int32_t* tokens, int m, uint16_t* out_f16);
+/* hiddenRows (SFV:4392): the normed rows the last step left behind (volatile). */
+int sl_hidden_rows(sl_engine* e, int m, uint16_t* out_f16);
+/* Logits of row m of the last sl_step_argmax (the reference keeps them in HeadBufs.logits, SFV:3783). */
+int sl_logits_row(sl_engine* e, int m, uint16_t* out_f16 /* [vocab] */);
+/* engine.logits (SeedlessEngine.swift:180): lm_head + argmax over already-normed rows; used for
+ * the first token after prefill (TellRuntime.swift:724-727). */
+int sl_head_argmax(sl_engine* e, const uint16_t* normed_f16, int m, int32_t* out);
+
+/* snapshot / rollbackOneStep (SFV:4039-4047): undo exactly one forward made after the snapshot. */
+int sl_snapshot(sl_engine* e, sl_snap* s);
+int sl_rollback_one_step(sl_engine* e, const sl_snap* s);
+/* fullSnapshot / fullRestore (SFV:4053-4068): arbitrary rewind; KV by length, GDN deep copy. */
+int sl_full_snapshot(sl_engine* e, sl_full_snap** out);
+int sl_full_restore(sl_engine* e, const sl_full_snap* s);
+void sl_full_snap_free(sl_full_snap* s);
+/* persistentStateData / restorePersistentState (SFV:4084-4154): "QWS1" little-endian blob. */
+size_t sl_persist_size(sl_engine* e);
+int sl_persist_write(sl_engine* e, void* dst, size_t cap);
+int sl_persist_restore(sl_engine* e, const void* src, size_t len);
+
+/* readLayerCache (SFV:4381).  GDN layer: a = conv history [3, 8192] fp16 (oldest first),
+ * b = recurrent state [32, 128, 128] fp32 ([hv][dv][dk]).  Attention layer: a = K [2, len, 256]
+ * fp16 (post-RoPE), b = V [2, len, 256] fp16.  Either pointer may be NULL. */
+int sl_read_layer_cache(sl_engine* e, int layer, void* a, void* b);
+/* Preloaded caches (the `caches:` argument of SFV:3368).  For attention layers `len` keys are
+ * written and the engine's sequence position becomes `len` (all attention layers share it). */
+int sl_load_layer_cache(sl_engine* e, int layer, const void* a, const void* b, int len);
+int sl_position(const sl_engine* e);
+
+/* indsCaptureHook (SFV:3366): routing of the last forward, layer `layer`: [m, 8] each. */
+int sl_read_route(sl_engine* e, int layer, int m, int32_t* inds, uint16_t* scores_f16);
+
+/* Per-block entry points used by the reference's block-level tests and by the single-block
+ * workloads: fusedMoEBlockRows (SFV:1986), fusedGdnLayerRows (SFV:3065), fusedAttnLayerRows
+ * (SFV:2460).  x is the already-normed input [m, 2048]; out is the block output before the
+ * residual add.  They run on layer `layer` of the engine and advance only that layer's caches
+ * (an attention block call advances the engine position by m). */
+int sl_moe_block_rows(sl_engine* e, int layer, const uint16_t* x_f16, int m, uint16_t* out_f16);
+int sl_gdn_layer_rows(sl_engine* e, int layer, const uint16_t* x_f16, int m, uint16_t* out_f16);
+int sl_attn_layer_rows(sl_engine* e, int layer, const uint16_t* x_f16, int m, uint16_t* out_f16);
+
+/* Greedy loop standing in for Tell.runSpecLoop without drafts (TellRuntime.swift:716-802):
+ * prefill the prompt in chunks of <= max_m rows through sl_forward_tokens, first token = argmax
+ * of lm_head on the last normed row, then sl_chained_step_argmax in chains of `chain_k`. */
+int sl_greedy_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_new, int chain_k,
+                       int32_t* out);
+
+/* Timing of the most recent step on the engine's stream, measured with HIP events
+ * (profLastGPUMs, SFV:3137). */
+float sl_last_gpu_ms(const sl_engine* e);
+/* The HIP stream (hipStream_t) the engine launches on. */
+void* sl_stream(sl_engine* e);
+
+/* ---- synthetic checkpoints (seeded, no file I/O) --------------------------------------------
+ * Fills device tensors with N(0, sigma) weights quantized by the MLX affine rule, group 64.
+ * Element (row, col) of tensor `seed` is a pure function of (seed, row*k + col), so any slice can
+ * be regenerated independently and a host implementation of the same rule gives the same bytes. */
+int sl_synth_q4(uint32_t* w_dev, uint16_t* scales_dev, uint16_t* biases_dev,
+                int64_t n, int32_t k, uint64_t seed, float sigma, void* stream);
+/* fp16 tensor: value = mean + sigma * normal. */
+int sl_synth_f16(uint16_t* dst_dev, int64_t count, uint64_t seed, float mean, float sigma, void* stream);
+/* fp32 tensor: value = mean + sigma * normal. */
+int sl_synth_f32(float* dst_dev, int64_t count, uint64_t seed, float mean, float sigma, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SEEDLESS_HIP_H */
