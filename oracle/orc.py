@@ -59,6 +59,9 @@ def _load():
         "orc_sdpa": (None, [vp, vp, vp, i32, vp]),
         "orc_rope_entry": (None, [i32, i32, C.POINTER(f32), C.POINTER(f32)]),
         "orc_norm_rope": (None, [vp, vp, i32, vp]),
+        "orc_delta_step": (None, [vp, vp, vp, vp, vp, vp, i32, i32, vp]),
+        "orc_gdn_beta": (f32, [f32]), "orc_gdn_decay": (f32, [f32, f32, f32]),
+        "orc_conv_silu": (f32, [vp, vp]),
         "orc_synth_q4": (None, [vp, vp, vp, i64, i32, u64, f32]),
         "orc_synth_f16": (None, [vp, i64, u64, f32, f32]),
         "orc_synth_f32": (None, [vp, i64, u64, f32, f32]),

@@ -225,6 +225,36 @@ static void moe_block_rows(Engine& e, int li, const float* x, int M, float* out)
   }
 }
 
+// One head of the gated delta rule (GatedDelta.swift:92-112): per state row dv,
+// s *= g; kv = sum s*k; delta = (v - kv)*beta; s += k*delta; y = sum s*q.  Canonical order: 32
+// lanes x 4 contiguous dk, fmaf chains, tree over the 32 lanes; y rounded to half.
+static void delta_head_step(float* state, const float* qh, const float* kh, const float* v, float g, float beta, float* y) {
+  for (int dv = 0; dv < GD; ++dv) {
+    float* s = &state[(size_t)dv * GD];
+    float p[32];
+    for (int l = 0; l < 32; ++l) {
+      float acc = 0.0f;
+      for (int i = 0; i < 4; ++i) { s[4 * l + i] = s[4 * l + i] * g; acc = std::fmaf(s[4 * l + i], kh[4 * l + i], acc); }
+      p[l] = acc;
+    }
+    const float kv = tree_sum(p, 32);
+    const float delta = (v[dv] - kv) * beta;
+    for (int l = 0; l < 32; ++l) {
+      float acc = 0.0f;
+      for (int i = 0; i < 4; ++i) { s[4 * l + i] = std::fmaf(kh[4 * l + i], delta, s[4 * l + i]); acc = std::fmaf(s[4 * l + i], qh[4 * l + i], acc); }
+      p[l] = acc;
+    }
+    y[dv] = f16r(tree_sum(p, 32));
+  }
+}
+static inline float gdn_beta(float b) { return sigmoid16(b); }
+static inline float gdn_decay(float a, float a_log, float dt_bias) { return exp_c(-(exp_c(a_log) * softplus_c(a + dt_bias))); }
+static inline float conv_silu(const float* win, const float* w) {
+  float acc = 0.0f;
+  for (int k = 0; k < CK; ++k) acc = std::fmaf(win[k], w[k], acc);
+  return f16r(acc * sigmoid32(acc));
+}
+
 // ------------------------------------------------------------------------------------------------
 // Gated-DeltaNet layer (SeedlessVerifyForward.swift:115-169).
 //   conv + silu + history shift: SeedlessFusedVerify.swift:634-663 (fp32 taps, tap k multiplies
@@ -247,9 +277,9 @@ static void gdn_layer_rows(Engine& e, int li, const float* x, int M, float* out)
   const float qs = f16r(1.0f / 128.0f), ks = f16r(0.08838834764831845f);
   for (int m = 0; m < M; ++m) {
     for (int ch = 0; ch < CD; ++ch) {
-      float acc = 0.0f;
-      for (int k = 0; k < CK; ++k) acc = std::fmaf(cat[(size_t)(m + k) * CD + ch], w.conv1d_w[ch * CK + k], acc);
-      conv[ch] = f16r(acc * sigmoid32(acc));
+      float win[CK];
+      for (int k = 0; k < CK; ++k) win[k] = cat[(size_t)(m + k) * CD + ch];
+      conv[ch] = conv_silu(win, &w.conv1d_w[ch * CK]);
     }
     for (int hk = 0; hk < HK; ++hk) {
       const float* q = &conv[hk * GD];
@@ -263,28 +293,11 @@ static void gdn_layer_rows(Engine& e, int li, const float* x, int M, float* out)
     const float* v = &conv[2 * KEYDIM];
 #pragma omp parallel for schedule(static)
     for (int hv = 0; hv < HV; ++hv) {
-      const float beta = sigmoid16(bP[(size_t)m * HV + hv]);
-      const float sp = softplus_c(aP[(size_t)m * HV + hv] + w.dt_bias[hv]);
-      const float g = exp_c(-(exp_c(w.a_log[hv]) * sp));
+      const float beta = gdn_beta(bP[(size_t)m * HV + hv]);
+      const float g = gdn_decay(aP[(size_t)m * HV + hv], w.a_log[hv], w.dt_bias[hv]);
       const float* qh = &qn[(hv / (HV / HK)) * GD];
       const float* kh = &kn[(hv / (HV / HK)) * GD];
-      for (int dv = 0; dv < GD; ++dv) {
-        float* s = &c.state[((size_t)hv * GD + dv) * GD];
-        float p[32];
-        for (int l = 0; l < 32; ++l) {
-          float acc = 0.0f;
-          for (int i = 0; i < 4; ++i) { s[4 * l + i] = s[4 * l + i] * g; acc = std::fmaf(s[4 * l + i], kh[4 * l + i], acc); }
-          p[l] = acc;
-        }
-        const float kv = tree_sum(p, 32);
-        const float delta = (v[hv * GD + dv] - kv) * beta;
-        for (int l = 0; l < 32; ++l) {
-          float acc = 0.0f;
-          for (int i = 0; i < 4; ++i) { s[4 * l + i] = std::fmaf(kh[4 * l + i], delta, s[4 * l + i]); acc = std::fmaf(s[4 * l + i], qh[4 * l + i], acc); }
-          p[l] = acc;
-        }
-        y[hv * GD + dv] = f16r(tree_sum(p, 32));
-      }
+      delta_head_step(&c.state[(size_t)hv * GD * GD], qh, kh, &v[hv * GD], g, beta, &y[hv * GD]);
     }
     for (int hv = 0; hv < HV; ++hv) {
       const float inv = inv_rms(&y[hv * GD], GD);
@@ -685,6 +698,18 @@ void orc_norm_rope(const uint16_t* x, const uint16_t* w, int pos, uint16_t* out)
   norm_rope(e, xf, w, pos, of);
   for (int d = 0; d < HD; ++d) out[d] = f2h(of[d]);
 }
+
+// Gated delta rule on nhv value heads sharing nhk key heads; q, k: [nhk,128] half values as
+// float, v: [nhv,128], state: [nhv,128,128] updated in place, y: [nhv,128].
+void orc_delta_step(float* state, const float* q, const float* k, const float* v, const float* g, const float* beta,
+                    int nhk, int nhv, float* y) {
+  for (int hv = 0; hv < nhv; ++hv)
+    delta_head_step(state + (size_t)hv * GD * GD, q + (hv / (nhv / nhk)) * GD, k + (hv / (nhv / nhk)) * GD,
+                    v + hv * GD, g[hv], beta[hv], y + hv * GD);
+}
+float orc_gdn_beta(float b) { return gdn_beta(b); }
+float orc_gdn_decay(float a, float a_log, float dt_bias) { return gdn_decay(a, a_log, dt_bias); }
+float orc_conv_silu(const float* win, const float* w) { return conv_silu(win, w); }
 
 // ---- synthetic tensors: the host statement of sl_synth_q4 / sl_synth_f16 / sl_synth_f32 -----------
 // MLX affine quantisation rule, group 64 (as published for mlx.core.quantize, mode "affine").

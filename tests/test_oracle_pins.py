@@ -1,0 +1,484 @@
+"""Pins for the CPU oracle.  The reference holds no golden vectors for this path, so each oracle
+function is checked against something it does not share code with: closed forms, special cases
+that reduce to a textbook result, brute force in float64, numpy / scipy / the gated-delta rule
+shipped in `transformers`, and tests/ref_f64.py (a float64 statement of the reference's MLX op
+graph).  The checks are chosen so that a dropped term, a wrong sign or index, or a transposed
+operand fails at least one of them.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import orc
+from qwisp_amd.synth import ModelConfig
+from tests.ref_f64 import RefModel
+
+dll = orc.dll
+rng = np.random.default_rng(1234)
+
+
+def h2u(x):
+    return np.asarray(x, np.float16).view(np.uint16)
+
+
+# ---- scalar arithmetic ----------------------------------------------------------------------------
+def test_half_conversion_matches_numpy_bit_for_bit():
+    vals = np.concatenate([
+        rng.normal(0, 1, 20000), rng.normal(0, 1e-4, 5000), rng.normal(0, 3e4, 5000),
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e9, -1e9, 5.96e-8, 2.98e-8, 2.9802322e-8,
+                  2.9802326e-8, 6.1e-5, 6.0975e-5, 1.0009765625, 1.00048828125, 1.00146484375, np.inf, -np.inf])
+    ]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    for v, w in zip(vals, want):
+        assert dll.orc_f2h(float(v)) == int(w), v
+        assert dll.orc_f2h_soft(float(v)) == int(w), v
+    for hbits in list(range(0, 0x7c00, 7)) + [0x7c00, 0xfc00, 0x8000, 1, 0x3ff, 0x400]:
+        want32 = np.array([hbits], np.uint16).view(np.float16).astype(np.float32)[0]
+        assert dll.orc_h2f(hbits) == want32
+        assert dll.orc_h2f_soft(hbits) == want32
+
+
+def test_exp_against_float64():
+    x = np.concatenate([rng.uniform(-86, 88.7, 200000), rng.uniform(-1, 1, 50000), [0.0, -0.0, 1.0, -1.0]]).astype(np.float32)
+    y = np.empty_like(x)
+    dll.orc_exp_vec(orc.p(x), orc.p(y), x.size)
+    want = np.exp(x.astype(np.float64))
+    rel = np.abs(y.astype(np.float64) - want) / want
+    assert rel.max() < 2.5e-7, rel.max()
+    assert dll.orc_exp(0.0) == 1.0
+    assert dll.orc_exp(88.8) == np.inf and dll.orc_exp(1e30) == np.inf
+    assert dll.orc_exp(-86.1) == 0.0 and dll.orc_exp(-np.inf) == 0.0
+    xs = np.sort(rng.uniform(-20, 20, 20000)).astype(np.float32)
+    ys = np.empty_like(xs)
+    dll.orc_exp_vec(orc.p(xs), orc.p(ys), xs.size)
+    assert np.all(np.diff(ys) >= 0), "exp must be monotone on a sorted sample"
+
+
+def test_log_against_float64():
+    x = np.concatenate([np.exp(rng.uniform(-17, 20, 200000)), rng.uniform(1, 2, 50000), [1.0, 2.0, 0.5, 1.4142135, 1.4142136]]).astype(np.float32)
+    y = np.empty_like(x)
+    dll.orc_log_vec(orc.p(x), orc.p(y), x.size)
+    want = np.log(x.astype(np.float64))
+    err = np.abs(y.astype(np.float64) - want)
+    assert np.all(err <= 2.5e-7 * np.maximum(1.0, np.abs(want))), err.max()
+    assert dll.orc_log(1.0) == 0.0
+
+
+def test_sigmoid_softplus_decay():
+    for x in rng.normal(0, 4, 2000).astype(np.float32):
+        x = float(x)
+        ref = 1.0 / (1.0 + np.exp(-np.float64(x)))
+        assert abs(dll.orc_sigmoid32(x) - ref) < 2e-7
+        xh = float(np.float16(x))
+        refh = 1.0 / (1.0 + np.exp(-np.float64(xh)))
+        s16 = dll.orc_sigmoid16(xh)
+        assert s16 == float(np.float16(s16)), "sigmoid16 must return a half value"
+        assert abs(s16 - refh) < 1.5e-3
+        assert abs(dll.orc_softplus(x) - np.log1p(np.exp(np.float64(x)))) < 4e-7 * max(1.0, abs(x))
+    # stable form: s(-x) + s(x) == 1 up to one rounding, and the large-|x| limits
+    assert dll.orc_sigmoid32(100.0) == 1.0 and dll.orc_sigmoid32(-100.0) == 0.0
+    assert dll.orc_sigmoid16(20.0) == 1.0 and dll.orc_sigmoid16(-20.0) == 0.0
+    assert dll.orc_sigmoid16(0.0) == 0.5
+    # g = exp(-exp(A_log) * softplus(a + dt_bias))  (GatedDelta.swift:12-15)
+    for a, al, dt in rng.normal(0, 1, (500, 3)):
+        ref = np.exp(-np.exp(al) * np.log1p(np.exp(a + dt)))
+        got = dll.orc_gdn_decay(float(np.float32(a)), float(np.float32(al)), float(np.float32(dt)))
+        assert abs(got - ref) < 1e-6
+        assert 0.0 <= got <= 1.0
+
+
+def test_normal_quantile_against_scipy():
+    from scipy.stats import norm
+    p = np.concatenate([rng.uniform(0, 1, 100000), [2.0 ** -24, 1 - 2.0 ** -24, 0.5, 0.075, 0.925, 0.0751, 0.9249]]).astype(np.float32)
+    p = p[(p > 0) & (p < 1)]
+    y = np.empty_like(p)
+    dll.orc_ppnd7_vec(orc.p(p), orc.p(y), p.size)
+    want = norm.ppf(p.astype(np.float64))
+    err = np.abs(y - want)
+    # single-precision evaluation of a 1e-7 approximation; tails amplify the rounding of p itself
+    assert np.all(err <= 3e-6 * np.maximum(1.0, np.abs(want)) + 2e-6), err.max()
+    assert dll.orc_ppnd7(0.5) == 0.0
+
+
+def test_generator_statistics_and_independence():
+    n = 400000
+    x = orc.synth_f32((n,), 77, 0.0, 1.0)
+    assert abs(x.mean()) < 5e-3 and abs(x.std() - 1.0) < 5e-3
+    assert abs(((x - x.mean()) ** 3).mean()) < 2e-2
+    assert abs(((x - x.mean()) ** 4).mean() - 3.0) < 5e-2
+    y = orc.synth_f32((n,), 78, 0.0, 1.0)
+    assert abs(np.corrcoef(x, y)[0, 1]) < 5e-3
+    assert abs(np.corrcoef(x[:-1], x[1:])[0, 1]) < 5e-3
+    # element i depends only on (seed, i): a prefix of a longer tensor is identical
+    assert np.array_equal(orc.synth_f32((1000,), 77, 0.0, 1.0), x[:1000])
+    # mean/sigma are applied as mean + sigma*z
+    z = orc.synth_f32((1000,), 5, 0.0, 1.0)
+    assert np.array_equal(orc.synth_f32((1000,), 5, 1.0, 0.5), (np.float32(1.0) + np.float32(0.5) * z).astype(np.float32))
+
+
+def test_affine_quantizer_invariants():
+    n, k = 64, 512
+    w, s, b = orc.synth_q4(n, k, 9, 0.02)
+    src = (np.float32(0.02) * orc.synth_f32((n * k,), 9, 0.0, 1.0)).reshape(n, k)
+    d = orc.dequant(w, s, b)
+    sc = np.repeat(np.abs(s.astype(np.float64)), 64, axis=1)
+    bi = np.repeat(np.abs(b.astype(np.float64)), 64, axis=1)
+    nib = (w[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))[None, None, :]) & 15
+    flat = nib.reshape(n, k)
+    # reconstruction within half a step (plus the fp16 rounding of scale and bias); the rule pins
+    # the larger-magnitude end of the group to code 0 exactly and re-derives the step from it, so
+    # the far end may clip at code 15 by up to about one step
+    slack = 15 * sc * 2.0 ** -11 + bi * 2.0 ** -11 + 1e-9
+    err = np.abs(d - src)
+    assert np.all(err[flat < 15] <= 0.5 * sc[flat < 15] + slack[flat < 15])
+    assert np.all(err[flat == 15] <= 1.07 * sc[flat == 15] + slack[flat == 15])
+    # every group touches both ends of its range (the edge value is code 0, the far end 14..15)
+    nib = nib.reshape(n, k // 64, 64)
+    assert nib.min() == 0 and nib.max() == 15
+    assert np.all(nib.min(axis=2) == 0) and np.all(nib.max(axis=2) >= 14)
+    # the bias is the group extreme with the larger magnitude (MLX rule), up to fp16 rounding
+    g = src.reshape(n, k // 64, 64)
+    edge = np.where(np.abs(g.min(axis=2)) > np.abs(g.max(axis=2)), g.min(axis=2), g.max(axis=2))
+    assert np.allclose(b.astype(np.float64), edge, rtol=2.0 ** -10, atol=1e-8)
+
+
+# ---- GEMV ----------------------------------------------------------------------------------------
+@pytest.mark.parametrize("k", [512, 2048, 4096])
+def test_qmv_against_float64(k):
+    n = 48
+    w, s, b = orc.synth_q4(n, k, 21 + k, 0.02)
+    x = rng.normal(0, 1, k).astype(np.float16)
+    y32 = np.empty(n, np.float32)
+    dll.orc_qmv_f32(orc.p(x), orc.p(w), orc.p(s), orc.p(b), n, k, orc.p(y32))
+    d = orc.dequant(w, s, b)
+    want = d @ x.astype(np.float64)
+    bound = 4e-6 * (np.abs(d) @ np.abs(x.astype(np.float64))) + 1e-7
+    assert np.all(np.abs(y32 - want) <= bound), np.abs(y32 - want).max()
+    y16 = np.empty(n, np.float16)
+    dll.orc_qmv(orc.p(x), orc.p(w), orc.p(s), orc.p(b), n, k, orc.p(y16))
+    assert np.array_equal(y16, y32.astype(np.float16))
+
+
+@pytest.mark.parametrize("k", [512, 2048, 4096])
+def test_qmv_unit_vectors_pick_single_weights(k):
+    """x = e_j returns half(float32(s*q + b)) of exactly that weight: pins nibble order, word order,
+    group indexing and the row stride."""
+    n = 8
+    w, s, b = orc.synth_q4(n, k, 33, 0.02)
+    nib = ((w[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))[None, None, :]) & 15).reshape(n, k)
+    for j in list(rng.integers(0, k, 24)) + [0, 7, 8, 63, 64, k - 1]:
+        x = np.zeros(k, np.float16)
+        x[j] = 1.0
+        y = np.empty(n, np.float16)
+        dll.orc_qmv(orc.p(x), orc.p(w), orc.p(s), orc.p(b), n, k, orc.p(y))
+        want = (s[:, j // 64].astype(np.float64) * nib[:, j] + b[:, j // 64].astype(np.float64)).astype(np.float32).astype(np.float16)
+        assert np.array_equal(y, want), j
+
+
+def test_qmv_zero_codes_give_bias_times_sum():
+    n, k = 4, 2048
+    w = np.zeros((n, k // 8), np.uint32)
+    s = rng.normal(0, 0.01, (n, k // 64)).astype(np.float16)
+    b = rng.normal(0, 0.01, (n, k // 64)).astype(np.float16)
+    x = rng.normal(0, 1, k).astype(np.float16)
+    y = np.empty(n, np.float32)
+    dll.orc_qmv_f32(orc.p(x), orc.p(w), orc.p(s), orc.p(b), n, k, orc.p(y))
+    want = (b.astype(np.float64) * x.astype(np.float64).reshape(k // 64, 64).sum(axis=1)[None, :]).sum(axis=1)
+    assert np.allclose(y, want, rtol=0, atol=2e-5)
+
+
+def test_dense_and_rmsnorm_closed_forms():
+    k, n = 2048, 12
+    W = rng.normal(0, 0.02, (n, k)).astype(np.float16)
+    x = rng.normal(0, 1, k).astype(np.float16)
+    y = np.empty(n, np.float16)
+    dll.orc_dense_f16(orc.p(x), orc.p(W), n, k, orc.p(y))
+    want = W.astype(np.float64) @ x.astype(np.float64)
+    assert np.all(np.abs(y.astype(np.float64) - want) <= 2.0 ** -10 * np.abs(want) + 1e-5)
+    for D in (128, 256, 2048):
+        wv = rng.normal(1, 0.1, D).astype(np.float16)
+        xv = rng.normal(0, 2, D).astype(np.float16)
+        out = np.empty(D, np.float16)
+        dll.orc_rmsnorm(orc.p(xv), orc.p(wv), D, orc.p(out))
+        x64 = xv.astype(np.float64)
+        ref = wv.astype(np.float64) * x64 / np.sqrt(np.mean(x64 ** 2) + 1e-6)
+        assert np.all(np.abs(out - ref) <= 2.5 * 2.0 ** -11 * np.abs(ref) + 1e-6)
+        # constant input: out = w * half(c / sqrt(c^2 + eps)), rounded to half twice
+        c = np.float16(0.75)
+        xc = np.full(D, c, np.float16)
+        dll.orc_rmsnorm(orc.p(xc), orc.p(wv), D, orc.p(out))
+        inner = np.float16(np.float32(c) * np.float32(1.0 / np.sqrt(np.float64(c) ** 2 + 1e-6)))
+        want_c = (wv.astype(np.float32) * np.float32(inner)).astype(np.float16)
+        assert np.array_equal(out, want_c)
+
+
+# ---- router ----------------------------------------------------------------------------------------
+@pytest.mark.parametrize("E", [16, 64, 256])
+def test_route_brute_force_with_ties(E):
+    for trial in range(40):
+        lg = rng.normal(0, 1.5, E).astype(np.float16)
+        if trial % 2:
+            lg[rng.integers(0, E, 6)] = lg.max()       # ties among the leaders
+            lg[rng.integers(0, E, 6)] = np.sort(lg)[-8]  # ties at the selection boundary
+        inds = np.empty(8, np.int32)
+        sc = np.empty(8, np.float16)
+        dll.orc_route(orc.p(lg), E, orc.p(inds), orc.p(sc))
+        order = np.argsort(-lg.astype(np.float64), kind="stable")[:8]   # descending, lower index first on ties
+        assert np.array_equal(inds, order)
+        g = np.exp(lg.astype(np.float64) - lg.astype(np.float64).max())
+        g /= g.sum()
+        want = g[order] / g[order].sum()
+        assert np.all(np.abs(sc.astype(np.float64) - want) <= 3e-3 * want + 2e-4)
+        assert abs(sc.astype(np.float64).sum() - 1.0) < 4e-3
+
+
+def test_swiglu_against_float64():
+    g = rng.normal(0, 2, 4096).astype(np.float16)
+    u = rng.normal(0, 2, 4096).astype(np.float16)
+    out = np.empty(4096, np.float16)
+    dll.orc_swiglu(orc.p(g), orc.p(u), 4096, orc.p(out))
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    ref = g64 / (1 + np.exp(-g64)) * u64
+    assert np.all(np.abs(out - ref) <= 4 * 2.0 ** -11 * np.abs(ref) + 2e-3 * np.abs(u64) * (np.abs(g64) < 0.05) + 1e-6)
+    z = np.zeros(4, np.float16)
+    dll.orc_swiglu(orc.p(z), orc.p(u[:4].copy()), 4, orc.p(out))
+    assert np.all(out[:4] == 0)
+
+
+# ---- attention -------------------------------------------------------------------------------------
+@pytest.mark.parametrize("N", [1, 2, 63, 64, 65, 129, 300])
+def test_sdpa_against_float64(N):
+    q = rng.normal(0, 1, 256).astype(np.float16)
+    k = rng.normal(0, 1, (N, 256)).astype(np.float16)
+    v = rng.normal(0, 1, (N, 256)).astype(np.float16)
+    out = np.empty(256, np.float16)
+    dll.orc_sdpa(orc.p(q), orc.p(k), orc.p(v), N, orc.p(out))
+    s = (k.astype(np.float64) @ q.astype(np.float64)) / 16.0
+    p = np.exp(s - s.max())
+    p /= p.sum()
+    ref = p @ v.astype(np.float64)
+    assert np.all(np.abs(out - ref) <= 2.0 ** -10 * np.abs(ref) + 2e-5), np.abs(out - ref).max()
+    if N == 1:
+        assert np.array_equal(out, v[0]), "one key: softmax weight 1, output is the value row"
+
+
+def test_sdpa_equal_keys_average_values_and_ignore_the_tail():
+    N = 100
+    q = rng.normal(0, 1, 256).astype(np.float16)
+    k = np.tile(rng.normal(0, 1, (1, 256)).astype(np.float16), (N + 50, 1))
+    v = rng.normal(0, 1, (N + 50, 256)).astype(np.float16)
+    out = np.empty(256, np.float16)
+    dll.orc_sdpa(orc.p(q), orc.p(k), orc.p(v), N, orc.p(out))
+    ref = v[:N].astype(np.float64).mean(axis=0)
+    assert np.all(np.abs(out - ref) <= 2.0 ** -10 * np.abs(ref) + 2e-5)
+    v2 = v.copy()
+    v2[N:] = 1000.0                                    # rows past N must have no influence
+    k2 = k.copy()
+    k2[N:] = 50.0
+    out2 = np.empty(256, np.float16)
+    dll.orc_sdpa(orc.p(q), orc.p(k2), orc.p(v2), N, orc.p(out2))
+    assert np.array_equal(out, out2)
+
+
+def test_rope_table_and_rotation():
+    for pos, i in [(0, 0), (1, 0), (1, 31), (37, 5), (4095, 17), (32767, 0), (32767, 31)]:
+        c, s = C.c_float(), C.c_float()
+        dll.orc_rope_entry(pos, i, C.byref(c), C.byref(s))
+        ang = pos * (1e7 ** (-i / 32.0))
+        # the angle itself is formed in fp32 (SeedlessFusedVerify.swift:1241-1242)
+        tol = 2e-7 + abs(ang) * 1.3e-7
+        assert abs(c.value - np.cos(ang)) <= tol and abs(s.value - np.sin(ang)) <= tol
+    x = rng.normal(0, 1, 256).astype(np.float16)
+    w = rng.normal(1, 0.1, 256).astype(np.float16)
+    nr = np.empty(256, np.float16)
+    dll.orc_rmsnorm(orc.p(x), orc.p(w), 256, orc.p(nr))
+    out0 = np.empty(256, np.float16)
+    dll.orc_norm_rope(orc.p(x), orc.p(w), 0, orc.p(out0))
+    assert np.array_equal(out0, nr), "position 0 is the identity rotation"
+    pos = 1234
+    out = np.empty(256, np.float16)
+    dll.orc_norm_rope(orc.p(x), orc.p(w), pos, orc.p(out))
+    assert np.array_equal(out[64:], nr[64:]), "dims >= 64 are not rotated"
+    n64, o64 = nr.astype(np.float64), out.astype(np.float64)
+    ang = pos * (1e7 ** (-np.arange(32) / 32.0))
+    want_lo = n64[:32] * np.cos(ang) - n64[32:64] * np.sin(ang)
+    want_hi = n64[:32] * np.sin(ang) + n64[32:64] * np.cos(ang)
+    assert np.allclose(o64[:32], want_lo, atol=3e-3) and np.allclose(o64[32:64], want_hi, atol=3e-3)
+
+
+# ---- gated delta rule ------------------------------------------------------------------------------
+def _delta(state, q, k, v, g, beta, nhk=16, nhv=32):
+    st = np.ascontiguousarray(state, np.float32).copy()
+    y = np.empty((nhv, 128), np.float32)
+    args = [np.ascontiguousarray(a, np.float32) for a in (q, k, v, g, beta)]
+    dll.orc_delta_step(orc.p(st), *[orc.p(a) for a in args], nhk, nhv, orc.p(y))
+    return y, st
+
+
+def test_delta_rule_against_float64_and_transformers():
+    nhk, nhv = 16, 32
+    state = rng.normal(0, 0.1, (nhv, 128, 128)).astype(np.float32)
+    q = rng.normal(0, 0.01, (nhk, 128)).astype(np.float16).astype(np.float32)
+    k = rng.normal(0, 0.09, (nhk, 128)).astype(np.float16).astype(np.float32)
+    v = rng.normal(0, 1, (nhv, 128)).astype(np.float16).astype(np.float32)
+    g = rng.uniform(0.3, 1, nhv).astype(np.float32)
+    beta = rng.uniform(0, 1, nhv).astype(np.float32)
+    y, st = _delta(state, q, k, v, g, beta)
+    qq, kk = np.repeat(q, 2, 0).astype(np.float64), np.repeat(k, 2, 0).astype(np.float64)
+    S = state.astype(np.float64) * g[:, None, None]
+    kv = np.einsum("hvk,hk->hv", S, kk)
+    d = (v - kv) * beta[:, None]
+    S = S + kk[:, None, :] * d[:, :, None]
+    yref = np.einsum("hvk,hk->hv", S, qq)
+    assert np.allclose(st, S, rtol=1e-5, atol=1e-6)
+    assert np.all(np.abs(y - yref) <= 2.0 ** -10 * np.abs(yref) + 1e-6)
+    # the library statement of the same rule keeps the state transposed ([dk, dv]) and applies its
+    # own l2norm/scale, so feed it pre-normalised q/k with use_qk_l2norm_in_kernel=False
+    torch = pytest.importorskip("torch")
+    mod = pytest.importorskip("transformers.models.qwen3_5_moe.modeling_qwen3_5_moe")
+    fn = mod.torch_recurrent_gated_delta_rule
+    tq = torch.tensor(qq, dtype=torch.float32)[None, None] * (128 ** 0.5)   # it multiplies q by d_k^-1/2
+    tk = torch.tensor(kk, dtype=torch.float32)[None, None]
+    tv = torch.tensor(v, dtype=torch.float32)[None, None]
+    tg = torch.log(torch.tensor(g))[None, None]
+    tb = torch.tensor(beta)[None, None]
+    init = torch.tensor(state).transpose(1, 2)[None].contiguous()
+    out, last = fn(tq, tk, tv, tg, tb, initial_state=init, output_final_state=True, use_qk_l2norm_in_kernel=False)
+    assert np.allclose(out[0, 0].numpy(), yref, rtol=1e-4, atol=1e-5)
+    assert np.allclose(last[0].transpose(1, 2).numpy(), S, rtol=1e-4, atol=1e-5)
+
+
+def test_delta_rule_special_cases():
+    nhk, nhv = 16, 32
+    state = rng.normal(0, 0.1, (nhv, 128, 128)).astype(np.float32)
+    q = rng.normal(0, 0.1, (nhk, 128)).astype(np.float16).astype(np.float32)
+    k = rng.normal(0, 0.1, (nhk, 128)).astype(np.float16).astype(np.float32)
+    v = rng.normal(0, 1, (nhv, 128)).astype(np.float16).astype(np.float32)
+    g = rng.uniform(0.3, 1, nhv).astype(np.float32)
+    # beta = 0: pure decay, state' = g*state exactly, y = (g*state) q
+    y, st = _delta(state, q, k, v, g, np.zeros(nhv, np.float32))
+    assert np.array_equal(st, state * g[:, None, None])
+    # k = 0: the same state update, whatever beta is
+    y2, st2 = _delta(state, q, np.zeros_like(k), v, g, np.ones(nhv, np.float32))
+    assert np.array_equal(st2, state * g[:, None, None])
+    assert np.array_equal(y2, y)
+    # zero state, g = beta = 1, unit key e_j, query = key: associative recall returns v exactly
+    kk = np.zeros((nhk, 128), np.float32)
+    kk[:, 5] = 1.0
+    y3, st3 = _delta(np.zeros_like(state), kk, kk, v, np.ones(nhv, np.float32), np.ones(nhv, np.float32))
+    assert np.array_equal(y3, v)
+    assert np.array_equal(st3[:, :, 5], v) and np.count_nonzero(st3) == np.count_nonzero(v)
+
+
+def test_conv_silu_taps():
+    w = np.array([0.1, -0.2, 0.3, 0.7], np.float32)
+    win = np.array([0.0, 0.0, 0.0, 1.5], np.float32)          # cold history: only the newest tap
+    acc = np.float64(np.float32(1.5) * np.float32(0.7))
+    got = dll.orc_conv_silu(orc.p(win), orc.p(w))
+    assert abs(got - acc / (1 + np.exp(-acc))) < 1e-3
+    for _ in range(200):
+        win = rng.normal(0, 1, 4).astype(np.float16).astype(np.float32)
+        w = rng.normal(0, 0.5, 4).astype(np.float32)
+        acc = np.dot(win.astype(np.float64), w.astype(np.float64))
+        ref = acc / (1 + np.exp(-acc))
+        assert abs(dll.orc_conv_silu(orc.p(win), orc.p(w)) - ref) <= 2.0 ** -10 * abs(ref) + 1e-6
+
+
+# ---- whole engine against the float64 graph --------------------------------------------------------
+@pytest.fixture(scope="module")
+def small_model():
+    cfg = ModelConfig(n_layers=4, n_experts=16, vocab=2048)
+    return cfg, orc.generate_host(cfg)
+
+
+def test_engine_against_float64_graph(small_model):
+    """Four layers (3 GDN + 1 attention, as layers 0-3 of the real layout), 6 decode steps.  The
+    oracle rounds to fp16 at every stage; the float64 graph does not.  Measured: the normed hidden
+    state agrees to about 0.5% rms whenever both pick the same experts, and the expert sets differ
+    only where the float64 margin at the selection boundary is below fp16 noise (< 0.02 logits)."""
+    cfg, t = small_model
+    o = orc.Oracle(cfg, t, max_m=4, max_seq_len=32)
+    ref = RefModel(cfg, t)
+    toks = [5, 77, 1999, 0, 1024, 333]
+    clean = 0
+    for step, tok in enumerate(toks):
+        got_tok = o.step_argmax([tok])[0]
+        h, n, logits = ref.step(tok)
+        same_routes = True
+        for li in range(cfg.n_layers):
+            inds, sc = o.read_route(li, 1)
+            rinds, rsc, rlog = ref.route[li]
+            srt = np.sort(rlog)
+            if set(inds[0].tolist()) != set(rinds.tolist()):
+                # a flip is legitimate only at a near-tie, and only the first one in a step is
+                # judged (later layers then see a different input)
+                assert not same_routes or srt[-8] - srt[-9] < 0.02, (step, li, srt[-8] - srt[-9])
+                same_routes = False
+            elif same_routes and np.min(np.diff(np.sort(rlog[rinds]))) > 0.02:
+                assert np.array_equal(inds[0], rinds), "descending-logit order"
+                assert np.allclose(sc[0].astype(np.float64), rsc, rtol=0.03, atol=2e-3)
+        if not same_routes:
+            continue
+        clean += 1
+        got_n = o.hidden_rows(1)[0].astype(np.float64)
+        scale = np.sqrt(np.mean(n ** 2))
+        assert np.sqrt(np.mean((got_n - n) ** 2)) < 0.01 * scale, (step, scale)
+        assert np.max(np.abs(got_n - n)) < 0.04 * scale, (step, np.max(np.abs(got_n - n)), scale)
+        got_lg = o.logits_row(0).astype(np.float64)
+        assert np.sqrt(np.mean((got_lg - logits) ** 2)) < 0.02 * np.std(logits)
+        top2 = np.sort(logits)[-2:]
+        if top2[1] - top2[0] > 0.1 * np.std(logits):
+            assert got_tok == int(np.argmax(logits))
+    assert clean >= 4
+    # caches: recurrent state and KV agree with the float64 graph
+    for li in range(cfg.n_layers):
+        a, b = o.read_layer_cache(li)
+        if cfg.is_linear(li):
+            assert np.allclose(a.astype(np.float64), ref.cache[li]["conv"], atol=0.03 * np.abs(ref.cache[li]["conv"]).max())
+            assert np.allclose(b, ref.cache[li]["state"], atol=0.03 * np.abs(ref.cache[li]["state"]).max())
+        else:
+            assert a.shape == (2, len(toks), 256)
+            assert np.allclose(a.astype(np.float64), ref.cache[li]["k"], atol=0.03 * np.abs(ref.cache[li]["k"]).max())
+            assert np.allclose(b.astype(np.float64), ref.cache[li]["v"], atol=0.03 * np.abs(ref.cache[li]["v"]).max())
+
+
+def test_rows_equal_single_steps_and_chain(small_model):
+    """M-row forward == M single-row forwards (SeedlessVerifyTests.swift:613), chained == stepped
+    (:2445): tokens, logits and every cache bit-for-bit."""
+    cfg, t = small_model
+    a = orc.Oracle(cfg, t, max_m=4, max_seq_len=32)
+    b = orc.Oracle(cfg, t, max_m=4, max_seq_len=32)
+    toks = [9, 8, 7, 6]
+    ta = a.step_argmax(toks)
+    tb = [b.step_argmax([x])[0] for x in toks]
+    assert ta.tolist() == tb
+    assert np.array_equal(a.logits_row(3), b.logits_row(0))
+    ca = a.chained_step_argmax(int(ta[-1]), 3)
+    cb = []
+    cur = tb[-1]
+    for _ in range(3):
+        cur = int(b.step_argmax([cur])[0])
+        cb.append(cur)
+    assert ca.tolist() == cb
+    for li in range(cfg.n_layers):
+        for x, y in zip(a.read_layer_cache(li), b.read_layer_cache(li)):
+            assert np.array_equal(x.view(np.uint8), y.view(np.uint8))
+
+
+def test_layer_pattern_and_rollback(small_model):
+    cfg, t = small_model
+    assert [cfg.is_linear(i) for i in range(8)] == [True, True, True, False, True, True, True, False]
+    o = orc.Oracle(cfg, t, max_m=4, max_seq_len=32)
+    o.step_argmax([1, 2])
+    before = [o.read_layer_cache(li) for li in range(cfg.n_layers)]
+    first = o.step_argmax([3])
+    o.rollback_one_step(2)
+    assert o.position == 2
+    again = o.step_argmax([3])
+    assert first.tolist() == again.tolist()
+    o.rollback_one_step(2)
+    after = [o.read_layer_cache(li) for li in range(cfg.n_layers)]
+    for (a0, b0), (a1, b1) in zip(before, after):
+        assert np.array_equal(a0, a1) and np.array_equal(b0, b1)
