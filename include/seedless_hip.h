@@ -125,7 +125,7 @@ typedef struct sl_engine sl_engine;
 typedef struct sl_full_snap sl_full_snap;
 
 /* Per-layer KV lengths captured before one forward (SFV:4039 `Snapshot`). */
-typedef struct { int32_t kv_len; int32_t gdn_parity; } sl_snap;
+typedef struct { int32_t kv_len; int32_t reserved; } sl_snap;
 
 /* SeedlessFusedForward.init (SFV:3368) + attachHead (SFV:3799).  Copies every tensor into
  * device memory in the engine's own layout; the caller may free its tensors afterwards.

@@ -52,7 +52,7 @@ class ModelDesc(C.Structure):
 
 
 class Snap(C.Structure):
-    _fields_ = [("kv_len", C.c_int32), ("gdn_parity", C.c_int32)]
+    _fields_ = [("kv_len", C.c_int32), ("reserved", C.c_int32)]
 
 
 def _ptr(t):

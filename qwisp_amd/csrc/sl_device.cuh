@@ -1,0 +1,168 @@
+// Device-side scalar arithmetic and wave64 helpers for the Seedless kernels (gfx950).
+//
+// Every function here is built from IEEE binary32 +,-,*,/,sqrt, fmaf and integer operations only
+// and the translation unit is compiled with -ffp-contract=off, so results do not depend on how
+// a kernel is tiled.  Reductions follow one rule: lane partials are left-to-right fmaf chains
+// over contiguous elements, lanes are combined by an xor-butterfly (adjacent lanes first), which
+// is a balanced binary tree whose value is the same on every lane.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#define SL_DEV __device__ __forceinline__
+
+namespace sl {
+
+SL_DEV float f16r(float x) { return __half2float(__float2half_rn(x)); }
+SL_DEV float h2f(uint16_t h) { return __half2float(__ushort_as_half(h)); }
+SL_DEV uint16_t f2h(float x) { return __half_as_ushort(__float2half_rn(x)); }
+
+// exp: n = rint(x*log2 e), two-constant Cody-Waite reduction, degree-6 polynomial, 2^n applied in
+// two exact steps.  x > 88.72 -> +inf, x < -86 (or NaN) -> 0.
+SL_DEV float exp_c(float x) {
+  if (x > 88.72f) return __int_as_float(0x7f800000);
+  if (!(x >= -86.0f)) return 0.0f;
+  float n = rintf(x * 1.44269504f);
+  float r = fmaf(n, -0.693359375f, x);
+  r = fmaf(n, 2.12194440e-4f, r);
+  float p = 1.9875691500e-4f;
+  p = fmaf(p, r, 1.3981999507e-3f);
+  p = fmaf(p, r, 8.3334519073e-3f);
+  p = fmaf(p, r, 4.1665795894e-2f);
+  p = fmaf(p, r, 1.6666665459e-1f);
+  p = fmaf(p, r, 5.0000001201e-1f);
+  float y = fmaf(p, r * r, r) + 1.0f;
+  int ni = (int)n;
+  int a = ni >> 1, b = ni - a;
+  return (y * __int_as_float((a + 127) << 23)) * __int_as_float((b + 127) << 23);
+}
+
+// log for normal positive x: x = m*2^e, m in (sqrt(1/2), sqrt(2)], s = (m-1)/(m+1), odd series to s^9.
+SL_DEV float log_c(float x) {
+  uint32_t u = (uint32_t)__float_as_int(x);
+  int e = (int)((u >> 23) & 255u) - 127;
+  float m = __int_as_float((int)((u & 0x7fffffu) | 0x3f800000u));
+  if (m > 1.41421356f) { m = m * 0.5f; e += 1; }
+  float f = m - 1.0f;
+  float s = f / (2.0f + f);
+  float z = s * s;
+  float p = 0.2222222222f;
+  p = fmaf(p, z, 0.2857142857f);
+  p = fmaf(p, z, 0.4f);
+  p = fmaf(p, z, 0.6666666667f);
+  p = fmaf(p, z, 2.0f);
+  return fmaf((float)e, 0.69314718f, s * p);
+}
+
+SL_DEV float sigmoid32(float x) {
+  float y = 1.0f / (1.0f + exp_c(fabsf(x)));
+  return (x < 0.0f) ? y : (1.0f - y);
+}
+// Half-precision sigmoid: every operation rounded to half; x must be a half value.
+SL_DEV float sigmoid16(float x) {
+  float e = f16r(exp_c(fabsf(x)));
+  float d = f16r(1.0f + e);
+  float y = f16r(1.0f / d);
+  return (x < 0.0f) ? y : f16r(1.0f - y);
+}
+SL_DEV float softplus_c(float x) { return fmaxf(x, 0.0f) + log_c(1.0f + exp_c(-fabsf(x))); }
+SL_DEV float swiglu16(float g, float u) { return f16r(f16r(g * sigmoid16(g)) * u); }
+
+// ---- wave64 butterflies ---------------------------------------------------------------------------
+template <int WIDTH>
+SL_DEV float tree_sum(float v) {
+#pragma unroll
+  for (int m = 1; m < WIDTH; m <<= 1) v = v + __shfl_xor(v, m, 64);
+  return v;
+}
+template <int WIDTH>
+SL_DEV float tree_max(float v) {
+#pragma unroll
+  for (int m = 1; m < WIDTH; m <<= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+  return v;
+}
+
+// ---- 16-byte vector access -------------------------------------------------------------------------
+SL_DEV uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+SL_DEV void st16(void* p, uint4 v) { *reinterpret_cast<uint4*>(p) = v; }
+SL_DEV float lo_h(uint32_t u) { return h2f((uint16_t)(u & 0xffffu)); }
+SL_DEV float hi_h(uint32_t u) { return h2f((uint16_t)(u >> 16)); }
+// 8 halves (one uint4) -> 8 floats
+SL_DEV void unpack8(uint4 v, float* f) {
+  f[0] = lo_h(v.x); f[1] = hi_h(v.x); f[2] = lo_h(v.y); f[3] = hi_h(v.y);
+  f[4] = lo_h(v.z); f[5] = hi_h(v.z); f[6] = lo_h(v.w); f[7] = hi_h(v.w);
+}
+SL_DEV uint32_t pack2(float a, float b) { return (uint32_t)f2h(a) | ((uint32_t)f2h(b) << 16); }
+SL_DEV uint4 pack8(const float* f) {
+  return make_uint4(pack2(f[0], f[1]), pack2(f[2], f[3]), pack2(f[4], f[5]), pack2(f[6], f[7]));
+}
+
+// ---- one packed word against 8 activations ---------------------------------------------------------
+// dq = fmaf chain over the 8 nibbles, least significant first.
+SL_DEV float word_dot(uint32_t w, const float* x) {
+  float dq = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) dq = fmaf(x[i], (float)((w >> (4 * i)) & 15u), dq);
+  return dq;
+}
+// Four consecutive words of one group-half: t_j = fmaf(s, dq_j, b*sx_j); returns (t0+t1)+(t2+t3).
+SL_DEV float quad_term(uint4 w, uint32_t sb, const float* x /*32*/, const float* sx /*4*/) {
+  const float s = lo_h(sb), b = hi_h(sb);
+  float t0 = fmaf(s, word_dot(w.x, x), b * sx[0]);
+  float t1 = fmaf(s, word_dot(w.y, x + 8), b * sx[1]);
+  float t2 = fmaf(s, word_dot(w.z, x + 16), b * sx[2]);
+  float t3 = fmaf(s, word_dot(w.w, x + 24), b * sx[3]);
+  return (t0 + t1) + (t2 + t3);
+}
+// Left-to-right sums of each run of 8 activations.
+SL_DEV void word_sums(const float* x /*32*/, float* sx /*4*/) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s = s + x[8 * j + i];
+    sx[j] = s;
+  }
+}
+
+// ---- counter-based generator (the same rule a host implementation can state) -----------------------
+SL_DEV uint64_t hash64(uint64_t seed, uint64_t idx) {
+  uint64_t z = (idx + 1ull) * 0x9E3779B97F4A7C15ull ^ (seed * 0xD1B54A32D192ED03ull + 0x8CB92BA72F3D8DD7ull);
+  z ^= z >> 30; z *= 0xBF58476D1CE4E5B9ull;
+  z ^= z >> 27; z *= 0x94D049BB133111EBull;
+  z ^= z >> 31;
+  return z;
+}
+SL_DEV float uniform01(uint64_t seed, uint64_t idx) {
+  uint32_t k = (uint32_t)(hash64(seed, idx) >> 41);
+  return (float)(2u * k + 1u) * 5.9604644775390625e-8f;
+}
+// Wichura AS241 PPND7, single precision.
+SL_DEV float ppnd7(float p) {
+  float q = p - 0.5f;
+  if (fabsf(q) <= 0.425f) {
+    float r = 0.180625f - q * q;
+    float num = ((5.9109374720e+01f * r + 1.5929113202e+02f) * r + 5.0434271938e+01f) * r + 3.3871327179e+00f;
+    float den = ((6.7187563600e+01f * r + 7.8757757664e+01f) * r + 1.7895169469e+01f) * r + 1.0f;
+    return q * num / den;
+  }
+  float r = (q < 0.0f) ? p : (1.0f - p);
+  r = sqrtf(-log_c(r));
+  float v;
+  if (r <= 5.0f) {
+    r = r - 1.6f;
+    float num = ((1.7023821103e-01f * r + 1.3067284816e+00f) * r + 2.7568153900e+00f) * r + 1.4234372777e+00f;
+    float den = (1.2021132975e-01f * r + 7.3700164250e-01f) * r + 1.0f;
+    v = num / den;
+  } else {
+    r = r - 5.0f;
+    float num = ((1.7337203997e-02f * r + 4.2868294337e-01f) * r + 3.0812263860e+00f) * r + 6.6579051150e+00f;
+    float den = (1.2258202635e-02f * r + 2.4197894225e-01f) * r + 1.0f;
+    v = num / den;
+  }
+  return (q < 0.0f) ? -v : v;
+}
+SL_DEV float normal01(uint64_t seed, uint64_t idx) { return ppnd7(uniform01(seed, idx)); }
+
+}  // namespace sl

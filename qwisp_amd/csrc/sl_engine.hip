@@ -1,0 +1,742 @@
+// Host side of libseedless_hip.so: persistent device buffers, the per-step launch sequence and
+// the C ABI declared in include/seedless_hip.h.  Mirrors SeedlessFusedForward
+// (SeedlessFusedVerify.swift:3111-4470 in the reference): weights, caches and scratch are
+// allocated once at creation; a step enqueues its kernels on one stream and reads back int32
+// token ids.  No CPU fallback exists: without a GPU every entry point fails.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "sl_kernels.cuh"
+
+using namespace sl;
+
+namespace {
+
+struct DevQ4 {
+  uint32_t* w = nullptr;    // [n, k/8]
+  uint32_t* sb = nullptr;   // [n, k/64] {scale, bias}
+  int n = 0, k = 0;
+};
+
+struct LayerDev {
+  int is_linear = 0;
+  uint16_t *input_ln = nullptr, *post_ln = nullptr;
+  // Gated-DeltaNet
+  DevQ4 in_proj, out_proj;
+  float *conv_w = nullptr, *a_log = nullptr, *dt_bias = nullptr;
+  uint16_t* gdn_norm_w = nullptr;
+  uint16_t* hist[2] = {nullptr, nullptr};
+  float* state[2] = {nullptr, nullptr};
+  // attention
+  DevQ4 qkv, o_proj;
+  uint16_t *q_norm = nullptr, *k_norm = nullptr, *kcache = nullptr, *vcache = nullptr;
+  // MoE
+  uint16_t *router_w = nullptr, *sgate_w = nullptr;
+  DevQ4 sw_gate, sw_up, sw_down, sh_gate, sh_up, sh_down;
+  int32_t* route_inds = nullptr;
+  uint16_t* route_scores = nullptr;
+};
+
+constexpr size_t HIST_ELEMS = (size_t)(SL_CONV_K - 1) * SL_CONV_DIM;
+constexpr size_t STATE_ELEMS = (size_t)SL_GDN_HV * SL_GDN_D * SL_GDN_D;
+constexpr int MAX_CHAIN = 256;
+
+}  // namespace
+
+struct sl_full_snap {
+  int pos = 0;
+  std::vector<uint16_t*> hist;   // device copies, null for attention layers
+  std::vector<float*> state;
+};
+
+struct sl_engine {
+  int n_layers = 0, n_experts = 0, vocab = 0, max_m = 0, max_seq = 0, max_tiles = 0;
+  bool has_attn = false, has_head = false;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  std::vector<void*> allocs;
+  std::vector<LayerDev> layers;
+  DevQ4 embed, lm_head;
+  uint16_t* final_norm = nullptr;
+  float *rope_cos = nullptr, *rope_sin = nullptr;
+  // scratch
+  uint16_t *hA = nullptr, *hB = nullptr, *proj = nullptr, *ycore = nullptr, *qrot = nullptr, *mix = nullptr, *xn = nullptr;
+  uint16_t *rlogits = nullptr, *sgate = nullptr, *sh_act = nullptr, *act = nullptr, *moe_out = nullptr, *normed = nullptr;
+  uint16_t *logits = nullptr, *rows_out = nullptr;
+  float *pm = nullptr, *pl = nullptr, *po = nullptr, *cand_v = nullptr;
+  int32_t *cand_i = nullptr, *tok_in = nullptr, *tok_out = nullptr, *st = nullptr;
+  int n_cand = 0;
+  void* pinned = nullptr;        // host staging
+  size_t pinned_bytes = 0;
+  // host mirrors of the device step state
+  int pos = 0;
+  std::vector<int> parity;
+  float last_ms = 0.0f;
+  bool inject_failure = false;
+  std::string fault;
+};
+
+namespace {
+
+bool ok(sl_engine* e, hipError_t r, const char* what) {
+  if (r == hipSuccess) return true;
+  if (e->fault.empty()) e->fault = std::string(what) + ": " + hipGetErrorString(r);
+  return false;
+}
+#define SL_TRY(e, call) do { if (!ok((e), (call), #call)) return SL_ERR_DEVICE; } while (0)
+
+template <typename T>
+T* dalloc(sl_engine* e, size_t count, bool zero = false) {
+  void* p = nullptr;
+  if (!ok(e, hipMalloc(&p, count * sizeof(T) > 0 ? count * sizeof(T) : 16), "hipMalloc")) return nullptr;
+  e->allocs.push_back(p);
+  if (zero && !ok(e, hipMemsetAsync(p, 0, count * sizeof(T), e->stream), "hipMemsetAsync")) return nullptr;
+  return (T*)p;
+}
+bool copy_in(sl_engine* e, void* dst, const void* src, size_t bytes, int loc) {
+  return ok(e, hipMemcpyAsync(dst, src, bytes, loc == SL_LOC_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice, e->stream),
+            "hipMemcpyAsync(weights)") &&
+         (loc != SL_LOC_HOST || ok(e, hipStreamSynchronize(e->stream), "hipStreamSynchronize"));
+}
+template <typename T>
+T* upload(sl_engine* e, const void* src, size_t count, int loc) {
+  if (!src) { if (e->fault.empty()) e->fault = "null tensor in model description"; return nullptr; }
+  T* d = dalloc<T>(e, count);
+  if (!d || !copy_in(e, d, src, count * sizeof(T), loc)) return nullptr;
+  return d;
+}
+bool alloc_q4(sl_engine* e, DevQ4& d, int n, int k) {
+  d.n = n; d.k = k;
+  d.w = dalloc<uint32_t>(e, (size_t)n * (k / 8));
+  d.sb = dalloc<uint32_t>(e, (size_t)n * (k / 64));
+  return d.w && d.sb;
+}
+// Copies rows of `src` into rows [row_off, row_off + src.n) of `dst`, interleaving scale/bias.
+bool fill_q4(sl_engine* e, DevQ4& dst, int row_off, const sl_q4& src, int n, int k, int loc) {
+  if (!src.w || !src.scales || !src.biases || src.n != n || src.k != k || dst.k != k || row_off + n > dst.n) {
+    if (e->fault.empty()) e->fault = "quantized tensor missing or of the wrong shape";
+    return false;
+  }
+  const size_t wcount = (size_t)n * (k / 8), gcount = (size_t)n * (k / 64);
+  if (!copy_in(e, dst.w + (size_t)row_off * (k / 8), src.w, wcount * 4, loc)) return false;
+  uint32_t* out = dst.sb + (size_t)row_off * (k / 64);
+  if (loc == SL_LOC_HOST) {
+    std::vector<uint32_t> tmp(gcount);
+    for (size_t i = 0; i < gcount; ++i) tmp[i] = (uint32_t)src.scales[i] | ((uint32_t)src.biases[i] << 16);
+    return copy_in(e, out, tmp.data(), gcount * 4, SL_LOC_HOST);
+  }
+  hipLaunchKernelGGL(k_pack_sb, dim3((unsigned)((gcount + 255) / 256)), dim3(256), 0, e->stream, src.scales, src.biases, out, gcount);
+  return ok(e, hipGetLastError(), "k_pack_sb");
+}
+bool upload_q4(sl_engine* e, DevQ4& d, const sl_q4& src, int n, int k, int loc) {
+  return alloc_q4(e, d, n, k) && fill_q4(e, d, 0, src, n, k, loc);
+}
+
+void build_rope(std::vector<float>& c, std::vector<float>& s, int max_seq) {
+  c.resize((size_t)max_seq * 32); s.resize((size_t)max_seq * 32);
+  for (int i = 0; i < 32; ++i) {
+    // freq = theta^(-2i/64), theta = 1e7; the angle is formed in fp32 as in attn_q_prep_rows
+    // (SeedlessFusedVerify.swift:1240-1242), its cosine and sine are taken in double.
+    const float freq = (float)std::exp(-2.0 * (double)i / (double)SL_ROPE_DIM * std::log(1e7));
+    for (int p = 0; p < max_seq; ++p) {
+      const float ang = (float)p * freq;
+      c[(size_t)p * 32 + i] = (float)std::cos((double)ang);
+      s[(size_t)p * 32 + i] = (float)std::sin((double)ang);
+    }
+  }
+}
+
+int push_state(sl_engine* e, int layer_parity_only = -1) {
+  (void)layer_parity_only;
+  std::vector<int32_t> h(1 + e->n_layers);
+  h[0] = e->pos;
+  for (int i = 0; i < e->n_layers; ++i) h[1 + i] = e->parity[i];
+  std::memcpy(e->pinned, h.data(), h.size() * 4);
+  SL_TRY(e, hipMemcpyAsync(e->st, e->pinned, h.size() * 4, hipMemcpyHostToDevice, e->stream));
+  SL_TRY(e, hipStreamSynchronize(e->stream));
+  return SL_OK;
+}
+
+int guard(sl_engine* e) {
+  if (!e) return SL_ERR_ARG;
+  if (!e->fault.empty()) return SL_ERR_POISONED;
+  return SL_OK;
+}
+int check_rows(sl_engine* e, int m) {
+  if (m < 1 || m > e->max_m) return SL_ERR_ARG;
+  if (e->has_attn && e->pos + m > e->max_seq) return SL_ERR_ARG;
+  return SL_OK;
+}
+// Waits for the stream; the injected failure stands in for a failed submission.
+int finish(sl_engine* e, const char* what) {
+  hipError_t r = hipStreamSynchronize(e->stream);
+  if (r == hipSuccess) r = hipGetLastError();
+  if (e->inject_failure) {
+    e->inject_failure = false;
+    e->fault = std::string(what) + ": injected device failure";
+    return SL_ERR_DEVICE;
+  }
+  if (!ok(e, r, what)) return SL_ERR_DEVICE;
+  return SL_OK;
+}
+
+// ---- launch sequences -------------------------------------------------------------------------------
+void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
+  MoeAArgs a{};
+  a.ha = ha;
+  a.shg_w = L.sh_gate.w; a.shg_sb = L.sh_gate.sb; a.shu_w = L.sh_up.w; a.shu_sb = L.sh_up.sb;
+  a.router_w = L.router_w; a.sgate_w = L.sgate_w; a.E = e->n_experts;
+  a.sh_act = e->sh_act; a.rlogits = e->rlogits; a.sgate = e->sgate;
+  const int router_blocks = (e->n_experts + 1 + 15) / 16;
+  hipLaunchKernelGGL(k_moe_a, dim3(MOE_A_SHARED_BLOCKS + router_blocks, M), dim3(256), 0, e->stream, a);
+  MoeBArgs b{};
+  b.xn = e->xn; b.rlogits = e->rlogits; b.E = e->n_experts;
+  b.g_w = L.sw_gate.w; b.g_sb = L.sw_gate.sb; b.u_w = L.sw_up.w; b.u_sb = L.sw_up.sb;
+  b.act = e->act; b.inds = L.route_inds; b.scores = L.route_scores;
+  hipLaunchKernelGGL(k_moe_b, dim3(512, M), dim3(256), 0, e->stream, b);
+  MoeCArgs c{};
+  c.act = e->act; c.sh_act = e->sh_act; c.inds = L.route_inds; c.scores = L.route_scores; c.sgate = e->sgate;
+  c.d_w = L.sw_down.w; c.d_sb = L.sw_down.sb; c.shd_w = L.sh_down.w; c.shd_sb = L.sh_down.sb; c.out = e->moe_out;
+  hipLaunchKernelGGL(k_moe_c, dim3(256, M), dim3(128), 0, e->stream, c);
+}
+void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs& ha) {
+  hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_GDN_IN_N / 16, M), dim3(256), 0, e->stream, ha, L.in_proj.w, L.in_proj.sb,
+                     SL_GDN_IN_N, e->proj, PROJ_STRIDE);
+  GdnArgs g{};
+  g.proj = e->proj; g.conv_w = L.conv_w; g.a_log = L.a_log; g.dt_bias = L.dt_bias;
+  g.hist[0] = L.hist[0]; g.hist[1] = L.hist[1]; g.state[0] = L.state[0]; g.state[1] = L.state[1];
+  g.st = e->st + li;       // st[1] of this view = parity of layer li
+  g.ycore = e->ycore; g.M = M;
+  hipLaunchKernelGGL(k_gdn_core, dim3(256), dim3(256), 0, e->stream, g);
+  hipLaunchKernelGGL(k_qmv_gdn_out<2>, dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w,
+                     L.out_proj.w, L.out_proj.sb, H, e->mix);
+}
+void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
+  hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_ATT_QKV_N / 16, M), dim3(256), 0, e->stream, ha, L.qkv.w, L.qkv.sb,
+                     SL_ATT_QKV_N, e->proj, PROJ_STRIDE);
+  AttnPrepArgs p{};
+  p.proj = e->proj; p.q_norm = L.q_norm; p.k_norm = L.k_norm; p.rope_cos = e->rope_cos; p.rope_sin = e->rope_sin;
+  p.st = e->st; p.qrot = e->qrot; p.kcache = L.kcache; p.vcache = L.vcache; p.maxSeq = e->max_seq;
+  hipLaunchKernelGGL(k_attn_prep, dim3(18, M), dim3(64), 0, e->stream, p);
+  const int tiles = (e->pos + M + SDPA_TILE - 1) / SDPA_TILE;
+  SdpaArgs s{};
+  s.qrot = e->qrot; s.kcache = L.kcache; s.vcache = L.vcache; s.st = e->st; s.maxSeq = e->max_seq; s.maxTiles = e->max_tiles;
+  s.pm = e->pm; s.pl = e->pl; s.po = e->po;
+  hipLaunchKernelGGL(k_sdpa_tile, dim3(tiles, SL_ATT_KV, M), dim3(64), 0, e->stream, s);
+  SdpaMergeArgs g{};
+  g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore;
+  hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
+  hipLaunchKernelGGL((k_qmv_plain<2, 2>), dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, 4096, L.o_proj.w, L.o_proj.sb,
+                     H, e->mix, H);
+}
+// All layers over M rows held in hA.  On return the hidden state is hA + moe_out (residual pending).
+void launch_layers(sl_engine* e, int M) {
+  for (int li = 0; li < e->n_layers; ++li) {
+    LayerDev& L = e->layers[li];
+    HiddenArgs ha{e->hA, li > 0 ? e->moe_out : nullptr, L.input_ln, e->hB, nullptr};
+    if (L.is_linear) launch_gdn_mixer(e, L, li, M, ha);
+    else launch_attn_mixer(e, L, M, ha);
+    HiddenArgs hb{e->hB, e->mix, L.post_ln, e->hA, e->xn};
+    launch_moe(e, L, M, hb);
+  }
+}
+void advance(sl_engine* e, int M) {
+  hipLaunchKernelGGL(k_advance, dim3(1), dim3(64), 0, e->stream, e->st, M, e->n_layers);
+  e->pos += M;
+  for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
+}
+void launch_head(sl_engine* e, int M, const HiddenArgs& ha, int out_off, bool feed) {
+  hipLaunchKernelGGL(k_head, dim3(e->n_cand, M), dim3(256), 0, e->stream, ha, e->lm_head.w, e->lm_head.sb, e->vocab,
+                     e->logits, e->cand_v, e->cand_i);
+  hipLaunchKernelGGL(k_argmax_final, dim3(M), dim3(256), 0, e->stream, e->cand_v, e->cand_i, e->n_cand, e->tok_out, out_off,
+                     feed ? e->tok_in : (int32_t*)nullptr);
+}
+int to_device(sl_engine* e, void* dst, const void* src, size_t bytes) {
+  if (bytes > e->pinned_bytes) return SL_ERR_ARG;
+  std::memcpy(e->pinned, src, bytes);
+  SL_TRY(e, hipMemcpyAsync(dst, e->pinned, bytes, hipMemcpyHostToDevice, e->stream));
+  return SL_OK;
+}
+// Large transfers (caches, snapshots) go straight between the caller's memory and the device.
+int copy_sync(sl_engine* e, void* dst, const void* src, size_t bytes, hipMemcpyKind kind) {
+  SL_TRY(e, hipMemcpyAsync(dst, src, bytes, kind, e->stream));
+  SL_TRY(e, hipStreamSynchronize(e->stream));
+  return SL_OK;
+}
+
+bool shape_ok(const sl_q4& q, int n, int k) { return q.w && q.scales && q.biases && q.n == n && q.k == k; }
+
+}  // namespace
+
+extern "C" {
+
+int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** out) {
+  if (!d || !out || max_m < 1 || max_seq_len < 1 || d->n_layers < 1 || !d->layers) return SL_ERR_ARG;
+  if (d->n_experts < 8 || d->n_experts > SL_MAX_EXPERTS || (d->n_experts % 8) != 0) return SL_ERR_ARG;
+  if (d->location != SL_LOC_HOST && d->location != SL_LOC_DEVICE) return SL_ERR_ARG;
+  const bool has_head = d->embed.w != nullptr;
+  if (has_head && (d->vocab < 16 || (d->vocab % 16) != 0 || !shape_ok(d->embed, d->vocab, H) ||
+                   !shape_ok(d->lm_head, d->vocab, H) || !d->final_norm)) return SL_ERR_ARG;
+  int ndev = 0;
+  if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) return SL_ERR_DEVICE;
+
+  sl_engine* e = new sl_engine();
+  *out = e;   // returned even on failure so the caller can read sl_fault() and must sl_destroy()
+  e->n_layers = d->n_layers; e->n_experts = d->n_experts; e->vocab = has_head ? d->vocab : 0;
+  e->max_m = max_m; e->max_seq = max_seq_len; e->max_tiles = (max_seq_len + SDPA_TILE - 1) / SDPA_TILE;
+  e->has_head = has_head;
+  e->parity.assign(d->n_layers, 0);
+  SL_TRY(e, hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
+  SL_TRY(e, hipEventCreate(&e->ev0));
+  SL_TRY(e, hipEventCreate(&e->ev1));
+  const int loc = d->location, E = d->n_experts;
+  e->layers.resize(d->n_layers);
+  for (int i = 0; i < d->n_layers; ++i) {
+    const sl_layer_desc& s = d->layers[i];
+    LayerDev& L = e->layers[i];
+    L.is_linear = s.is_linear;
+    L.input_ln = upload<uint16_t>(e, s.input_ln, H, loc);
+    L.post_ln = upload<uint16_t>(e, s.post_ln, H, loc);
+    if (!L.input_ln || !L.post_ln) return SL_ERR_DEVICE;
+    if (s.is_linear) {
+      const sl_gdn_w& g = s.gdn;
+      if (!alloc_q4(e, L.in_proj, SL_GDN_IN_N, H)) return SL_ERR_DEVICE;
+      if (!fill_q4(e, L.in_proj, 0, g.in_proj_qkv, SL_CONV_DIM, H, loc) ||
+          !fill_q4(e, L.in_proj, SL_CONV_DIM, g.in_proj_z, 4096, H, loc) ||
+          !fill_q4(e, L.in_proj, SL_CONV_DIM + 4096, g.in_proj_b, SL_GDN_HV, H, loc) ||
+          !fill_q4(e, L.in_proj, SL_CONV_DIM + 4096 + SL_GDN_HV, g.in_proj_a, SL_GDN_HV, H, loc) ||
+          !upload_q4(e, L.out_proj, g.out_proj, H, 4096, loc)) return SL_ERR_ARG;
+      L.conv_w = upload<float>(e, g.conv1d_w, (size_t)SL_CONV_DIM * SL_CONV_K, loc);
+      L.a_log = upload<float>(e, g.a_log, SL_GDN_HV, loc);
+      L.dt_bias = upload<float>(e, g.dt_bias, SL_GDN_HV, loc);
+      L.gdn_norm_w = upload<uint16_t>(e, g.norm_w, SL_GDN_D, loc);
+      for (int p = 0; p < 2; ++p) {
+        L.hist[p] = dalloc<uint16_t>(e, HIST_ELEMS, true);
+        L.state[p] = dalloc<float>(e, STATE_ELEMS, true);
+      }
+      if (!L.conv_w || !L.a_log || !L.dt_bias || !L.gdn_norm_w || !L.hist[1] || !L.state[1]) return SL_ERR_DEVICE;
+    } else {
+      e->has_attn = true;
+      const sl_attn_w& a = s.attn;
+      if (!alloc_q4(e, L.qkv, SL_ATT_QKV_N, H)) return SL_ERR_DEVICE;
+      if (!fill_q4(e, L.qkv, 0, a.q_proj, 8192, H, loc) || !fill_q4(e, L.qkv, 8192, a.k_proj, 512, H, loc) ||
+          !fill_q4(e, L.qkv, 8192 + 512, a.v_proj, 512, H, loc) || !upload_q4(e, L.o_proj, a.o_proj, H, 4096, loc))
+        return SL_ERR_ARG;
+      L.q_norm = upload<uint16_t>(e, a.q_norm, SL_ATT_D, loc);
+      L.k_norm = upload<uint16_t>(e, a.k_norm, SL_ATT_D, loc);
+      L.kcache = dalloc<uint16_t>(e, (size_t)SL_ATT_KV * max_seq_len * SL_ATT_D, true);
+      L.vcache = dalloc<uint16_t>(e, (size_t)SL_ATT_KV * max_seq_len * SL_ATT_D, true);
+      if (!L.q_norm || !L.k_norm || !L.kcache || !L.vcache) return SL_ERR_DEVICE;
+    }
+    const sl_moe_w& w = s.moe;
+    L.router_w = upload<uint16_t>(e, w.router_w, (size_t)E * H, loc);
+    L.sgate_w = upload<uint16_t>(e, w.shared_gate_w, H, loc);
+    if (!L.router_w || !L.sgate_w) return SL_ERR_DEVICE;
+    if (!upload_q4(e, L.sw_gate, w.sw_gate, E * SL_MOE_I, H, loc) || !upload_q4(e, L.sw_up, w.sw_up, E * SL_MOE_I, H, loc) ||
+        !upload_q4(e, L.sw_down, w.sw_down, E * H, SL_MOE_I, loc) || !upload_q4(e, L.sh_gate, w.sh_gate, SL_MOE_I, H, loc) ||
+        !upload_q4(e, L.sh_up, w.sh_up, SL_MOE_I, H, loc) || !upload_q4(e, L.sh_down, w.sh_down, H, SL_MOE_I, loc))
+      return SL_ERR_ARG;
+    L.route_inds = dalloc<int32_t>(e, (size_t)max_m * 8, true);
+    L.route_scores = dalloc<uint16_t>(e, (size_t)max_m * 8, true);
+    if (!L.route_inds || !L.route_scores) return SL_ERR_DEVICE;
+  }
+  if (has_head) {
+    if (!upload_q4(e, e->embed, d->embed, d->vocab, H, loc) || !upload_q4(e, e->lm_head, d->lm_head, d->vocab, H, loc))
+      return SL_ERR_ARG;
+    e->final_norm = upload<uint16_t>(e, d->final_norm, H, loc);
+    e->n_cand = d->vocab / 16;
+    e->logits = dalloc<uint16_t>(e, (size_t)max_m * d->vocab);
+    e->cand_v = dalloc<float>(e, (size_t)max_m * e->n_cand);
+    e->cand_i = dalloc<int32_t>(e, (size_t)max_m * e->n_cand);
+    if (!e->final_norm || !e->logits || !e->cand_v || !e->cand_i) return SL_ERR_DEVICE;
+  }
+  if (e->has_attn) {
+    std::vector<float> c, s;
+    build_rope(c, s, max_seq_len);
+    e->rope_cos = upload<float>(e, c.data(), c.size(), SL_LOC_HOST);
+    e->rope_sin = upload<float>(e, s.data(), s.size(), SL_LOC_HOST);
+    e->pm = dalloc<float>(e, (size_t)max_m * 16 * e->max_tiles);
+    e->pl = dalloc<float>(e, (size_t)max_m * 16 * e->max_tiles);
+    e->po = dalloc<float>(e, (size_t)max_m * 16 * e->max_tiles * 256);
+    e->qrot = dalloc<uint16_t>(e, (size_t)max_m * 16 * 256);
+    if (!e->rope_cos || !e->rope_sin || !e->pm || !e->pl || !e->po || !e->qrot) return SL_ERR_DEVICE;
+  }
+  const size_t MH = (size_t)max_m * H;
+  e->hA = dalloc<uint16_t>(e, MH, true); e->hB = dalloc<uint16_t>(e, MH, true);
+  e->proj = dalloc<uint16_t>(e, (size_t)max_m * PROJ_STRIDE, true);
+  e->ycore = dalloc<uint16_t>(e, (size_t)max_m * 4096, true);
+  e->mix = dalloc<uint16_t>(e, MH, true); e->xn = dalloc<uint16_t>(e, MH, true);
+  e->rlogits = dalloc<uint16_t>(e, (size_t)max_m * 256, true); e->sgate = dalloc<uint16_t>(e, max_m, true);
+  e->sh_act = dalloc<uint16_t>(e, (size_t)max_m * 512, true); e->act = dalloc<uint16_t>(e, (size_t)max_m * 8 * 512, true);
+  e->moe_out = dalloc<uint16_t>(e, MH, true); e->normed = dalloc<uint16_t>(e, MH, true);
+  e->rows_out = dalloc<uint16_t>(e, MH, true);
+  e->tok_in = dalloc<int32_t>(e, max_m, true);
+  e->tok_out = dalloc<int32_t>(e, max_m > MAX_CHAIN ? max_m : MAX_CHAIN, true);
+  e->st = dalloc<int32_t>(e, 1 + d->n_layers, true);
+  if (!e->hA || !e->hB || !e->proj || !e->ycore || !e->mix || !e->xn || !e->rlogits || !e->sgate || !e->sh_act || !e->act ||
+      !e->moe_out || !e->normed || !e->rows_out || !e->tok_in || !e->tok_out || !e->st) return SL_ERR_DEVICE;
+  e->pinned_bytes = MH * 2 + 4096 + (size_t)d->n_layers * 4 + (size_t)MAX_CHAIN * 4;
+  SL_TRY(e, hipHostMalloc(&e->pinned, e->pinned_bytes, hipHostMallocDefault));
+  SL_TRY(e, hipStreamSynchronize(e->stream));
+  return SL_OK;
+}
+
+void sl_destroy(sl_engine* e) {
+  if (!e) return;
+  if (e->stream) (void)hipStreamSynchronize(e->stream);
+  for (void* p : e->allocs) (void)hipFree(p);
+  if (e->pinned) (void)hipHostFree(e->pinned);
+  if (e->ev0) (void)hipEventDestroy(e->ev0);
+  if (e->ev1) (void)hipEventDestroy(e->ev1);
+  if (e->stream) (void)hipStreamDestroy(e->stream);
+  delete e;
+}
+
+const char* sl_fault(const sl_engine* e) { return (e && !e->fault.empty()) ? e->fault.c_str() : nullptr; }
+void sl_inject_failure(sl_engine* e) { if (e) e->inject_failure = true; }
+int sl_position(const sl_engine* e) { return e ? e->pos : -1; }
+float sl_last_gpu_ms(const sl_engine* e) { return e ? e->last_ms : 0.0f; }
+void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
+
+static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, const char* what) {
+  if (bytes > e->pinned_bytes) return SL_ERR_ARG;
+  SL_TRY(e, hipMemcpyAsync(e->pinned, dev, bytes, hipMemcpyDeviceToHost, e->stream));
+  int r = finish(e, what);
+  if (r) return r;
+  std::memcpy(dst, e->pinned, bytes);
+  return SL_OK;
+}
+static void time_end(sl_engine* e) {
+  float ms = 0.0f;
+  if (hipEventElapsedTime(&ms, e->ev0, e->ev1) == hipSuccess) e->last_ms = ms;
+}
+
+int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!tokens || !out || !e->has_head) return SL_ERR_ARG;
+  r = check_rows(e, m); if (r) return r;
+  for (int i = 0; i < m; ++i) if (tokens[i] < 0 || tokens[i] >= e->vocab) return SL_ERR_ARG;
+  r = to_device(e, e->tok_in, tokens, (size_t)m * 4); if (r) return r;
+  SL_TRY(e, hipEventRecord(e->ev0, e->stream));
+  hipLaunchKernelGGL(k_embed, dim3(H / 256, m), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
+  launch_layers(e, m);
+  HiddenArgs ha{e->hA, e->moe_out, e->final_norm, e->hB, e->normed};
+  launch_head(e, m, ha, 0, false);
+  advance(e, m);
+  SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+  r = read_back(e, out, e->tok_out, (size_t)m * 4, "stepArgmax"); if (r) return r;
+  time_end(e);
+  return SL_OK;
+}
+
+int sl_chained_step_argmax(sl_engine* e, int32_t first, int k, int32_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!out || !e->has_head || k < 1 || k > MAX_CHAIN || first < 0 || first >= e->vocab) return SL_ERR_ARG;
+  if (e->has_attn && e->pos + k > e->max_seq) return SL_ERR_ARG;
+  r = to_device(e, e->tok_in, &first, 4); if (r) return r;
+  SL_TRY(e, hipEventRecord(e->ev0, e->stream));
+  for (int s = 0; s < k; ++s) {
+    hipLaunchKernelGGL(k_embed, dim3(H / 256, 1), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
+    launch_layers(e, 1);
+    HiddenArgs ha{e->hA, e->moe_out, e->final_norm, e->hB, e->normed};
+    launch_head(e, 1, ha, s, true);
+    advance(e, 1);
+  }
+  SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+  r = read_back(e, out, e->tok_out, (size_t)k * 4, "chainedStepArgmax"); if (r) return r;
+  time_end(e);
+  return SL_OK;
+}
+
+static int forward_common(sl_engine* e, int m, int final_norm, uint16_t* out, const char* what) {
+  SL_TRY(e, hipEventRecord(e->ev0, e->stream));
+  launch_layers(e, m);
+  HiddenArgs ha{e->hA, e->moe_out, final_norm ? e->final_norm : nullptr, final_norm ? e->hB : e->rows_out,
+                final_norm ? e->normed : nullptr};
+  hipLaunchKernelGGL(k_final_rows, dim3(m), dim3(64), 0, e->stream, ha);
+  advance(e, m);
+  SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+  int r = read_back(e, out, final_norm ? e->normed : e->rows_out, (size_t)m * H * 2, what); if (r) return r;
+  time_end(e);
+  return SL_OK;
+}
+int sl_forward_rows(sl_engine* e, const uint16_t* x, int m, int final_norm, uint16_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!x || !out || (final_norm && !e->final_norm)) return SL_ERR_ARG;
+  r = check_rows(e, m); if (r) return r;
+  r = to_device(e, e->hA, x, (size_t)m * H * 2); if (r) return r;
+  return forward_common(e, m, final_norm, out, "forwardRows");
+}
+int sl_forward_tokens(sl_engine* e, const int32_t* tokens, int m, uint16_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!tokens || !out || !e->has_head) return SL_ERR_ARG;
+  r = check_rows(e, m); if (r) return r;
+  for (int i = 0; i < m; ++i) if (tokens[i] < 0 || tokens[i] >= e->vocab) return SL_ERR_ARG;
+  r = to_device(e, e->tok_in, tokens, (size_t)m * 4); if (r) return r;
+  hipLaunchKernelGGL(k_embed, dim3(H / 256, m), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
+  return forward_common(e, m, 1, out, "forward");
+}
+int sl_hidden_rows(sl_engine* e, int m, uint16_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!out || m < 1 || m > e->max_m) return SL_ERR_ARG;
+  return read_back(e, out, e->normed, (size_t)m * H * 2, "hiddenRows");
+}
+int sl_logits_row(sl_engine* e, int m, uint16_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!out || !e->has_head || m < 0 || m >= e->max_m) return SL_ERR_ARG;
+  r = copy_sync(e, out, e->logits + (size_t)m * e->vocab, (size_t)e->vocab * 2, hipMemcpyDeviceToHost);
+  return r;
+}
+int sl_head_argmax(sl_engine* e, const uint16_t* normed, int m, int32_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!normed || !out || !e->has_head || m < 1 || m > e->max_m) return SL_ERR_ARG;
+  r = to_device(e, e->xn, normed, (size_t)m * H * 2); if (r) return r;
+  HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
+  launch_head(e, m, ha, 0, false);
+  return read_back(e, out, e->tok_out, (size_t)m * 4, "headArgmax");
+}
+
+int sl_snapshot(sl_engine* e, sl_snap* s) {
+  int r = guard(e); if (r) return r;
+  if (!s) return SL_ERR_ARG;
+  s->kv_len = e->pos; s->reserved = 0;
+  return SL_OK;
+}
+int sl_rollback_one_step(sl_engine* e, const sl_snap* s) {
+  int r = guard(e); if (r) return r;
+  if (!s || s->kv_len < 0 || s->kv_len > e->pos) return SL_ERR_ARG;
+  e->pos = s->kv_len;
+  for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
+  return push_state(e);
+}
+int sl_full_snapshot(sl_engine* e, sl_full_snap** out) {
+  int r = guard(e); if (r) return r;
+  if (!out) return SL_ERR_ARG;
+  sl_full_snap* s = new sl_full_snap();
+  s->pos = e->pos;
+  s->hist.assign(e->n_layers, nullptr); s->state.assign(e->n_layers, nullptr);
+  *out = s;
+  for (int i = 0; i < e->n_layers; ++i) {
+    LayerDev& L = e->layers[i];
+    if (!L.is_linear) continue;
+    SL_TRY(e, hipMalloc((void**)&s->hist[i], HIST_ELEMS * 2));
+    SL_TRY(e, hipMalloc((void**)&s->state[i], STATE_ELEMS * 4));
+    SL_TRY(e, hipMemcpyAsync(s->hist[i], L.hist[e->parity[i]], HIST_ELEMS * 2, hipMemcpyDeviceToDevice, e->stream));
+    SL_TRY(e, hipMemcpyAsync(s->state[i], L.state[e->parity[i]], STATE_ELEMS * 4, hipMemcpyDeviceToDevice, e->stream));
+  }
+  SL_TRY(e, hipStreamSynchronize(e->stream));
+  return SL_OK;
+}
+int sl_full_restore(sl_engine* e, const sl_full_snap* s) {
+  int r = guard(e); if (r) return r;
+  if (!s || (int)s->hist.size() != e->n_layers) return SL_ERR_ARG;
+  for (int i = 0; i < e->n_layers; ++i) {
+    LayerDev& L = e->layers[i];
+    if (!L.is_linear) continue;
+    if (!s->hist[i] || !s->state[i]) return SL_ERR_ARG;
+    SL_TRY(e, hipMemcpyAsync(L.hist[e->parity[i]], s->hist[i], HIST_ELEMS * 2, hipMemcpyDeviceToDevice, e->stream));
+    SL_TRY(e, hipMemcpyAsync(L.state[e->parity[i]], s->state[i], STATE_ELEMS * 4, hipMemcpyDeviceToDevice, e->stream));
+  }
+  e->pos = s->pos;
+  return push_state(e);
+}
+void sl_full_snap_free(sl_full_snap* s) {
+  if (!s) return;
+  for (auto p : s->hist) if (p) (void)hipFree(p);
+  for (auto p : s->state) if (p) (void)hipFree(p);
+  delete s;
+}
+
+// "QWS1" blob, little-endian (layout of persistentStateData, SeedlessFusedVerify.swift:4077-4111):
+// magic, format, nLayers, then per layer: flags (bit0 KV, bit1 GDN); KV: u32 KV, D, len, K bytes
+// (per head the used rows), V bytes; GDN: u32 convCount, stateCount, history bytes, state bytes.
+static const uint32_t PERSIST_MAGIC = 0x31535751u, PERSIST_FORMAT = 1u;
+size_t sl_persist_size(sl_engine* e) {
+  if (!e) return 0;
+  size_t n = 12;
+  for (auto& L : e->layers) {
+    n += 4;
+    if (L.is_linear) n += 8 + HIST_ELEMS * 2 + STATE_ELEMS * 4;
+    else n += 12 + 2 * (size_t)SL_ATT_KV * e->pos * SL_ATT_D * 2;
+  }
+  return n;
+}
+int sl_persist_write(sl_engine* e, void* dst, size_t cap) {
+  int r = guard(e); if (r) return r;
+  if (!dst || cap < sl_persist_size(e)) return SL_ERR_ARG;
+  uint8_t* p = (uint8_t*)dst;
+  auto u32 = [&](uint32_t v) { std::memcpy(p, &v, 4); p += 4; };
+  u32(PERSIST_MAGIC); u32(PERSIST_FORMAT); u32((uint32_t)e->n_layers);
+  for (int i = 0; i < e->n_layers; ++i) {
+    LayerDev& L = e->layers[i];
+    u32(L.is_linear ? 2u : 1u);
+    if (!L.is_linear) {
+      u32(SL_ATT_KV); u32(SL_ATT_D); u32((uint32_t)e->pos);
+      const size_t rb = (size_t)e->pos * SL_ATT_D * 2;
+      for (uint16_t* buf : {L.kcache, L.vcache})
+        for (int h = 0; h < SL_ATT_KV; ++h) {
+          if (rb) { r = copy_sync(e, p, buf + (size_t)h * e->max_seq * SL_ATT_D, rb, hipMemcpyDeviceToHost); if (r) return r; }
+          p += rb;
+        }
+    } else {
+      u32((uint32_t)HIST_ELEMS); u32((uint32_t)STATE_ELEMS);
+      r = copy_sync(e, p, L.hist[e->parity[i]], HIST_ELEMS * 2, hipMemcpyDeviceToHost); if (r) return r;
+      p += HIST_ELEMS * 2;
+      r = copy_sync(e, p, L.state[e->parity[i]], STATE_ELEMS * 4, hipMemcpyDeviceToHost); if (r) return r;
+      p += STATE_ELEMS * 4;
+    }
+  }
+  return SL_OK;
+}
+int sl_persist_restore(sl_engine* e, const void* src, size_t len) {
+  int r = guard(e); if (r) return r;
+  if (!src) return SL_ERR_ARG;
+  const uint8_t* p = (const uint8_t*)src;
+  const uint8_t* end = p + len;
+  auto u32 = [&](uint32_t& v) { if (end - p < 4) return false; std::memcpy(&v, p, 4); p += 4; return true; };
+  uint32_t v = 0;
+  if (!u32(v) || v != PERSIST_MAGIC || !u32(v) || v != PERSIST_FORMAT || !u32(v) || v != (uint32_t)e->n_layers) return SL_ERR_FORMAT;
+  int new_pos = e->has_attn ? -1 : e->pos;
+  for (int i = 0; i < e->n_layers; ++i) {
+    LayerDev& L = e->layers[i];
+    if (!u32(v) || v != (L.is_linear ? 2u : 1u)) return SL_ERR_FORMAT;
+    if (!L.is_linear) {
+      uint32_t kv = 0, dd = 0, ln = 0;
+      if (!u32(kv) || kv != SL_ATT_KV || !u32(dd) || dd != SL_ATT_D || !u32(ln) || ln > (uint32_t)e->max_seq) return SL_ERR_FORMAT;
+      if (new_pos >= 0 && (uint32_t)new_pos != ln) return SL_ERR_FORMAT;
+      new_pos = (int)ln;
+      const size_t rb = (size_t)ln * SL_ATT_D * 2;
+      for (uint16_t* buf : {L.kcache, L.vcache})
+        for (int h = 0; h < SL_ATT_KV; ++h) {
+          if ((size_t)(end - p) < rb) return SL_ERR_FORMAT;
+          if (rb) { r = copy_sync(e, buf + (size_t)h * e->max_seq * SL_ATT_D, p, rb, hipMemcpyHostToDevice); if (r) return r; }
+          p += rb;
+        }
+    } else {
+      uint32_t cc = 0, sc = 0;
+      if (!u32(cc) || cc != HIST_ELEMS || !u32(sc) || sc != STATE_ELEMS) return SL_ERR_FORMAT;
+      if ((size_t)(end - p) < HIST_ELEMS * 2 + STATE_ELEMS * 4) return SL_ERR_FORMAT;
+      r = copy_sync(e, L.hist[e->parity[i]], p, HIST_ELEMS * 2, hipMemcpyHostToDevice); if (r) return r;
+      p += HIST_ELEMS * 2;
+      r = copy_sync(e, L.state[e->parity[i]], p, STATE_ELEMS * 4, hipMemcpyHostToDevice); if (r) return r;
+      p += STATE_ELEMS * 4;
+    }
+  }
+  if (p != end) return SL_ERR_FORMAT;
+  if (new_pos >= 0) e->pos = new_pos;
+  return push_state(e);
+}
+
+int sl_read_layer_cache(sl_engine* e, int layer, void* a, void* b) {
+  int r = guard(e); if (r) return r;
+  if (layer < 0 || layer >= e->n_layers) return SL_ERR_ARG;
+  LayerDev& L = e->layers[layer];
+  if (L.is_linear) {
+    if (a) { r = copy_sync(e, a, L.hist[e->parity[layer]], HIST_ELEMS * 2, hipMemcpyDeviceToHost); if (r) return r; }
+    if (b) { r = copy_sync(e, b, L.state[e->parity[layer]], STATE_ELEMS * 4, hipMemcpyDeviceToHost); if (r) return r; }
+  } else {
+    const size_t rb = (size_t)e->pos * SL_ATT_D * 2;
+    for (int h = 0; h < SL_ATT_KV && rb; ++h) {
+      if (a) { r = copy_sync(e, (uint8_t*)a + h * rb, L.kcache + (size_t)h * e->max_seq * SL_ATT_D, rb, hipMemcpyDeviceToHost); if (r) return r; }
+      if (b) { r = copy_sync(e, (uint8_t*)b + h * rb, L.vcache + (size_t)h * e->max_seq * SL_ATT_D, rb, hipMemcpyDeviceToHost); if (r) return r; }
+    }
+  }
+  return SL_OK;
+}
+int sl_load_layer_cache(sl_engine* e, int layer, const void* a, const void* b, int len) {
+  int r = guard(e); if (r) return r;
+  if (layer < 0 || layer >= e->n_layers) return SL_ERR_ARG;
+  LayerDev& L = e->layers[layer];
+  if (L.is_linear) {
+    if (a) { r = copy_sync(e, L.hist[e->parity[layer]], a, HIST_ELEMS * 2, hipMemcpyHostToDevice); if (r) return r; }
+    if (b) { r = copy_sync(e, L.state[e->parity[layer]], b, STATE_ELEMS * 4, hipMemcpyHostToDevice); if (r) return r; }
+    return SL_OK;
+  }
+  if (len < 0 || len > e->max_seq) return SL_ERR_ARG;
+  const size_t rb = (size_t)len * SL_ATT_D * 2;
+  for (int h = 0; h < SL_ATT_KV && rb; ++h) {
+    if (a) { r = copy_sync(e, L.kcache + (size_t)h * e->max_seq * SL_ATT_D, (const uint8_t*)a + h * rb, rb, hipMemcpyHostToDevice); if (r) return r; }
+    if (b) { r = copy_sync(e, L.vcache + (size_t)h * e->max_seq * SL_ATT_D, (const uint8_t*)b + h * rb, rb, hipMemcpyHostToDevice); if (r) return r; }
+  }
+  e->pos = len;
+  return push_state(e);
+}
+
+int sl_read_route(sl_engine* e, int layer, int m, int32_t* inds, uint16_t* scores) {
+  int r = guard(e); if (r) return r;
+  if (layer < 0 || layer >= e->n_layers || m < 1 || m > e->max_m) return SL_ERR_ARG;
+  if (inds) { r = copy_sync(e, inds, e->layers[layer].route_inds, (size_t)m * 32, hipMemcpyDeviceToHost); if (r) return r; }
+  if (scores) { r = copy_sync(e, scores, e->layers[layer].route_scores, (size_t)m * 16, hipMemcpyDeviceToHost); if (r) return r; }
+  return SL_OK;
+}
+
+// ---- per-block entry points -----------------------------------------------------------------------
+int sl_moe_block_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!x || !out || layer < 0 || layer >= e->n_layers || m < 1 || m > e->max_m) return SL_ERR_ARG;
+  r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
+  SL_TRY(e, hipEventRecord(e->ev0, e->stream));
+  HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
+  launch_moe(e, e->layers[layer], m, ha);
+  SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+  r = read_back(e, out, e->moe_out, (size_t)m * H * 2, "moeBlockRows"); if (r) return r;
+  time_end(e);
+  return SL_OK;
+}
+int sl_gdn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!x || !out || layer < 0 || layer >= e->n_layers || m < 1 || m > e->max_m || !e->layers[layer].is_linear) return SL_ERR_ARG;
+  r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
+  SL_TRY(e, hipEventRecord(e->ev0, e->stream));
+  HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
+  launch_gdn_mixer(e, e->layers[layer], layer, m, ha);
+  SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+  r = read_back(e, out, e->mix, (size_t)m * H * 2, "gdnLayerRows"); if (r) return r;
+  time_end(e);
+  e->parity[layer] ^= 1;
+  return push_state(e);
+}
+int sl_attn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!x || !out || layer < 0 || layer >= e->n_layers || e->layers[layer].is_linear) return SL_ERR_ARG;
+  r = check_rows(e, m); if (r) return r;
+  r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
+  SL_TRY(e, hipEventRecord(e->ev0, e->stream));
+  HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
+  launch_attn_mixer(e, e->layers[layer], m, ha);
+  SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+  r = read_back(e, out, e->mix, (size_t)m * H * 2, "attnLayerRows"); if (r) return r;
+  time_end(e);
+  e->pos += m;
+  return push_state(e);
+}
+
+int sl_greedy_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_new, int chain_k, int32_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!prompt || n_prompt < 1 || n_new < 0 || (n_new > 0 && !out) || !e->has_head) return SL_ERR_ARG;
+  if (chain_k < 1) chain_k = 1;
+  if (chain_k > MAX_CHAIN) chain_k = MAX_CHAIN;
+  std::vector<uint16_t> nr((size_t)e->max_m * H);
+  int done = 0, last_m = 0;
+  while (done < n_prompt) {
+    last_m = n_prompt - done < e->max_m ? n_prompt - done : e->max_m;
+    r = sl_forward_tokens(e, prompt + done, last_m, nr.data()); if (r) return r;
+    done += last_m;
+  }
+  if (n_new == 0) return SL_OK;
+  r = sl_head_argmax(e, nr.data() + (size_t)(last_m - 1) * H, 1, &out[0]); if (r) return r;
+  int have = 1;
+  while (have < n_new) {
+    const int k = n_new - have < chain_k ? n_new - have : chain_k;
+    r = sl_chained_step_argmax(e, out[have - 1], k, out + have); if (r) return r;
+    have += k;
+  }
+  return SL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,760 @@
+// Decode kernels for the Seedless engine on gfx950 (wave64).  Row m of an M-row forward is
+// blockIdx.y (or .z); every per-row computation is independent of M, which is what makes an
+// M-row verify step equal M single-row steps bit for bit.
+//
+// Reduction order shared by all kernels (and by the CPU checker used in the tests):
+//  * 4-bit dot, K = 2048*NBLK: lane l owns words 4l..4l+3 of each 2048-element block (one 16-byte
+//    load), word term t = fmaf(s, dq, b*sx), lane partial = sum over blocks of (t0+t1)+(t2+t3),
+//    then a 64-lane butterfly.  K = 512: the same with 16 lanes per row, four rows per wave.
+//  * dense fp16 dot / sum of squares over 2048: lane l owns elements 32l..32l+31, fmaf chain, butterfly.
+//  * sum of squares over 128 or 256: 64 leaves of 2 or 4 contiguous elements, balanced tree.
+#pragma once
+#include "sl_device.cuh"
+#include "../../include/seedless_hip.h"
+
+namespace sl {
+
+constexpr int H = SL_H;
+constexpr float EPS = 1e-6f;
+constexpr int PROJ_STRIDE = SL_GDN_IN_N;     // row stride of the projection scratch (>= 9216)
+constexpr int SDPA_TILE = 64;
+constexpr int KT_STRIDE = 264;               // halves per staged key row (256 + 8 pad)
+
+// -------------------------------------------------------------------------------------------------
+// Hidden-row prologue: x = half(h + r) (optional), optional rmsnorm with weight w.
+// Reference: resid_add + rmsnorm fused as gdn_resid_postnorm_rows, SeedlessFusedVerify.swift:943-1001.
+// -------------------------------------------------------------------------------------------------
+SL_DEV void load32(const uint16_t* p, float* x) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) unpack8(ld16(p + 8 * j), x + 8 * j);
+}
+SL_DEV void store32(uint16_t* p, const float* x) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) st16(p + 8 * j, pack8(x + 8 * j));
+}
+SL_DEV float inv_rms_2048(const float* x) {
+  float ss = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) ss = fmaf(x[i], x[i], ss);
+  ss = tree_sum<64>(ss);
+  return 1.0f / sqrtf(ss / 2048.0f + EPS);
+}
+struct HiddenArgs {
+  const uint16_t* h_in;    // [M, 2048]
+  const uint16_t* r_in;    // [M, 2048] residual to add first, or null
+  const uint16_t* lnw;     // [2048] norm weight, or null for "x is used as given"
+  uint16_t* h_out;         // [M, 2048] receives half(h + r) (written once per row), or null
+  uint16_t* xn_out;        // [M, 2048] receives the normed row (written once per row), or null
+};
+// Every wave of the grid calls this; `writer` selects the single wave that stores the outputs.
+SL_DEV void hidden_prologue(const HiddenArgs& a, int m, int lane, bool writer, float* x) {
+  load32(a.h_in + (size_t)m * H + 32 * lane, x);
+  if (a.r_in) {
+    float r[32];
+    load32(a.r_in + (size_t)m * H + 32 * lane, r);
+#pragma unroll
+    for (int i = 0; i < 32; ++i) x[i] = f16r(x[i] + r[i]);
+  }
+  if (writer && a.h_out) store32(a.h_out + (size_t)m * H + 32 * lane, x);
+  if (a.lnw) {
+    const float inv = inv_rms_2048(x);
+    float w[32];
+    load32(a.lnw + 32 * lane, w);
+#pragma unroll
+    for (int i = 0; i < 32; ++i) x[i] = f16r(w[i] * f16r(x[i] * inv));
+  }
+  if (writer && a.xn_out) store32(a.xn_out + (size_t)m * H + 32 * lane, x);
+}
+
+// -------------------------------------------------------------------------------------------------
+// 4-bit dots.  W: packed words [rows, K/8]; SB: {scale, bias} half pairs [rows, K/64].
+// Reference arithmetic: qmm4, SeedlessMetalForward.swift:238-310.
+// -------------------------------------------------------------------------------------------------
+template <int NBLK, int R>
+SL_DEV void qdot_rows(const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB, const size_t* rows, int lane,
+                      const float* x, const float* sx, float* out) {
+  constexpr int WPR = NBLK * 256, GPR = NBLK * 32;
+  uint4 wv[R][NBLK];
+  uint32_t sb[R][NBLK];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b) {
+      wv[r][b] = ld16(W + rows[r] * WPR + b * 256 + 4 * lane);
+      sb[r][b] = SB[rows[r] * GPR + b * 32 + (lane >> 1)];
+    }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float acc = quad_term(wv[r][0], sb[r][0], x, sx);
+#pragma unroll
+    for (int b = 1; b < NBLK; ++b) acc = acc + quad_term(wv[r][b], sb[r][b], x + 32 * b, sx + 4 * b);
+    out[r] = tree_sum<64>(acc);
+  }
+}
+// K = 512: 16 lanes per row; li = lane & 15 owns words 4li..4li+3.  Result valid on all 16 lanes.
+SL_DEV float qdot512(const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB, size_t row, int li, const float* x,
+                     const float* sx) {
+  const uint4 wv = ld16(W + row * 64 + 4 * li);
+  const uint32_t sb = SB[row * 8 + (li >> 1)];
+  return tree_sum<16>(quad_term(wv, sb, x, sx));
+}
+// Dense fp16 row against the lane's 32 activations (router gate, shared-expert gate).
+SL_DEV float dense_dot(const uint16_t* __restrict__ wrow, int lane, const float* x) {
+  float w[32];
+  load32(wrow + 32 * lane, w);
+  float acc = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) acc = fmaf(x[i], w[i], acc);
+  return tree_sum<64>(acc);
+}
+
+// -------------------------------------------------------------------------------------------------
+// embed_rows_q4 (SeedlessFusedVerify.swift:556-570): h = half(half(s*nib) + b).
+// -------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_embed(const int32_t* __restrict__ tokens, const uint32_t* __restrict__ W,
+                                               const uint32_t* __restrict__ SB, uint16_t* __restrict__ h) {
+  const int m = blockIdx.y, j = blockIdx.x * 256 + threadIdx.x;
+  const size_t tok = (size_t)tokens[m];
+  const uint32_t w = W[tok * 256 + (j >> 3)];
+  const uint32_t sb = SB[tok * 32 + (j >> 6)];
+  const float nib = (float)((w >> (4 * (j & 7))) & 15u);
+  h[(size_t)m * H + j] = f2h(f16r(lo_h(sb) * nib) + hi_h(sb));
+}
+
+// -------------------------------------------------------------------------------------------------
+// Projection with the hidden prologue: y[m, n] = half(dot(x_m, W[n])), K = 2048.
+// Used for the GDN in-proj (qkv|z|b|a concatenated, SeedlessFusedVerify.swift:690) and the
+// attention q|k|v projection.  4 waves x R rows per workgroup.
+// -------------------------------------------------------------------------------------------------
+template <int R>
+__global__ __launch_bounds__(256) void k_qmv_hidden(HiddenArgs ha, const uint32_t* __restrict__ W,
+                                                    const uint32_t* __restrict__ SB, int N, uint16_t* __restrict__ y,
+                                                    int y_stride) {
+  const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float x[32], sx[4];
+  hidden_prologue(ha, m, lane, blockIdx.x == 0 && wave == 0, x);
+  word_sums(x, sx);
+  const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * R;
+  if (row0 >= (size_t)N) return;
+  size_t rows[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) rows[r] = row0 + r;
+  float out[R];
+  qdot_rows<1, R>(W, SB, rows, lane, x, sx, out);
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) y[(size_t)m * y_stride + row0 + r] = f2h(out[r]);
+  }
+}
+
+// Plain projection from an fp16 activation buffer, K = 2048*NBLK (attention o_proj: NBLK = 2).
+template <int NBLK, int R>
+__global__ __launch_bounds__(256) void k_qmv_plain(const uint16_t* __restrict__ xin, int x_stride,
+                                                   const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB,
+                                                   int N, uint16_t* __restrict__ y, int y_stride) {
+  const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float x[32 * NBLK], sx[4 * NBLK];
+#pragma unroll
+  for (int b = 0; b < NBLK; ++b) {
+    load32(xin + (size_t)m * x_stride + b * 2048 + 32 * lane, x + 32 * b);
+    word_sums(x + 32 * b, sx + 4 * b);
+  }
+  const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * R;
+  if (row0 >= (size_t)N) return;
+  size_t rows[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) rows[r] = row0 + r;
+  float out[R];
+  qdot_rows<NBLK, R>(W, SB, rows, lane, x, sx, out);
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) y[(size_t)m * y_stride + row0 + r] = f2h(out[r]);
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Gated-DeltaNet core: causal conv(4)+SiLU+history shift, q/k head norms and scales, beta and
+// decay, and the gated delta rule with the fp32 state in registers, M rows in sequence.
+// References: conv_shift_fused_rows SeedlessFusedVerify.swift:634-663; gdn_prep_rows :839-938;
+// gated_delta_step GatedDelta.swift:63-124.
+// Grid: 32 value heads x 8 slices of 16 state rows; 4 waves, each wave 2 x 2 rows, a row = 32
+// lanes x 4 contiguous dk.  State layout [hv][dv][dk] fp32, ping-pong selected by st[1].
+// -------------------------------------------------------------------------------------------------
+struct GdnArgs {
+  const uint16_t* proj;      // [M, PROJ_STRIDE]: qkv 8192 | z 4096 | b 32 | a 32
+  const float* conv_w;       // [8192, 4]
+  const float* a_log;        // [32]
+  const float* dt_bias;      // [32]
+  uint16_t* hist[2];         // [3, 8192] each
+  float* state[2];           // [32, 128, 128] each
+  const int32_t* st;         // st[1] = parity: read side
+  uint16_t* ycore;           // [M, 4096]
+  int M;
+};
+SL_DEV float conv_tap(const GdnArgs& a, const uint16_t* hin, int row, int ch) {
+  // row of the concatenation [hist(3) | qkv(M)]
+  return (row < 3) ? h2f(hin[row * SL_CONV_DIM + ch]) : h2f(a.proj[(size_t)(row - 3) * PROJ_STRIDE + ch]);
+}
+SL_DEV float conv_silu(const GdnArgs& a, const uint16_t* hin, int t, int ch) {
+  float acc = 0.0f;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) acc = fmaf(conv_tap(a, hin, t + k, ch), a.conv_w[ch * 4 + k], acc);
+  return f16r(acc * sigmoid32(acc));
+}
+__global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
+  __shared__ float s_q[128], s_k[128], s_v[16], s_gb[2];
+  const int hv = blockIdx.x >> 3, dvb = blockIdx.x & 7, hk = hv >> 1;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+  const int par = a.st[1];
+  const uint16_t* hin = a.hist[par];
+  uint16_t* hout = a.hist[par ^ 1];
+  const float* sin_ = a.state[par];
+  float* sout = a.state[par ^ 1];
+
+  float s[2][4];
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int dv = dvb * 16 + wave * 4 + it * 2 + half;
+    const float4 v = *reinterpret_cast<const float4*>(sin_ + ((size_t)hv * 128 + dv) * 128 + 4 * l32);
+    s[it][0] = v.x; s[it][1] = v.y; s[it][2] = v.z; s[it][3] = v.w;
+  }
+  const int qk_ch = (tid < 128) ? (hk * 128 + tid) : (2048 + hk * 128 + (tid - 128));
+  const int v_ch = 4096 + hv * 128 + dvb * 16 + (tid & 15);
+
+  for (int t = 0; t < a.M; ++t) {
+    const float c = conv_silu(a, hin, t, qk_ch);
+    if (tid < 128) s_q[tid] = c; else s_k[tid - 128] = c;
+    if (tid < 16) s_v[tid] = conv_silu(a, hin, t, v_ch);
+    __syncthreads();
+    if (wave < 2) {
+      // weightless rmsnorm over 128, then the key/query scale, both rounded to half
+      float* buf = wave ? s_k : s_q;
+      const float x0 = buf[2 * lane], x1 = buf[2 * lane + 1];
+      float ss = fmaf(x1, x1, fmaf(x0, x0, 0.0f));
+      ss = tree_sum<64>(ss);
+      const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
+      const float sc = wave ? f16r(0.08838834764831845f) : f16r(0.0078125f);
+      const float y0 = f16r(sc * f16r(x0 * inv)), y1 = f16r(sc * f16r(x1 * inv));
+      buf[2 * lane] = y0; buf[2 * lane + 1] = y1;
+    } else if (tid == 128) {
+      const float bP = h2f(a.proj[(size_t)t * PROJ_STRIDE + 12288 + hv]);
+      const float aP = h2f(a.proj[(size_t)t * PROJ_STRIDE + 12320 + hv]);
+      s_gb[0] = exp_c(-(exp_c(a.a_log[hv]) * softplus_c(aP + a.dt_bias[hv])));
+      s_gb[1] = sigmoid16(bP);
+    }
+    __syncthreads();
+    const float g = s_gb[0], beta = s_gb[1];
+    const float4 k4 = *reinterpret_cast<const float4*>(&s_k[4 * l32]);
+    const float4 q4 = *reinterpret_cast<const float4*>(&s_q[4 * l32]);
+    const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, qq[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int dvl = wave * 4 + it * 2 + half;
+      float acc = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { s[it][i] = s[it][i] * g; acc = fmaf(s[it][i], kk[i], acc); }
+      const float kv = tree_sum<32>(acc);
+      const float delta = (s_v[dvl] - kv) * beta;
+      acc = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { s[it][i] = fmaf(kk[i], delta, s[it][i]); acc = fmaf(s[it][i], qq[i], acc); }
+      const float y = tree_sum<32>(acc);
+      if (l32 == 0) a.ycore[(size_t)t * 4096 + hv * 128 + dvb * 16 + dvl] = f2h(y);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int dv = dvb * 16 + wave * 4 + it * 2 + half;
+    *reinterpret_cast<float4*>(sout + ((size_t)hv * 128 + dv) * 128 + 4 * l32) = make_float4(s[it][0], s[it][1], s[it][2], s[it][3]);
+  }
+  // history shift: rows M..M+2 of [hist | qkv]; each channel written by exactly one workgroup
+  if ((hv & 1) == 0 && dvb == 0) {
+#pragma unroll
+    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + qk_ch] = f2h(conv_tap(a, hin, a.M + j, qk_ch));
+  }
+  if (tid < 16) {
+#pragma unroll
+    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + v_ch] = f2h(conv_tap(a, hin, a.M + j, v_ch));
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// GDN out-proj with the gated rmsnorm as prologue: x = half(silu(z) * (w * half(y*inv))) per value
+// head, then the K = 4096 4-bit dot.  Reference: gdn_norm_gate_rows SeedlessFusedVerify.swift:768-812.
+// -------------------------------------------------------------------------------------------------
+template <int R>
+__global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict__ ycore, const uint16_t* __restrict__ proj,
+                                                     const uint16_t* __restrict__ norm_w, const uint32_t* __restrict__ W,
+                                                     const uint32_t* __restrict__ SB, int N, uint16_t* __restrict__ y) {
+  const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float x[64], sx[8];
+  float nw[32];
+  load32(norm_w + 32 * (lane & 3), nw);
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    float* xb = x + 32 * b;
+    load32(ycore + (size_t)m * 4096 + b * 2048 + 32 * lane, xb);
+    float leaf[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) leaf[j] = fmaf(xb[2 * j + 1], xb[2 * j + 1], fmaf(xb[2 * j], xb[2 * j], 0.0f));
+#pragma unroll
+    for (int st = 1; st < 16; st <<= 1)
+#pragma unroll
+      for (int j = 0; j < 16; j += 2 * st) leaf[j] = leaf[j] + leaf[j + st];
+    const float ss = tree_sum<4>(leaf[0]);
+    const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
+    float z[32];
+    load32(proj + (size_t)m * PROJ_STRIDE + 8192 + b * 2048 + 32 * lane, z);
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      const float nrm = f16r(nw[i] * f16r(xb[i] * inv));
+      xb[i] = f16r((z[i] * sigmoid32(z[i])) * nrm);
+    }
+    word_sums(xb, sx + 4 * b);
+  }
+  const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * R;
+  if (row0 >= (size_t)N) return;
+  size_t rows[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) rows[r] = row0 + r;
+  float out[R];
+  qdot_rows<2, R>(W, SB, rows, lane, x, sx, out);
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) y[(size_t)m * H + row0 + r] = f2h(out[r]);
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// MoE stage A: residual + post-attention norm, then in one launch the shared expert's gate/up
+// with SwiGLU (64 workgroups), the fp16 router gate rows and the shared-expert gate row.
+// References: MoEBlock.swift:69-97; shared expert SeedlessFusedVerify.swift:1859-1871.
+// -------------------------------------------------------------------------------------------------
+struct MoeAArgs {
+  HiddenArgs ha;
+  const uint32_t *shg_w, *shg_sb, *shu_w, *shu_sb;   // shared gate_proj / up_proj [512, 2048]
+  const uint16_t* router_w;                          // [E, 2048]
+  const uint16_t* sgate_w;                           // [2048]
+  int E;
+  uint16_t* sh_act;                                  // [M, 512]
+  uint16_t* rlogits;                                 // [M, 256]
+  uint16_t* sgate;                                   // [M]
+};
+constexpr int MOE_A_SHARED_BLOCKS = 64;
+__global__ __launch_bounds__(256) void k_moe_a(MoeAArgs a) {
+  const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float x[32], sx[4];
+  hidden_prologue(a.ha, m, lane, blockIdx.x == 0 && wave == 0, x);
+  if (blockIdx.x < MOE_A_SHARED_BLOCKS) {
+    word_sums(x, sx);
+    const size_t i0 = ((size_t)blockIdx.x * 4 + wave) * 2;
+    const size_t rows[2] = {i0, i0 + 1};
+    float g[2], u[2];
+    qdot_rows<1, 2>(a.shg_w, a.shg_sb, rows, lane, x, sx, g);
+    qdot_rows<1, 2>(a.shu_w, a.shu_sb, rows, lane, x, sx, u);
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < 2; ++r) a.sh_act[(size_t)m * 512 + i0 + r] = f2h(swiglu16(f16r(g[r]), f16r(u[r])));
+    }
+  } else {
+    const int row0 = ((blockIdx.x - MOE_A_SHARED_BLOCKS) * 4 + wave) * 4;
+    for (int r = 0; r < 4; ++r) {
+      const int row = row0 + r;
+      if (row < a.E) {
+        const float v = dense_dot(a.router_w + (size_t)row * H, lane, x);
+        if (lane == 0) a.rlogits[(size_t)m * 256 + row] = f2h(v);
+      } else if (row == a.E) {
+        const float v = dense_dot(a.sgate_w, lane, x);
+        if (lane == 0) a.sgate[m] = f2h(v);
+      }
+    }
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Router: softmax over the half logits, gates rounded to half, 8 x arg-max of the raw logits
+// (ties to the lower index), half renormalisation.  One wave; lane l owns experts 4l..4l+3.
+// Reference: route_top8_rows SeedlessFusedVerify.swift:191-213.
+// -------------------------------------------------------------------------------------------------
+SL_DEV void route_wave(const uint16_t* __restrict__ logits, int E, int lane, int* inds, float* scores) {
+  const float NEG = -__int_as_float(0x7f800000);
+  float lg[4], ex[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) lg[i] = (4 * lane + i < E) ? h2f(logits[4 * lane + i]) : NEG;
+  const float mx = tree_max<64>(fmaxf(fmaxf(lg[0], lg[1]), fmaxf(lg[2], lg[3])));
+#pragma unroll
+  for (int i = 0; i < 4; ++i) ex[i] = (4 * lane + i < E) ? exp_c(lg[i] - mx) : 0.0f;
+  const float Z = tree_sum<64>(((ex[0] + ex[1]) + ex[2]) + ex[3]);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    float bv = lg[0]; int bi = 4 * lane;
+#pragma unroll
+    for (int i = 1; i < 4; ++i) if (lg[i] > bv) { bv = lg[i]; bi = 4 * lane + i; }
+#pragma unroll
+    for (int msk = 1; msk < 64; msk <<= 1) {
+      const float ov = __shfl_xor(bv, msk, 64);
+      const int oi = __shfl_xor(bi, msk, 64);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    const int sub = bi & 3;
+    const float mine = (sub == 0) ? ex[0] : (sub == 1) ? ex[1] : (sub == 2) ? ex[2] : ex[3];
+    const float e = __shfl(mine, bi >> 2, 64);
+    inds[k] = bi;
+    scores[k] = f16r(e / Z);
+    if ((bi >> 2) == lane) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) if (i == sub) lg[i] = NEG;
+    }
+  }
+  float ss = 0.0f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) ss = f16r(ss + scores[k]);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) scores[k] = f16r(scores[k] / ss);
+}
+
+// MoE stage B: routing + the 8 routed experts' gate/up with SwiGLU.
+// Reference: gqmm4_swiglu_rows SeedlessMetalForward.swift:1419-1460.
+struct MoeBArgs {
+  const uint16_t* xn;          // [M, 2048] post-normed rows
+  const uint16_t* rlogits;     // [M, 256]
+  int E;
+  const uint32_t *g_w, *g_sb, *u_w, *u_sb;   // [E*512, 2048]
+  uint16_t* act;               // [M, 8, 512]
+  int32_t* inds;               // [M, 8]
+  uint16_t* scores;            // [M, 8]
+};
+__global__ __launch_bounds__(256) void k_moe_b(MoeBArgs a) {
+  __shared__ int s_inds[8];
+  const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (wave == 0) {
+    int inds[8]; float sc[8];
+    route_wave(a.rlogits + (size_t)m * 256, a.E, lane, inds, sc);
+    if (lane == 0) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        s_inds[k] = inds[k];
+        if (blockIdx.x == 0) { a.inds[m * 8 + k] = inds[k]; a.scores[m * 8 + k] = f2h(sc[k]); }
+      }
+    }
+  }
+  float x[32], sx[4];
+  load32(a.xn + (size_t)m * H + 32 * lane, x);
+  word_sums(x, sx);
+  __syncthreads();
+  const int p0 = (blockIdx.x * 4 + wave) * 2;          // pair index in [0, 8*512)
+  const int k = p0 >> 9, i0 = p0 & 511;
+  const size_t base = (size_t)s_inds[k] * 512 + i0;
+  const size_t rows[2] = {base, base + 1};
+  float g[2], u[2];
+  qdot_rows<1, 2>(a.g_w, a.g_sb, rows, lane, x, sx, g);
+  qdot_rows<1, 2>(a.u_w, a.u_sb, rows, lane, x, sx, u);
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) a.act[((size_t)m * 8 + k) * 512 + i0 + r] = f2h(swiglu16(f16r(g[r]), f16r(u[r])));
+  }
+}
+
+// MoE stage C: routed down-proj, half-precision combine in routing order, shared down-proj and the
+// sigmoid-gated shared add.  References: gqmm4_rows SeedlessMetalForward.swift:4017; combine_rows
+// SeedlessFusedVerify.swift:462-470; shared_gate_combine_rows :1051-1109.
+struct MoeCArgs {
+  const uint16_t* act;         // [M, 8, 512]
+  const uint16_t* sh_act;      // [M, 512]
+  const int32_t* inds;         // [M, 8]
+  const uint16_t* scores;      // [M, 8]
+  const uint16_t* sgate;       // [M]
+  const uint32_t *d_w, *d_sb;  // [E*2048, 512]
+  const uint32_t *shd_w, *shd_sb;   // [2048, 512]
+  uint16_t* out;               // [M, 2048]
+};
+__global__ __launch_bounds__(128) void k_moe_c(MoeCArgs a) {
+  const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane >> 4, li = lane & 15;
+  const int n = (blockIdx.x * 2 + wave) * 4 + sub;
+  float acc = 0.0f;
+  float x[32], sx[4];
+#pragma unroll 1
+  for (int k = 0; k < 8; ++k) {
+    load32(a.act + ((size_t)m * 8 + k) * 512 + 32 * li, x);
+    word_sums(x, sx);
+    const size_t row = (size_t)a.inds[m * 8 + k] * 2048 + n;
+    const float d = f16r(qdot512(a.d_w, a.d_sb, row, li, x, sx));
+    acc = f16r(acc + f16r(d * h2f(a.scores[m * 8 + k])));
+  }
+  load32(a.sh_act + (size_t)m * 512 + 32 * li, x);
+  word_sums(x, sx);
+  const float sy = f16r(qdot512(a.shd_w, a.shd_sb, (size_t)n, li, x, sx));
+  const float s = sigmoid16(h2f(a.sgate[m]));
+  if (li == 0) a.out[(size_t)m * H + n] = f2h(f16r(acc + f16r(s * sy)));
+}
+
+// -------------------------------------------------------------------------------------------------
+// Attention prep: per-head rmsnorm with weight, partial NeoX RoPE on the first 64 dims from a
+// (cos, sin) table, K and V appended to the cache.  Blocks 0..15: query heads; 16..17: kv heads.
+// References: attn_q_prep_rows / attn_k_prep_rows SeedlessFusedVerify.swift:1183-1330; write_kv_rows :487.
+// -------------------------------------------------------------------------------------------------
+struct AttnPrepArgs {
+  const uint16_t* proj;        // [M, PROJ_STRIDE]: q(+gate) 16x512 | k 2x256 | v 2x256
+  const uint16_t *q_norm, *k_norm;
+  const float *rope_cos, *rope_sin;   // [maxSeq, 32]
+  const int32_t* st;           // st[0] = position of row 0
+  uint16_t* qrot;              // [M, 16, 256]
+  uint16_t *kcache, *vcache;   // [2, maxSeq, 256]
+  int maxSeq;
+};
+__global__ __launch_bounds__(64) void k_attn_prep(AttnPrepArgs a) {
+  __shared__ float s_n[256];
+  const int m = blockIdx.y, hb = blockIdx.x, lane = threadIdx.x;
+  const int pos = a.st[0] + m;
+  const bool isq = hb < 16;
+  const uint16_t* src = a.proj + (size_t)m * PROJ_STRIDE + (isq ? hb * 512 : 8192 + (hb - 16) * 256);
+  const uint16_t* nw = isq ? a.q_norm : a.k_norm;
+  const uint2 raw = *reinterpret_cast<const uint2*>(src + 4 * lane);
+  const uint2 wraw = *reinterpret_cast<const uint2*>(nw + 4 * lane);
+  const float xv[4] = {lo_h(raw.x), hi_h(raw.x), lo_h(raw.y), hi_h(raw.y)};
+  const float wv[4] = {lo_h(wraw.x), hi_h(wraw.x), lo_h(wraw.y), hi_h(wraw.y)};
+  float ss = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) ss = fmaf(xv[i], xv[i], ss);
+  ss = tree_sum<64>(ss);
+  const float inv = 1.0f / sqrtf(ss / 256.0f + EPS);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) s_n[4 * lane + i] = f16r(wv[i] * f16r(xv[i] * inv));
+  __syncthreads();
+  float o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = 4 * lane + i;
+    if (d >= SL_ROPE_DIM) { o[i] = s_n[d]; continue; }
+    const int ii = d & 31;
+    const float c = a.rope_cos[(size_t)pos * 32 + ii], s = a.rope_sin[(size_t)pos * 32 + ii];
+    const float x0 = s_n[ii], x1 = s_n[ii + 32];
+    o[i] = (d < 32) ? f16r(fmaf(-x1, s, x0 * c)) : f16r(fmaf(x1, c, x0 * s));
+  }
+  const uint2 packed = make_uint2(pack2(o[0], o[1]), pack2(o[2], o[3]));
+  if (isq) {
+    *reinterpret_cast<uint2*>(a.qrot + ((size_t)m * 16 + hb) * 256 + 4 * lane) = packed;
+  } else {
+    const int h = hb - 16;
+    const size_t off = ((size_t)h * a.maxSeq + pos) * 256 + 4 * lane;
+    *reinterpret_cast<uint2*>(a.kcache + off) = packed;
+    *reinterpret_cast<uint2*>(a.vcache + off) =
+        *reinterpret_cast<const uint2*>(a.proj + (size_t)m * PROJ_STRIDE + 8192 + 512 + h * 256 + 4 * lane);
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Decode attention, tile pass: one wave per (key tile of 64, kv head, row).  The tile's keys are
+// staged in LDS; lane j scores key j against the 8 query heads of the group (a balanced tree over
+// 64 leaves of 4 dims), then p = exp(s - tile max), l = butterfly sum of p, o = fmaf chain over
+// the tile's keys with V rows read coalesced.  Reference semantics: sdpa_rows
+// SeedlessMetalForward.swift:4922-4989 (q scaled by 1/16, fp32 softmax).
+// -------------------------------------------------------------------------------------------------
+struct SdpaArgs {
+  const uint16_t* qrot;        // [M, 16, 256]
+  const uint16_t *kcache, *vcache;
+  const int32_t* st;
+  int maxSeq, maxTiles;
+  float *pm, *pl;              // [M, 16, maxTiles]
+  float* po;                   // [M, 16, maxTiles, 256]
+};
+__global__ __launch_bounds__(64) void k_sdpa_tile(SdpaArgs a) {
+  __shared__ __align__(16) uint16_t s_k[SDPA_TILE * KT_STRIDE];
+  __shared__ __align__(16) float s_q[8 * 256];
+  const int tile = blockIdx.x, kvh = blockIdx.y, m = blockIdx.z, lane = threadIdx.x;
+  const int N = a.st[0] + m + 1;
+  const int j0 = tile * SDPA_TILE;
+  if (j0 >= N) return;
+  const int nk = min(SDPA_TILE, N - j0);
+  const uint16_t* kbase = a.kcache + ((size_t)kvh * a.maxSeq + j0) * 256;
+  const uint16_t* vbase = a.vcache + ((size_t)kvh * a.maxSeq + j0) * 256;
+  // stage keys (rows >= nk are never read) and the group's 8 scaled queries
+  for (int it = 0; it < 32; ++it) {
+    const int row = it * 2 + (lane >> 5), c8 = (lane & 31) * 8;
+    if (row < nk) st16(&s_k[row * KT_STRIDE + c8], ld16(kbase + (size_t)row * 256 + c8));
+  }
+  for (int it = 0; it < 4; ++it) {
+    const int idx = (it * 64 + lane) * 8;            // 0..2047 step 8
+    float f[8];
+    unpack8(ld16(a.qrot + ((size_t)m * 16 + kvh * 8) * 256 + idx), f);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s_q[idx + i] = 0.0625f * f[i];
+  }
+  __syncthreads();
+  const float NEG = -__int_as_float(0x7f800000);
+  float sc[8];
+  {
+    float stk[8][7];
+    const uint16_t* kr = &s_k[(lane < nk ? lane : 0) * KT_STRIDE];
+#pragma unroll
+    for (int leaf = 0; leaf < 64; ++leaf) {
+      const uint2 kraw = *reinterpret_cast<const uint2*>(kr + 4 * leaf);
+      const float kf[4] = {lo_h(kraw.x), hi_h(kraw.x), lo_h(kraw.y), hi_h(kraw.y)};
+#pragma unroll
+      for (int h = 0; h < 8; ++h) {
+        const float4 q4 = *reinterpret_cast<const float4*>(&s_q[h * 256 + 4 * leaf]);
+        float node = fmaf(q4.x, kf[0], 0.0f);
+        node = fmaf(q4.y, kf[1], node);
+        node = fmaf(q4.z, kf[2], node);
+        node = fmaf(q4.w, kf[3], node);
+        int c = leaf, lvl = 0;
+        while (c & 1) { node = stk[h][lvl] + node; c >>= 1; ++lvl; }
+        stk[h][lvl] = node;
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < 8; ++h) sc[h] = (lane < nk) ? stk[h][6] : NEG;
+  }
+  float p[8], o[8][4];
+#pragma unroll
+  for (int h = 0; h < 8; ++h) {
+    const float mx = tree_max<64>(sc[h]);
+    p[h] = (lane < nk) ? exp_c(sc[h] - mx) : 0.0f;
+    const float l = tree_sum<64>(p[h]);
+    if (lane == 0) {
+      const size_t pi = ((size_t)m * 16 + kvh * 8 + h) * a.maxTiles + tile;
+      a.pm[pi] = mx; a.pl[pi] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[h][i] = 0.0f;
+  }
+  for (int j = 0; j < nk; ++j) {
+    const uint2 vraw = *reinterpret_cast<const uint2*>(vbase + (size_t)j * 256 + 4 * lane);
+    const float vf[4] = {lo_h(vraw.x), hi_h(vraw.x), lo_h(vraw.y), hi_h(vraw.y)};
+#pragma unroll
+    for (int h = 0; h < 8; ++h) {
+      const float pj = __shfl(p[h], j, 64);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[h][i] = fmaf(pj, vf[i], o[h][i]);
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < 8; ++h) {
+    const size_t pi = ((size_t)m * 16 + kvh * 8 + h) * a.maxTiles + tile;
+    *reinterpret_cast<float4*>(a.po + pi * 256 + 4 * lane) = make_float4(o[h][0], o[h][1], o[h][2], o[h][3]);
+  }
+}
+
+// Merge pass + output gate: tiles combined in order with the global max, out = half(O/L),
+// gated = out * sigmoid16(gate) with the gate half of the q projection (sigmoid_mul,
+// SeedlessMetalForward.swift:1012-1022).
+struct SdpaMergeArgs {
+  const float *pm, *pl, *po;
+  const uint16_t* proj;        // gate at [m, h*512 + 256 + d]
+  const int32_t* st;
+  int maxTiles;
+  uint16_t* gated;             // [M, 4096]
+};
+__global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
+  const int h = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;
+  const int N = a.st[0] + m + 1;
+  const int nt = (N + SDPA_TILE - 1) / SDPA_TILE;
+  const size_t base = ((size_t)m * 16 + h) * a.maxTiles;
+  float Mx = -__int_as_float(0x7f800000);
+  for (int t = 0; t < nt; ++t) Mx = fmaxf(Mx, a.pm[base + t]);
+  float L = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int t = 0; t < nt; ++t) {
+    const float f = exp_c(a.pm[base + t] - Mx);
+    L = fmaf(a.pl[base + t], f, L);
+    const float4 o = *reinterpret_cast<const float4*>(a.po + (base + t) * 256 + 4 * lane);
+    O[0] = fmaf(o.x, f, O[0]); O[1] = fmaf(o.y, f, O[1]); O[2] = fmaf(o.z, f, O[2]); O[3] = fmaf(o.w, f, O[3]);
+  }
+  const uint2 graw = *reinterpret_cast<const uint2*>(a.proj + (size_t)m * PROJ_STRIDE + h * 512 + 256 + 4 * lane);
+  const float gt[4] = {lo_h(graw.x), hi_h(graw.x), lo_h(graw.y), hi_h(graw.y)};
+  float r[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = f16r(f16r(O[i] / L) * sigmoid16(gt[i]));
+  *reinterpret_cast<uint2*>(a.gated + (size_t)m * 4096 + h * 256 + 4 * lane) = make_uint2(pack2(r[0], r[1]), pack2(r[2], r[3]));
+}
+
+// -------------------------------------------------------------------------------------------------
+// Head: residual + final norm + lm_head with the arg-max folded into the epilogue.  Each
+// workgroup stores its 16 logits and one (value, index) candidate; k_argmax_final picks the
+// first maximum.  References: SeedlessFusedVerify.swift:3855-3876, argmax_rows :572-596.
+// -------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_head(HiddenArgs ha, const uint32_t* __restrict__ W,
+                                              const uint32_t* __restrict__ SB, int V, uint16_t* __restrict__ logits,
+                                              float* __restrict__ cand_v, int32_t* __restrict__ cand_i) {
+  __shared__ float s_v[4];
+  __shared__ int s_i[4];
+  const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float x[32], sx[4];
+  hidden_prologue(ha, m, lane, blockIdx.x == 0 && wave == 0, x);
+  word_sums(x, sx);
+  const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * 4;
+  float bv = -__int_as_float(0x7f800000);
+  int bi = 0x7fffffff;
+  if (row0 < (size_t)V) {
+    const size_t rows[4] = {row0, row0 + 1, row0 + 2, row0 + 3};
+    float out[4];
+    qdot_rows<1, 4>(W, SB, rows, lane, x, sx, out);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float v = f16r(out[r]);
+      if (v > bv) { bv = v; bi = (int)(row0 + r); }
+    }
+    if (lane == 0) {
+      const uint2 pk = make_uint2(pack2(out[0], out[1]), pack2(out[2], out[3]));
+      *reinterpret_cast<uint2*>(logits + (size_t)m * V + row0) = pk;
+    }
+  }
+  if (lane == 0) { s_v[wave] = bv; s_i[wave] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < 4; ++w) if (s_v[w] > bv) { bv = s_v[w]; bi = s_i[w]; }
+    cand_v[(size_t)m * gridDim.x + blockIdx.x] = bv;
+    cand_i[(size_t)m * gridDim.x + blockIdx.x] = bi;
+  }
+}
+__global__ __launch_bounds__(256) void k_argmax_final(const float* __restrict__ cand_v, const int32_t* __restrict__ cand_i,
+                                                      int ncand, int32_t* __restrict__ tok_out, int out_off,
+                                                      int32_t* __restrict__ feed) {
+  __shared__ float s_v[256];
+  __shared__ int s_i[256];
+  const int m = blockIdx.x, tid = threadIdx.x;
+  float bv = -__int_as_float(0x7f800000);
+  int bi = 0x7fffffff;
+  for (int c = tid; c < ncand; c += 256) {
+    const float v = cand_v[(size_t)m * ncand + c];
+    const int i = cand_i[(size_t)m * ncand + c];
+    if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+  }
+  s_v[tid] = bv; s_i[tid] = bi;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if (tid < s) {
+      const float ov = s_v[tid + s]; const int oi = s_i[tid + s];
+      if (ov > s_v[tid] || (ov == s_v[tid] && oi < s_i[tid])) { s_v[tid] = ov; s_i[tid] = oi; }
+    }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    tok_out[out_off + m] = s_i[0];
+    if (feed) feed[0] = s_i[0];
+  }
+}
+
+// Residual + optional final norm, rows out (forwardRows, SeedlessFusedVerify.swift:3641-3660).
+__global__ __launch_bounds__(64) void k_final_rows(HiddenArgs ha) {
+  float x[32];
+  hidden_prologue(ha, blockIdx.x, threadIdx.x, true, x);
+}
+
+// Step state st = {position, parity[0..n_layers)}: the position advances by M and every layer's
+// ping-pong side flips (attention layers ignore theirs).
+__global__ void k_advance(int32_t* st, int M, int n_layers) {
+  const int t = threadIdx.x;
+  if (t == 0) st[0] += M;
+  for (int i = t; i < n_layers; i += blockDim.x) st[1 + i] ^= 1;
+}
+// {scale, bias} interleave: the engine keeps one 32-bit pair per quantisation group.
+__global__ __launch_bounds__(256) void k_pack_sb(const uint16_t* __restrict__ s, const uint16_t* __restrict__ b,
+                                                 uint32_t* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = (uint32_t)s[i] | ((uint32_t)b[i] << 16);
+}
+
+}  // namespace sl
