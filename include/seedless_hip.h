@@ -191,6 +191,13 @@ int sl_moe_block_rows(sl_engine* e, int layer, const uint16_t* x_f16, int m, uin
 int sl_gdn_layer_rows(sl_engine* e, int layer, const uint16_t* x_f16, int m, uint16_t* out_f16);
 int sl_attn_layer_rows(sl_engine* e, int layer, const uint16_t* x_f16, int m, uint16_t* out_f16);
 
+/* Test hook in the spirit of the reference's diagnostic buffers (diagRouteBufs, SFV:3486): copies
+ * `count` fp16 elements of an internal scratch buffer left by the last launch sequence.
+ * which: 0 projection rows (stride 12352), 1 GDN core output / gated attention output (stride 4096),
+ * 2 rotated queries, 3 mixer output, 4 post-normed rows, 5 routed activations, 6 shared activations,
+ * 7 router logits (stride 256), 8 MoE output. */
+int sl_debug_scratch(sl_engine* e, int which, uint16_t* out_f16, size_t count);
+
 /* Greedy loop standing in for Tell.runSpecLoop without drafts (TellRuntime.swift:716-802):
  * prefill the prompt in chunks of <= max_m rows through sl_forward_tokens, first token = argmax
  * of lm_head on the last normed row, then sl_chained_step_argmax in chains of `chain_k`. */
@@ -213,6 +220,11 @@ int sl_synth_q4(uint32_t* w_dev, uint16_t* scales_dev, uint16_t* biases_dev,
 int sl_synth_f16(uint16_t* dst_dev, int64_t count, uint64_t seed, float mean, float sigma, void* stream);
 /* fp32 tensor: value = mean + sigma * normal. */
 int sl_synth_f32(float* dst_dev, int64_t count, uint64_t seed, float mean, float sigma, void* stream);
+
+/* Self-test of the device arithmetic: y[i] = op(x[i]) evaluated on the GPU (host arrays in/out).
+ * op: 0 exp, 1 log, 2 sigmoid (fp32), 3 sigmoid (half), 4 softplus, 5 round-to-half,
+ * 6 1/sqrt(x/128 + 1e-6), 7 half(x*sigmoid(x)), 8 normal quantile. */
+int sl_selftest_math(int op, const float* x_host, float* y_host, int64_t n);
 
 #ifdef __cplusplus
 }

@@ -50,6 +50,7 @@ def _load():
         "orc_hash64": (u64, [u64, u64]), "orc_normal01": (f32, [u64, u64]),
         "orc_exp_vec": (None, [vp, vp, i64]), "orc_log_vec": (None, [vp, vp, i64]),
         "orc_ppnd7_vec": (None, [vp, vp, i64]),
+        "orc_map_vec": (None, [i32, vp, vp, i64]),
         "orc_qmv": (None, [vp, vp, vp, vp, i32, i32, vp]),
         "orc_qmv_f32": (None, [vp, vp, vp, vp, i32, i32, vp]),
         "orc_dense_f16": (None, [vp, vp, i32, i32, vp]),

@@ -642,6 +642,25 @@ uint64_t orc_hash64(uint64_t seed, uint64_t idx) { return hash64(seed, idx); }
 float orc_normal01(uint64_t seed, uint64_t idx) { return normal01(seed, idx); }
 void orc_exp_vec(const float* x, float* y, int64_t n) { for (int64_t i = 0; i < n; ++i) y[i] = exp_c(x[i]); }
 void orc_log_vec(const float* x, float* y, int64_t n) { for (int64_t i = 0; i < n; ++i) y[i] = log_c(x[i]); }
+// y[i] = op(x[i]); op numbering as in sl_selftest_math.
+void orc_map_vec(int op, const float* x, float* y, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) {
+    const float v = x[i];
+    float r;
+    switch (op) {
+      case 0: r = exp_c(v); break;
+      case 1: r = log_c(v); break;
+      case 2: r = sigmoid32(v); break;
+      case 3: r = sigmoid16(v); break;
+      case 4: r = softplus_c(v); break;
+      case 5: r = f16r(v); break;
+      case 6: r = 1.0f / std::sqrt(v / 128.0f + EPS); break;
+      case 7: r = f16r(v * sigmoid32(v)); break;
+      default: r = ppnd7(v); break;
+    }
+    y[i] = r;
+  }
+}
 void orc_ppnd7_vec(const float* x, float* y, int64_t n) { for (int64_t i = 0; i < n; ++i) y[i] = ppnd7(x[i]); }
 
 void orc_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* s, const uint16_t* b, int n, int k, uint16_t* y) {

@@ -14,9 +14,14 @@
 
 namespace sl {
 
-SL_DEV float f16r(float x) { return __half2float(__float2half_rn(x)); }
+// Rounding to half is always a separate step applied to an already-rounded fp32 value.  The empty
+// asm keeps the compiler from folding the producing fp32 multiply/add into a mixed-precision
+// instruction that rounds the exact result to half once (v_fma_mixlo_f16), which differs from
+// fp32-then-half rounding in about 6e-5 of cases.
+SL_DEV float opaque(float x) { asm("" : "+v"(x)); return x; }
+SL_DEV float f16r(float x) { return __half2float(__float2half_rn(opaque(x))); }
 SL_DEV float h2f(uint16_t h) { return __half2float(__ushort_as_half(h)); }
-SL_DEV uint16_t f2h(float x) { return __half_as_ushort(__float2half_rn(x)); }
+SL_DEV uint16_t f2h(float x) { return __half_as_ushort(__float2half_rn(opaque(x))); }
 
 // exp: n = rint(x*log2 e), two-constant Cody-Waite reduction, degree-6 polynomial, 2^n applied in
 // two exact steps.  x > 88.72 -> +inf, x < -86 (or NaN) -> 0.

@@ -716,6 +716,26 @@ int sl_attn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16
   return push_state(e);
 }
 
+// Test hook: copy `count` fp16 elements of one internal scratch buffer of the last launch sequence.
+int sl_debug_scratch(sl_engine* e, int which, uint16_t* out, size_t count) {
+  int r = guard(e); if (r) return r;
+  const uint16_t* src = nullptr;
+  switch (which) {
+    case 0: src = e->proj; break;
+    case 1: src = e->ycore; break;
+    case 2: src = e->qrot; break;
+    case 3: src = e->mix; break;
+    case 4: src = e->xn; break;
+    case 5: src = e->act; break;
+    case 6: src = e->sh_act; break;
+    case 7: src = e->rlogits; break;
+    case 8: src = e->moe_out; break;
+    default: return SL_ERR_ARG;
+  }
+  if (!src || !out) return SL_ERR_ARG;
+  return copy_sync(e, out, src, count * 2, hipMemcpyDeviceToHost);
+}
+
 int sl_greedy_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_new, int chain_k, int32_t* out) {
   int r = guard(e); if (r) return r;
   if (!prompt || n_prompt < 1 || n_new < 0 || (n_new > 0 && !out) || !e->has_head) return SL_ERR_ARG;

@@ -52,6 +52,26 @@ __global__ __launch_bounds__(256) void k_synth_f32(float* __restrict__ dst, int6
   if (i < n) dst[i] = mean + sigma * normal01(seed, (uint64_t)i);
 }
 
+// Applies one scalar routine of sl_device.cuh to an array (self-test of the device arithmetic).
+__global__ __launch_bounds__(256) void k_math(int op, const float* __restrict__ x, float* __restrict__ y, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float v = x[i];
+  float r;
+  switch (op) {
+    case 0: r = exp_c(v); break;
+    case 1: r = log_c(v); break;
+    case 2: r = sigmoid32(v); break;
+    case 3: r = sigmoid16(v); break;
+    case 4: r = softplus_c(v); break;
+    case 5: r = f16r(v); break;
+    case 6: r = 1.0f / sqrtf(v / 128.0f + 1e-6f); break;
+    case 7: r = f16r(v * sigmoid32(v)); break;
+    default: r = ppnd7(v); break;
+  }
+  y[i] = r;
+}
+
 static int launch_status() { return hipGetLastError() == hipSuccess ? SL_OK : SL_ERR_DEVICE; }
 
 extern "C" int sl_synth_q4(uint32_t* w, uint16_t* s, uint16_t* b, int64_t n, int32_t k, uint64_t seed, float sigma,
@@ -74,4 +94,18 @@ extern "C" int sl_synth_f32(float* dst, int64_t count, uint64_t seed, float mean
   hipLaunchKernelGGL(k_synth_f32, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, (hipStream_t)stream, dst, count,
                      seed, mean, sigma);
   return launch_status();
+}
+
+extern "C" int sl_selftest_math(int op, const float* x_host, float* y_host, int64_t n) {
+  if (!x_host || !y_host || n < 1) return SL_ERR_ARG;
+  float *dx = nullptr, *dy = nullptr;
+  if (hipMalloc((void**)&dx, n * 4) != hipSuccess) return SL_ERR_DEVICE;
+  if (hipMalloc((void**)&dy, n * 4) != hipSuccess) { (void)hipFree(dx); return SL_ERR_DEVICE; }
+  int rc = SL_ERR_DEVICE;
+  if (hipMemcpy(dx, x_host, n * 4, hipMemcpyHostToDevice) == hipSuccess) {
+    hipLaunchKernelGGL(k_math, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, nullptr, op, dx, dy, n);
+    if (hipGetLastError() == hipSuccess && hipMemcpy(y_host, dy, n * 4, hipMemcpyDeviceToHost) == hipSuccess) rc = SL_OK;
+  }
+  (void)hipFree(dx); (void)hipFree(dy);
+  return rc;
 }

@@ -180,6 +180,12 @@ class SeedlessFusedForward:
             return None, None
         return inds, sc
 
+    def debug_scratch(self, which, count):
+        out = np.empty(count, np.float16)
+        if self.lib.dll.sl_debug_scratch(self.h, which, _p(out), count) != abi.SL_OK:
+            return None
+        return out
+
     def _block(self, fn, layer, x):
         x = np.ascontiguousarray(x, np.float16).reshape(-1, abi.H)
         out = np.empty_like(x)

@@ -40,9 +40,11 @@ SIGNATURES = {
     "sl_moe_block_rows": (_i32, [_vp, _i32, _vp, _i32, _vp]),
     "sl_gdn_layer_rows": (_i32, [_vp, _i32, _vp, _i32, _vp]),
     "sl_attn_layer_rows": (_i32, [_vp, _i32, _vp, _i32, _vp]),
+    "sl_debug_scratch": (_i32, [_vp, _i32, _vp, _sz]),
     "sl_greedy_generate": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp]),
     "sl_last_gpu_ms": (_f32, [_vp]),
     "sl_stream": (_vp, [_vp]),
+    "sl_selftest_math": (_i32, [_i32, _vp, _vp, _i64]),
     "sl_synth_q4": (_i32, [_vp, _vp, _vp, _i64, _i32, _u64, _f32, _vp]),
     "sl_synth_f16": (_i32, [_vp, _i64, _u64, _f32, _f32, _vp]),
     "sl_synth_f32": (_i32, [_vp, _i64, _u64, _f32, _f32, _vp]),

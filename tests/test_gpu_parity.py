@@ -26,6 +26,26 @@ def xrows(m, seed, scale=1.0):
     return (np.random.default_rng(seed).normal(0, scale, (m, abi.H))).astype(np.float16)
 
 
+# ---- scalar arithmetic on the device ----------------------------------------------------------------
+def test_device_math_equals_oracle(env):
+    """exp/log/sigmoid/softplus/half rounding/normal quantile evaluated on the GPU give the oracle's
+    bits.  Op 7, half(x*sigmoid(x)), is the case that differs when a compiler folds the fp32
+    multiply and the rounding to half into one mixed-precision instruction."""
+    orc, lib = env["orc"], env["lib"]
+    r = np.random.default_rng(7)
+    n = 1 << 19
+    x = r.uniform(-30, 30, n).astype(np.float32)
+    cases = {0: x, 1: np.exp(x / 2).astype(np.float32), 2: x / 3, 3: (x / 3).astype(np.float16).astype(np.float32),
+             4: x / 3, 5: x * 1e-3, 6: np.abs(x) + 1e-3, 7: r.normal(0, 1.5, n).astype(np.float32),
+             8: r.uniform(0, 1, n).astype(np.float32)}
+    for op, xs in cases.items():
+        xs = np.ascontiguousarray(xs, np.float32)
+        g, c = np.empty_like(xs), np.empty_like(xs)
+        lib.check(lib.dll.sl_selftest_math(op, xs.ctypes.data, g.ctypes.data, xs.size), "sl_selftest_math")
+        orc.dll.orc_map_vec(op, xs.ctypes.data, c.ctypes.data, xs.size)
+        assert same_bits(g, c), (op, first_diff(g.view(np.uint32), c.view(np.uint32)))
+
+
 # ---- generator -----------------------------------------------------------------------------------
 def test_generator_device_equals_host(env):
     torch, orc, lib = env["torch"], env["orc"], env["lib"]
