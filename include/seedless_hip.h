@@ -209,6 +209,11 @@ int sl_greedy_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_
 float sl_last_gpu_ms(const sl_engine* e);
 /* The HIP stream (hipStream_t) the engine launches on. */
 void* sl_stream(sl_engine* e);
+/* Per-kernel timing in the manner of forwardRowsProfiled (SFV:4352): while enabled, every launch of
+ * the lm_head kernel is bracketed by HIP events on the engine's stream; the read call returns the
+ * summed duration and the number of launches since it was enabled. */
+int sl_profile_head(sl_engine* e, int enable);
+int sl_profile_head_read(sl_engine* e, double* ms_sum, int64_t* launches);
 
 /* ---- synthetic checkpoints (seeded, no file I/O) --------------------------------------------
  * Fills device tensors with N(0, sigma) weights quantized by the MLX affine rule, group 64.

@@ -77,6 +77,12 @@ struct sl_engine {
   int pos = 0;
   std::vector<int> parity;
   float last_ms = 0.0f;
+  // optional HIP-event timing of the lm_head kernel, one event pair per step of a chain
+  bool profile_head = false;
+  std::vector<hipEvent_t> head_ev;      // 2 * MAX_CHAIN
+  int head_pending = 0;
+  double head_ms_sum = 0.0;
+  long head_launches = 0;
   bool inject_failure = false;
   std::string fault;
 };
@@ -251,8 +257,11 @@ void advance(sl_engine* e, int M) {
   for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
 }
 void launch_head(sl_engine* e, int M, const HiddenArgs& ha, int out_off, bool feed) {
+  const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
+  if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
   hipLaunchKernelGGL(k_head, dim3(e->n_cand, M), dim3(256), 0, e->stream, ha, e->lm_head.w, e->lm_head.sb, e->vocab,
                      e->logits, e->cand_v, e->cand_i);
+  if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
   hipLaunchKernelGGL(k_argmax_final, dim3(M), dim3(256), 0, e->stream, e->cand_v, e->cand_i, e->n_cand, e->tok_out, out_off,
                      feed ? e->tok_in : (int32_t*)nullptr);
 }
@@ -391,6 +400,7 @@ void sl_destroy(sl_engine* e) {
   if (e->stream) (void)hipStreamSynchronize(e->stream);
   for (void* p : e->allocs) (void)hipFree(p);
   if (e->pinned) (void)hipHostFree(e->pinned);
+  for (hipEvent_t ev : e->head_ev) (void)hipEventDestroy(ev);
   if (e->ev0) (void)hipEventDestroy(e->ev0);
   if (e->ev1) (void)hipEventDestroy(e->ev1);
   if (e->stream) (void)hipStreamDestroy(e->stream);
@@ -402,6 +412,21 @@ void sl_inject_failure(sl_engine* e) { if (e) e->inject_failure = true; }
 int sl_position(const sl_engine* e) { return e ? e->pos : -1; }
 float sl_last_gpu_ms(const sl_engine* e) { return e ? e->last_ms : 0.0f; }
 void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
+int sl_profile_head(sl_engine* e, int enable) {
+  int r = guard(e); if (r) return r;
+  if (enable && e->head_ev.empty()) {
+    e->head_ev.resize(2 * MAX_CHAIN, nullptr);
+    for (auto& ev : e->head_ev) SL_TRY(e, hipEventCreate(&ev));
+  }
+  e->profile_head = enable != 0;
+  e->head_pending = 0; e->head_ms_sum = 0.0; e->head_launches = 0;
+  return SL_OK;
+}
+int sl_profile_head_read(sl_engine* e, double* ms_sum, int64_t* launches) {
+  if (!e || !ms_sum || !launches) return SL_ERR_ARG;
+  *ms_sum = e->head_ms_sum; *launches = e->head_launches;
+  return SL_OK;
+}
 
 static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, const char* what) {
   if (bytes > e->pinned_bytes) return SL_ERR_ARG;
@@ -414,6 +439,9 @@ static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, con
 static void time_end(sl_engine* e) {
   float ms = 0.0f;
   if (hipEventElapsedTime(&ms, e->ev0, e->ev1) == hipSuccess) e->last_ms = ms;
+  for (int i = 0; i < e->head_pending; ++i)
+    if (hipEventElapsedTime(&ms, e->head_ev[2 * i], e->head_ev[2 * i + 1]) == hipSuccess) { e->head_ms_sum += ms; e->head_launches++; }
+  e->head_pending = 0;
 }
 
 int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {

@@ -71,6 +71,14 @@ class SeedlessFusedForward:
     def last_gpu_ms(self):
         return self.lib.dll.sl_last_gpu_ms(self.h)
 
+    def profile_head(self, enable=True):
+        return self.lib.dll.sl_profile_head(self.h, int(enable)) == abi.SL_OK
+
+    def profile_head_read(self):
+        ms, n = C.c_double(), C.c_int64()
+        self.lib.dll.sl_profile_head_read(self.h, C.byref(ms), C.byref(n))
+        return ms.value, n.value
+
     # -- steps --------------------------------------------------------------------------------------
     def step_argmax(self, tokens):
         tok = np.ascontiguousarray(tokens, np.int32)
