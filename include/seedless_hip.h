@@ -209,8 +209,13 @@ int sl_greedy_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_
 float sl_last_gpu_ms(const sl_engine* e);
 /* The HIP stream (hipStream_t) the engine launches on. */
 void* sl_stream(sl_engine* e);
+/* Batch-1 steps run as one persistent kernel launch per token when the device has at least 256
+ * compute units (the reference's counterpart is the one-command-buffer step, SFV:3881-3890);
+ * 0 switches to the kernel-per-stage sequence used for M > 1.  Both give identical results. */
+int sl_set_persistent(sl_engine* e, int enable);
+
 /* Per-kernel timing in the manner of forwardRowsProfiled (SFV:4352): while enabled, every launch of
- * the lm_head kernel is bracketed by HIP events on the engine's stream; the read call returns the
+ * the dominant kernel (the persistent step kernel, or lm_head in the kernel-per-stage sequence) is bracketed by HIP events on the engine's stream; the read call returns the
  * summed duration and the number of launches since it was enabled. */
 int sl_profile_head(sl_engine* e, int enable);
 int sl_profile_head_read(sl_engine* e, double* ms_sum, int64_t* launches);

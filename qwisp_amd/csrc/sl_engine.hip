@@ -11,7 +11,7 @@
 #include <string>
 #include <vector>
 
-#include "sl_kernels.cuh"
+#include "sl_decode.cuh"
 
 using namespace sl;
 
@@ -71,6 +71,10 @@ struct sl_engine {
   float *pm = nullptr, *pl = nullptr, *po = nullptr, *cand_v = nullptr;
   int32_t *cand_i = nullptr, *tok_in = nullptr, *tok_out = nullptr, *st = nullptr;
   int n_cand = 0;
+  // persistent single-token kernel
+  DecodeP* dec_params = nullptr;   // device copy
+  unsigned* dec_bar = nullptr;
+  int dec_grid = 0;                // 0 = not available (fewer than 256 compute units)
   void* pinned = nullptr;        // host staging
   size_t pinned_bytes = 0;
   // host mirrors of the device step state
@@ -83,6 +87,7 @@ struct sl_engine {
   int head_pending = 0;
   double head_ms_sum = 0.0;
   long head_launches = 0;
+  bool use_persistent = true;
   bool inject_failure = false;
   std::string fault;
 };
@@ -265,6 +270,24 @@ void launch_head(sl_engine* e, int M, const HiddenArgs& ha, int out_off, bool fe
   hipLaunchKernelGGL(k_argmax_final, dim3(M), dim3(256), 0, e->stream, e->cand_v, e->cand_i, e->n_cand, e->tok_out, out_off,
                      feed ? e->tok_in : (int32_t*)nullptr);
 }
+// One batch-1 step in a single persistent launch; host mirrors advance as the kernel's own update does.
+void launch_decode(sl_engine* e, int out_off, bool feed) {
+  const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
+  if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
+  hipLaunchKernelGGL(k_decode, dim3(e->dec_grid), dim3(DEC_THREADS), 0, e->stream, e->dec_params, out_off, feed ? 1 : 0);
+  if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
+  e->pos += 1;
+  for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
+}
+// After a persistent step: a workgroup that gave up waiting leaves the abort word set.
+int check_decode_abort(sl_engine* e) {
+  unsigned flag = 0;
+  SL_TRY(e, hipMemcpyAsync(e->pinned, e->dec_bar + 32, 4, hipMemcpyDeviceToHost, e->stream));
+  SL_TRY(e, hipStreamSynchronize(e->stream));
+  std::memcpy(&flag, e->pinned, 4);
+  if (flag) { if (e->fault.empty()) e->fault = "persistent decode kernel: grid barrier timed out"; return SL_ERR_DEVICE; }
+  return SL_OK;
+}
 int to_device(sl_engine* e, void* dst, const void* src, size_t bytes) {
   if (bytes > e->pinned_bytes) return SL_ERR_ARG;
   std::memcpy(e->pinned, src, bytes);
@@ -360,8 +383,8 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
     e->final_norm = upload<uint16_t>(e, d->final_norm, H, loc);
     e->n_cand = d->vocab / 16;
     e->logits = dalloc<uint16_t>(e, (size_t)max_m * d->vocab);
-    e->cand_v = dalloc<float>(e, (size_t)max_m * e->n_cand);
-    e->cand_i = dalloc<int32_t>(e, (size_t)max_m * e->n_cand);
+    e->cand_v = dalloc<float>(e, (size_t)max_m * e->n_cand + 1024);
+    e->cand_i = dalloc<int32_t>(e, (size_t)max_m * e->n_cand + 1024);
     if (!e->final_norm || !e->logits || !e->cand_v || !e->cand_i) return SL_ERR_DEVICE;
   }
   if (e->has_attn) {
@@ -389,6 +412,47 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
   e->st = dalloc<int32_t>(e, 1 + d->n_layers, true);
   if (!e->hA || !e->hB || !e->proj || !e->ycore || !e->mix || !e->xn || !e->rlogits || !e->sgate || !e->sh_act || !e->act ||
       !e->moe_out || !e->normed || !e->rows_out || !e->tok_in || !e->tok_out || !e->st) return SL_ERR_DEVICE;
+  if (has_head) {
+    int ncu = 0;
+    SL_TRY(e, hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, 0));
+    if (ncu >= 256) {
+      std::vector<LayerP> lp(d->n_layers);
+      for (int i = 0; i < d->n_layers; ++i) {
+        const LayerDev& L = e->layers[i];
+        LayerP& q = lp[i];
+        std::memset(&q, 0, sizeof(q));
+        q.is_linear = L.is_linear; q.input_ln = L.input_ln; q.post_ln = L.post_ln;
+        if (L.is_linear) {
+          q.in_w = L.in_proj.w; q.in_sb = L.in_proj.sb; q.out_w = L.out_proj.w; q.out_sb = L.out_proj.sb;
+          q.conv_w = L.conv_w; q.a_log = L.a_log; q.dt_bias = L.dt_bias; q.gdn_norm_w = L.gdn_norm_w;
+          q.hist[0] = L.hist[0]; q.hist[1] = L.hist[1]; q.state[0] = L.state[0]; q.state[1] = L.state[1];
+        } else {
+          q.in_w = L.qkv.w; q.in_sb = L.qkv.sb; q.out_w = L.o_proj.w; q.out_sb = L.o_proj.sb;
+          q.q_norm = L.q_norm; q.k_norm = L.k_norm; q.kcache = L.kcache; q.vcache = L.vcache;
+        }
+        q.router_w = L.router_w; q.sgate_w = L.sgate_w;
+        q.swg_w = L.sw_gate.w; q.swg_sb = L.sw_gate.sb; q.swu_w = L.sw_up.w; q.swu_sb = L.sw_up.sb;
+        q.swd_w = L.sw_down.w; q.swd_sb = L.sw_down.sb; q.shg_w = L.sh_gate.w; q.shg_sb = L.sh_gate.sb;
+        q.shu_w = L.sh_up.w; q.shu_sb = L.sh_up.sb; q.shd_w = L.sh_down.w; q.shd_sb = L.sh_down.sb;
+        q.route_inds = L.route_inds; q.route_scores = L.route_scores;
+      }
+      LayerP* dl = upload<LayerP>(e, lp.data(), lp.size(), SL_LOC_HOST);
+      e->dec_bar = dalloc<unsigned>(e, 4096, true);
+      if (!dl || !e->dec_bar) return SL_ERR_DEVICE;
+      DecodeP P;
+      std::memset(&P, 0, sizeof(P));
+      P.n_layers = d->n_layers; P.E = E; P.vocab = d->vocab; P.max_seq = max_seq_len; P.max_tiles = e->max_tiles;
+      P.layers = dl; P.emb_w = e->embed.w; P.emb_sb = e->embed.sb; P.lm_w = e->lm_head.w; P.lm_sb = e->lm_head.sb;
+      P.final_norm = e->final_norm; P.rope_cos = e->rope_cos; P.rope_sin = e->rope_sin;
+      P.hA = e->hA; P.hB = e->hB; P.proj = e->proj; P.ycore = e->ycore; P.mix = e->mix; P.rlogits = e->rlogits;
+      P.sgate = e->sgate; P.sh_act = e->sh_act; P.act = e->act; P.moe_out = e->moe_out; P.normed = e->normed;
+      P.logits = e->logits; P.pm = e->pm; P.pl = e->pl; P.po = e->po; P.cand_v = e->cand_v; P.cand_i = e->cand_i;
+      P.tok_in = e->tok_in; P.tok_out = e->tok_out; P.st = e->st; P.bar = e->dec_bar;
+      e->dec_params = upload<DecodeP>(e, &P, 1, SL_LOC_HOST);
+      if (!e->dec_params) return SL_ERR_DEVICE;
+      e->dec_grid = 256;
+    }
+  }
   e->pinned_bytes = MH * 2 + 4096 + (size_t)d->n_layers * 4 + (size_t)MAX_CHAIN * 4;
   SL_TRY(e, hipHostMalloc(&e->pinned, e->pinned_bytes, hipHostMallocDefault));
   SL_TRY(e, hipStreamSynchronize(e->stream));
@@ -412,6 +476,11 @@ void sl_inject_failure(sl_engine* e) { if (e) e->inject_failure = true; }
 int sl_position(const sl_engine* e) { return e ? e->pos : -1; }
 float sl_last_gpu_ms(const sl_engine* e) { return e ? e->last_ms : 0.0f; }
 void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
+int sl_set_persistent(sl_engine* e, int enable) {
+  int r = guard(e); if (r) return r;
+  e->use_persistent = enable != 0;
+  return SL_OK;
+}
 int sl_profile_head(sl_engine* e, int enable) {
   int r = guard(e); if (r) return r;
   if (enable && e->head_ev.empty()) {
@@ -451,13 +520,19 @@ int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
   for (int i = 0; i < m; ++i) if (tokens[i] < 0 || tokens[i] >= e->vocab) return SL_ERR_ARG;
   r = to_device(e, e->tok_in, tokens, (size_t)m * 4); if (r) return r;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
-  hipLaunchKernelGGL(k_embed, dim3(H / 256, m), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
-  launch_layers(e, m);
-  HiddenArgs ha{e->hA, e->moe_out, e->final_norm, e->hB, e->normed};
-  launch_head(e, m, ha, 0, false);
-  advance(e, m);
+  const bool persistent = (m == 1 && e->dec_grid > 0 && e->use_persistent);
+  if (persistent) {
+    launch_decode(e, 0, false);
+  } else {
+    hipLaunchKernelGGL(k_embed, dim3(H / 256, m), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
+    launch_layers(e, m);
+    HiddenArgs ha{e->hA, e->moe_out, e->final_norm, e->hB, e->normed};
+    launch_head(e, m, ha, 0, false);
+    advance(e, m);
+  }
   SL_TRY(e, hipEventRecord(e->ev1, e->stream));
   r = read_back(e, out, e->tok_out, (size_t)m * 4, "stepArgmax"); if (r) return r;
+  if (persistent) { r = check_decode_abort(e); if (r) return r; }
   time_end(e);
   return SL_OK;
 }
@@ -468,7 +543,9 @@ int sl_chained_step_argmax(sl_engine* e, int32_t first, int k, int32_t* out) {
   if (e->has_attn && e->pos + k > e->max_seq) return SL_ERR_ARG;
   r = to_device(e, e->tok_in, &first, 4); if (r) return r;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
+  const bool persistent = (e->dec_grid > 0 && e->use_persistent);
   for (int s = 0; s < k; ++s) {
+    if (persistent) { launch_decode(e, s, true); continue; }
     hipLaunchKernelGGL(k_embed, dim3(H / 256, 1), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
     launch_layers(e, 1);
     HiddenArgs ha{e->hA, e->moe_out, e->final_norm, e->hB, e->normed};
@@ -477,6 +554,7 @@ int sl_chained_step_argmax(sl_engine* e, int32_t first, int k, int32_t* out) {
   }
   SL_TRY(e, hipEventRecord(e->ev1, e->stream));
   r = read_back(e, out, e->tok_out, (size_t)k * 4, "chainedStepArgmax"); if (r) return r;
+  if (persistent) { r = check_decode_abort(e); if (r) return r; }
   time_end(e);
   return SL_OK;
 }

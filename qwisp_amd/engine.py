@@ -71,6 +71,9 @@ class SeedlessFusedForward:
     def last_gpu_ms(self):
         return self.lib.dll.sl_last_gpu_ms(self.h)
 
+    def set_persistent(self, enable=True):
+        return self.lib.dll.sl_set_persistent(self.h, int(enable)) == abi.SL_OK
+
     def profile_head(self, enable=True):
         return self.lib.dll.sl_profile_head(self.h, int(enable)) == abi.SL_OK
 

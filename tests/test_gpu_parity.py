@@ -190,6 +190,31 @@ def test_rows_equal_single_steps_and_chain(env, small_model):
             assert same_bits(x, y), li
 
 
+def test_persistent_step_equals_kernel_per_stage(env, small_model):
+    """Batch-1 steps run as one persistent launch; with it switched off the same steps run as the
+    kernel-per-stage sequence used for M > 1.  Tokens, logits and caches must be identical."""
+    cfg, dev, host = small_model
+    a = env["Engine"](cfg, dev, max_m=4, max_seq_len=160)
+    b = env["Engine"](cfg, dev, max_m=4, max_seq_len=160)
+    assert b.set_persistent(False)
+    for eng in (a, b):
+        assert eng.step_argmax([100, 200, 300]) is not None, eng.gpu_fault
+    ta = a.chained_step_argmax(7, 70)          # crosses the 64-key tile boundary
+    tb = b.chained_step_argmax(7, 70)
+    assert ta is not None and tb is not None, (a.gpu_fault, b.gpu_fault)
+    assert ta.tolist() == tb.tolist()
+    sa, sb = a.step_argmax([int(ta[-1])]), b.step_argmax([int(tb[-1])])
+    assert sa.tolist() == sb.tolist()
+    assert same_bits(a.logits_row(0), b.logits_row(0))
+    assert same_bits(a.hidden_rows(1), b.hidden_rows(1))
+    for li in range(cfg.n_layers):
+        for x, y in zip(a.read_layer_cache(li), b.read_layer_cache(li)):
+            assert same_bits(x, y), (li, first_diff(x, y))
+        ia, sca = a.read_route(li, 1)
+        ib, scb = b.read_route(li, 1)
+        assert np.array_equal(ia, ib) and same_bits(sca, scb)
+
+
 def test_forward_rows_and_head(env, small_model):
     cfg, dev, host = small_model
     eng = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)
