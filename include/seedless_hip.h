@@ -214,6 +214,10 @@ void* sl_stream(sl_engine* e);
  * 0 switches to the kernel-per-stage sequence used for M > 1.  Both give identical results. */
 int sl_set_persistent(sl_engine* e, int enable);
 
+/* Diagnostic: while enabled, workgroup 0 of the persistent kernel records a 100 MHz clock stamp after
+ * every grid barrier; the call copies out[0] = number of stamps and out[1..] = stamps of the last step. */
+int sl_debug_stage_clock(sl_engine* e, int enable, unsigned long long* out, int cap);
+
 /* Per-kernel timing in the manner of forwardRowsProfiled (SFV:4352): while enabled, every launch of
  * the dominant kernel (the persistent step kernel, or lm_head in the kernel-per-stage sequence) is bracketed by HIP events on the engine's stream; the read call returns the
  * summed duration and the number of launches since it was enabled. */

@@ -104,21 +104,42 @@ SL_DEV uint4 pack8(const float* f) {
 }
 
 // ---- one packed word against 8 activations ---------------------------------------------------------
-// dq = fmaf chain over the 8 nibbles, least significant first.
-SL_DEV float word_dot(uint32_t w, const float* x) {
+// The 8 activations arrive as 4 packed half pairs.  Masking the word with 0x000F000F leaves two
+// halves whose bit patterns are the nibbles j and j+4: as (subnormal) half values they equal
+// q * 2^-24 exactly, so the products x*q*2^-24 and their fp32 fmaf chain are the chain of x*q scaled
+// by a power of two -- same rounding, no integer-to-float conversion.  The compiler folds the half
+// operands into v_fma_mix_f32.  The 2^24 is returned to the scale: t = fmaf(s*2^24, dq', b*sx).
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+SL_DEV h2_t as_h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
+// dq' = 2^-24 * (fmaf chain over the 8 nibbles, least significant first)
+SL_DEV float word_dot(uint32_t w, const uint32_t* xp /*4 packed pairs*/) {
+  const h2_t m0 = as_h2(w & 0x000F000Fu), m1 = as_h2((w >> 4) & 0x000F000Fu);
+  const h2_t m2 = as_h2((w >> 8) & 0x000F000Fu), m3 = as_h2((w >> 12) & 0x000F000Fu);
+  const h2_t x0 = as_h2(xp[0]), x1 = as_h2(xp[1]), x2 = as_h2(xp[2]), x3 = as_h2(xp[3]);
   float dq = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) dq = fmaf(x[i], (float)((w >> (4 * i)) & 15u), dq);
+  dq = fmaf((float)x0.x, (float)m0.x, dq);
+  dq = fmaf((float)x0.y, (float)m1.x, dq);
+  dq = fmaf((float)x1.x, (float)m2.x, dq);
+  dq = fmaf((float)x1.y, (float)m3.x, dq);
+  dq = fmaf((float)x2.x, (float)m0.y, dq);
+  dq = fmaf((float)x2.y, (float)m1.y, dq);
+  dq = fmaf((float)x3.x, (float)m2.y, dq);
+  dq = fmaf((float)x3.y, (float)m3.y, dq);
   return dq;
 }
 // Four consecutive words of one group-half: t_j = fmaf(s, dq_j, b*sx_j); returns (t0+t1)+(t2+t3).
-SL_DEV float quad_term(uint4 w, uint32_t sb, const float* x /*32*/, const float* sx /*4*/) {
-  const float s = lo_h(sb), b = hi_h(sb);
-  float t0 = fmaf(s, word_dot(w.x, x), b * sx[0]);
-  float t1 = fmaf(s, word_dot(w.y, x + 8), b * sx[1]);
-  float t2 = fmaf(s, word_dot(w.z, x + 16), b * sx[2]);
-  float t3 = fmaf(s, word_dot(w.w, x + 24), b * sx[3]);
+SL_DEV float quad_term(uint4 w, uint32_t sb, const uint32_t* xp /*16 packed pairs*/, const float* sx /*4*/) {
+  const float s = lo_h(sb) * 16777216.0f, b = hi_h(sb);
+  float t0 = fmaf(s, word_dot(w.x, xp), b * sx[0]);
+  float t1 = fmaf(s, word_dot(w.y, xp + 4), b * sx[1]);
+  float t2 = fmaf(s, word_dot(w.z, xp + 8), b * sx[2]);
+  float t3 = fmaf(s, word_dot(w.w, xp + 12), b * sx[3]);
   return (t0 + t1) + (t2 + t3);
+}
+// 32 half-valued floats -> 16 packed pairs (exact)
+SL_DEV void pack_x(const float* x, uint32_t* xp) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) xp[i] = pack2(x[2 * i], x[2 * i + 1]);
 }
 // Left-to-right sums of each run of 8 activations.
 SL_DEV void word_sums(const float* x /*32*/, float* sx /*4*/) {

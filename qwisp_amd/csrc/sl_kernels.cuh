@@ -72,7 +72,7 @@ SL_DEV void hidden_prologue(const HiddenArgs& a, int m, int lane, bool writer, f
 // -------------------------------------------------------------------------------------------------
 template <int NBLK, int R>
 SL_DEV void qdot_rows(const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB, const size_t* rows, int lane,
-                      const float* x, const float* sx, float* out) {
+                      const uint32_t* xp, const float* sx, float* out) {
   constexpr int WPR = NBLK * 256, GPR = NBLK * 32;
   uint4 wv[R][NBLK];
   uint32_t sb[R][NBLK];
@@ -85,18 +85,18 @@ SL_DEV void qdot_rows(const uint32_t* __restrict__ W, const uint32_t* __restrict
     }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    float acc = quad_term(wv[r][0], sb[r][0], x, sx);
+    float acc = quad_term(wv[r][0], sb[r][0], xp, sx);
 #pragma unroll
-    for (int b = 1; b < NBLK; ++b) acc = acc + quad_term(wv[r][b], sb[r][b], x + 32 * b, sx + 4 * b);
+    for (int b = 1; b < NBLK; ++b) acc = acc + quad_term(wv[r][b], sb[r][b], xp + 16 * b, sx + 4 * b);
     out[r] = tree_sum<64>(acc);
   }
 }
 // K = 512: 16 lanes per row; li = lane & 15 owns words 4li..4li+3.  Result valid on all 16 lanes.
-SL_DEV float qdot512(const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB, size_t row, int li, const float* x,
-                     const float* sx) {
+SL_DEV float qdot512(const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB, size_t row, int li,
+                     const uint32_t* xp, const float* sx) {
   const uint4 wv = ld16(W + row * 64 + 4 * li);
   const uint32_t sb = SB[row * 8 + (li >> 1)];
-  return tree_sum<16>(quad_term(wv, sb, x, sx));
+  return tree_sum<16>(quad_term(wv, sb, xp, sx));
 }
 // Dense fp16 row against the lane's 32 activations (router gate, shared-expert gate).
 SL_DEV float dense_dot(const uint16_t* __restrict__ wrow, int lane, const float* x) {
@@ -134,13 +134,15 @@ __global__ __launch_bounds__(256) void k_qmv_hidden(HiddenArgs ha, const uint32_
   float x[32], sx[4];
   hidden_prologue(ha, m, lane, blockIdx.x == 0 && wave == 0, x);
   word_sums(x, sx);
+  uint32_t xp[16];
+  pack_x(x, xp);
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * R;
   if (row0 >= (size_t)N) return;
   size_t rows[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) rows[r] = row0 + r;
   float out[R];
-  qdot_rows<1, R>(W, SB, rows, lane, x, sx, out);
+  qdot_rows<1, R>(W, SB, rows, lane, xp, sx, out);
   if (lane == 0) {
 #pragma unroll
     for (int r = 0; r < R; ++r) y[(size_t)m * y_stride + row0 + r] = f2h(out[r]);
@@ -153,11 +155,14 @@ __global__ __launch_bounds__(256) void k_qmv_plain(const uint16_t* __restrict__ 
                                                    const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB,
                                                    int N, uint16_t* __restrict__ y, int y_stride) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float x[32 * NBLK], sx[4 * NBLK];
+  float sx[4 * NBLK];
+  uint32_t xp[16 * NBLK];
 #pragma unroll
   for (int b = 0; b < NBLK; ++b) {
-    load32(xin + (size_t)m * x_stride + b * 2048 + 32 * lane, x + 32 * b);
-    word_sums(x + 32 * b, sx + 4 * b);
+    float x[32];
+    load32(xin + (size_t)m * x_stride + b * 2048 + 32 * lane, x);
+    word_sums(x, sx + 4 * b);
+    pack_x(x, xp + 16 * b);
   }
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * R;
   if (row0 >= (size_t)N) return;
@@ -165,7 +170,7 @@ __global__ __launch_bounds__(256) void k_qmv_plain(const uint16_t* __restrict__ 
 #pragma unroll
   for (int r = 0; r < R; ++r) rows[r] = row0 + r;
   float out[R];
-  qdot_rows<NBLK, R>(W, SB, rows, lane, x, sx, out);
+  qdot_rows<NBLK, R>(W, SB, rows, lane, xp, sx, out);
   if (lane == 0) {
 #pragma unroll
     for (int r = 0; r < R; ++r) y[(size_t)m * y_stride + row0 + r] = f2h(out[r]);
@@ -288,12 +293,13 @@ __global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict_
                                                      const uint16_t* __restrict__ norm_w, const uint32_t* __restrict__ W,
                                                      const uint32_t* __restrict__ SB, int N, uint16_t* __restrict__ y) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float x[64], sx[8];
+  float sx[8];
+  uint32_t xp[32];
   float nw[32];
   load32(norm_w + 32 * (lane & 3), nw);
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
-    float* xb = x + 32 * b;
+    float xb[32];
     load32(ycore + (size_t)m * 4096 + b * 2048 + 32 * lane, xb);
     float leaf[16];
 #pragma unroll
@@ -312,6 +318,7 @@ __global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict_
       xb[i] = f16r((z[i] * sigmoid32(z[i])) * nrm);
     }
     word_sums(xb, sx + 4 * b);
+    pack_x(xb, xp + 16 * b);
   }
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * R;
   if (row0 >= (size_t)N) return;
@@ -319,7 +326,7 @@ __global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict_
 #pragma unroll
   for (int r = 0; r < R; ++r) rows[r] = row0 + r;
   float out[R];
-  qdot_rows<2, R>(W, SB, rows, lane, x, sx, out);
+  qdot_rows<2, R>(W, SB, rows, lane, xp, sx, out);
   if (lane == 0) {
 #pragma unroll
     for (int r = 0; r < R; ++r) y[(size_t)m * H + row0 + r] = f2h(out[r]);
@@ -348,11 +355,13 @@ __global__ __launch_bounds__(256) void k_moe_a(MoeAArgs a) {
   hidden_prologue(a.ha, m, lane, blockIdx.x == 0 && wave == 0, x);
   if (blockIdx.x < MOE_A_SHARED_BLOCKS) {
     word_sums(x, sx);
+    uint32_t xp[16];
+    pack_x(x, xp);
     const size_t i0 = ((size_t)blockIdx.x * 4 + wave) * 2;
     const size_t rows[2] = {i0, i0 + 1};
     float g[2], u[2];
-    qdot_rows<1, 2>(a.shg_w, a.shg_sb, rows, lane, x, sx, g);
-    qdot_rows<1, 2>(a.shu_w, a.shu_sb, rows, lane, x, sx, u);
+    qdot_rows<1, 2>(a.shg_w, a.shg_sb, rows, lane, xp, sx, g);
+    qdot_rows<1, 2>(a.shu_w, a.shu_sb, rows, lane, xp, sx, u);
     if (lane == 0) {
 #pragma unroll
       for (int r = 0; r < 2; ++r) a.sh_act[(size_t)m * 512 + i0 + r] = f2h(swiglu16(f16r(g[r]), f16r(u[r])));
@@ -377,7 +386,7 @@ __global__ __launch_bounds__(256) void k_moe_a(MoeAArgs a) {
 // (ties to the lower index), half renormalisation.  One wave; lane l owns experts 4l..4l+3.
 // Reference: route_top8_rows SeedlessFusedVerify.swift:191-213.
 // -------------------------------------------------------------------------------------------------
-SL_DEV void route_wave(const uint16_t* __restrict__ logits, int E, int lane, int* inds, float* scores) {
+SL_DEV void route_wave(const uint16_t* __restrict__ logits, int E, int lane, int* inds /*LDS [8]*/, float* scores /*LDS [8]*/) {
   const float NEG = -__int_as_float(0x7f800000);
   float lg[4], ex[4];
 #pragma unroll
@@ -386,7 +395,7 @@ SL_DEV void route_wave(const uint16_t* __restrict__ logits, int E, int lane, int
 #pragma unroll
   for (int i = 0; i < 4; ++i) ex[i] = (4 * lane + i < E) ? exp_c(lg[i] - mx) : 0.0f;
   const float Z = tree_sum<64>(((ex[0] + ex[1]) + ex[2]) + ex[3]);
-#pragma unroll
+#pragma unroll 1
   for (int k = 0; k < 8; ++k) {
     float bv = lg[0]; int bi = 4 * lane;
 #pragma unroll
@@ -400,18 +409,17 @@ SL_DEV void route_wave(const uint16_t* __restrict__ logits, int E, int lane, int
     const int sub = bi & 3;
     const float mine = (sub == 0) ? ex[0] : (sub == 1) ? ex[1] : (sub == 2) ? ex[2] : ex[3];
     const float e = __shfl(mine, bi >> 2, 64);
-    inds[k] = bi;
-    scores[k] = f16r(e / Z);
+    if (lane == 0) { inds[k] = bi; scores[k] = f16r(e / Z); }
     if ((bi >> 2) == lane) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) if (i == sub) lg[i] = NEG;
     }
   }
-  float ss = 0.0f;
-#pragma unroll
-  for (int k = 0; k < 8; ++k) ss = f16r(ss + scores[k]);
-#pragma unroll
-  for (int k = 0; k < 8; ++k) scores[k] = f16r(scores[k] / ss);
+  if (lane == 0) {
+    float ss = 0.0f;
+    for (int k = 0; k < 8; ++k) ss = f16r(ss + scores[k]);
+    for (int k = 0; k < 8; ++k) scores[k] = f16r(scores[k] / ss);
+  }
 }
 
 // MoE stage B: routing + the 8 routed experts' gate/up with SwiGLU.
@@ -427,29 +435,27 @@ struct MoeBArgs {
 };
 __global__ __launch_bounds__(256) void k_moe_b(MoeBArgs a) {
   __shared__ int s_inds[8];
+  __shared__ float s_sc[8];
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (wave == 0) {
-    int inds[8]; float sc[8];
-    route_wave(a.rlogits + (size_t)m * 256, a.E, lane, inds, sc);
-    if (lane == 0) {
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        s_inds[k] = inds[k];
-        if (blockIdx.x == 0) { a.inds[m * 8 + k] = inds[k]; a.scores[m * 8 + k] = f2h(sc[k]); }
-      }
+    route_wave(a.rlogits + (size_t)m * 256, a.E, lane, s_inds, s_sc);
+    if (lane == 0 && blockIdx.x == 0) {
+      for (int k = 0; k < 8; ++k) { a.inds[m * 8 + k] = s_inds[k]; a.scores[m * 8 + k] = f2h(s_sc[k]); }
     }
   }
   float x[32], sx[4];
   load32(a.xn + (size_t)m * H + 32 * lane, x);
   word_sums(x, sx);
+  uint32_t xp[16];
+  pack_x(x, xp);
   __syncthreads();
   const int p0 = (blockIdx.x * 4 + wave) * 2;          // pair index in [0, 8*512)
   const int k = p0 >> 9, i0 = p0 & 511;
   const size_t base = (size_t)s_inds[k] * 512 + i0;
   const size_t rows[2] = {base, base + 1};
   float g[2], u[2];
-  qdot_rows<1, 2>(a.g_w, a.g_sb, rows, lane, x, sx, g);
-  qdot_rows<1, 2>(a.u_w, a.u_sb, rows, lane, x, sx, u);
+  qdot_rows<1, 2>(a.g_w, a.g_sb, rows, lane, xp, sx, g);
+  qdot_rows<1, 2>(a.u_w, a.u_sb, rows, lane, xp, sx, u);
   if (lane == 0) {
 #pragma unroll
     for (int r = 0; r < 2; ++r) a.act[((size_t)m * 8 + k) * 512 + i0 + r] = f2h(swiglu16(f16r(g[r]), f16r(u[r])));
@@ -475,17 +481,20 @@ __global__ __launch_bounds__(128) void k_moe_c(MoeCArgs a) {
   const int n = (blockIdx.x * 2 + wave) * 4 + sub;
   float acc = 0.0f;
   float x[32], sx[4];
+  uint32_t xp[16];
 #pragma unroll 1
   for (int k = 0; k < 8; ++k) {
     load32(a.act + ((size_t)m * 8 + k) * 512 + 32 * li, x);
     word_sums(x, sx);
+    pack_x(x, xp);
     const size_t row = (size_t)a.inds[m * 8 + k] * 2048 + n;
-    const float d = f16r(qdot512(a.d_w, a.d_sb, row, li, x, sx));
+    const float d = f16r(qdot512(a.d_w, a.d_sb, row, li, xp, sx));
     acc = f16r(acc + f16r(d * h2f(a.scores[m * 8 + k])));
   }
   load32(a.sh_act + (size_t)m * 512 + 32 * li, x);
   word_sums(x, sx);
-  const float sy = f16r(qdot512(a.shd_w, a.shd_sb, (size_t)n, li, x, sx));
+  pack_x(x, xp);
+  const float sy = f16r(qdot512(a.shd_w, a.shd_sb, (size_t)n, li, xp, sx));
   const float s = sigmoid16(h2f(a.sgate[m]));
   if (li == 0) a.out[(size_t)m * H + n] = f2h(f16r(acc + f16r(s * sy)));
 }
@@ -683,13 +692,15 @@ __global__ __launch_bounds__(256) void k_head(HiddenArgs ha, const uint32_t* __r
   float x[32], sx[4];
   hidden_prologue(ha, m, lane, blockIdx.x == 0 && wave == 0, x);
   word_sums(x, sx);
+  uint32_t xp[16];
+  pack_x(x, xp);
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * 4;
   float bv = -__int_as_float(0x7f800000);
   int bi = 0x7fffffff;
   if (row0 < (size_t)V) {
     const size_t rows[4] = {row0, row0 + 1, row0 + 2, row0 + 3};
     float out[4];
-    qdot_rows<1, 4>(W, SB, rows, lane, x, sx, out);
+    qdot_rows<1, 4>(W, SB, rows, lane, xp, sx, out);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const float v = f16r(out[r]);
