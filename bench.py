@@ -6,9 +6,9 @@ The model is synthetic (seeded, generated in HBM); a 512-token uniform-random pr
 before the timed region; tokens feed back on the device in chains, as the reference's default
 decode does (chainedStepArgmax, K = 8).
 
-Prints one JSON line: throughput, the roofline of the dominant kernel (lm_head GEMV+argmax, timed
-with HIP events on the engine's stream), the whole-step HBM fraction, and the CPU baseline (the
-oracle, timed on this host's cores on a bounded sample of the same workload).
+Prints one JSON line: throughput, the roofline of the dominant kernel (the persistent step kernel
+k_decode, which runs a whole token; timed with HIP events on the engine's stream), and the CPU
+baseline (the oracle, timed on this host's cores on a bounded sample of the same workload).
 """
 import argparse
 import json
@@ -22,6 +22,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 PROMPT_LEN = 512
+# HBM bytes per k_decode launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/), or None until measured
+TRAFFIC_BYTES_PER_LAUNCH = None
 
 
 def step_bytes(cfg, ctx):
@@ -47,6 +49,8 @@ def main():
     ap.add_argument("--chain", type=int, default=8, help="tokens per on-device chain")
     ap.add_argument("--layers", type=int, default=40, help="for quick functional runs only")
     ap.add_argument("--cpu-tokens", type=int, default=4, help="decode tokens timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="only run a plain device copy of this many MiB (reference for rocprofv3 FETCH_SIZE/WRITE_SIZE) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
@@ -56,6 +60,15 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs the MI355X; no GPU is visible.")
     torch.cuda.set_device(0)
+    if args.copy_calibration:
+        n = args.copy_calibration << 20
+        src = torch.full((n,), 3, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes": n, "copies": 3}))
+        return
     from qwisp_amd import lib, synth
     from qwisp_amd.engine import SeedlessFusedForward
 
@@ -105,7 +118,7 @@ def main():
     ms_step = elapsed * 1e3 / args.steps
     tok_s = args.steps / elapsed
     head_avg_ms = head_ms / max(head_n, 1)
-    head_gbs = head_b / (head_avg_ms * 1e-3) / 1e9 if head_n else 0.0
+    head_gbs = total_b / (head_avg_ms * 1e-3) / 1e9 if head_n else 0.0
     step_gbs = total_b / (ms_step * 1e-3) / 1e9
 
     cpu = None
@@ -132,9 +145,9 @@ def main():
         "config": {"workload": f"{cfg.n_layers}-layer 35B-A3B hybrid (3 GDN : 1 attention, 256-expert top-8 MoE + shared), "
                                f"vocab {cfg.vocab}, 4-bit g64; greedy decode after a {PROMPT_LEN}-token prompt, batch 1",
                    "chain_k": args.chain, "context": [PROMPT_LEN + args.warmup, PROMPT_LEN + args.warmup + args.steps]},
-        "roofline": {"bound": "hbm", "kernel": "k_head (lm_head 4-bit GEMV + argmax)", "achieved": head_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": head_gbs / HBM_PEAK_GBS, "traffic": None,
-                     "launches": head_n, "avg_ms": head_avg_ms, "bytes_per_launch": head_b},
+        "roofline": {"bound": "hbm", "kernel": "k_decode (persistent batch-1 step: 40 layers + lm_head + argmax)",
+                     "achieved": head_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head_gbs / HBM_PEAK_GBS,
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH, "launches": head_n, "avg_ms": head_avg_ms, "bytes_per_launch": total_b},
         "step_hbm": {"bytes_per_token": total_b, "achieved_GBs": step_gbs, "frac_of_peak": step_gbs / HBM_PEAK_GBS},
         "cpu_baseline": cpu,
         "setup_s": {"generate": t_gen, "prefill_512": t_prefill},

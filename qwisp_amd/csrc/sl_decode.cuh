@@ -208,7 +208,7 @@ SL_DEV void lds_get_x(int b, int lane, uint32_t* xp, float* sx) {
 }
 
 // Hidden prologue, run by one wave: x = half(h + r), optional rmsnorm, result into LDS.
-__device__ __noinline__ void dec_hidden(const uint16_t* h_in, const uint16_t* r_in, const uint16_t* lnw, uint16_t* h_out,
+SL_DEV void dec_hidden(const uint16_t* h_in, const uint16_t* r_in, const uint16_t* lnw, uint16_t* h_out,
                                         uint16_t* xn_out, int writer) {
   const int lane = threadIdx.x & 63;
   float x[32], w[32];
@@ -254,7 +254,7 @@ struct F4 { float v[4]; };
 struct F2 { float v[2]; };
 // The three dot shapes of a step, each compiled once (arguments travel in registers):
 // 4 rows x 2048, 2 rows x 2048, 1 row x 4096.
-__device__ __noinline__ F4 dot_1x4_(uint4 w0, uint4 w1, uint4 w2, uint4 w3, uint32_t s0, uint32_t s1, uint32_t s2, uint32_t s3) {
+SL_DEV F4 dot_1x4_(uint4 w0, uint4 w1, uint4 w2, uint4 w3, uint32_t s0, uint32_t s1, uint32_t s2, uint32_t s3) {
   const int lane = threadIdx.x & 63;
   uint32_t x[16]; float sx[4];
   lds_get_x(0, lane, x, sx);
@@ -265,7 +265,7 @@ __device__ __noinline__ F4 dot_1x4_(uint4 w0, uint4 w1, uint4 w2, uint4 w3, uint
   o.v[3] = tree_sum<64>(quad_term(w3, s3, x, sx));
   return o;
 }
-__device__ __noinline__ F2 dot_1x2_(uint4 w0, uint4 w1, uint32_t s0, uint32_t s1) {
+SL_DEV F2 dot_1x2_(uint4 w0, uint4 w1, uint32_t s0, uint32_t s1) {
   const int lane = threadIdx.x & 63;
   uint32_t x[16]; float sx[4];
   lds_get_x(0, lane, x, sx);
@@ -274,7 +274,7 @@ __device__ __noinline__ F2 dot_1x2_(uint4 w0, uint4 w1, uint32_t s0, uint32_t s1
   o.v[1] = tree_sum<64>(quad_term(w1, s1, x, sx));
   return o;
 }
-__device__ __noinline__ float dot_2x1_(uint4 w0, uint4 w1, uint32_t s0, uint32_t s1) {
+SL_DEV float dot_2x1_(uint4 w0, uint4 w1, uint32_t s0, uint32_t s1) {
   const int lane = threadIdx.x & 63;
   uint32_t x[16]; float sx[4];
   lds_get_x(0, lane, x, sx);
@@ -293,7 +293,7 @@ SL_DEV float dot_2x1(const WRegs<2, 1>& r) { return dot_2x1_(r.w[0][0], r.w[0][1
                 (void)tid; (void)lane; (void)wave; (void)wg; (void)G; (void)NW; (void)gw
 
 // stage 1: input norm + in-projection (GDN qkv|z|b|a or attention q|k|v); wave gw owns rows gw + j*NW
-__device__ __noinline__ bool stage_in(const DecodeP& P, const LayerP& Y, int li, int pos) {
+SL_DEV bool stage_in(const DecodeP& P, const LayerP& Y, int li, int pos) {
   DEC_IDS;
   const int N = Y.is_linear ? SL_GDN_IN_N : SL_ATT_QKV_N;
   WRegs<1, 4> wr;
@@ -343,7 +343,7 @@ __device__ __noinline__ bool stage_in(const DecodeP& P, const LayerP& Y, int li,
 }
 
 // GDN stage 2: conv + prep + gated delta rule; 256 units of (value head, 16 state rows)
-__device__ __noinline__ bool stage_gdn(const DecodeP& P, const LayerP& Y, int li) {
+SL_DEV bool stage_gdn(const DecodeP& P, const LayerP& Y, int li) {
   DEC_IDS;
   Lds& L = g_L;
   const int par = P.st[1 + li];
@@ -436,7 +436,7 @@ __device__ __noinline__ bool stage_gdn(const DecodeP& P, const LayerP& Y, int li
 
 // K = 4096 projection: GDN out_proj with the gated rmsnorm as prologue, or attention o_proj after the
 // tile merge (done by workgroup 0 in an extra barrier phase).
-__device__ __noinline__ bool stage_out(const DecodeP& P, const LayerP& Y, int nt) {
+SL_DEV bool stage_out(const DecodeP& P, const LayerP& Y, int nt) {
   DEC_IDS;
   const float NEG = -__int_as_float(0x7f800000);
   WRegs<2, 1> wr;
@@ -515,7 +515,7 @@ __device__ __noinline__ bool stage_out(const DecodeP& P, const LayerP& Y, int nt
 }
 
 // 8 leaves (32 dims) of the score tree of one key against one query head: balanced sub-tree.
-__device__ __noinline__ float score_leaf8(const uint16_t* kr, const float* qh) {
+SL_DEV float score_leaf8(const uint16_t* kr, const float* qh) {
   float n[8];
 #pragma unroll
   for (int l = 0; l < 8; ++l) {
@@ -529,7 +529,7 @@ __device__ __noinline__ float score_leaf8(const uint16_t* kr, const float* qh) {
 }
 
 // attention stage 2: q/k prep, KV append, tile pass; units of (key tile, kv head)
-__device__ __noinline__ bool stage_sdpa(const DecodeP& P, const LayerP& Y, int pos) {
+SL_DEV bool stage_sdpa(const DecodeP& P, const LayerP& Y, int pos) {
   DEC_IDS;
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
@@ -644,7 +644,7 @@ __device__ __noinline__ bool stage_sdpa(const DecodeP& P, const LayerP& Y, int p
 }
 
 // MoE stage A: post norm; router rows (waves 0..E-1), shared-gate row (wave E), shared gate/up pairs (waves 512..1023)
-__device__ __noinline__ bool stage_moe_a(const DecodeP& P, const LayerP& Y) {
+SL_DEV bool stage_moe_a(const DecodeP& P, const LayerP& Y) {
   DEC_IDS;
   const bool is_dense = gw <= P.E;
   const bool is_pair = gw >= 512 && gw < 1024;
@@ -675,7 +675,7 @@ __device__ __noinline__ bool stage_moe_a(const DecodeP& P, const LayerP& Y) {
 }
 
 // MoE stage B: routing (one wave per workgroup) + routed gate/up + SwiGLU; xs still holds the post-normed row
-__device__ __noinline__ bool stage_moe_b(const DecodeP& P, const LayerP& Y) {
+SL_DEV bool stage_moe_b(const DecodeP& P, const LayerP& Y) {
   DEC_IDS;
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
@@ -755,7 +755,7 @@ __device__ __noinline__ bool stage_moe_b(const DecodeP& P, const LayerP& Y) {
 
 // MoE stage C: down-projections, half-precision combine in routing order, gated shared add.
 // Units (quad of 4 outputs, slot): slots 0..7 routed experts, slot 8 shared; 2 quads per workgroup.
-__device__ __noinline__ bool stage_moe_c(const DecodeP& P, const LayerP& Y, const uint32_t* next_w, const uint32_t* next_sb,
+SL_DEV bool stage_moe_c(const DecodeP& P, const LayerP& Y, const uint32_t* next_w, const uint32_t* next_sb,
                                          int next_n, int next_contig) {
   DEC_IDS;
   Lds& L = g_L;
@@ -819,7 +819,7 @@ __device__ __noinline__ bool stage_moe_c(const DecodeP& P, const LayerP& Y, cons
 
 // head: final norm + lm_head + argmax.  Each wave owns a contiguous chunk of 64 vocabulary rows, 4 at a
 // time with the next group prefetched; candidates are reduced per workgroup, then by workgroup 0.
-__device__ __noinline__ bool stage_head(const DecodeP& P, int pos, int out_off, int feed) {
+SL_DEV bool stage_head(const DecodeP& P, int pos, int out_off, int feed) {
   DEC_IDS;
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
