@@ -11,7 +11,7 @@
 #include <string>
 #include <vector>
 
-#include "sl_decode.cuh"
+#include "sl_flow.cuh"
 
 using namespace sl;
 
@@ -77,6 +77,9 @@ struct sl_engine {
   unsigned long long* dec_tstamp = nullptr;
   unsigned* dec_bar = nullptr;
   int dec_grid = 0;                // 0 = not available (fewer than 256 compute units)
+  FlowP* flow_params = nullptr;    // device copy of the dataflow variant's parameters
+  FlowP flow_host;
+  bool use_flow = true;
   void* pinned = nullptr;        // host staging
   size_t pinned_bytes = 0;
   // host mirrors of the device step state
@@ -277,7 +280,10 @@ void launch_decode(sl_engine* e, int out_off, bool feed) {
   const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
   hipLaunchKernelGGL(k_embed, dim3(H / 256, 1), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
-  hipLaunchKernelGGL(k_decode, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->dec_params, out_off, feed ? 1 : 0);
+  if (e->use_flow)
+    hipLaunchKernelGGL(k_decode_flow, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0);
+  else
+    hipLaunchKernelGGL(k_decode, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->dec_params, out_off, feed ? 1 : 0);
   if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
   e->pos += 1;
   for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
@@ -418,7 +424,7 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
   if (has_head) {
     int ncu = 0;
     SL_TRY(e, hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, 0));
-    if (ncu >= 256) {
+    if (ncu >= 256 && d->n_layers <= FLOW_MAX_LAYERS) {
       std::vector<LayerP> lp(d->n_layers);
       for (int i = 0; i < d->n_layers; ++i) {
         const LayerDev& L = e->layers[i];
@@ -456,6 +462,24 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
       e->dec_params = upload<DecodeP>(e, &P, 1, SL_LOC_HOST);
       if (!e->dec_params) return SL_ERR_DEVICE;
       SL_TRY(e, hipFuncSetAttribute((const void*)k_decode, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
+      {
+        FlowP F;
+        std::memset(&F, 0, sizeof(F));
+        F.d = P;
+        F.th[0] = dalloc<uint32_t>(e, H, true); F.th[1] = dalloc<uint32_t>(e, H, true);
+        F.tproj = dalloc<uint32_t>(e, PROJ_STRIDE, true); F.tycore = dalloc<uint32_t>(e, 4096, true);
+        F.tmix = dalloc<uint32_t>(e, H, true); F.trlog = dalloc<uint32_t>(e, 256, true); F.tsg = dalloc<uint32_t>(e, 4, true);
+        F.tsh = dalloc<uint32_t>(e, 512, true); F.tact = dalloc<uint32_t>(e, 8 * 512, true); F.tmoe = dalloc<uint32_t>(e, H, true);
+        F.tml = dalloc<uint4>(e, (size_t)SL_ATT_HEADS * e->max_tiles, true);
+        F.tpo = dalloc<uint4>(e, (size_t)SL_ATT_HEADS * e->max_tiles * 128, true);
+        F.tcand = dalloc<uint4>(e, 256, true);
+        if (!F.th[0] || !F.th[1] || !F.tproj || !F.tycore || !F.tmix || !F.trlog || !F.tsg || !F.tsh || !F.tact || !F.tmoe ||
+            !F.tml || !F.tpo || !F.tcand) return SL_ERR_DEVICE;
+        e->flow_host = F;
+        e->flow_params = upload<FlowP>(e, &F, 1, SL_LOC_HOST);
+        if (!e->flow_params) return SL_ERR_DEVICE;
+        SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
+      }
       e->dec_grid = 256;
     }
   }
@@ -485,6 +509,7 @@ void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
 int sl_set_persistent(sl_engine* e, int enable) {
   int r = guard(e); if (r) return r;
   e->use_persistent = enable != 0;
+  e->use_flow = enable != 2;          // 2 = the barrier-separated variant of the single-launch step
   return SL_OK;
 }
 // Test/diagnostic hook: per-barrier clock stamps (100 MHz ticks) of workgroup 0 for the steps run while
@@ -496,6 +521,8 @@ int sl_debug_stage_clock(sl_engine* e, int enable, unsigned long long* out, int 
     r = copy_sync(e, out, e->dec_tstamp, (size_t)(cap < 2048 + 8192 ? cap : 2048 + 8192) * 8, hipMemcpyDeviceToHost); if (r) return r;
   }
   e->dec_host.tstamp = enable ? e->dec_tstamp : nullptr;
+  e->flow_host.d.tstamp = e->dec_host.tstamp;
+  r = copy_sync(e, e->flow_params, &e->flow_host, sizeof(FlowP), hipMemcpyHostToDevice); if (r) return r;
   return copy_sync(e, e->dec_params, &e->dec_host, sizeof(DecodeP), hipMemcpyHostToDevice);
 }
 int sl_profile_head(sl_engine* e, int enable) {

@@ -1,0 +1,924 @@
+// Dataflow variant of the persistent batch-1 step: no grid barriers.
+//
+// Every value a stage hands to the next one travels with a tag that names the stage instance that
+// produced it (layer, stage, launch): fp16 activations as 32-bit words {half, tag16}, fp32 attention
+// partials and arg-max candidates as 16-byte chunks {v0, v1, tag, tag}.  A consumer simply loads the
+// words it needs (sc1, coherent across XCDs) and retries until all tags are the expected ones, so a
+// dependency costs one store->load hop instead of "store, wait for the ack, two atomic hops, a flag
+// hop, then fetch".  Producers never wait.  Buffers are reused every layer; this is safe because
+// between the last reader of a buffer and its next writer there is always a stage to which every
+// workgroup contributes (in-proj, routed gate/up, down-proj), and a writer only runs after it has
+// consumed that stage's complete output.
+//
+// Arithmetic, reduction order and work split are those of sl_decode.cuh / sl_kernels.cuh.
+#pragma once
+#include "sl_decode.cuh"
+
+namespace sl {
+
+struct FlowP {
+  DecodeP d;
+  uint32_t *th[2];      // hidden rows A/B                 [2048] {half, tag}
+  uint32_t *tproj;      // projection output               [12352]
+  uint32_t *tycore;     // GDN core out / gated attn out   [4096]
+  uint32_t *tmix;       // mixer output                    [2048]
+  uint32_t *trlog;      // router logits                   [256]
+  uint32_t *tsg;        // shared-gate logit               [4]
+  uint32_t *tsh;        // shared expert activations       [512]
+  uint32_t *tact;       // routed activations              [8*512]
+  uint32_t *tmoe;       // MoE output                      [2048]
+  uint4 *tml;           // attention {max, sum, tag, tag}  [16][max_tiles]
+  uint4 *tpo;           // attention {o[2c], o[2c+1], tag, tag}  [16][max_tiles][128]
+  uint4 *tcand;         // {value, index, tag, tag}        [256]
+};
+
+// Parameters live in LDS for the whole launch.  Reading them there (ds_read + readfirstlane) does not
+// pass through the vector-memory return queue, so fetching a pointer never waits behind the weight
+// loads that are in flight, and the scalar cache is not asked for a new line every stage.
+constexpr int FLOW_MAX_LAYERS = 64;
+struct FlowLds {
+  FlowP F;
+  LayerP layers[FLOW_MAX_LAYERS];
+  unsigned long long parity;      // bit l = which copy of layer l's recurrent state / history is current
+  int pos;
+  uint32_t base;
+};
+__shared__ FlowLds g_K;
+
+template <typename T>
+SL_DEV T uni(const T& r) {
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "parameter fields are 4 or 8 bytes");
+  if constexpr (sizeof(T) == 4) {
+    const uint32_t v = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const uint32_t*>(&r));
+    return __builtin_bit_cast(T, v);
+  } else {
+    const uint2 v = *reinterpret_cast<const uint2*>(&r);
+    const unsigned long long u = (unsigned long long)(uint32_t)__builtin_amdgcn_readfirstlane(v.x) |
+                                 ((unsigned long long)(uint32_t)__builtin_amdgcn_readfirstlane(v.y) << 32);
+    return __builtin_bit_cast(T, u);
+  }
+}
+
+// Thread and workgroup ids pass through an empty volatile asm in every stage: index arithmetic derived
+// from them is then recomputed where it is used instead of being hoisted out of the layer loop, kept live
+// across all stages and spilled (a spill reload is a vector-memory load and would queue behind the weight
+// prefetch).
+SL_DEV int fresh_v(int x) { asm volatile("" : "+v"(x)); return x; }
+SL_DEV int fresh_s(int x) { asm volatile("" : "+s"(x)); return x; }
+
+enum { FS_IN = 0, FS_CORE = 1, FS_MERGE = 2, FS_OUT = 3, FS_A = 4, FS_B = 5, FS_C = 6 };
+constexpr unsigned FLOW_SPIN_LIMIT = 1u << 19;
+
+// `base` counts stage instances over all launches (32 bits, advanced by 8*(layers+1) per launch).
+SL_DEV uint32_t flow_tag(uint32_t base, int layer, int stage) { return 0x8000u | ((base + (uint32_t)(layer * 8 + stage)) & 0x7fffu); }
+// 16-byte chunks carry the whole counter: their slots are not rewritten every layer (a key tile beyond
+// the current position keeps what an earlier, longer sequence left there).
+SL_DEV uint32_t flow_tag32(uint32_t base, int layer, int stage) { return 0x80000000u | (base + (uint32_t)(layer * 8 + stage)); }
+SL_DEV uint32_t tagged(float v, uint32_t tag) { return (uint32_t)f2h(v) | (tag << 16); }
+SL_DEV bool tag_ok(uint32_t w, uint32_t tag) { return (w >> 16) == tag; }
+
+SL_DEV uint32_t ldw1(rsrc_t r, int idx) { return __builtin_amdgcn_raw_buffer_load_b32(r, idx * 4, 0, CO_SC1); }
+SL_DEV uint2 ldw2(rsrc_t r, int idx) { const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, idx * 4, 0, CO_SC1); return make_uint2(v.x, v.y); }
+SL_DEV uint4 ldw4(rsrc_t r, int idx) { const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, idx * 4, 0, CO_SC1); return make_uint4(v.x, v.y, v.z, v.w); }
+SL_DEV void stw1(rsrc_t r, int idx, uint32_t w) { __builtin_amdgcn_raw_buffer_store_b32(w, r, idx * 4, 0, CO_SC1); }
+SL_DEV void stw2(rsrc_t r, int idx, uint32_t a, uint32_t b) {
+  u32x2_t v; v.x = a; v.y = b;
+  __builtin_amdgcn_raw_buffer_store_b64(v, r, idx * 4, 0, CO_SC1);
+}
+SL_DEV void stw4(rsrc_t r, int idx, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  u32x4_t v; v.x = a; v.y = b; v.z = c; v.w = d;
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, idx * 4, 0, CO_SC1);
+}
+
+// Diagnostic clock stamps (100 MHz) of workgroups 0 and 100: (clock << 16) | id << 8 | min(v, 255).
+SL_DEV void fstamp(const DecodeP& P, unsigned id, unsigned v) {
+  if (uni(P.tstamp) && threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == 100)) {
+    const int n = g_L.bar.nts;
+    if (n < 2040) { uni(P.tstamp)[(blockIdx.x ? 2048 : 0) + 1 + n] = ((unsigned long long)wall_clock64() << 16) | (id << 8) | (v > 255u ? 255u : v); g_L.bar.nts = n + 1; }
+  }
+}
+// One polling round's verdict for the whole workgroup.  Returns 1 = all tags present, 0 = retry,
+// -1 = give up (spin limit reached here, or another workgroup raised the abort word).
+SL_DEV int flow_round(bool ok, unsigned& spins, unsigned* abort_word) {
+  if (__syncthreads_and(ok ? 1 : 0)) return 1;
+  ++spins;
+  int stop = 0;
+  if (threadIdx.x == 0 && (spins > FLOW_SPIN_LIMIT || ((spins & 255u) == 0 && ld_co32(abort_word) != 0))) {
+    st_co32(abort_word, 1u);
+    stop = 1;
+  }
+  if (__syncthreads_or(stop)) return -1;
+  __builtin_amdgcn_s_sleep(1);
+  return 0;
+}
+
+// Prologue on the whole workgroup: thread t owns elements 2t, 2t+1 of the hidden row.
+//   h' = half(h + r); x = w * half(h' * inv_rms(h')) -> packed into LDS with the word sums.
+// Sum of squares keeps the canonical order: wave 0, lane l chains its 32 contiguous elements.
+SL_DEV void flow_prologue(float h0, float h1, bool has_r, float r0, float r1, uint32_t lnw_pair, bool writer,
+                          rsrc_t h_out, uint32_t tag_out, uint16_t* xn_plain) {
+  const int tid = fresh_v(threadIdx.x), lane = tid & 63, wave = tid >> 6;
+  uint32_t* hs = reinterpret_cast<uint32_t*>(g_L.sq);          // 1024 words of scratch (attention's query area)
+  if (has_r) { h0 = f16r(h0 + r0); h1 = f16r(h1 + r1); }
+  hs[tid + (tid >> 4)] = pack2(h0, h1);       // 17-word lane stride: conflict-free for the chain below
+  if (writer) stw2(h_out, 2 * tid, tagged(h0, tag_out), tagged(h1, tag_out));
+  __syncthreads();
+  if (wave == 0) {
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const uint32_t w = hs[17 * lane + i];
+      const float a = lo_h(w), b = hi_h(w);
+      ss = fmaf(a, a, ss);
+      ss = fmaf(b, b, ss);
+    }
+    ss = tree_sum<64>(ss);
+    if (lane == 0) g_L.gb[0] = 1.0f / sqrtf(ss / 2048.0f + EPS);
+  }
+  __syncthreads();
+  const float inv = g_L.gb[0];
+  const float y0 = f16r(lo_h(lnw_pair) * f16r(h0 * inv)), y1 = f16r(hi_h(lnw_pair) * f16r(h1 * inv));
+  g_L.xs[(tid & 15) * 64 + (tid >> 4)] = pack2(y0, y1);
+  // left-to-right sum over each word of 8 elements = 4 consecutive threads
+  const int q = tid & 3;
+  float s = (0.0f + y0) + y1;
+#pragma unroll
+  for (int r = 1; r < 4; ++r) {
+    const float v = __shfl_up(s, 1, 64);
+    if (q == r) s = (v + y0) + y1;
+  }
+  if (q == 3) g_L.sxs[((tid & 15) >> 2) * 64 + (tid >> 4)] = s;
+  if (writer && xn_plain) *reinterpret_cast<uint32_t*>(xn_plain + 2 * tid) = pack2(y0, y1);
+  __syncthreads();
+}
+
+#define FLOW_IDS const int tid = fresh_v(threadIdx.x), lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); \
+                 const int wg = fresh_s(blockIdx.x), G = fresh_s(gridDim.x), NW = G * DEC_WAVES, gw = wg * DEC_WAVES + wave; \
+                 (void)tid; (void)lane; (void)wave; (void)wg; (void)G; (void)NW; (void)gw
+
+// ---- stage 1: input norm + in-projection ------------------------------------------------------------
+SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base) {
+  FLOW_IDS;
+  const DecodeP& P = F.d;
+  const int N = uni(Y.is_linear) ? SL_GDN_IN_N : SL_ATT_QKV_N;
+  WRegs<1, 4> wr;
+  bool valid[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    valid[j] = gw + j * NW < N;
+    wload_row<1>(wr.w[j], wr.sb[j], uni(Y.in_w), uni(Y.in_sb), (size_t)(valid[j] ? gw + j * NW : 0), valid[j], lane);
+  }
+  const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.input_ln) + 2 * tid);
+  // first touches of the next stage: this workgroup's recurrent-state rows, or its key/value tile
+  if (uni(Y.is_linear)) {
+    if (wg < 256 && wave < 8) {
+      const int hv = wg >> 3, dvb = wg & 7, par = (int)((uni(g_K.parity) >> li) & 1ull);
+      l2_touch(uni(Y.state[par]) + ((size_t)hv * 128 + dvb * 16 + wave * 2) * 128, 8, lane);
+    }
+  } else {
+    const int nt = (pos + SDPA_TILE) / SDPA_TILE;
+    if (wg < nt * SL_ATT_KV) {
+      const int tile = wg >> 1, kvh = wg & 1;
+      const int row = tile * SDPA_TILE + wave * 4 + (lane >> 2);
+      if (lane < 16 && row < pos) {
+        const size_t off = ((size_t)kvh * uni(P.max_seq) + row) * 256 + (size_t)(lane & 3) * 64;
+        (void)*reinterpret_cast<const volatile uint32_t*>(uni(Y.kcache) + off);
+        (void)*reinterpret_cast<const volatile uint32_t*>(uni(Y.vcache) + off);
+      }
+    }
+  }
+  float h0, h1, r0 = 0.0f, r1 = 0.0f;
+  if (li == 0) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(uni(P.hA) + 2 * tid);   // embedded row from k_embed
+    h0 = lo_h(w); h1 = hi_h(w);
+  } else {
+    const uint32_t th = flow_tag(base, li - 1, FS_A), tr = flow_tag(base, li - 1, FS_C);
+    const rsrc_t rh = co_rsrc(uni(F.th[0])), rr = co_rsrc(uni(F.tmoe));
+    unsigned spins = 0;
+    fstamp(P, 0, 0);
+    for (;;) {
+      const uint2 a = ldw2(rh, 2 * tid), b = ldw2(rr, 2 * tid);
+      const bool ok = tag_ok(a.x, th) && tag_ok(a.y, th) && tag_ok(b.x, tr) && tag_ok(b.y, tr);
+      h0 = lo_h(a.x); h1 = lo_h(a.y); r0 = lo_h(b.x); r1 = lo_h(b.y);
+      const int v = flow_round(ok, spins, uni(P.bar) + 32);
+      if (v > 0) break;
+      if (v < 0) return false;
+    }
+    fstamp(P, 1, spins);
+  }
+  const uint32_t tin = flow_tag(base, li, FS_IN);
+  flow_prologue(h0, h1, li > 0, r0, r1, lnw, wg == 0, co_rsrc(uni(F.th[1])), tin, nullptr);
+  const F4 o = dot_1x4(wr);
+  if (lane == 0) {
+    const rsrc_t rp = co_rsrc(uni(F.tproj));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) if (valid[j]) stw1(rp, gw + j * NW, tagged(o.v[j], tin));
+  }
+  return true;
+}
+
+// ---- GDN stage 2: conv + prep + gated delta rule ------------------------------------------------------
+SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
+  FLOW_IDS;
+  const DecodeP& P = F.d;
+  Lds& L = g_L;
+  if (wg >= 256) return true;
+  const int par = (int)((uni(g_K.parity) >> li) & 1ull);
+  const uint16_t* hin = uni(Y.hist[par]);
+  uint16_t* hout = uni(Y.hist[par ^ 1]);
+  const int hv = wg >> 3, dvb = wg & 7, hk = hv >> 1;
+  const int half = lane >> 5, l32 = lane & 31;
+  float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (wave < 8) {
+    const int dv = dvb * 16 + wave * 2 + half;
+    const float4 v4 = *reinterpret_cast<const float4*>(uni(Y.state[par]) + ((size_t)hv * 128 + dv) * 128 + 4 * l32);
+    s[0] = v4.x; s[1] = v4.y; s[2] = v4.z; s[3] = v4.w;
+  }
+  int ch = -1;
+  if (tid < 128) ch = hk * 128 + tid;
+  else if (tid < 256) ch = 2048 + hk * 128 + (tid - 128);
+  else if (tid < 272) ch = 4096 + hv * 128 + dvb * 16 + (tid - 256);
+  else if (tid == 272) ch = 12288 + hv;       // beta logit
+  else if (tid == 273) ch = 12320 + hv;       // decay logit
+  float tap[3] = {0.0f, 0.0f, 0.0f}, cw[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (tid < 272) {
+#pragma unroll
+    for (int k = 0; k < 3; ++k) tap[k] = h2f(hin[k * SL_CONV_DIM + ch]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) cw[k] = uni(Y.conv_w)[ch * 4 + k];
+  }
+  {
+    const size_t orow[1] = {(size_t)(gw < H ? gw : 0)}; const bool ov[1] = {gw < H};
+    l2_touch_rows<2>(uni(Y.out_w), uni(Y.out_sb), orow, ov, 1, lane);
+  }
+  float newest = 0.0f;
+  {
+    const uint32_t tin = flow_tag(base, li, FS_IN);
+    const rsrc_t rp = co_rsrc(uni(F.tproj));
+    unsigned spins = 0;
+    fstamp(P, 2, 0);
+    for (;;) {
+      bool ok = true;
+      if (ch >= 0) { const uint32_t w = ldw1(rp, ch); ok = tag_ok(w, tin); newest = lo_h(w); }
+      const int v = flow_round(ok, spins, uni(P.bar) + 32);
+      if (v > 0) break;
+      if (v < 0) return false;
+    }
+    fstamp(P, 3, spins);
+  }
+  if (tid < 272) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) acc = fmaf(tap[k], cw[k], acc);
+    acc = fmaf(newest, cw[3], acc);
+    const float c = f16r(acc * sigmoid32(acc));
+    if (tid < 128) L.q[tid] = c; else if (tid < 256) L.k[tid - 128] = c; else L.v[tid - 256] = c;
+  } else if (tid == 272) {
+    L.gb[1] = sigmoid16(newest);
+  } else if (tid == 273) {
+    L.gb[0] = exp_c(-(exp_c(uni(Y.a_log)[hv]) * softplus_c(newest + uni(Y.dt_bias)[hv])));
+  }
+  __syncthreads();
+  if (wave < 2) {
+    float* buf = wave ? L.k : L.q;
+    const float x0 = buf[2 * lane], x1 = buf[2 * lane + 1];
+    float ss = fmaf(x1, x1, fmaf(x0, x0, 0.0f));
+    ss = tree_sum<64>(ss);
+    const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
+    const float sc = wave ? f16r(0.08838834764831845f) : f16r(0.0078125f);
+    const float y0 = f16r(sc * f16r(x0 * inv)), y1 = f16r(sc * f16r(x1 * inv));
+    buf[2 * lane] = y0; buf[2 * lane + 1] = y1;
+  }
+  __syncthreads();
+  if (wave < 8) {
+    const float g = L.gb[0], beta = L.gb[1];
+    const int dvl = wave * 2 + half;
+    float kk[4], qq[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { kk[i] = L.k[4 * l32 + i]; qq[i] = L.q[4 * l32 + i]; }
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { s[i] = s[i] * g; acc = fmaf(s[i], kk[i], acc); }
+    const float kv = tree_sum<32>(acc);
+    const float delta = (L.v[dvl] - kv) * beta;
+    acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { s[i] = fmaf(kk[i], delta, s[i]); acc = fmaf(s[i], qq[i], acc); }
+    const float y = tree_sum<32>(acc);
+    const int dv = dvb * 16 + dvl;
+    if (l32 == 0) stw1(co_rsrc(uni(F.tycore)), hv * 128 + dv, tagged(y, flow_tag(base, li, FS_CORE)));
+    *reinterpret_cast<float4*>(uni(Y.state[par ^ 1]) + ((size_t)hv * 128 + dv) * 128 + 4 * l32) = make_float4(s[0], s[1], s[2], s[3]);
+  }
+  if (tid < 272 && (tid >= 256 || ((hv & 1) == 0 && dvb == 0))) {
+    hout[ch] = f2h(tap[1]);
+    hout[SL_CONV_DIM + ch] = f2h(tap[2]);
+    hout[2 * SL_CONV_DIM + ch] = f2h(newest);
+  }
+  __syncthreads();
+  return true;
+}
+
+// ---- attention stage 2: q/k prep, KV append, tile pass ---------------------------------------------------
+SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base) {
+  FLOW_IDS;
+  const DecodeP& P = F.d;
+  Lds& L = g_L;
+  const float NEG = -__int_as_float(0x7f800000);
+  const int N = pos + 1, nt = (N + SDPA_TILE - 1) / SDPA_TILE;
+  {
+    const size_t orow[1] = {(size_t)(gw < H ? gw : 0)}; const bool ov[1] = {gw < H};
+    l2_touch_rows<2>(uni(Y.out_w), uni(Y.out_sb), orow, ov, 1, lane);
+  }
+  const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag32(base, li, FS_CORE);
+  for (int u = wg; u < nt * SL_ATT_KV; u += G) {
+    const int tile = u >> 1, kvh = u & 1;
+    const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
+    const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
+    const uint16_t* kbase = uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + j0) * 256;
+    const uint16_t* vbase = uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + j0) * 256;
+    __syncthreads();                    // the key tile aliases the activation vector the in-projection just read
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int row = it * 32 + (tid >> 5), c8 = (tid & 31) * 8;
+      if (row < nk && j0 + row != pos) {
+        st16(&L.kt[row * KT_STRIDE + c8], ld16(kbase + (size_t)row * 256 + c8));
+        st16(&g_vt[row * 256 + c8], ld16(vbase + (size_t)row * 256 + c8));
+      }
+    }
+    // waves 0..7: query heads of the group; wave 8: new key; wave 9: new value -- 4 tagged words per lane
+    const int src = wave < 8 ? (kvh * 8 + wave) * 512 : (wave == 8 ? 8192 + kvh * 256 : 8192 + 512 + kvh * 256);
+    uint4 w4 = make_uint4(0, 0, 0, 0);
+    {
+      const rsrc_t rp = co_rsrc(uni(F.tproj));
+      unsigned spins = 0;
+    fstamp(P, 4, 0);
+      for (;;) {
+        bool ok = true;
+        if (wave < 10) { w4 = ldw4(rp, src + 4 * lane); ok = tag_ok(w4.x, tin) && tag_ok(w4.y, tin) && tag_ok(w4.z, tin) && tag_ok(w4.w, tin); }
+        const int v = flow_round(ok, spins, uni(P.bar) + 32);
+        if (v > 0) break;
+        if (v < 0) return false;
+      }
+      fstamp(P, 5, spins);
+    }
+    if (wave < 9) {
+      const bool isq = wave < 8;
+      const uint16_t* nwp = isq ? uni(Y.q_norm) : uni(Y.k_norm);
+      const float xv[4] = {lo_h(w4.x), lo_h(w4.y), lo_h(w4.z), lo_h(w4.w)};
+      float wv[4];
+      const uint2 wraw = *reinterpret_cast<const uint2*>(nwp + 4 * lane);
+      wv[0] = lo_h(wraw.x); wv[1] = hi_h(wraw.x); wv[2] = lo_h(wraw.y); wv[3] = hi_h(wraw.y);
+      float ss = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ss = fmaf(xv[i], xv[i], ss);
+      ss = tree_sum<64>(ss);
+      const float inv = 1.0f / sqrtf(ss / 256.0f + EPS);
+      float* dst = isq ? &L.sq[wave * 256] : L.knew;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dst[4 * lane + i] = f16r(wv[i] * f16r(xv[i] * inv));
+      float o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = dst[4 * lane + i];
+      if (lane < 16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int d = 4 * lane + i, ii = d & 31;
+          const float c = uni(P.rope_cos)[(size_t)pos * 32 + ii], sn = uni(P.rope_sin)[(size_t)pos * 32 + ii];
+          const float x0 = dst[ii], x1 = dst[ii + 32];
+          o[i] = (d < 32) ? f16r(fmaf(-x1, sn, x0 * c)) : f16r(fmaf(x1, c, x0 * sn));
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dst[4 * lane + i] = isq ? 0.0625f * o[i] : o[i];
+      if (!isq && has_new) {
+        st_co_h4(co_rsrc(uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 4 * lane, o);
+        *reinterpret_cast<uint2*>(&L.kt[(pos - j0) * KT_STRIDE + 4 * lane]) = make_uint2(pack2(o[0], o[1]), pack2(o[2], o[3]));
+      }
+    } else if (wave == 9 && has_new) {
+      const uint32_t a = (w4.x & 0xffffu) | (w4.y << 16), b = (w4.z & 0xffffu) | (w4.w << 16);
+      stw2(co_rsrc(uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 2 * lane, a, b);
+      *reinterpret_cast<uint2*>(&g_vt[(pos - j0) * 256 + 4 * lane]) = make_uint2(a, b);
+    }
+    __syncthreads();
+    {
+      const int h = wave >> 1, half = wave & 1;
+      const uint16_t* kr = &L.kt[(lane < nk ? lane : 0) * KT_STRIDE + 128 * half];
+      const float* qh = &L.sq[h * 256 + 128 * half];
+      const float g0 = score_leaf8(kr, qh), g1 = score_leaf8(kr + 32, qh + 32);
+      const float g2 = score_leaf8(kr + 64, qh + 64), g3 = score_leaf8(kr + 96, qh + 96);
+      L.part[wave * 64 + lane] = (g0 + g1) + (g2 + g3);
+    }
+    __syncthreads();
+    if ((wave & 1) == 0) {
+      const int h = wave >> 1;
+      const float dotv = L.part[wave * 64 + lane] + L.part[(wave + 1) * 64 + lane];
+      const float sc = (lane < nk) ? dotv : NEG;
+      const float mx = tree_max<64>(sc);
+      const float p = (lane < nk) ? exp_c(sc - mx) : 0.0f;
+      const float l = tree_sum<64>(p);
+      L.sm[h * 64 + lane] = p;
+      const int head = kvh * 8 + h;
+      if (lane == 0) stw4(co_rsrc(uni(F.tml)), (head * uni(P.max_tiles) + tile) * 4, __float_as_uint(mx), __float_as_uint(l), tcore, tcore);
+    }
+    __syncthreads();
+    {
+      const int h = wave >> 1, half = wave & 1;
+      float o0 = 0.0f, o1 = 0.0f;
+      const uint16_t* vt = &g_vt[128 * half + 2 * lane];
+      const float* pw = &L.sm[h * 64];
+      for (int j = 0; j < nk; ++j) {
+        const uint32_t vv = *reinterpret_cast<const uint32_t*>(vt + j * 256);
+        const float pj = pw[j];
+        o0 = fmaf(pj, lo_h(vv), o0);
+        o1 = fmaf(pj, hi_h(vv), o1);
+      }
+      const int head = kvh * 8 + h;
+      stw4(co_rsrc(uni(F.tpo)), ((head * uni(P.max_tiles) + tile) * 128 + 64 * half + lane) * 4, __float_as_uint(o0), __float_as_uint(o1), tcore, tcore);
+    }
+    __syncthreads();
+  }
+  return true;
+}
+
+// ---- K = 4096 projection (GDN out_proj with gated rmsnorm prologue / attention merge + o_proj) ---------
+SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t base) {
+  FLOW_IDS;
+  const DecodeP& P = F.d;
+  const bool lin = uni(Y.is_linear) != 0;
+  const float NEG = -__int_as_float(0x7f800000);
+  WRegs<2, 1> wr;
+  const bool valid = gw < H;
+  wload_row<2>(wr.w[0], wr.sb[0], uni(Y.out_w), uni(Y.out_sb), (size_t)(valid ? gw : 0), valid, lane);
+  if (gw <= uni(P.E)) l2_touch((gw < uni(P.E) ? uni(Y.router_w) + (size_t)gw * H : uni(Y.sgate_w)), 32, lane);
+  if (gw >= 512 && gw < 1024) {
+    const size_t pr[1] = {(size_t)(gw - 512)}; const bool pv[1] = {true};
+    l2_touch_rows<1>(uni(Y.shg_w), uni(Y.shg_sb), pr, pv, 1, lane);
+    l2_touch_rows<1>(uni(Y.shu_w), uni(Y.shu_sb), pr, pv, 1, lane);
+  }
+  const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
+  const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
+  if (!lin && wg == 0) {
+    // merge the attention tiles of head `wave` in order with the global max (each wave polls on its own)
+    const int h = wave, slot0 = h * uni(P.max_tiles);
+    const rsrc_t rml = co_rsrc(uni(F.tml)), rpo = co_rsrc(uni(F.tpo));
+    int fail = 0;
+    float Mx = NEG;
+    for (int t = 0; t < nt && !fail; ++t) {
+      unsigned spins = 0;
+      for (;;) {
+        const uint4 m = ldw4(rml, (slot0 + t) * 4);
+        if (m.z == tcore32 && m.w == tcore32) { Mx = fmaxf(Mx, __uint_as_float(m.x)); break; }
+        if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+        __builtin_amdgcn_s_sleep(1);
+      }
+    }
+    float Ls = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int t = 0; t < nt && !fail; ++t) {
+      const uint4 m = ldw4(rml, (slot0 + t) * 4);          // tags verified above
+      const float f = exp_c(__uint_as_float(m.x) - Mx);
+      Ls = fmaf(__uint_as_float(m.y), f, Ls);
+      unsigned spins = 0;
+      for (;;) {
+        const uint4 a = ldw4(rpo, ((slot0 + t) * 128 + 2 * lane) * 4), b = ldw4(rpo, ((slot0 + t) * 128 + 2 * lane + 1) * 4);
+        const bool ok = a.z == tcore32 && a.w == tcore32 && b.z == tcore32 && b.w == tcore32;
+        if (__all(ok ? 1 : 0)) {
+          O[0] = fmaf(__uint_as_float(a.x), f, O[0]); O[1] = fmaf(__uint_as_float(a.y), f, O[1]);
+          O[2] = fmaf(__uint_as_float(b.x), f, O[2]); O[3] = fmaf(__uint_as_float(b.y), f, O[3]);
+          break;
+        }
+        if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+        __builtin_amdgcn_s_sleep(1);
+      }
+    }
+    // the output gate sits in the q projection of this step
+    const rsrc_t rp = co_rsrc(uni(F.tproj));
+    uint4 g4 = make_uint4(0, 0, 0, 0);
+    for (unsigned spins = 0; !fail;) {
+      g4 = ldw4(rp, h * 512 + 256 + 4 * lane);
+      if (__all((tag_ok(g4.x, tin) && tag_ok(g4.y, tin) && tag_ok(g4.z, tin) && tag_ok(g4.w, tin)) ? 1 : 0)) break;
+      if (++spins > FLOW_SPIN_LIMIT) fail = 1;
+    }
+    if (fail) st_co32(uni(P.bar) + 32, 1u);
+    const float gt[4] = {lo_h(g4.x), lo_h(g4.y), lo_h(g4.z), lo_h(g4.w)};
+    uint32_t r[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = tagged(f16r(f16r(O[i] / Ls) * sigmoid16(gt[i])), tmerge);
+    if (!fail) stw4(co_rsrc(uni(F.tycore)), h * 256 + 4 * lane, r[0], r[1], r[2], r[3]);
+  }
+  // every thread prepares 4 consecutive elements of the 4096-long activation
+  const int e0 = 256 * wave + 4 * lane;
+  float out[4], z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  {
+    const uint32_t ty = lin ? tcore : tmerge;
+    const rsrc_t ry = co_rsrc(uni(F.tycore)), rz = co_rsrc(uni(F.tproj));
+    unsigned spins = 0;
+    fstamp(P, 6, 0);
+    for (;;) {
+      const uint4 a = ldw4(ry, e0);
+      bool ok = tag_ok(a.x, ty) && tag_ok(a.y, ty) && tag_ok(a.z, ty) && tag_ok(a.w, ty);
+      out[0] = lo_h(a.x); out[1] = lo_h(a.y); out[2] = lo_h(a.z); out[3] = lo_h(a.w);
+      if (lin) {
+        const uint4 b = ldw4(rz, 8192 + e0);
+        ok = ok && tag_ok(b.x, tin) && tag_ok(b.y, tin) && tag_ok(b.z, tin) && tag_ok(b.w, tin);
+        z[0] = lo_h(b.x); z[1] = lo_h(b.y); z[2] = lo_h(b.z); z[3] = lo_h(b.w);
+      }
+      const int v = flow_round(ok, spins, uni(P.bar) + 32);
+      if (v > 0) break;
+      if (v < 0) return false;
+    }
+    fstamp(P, 7, spins);
+  }
+  if (lin) {
+    float nw[4];
+    const uint2 wraw = *reinterpret_cast<const uint2*>(uni(Y.gdn_norm_w) + (e0 & 127));
+    nw[0] = lo_h(wraw.x); nw[1] = hi_h(wraw.x); nw[2] = lo_h(wraw.y); nw[3] = hi_h(wraw.y);
+    const float la = fmaf(out[1], out[1], fmaf(out[0], out[0], 0.0f));
+    const float lb = fmaf(out[3], out[3], fmaf(out[2], out[2], 0.0f));
+    const float ss = tree_sum<32>(la + lb);
+    const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float nrm = f16r(nw[i] * f16r(out[i] * inv));
+      out[i] = f16r((z[i] * sigmoid32(z[i])) * nrm);
+    }
+  }
+  {
+    const int b = e0 >> 11, r = e0 & 2047, lo = r >> 5, i0 = r & 31;
+    g_L.xs[(16 * b + (i0 >> 1)) * 64 + lo] = pack2(out[0], out[1]);
+    g_L.xs[(16 * b + (i0 >> 1) + 1) * 64 + lo] = pack2(out[2], out[3]);
+    float sfirst = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sfirst = sfirst + out[i];
+    float srest = __shfl_up(sfirst, 1, 64);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) srest = srest + out[i];
+    if (lane & 1) g_L.sxs[(4 * b + (i0 >> 3)) * 64 + lo] = srest;
+  }
+  __syncthreads();
+  const float o = dot_2x1(wr);
+  if (lane == 0 && valid) stw1(co_rsrc(uni(F.tmix)), gw, tagged(o, flow_tag(base, li, FS_OUT)));
+  return true;
+}
+
+// ---- MoE stage A -------------------------------------------------------------------------------------
+SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
+  FLOW_IDS;
+  const DecodeP& P = F.d;
+  const bool is_dense = gw <= uni(P.E);
+  const bool is_pair = gw >= 512 && gw < 1024;
+  float dw[32];
+  WRegs<1, 2> wr;
+  const size_t prow = is_pair ? (size_t)(gw - 512) : 0;
+  wload_row<1>(wr.w[0], wr.sb[0], uni(Y.shg_w), uni(Y.shg_sb), prow, is_pair, lane);
+  wload_row<1>(wr.w[1], wr.sb[1], uni(Y.shu_w), uni(Y.shu_sb), prow, is_pair, lane);
+  if (is_dense) load32((gw < uni(P.E) ? uni(Y.router_w) + (size_t)gw * H : uni(Y.sgate_w)) + 32 * lane, dw);
+  const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.post_ln) + 2 * tid);
+  float h0, h1, r0, r1;
+  {
+    const uint32_t th = flow_tag(base, li, FS_IN), tr = flow_tag(base, li, FS_OUT);
+    const rsrc_t rh = co_rsrc(uni(F.th[1])), rr = co_rsrc(uni(F.tmix));
+    unsigned spins = 0;
+    fstamp(P, 8, 0);
+    for (;;) {
+      const uint2 a = ldw2(rh, 2 * tid), b = ldw2(rr, 2 * tid);
+      const bool ok = tag_ok(a.x, th) && tag_ok(a.y, th) && tag_ok(b.x, tr) && tag_ok(b.y, tr);
+      h0 = lo_h(a.x); h1 = lo_h(a.y); r0 = lo_h(b.x); r1 = lo_h(b.y);
+      const int v = flow_round(ok, spins, uni(P.bar) + 32);
+      if (v > 0) break;
+      if (v < 0) return false;
+    }
+    fstamp(P, 9, spins);
+  }
+  const uint32_t ta = flow_tag(base, li, FS_A);
+  flow_prologue(h0, h1, true, r0, r1, lnw, wg == 0, co_rsrc(uni(F.th[0])), ta, nullptr);
+  if (is_dense) {
+    uint32_t xp[16]; float sx[4];
+    lds_get_x(0, lane, xp, sx);
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { acc = fmaf(lo_h(xp[i]), dw[2 * i], acc); acc = fmaf(hi_h(xp[i]), dw[2 * i + 1], acc); }
+    acc = tree_sum<64>(acc);
+    if (lane == 0) { if (gw < uni(P.E)) stw1(co_rsrc(uni(F.trlog)), gw, tagged(acc, ta)); else stw1(co_rsrc(uni(F.tsg)), 0, tagged(acc, ta)); }
+  }
+  if (is_pair) {
+    const F2 gu = dot_1x2(wr);
+    if (lane == 0) stw1(co_rsrc(uni(F.tsh)), (int)prow, tagged(swiglu16(f16r(gu.v[0]), f16r(gu.v[1])), ta));
+  }
+  return true;
+}
+
+// ---- MoE stage B: routing + routed gate/up + SwiGLU -------------------------------------------------------
+SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
+  FLOW_IDS;
+  const DecodeP& P = F.d;
+  Lds& L = g_L;
+  const float NEG = -__int_as_float(0x7f800000);
+  float* lg = L.part;
+  float* ex = L.part + 256;
+  int* cnt = reinterpret_cast<int*>(g_vt);
+  // Non-finite logits rank no expert below 8; the slots then keep these in-range defaults.
+  if (tid < 8) { L.inds[tid] = tid; L.scores[tid] = 0.0f; }
+  {
+    const uint32_t ta = flow_tag(base, li, FS_A);
+    const rsrc_t rl = co_rsrc(uni(F.trlog));
+    unsigned spins = 0;
+    fstamp(P, 10, 0);
+    for (;;) {
+      bool ok = true;
+      float v0 = NEG;
+      if (tid < uni(P.E)) { const uint32_t w = ldw1(rl, tid); ok = tag_ok(w, ta); v0 = lo_h(w); }
+      if (tid < 256) lg[tid] = v0;
+      const int v = flow_round(ok, spins, uni(P.bar) + 32);
+      if (v > 0) break;
+      if (v < 0) return false;
+    }
+    fstamp(P, 11, spins);
+  }
+  {
+    const int e = tid & 255, part = tid >> 8;
+    const float me = lg[e];
+    int c = 0;
+#pragma unroll 8
+    for (int j = 64 * part; j < 64 * part + 64; ++j) {
+      const float o = lg[j];
+      c += (o > me || (o == me && j < e)) ? 1 : 0;
+    }
+    cnt[part * 256 + e] = c;
+  }
+  if (wave == 0) {
+    float v[4], x4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = lg[4 * lane + i];
+    const float mx = tree_max<64>(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { x4[i] = (4 * lane + i < uni(P.E)) ? exp_c(v[i] - mx) : 0.0f; ex[4 * lane + i] = x4[i]; }
+    const float Z = tree_sum<64>(((x4[0] + x4[1]) + x4[2]) + x4[3]);
+    if (lane == 0) L.gb[0] = Z;
+  }
+  __syncthreads();
+  if (tid < 256) {
+    const int rank = cnt[tid] + cnt[256 + tid] + cnt[512 + tid] + cnt[768 + tid];
+    if (rank < 8 && tid < uni(P.E)) { L.inds[rank] = tid; L.scores[rank] = f16r(ex[tid] / L.gb[0]); }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float ss = 0.0f;
+    for (int k = 0; k < 8; ++k) ss = f16r(ss + L.scores[k]);
+    for (int k = 0; k < 8; ++k) L.scores[k] = f16r(L.scores[k] / ss);
+    if (wg == 0) for (int k = 0; k < 8; ++k) { uni(Y.route_inds)[k] = L.inds[k]; uni(Y.route_scores)[k] = f2h(L.scores[k]); }
+  }
+  const int p = gw;
+  WRegs<1, 2> wr;
+  int k = 0, i = 0;
+  const bool active = p < 8 * 512;
+  if (active) {
+    k = p >> 9; i = p & 511;
+    const size_t row = (size_t)L.inds[k] * 512 + i;
+    wload_row<1>(wr.w[0], wr.sb[0], uni(Y.swg_w), uni(Y.swg_sb), row, true, lane);
+    wload_row<1>(wr.w[1], wr.sb[1], uni(Y.swu_w), uni(Y.swu_sb), row, true, lane);
+  }
+#pragma unroll
+  for (int qq = 0; qq < 2; ++qq) {
+    const int un = wave + 16 * qq, ql = un / 9, slot = un % 9;
+    if (ql < 2 && slot < 8) {
+      const size_t row = (size_t)L.inds[slot] * 2048 + (size_t)(wg * 2 + ql) * 4;
+      l2_touch(uni(Y.swd_w) + row * 64, 8, lane);
+      if (lane == 8) (void)*reinterpret_cast<const volatile uint32_t*>(uni(Y.swd_sb) + row * 8);
+    }
+  }
+  __syncthreads();
+  if (active) {
+    const F2 gu = dot_1x2(wr);
+    if (lane == 0) stw1(co_rsrc(uni(F.tact)), k * 512 + i, tagged(swiglu16(f16r(gu.v[0]), f16r(gu.v[1])), flow_tag(base, li, FS_B)));
+  }
+  return true;
+}
+
+// ---- MoE stage C: down-projections, half combine, gated shared add ---------------------------------------
+SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, const uint32_t* next_w, const uint32_t* next_sb,
+                       int next_n, int next_contig) {
+  FLOW_IDS;
+  const DecodeP& P = F.d;
+  Lds& L = g_L;
+  const int sub = lane >> 4, li16 = lane & 15;
+  {
+    size_t rows[4]; bool rv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const long r = next_contig ? (long)gw * 64 + j : (long)gw + (long)j * NW;
+      rv[j] = r < next_n; rows[j] = rv[j] ? (size_t)r : 0;
+    }
+    l2_touch_rows<1>(next_w, next_sb, rows, rv, 4, lane);
+  }
+  const uint32_t ta = flow_tag(base, li, FS_A), tb = flow_tag(base, li, FS_B);
+  float sgate_logit = 0.0f;
+#pragma unroll
+  for (int qq = 0; qq < 2; ++qq) {
+    const int un = wave + 16 * qq, ql = un / 9, slot = un % 9;
+    const int quad = wg * 2 + ql;
+    const bool has = ql < 2;
+    uint4 wv = make_uint4(0, 0, 0, 0); uint32_t sbv = 0;
+    if (has) {
+      // the routed rows were touched into L2 during stage B; the shared rows do not depend on routing
+      const size_t row = (slot < 8 ? (size_t)L.inds[slot] * 2048 : 0) + (size_t)quad * 4 + sub;
+      const uint32_t* W = slot < 8 ? uni(Y.swd_w) : uni(Y.shd_w);
+      const uint32_t* SB = slot < 8 ? uni(Y.swd_sb) : uni(Y.shd_sb);
+      wv = ld16(W + row * 64 + 4 * li16);
+      sbv = SB[row * 8 + (li16 >> 1)];
+    }
+    float x[32];
+    {
+      const rsrc_t rx = co_rsrc(slot < 8 ? uni(F.tact) + slot * 512 : uni(F.tsh));
+      const uint32_t tx = slot < 8 ? tb : ta;
+      const rsrc_t rg = co_rsrc(uni(F.tsg));
+      unsigned spins = 0;
+    fstamp(P, 12, 0);
+      for (;;) {
+        bool ok = true;
+        if (has) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const uint4 w = ldw4(rx, 32 * li16 + 4 * j);
+            ok = ok && tag_ok(w.x, tx) && tag_ok(w.y, tx) && tag_ok(w.z, tx) && tag_ok(w.w, tx);
+            x[4 * j] = lo_h(w.x); x[4 * j + 1] = lo_h(w.y); x[4 * j + 2] = lo_h(w.z); x[4 * j + 3] = lo_h(w.w);
+          }
+        }
+        if (qq == 0 && tid < 8) { const uint32_t w = ldw1(rg, 0); ok = ok && tag_ok(w, ta); sgate_logit = lo_h(w); }
+        const int v = flow_round(ok, spins, uni(P.bar) + 32);
+        if (v > 0) break;
+        if (v < 0) return false;
+      }
+      fstamp(P, 13, spins);
+    }
+    if (has) {
+      float sx[4];
+      uint32_t xp[16];
+      word_sums(x, sx);
+      pack_x(x, xp);
+      const float d = tree_sum<16>(quad_term(wv, sbv, xp, sx));
+      if (li16 == 0) L.dbuf[(ql * 9 + slot) * 4 + sub] = f16r(d);
+    }
+  }
+  __syncthreads();
+  if (tid < 8) {
+    const int ql = tid >> 2, sb4 = tid & 3;
+    const int quad = wg * 2 + ql;
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc = f16r(acc + f16r(L.dbuf[(ql * 9 + k) * 4 + sb4] * L.scores[k]));
+    const float s = sigmoid16(sgate_logit);
+    stw1(co_rsrc(uni(F.tmoe)), quad * 4 + sb4, tagged(f16r(acc + f16r(s * L.dbuf[(ql * 9 + 8) * 4 + sb4])), flow_tag(base, li, FS_C)));
+  }
+  __syncthreads();
+  return true;
+}
+
+// ---- head -------------------------------------------------------------------------------------------
+SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t base) {
+  FLOW_IDS;
+  const DecodeP& P = F.d;
+  Lds& L = g_L;
+  const float NEG = -__int_as_float(0x7f800000);
+  const int nchunks = (uni(P.vocab) + 63) / 64;
+  const int nl = uni(P.n_layers);
+  float bv = NEG; int bi = 0x7fffffff;
+  WRegs<1, 4> cur, nxt;
+  auto load_group = [&](WRegs<1, 4>& r, int chunk, int g4) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const long row = (long)chunk * 64 + g4 * 4 + j;
+      const bool v = chunk < nchunks && row < uni(P.vocab);
+      wload_row<1>(r.w[j], r.sb[j], uni(P.lm_w), uni(P.lm_sb), (size_t)(v ? row : 0), v, lane);
+    }
+  };
+  load_group(cur, gw, 0);
+  const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(P.final_norm) + 2 * tid);
+  float h0, h1, r0, r1;
+  {
+    const uint32_t th = flow_tag(base, nl - 1, FS_A), tr = flow_tag(base, nl - 1, FS_C);
+    const rsrc_t rh = co_rsrc(uni(F.th[0])), rr = co_rsrc(uni(F.tmoe));
+    unsigned spins = 0;
+    fstamp(P, 14, 0);
+    for (;;) {
+      const uint2 a = ldw2(rh, 2 * tid), b = ldw2(rr, 2 * tid);
+      const bool ok = tag_ok(a.x, th) && tag_ok(a.y, th) && tag_ok(b.x, tr) && tag_ok(b.y, tr);
+      h0 = lo_h(a.x); h1 = lo_h(a.y); r0 = lo_h(b.x); r1 = lo_h(b.y);
+      const int v = flow_round(ok, spins, uni(P.bar) + 32);
+      if (v > 0) break;
+      if (v < 0) return false;
+    }
+    fstamp(P, 15, spins);
+  }
+  const uint32_t thd = flow_tag(base, nl, 0), thd32 = flow_tag32(base, nl, 0);
+  flow_prologue(h0, h1, true, r0, r1, lnw, wg == 0, co_rsrc(uni(F.th[1])), thd, uni(P.normed));
+  for (int chunk = gw; chunk < nchunks; chunk += NW) {
+#pragma unroll 1
+    for (int g4 = 0; g4 < 16; ++g4) {
+      int nchunk = chunk, ng = g4 + 1;
+      if (ng == 16) { ng = 0; nchunk = chunk + NW; }
+      load_group(nxt, nchunk, ng);
+      const F4 o = dot_1x4(cur);
+      const long r0w = (long)chunk * 64 + g4 * 4;
+      if (r0w < uni(P.vocab)) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float v = f16r(o.v[j]);
+          if (v > bv) { bv = v; bi = (int)(r0w + j); }
+        }
+        if (lane == 0) *reinterpret_cast<uint2*>(uni(P.logits) + r0w) = make_uint2(pack2(o.v[0], o.v[1]), pack2(o.v[2], o.v[3]));
+      }
+      cur = nxt;
+    }
+  }
+  if (lane == 0) { L.red[wave] = bv; L.ired[wave] = bi; }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < DEC_WAVES; ++w)
+      if (L.red[w] > bv || (L.red[w] == bv && L.ired[w] < bi)) { bv = L.red[w]; bi = L.ired[w]; }
+    stw4(co_rsrc(uni(F.tcand)), wg * 4, __float_as_uint(bv), (uint32_t)bi, thd32, thd32);
+  }
+  if (wg != 0) return true;
+  float v = NEG; int i = 0x7fffffff;
+  {
+    const rsrc_t rc = co_rsrc(uni(F.tcand));
+    unsigned spins = 0;
+    fstamp(P, 16, 0);
+    for (;;) {
+      bool ok = true;
+      if (tid < G) { const uint4 c = ldw4(rc, tid * 4); ok = c.z == thd32 && c.w == thd32; v = __uint_as_float(c.x); i = (int)c.y; }
+      const int r = flow_round(ok, spins, uni(P.bar) + 32);
+      if (r > 0) break;
+      if (r < 0) return false;
+    }
+    fstamp(P, 17, spins);
+  }
+#pragma unroll
+  for (int msk = 1; msk < 64; msk <<= 1) {
+    const float ov = __shfl_xor(v, msk, 64); const int oi = __shfl_xor(i, msk, 64);
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+  }
+  __syncthreads();
+  if (lane == 0) { L.red[wave] = v; L.ired[wave] = i; }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < DEC_WAVES; ++w)
+      if (L.red[w] > v || (L.red[w] == v && L.ired[w] < i)) { v = L.red[w]; i = L.ired[w]; }
+    uni(P.tok_out)[out_off] = i;
+    if (feed) uni(P.tok_in)[0] = i;
+    uni(P.st)[0] = pos + 1;
+    st_co32(uni(P.bar) + 16, base + (uint32_t)(nl + 1) * 8u);
+  }
+  for (int l = tid; l < nl; l += DEC_THREADS) uni(P.st)[1 + l] ^= 1;
+  return true;
+}
+
+// ---- the kernel: hA already holds the embedded token row (k_embed) --------------------------------------
+__global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __restrict__ Fp, int out_off, int feed) {
+  {
+    const int tid = threadIdx.x;
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(Fp);
+    uint32_t* dst = reinterpret_cast<uint32_t*>(&g_K.F);
+    for (int i = tid; i < (int)(sizeof(FlowP) / 4); i += DEC_THREADS) dst[i] = src[i];
+    const int nl = Fp->d.n_layers;
+    const uint32_t* lsrc = reinterpret_cast<const uint32_t*>(Fp->d.layers);
+    uint32_t* ldst = reinterpret_cast<uint32_t*>(g_K.layers);
+    for (int i = tid; i < nl * (int)(sizeof(LayerP) / 4); i += DEC_THREADS) ldst[i] = lsrc[i];
+    if (tid < 64) {
+      const int bit = (tid < nl) ? (Fp->d.st[1 + tid] & 1) : 0;
+      const unsigned long long m = __ballot(bit);
+      if (tid == 0) { g_K.parity = m; g_K.pos = Fp->d.st[0]; g_K.base = ld_co32(Fp->d.bar + 16); g_L.bar.nts = 0; }
+    }
+    __syncthreads();
+  }
+  const FlowP& F = g_K.F;
+  const DecodeP& P = F.d;
+  const uint32_t base = uni(g_K.base);
+  const int pos = uni(g_K.pos);
+  const int nl = uni(P.n_layers);
+  for (int li = 0; li < nl; ++li) {
+    const LayerP& Y = g_K.layers[li];
+    const int is_linear = uni(Y.is_linear);
+    if (!flow_in(F, Y, li, pos, base)) return;
+    if (is_linear) {
+      if (!flow_gdn(F, Y, li, base)) return;
+      if (!flow_out(F, Y, li, 0, base)) return;
+    } else {
+      if (!flow_sdpa(F, Y, li, pos, base)) return;
+      if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base)) return;
+    }
+    if (!flow_moe_a(F, Y, li, base)) return;
+    if (!flow_moe_b(F, Y, li, base)) return;
+    {
+      const bool last = li + 1 == nl;
+      const LayerP& Z = g_K.layers[last ? li : li + 1];
+      if (!flow_moe_c(F, Y, li, base, last ? uni(P.lm_w) : uni(Z.in_w), last ? uni(P.lm_sb) : uni(Z.in_sb),
+                      last ? uni(P.vocab) : (uni(Z.is_linear) ? SL_GDN_IN_N : SL_ATT_QKV_N), last ? 1 : 0)) return;
+    }
+  }
+  flow_head(F, pos, out_off, feed, base);
+  fstamp(P, 18, 0);
+  if (uni(P.tstamp) && threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == 100))
+    uni(P.tstamp)[blockIdx.x ? 2048 : 0] = (unsigned long long)g_L.bar.nts;
+}
+
+}  // namespace sl
