@@ -7,7 +7,7 @@ before the timed region; tokens feed back on the device in chains, as the refere
 decode does (chainedStepArgmax, K = 8).
 
 Prints one JSON line: throughput, the roofline of the dominant kernel (the persistent step kernel
-k_decode, which runs a whole token; timed with HIP events on the engine's stream), and the CPU
+k_decode_flow, which runs a whole token; timed with HIP events on the engine's stream), and the CPU
 baseline (the oracle, timed on this host's cores on a bounded sample of the same workload).
 """
 import argparse
@@ -22,8 +22,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 PROMPT_LEN = 512
-# HBM bytes per k_decode launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/), or None until measured
-TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per k_decode_flow launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/), or None until measured
+TRAFFIC_BYTES_PER_LAUNCH = 1950521354   # 2 x FETCH_SIZE (copy-calibrated) + WRITE_SIZE, in bytes, at context ~525
 
 
 def step_bytes(cfg, ctx):
@@ -145,7 +145,7 @@ def main():
         "config": {"workload": f"{cfg.n_layers}-layer 35B-A3B hybrid (3 GDN : 1 attention, 256-expert top-8 MoE + shared), "
                                f"vocab {cfg.vocab}, 4-bit g64; greedy decode after a {PROMPT_LEN}-token prompt, batch 1",
                    "chain_k": args.chain, "context": [PROMPT_LEN + args.warmup, PROMPT_LEN + args.warmup + args.steps]},
-        "roofline": {"bound": "hbm", "kernel": "k_decode (persistent batch-1 step: 40 layers + lm_head + argmax)",
+        "roofline": {"bound": "hbm", "kernel": "k_decode_flow (persistent batch-1 step: 40 layers + lm_head + argmax)",
                      "achieved": head_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head_gbs / HBM_PEAK_GBS,
                      "traffic": TRAFFIC_BYTES_PER_LAUNCH, "launches": head_n, "avg_ms": head_avg_ms, "bytes_per_launch": total_b},
         "step_hbm": {"bytes_per_token": total_b, "achieved_GBs": step_gbs, "frac_of_peak": step_gbs / HBM_PEAK_GBS},
