@@ -12,6 +12,7 @@
 //
 // Arithmetic, reduction order and work split are those of sl_decode.cuh / sl_kernels.cuh.
 #pragma once
+#include <type_traits>
 #include "sl_decode.cuh"
 
 namespace sl {
@@ -55,7 +56,15 @@ SL_DEV T uni(const T& r) {
     const uint2 v = *reinterpret_cast<const uint2*>(&r);
     const unsigned long long u = (unsigned long long)(uint32_t)__builtin_amdgcn_readfirstlane(v.x) |
                                  ((unsigned long long)(uint32_t)__builtin_amdgcn_readfirstlane(v.y) << 32);
-    return __builtin_bit_cast(T, u);
+    if constexpr (std::is_pointer<T>::value) {
+      // Every pointer parameter is device memory.  Saying so keeps accesses through it on the vector-memory
+      // counter only; a generic ("flat") access would also count as an LDS operation, and the next parameter
+      // read from LDS would then wait for it to come back from HBM.
+      typedef typename std::remove_pointer<T>::type E;
+      return (T)(E __attribute__((address_space(1)))*)u;
+    } else {
+      return __builtin_bit_cast(T, u);
+    }
   }
 }
 
@@ -65,6 +74,34 @@ SL_DEV T uni(const T& r) {
 // prefetch).
 SL_DEV int fresh_v(int x) { asm volatile("" : "+v"(x)); return x; }
 SL_DEV int fresh_s(int x) { asm volatile("" : "+s"(x)); return x; }
+
+// A touch pulls a line into this XCD's L2 (and its translation into the TLB) one stage ahead.  It is an
+// ordinary load of one dword whose value goes to touch_done() later, at a point where the wave has already
+// waited for younger loads; nothing is done with the value.  (A volatile load would be waited for at once.)
+SL_DEV uint32_t ftouch(const void* p, bool on) {
+  uint32_t v = 0;
+  if (on) v = *reinterpret_cast<const uint32_t*>(p);
+  return v;
+}
+SL_DEV void touch_done(uint32_t v) { asm volatile("" ::"v"(v)); }
+SL_DEV void touch_done(uint2 v) { touch_done(v.x); touch_done(v.y); }
+// Rows of K = 2048*NBLK of a 4-bit matrix: 8*NBLK lines of weights per row (x) and the row's scale line (y).
+template <int NBLK>
+SL_DEV uint2 ftouch_rows(const uint32_t* W, const uint32_t* SB, const size_t* rows, const bool* valid, int nrows, int lane) {
+  constexpr int LPR = 8 * NBLK;
+  const int r = lane / LPR, l = lane % LPR;
+  bool onw = false, ons = false;
+  size_t rw = 0, rs = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (j < nrows && r == j && valid[j]) { onw = true; rw = rows[j]; }
+    if (j < nrows && lane == j && valid[j]) { ons = true; rs = rows[j]; }
+  }
+  uint2 t;
+  t.x = ftouch(reinterpret_cast<const char*>(W + rw * (NBLK * 256)) + 128 * l, onw);
+  t.y = ftouch(SB + rs * (NBLK * 32), ons);
+  return t;
+}
 
 enum { FS_IN = 0, FS_CORE = 1, FS_MERGE = 2, FS_OUT = 3, FS_A = 4, FS_B = 5, FS_C = 6 };
 constexpr unsigned FLOW_SPIN_LIMIT = 1u << 19;
@@ -170,21 +207,22 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.input_ln) + 2 * tid);
   // first touches of the next stage: this workgroup's recurrent-state rows, or its key/value tile
+  uint32_t t0 = 0, t1 = 0;
   if (uni(Y.is_linear)) {
     if (wg < 256 && wave < 8) {
       const int hv = wg >> 3, dvb = wg & 7, par = (int)((uni(g_K.parity) >> li) & 1ull);
-      l2_touch(uni(Y.state[par]) + ((size_t)hv * 128 + dvb * 16 + wave * 2) * 128, 8, lane);
+      t0 = ftouch(uni(Y.state[par]) + ((size_t)hv * 128 + dvb * 16 + wave * 2) * 128 + 32 * lane, lane < 8);
     }
   } else {
     const int nt = (pos + SDPA_TILE) / SDPA_TILE;
     if (wg < nt * SL_ATT_KV) {
+      // rows already in the arena only (the row of this step is written later): 4 rows x 4 lines per wave
       const int tile = wg >> 1, kvh = wg & 1;
       const int row = tile * SDPA_TILE + wave * 4 + (lane >> 2);
-      if (lane < 16 && row < pos) {
-        const size_t off = ((size_t)kvh * uni(P.max_seq) + row) * 256 + (size_t)(lane & 3) * 64;
-        (void)*reinterpret_cast<const volatile uint32_t*>(uni(Y.kcache) + off);
-        (void)*reinterpret_cast<const volatile uint32_t*>(uni(Y.vcache) + off);
-      }
+      const bool on = lane < 16 && row < pos;
+      const size_t off = on ? ((size_t)kvh * uni(P.max_seq) + row) * 256 + (size_t)(lane & 3) * 64 : 0;
+      t0 = ftouch(uni(Y.kcache) + off, on);
+      t1 = ftouch(uni(Y.vcache) + off, on);
     }
   }
   float h0, h1, r0 = 0.0f, r1 = 0.0f;
@@ -208,6 +246,7 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   }
   const uint32_t tin = flow_tag(base, li, FS_IN);
   flow_prologue(h0, h1, li > 0, r0, r1, lnw, wg == 0, co_rsrc(uni(F.th[1])), tin, nullptr);
+  touch_done(t0); touch_done(t1);
   const F4 o = dot_1x4(wr);
   if (lane == 0) {
     const rsrc_t rp = co_rsrc(uni(F.tproj));
@@ -240,16 +279,19 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   else if (tid < 272) ch = 4096 + hv * 128 + dvb * 16 + (tid - 256);
   else if (tid == 272) ch = 12288 + hv;       // beta logit
   else if (tid == 273) ch = 12320 + hv;       // decay logit
-  float tap[3] = {0.0f, 0.0f, 0.0f}, cw[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  // history taps stay raw until the wait is over: converting them here would wait for the loads
+  uint16_t traw[3] = {0, 0, 0};
+  float cw[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   if (tid < 272) {
 #pragma unroll
-    for (int k = 0; k < 3; ++k) tap[k] = h2f(hin[k * SL_CONV_DIM + ch]);
-#pragma unroll
-    for (int k = 0; k < 4; ++k) cw[k] = uni(Y.conv_w)[ch * 4 + k];
+    for (int k = 0; k < 3; ++k) traw[k] = hin[k * SL_CONV_DIM + ch];
+    const float4 c4 = *reinterpret_cast<const float4*>(uni(Y.conv_w) + ch * 4);
+    cw[0] = c4.x; cw[1] = c4.y; cw[2] = c4.z; cw[3] = c4.w;
   }
+  uint2 tt;
   {
     const size_t orow[1] = {(size_t)(gw < H ? gw : 0)}; const bool ov[1] = {gw < H};
-    l2_touch_rows<2>(uni(Y.out_w), uni(Y.out_sb), orow, ov, 1, lane);
+    tt = ftouch_rows<2>(uni(Y.out_w), uni(Y.out_sb), orow, ov, 1, lane);
   }
   float newest = 0.0f;
   {
@@ -266,6 +308,8 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     }
     fstamp(P, 3, spins);
   }
+  touch_done(tt);
+  const float tap[3] = {h2f(traw[0]), h2f(traw[1]), h2f(traw[2])};
   if (tid < 272) {
     float acc = 0.0f;
 #pragma unroll
@@ -325,9 +369,10 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
   const int N = pos + 1, nt = (N + SDPA_TILE - 1) / SDPA_TILE;
+  uint2 tt;
   {
     const size_t orow[1] = {(size_t)(gw < H ? gw : 0)}; const bool ov[1] = {gw < H};
-    l2_touch_rows<2>(uni(Y.out_w), uni(Y.out_sb), orow, ov, 1, lane);
+    tt = ftouch_rows<2>(uni(Y.out_w), uni(Y.out_sb), orow, ov, 1, lane);
   }
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag32(base, li, FS_CORE);
   for (int u = wg; u < nt * SL_ATT_KV; u += G) {
@@ -361,6 +406,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       }
       fstamp(P, 5, spins);
     }
+    touch_done(tt);
     if (wave < 9) {
       const bool isq = wave < 8;
       const uint16_t* nwp = isq ? uni(Y.q_norm) : uni(Y.k_norm);
@@ -449,11 +495,13 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   WRegs<2, 1> wr;
   const bool valid = gw < H;
   wload_row<2>(wr.w[0], wr.sb[0], uni(Y.out_w), uni(Y.out_sb), (size_t)(valid ? gw : 0), valid, lane);
-  if (gw <= uni(P.E)) l2_touch((gw < uni(P.E) ? uni(Y.router_w) + (size_t)gw * H : uni(Y.sgate_w)), 32, lane);
+  uint32_t ta0 = 0;
+  uint2 ta1 = make_uint2(0, 0), ta2 = make_uint2(0, 0);
+  if (gw <= uni(P.E)) ta0 = ftouch((gw < uni(P.E) ? uni(Y.router_w) + (size_t)gw * H : uni(Y.sgate_w)) + 64 * lane, lane < 32);
   if (gw >= 512 && gw < 1024) {
     const size_t pr[1] = {(size_t)(gw - 512)}; const bool pv[1] = {true};
-    l2_touch_rows<1>(uni(Y.shg_w), uni(Y.shg_sb), pr, pv, 1, lane);
-    l2_touch_rows<1>(uni(Y.shu_w), uni(Y.shu_sb), pr, pv, 1, lane);
+    ta1 = ftouch_rows<1>(uni(Y.shg_w), uni(Y.shg_sb), pr, pv, 1, lane);
+    ta2 = ftouch_rows<1>(uni(Y.shu_w), uni(Y.shu_sb), pr, pv, 1, lane);
   }
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
@@ -528,6 +576,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     }
     fstamp(P, 7, spins);
   }
+  touch_done(ta0); touch_done(ta1); touch_done(ta2);
   if (lin) {
     float nw[4];
     const uint2 wraw = *reinterpret_cast<const uint2*>(uni(Y.gdn_norm_w) + (e0 & 127));
@@ -608,40 +657,52 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
 }
 
 // ---- MoE stage B: routing + routed gate/up + SwiGLU -------------------------------------------------------
-SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
+// Order key of a router logit: larger logit first, lower expert index first on ties (+0 and -0 tie).
+SL_DEV uint32_t route_key(uint32_t hbits, int e) {
+  uint32_t u = hbits & 0xffffu;
+  if ((u & 0x7fffu) == 0) u = 0;
+  u = (u & 0x8000u) ? (~u & 0xffffu) : (u | 0x8000u);
+  return (u << 8) | (uint32_t)(255 - e);
+}
+SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, uint32_t* carry /*4*/) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
-  float* lg = L.part;
-  float* ex = L.part + 256;
-  int* cnt = reinterpret_cast<int*>(g_vt);
+  float* lg = L.part;                                   // [256] logits
+  float* ex = L.part + 256;                             // [256] exp(logit - max)
+  uint32_t* key = reinterpret_cast<uint32_t*>(L.part + 512);   // [256] order keys
+  int* cnt = reinterpret_cast<int*>(g_vt);              // [4][256] partial rank counts (the value tile is idle here)
   // Non-finite logits rank no expert below 8; the slots then keep these in-range defaults.
   if (tid < 8) { L.inds[tid] = tid; L.scores[tid] = 0.0f; }
   {
     const uint32_t ta = flow_tag(base, li, FS_A);
     const rsrc_t rl = co_rsrc(uni(F.trlog));
+    const int E = uni(P.E);
     unsigned spins = 0;
     fstamp(P, 10, 0);
     for (;;) {
       bool ok = true;
       float v0 = NEG;
-      if (tid < uni(P.E)) { const uint32_t w = ldw1(rl, tid); ok = tag_ok(w, ta); v0 = lo_h(w); }
-      if (tid < 256) lg[tid] = v0;
+      uint32_t k0 = 0;
+      if (tid < E) { const uint32_t w = ldw1(rl, tid); ok = tag_ok(w, ta); v0 = lo_h(w); k0 = route_key(w, tid); }
+      if (tid < 256) { lg[tid] = v0; key[tid] = k0; }
       const int v = flow_round(ok, spins, uni(P.bar) + 32);
       if (v > 0) break;
       if (v < 0) return false;
     }
     fstamp(P, 11, spins);
   }
+  // The 8 selected experts in routing order are the experts of rank 0..7, so each expert's rank is counted
+  // directly: threads (part, e) count the keys of one quarter that precede e; wave 0 forms the softmax sums.
   {
     const int e = tid & 255, part = tid >> 8;
-    const float me = lg[e];
+    const uint32_t me = key[e];
     int c = 0;
-#pragma unroll 8
-    for (int j = 64 * part; j < 64 * part + 64; ++j) {
-      const float o = lg[j];
-      c += (o > me || (o == me && j < e)) ? 1 : 0;
+#pragma unroll
+    for (int j = 0; j < 64; j += 4) {
+      const uint4 o = *reinterpret_cast<const uint4*>(&key[64 * part + j]);
+      c += (o.x > me) ? 1 : 0; c += (o.y > me) ? 1 : 0; c += (o.z > me) ? 1 : 0; c += (o.w > me) ? 1 : 0;
     }
     cnt[part * 256 + e] = c;
   }
@@ -661,12 +722,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     if (rank < 8 && tid < uni(P.E)) { L.inds[rank] = tid; L.scores[rank] = f16r(ex[tid] / L.gb[0]); }
   }
   __syncthreads();
-  if (tid == 0) {
-    float ss = 0.0f;
-    for (int k = 0; k < 8; ++k) ss = f16r(ss + L.scores[k]);
-    for (int k = 0; k < 8; ++k) L.scores[k] = f16r(L.scores[k] / ss);
-    if (wg == 0) for (int k = 0; k < 8; ++k) { uni(Y.route_inds)[k] = L.inds[k]; uni(Y.route_scores)[k] = f2h(L.scores[k]); }
-  }
+  // this wave's gate/up pair (issued as soon as the indices are known), then first touches of its down rows
   const int p = gw;
   WRegs<1, 2> wr;
   int k = 0, i = 0;
@@ -680,13 +736,17 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
 #pragma unroll
   for (int qq = 0; qq < 2; ++qq) {
     const int un = wave + 16 * qq, ql = un / 9, slot = un % 9;
-    if (ql < 2 && slot < 8) {
-      const size_t row = (size_t)L.inds[slot] * 2048 + (size_t)(wg * 2 + ql) * 4;
-      l2_touch(uni(Y.swd_w) + row * 64, 8, lane);
-      if (lane == 8) (void)*reinterpret_cast<const volatile uint32_t*>(uni(Y.swd_sb) + row * 8);
-    }
+    const bool on = ql < 2 && slot < 8;
+    const size_t row = on ? (size_t)L.inds[slot] * 2048 + (size_t)(wg * 2 + ql) * 4 : 0;
+    carry[2 * qq] = ftouch(reinterpret_cast<const char*>(uni(Y.swd_w) + row * 64) + 128 * lane, on && lane < 8);
+    carry[2 * qq + 1] = ftouch(uni(Y.swd_sb) + row * 8, on && lane == 8);
   }
-  __syncthreads();
+  if (tid == 0) {
+    float ss = 0.0f;
+    for (int kk = 0; kk < 8; ++kk) ss = f16r(ss + L.scores[kk]);
+    for (int kk = 0; kk < 8; ++kk) L.scores[kk] = f16r(L.scores[kk] / ss);
+    if (wg == 0) for (int kk = 0; kk < 8; ++kk) { uni(Y.route_inds)[kk] = L.inds[kk]; uni(Y.route_scores)[kk] = f2h(L.scores[kk]); }
+  }
   if (active) {
     const F2 gu = dot_1x2(wr);
     if (lane == 0) stw1(co_rsrc(uni(F.tact)), k * 512 + i, tagged(swiglu16(f16r(gu.v[0]), f16r(gu.v[1])), flow_tag(base, li, FS_B)));
@@ -695,12 +755,17 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
 }
 
 // ---- MoE stage C: down-projections, half combine, gated shared add ---------------------------------------
+// Units (quad of 4 outputs, slot): slots 0..7 routed experts, slot 8 shared; 2 quads per workgroup.  The nine
+// activation rows are fetched once per workgroup into LDS (packed pairs, 20-word stride per 32 elements).
+constexpr int XC_STRIDE = 20;
 SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, const uint32_t* next_w, const uint32_t* next_sb,
-                       int next_n, int next_contig) {
+                       int next_n, int next_contig, const uint32_t* carry /*4*/) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   Lds& L = g_L;
+  uint32_t* xc = reinterpret_cast<uint32_t*>(g_vt);      // [9][16][XC_STRIDE]
   const int sub = lane >> 4, li16 = lane & 15;
+  uint2 tn;
   {
     size_t rows[4]; bool rv[4];
 #pragma unroll
@@ -708,54 +773,69 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
       const long r = next_contig ? (long)gw * 64 + j : (long)gw + (long)j * NW;
       rv[j] = r < next_n; rows[j] = rv[j] ? (size_t)r : 0;
     }
-    l2_touch_rows<1>(next_w, next_sb, rows, rv, 4, lane);
+    tn = ftouch_rows<1>(next_w, next_sb, rows, rv, 4, lane);
   }
   const uint32_t ta = flow_tag(base, li, FS_A), tb = flow_tag(base, li, FS_B);
-  float sgate_logit = 0.0f;
+  // weights of this wave's (up to) two units: routed rows were touched during stage B
+  uint4 wv[2]; uint32_t sbv[2];
 #pragma unroll
   for (int qq = 0; qq < 2; ++qq) {
     const int un = wave + 16 * qq, ql = un / 9, slot = un % 9;
-    const int quad = wg * 2 + ql;
-    const bool has = ql < 2;
-    uint4 wv = make_uint4(0, 0, 0, 0); uint32_t sbv = 0;
-    if (has) {
-      // the routed rows were touched into L2 during stage B; the shared rows do not depend on routing
-      const size_t row = (slot < 8 ? (size_t)L.inds[slot] * 2048 : 0) + (size_t)quad * 4 + sub;
+    wv[qq] = make_uint4(0, 0, 0, 0); sbv[qq] = 0;
+    if (ql < 2) {
+      const size_t row = (slot < 8 ? (size_t)L.inds[slot] * 2048 : 0) + (size_t)(wg * 2 + ql) * 4 + sub;
       const uint32_t* W = slot < 8 ? uni(Y.swd_w) : uni(Y.shd_w);
       const uint32_t* SB = slot < 8 ? uni(Y.swd_sb) : uni(Y.shd_sb);
-      wv = ld16(W + row * 64 + 4 * li16);
-      sbv = SB[row * 8 + (li16 >> 1)];
+      wv[qq] = ld16(W + row * 64 + 4 * li16);
+      sbv[qq] = SB[row * 8 + (li16 >> 1)];
     }
-    float x[32];
-    {
-      const rsrc_t rx = co_rsrc(slot < 8 ? uni(F.tact) + slot * 512 : uni(F.tsh));
-      const uint32_t tx = slot < 8 ? tb : ta;
-      const rsrc_t rg = co_rsrc(uni(F.tsg));
-      unsigned spins = 0;
+  }
+  float sgate_logit = 0.0f;
+  uint4 a4 = make_uint4(0, 0, 0, 0), s4 = make_uint4(0, 0, 0, 0);
+  {
+    const rsrc_t ra = co_rsrc(uni(F.tact)), rs = co_rsrc(uni(F.tsh)), rg = co_rsrc(uni(F.tsg));
+    unsigned spins = 0;
     fstamp(P, 12, 0);
-      for (;;) {
-        bool ok = true;
-        if (has) {
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const uint4 w = ldw4(rx, 32 * li16 + 4 * j);
-            ok = ok && tag_ok(w.x, tx) && tag_ok(w.y, tx) && tag_ok(w.z, tx) && tag_ok(w.w, tx);
-            x[4 * j] = lo_h(w.x); x[4 * j + 1] = lo_h(w.y); x[4 * j + 2] = lo_h(w.z); x[4 * j + 3] = lo_h(w.w);
-          }
-        }
-        if (qq == 0 && tid < 8) { const uint32_t w = ldw1(rg, 0); ok = ok && tag_ok(w, ta); sgate_logit = lo_h(w); }
-        const int v = flow_round(ok, spins, uni(P.bar) + 32);
-        if (v > 0) break;
-        if (v < 0) return false;
-      }
-      fstamp(P, 13, spins);
+    for (;;) {
+      a4 = ldw4(ra, 4 * tid);
+      bool ok = tag_ok(a4.x, tb) && tag_ok(a4.y, tb) && tag_ok(a4.z, tb) && tag_ok(a4.w, tb);
+      if (tid < 128) { s4 = ldw4(rs, 4 * tid); ok = ok && tag_ok(s4.x, ta) && tag_ok(s4.y, ta) && tag_ok(s4.z, ta) && tag_ok(s4.w, ta); }
+      if (tid < 8) { const uint32_t w = ldw1(rg, 0); ok = ok && tag_ok(w, ta); sgate_logit = lo_h(w); }
+      const int v = flow_round(ok, spins, uni(P.bar) + 32);
+      if (v > 0) break;
+      if (v < 0) return false;
     }
-    if (has) {
-      float sx[4];
+    fstamp(P, 13, spins);
+  }
+  touch_done(tn);
+  touch_done(carry[0]); touch_done(carry[1]); touch_done(carry[2]); touch_done(carry[3]);
+  {
+    // thread t holds elements 4(t%128).. of slot t/128: packed pairs 2(t%128), 2(t%128)+1
+    const int slot = tid >> 7, pi = 2 * (tid & 127);
+    *reinterpret_cast<uint2*>(&xc[(slot * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
+        make_uint2((a4.x & 0xffffu) | (a4.y << 16), (a4.z & 0xffffu) | (a4.w << 16));
+    if (tid < 128)
+      *reinterpret_cast<uint2*>(&xc[(8 * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
+          make_uint2((s4.x & 0xffffu) | (s4.y << 16), (s4.z & 0xffffu) | (s4.w << 16));
+  }
+  __syncthreads();
+#pragma unroll
+  for (int qq = 0; qq < 2; ++qq) {
+    const int un = wave + 16 * qq, ql = un / 9, slot = un % 9;
+    if (ql < 2) {
       uint32_t xp[16];
-      word_sums(x, sx);
-      pack_x(x, xp);
-      const float d = tree_sum<16>(quad_term(wv, sbv, xp, sx));
+      const uint4* src = reinterpret_cast<const uint4*>(&xc[(slot * 16 + li16) * XC_STRIDE]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { const uint4 q = src[j]; xp[4 * j] = q.x; xp[4 * j + 1] = q.y; xp[4 * j + 2] = q.z; xp[4 * j + 3] = q.w; }
+      float sx[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float sacc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { sacc = sacc + lo_h(xp[4 * j + i]); sacc = sacc + hi_h(xp[4 * j + i]); }
+        sx[j] = sacc;
+      }
+      const float d = tree_sum<16>(quad_term(wv[qq], sbv[qq], xp, sx));
       if (li16 == 0) L.dbuf[(ql * 9 + slot) * 4 + sub] = f16r(d);
     }
   }
@@ -907,12 +987,13 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
       if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base)) return;
     }
     if (!flow_moe_a(F, Y, li, base)) return;
-    if (!flow_moe_b(F, Y, li, base)) return;
+    uint32_t carry[4];
+    if (!flow_moe_b(F, Y, li, base, carry)) return;
     {
       const bool last = li + 1 == nl;
       const LayerP& Z = g_K.layers[last ? li : li + 1];
       if (!flow_moe_c(F, Y, li, base, last ? uni(P.lm_w) : uni(Z.in_w), last ? uni(P.lm_sb) : uni(Z.in_sb),
-                      last ? uni(P.vocab) : (uni(Z.is_linear) ? SL_GDN_IN_N : SL_ATT_QKV_N), last ? 1 : 0)) return;
+                      last ? uni(P.vocab) : (uni(Z.is_linear) ? SL_GDN_IN_N : SL_ATT_QKV_N), last ? 1 : 0, carry)) return;
     }
   }
   flow_head(F, pos, out_off, feed, base);
