@@ -74,19 +74,55 @@ SL_DEV float sigmoid16(float x) {
 SL_DEV float softplus_c(float x) { return fmaxf(x, 0.0f) + log_c(1.0f + exp_c(-fabsf(x))); }
 SL_DEV float swiglu16(float g, float u) { return f16r(f16r(g * sigmoid16(g)) * u); }
 
-// ---- wave64 butterflies ---------------------------------------------------------------------------
+// ---- wave64 reductions ------------------------------------------------------------------------------
+// The value of every reduction is that of the xor-butterfly (partners at distance 1, 2, 4, ... combined in
+// that order), which is a balanced binary tree over adjacent lanes.  After step k all 2^k lanes of a group
+// hold the same value, so a lane may take its partner group's value from ANY lane of that group and, the
+// operation being commutative, gets the same bits.  That lets the first four steps run as DPP operand
+// modifiers (quad permutes, half-row mirror, row mirror: no LDS round trip) and the last two as reads of one
+// lane per 16-lane row.
+template <int CTRL>
+SL_DEV float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int CTRL>
+SL_DEV uint32_t dpp_u(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+}
+constexpr int DPP_XOR1 = 0xB1;          // quad_perm [1,0,3,2]
+constexpr int DPP_XOR2 = 0x4E;          // quad_perm [2,3,0,1]
+constexpr int DPP_HALF_MIRROR = 0x141;  // lane i <-> 7-i within 8
+constexpr int DPP_MIRROR = 0x140;       // lane i <-> 15-i within 16
+constexpr int DPP_SHR1 = 0x111;         // lane i takes lane i-1 within its 16-lane row
+SL_DEV float row_lane_f(float v, int lane) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane)); }
+
 template <int WIDTH>
 SL_DEV float tree_sum(float v) {
-#pragma unroll
-  for (int m = 1; m < WIDTH; m <<= 1) v = v + __shfl_xor(v, m, 64);
-  return v;
+  static_assert(WIDTH == 4 || WIDTH == 8 || WIDTH == 16 || WIDTH == 32 || WIDTH == 64, "group sizes used by the kernels");
+  v = v + dpp_f<DPP_XOR1>(v);
+  v = v + dpp_f<DPP_XOR2>(v);
+  if constexpr (WIDTH == 4) return v;
+  v = v + dpp_f<DPP_HALF_MIRROR>(v);
+  if constexpr (WIDTH == 8) return v;
+  v = v + dpp_f<DPP_MIRROR>(v);
+  if constexpr (WIDTH == 16) return v;
+  const float r0 = row_lane_f(v, 0), r1 = row_lane_f(v, 16), r2 = row_lane_f(v, 32), r3 = row_lane_f(v, 48);
+  const float lo = r0 + r1, hi = r2 + r3;
+  if constexpr (WIDTH == 32) return (__lane_id() < 32) ? lo : hi;
+  return lo + hi;
 }
 template <int WIDTH>
 SL_DEV float tree_max(float v) {
-#pragma unroll
-  for (int m = 1; m < WIDTH; m <<= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
-  return v;
+  static_assert(WIDTH == 64, "group sizes used by the kernels");
+  v = fmaxf(v, dpp_f<DPP_XOR1>(v));
+  v = fmaxf(v, dpp_f<DPP_XOR2>(v));
+  v = fmaxf(v, dpp_f<DPP_HALF_MIRROR>(v));
+  v = fmaxf(v, dpp_f<DPP_MIRROR>(v));
+  const float r0 = row_lane_f(v, 0), r1 = row_lane_f(v, 16), r2 = row_lane_f(v, 32), r3 = row_lane_f(v, 48);
+  return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 }
+// Value of the previous lane (lanes 0, 16, 32, 48 get 0): for left-to-right chains inside a 16-lane row.
+SL_DEV float prev_lane(float v) { return dpp_f<DPP_SHR1>(v); }
 
 // ---- 16-byte vector access -------------------------------------------------------------------------
 SL_DEV uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }

@@ -181,7 +181,7 @@ SL_DEV void flow_prologue(float h0, float h1, bool has_r, float r0, float r1, ui
   float s = (0.0f + y0) + y1;
 #pragma unroll
   for (int r = 1; r < 4; ++r) {
-    const float v = __shfl_up(s, 1, 64);
+    const float v = prev_lane(s);
     if (q == r) s = (v + y0) + y1;
   }
   if (q == 3) g_L.sxs[((tid & 15) >> 2) * 64 + (tid >> 4)] = s;
@@ -598,7 +598,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     float sfirst = 0.0f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) sfirst = sfirst + out[i];
-    float srest = __shfl_up(sfirst, 1, 64);
+    float srest = prev_lane(sfirst);
 #pragma unroll
     for (int i = 0; i < 4; ++i) srest = srest + out[i];
     if (lane & 1) g_L.sxs[(4 * b + (i0 >> 3)) * 64 + lo] = srest;
@@ -672,9 +672,6 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
   float* lg = L.part;                                   // [256] logits
   float* ex = L.part + 256;                             // [256] exp(logit - max)
   uint32_t* key = reinterpret_cast<uint32_t*>(L.part + 512);   // [256] order keys
-  int* cnt = reinterpret_cast<int*>(g_vt);              // [4][256] partial rank counts (the value tile is idle here)
-  // Non-finite logits rank no expert below 8; the slots then keep these in-range defaults.
-  if (tid < 8) { L.inds[tid] = tid; L.scores[tid] = 0.0f; }
   {
     const uint32_t ta = flow_tag(base, li, FS_A);
     const rsrc_t rl = co_rsrc(uni(F.trlog));
@@ -693,20 +690,26 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
     }
     fstamp(P, 11, spins);
   }
-  // The 8 selected experts in routing order are the experts of rank 0..7, so each expert's rank is counted
-  // directly: threads (part, e) count the keys of one quarter that precede e; wave 0 forms the softmax sums.
-  {
-    const int e = tid & 255, part = tid >> 8;
-    const uint32_t me = key[e];
-    int c = 0;
-#pragma unroll
-    for (int j = 0; j < 64; j += 4) {
-      const uint4 o = *reinterpret_cast<const uint4*>(&key[64 * part + j]);
-      c += (o.x > me) ? 1 : 0; c += (o.y > me) ? 1 : 0; c += (o.z > me) ? 1 : 0; c += (o.w > me) ? 1 : 0;
-    }
-    cnt[part * 256 + e] = c;
-  }
+  // Wave 0 picks the 8 largest keys in order (max, remove, repeat; the wave-wide max is a DPP reduction plus
+  // one lane per row); wave 1 forms the softmax sums meanwhile.
   if (wave == 0) {
+    const uint4 k4 = *reinterpret_cast<const uint4*>(&key[4 * lane]);
+    uint32_t k[4] = {k4.x, k4.y, k4.z, k4.w};
+    const int E = uni(P.E);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      uint32_t m = max(max(k[0], k[1]), max(k[2], k[3]));
+      m = max(m, dpp_u<DPP_XOR1>(m));
+      m = max(m, dpp_u<DPP_XOR2>(m));
+      m = max(m, dpp_u<DPP_HALF_MIRROR>(m));
+      m = max(m, dpp_u<DPP_MIRROR>(m));
+      const uint32_t M = max(max((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
+                             max((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) k[i] = (k[i] == M) ? 0u : k[i];
+      if (lane == 0) L.inds[r] = min(255 - (int)(M & 255u), E - 1);
+    }
+  } else if (wave == 1) {
     float v[4], x4[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = lg[4 * lane + i];
@@ -717,11 +720,15 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
     if (lane == 0) L.gb[0] = Z;
   }
   __syncthreads();
-  if (tid < 256) {
-    const int rank = cnt[tid] + cnt[256 + tid] + cnt[512 + tid] + cnt[768 + tid];
-    if (rank < 8 && tid < uni(P.E)) { L.inds[rank] = tid; L.scores[rank] = f16r(ex[tid] / L.gb[0]); }
+  if (tid == 0) {
+    float sc[8], ss = 0.0f;
+    const float Z = L.gb[0];
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) { sc[kk] = f16r(ex[L.inds[kk]] / Z); ss = f16r(ss + sc[kk]); }
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) L.scores[kk] = f16r(sc[kk] / ss);
+    if (wg == 0) for (int kk = 0; kk < 8; ++kk) { uni(Y.route_inds)[kk] = L.inds[kk]; uni(Y.route_scores)[kk] = f2h(L.scores[kk]); }
   }
-  __syncthreads();
   // this wave's gate/up pair (issued as soon as the indices are known), then first touches of its down rows
   const int p = gw;
   WRegs<1, 2> wr;
@@ -740,12 +747,6 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
     const size_t row = on ? (size_t)L.inds[slot] * 2048 + (size_t)(wg * 2 + ql) * 4 : 0;
     carry[2 * qq] = ftouch(reinterpret_cast<const char*>(uni(Y.swd_w) + row * 64) + 128 * lane, on && lane < 8);
     carry[2 * qq + 1] = ftouch(uni(Y.swd_sb) + row * 8, on && lane == 8);
-  }
-  if (tid == 0) {
-    float ss = 0.0f;
-    for (int kk = 0; kk < 8; ++kk) ss = f16r(ss + L.scores[kk]);
-    for (int kk = 0; kk < 8; ++kk) L.scores[kk] = f16r(L.scores[kk] / ss);
-    if (wg == 0) for (int kk = 0; kk < 8; ++kk) { uni(Y.route_inds)[kk] = L.inds[kk]; uni(Y.route_scores)[kk] = f2h(L.scores[kk]); }
   }
   if (active) {
     const F2 gu = dot_1x2(wr);
