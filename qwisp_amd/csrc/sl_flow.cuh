@@ -207,24 +207,6 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.input_ln) + 2 * tid);
   // first touches of the next stage: this workgroup's recurrent-state rows, or its key/value tile
-  uint32_t t0 = 0, t1 = 0;
-  if (uni(Y.is_linear)) {
-    if (wg < 256 && wave < 8) {
-      const int hv = wg >> 3, dvb = wg & 7, par = (int)((uni(g_K.parity) >> li) & 1ull);
-      t0 = ftouch(uni(Y.state[par]) + ((size_t)hv * 128 + dvb * 16 + wave * 2) * 128 + 32 * lane, lane < 8);
-    }
-  } else {
-    const int nt = (pos + SDPA_TILE) / SDPA_TILE;
-    if (wg < nt * SL_ATT_KV) {
-      // rows already in the arena only (the row of this step is written later): 4 rows x 4 lines per wave
-      const int tile = wg >> 1, kvh = wg & 1;
-      const int row = tile * SDPA_TILE + wave * 4 + (lane >> 2);
-      const bool on = lane < 16 && row < pos;
-      const size_t off = on ? ((size_t)kvh * uni(P.max_seq) + row) * 256 + (size_t)(lane & 3) * 64 : 0;
-      t0 = ftouch(uni(Y.kcache) + off, on);
-      t1 = ftouch(uni(Y.vcache) + off, on);
-    }
-  }
   float h0, h1, r0 = 0.0f, r1 = 0.0f;
   if (li == 0) {
     const uint32_t w = *reinterpret_cast<const uint32_t*>(uni(P.hA) + 2 * tid);   // embedded row from k_embed
@@ -246,7 +228,6 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   }
   const uint32_t tin = flow_tag(base, li, FS_IN);
   flow_prologue(h0, h1, li > 0, r0, r1, lnw, wg == 0, co_rsrc(uni(F.th[1])), tin, nullptr);
-  touch_done(t0); touch_done(t1);
   const F4 o = dot_1x4(wr);
   if (lane == 0) {
     const rsrc_t rp = co_rsrc(uni(F.tproj));
@@ -288,11 +269,6 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     const float4 c4 = *reinterpret_cast<const float4*>(uni(Y.conv_w) + ch * 4);
     cw[0] = c4.x; cw[1] = c4.y; cw[2] = c4.z; cw[3] = c4.w;
   }
-  uint2 tt;
-  {
-    const size_t orow[1] = {(size_t)(gw < H ? gw : 0)}; const bool ov[1] = {gw < H};
-    tt = ftouch_rows<2>(uni(Y.out_w), uni(Y.out_sb), orow, ov, 1, lane);
-  }
   float newest = 0.0f;
   {
     const uint32_t tin = flow_tag(base, li, FS_IN);
@@ -308,7 +284,6 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     }
     fstamp(P, 3, spins);
   }
-  touch_done(tt);
   const float tap[3] = {h2f(traw[0]), h2f(traw[1]), h2f(traw[2])};
   if (tid < 272) {
     float acc = 0.0f;
@@ -369,11 +344,6 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
   const int N = pos + 1, nt = (N + SDPA_TILE - 1) / SDPA_TILE;
-  uint2 tt;
-  {
-    const size_t orow[1] = {(size_t)(gw < H ? gw : 0)}; const bool ov[1] = {gw < H};
-    tt = ftouch_rows<2>(uni(Y.out_w), uni(Y.out_sb), orow, ov, 1, lane);
-  }
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag32(base, li, FS_CORE);
   for (int u = wg; u < nt * SL_ATT_KV; u += G) {
     const int tile = u >> 1, kvh = u & 1;
@@ -406,8 +376,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       }
       fstamp(P, 5, spins);
     }
-    touch_done(tt);
-    if (wave < 9) {
+      if (wave < 9) {
       const bool isq = wave < 8;
       const uint16_t* nwp = isq ? uni(Y.q_norm) : uni(Y.k_norm);
       const float xv[4] = {lo_h(w4.x), lo_h(w4.y), lo_h(w4.z), lo_h(w4.w)};
@@ -495,14 +464,6 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   WRegs<2, 1> wr;
   const bool valid = gw < H;
   wload_row<2>(wr.w[0], wr.sb[0], uni(Y.out_w), uni(Y.out_sb), (size_t)(valid ? gw : 0), valid, lane);
-  uint32_t ta0 = 0;
-  uint2 ta1 = make_uint2(0, 0), ta2 = make_uint2(0, 0);
-  if (gw <= uni(P.E)) ta0 = ftouch((gw < uni(P.E) ? uni(Y.router_w) + (size_t)gw * H : uni(Y.sgate_w)) + 64 * lane, lane < 32);
-  if (gw >= 512 && gw < 1024) {
-    const size_t pr[1] = {(size_t)(gw - 512)}; const bool pv[1] = {true};
-    ta1 = ftouch_rows<1>(uni(Y.shg_w), uni(Y.shg_sb), pr, pv, 1, lane);
-    ta2 = ftouch_rows<1>(uni(Y.shu_w), uni(Y.shu_sb), pr, pv, 1, lane);
-  }
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
   if (!lin && wg == 0) {
@@ -576,7 +537,6 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     }
     fstamp(P, 7, spins);
   }
-  touch_done(ta0); touch_done(ta1); touch_done(ta2);
   if (lin) {
     float nw[4];
     const uint2 wraw = *reinterpret_cast<const uint2*>(uni(Y.gdn_norm_w) + (e0 & 127));
@@ -615,12 +575,16 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   const DecodeP& P = F.d;
   const bool is_dense = gw <= uni(P.E);
   const bool is_pair = gw >= 512 && gw < 1024;
-  float dw[32];
+  uint4 dwr[4] = {};                      // dense fp16 row, kept packed until the wait is over
   WRegs<1, 2> wr;
   const size_t prow = is_pair ? (size_t)(gw - 512) : 0;
   wload_row<1>(wr.w[0], wr.sb[0], uni(Y.shg_w), uni(Y.shg_sb), prow, is_pair, lane);
   wload_row<1>(wr.w[1], wr.sb[1], uni(Y.shu_w), uni(Y.shu_sb), prow, is_pair, lane);
-  if (is_dense) load32((gw < uni(P.E) ? uni(Y.router_w) + (size_t)gw * H : uni(Y.sgate_w)) + 32 * lane, dw);
+  if (is_dense) {
+    const uint16_t* drow = (gw < uni(P.E) ? uni(Y.router_w) + (size_t)gw * H : uni(Y.sgate_w)) + 32 * lane;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dwr[j] = ld16(drow + 8 * j);
+  }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.post_ln) + 2 * tid);
   float h0, h1, r0, r1;
   {
@@ -643,9 +607,11 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   if (is_dense) {
     uint32_t xp[16]; float sx[4];
     lds_get_x(0, lane, xp, sx);
+    const uint32_t dww[16] = {dwr[0].x, dwr[0].y, dwr[0].z, dwr[0].w, dwr[1].x, dwr[1].y, dwr[1].z, dwr[1].w,
+                              dwr[2].x, dwr[2].y, dwr[2].z, dwr[2].w, dwr[3].x, dwr[3].y, dwr[3].z, dwr[3].w};
     float acc = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { acc = fmaf(lo_h(xp[i]), dw[2 * i], acc); acc = fmaf(hi_h(xp[i]), dw[2 * i + 1], acc); }
+    for (int i = 0; i < 16; ++i) { acc = fmaf(lo_h(xp[i]), lo_h(dww[i]), acc); acc = fmaf(hi_h(xp[i]), hi_h(dww[i]), acc); }
     acc = tree_sum<64>(acc);
     if (lane == 0) { if (gw < uni(P.E)) stw1(co_rsrc(uni(F.trlog)), gw, tagged(acc, ta)); else stw1(co_rsrc(uni(F.tsg)), 0, tagged(acc, ta)); }
   }
@@ -766,16 +732,6 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
   Lds& L = g_L;
   uint32_t* xc = reinterpret_cast<uint32_t*>(g_vt);      // [9][16][XC_STRIDE]
   const int sub = lane >> 4, li16 = lane & 15;
-  uint2 tn;
-  {
-    size_t rows[4]; bool rv[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const long r = next_contig ? (long)gw * 64 + j : (long)gw + (long)j * NW;
-      rv[j] = r < next_n; rows[j] = rv[j] ? (size_t)r : 0;
-    }
-    tn = ftouch_rows<1>(next_w, next_sb, rows, rv, 4, lane);
-  }
   const uint32_t ta = flow_tag(base, li, FS_A), tb = flow_tag(base, li, FS_B);
   // weights of this wave's (up to) two units: routed rows were touched during stage B
   uint4 wv[2]; uint32_t sbv[2];
@@ -808,7 +764,6 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
     }
     fstamp(P, 13, spins);
   }
-  touch_done(tn);
   touch_done(carry[0]); touch_done(carry[1]); touch_done(carry[2]); touch_done(carry[3]);
   {
     // thread t holds elements 4(t%128).. of slot t/128: packed pairs 2(t%128), 2(t%128)+1
