@@ -466,14 +466,13 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
         FlowP F;
         std::memset(&F, 0, sizeof(F));
         F.d = P;
-        F.th[0] = dalloc<uint32_t>(e, H, true); F.th[1] = dalloc<uint32_t>(e, H, true);
         F.tproj = dalloc<uint32_t>(e, PROJ_STRIDE, true); F.tycore = dalloc<uint32_t>(e, 4096, true);
         F.tmix = dalloc<uint32_t>(e, H, true); F.trlog = dalloc<uint32_t>(e, 256, true); F.tsg = dalloc<uint32_t>(e, 4, true);
         F.tsh = dalloc<uint32_t>(e, 512, true); F.tact = dalloc<uint32_t>(e, 8 * 512, true); F.tmoe = dalloc<uint32_t>(e, H, true);
         F.tml = dalloc<uint4>(e, (size_t)SL_ATT_HEADS * e->max_tiles, true);
         F.tpo = dalloc<uint4>(e, (size_t)SL_ATT_HEADS * e->max_tiles * 128, true);
         F.tcand = dalloc<uint4>(e, 256, true);
-        if (!F.th[0] || !F.th[1] || !F.tproj || !F.tycore || !F.tmix || !F.trlog || !F.tsg || !F.tsh || !F.tact || !F.tmoe ||
+        if (!F.tproj || !F.tycore || !F.tmix || !F.trlog || !F.tsg || !F.tsh || !F.tact || !F.tmoe ||
             !F.tml || !F.tpo || !F.tcand) return SL_ERR_DEVICE;
         e->flow_host = F;
         e->flow_params = upload<FlowP>(e, &F, 1, SL_LOC_HOST);

@@ -19,7 +19,6 @@ namespace sl {
 
 struct FlowP {
   DecodeP d;
-  uint32_t *th[2];      // hidden rows A/B                 [2048] {half, tag}
   uint32_t *tproj;      // projection output               [12352]
   uint32_t *tycore;     // GDN core out / gated attn out   [4096]
   uint32_t *tmix;       // mixer output                    [2048]
@@ -149,16 +148,15 @@ SL_DEV int flow_round(bool ok, unsigned& spins, unsigned* abort_word) {
   return 0;
 }
 
-// Prologue on the whole workgroup: thread t owns elements 2t, 2t+1 of the hidden row.
-//   h' = half(h + r); x = w * half(h' * inv_rms(h')) -> packed into LDS with the word sums.
+// Prologue on the whole workgroup: thread t owns elements 2t, 2t+1 of the hidden row and keeps them in
+// registers from stage to stage (every workgroup follows the whole residual stream, so it is never exchanged).
+//   h' = half(h + r) (returned in h0, h1); x = w * half(h' * inv_rms(h')) -> packed into LDS with the word sums.
 // Sum of squares keeps the canonical order: wave 0, lane l chains its 32 contiguous elements.
-SL_DEV void flow_prologue(float h0, float h1, bool has_r, float r0, float r1, uint32_t lnw_pair, bool writer,
-                          rsrc_t h_out, uint32_t tag_out, uint16_t* xn_plain) {
+SL_DEV void flow_prologue(float& h0, float& h1, bool has_r, float r0, float r1, uint32_t lnw_pair, uint16_t* xn_plain) {
   const int tid = fresh_v(threadIdx.x), lane = tid & 63, wave = tid >> 6;
   uint32_t* hs = reinterpret_cast<uint32_t*>(g_L.sq);          // 1024 words of scratch (attention's query area)
   if (has_r) { h0 = f16r(h0 + r0); h1 = f16r(h1 + r1); }
   hs[tid + (tid >> 4)] = pack2(h0, h1);       // 17-word lane stride: conflict-free for the chain below
-  if (writer) stw2(h_out, 2 * tid, tagged(h0, tag_out), tagged(h1, tag_out));
   __syncthreads();
   if (wave == 0) {
     float ss = 0.0f;
@@ -185,7 +183,7 @@ SL_DEV void flow_prologue(float h0, float h1, bool has_r, float r0, float r1, ui
     if (q == r) s = (v + y0) + y1;
   }
   if (q == 3) g_L.sxs[((tid & 15) >> 2) * 64 + (tid >> 4)] = s;
-  if (writer && xn_plain) *reinterpret_cast<uint32_t*>(xn_plain + 2 * tid) = pack2(y0, y1);
+  if (xn_plain) *reinterpret_cast<uint32_t*>(xn_plain + 2 * tid) = pack2(y0, y1);
   __syncthreads();
 }
 
@@ -194,7 +192,7 @@ SL_DEV void flow_prologue(float h0, float h1, bool has_r, float r0, float r1, ui
                  (void)tid; (void)lane; (void)wave; (void)wg; (void)G; (void)NW; (void)gw
 
 // ---- stage 1: input norm + in-projection ------------------------------------------------------------
-SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base) {
+SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base, float& h0, float& h1) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   const int N = uni(Y.is_linear) ? SL_GDN_IN_N : SL_ATT_QKV_N;
@@ -207,19 +205,19 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.input_ln) + 2 * tid);
   // first touches of the next stage: this workgroup's recurrent-state rows, or its key/value tile
-  float h0, h1, r0 = 0.0f, r1 = 0.0f;
+  float r0 = 0.0f, r1 = 0.0f;
   if (li == 0) {
     const uint32_t w = *reinterpret_cast<const uint32_t*>(uni(P.hA) + 2 * tid);   // embedded row from k_embed
     h0 = lo_h(w); h1 = hi_h(w);
   } else {
-    const uint32_t th = flow_tag(base, li - 1, FS_A), tr = flow_tag(base, li - 1, FS_C);
-    const rsrc_t rh = co_rsrc(uni(F.th[0])), rr = co_rsrc(uni(F.tmoe));
+    const uint32_t tr = flow_tag(base, li - 1, FS_C);
+    const rsrc_t rr = co_rsrc(uni(F.tmoe));
     unsigned spins = 0;
     fstamp(P, 0, 0);
     for (;;) {
-      const uint2 a = ldw2(rh, 2 * tid), b = ldw2(rr, 2 * tid);
-      const bool ok = tag_ok(a.x, th) && tag_ok(a.y, th) && tag_ok(b.x, tr) && tag_ok(b.y, tr);
-      h0 = lo_h(a.x); h1 = lo_h(a.y); r0 = lo_h(b.x); r1 = lo_h(b.y);
+      const uint2 b = ldw2(rr, 2 * tid);
+      const bool ok = tag_ok(b.x, tr) && tag_ok(b.y, tr);
+      r0 = lo_h(b.x); r1 = lo_h(b.y);
       const int v = flow_round(ok, spins, uni(P.bar) + 32);
       if (v > 0) break;
       if (v < 0) return false;
@@ -227,7 +225,7 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
     fstamp(P, 1, spins);
   }
   const uint32_t tin = flow_tag(base, li, FS_IN);
-  flow_prologue(h0, h1, li > 0, r0, r1, lnw, wg == 0, co_rsrc(uni(F.th[1])), tin, nullptr);
+  flow_prologue(h0, h1, li > 0, r0, r1, lnw, nullptr);
   const F4 o = dot_1x4(wr);
   if (lane == 0) {
     const rsrc_t rp = co_rsrc(uni(F.tproj));
@@ -570,7 +568,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
 }
 
 // ---- MoE stage A -------------------------------------------------------------------------------------
-SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
+SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, float& h0, float& h1) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   const bool is_dense = gw <= uni(P.E);
@@ -586,16 +584,16 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     for (int j = 0; j < 4; ++j) dwr[j] = ld16(drow + 8 * j);
   }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.post_ln) + 2 * tid);
-  float h0, h1, r0, r1;
+  float r0, r1;
   {
-    const uint32_t th = flow_tag(base, li, FS_IN), tr = flow_tag(base, li, FS_OUT);
-    const rsrc_t rh = co_rsrc(uni(F.th[1])), rr = co_rsrc(uni(F.tmix));
+    const uint32_t tr = flow_tag(base, li, FS_OUT);
+    const rsrc_t rr = co_rsrc(uni(F.tmix));
     unsigned spins = 0;
     fstamp(P, 8, 0);
     for (;;) {
-      const uint2 a = ldw2(rh, 2 * tid), b = ldw2(rr, 2 * tid);
-      const bool ok = tag_ok(a.x, th) && tag_ok(a.y, th) && tag_ok(b.x, tr) && tag_ok(b.y, tr);
-      h0 = lo_h(a.x); h1 = lo_h(a.y); r0 = lo_h(b.x); r1 = lo_h(b.y);
+      const uint2 b = ldw2(rr, 2 * tid);
+      const bool ok = tag_ok(b.x, tr) && tag_ok(b.y, tr);
+      r0 = lo_h(b.x); r1 = lo_h(b.y);
       const int v = flow_round(ok, spins, uni(P.bar) + 32);
       if (v > 0) break;
       if (v < 0) return false;
@@ -603,7 +601,7 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     fstamp(P, 9, spins);
   }
   const uint32_t ta = flow_tag(base, li, FS_A);
-  flow_prologue(h0, h1, true, r0, r1, lnw, wg == 0, co_rsrc(uni(F.th[0])), ta, nullptr);
+  flow_prologue(h0, h1, true, r0, r1, lnw, nullptr);
   if (is_dense) {
     uint32_t xp[16]; float sx[4];
     lds_get_x(0, lane, xp, sx);
@@ -810,7 +808,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
 }
 
 // ---- head -------------------------------------------------------------------------------------------
-SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t base) {
+SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t base, float h0, float h1) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   Lds& L = g_L;
@@ -829,24 +827,24 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
   };
   load_group(cur, gw, 0);
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(P.final_norm) + 2 * tid);
-  float h0, h1, r0, r1;
+  float r0, r1;
   {
-    const uint32_t th = flow_tag(base, nl - 1, FS_A), tr = flow_tag(base, nl - 1, FS_C);
-    const rsrc_t rh = co_rsrc(uni(F.th[0])), rr = co_rsrc(uni(F.tmoe));
+    const uint32_t tr = flow_tag(base, nl - 1, FS_C);
+    const rsrc_t rr = co_rsrc(uni(F.tmoe));
     unsigned spins = 0;
     fstamp(P, 14, 0);
     for (;;) {
-      const uint2 a = ldw2(rh, 2 * tid), b = ldw2(rr, 2 * tid);
-      const bool ok = tag_ok(a.x, th) && tag_ok(a.y, th) && tag_ok(b.x, tr) && tag_ok(b.y, tr);
-      h0 = lo_h(a.x); h1 = lo_h(a.y); r0 = lo_h(b.x); r1 = lo_h(b.y);
+      const uint2 b = ldw2(rr, 2 * tid);
+      const bool ok = tag_ok(b.x, tr) && tag_ok(b.y, tr);
+      r0 = lo_h(b.x); r1 = lo_h(b.y);
       const int v = flow_round(ok, spins, uni(P.bar) + 32);
       if (v > 0) break;
       if (v < 0) return false;
     }
     fstamp(P, 15, spins);
   }
-  const uint32_t thd = flow_tag(base, nl, 0), thd32 = flow_tag32(base, nl, 0);
-  flow_prologue(h0, h1, true, r0, r1, lnw, wg == 0, co_rsrc(uni(F.th[1])), thd, uni(P.normed));
+  const uint32_t thd32 = flow_tag32(base, nl, 0);
+  flow_prologue(h0, h1, true, r0, r1, lnw, wg == 0 ? uni(P.normed) : nullptr);
   for (int chunk = gw; chunk < nchunks; chunk += NW) {
 #pragma unroll 1
     for (int g4 = 0; g4 < 16; ++g4) {
@@ -931,10 +929,11 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
   const uint32_t base = uni(g_K.base);
   const int pos = uni(g_K.pos);
   const int nl = uni(P.n_layers);
+  float h0 = 0.0f, h1 = 0.0f;          // this thread's two elements of the residual stream
   for (int li = 0; li < nl; ++li) {
     const LayerP& Y = g_K.layers[li];
     const int is_linear = uni(Y.is_linear);
-    if (!flow_in(F, Y, li, pos, base)) return;
+    if (!flow_in(F, Y, li, pos, base, h0, h1)) return;
     if (is_linear) {
       if (!flow_gdn(F, Y, li, base)) return;
       if (!flow_out(F, Y, li, 0, base)) return;
@@ -942,7 +941,7 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
       if (!flow_sdpa(F, Y, li, pos, base)) return;
       if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base)) return;
     }
-    if (!flow_moe_a(F, Y, li, base)) return;
+    if (!flow_moe_a(F, Y, li, base, h0, h1)) return;
     uint32_t carry[4];
     if (!flow_moe_b(F, Y, li, base, carry)) return;
     {
@@ -952,7 +951,7 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
                       last ? uni(P.vocab) : (uni(Z.is_linear) ? SL_GDN_IN_N : SL_ATT_QKV_N), last ? 1 : 0, carry)) return;
     }
   }
-  flow_head(F, pos, out_off, feed, base);
+  flow_head(F, pos, out_off, feed, base, h0, h1);
   fstamp(P, 18, 0);
   if (uni(P.tstamp) && threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == 100))
     uni(P.tstamp)[blockIdx.x ? 2048 : 0] = (unsigned long long)g_L.bar.nts;
