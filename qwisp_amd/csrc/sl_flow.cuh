@@ -187,9 +187,38 @@ SL_DEV void flow_prologue(float& h0, float& h1, bool has_r, float r0, float r1, 
   __syncthreads();
 }
 
+// Stores of a wave are acknowledged in order with its loads, so a wave that has just published results cannot
+// finish a poll before the write has travelled to memory and back.  All tagged results of a stage are therefore
+// gathered in LDS and written by wave 15 (full 64-byte lines), and wave 15 never takes part in a poll.
+constexpr int PUB_WAVE = DEC_WAVES - 1;
+
 #define FLOW_IDS const int tid = fresh_v(threadIdx.x), lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); \
                  const int wg = fresh_s(blockIdx.x), G = fresh_s(gridDim.x), NW = G * DEC_WAVES, gw = wg * DEC_WAVES + wave; \
                  (void)tid; (void)lane; (void)wave; (void)wg; (void)G; (void)NW; (void)gw
+
+// Waves 0..7 poll a 2048-long tagged vector (4 words per thread); every thread then takes the pair it owns.
+SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, float& r0, float& r1, unsigned id) {
+  const int tid = fresh_v(threadIdx.x);
+  uint32_t* rs = reinterpret_cast<uint32_t*>(g_L.part);       // [1024] packed pairs
+  const rsrc_t rr = co_rsrc(vec);
+  unsigned spins = 0;
+  fstamp(P, id, 0);
+  for (;;) {
+    bool ok = true;
+    if (tid < 512) {
+      const uint4 b = ldw4(rr, 4 * tid);
+      ok = tag_ok(b.x, tag) && tag_ok(b.y, tag) && tag_ok(b.z, tag) && tag_ok(b.w, tag);
+      *reinterpret_cast<uint2*>(&rs[2 * tid]) = make_uint2((b.x & 0xffffu) | (b.y << 16), (b.z & 0xffffu) | (b.w << 16));
+    }
+    const int v = flow_round(ok, spins, uni(P.bar) + 32);
+    if (v > 0) break;
+    if (v < 0) return false;
+  }
+  fstamp(P, id + 1, spins);
+  const uint32_t w = rs[tid];
+  r0 = lo_h(w); r1 = hi_h(w);
+  return true;
+}
 
 // ---- stage 1: input norm + in-projection ------------------------------------------------------------
 SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base, float& h0, float& h1) {
@@ -210,27 +239,19 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
     const uint32_t w = *reinterpret_cast<const uint32_t*>(uni(P.hA) + 2 * tid);   // embedded row from k_embed
     h0 = lo_h(w); h1 = hi_h(w);
   } else {
-    const uint32_t tr = flow_tag(base, li - 1, FS_C);
-    const rsrc_t rr = co_rsrc(uni(F.tmoe));
-    unsigned spins = 0;
-    fstamp(P, 0, 0);
-    for (;;) {
-      const uint2 b = ldw2(rr, 2 * tid);
-      const bool ok = tag_ok(b.x, tr) && tag_ok(b.y, tr);
-      r0 = lo_h(b.x); r1 = lo_h(b.y);
-      const int v = flow_round(ok, spins, uni(P.bar) + 32);
-      if (v > 0) break;
-      if (v < 0) return false;
-    }
-    fstamp(P, 1, spins);
+    if (!poll_vec2048(P, uni(F.tmoe), flow_tag(base, li - 1, FS_C), r0, r1, 0)) return false;
   }
   const uint32_t tin = flow_tag(base, li, FS_IN);
   flow_prologue(h0, h1, li > 0, r0, r1, lnw, nullptr);
   const F4 o = dot_1x4(wr);
   if (lane == 0) {
-    const rsrc_t rp = co_rsrc(uni(F.tproj));
 #pragma unroll
-    for (int j = 0; j < 4; ++j) if (valid[j]) stw1(rp, gw + j * NW, tagged(o.v[j], tin));
+    for (int j = 0; j < 4; ++j) g_L.pub[j * 16 + wave] = tagged(o.v[j], tin);
+  }
+  __syncthreads();
+  if (wave == PUB_WAVE) {
+    const int row = wg * DEC_WAVES + (lane & 15) + (lane >> 4) * NW;      // four runs of 16 consecutive rows
+    if (row < N) stw1(co_rsrc(uni(F.tproj)), row, g_L.pub[lane]);
   }
   return true;
 }
@@ -323,7 +344,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     for (int i = 0; i < 4; ++i) { s[i] = fmaf(kk[i], delta, s[i]); acc = fmaf(s[i], qq[i], acc); }
     const float y = tree_sum<32>(acc);
     const int dv = dvb * 16 + dvl;
-    if (l32 == 0) stw1(co_rsrc(uni(F.tycore)), hv * 128 + dv, tagged(y, flow_tag(base, li, FS_CORE)));
+    if (l32 == 0) L.pub[dvl] = tagged(y, flow_tag(base, li, FS_CORE));
     *reinterpret_cast<float4*>(uni(Y.state[par ^ 1]) + ((size_t)hv * 128 + dv) * 128 + 4 * l32) = make_float4(s[0], s[1], s[2], s[3]);
   }
   if (tid < 272 && (tid >= 256 || ((hv & 1) == 0 && dvb == 0))) {
@@ -332,6 +353,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     hout[2 * SL_CONV_DIM + ch] = f2h(newest);
   }
   __syncthreads();
+  if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tycore)), hv * 128 + dvb * 16 + lane, L.pub[lane]);
   return true;
 }
 
@@ -512,28 +534,41 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     for (int i = 0; i < 4; ++i) r[i] = tagged(f16r(f16r(O[i] / Ls) * sigmoid16(gt[i])), tmerge);
     if (!fail) stw4(co_rsrc(uni(F.tycore)), h * 256 + 4 * lane, r[0], r[1], r[2], r[3]);
   }
-  // every thread prepares 4 consecutive elements of the 4096-long activation
+  // every thread prepares 4 consecutive elements of the 4096-long activation; waves 0..7 fetch them, for
+  // themselves and for the wave 8 above (handed over through LDS)
   const int e0 = 256 * wave + 4 * lane;
   float out[4], z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   {
+    uint4* ystage = reinterpret_cast<uint4*>(g_vt);            // [512] y chunks, [512] z chunks of waves 8..15
     const uint32_t ty = lin ? tcore : tmerge;
     const rsrc_t ry = co_rsrc(uni(F.tycore)), rz = co_rsrc(uni(F.tproj));
+    uint4 a = make_uint4(0, 0, 0, 0), b = make_uint4(0, 0, 0, 0);
     unsigned spins = 0;
     fstamp(P, 6, 0);
     for (;;) {
-      const uint4 a = ldw4(ry, e0);
-      bool ok = tag_ok(a.x, ty) && tag_ok(a.y, ty) && tag_ok(a.z, ty) && tag_ok(a.w, ty);
-      out[0] = lo_h(a.x); out[1] = lo_h(a.y); out[2] = lo_h(a.z); out[3] = lo_h(a.w);
-      if (lin) {
-        const uint4 b = ldw4(rz, 8192 + e0);
-        ok = ok && tag_ok(b.x, tin) && tag_ok(b.y, tin) && tag_ok(b.z, tin) && tag_ok(b.w, tin);
-        z[0] = lo_h(b.x); z[1] = lo_h(b.y); z[2] = lo_h(b.z); z[3] = lo_h(b.w);
+      bool ok = true;
+      if (wave < 8) {
+        a = ldw4(ry, e0);
+        const uint4 a2 = ldw4(ry, e0 + 2048);
+        ok = tag_ok(a.x, ty) && tag_ok(a.y, ty) && tag_ok(a.z, ty) && tag_ok(a.w, ty) &&
+             tag_ok(a2.x, ty) && tag_ok(a2.y, ty) && tag_ok(a2.z, ty) && tag_ok(a2.w, ty);
+        ystage[tid] = a2;
+        if (lin) {
+          b = ldw4(rz, 8192 + e0);
+          const uint4 b2 = ldw4(rz, 8192 + e0 + 2048);
+          ok = ok && tag_ok(b.x, tin) && tag_ok(b.y, tin) && tag_ok(b.z, tin) && tag_ok(b.w, tin) &&
+               tag_ok(b2.x, tin) && tag_ok(b2.y, tin) && tag_ok(b2.z, tin) && tag_ok(b2.w, tin);
+          ystage[512 + tid] = b2;
+        }
       }
       const int v = flow_round(ok, spins, uni(P.bar) + 32);
       if (v > 0) break;
       if (v < 0) return false;
     }
     fstamp(P, 7, spins);
+    if (wave >= 8) { a = ystage[tid - 512]; if (lin) b = ystage[tid]; }
+    out[0] = lo_h(a.x); out[1] = lo_h(a.y); out[2] = lo_h(a.z); out[3] = lo_h(a.w);
+    z[0] = lo_h(b.x); z[1] = lo_h(b.y); z[2] = lo_h(b.z); z[3] = lo_h(b.w);
   }
   if (lin) {
     float nw[4];
@@ -563,7 +598,11 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   }
   __syncthreads();
   const float o = dot_2x1(wr);
-  if (lane == 0 && valid) stw1(co_rsrc(uni(F.tmix)), gw, tagged(o, flow_tag(base, li, FS_OUT)));
+  if (wg * DEC_WAVES < H) {                       // uniform per workgroup
+    if (lane == 0) g_L.pub[wave] = tagged(o, flow_tag(base, li, FS_OUT));
+    __syncthreads();
+    if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tmix)), wg * DEC_WAVES + lane, g_L.pub[lane]);
+  }
   return true;
 }
 
@@ -585,21 +624,7 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
   }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.post_ln) + 2 * tid);
   float r0, r1;
-  {
-    const uint32_t tr = flow_tag(base, li, FS_OUT);
-    const rsrc_t rr = co_rsrc(uni(F.tmix));
-    unsigned spins = 0;
-    fstamp(P, 8, 0);
-    for (;;) {
-      const uint2 b = ldw2(rr, 2 * tid);
-      const bool ok = tag_ok(b.x, tr) && tag_ok(b.y, tr);
-      r0 = lo_h(b.x); r1 = lo_h(b.y);
-      const int v = flow_round(ok, spins, uni(P.bar) + 32);
-      if (v > 0) break;
-      if (v < 0) return false;
-    }
-    fstamp(P, 9, spins);
-  }
+  if (!poll_vec2048(P, uni(F.tmix), flow_tag(base, li, FS_OUT), r0, r1, 8)) return false;
   const uint32_t ta = flow_tag(base, li, FS_A);
   flow_prologue(h0, h1, true, r0, r1, lnw, nullptr);
   if (is_dense) {
@@ -611,11 +636,23 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
 #pragma unroll
     for (int i = 0; i < 16; ++i) { acc = fmaf(lo_h(xp[i]), lo_h(dww[i]), acc); acc = fmaf(hi_h(xp[i]), hi_h(dww[i]), acc); }
     acc = tree_sum<64>(acc);
-    if (lane == 0) { if (gw < uni(P.E)) stw1(co_rsrc(uni(F.trlog)), gw, tagged(acc, ta)); else stw1(co_rsrc(uni(F.tsg)), 0, tagged(acc, ta)); }
+    if (lane == 0) g_L.pub[wave] = tagged(acc, ta);
   }
   if (is_pair) {
     const F2 gu = dot_1x2(wr);
-    if (lane == 0) stw1(co_rsrc(uni(F.tsh)), (int)prow, tagged(swiglu16(f16r(gu.v[0]), f16r(gu.v[1])), ta));
+    if (lane == 0) g_L.pub[wave] = tagged(swiglu16(f16r(gu.v[0]), f16r(gu.v[1])), ta);
+  }
+  {
+    const int g0 = wg * DEC_WAVES, E = uni(P.E);
+    if (g0 <= E || (g0 >= 512 && g0 < 1024)) {     // uniform per workgroup: it holds router rows, the gate row or pairs
+      __syncthreads();
+      if (wave == PUB_WAVE && lane < 16) {
+        const int g = g0 + lane;
+        if (g < E) stw1(co_rsrc(uni(F.trlog)), g, g_L.pub[lane]);
+        else if (g == E) stw1(co_rsrc(uni(F.tsg)), 0, g_L.pub[lane]);
+        else if (g >= 512 && g < 1024) stw1(co_rsrc(uni(F.tsh)), g - 512, g_L.pub[lane]);
+      }
+    }
   }
   return true;
 }
@@ -714,8 +751,10 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
   }
   if (active) {
     const F2 gu = dot_1x2(wr);
-    if (lane == 0) stw1(co_rsrc(uni(F.tact)), k * 512 + i, tagged(swiglu16(f16r(gu.v[0]), f16r(gu.v[1])), flow_tag(base, li, FS_B)));
+    if (lane == 0) L.pub[wave] = tagged(swiglu16(f16r(gu.v[0]), f16r(gu.v[1])), flow_tag(base, li, FS_B));
   }
+  __syncthreads();
+  if (wave == PUB_WAVE && lane < 16 && wg * DEC_WAVES + lane < 8 * 512) stw1(co_rsrc(uni(F.tact)), wg * DEC_WAVES + lane, L.pub[lane]);
   return true;
 }
 
@@ -745,34 +784,38 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
       sbv[qq] = SB[row * 8 + (li16 >> 1)];
     }
   }
-  float sgate_logit = 0.0f;
-  uint4 a4 = make_uint4(0, 0, 0, 0), s4 = make_uint4(0, 0, 0, 0);
   {
+    // waves 0..7 fetch the nine activation rows (8 x 512 routed + 512 shared) and the shared-gate logit
     const rsrc_t ra = co_rsrc(uni(F.tact)), rs = co_rsrc(uni(F.tsh)), rg = co_rsrc(uni(F.tsg));
     unsigned spins = 0;
     fstamp(P, 12, 0);
     for (;;) {
-      a4 = ldw4(ra, 4 * tid);
-      bool ok = tag_ok(a4.x, tb) && tag_ok(a4.y, tb) && tag_ok(a4.z, tb) && tag_ok(a4.w, tb);
-      if (tid < 128) { s4 = ldw4(rs, 4 * tid); ok = ok && tag_ok(s4.x, ta) && tag_ok(s4.y, ta) && tag_ok(s4.z, ta) && tag_ok(s4.w, ta); }
-      if (tid < 8) { const uint32_t w = ldw1(rg, 0); ok = ok && tag_ok(w, ta); sgate_logit = lo_h(w); }
+      bool ok = true;
+      if (wave < 8) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          // thread t holds elements 4(t%128).. of slot t/128: packed pairs 2(t%128), 2(t%128)+1
+          const int t = tid + 512 * c, slot = t >> 7, pi = 2 * (t & 127);
+          const uint4 a4 = ldw4(ra, 4 * t);
+          ok = ok && tag_ok(a4.x, tb) && tag_ok(a4.y, tb) && tag_ok(a4.z, tb) && tag_ok(a4.w, tb);
+          *reinterpret_cast<uint2*>(&xc[(slot * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
+              make_uint2((a4.x & 0xffffu) | (a4.y << 16), (a4.z & 0xffffu) | (a4.w << 16));
+        }
+        if (tid < 128) {
+          const int pi = 2 * tid;
+          const uint4 s4 = ldw4(rs, 4 * tid);
+          ok = ok && tag_ok(s4.x, ta) && tag_ok(s4.y, ta) && tag_ok(s4.z, ta) && tag_ok(s4.w, ta);
+          *reinterpret_cast<uint2*>(&xc[(8 * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
+              make_uint2((s4.x & 0xffffu) | (s4.y << 16), (s4.z & 0xffffu) | (s4.w << 16));
+        }
+        if (tid == 0) { const uint32_t w = ldw1(rg, 0); ok = ok && tag_ok(w, ta); L.gb[1] = lo_h(w); }
+      }
       const int v = flow_round(ok, spins, uni(P.bar) + 32);
       if (v > 0) break;
       if (v < 0) return false;
     }
     fstamp(P, 13, spins);
   }
-  touch_done(carry[0]); touch_done(carry[1]); touch_done(carry[2]); touch_done(carry[3]);
-  {
-    // thread t holds elements 4(t%128).. of slot t/128: packed pairs 2(t%128), 2(t%128)+1
-    const int slot = tid >> 7, pi = 2 * (tid & 127);
-    *reinterpret_cast<uint2*>(&xc[(slot * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
-        make_uint2((a4.x & 0xffffu) | (a4.y << 16), (a4.z & 0xffffu) | (a4.w << 16));
-    if (tid < 128)
-      *reinterpret_cast<uint2*>(&xc[(8 * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
-          make_uint2((s4.x & 0xffffu) | (s4.y << 16), (s4.z & 0xffffu) | (s4.w << 16));
-  }
-  __syncthreads();
 #pragma unroll
   for (int qq = 0; qq < 2; ++qq) {
     const int un = wave + 16 * qq, ql = un / 9, slot = un % 9;
@@ -794,13 +837,13 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
     }
   }
   __syncthreads();
-  if (tid < 8) {
-    const int ql = tid >> 2, sb4 = tid & 3;
+  if (wave == PUB_WAVE && lane < 8) {
+    const int ql = lane >> 2, sb4 = lane & 3;
     const int quad = wg * 2 + ql;
     float acc = 0.0f;
 #pragma unroll
     for (int k = 0; k < 8; ++k) acc = f16r(acc + f16r(L.dbuf[(ql * 9 + k) * 4 + sb4] * L.scores[k]));
-    const float s = sigmoid16(sgate_logit);
+    const float s = sigmoid16(L.gb[1]);
     stw1(co_rsrc(uni(F.tmoe)), quad * 4 + sb4, tagged(f16r(acc + f16r(s * L.dbuf[(ql * 9 + 8) * 4 + sb4])), flow_tag(base, li, FS_C)));
   }
   __syncthreads();
@@ -828,21 +871,7 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
   load_group(cur, gw, 0);
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(P.final_norm) + 2 * tid);
   float r0, r1;
-  {
-    const uint32_t tr = flow_tag(base, nl - 1, FS_C);
-    const rsrc_t rr = co_rsrc(uni(F.tmoe));
-    unsigned spins = 0;
-    fstamp(P, 14, 0);
-    for (;;) {
-      const uint2 b = ldw2(rr, 2 * tid);
-      const bool ok = tag_ok(b.x, tr) && tag_ok(b.y, tr);
-      r0 = lo_h(b.x); r1 = lo_h(b.y);
-      const int v = flow_round(ok, spins, uni(P.bar) + 32);
-      if (v > 0) break;
-      if (v < 0) return false;
-    }
-    fstamp(P, 15, spins);
-  }
+  if (!poll_vec2048(P, uni(F.tmoe), flow_tag(base, nl - 1, FS_C), r0, r1, 14)) return false;
   const uint32_t thd32 = flow_tag32(base, nl, 0);
   flow_prologue(h0, h1, true, r0, r1, lnw, wg == 0 ? uni(P.normed) : nullptr);
   for (int chunk = gw; chunk < nchunks; chunk += NW) {
@@ -866,7 +895,8 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
   }
   if (lane == 0) { L.red[wave] = bv; L.ired[wave] = bi; }
   __syncthreads();
-  if (tid == 0) {
+  if (wave == PUB_WAVE && lane == 0) {
+    bv = L.red[0]; bi = L.ired[0];
     for (int w = 1; w < DEC_WAVES; ++w)
       if (L.red[w] > bv || (L.red[w] == bv && L.ired[w] < bi)) { bv = L.red[w]; bi = L.ired[w]; }
     stw4(co_rsrc(uni(F.tcand)), wg * 4, __float_as_uint(bv), (uint32_t)bi, thd32, thd32);
