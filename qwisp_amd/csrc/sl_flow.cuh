@@ -133,17 +133,24 @@ SL_DEV void fstamp(const DecodeP& P, unsigned id, unsigned v) {
     if (n < 2040) { uni(P.tstamp)[(blockIdx.x ? 2048 : 0) + 1 + n] = ((unsigned long long)wall_clock64() << 16) | (id << 8) | (v > 255u ? 255u : v); g_L.bar.nts = n + 1; }
   }
 }
-// One polling round's verdict for the whole workgroup.  Returns 1 = all tags present, 0 = retry,
-// -1 = give up (spin limit reached here, or another workgroup raised the abort word).
+// One polling round's verdict for the whole workgroup: 1 = all tags present, 0 = retry, -1 = give up (spin
+// limit reached here, or another workgroup raised the abort word).  One barrier per round: a wave with a
+// missing tag marks slot (round % 3) in LDS before the barrier, everybody reads it after, and thread 0 then
+// clears the slot of the round before (nobody can still be reading that one), so a successful round leaves
+// all three slots clear for the next stage.
 SL_DEV int flow_round(bool ok, unsigned& spins, unsigned* abort_word) {
-  if (__syncthreads_and(ok ? 1 : 0)) return 1;
-  ++spins;
-  int stop = 0;
-  if (threadIdx.x == 0 && (spins > FLOW_SPIN_LIMIT || ((spins & 255u) == 0 && ld_co32(abort_word) != 0))) {
+  const unsigned slot = spins % 3u;
+  if (!__all(ok ? 1 : 0) && (threadIdx.x & 63) == 0) g_L.pf[slot] = 1;
+  if (threadIdx.x == 0 && (spins > FLOW_SPIN_LIMIT || ((spins & 63u) == 63u && ld_co32(abort_word) != 0))) {
     st_co32(abort_word, 1u);
-    stop = 1;
+    g_L.pf[3] = 1;
   }
-  if (__syncthreads_or(stop)) return -1;
+  __syncthreads();
+  const int failed = g_L.pf[slot], dead = g_L.pf[3];
+  if (threadIdx.x == 0) g_L.pf[(spins + 2u) % 3u] = 0;
+  if (dead) return -1;
+  if (!failed) return 1;
+  ++spins;
   __builtin_amdgcn_s_sleep(1);
   return 0;
 }
@@ -253,6 +260,7 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
     const int row = wg * DEC_WAVES + (lane & 15) + (lane >> 4) * NW;      // four runs of 16 consecutive rows
     if (row < N) stw1(co_rsrc(uni(F.tproj)), row, g_L.pub[lane]);
   }
+ 
   return true;
 }
 
@@ -354,6 +362,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   }
   __syncthreads();
   if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tycore)), hv * 128 + dvb * 16 + lane, L.pub[lane]);
+ 
   return true;
 }
 
@@ -472,6 +481,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
     }
     __syncthreads();
   }
+ 
   return true;
 }
 
@@ -603,6 +613,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     __syncthreads();
     if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tmix)), wg * DEC_WAVES + lane, g_L.pub[lane]);
   }
+ 
   return true;
 }
 
@@ -654,6 +665,7 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
       }
     }
   }
+ 
   return true;
 }
 
@@ -755,6 +767,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
   }
   __syncthreads();
   if (wave == PUB_WAVE && lane < 16 && wg * DEC_WAVES + lane < 8 * 512) stw1(co_rsrc(uni(F.tact)), wg * DEC_WAVES + lane, L.pub[lane]);
+ 
   return true;
 }
 
@@ -847,6 +860,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
     stw1(co_rsrc(uni(F.tmoe)), quad * 4 + sb4, tagged(f16r(acc + f16r(s * L.dbuf[(ql * 9 + 8) * 4 + sb4])), flow_tag(base, li, FS_C)));
   }
   __syncthreads();
+ 
   return true;
 }
 
@@ -951,6 +965,7 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
       const int bit = (tid < nl) ? (Fp->d.st[1 + tid] & 1) : 0;
       const unsigned long long m = __ballot(bit);
       if (tid == 0) { g_K.parity = m; g_K.pos = Fp->d.st[0]; g_K.base = ld_co32(Fp->d.bar + 16); g_L.bar.nts = 0; }
+      if (tid < 4) g_L.pf[tid] = 0;
     }
     __syncthreads();
   }
