@@ -265,19 +265,22 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
 }
 
 // ---- GDN stage 2: conv + prep + gated delta rule ------------------------------------------------------
-SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
+// New conv-history samples of a thread's channel; written to memory by the next stage once its poll is over
+// (a store issued here would hold up that poll until it is acknowledged).
+struct GdnHist { uint32_t t12; uint32_t tnew; };
+SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, GdnHist& gh) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   Lds& L = g_L;
   if (wg >= 256) return true;
   const int par = (int)((uni(g_K.parity) >> li) & 1ull);
   const uint16_t* hin = uni(Y.hist[par]);
-  uint16_t* hout = uni(Y.hist[par ^ 1]);
   const int hv = wg >> 3, dvb = wg & 7, hk = hv >> 1;
   const int half = lane >> 5, l32 = lane & 31;
+  // waves 8..15 hold the recurrent state (they take no part in this stage's or the next stage's poll)
   float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (wave < 8) {
-    const int dv = dvb * 16 + wave * 2 + half;
+  if (wave >= 8) {
+    const int dv = dvb * 16 + (wave - 8) * 2 + half;
     const float4 v4 = *reinterpret_cast<const float4*>(uni(Y.state[par]) + ((size_t)hv * 128 + dv) * 128 + 4 * l32);
     s[0] = v4.x; s[1] = v4.y; s[2] = v4.z; s[3] = v4.w;
   }
@@ -336,9 +339,9 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     buf[2 * lane] = y0; buf[2 * lane + 1] = y1;
   }
   __syncthreads();
-  if (wave < 8) {
+  if (wave >= 8) {
     const float g = L.gb[0], beta = L.gb[1];
-    const int dvl = wave * 2 + half;
+    const int dvl = (wave - 8) * 2 + half;
     float kk[4], qq[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) { kk[i] = L.k[4 * l32 + i]; qq[i] = L.q[4 * l32 + i]; }
@@ -355,11 +358,8 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     if (l32 == 0) L.pub[dvl] = tagged(y, flow_tag(base, li, FS_CORE));
     *reinterpret_cast<float4*>(uni(Y.state[par ^ 1]) + ((size_t)hv * 128 + dv) * 128 + 4 * l32) = make_float4(s[0], s[1], s[2], s[3]);
   }
-  if (tid < 272 && (tid >= 256 || ((hv & 1) == 0 && dvb == 0))) {
-    hout[ch] = f2h(tap[1]);
-    hout[SL_CONV_DIM + ch] = f2h(tap[2]);
-    hout[2 * SL_CONV_DIM + ch] = f2h(newest);
-  }
+  gh.t12 = (uint32_t)traw[1] | ((uint32_t)traw[2] << 16);
+  gh.tnew = f2h(newest);
   __syncthreads();
   if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tycore)), hv * 128 + dvb * 16 + lane, L.pub[lane]);
  
@@ -486,7 +486,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
 }
 
 // ---- K = 4096 projection (GDN out_proj with gated rmsnorm prologue / attention merge + o_proj) ---------
-SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t base) {
+SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t base, const GdnHist& gh) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   const bool lin = uni(Y.is_linear) != 0;
@@ -577,6 +577,18 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     }
     fstamp(P, 7, spins);
     if (wave >= 8) { a = ystage[tid - 512]; if (lin) b = ystage[tid]; }
+    if (lin && tid < 272) {
+      // history shift of the linear-attention layer: rows 1,2 of the old history and the new sample (each
+      // channel is written by one workgroup)
+      const int hv = wg >> 3, dvb = wg & 7, hk = hv >> 1;
+      const int ch = tid < 128 ? hk * 128 + tid : (tid < 256 ? 2048 + hk * 128 + (tid - 128) : 4096 + hv * 128 + dvb * 16 + (tid - 256));
+      if (tid >= 256 || ((hv & 1) == 0 && dvb == 0)) {
+        uint16_t* hout = uni(Y.hist[(int)(((uni(g_K.parity) >> li) & 1ull) ^ 1ull)]);
+        hout[ch] = (uint16_t)(gh.t12 & 0xffffu);
+        hout[SL_CONV_DIM + ch] = (uint16_t)(gh.t12 >> 16);
+        hout[2 * SL_CONV_DIM + ch] = (uint16_t)gh.tnew;
+      }
+    }
     out[0] = lo_h(a.x); out[1] = lo_h(a.y); out[2] = lo_h(a.z); out[3] = lo_h(a.w);
     z[0] = lo_h(b.x); z[1] = lo_h(b.y); z[2] = lo_h(b.z); z[3] = lo_h(b.w);
   }
@@ -979,12 +991,13 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
     const LayerP& Y = g_K.layers[li];
     const int is_linear = uni(Y.is_linear);
     if (!flow_in(F, Y, li, pos, base, h0, h1)) return;
+    GdnHist gh = {0u, 0u};
     if (is_linear) {
-      if (!flow_gdn(F, Y, li, base)) return;
-      if (!flow_out(F, Y, li, 0, base)) return;
+      if (!flow_gdn(F, Y, li, base, gh)) return;
+      if (!flow_out(F, Y, li, 0, base, gh)) return;
     } else {
       if (!flow_sdpa(F, Y, li, pos, base)) return;
-      if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base)) return;
+      if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh)) return;
     }
     if (!flow_moe_a(F, Y, li, base, h0, h1)) return;
     uint32_t carry[4];
