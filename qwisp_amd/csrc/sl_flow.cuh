@@ -221,7 +221,6 @@ SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, fl
     if (v > 0) break;
     if (v < 0) return false;
   }
-  fstamp(P, id + 1, spins);
   const uint32_t w = rs[tid];
   r0 = lo_h(w); r1 = hi_h(w);
   return true;
@@ -260,6 +259,7 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
     const int row = wg * DEC_WAVES + (lane & 15) + (lane >> 4) * NW;      // four runs of 16 consecutive rows
     if (row < N) stw1(co_rsrc(uni(F.tproj)), row, g_L.pub[lane]);
   }
+ 
  
   return true;
 }
@@ -362,6 +362,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
   gh.tnew = f2h(newest);
   __syncthreads();
   if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tycore)), hv * 128 + dvb * 16 + lane, L.pub[lane]);
+ 
  
   return true;
 }
@@ -482,7 +483,24 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
     __syncthreads();
   }
  
+ 
   return true;
+}
+
+// History shift of a linear-attention layer: rows 1,2 of the old history and the new sample (each channel is
+// written by one workgroup).
+SL_DEV void store_hist(const LayerP& Y, int li, const GdnHist& gh) {
+  const int tid = fresh_v(threadIdx.x), wg = fresh_s(blockIdx.x);
+  if (tid < 272) {
+    const int hv = wg >> 3, dvb = wg & 7, hk = hv >> 1;
+    const int ch = tid < 128 ? hk * 128 + tid : (tid < 256 ? 2048 + hk * 128 + (tid - 128) : 4096 + hv * 128 + dvb * 16 + (tid - 256));
+    if (tid >= 256 || ((hv & 1) == 0 && dvb == 0)) {
+      uint16_t* hout = uni(Y.hist[(int)(((uni(g_K.parity) >> li) & 1ull) ^ 1ull)]);
+      hout[ch] = (uint16_t)(gh.t12 & 0xffffu);
+      hout[SL_CONV_DIM + ch] = (uint16_t)(gh.t12 >> 16);
+      hout[2 * SL_CONV_DIM + ch] = (uint16_t)gh.tnew;
+    }
+  }
 }
 
 // ---- K = 4096 projection (GDN out_proj with gated rmsnorm prologue / attention merge + o_proj) ---------
@@ -544,6 +562,10 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     for (int i = 0; i < 4; ++i) r[i] = tagged(f16r(f16r(O[i] / Ls) * sigmoid16(gt[i])), tmerge);
     if (!fail) stw4(co_rsrc(uni(F.tycore)), h * 256 + 4 * lane, r[0], r[1], r[2], r[3]);
   }
+  if (wg * DEC_WAVES >= H) {                       // no output row here (uniform per workgroup): nothing to fetch
+    if (lin) store_hist(Y, li, gh);
+    return true;
+  }
   // every thread prepares 4 consecutive elements of the 4096-long activation; waves 0..7 fetch them, for
   // themselves and for the wave 8 above (handed over through LDS)
   const int e0 = 256 * wave + 4 * lane;
@@ -577,18 +599,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     }
     fstamp(P, 7, spins);
     if (wave >= 8) { a = ystage[tid - 512]; if (lin) b = ystage[tid]; }
-    if (lin && tid < 272) {
-      // history shift of the linear-attention layer: rows 1,2 of the old history and the new sample (each
-      // channel is written by one workgroup)
-      const int hv = wg >> 3, dvb = wg & 7, hk = hv >> 1;
-      const int ch = tid < 128 ? hk * 128 + tid : (tid < 256 ? 2048 + hk * 128 + (tid - 128) : 4096 + hv * 128 + dvb * 16 + (tid - 256));
-      if (tid >= 256 || ((hv & 1) == 0 && dvb == 0)) {
-        uint16_t* hout = uni(Y.hist[(int)(((uni(g_K.parity) >> li) & 1ull) ^ 1ull)]);
-        hout[ch] = (uint16_t)(gh.t12 & 0xffffu);
-        hout[SL_CONV_DIM + ch] = (uint16_t)(gh.t12 >> 16);
-        hout[2 * SL_CONV_DIM + ch] = (uint16_t)gh.tnew;
-      }
-    }
+    if (lin) store_hist(Y, li, gh);
     out[0] = lo_h(a.x); out[1] = lo_h(a.y); out[2] = lo_h(a.z); out[3] = lo_h(a.w);
     z[0] = lo_h(b.x); z[1] = lo_h(b.y); z[2] = lo_h(b.z); z[3] = lo_h(b.w);
   }
@@ -625,6 +636,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     __syncthreads();
     if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tmix)), wg * DEC_WAVES + lane, g_L.pub[lane]);
   }
+ 
  
   return true;
 }
@@ -677,6 +689,7 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
       }
     }
   }
+ 
  
   return true;
 }
@@ -780,6 +793,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
   __syncthreads();
   if (wave == PUB_WAVE && lane < 16 && wg * DEC_WAVES + lane < 8 * 512) stw1(co_rsrc(uni(F.tact)), wg * DEC_WAVES + lane, L.pub[lane]);
  
+ 
   return true;
 }
 
@@ -795,13 +809,15 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
   uint32_t* xc = reinterpret_cast<uint32_t*>(g_vt);      // [9][16][XC_STRIDE]
   const int sub = lane >> 4, li16 = lane & 15;
   const uint32_t ta = flow_tag(base, li, FS_A), tb = flow_tag(base, li, FS_B);
-  // weights of this wave's (up to) two units: routed rows were touched during stage B
+  // Waves 0..5 poll, waves 6..14 own the 18 units (two each) and fetch their down-projection rows now (they
+  // do not poll, so the cold expert rows hold nobody up), wave 15 combines and publishes.
+  const bool unit_wave = wave >= 6 && wave < 15;
   uint4 wv[2]; uint32_t sbv[2];
 #pragma unroll
   for (int qq = 0; qq < 2; ++qq) {
-    const int un = wave + 16 * qq, ql = un / 9, slot = un % 9;
+    const int un = (wave - 6) * 2 + qq, ql = un / 9, slot = un % 9;
     wv[qq] = make_uint4(0, 0, 0, 0); sbv[qq] = 0;
-    if (ql < 2) {
+    if (unit_wave) {
       const size_t row = (slot < 8 ? (size_t)L.inds[slot] * 2048 : 0) + (size_t)(wg * 2 + ql) * 4 + sub;
       const uint32_t* W = slot < 8 ? uni(Y.swd_w) : uni(Y.shd_w);
       const uint32_t* SB = slot < 8 ? uni(Y.swd_sb) : uni(Y.shd_sb);
@@ -810,28 +826,22 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
     }
   }
   {
-    // waves 0..7 fetch the nine activation rows (8 x 512 routed + 512 shared) and the shared-gate logit
+    // the nine activation rows (8 x 512 routed + 512 shared) are 1152 chunks of 4 tagged words: 3 per thread
     const rsrc_t ra = co_rsrc(uni(F.tact)), rs = co_rsrc(uni(F.tsh)), rg = co_rsrc(uni(F.tsg));
     unsigned spins = 0;
     fstamp(P, 12, 0);
     for (;;) {
       bool ok = true;
-      if (wave < 8) {
+      if (wave < 6) {
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          // thread t holds elements 4(t%128).. of slot t/128: packed pairs 2(t%128), 2(t%128)+1
-          const int t = tid + 512 * c, slot = t >> 7, pi = 2 * (t & 127);
-          const uint4 a4 = ldw4(ra, 4 * t);
-          ok = ok && tag_ok(a4.x, tb) && tag_ok(a4.y, tb) && tag_ok(a4.z, tb) && tag_ok(a4.w, tb);
+        for (int c = 0; c < 3; ++c) {
+          // chunk t holds elements 4(t%128).. of slot t/128 (slot 8 = shared): packed pairs 2(t%128), 2(t%128)+1
+          const int t = tid + 384 * c, slot = t >> 7, pi = 2 * (t & 127);
+          const uint4 a4 = (slot < 8) ? ldw4(ra, 4 * t) : ldw4(rs, 4 * (t & 127));
+          const uint32_t tx = (slot < 8) ? tb : ta;
+          ok = ok && tag_ok(a4.x, tx) && tag_ok(a4.y, tx) && tag_ok(a4.z, tx) && tag_ok(a4.w, tx);
           *reinterpret_cast<uint2*>(&xc[(slot * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
               make_uint2((a4.x & 0xffffu) | (a4.y << 16), (a4.z & 0xffffu) | (a4.w << 16));
-        }
-        if (tid < 128) {
-          const int pi = 2 * tid;
-          const uint4 s4 = ldw4(rs, 4 * tid);
-          ok = ok && tag_ok(s4.x, ta) && tag_ok(s4.y, ta) && tag_ok(s4.z, ta) && tag_ok(s4.w, ta);
-          *reinterpret_cast<uint2*>(&xc[(8 * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
-              make_uint2((s4.x & 0xffffu) | (s4.y << 16), (s4.z & 0xffffu) | (s4.w << 16));
         }
         if (tid == 0) { const uint32_t w = ldw1(rg, 0); ok = ok && tag_ok(w, ta); L.gb[1] = lo_h(w); }
       }
@@ -843,8 +853,8 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
   }
 #pragma unroll
   for (int qq = 0; qq < 2; ++qq) {
-    const int un = wave + 16 * qq, ql = un / 9, slot = un % 9;
-    if (ql < 2) {
+    const int un = (wave - 6) * 2 + qq, ql = un / 9, slot = un % 9;
+    if (unit_wave) {
       uint32_t xp[16];
       const uint4* src = reinterpret_cast<const uint4*>(&xc[(slot * 16 + li16) * XC_STRIDE]);
 #pragma unroll
@@ -872,6 +882,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
     stw1(co_rsrc(uni(F.tmoe)), quad * 4 + sb4, tagged(f16r(acc + f16r(s * L.dbuf[(ql * 9 + 8) * 4 + sb4])), flow_tag(base, li, FS_C)));
   }
   __syncthreads();
+ 
  
   return true;
 }
