@@ -72,14 +72,11 @@ struct sl_engine {
   int32_t *cand_i = nullptr, *tok_in = nullptr, *tok_out = nullptr, *st = nullptr;
   int n_cand = 0;
   // persistent single-token kernel
-  DecodeP* dec_params = nullptr;   // device copy
-  DecodeP dec_host;                // host copy
   unsigned long long* dec_tstamp = nullptr;
   unsigned* dec_bar = nullptr;
   int dec_grid = 0;                // 0 = not available (fewer than 256 compute units)
-  FlowP* flow_params = nullptr;    // device copy of the dataflow variant's parameters
+  FlowP* flow_params = nullptr;    // device copy of the single-launch step's parameters
   FlowP flow_host;
-  bool use_flow = true;
   void* pinned = nullptr;        // host staging
   size_t pinned_bytes = 0;
   // host mirrors of the device step state
@@ -280,10 +277,7 @@ void launch_decode(sl_engine* e, int out_off, bool feed) {
   const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
   hipLaunchKernelGGL(k_embed, dim3(H / 256, 1), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
-  if (e->use_flow)
-    hipLaunchKernelGGL(k_decode_flow, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0);
-  else
-    hipLaunchKernelGGL(k_decode, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->dec_params, out_off, feed ? 1 : 0);
+  hipLaunchKernelGGL(k_decode_flow, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0);
   if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
   e->pos += 1;
   for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
@@ -458,10 +452,6 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
       P.logits = e->logits; P.pm = e->pm; P.pl = e->pl; P.po = e->po; P.cand_v = e->cand_v; P.cand_i = e->cand_i;
       P.tok_in = e->tok_in; P.tok_out = e->tok_out; P.st = e->st; P.bar = e->dec_bar;
       e->dec_tstamp = dalloc<unsigned long long>(e, 2048 + 16 * 256 * 2, true);
-      e->dec_host = P;
-      e->dec_params = upload<DecodeP>(e, &P, 1, SL_LOC_HOST);
-      if (!e->dec_params) return SL_ERR_DEVICE;
-      SL_TRY(e, hipFuncSetAttribute((const void*)k_decode, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
       {
         FlowP F;
         std::memset(&F, 0, sizeof(F));
@@ -508,21 +498,18 @@ void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
 int sl_set_persistent(sl_engine* e, int enable) {
   int r = guard(e); if (r) return r;
   e->use_persistent = enable != 0;
-  e->use_flow = enable != 2;          // 2 = the barrier-separated variant of the single-launch step
   return SL_OK;
 }
 // Test/diagnostic hook: per-barrier clock stamps (100 MHz ticks) of workgroup 0 for the steps run while
 // enabled; out[0] = count, out[1..] = stamps.
 int sl_debug_stage_clock(sl_engine* e, int enable, unsigned long long* out, int cap) {
   int r = guard(e); if (r) return r;
-  if (!e->dec_params) return SL_ERR_UNSUPPORTED;
+  if (!e->flow_params) return SL_ERR_UNSUPPORTED;
   if (out && cap > 0) {
     r = copy_sync(e, out, e->dec_tstamp, (size_t)(cap < 2048 + 8192 ? cap : 2048 + 8192) * 8, hipMemcpyDeviceToHost); if (r) return r;
   }
-  e->dec_host.tstamp = enable ? e->dec_tstamp : nullptr;
-  e->flow_host.d.tstamp = e->dec_host.tstamp;
-  r = copy_sync(e, e->flow_params, &e->flow_host, sizeof(FlowP), hipMemcpyHostToDevice); if (r) return r;
-  return copy_sync(e, e->dec_params, &e->dec_host, sizeof(DecodeP), hipMemcpyHostToDevice);
+  e->flow_host.d.tstamp = enable ? e->dec_tstamp : nullptr;
+  return copy_sync(e, e->flow_params, &e->flow_host, sizeof(FlowP), hipMemcpyHostToDevice);
 }
 int sl_profile_head(sl_engine* e, int enable) {
   int r = guard(e); if (r) return r;

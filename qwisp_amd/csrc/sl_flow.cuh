@@ -515,36 +515,60 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
   if (!lin && wg == 0) {
-    // merge the attention tiles of head `wave` in order with the global max (each wave polls on its own)
+    // Merge the attention tiles of head `wave` in order with the global max (each wave polls on its own).
+    // The round trips are batched: lane i fetches {max, sum} of tile t0+i (64 tiles per load), the per-dim
+    // partials of 4 tiles are in flight at a time; the accumulation itself runs in tile order.
     const int h = wave, slot0 = h * uni(P.max_tiles);
     const rsrc_t rml = co_rsrc(uni(F.tml)), rpo = co_rsrc(uni(F.tpo));
     int fail = 0;
     float Mx = NEG;
-    for (int t = 0; t < nt && !fail; ++t) {
+    for (int t0 = 0; t0 < nt && !fail; t0 += 64) {
+      const bool mine = t0 + lane < nt;
       unsigned spins = 0;
       for (;;) {
-        const uint4 m = ldw4(rml, (slot0 + t) * 4);
-        if (m.z == tcore32 && m.w == tcore32) { Mx = fmaxf(Mx, __uint_as_float(m.x)); break; }
+        bool ok = true;
+        float pm = NEG;
+        if (mine) { const uint4 m = ldw4(rml, (slot0 + t0 + lane) * 4); ok = m.z == tcore32 && m.w == tcore32; pm = __uint_as_float(m.x); }
+        if (__all(ok ? 1 : 0)) { Mx = fmaxf(Mx, tree_max<64>(pm)); break; }
         if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
         __builtin_amdgcn_s_sleep(1);
       }
     }
     float Ls = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int t = 0; t < nt && !fail; ++t) {
-      const uint4 m = ldw4(rml, (slot0 + t) * 4);          // tags verified above
-      const float f = exp_c(__uint_as_float(m.x) - Mx);
-      Ls = fmaf(__uint_as_float(m.y), f, Ls);
-      unsigned spins = 0;
-      for (;;) {
-        const uint4 a = ldw4(rpo, ((slot0 + t) * 128 + 2 * lane) * 4), b = ldw4(rpo, ((slot0 + t) * 128 + 2 * lane + 1) * 4);
-        const bool ok = a.z == tcore32 && a.w == tcore32 && b.z == tcore32 && b.w == tcore32;
-        if (__all(ok ? 1 : 0)) {
-          O[0] = fmaf(__uint_as_float(a.x), f, O[0]); O[1] = fmaf(__uint_as_float(a.y), f, O[1]);
-          O[2] = fmaf(__uint_as_float(b.x), f, O[2]); O[3] = fmaf(__uint_as_float(b.y), f, O[3]);
-          break;
+    for (int t0 = 0; t0 < nt && !fail; t0 += 64) {
+      float fl = 0.0f, pl = 0.0f;                         // lane i: scale and sum of tile t0+i (tags verified above)
+      if (t0 + lane < nt) {
+        const uint4 m = ldw4(rml, (slot0 + t0 + lane) * 4);
+        fl = exp_c(__uint_as_float(m.x) - Mx); pl = __uint_as_float(m.y);
+      }
+      const int cnt = min(64, nt - t0);
+      for (int u0 = 0; u0 < cnt && !fail; u0 += 4) {
+        uint4 a[4], b[4];
+        unsigned spins = 0;
+        for (;;) {
+          bool ok = true;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            if (u0 + u < cnt) {
+              const int t = slot0 + t0 + u0 + u;
+              a[u] = ldw4(rpo, (t * 128 + 2 * lane) * 4); b[u] = ldw4(rpo, (t * 128 + 2 * lane + 1) * 4);
+              ok = ok && a[u].z == tcore32 && a[u].w == tcore32 && b[u].z == tcore32 && b[u].w == tcore32;
+            }
+          }
+          if (__all(ok ? 1 : 0)) break;
+          if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+          __builtin_amdgcn_s_sleep(1);
         }
-        if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
-        __builtin_amdgcn_s_sleep(1);
+        if (fail) break;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (u0 + u < cnt) {
+            const float f = row_lane_f(fl, u0 + u), l = row_lane_f(pl, u0 + u);
+            Ls = fmaf(l, f, Ls);
+            O[0] = fmaf(__uint_as_float(a[u].x), f, O[0]); O[1] = fmaf(__uint_as_float(a[u].y), f, O[1]);
+            O[2] = fmaf(__uint_as_float(b[u].x), f, O[2]); O[3] = fmaf(__uint_as_float(b[u].y), f, O[3]);
+          }
+        }
       }
     }
     // the output gate sits in the q projection of this step

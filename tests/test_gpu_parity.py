@@ -215,6 +215,27 @@ def test_persistent_step_equals_kernel_per_stage(env, small_model):
         assert np.array_equal(ia, ib) and same_bits(sca, scb)
 
 
+def test_persistent_step_long_context(env, small_model):
+    """More than 64 key tiles per head (context > 4096): the single-launch step merges the tiles in two
+    batches of lanes.  Same tokens, logits and caches as the kernel-per-stage sequence."""
+    cfg, dev, host = small_model
+    a = env["Engine"](cfg, dev, max_m=64, max_seq_len=4352)
+    b = env["Engine"](cfg, dev, max_m=64, max_seq_len=4352)
+    assert b.set_persistent(False)
+    toks = np.random.default_rng(77).integers(0, cfg.vocab, 4150).astype(np.int32)
+    for eng in (a, b):
+        for i in range(0, len(toks), 64):
+            assert eng.step_argmax(toks[i:i + 64]) is not None, eng.gpu_fault
+    ta = a.chained_step_argmax(11, 20)         # crosses the 65th tile boundary (position 4160)
+    tb = b.chained_step_argmax(11, 20)
+    assert ta is not None and tb is not None, (a.gpu_fault, b.gpu_fault)
+    assert ta.tolist() == tb.tolist()
+    assert same_bits(a.logits_row(0), b.logits_row(0))
+    for li in range(cfg.n_layers):
+        for x, y in zip(a.read_layer_cache(li), b.read_layer_cache(li)):
+            assert same_bits(x, y), (li, first_diff(x, y))
+
+
 def test_forward_rows_and_head(env, small_model):
     cfg, dev, host = small_model
     eng = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)
