@@ -1,16 +1,18 @@
-// Dataflow variant of the persistent batch-1 step: no grid barriers.
+// Single-launch batch-1 decode step for gfx950: 256 workgroups x 1024 threads follow one token through all
+// layers, the final norm, lm_head and the arg-max.  There are no grid barriers.
 //
 // Every value a stage hands to the next one travels with a tag that names the stage instance that
 // produced it (layer, stage, launch): fp16 activations as 32-bit words {half, tag16}, fp32 attention
-// partials and arg-max candidates as 16-byte chunks {v0, v1, tag, tag}.  A consumer simply loads the
-// words it needs (sc1, coherent across XCDs) and retries until all tags are the expected ones, so a
-// dependency costs one store->load hop instead of "store, wait for the ack, two atomic hops, a flag
-// hop, then fetch".  Producers never wait.  Buffers are reused every layer; this is safe because
-// between the last reader of a buffer and its next writer there is always a stage to which every
-// workgroup contributes (in-proj, routed gate/up, down-proj), and a writer only runs after it has
-// consumed that stage's complete output.
+// partials and arg-max candidates as 16-byte chunks {v0, v1, tag, tag}.  A consumer loads the words it
+// needs (sc1, coherent across XCDs) and retries until all tags are the expected ones; producers never wait.
+// Buffers are reused every layer; this is safe because between the last reader of a buffer and its next
+// writer there is always a stage to which every workgroup contributes (in-proj, routed gate/up, down-proj),
+// and a writer only runs after it has consumed that stage's complete output.
 //
-// Arithmetic, reduction order and work split are those of sl_decode.cuh / sl_kernels.cuh.
+// The residual stream is not exchanged: every workgroup computes all of it (thread t keeps elements 2t, 2t+1
+// in registers), only projection outputs travel.
+//
+// Arithmetic and reduction order are those of sl_kernels.cuh (shared helpers in sl_device.cuh).
 #pragma once
 #include <type_traits>
 #include "sl_decode.cuh"
