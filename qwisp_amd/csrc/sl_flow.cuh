@@ -448,12 +448,29 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
     }
     __syncthreads();
     {
+      // scores: wave (head, half) takes the 32 leaves of its half of the 256 dims, lane j is key j.  The 128
+      // query values sit two per lane and reach the multiply as scalar operands (readlane), so LDS only
+      // serves the key rows.
       const int h = wave >> 1, half = wave & 1;
       const uint16_t* kr = &L.kt[(lane < nk ? lane : 0) * KT_STRIDE + 128 * half];
-      const float* qh = &L.sq[h * 256 + 128 * half];
-      const float g0 = score_leaf8(kr, qh), g1 = score_leaf8(kr + 32, qh + 32);
-      const float g2 = score_leaf8(kr + 64, qh + 64), g3 = score_leaf8(kr + 96, qh + 96);
-      L.part[wave * 64 + lane] = (g0 + g1) + (g2 + g3);
+      const float qa = L.sq[h * 256 + 128 * half + lane], qb = L.sq[h * 256 + 128 * half + 64 + lane];
+      float g[4];
+#pragma unroll
+      for (int gi = 0; gi < 4; ++gi) {
+        float n[8];
+#pragma unroll
+        for (int l = 0; l < 8; ++l) {
+          const int d = 32 * gi + 4 * l;                 // first dim of the leaf within the half
+          const float qv = d < 64 ? qa : qb;
+          const uint2 kraw = *reinterpret_cast<const uint2*>(kr + d);
+          float node = fmaf(row_lane_f(qv, (d & 63)), lo_h(kraw.x), 0.0f);
+          node = fmaf(row_lane_f(qv, (d & 63) + 1), hi_h(kraw.x), node);
+          node = fmaf(row_lane_f(qv, (d & 63) + 2), lo_h(kraw.y), node);
+          n[l] = fmaf(row_lane_f(qv, (d & 63) + 3), hi_h(kraw.y), node);
+        }
+        g[gi] = ((n[0] + n[1]) + (n[2] + n[3])) + ((n[4] + n[5]) + (n[6] + n[7]));
+      }
+      L.part[wave * 64 + lane] = (g[0] + g[1]) + (g[2] + g[3]);
     }
     __syncthreads();
     if ((wave & 1) == 0) {
@@ -472,10 +489,10 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       const int h = wave >> 1, half = wave & 1;
       float o0 = 0.0f, o1 = 0.0f;
       const uint16_t* vt = &g_vt[128 * half + 2 * lane];
-      const float* pw = &L.sm[h * 64];
+      const float pmine = L.sm[h * 64 + lane];            // weight of key `lane`; handed out by readlane below
       for (int j = 0; j < nk; ++j) {
         const uint32_t vv = *reinterpret_cast<const uint32_t*>(vt + j * 256);
-        const float pj = pw[j];
+        const float pj = row_lane_f(pmine, j);
         o0 = fmaf(pj, lo_h(vv), o0);
         o1 = fmaf(pj, hi_h(vv), o1);
       }
@@ -601,6 +618,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     const uint32_t ty = lin ? tcore : tmerge;
     const rsrc_t ry = co_rsrc(uni(F.tycore)), rz = co_rsrc(uni(F.tproj));
     uint4 a = make_uint4(0, 0, 0, 0), b = make_uint4(0, 0, 0, 0);
+    bool zdone = false;
     unsigned spins = 0;
     fstamp(P, 6, 0);
     for (;;) {
@@ -611,11 +629,12 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
         ok = tag_ok(a.x, ty) && tag_ok(a.y, ty) && tag_ok(a.z, ty) && tag_ok(a.w, ty) &&
              tag_ok(a2.x, ty) && tag_ok(a2.y, ty) && tag_ok(a2.z, ty) && tag_ok(a2.w, ty);
         ystage[tid] = a2;
-        if (lin) {
+        if (lin && !zdone) {                      // the gate values were published a stage earlier: fetched once
           b = ldw4(rz, 8192 + e0);
           const uint4 b2 = ldw4(rz, 8192 + e0 + 2048);
-          ok = ok && tag_ok(b.x, tin) && tag_ok(b.y, tin) && tag_ok(b.z, tin) && tag_ok(b.w, tin) &&
-               tag_ok(b2.x, tin) && tag_ok(b2.y, tin) && tag_ok(b2.z, tin) && tag_ok(b2.w, tin);
+          zdone = tag_ok(b.x, tin) && tag_ok(b.y, tin) && tag_ok(b.z, tin) && tag_ok(b.w, tin) &&
+                  tag_ok(b2.x, tin) && tag_ok(b2.y, tin) && tag_ok(b2.z, tin) && tag_ok(b2.w, tin);
+          ok = ok && zdone;
           ystage[512 + tid] = b2;
         }
       }
