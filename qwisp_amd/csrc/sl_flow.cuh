@@ -463,10 +463,11 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
           const int d = 32 * gi + 4 * l;                 // first dim of the leaf within the half
           const float qv = d < 64 ? qa : qb;
           const uint2 kraw = *reinterpret_cast<const uint2*>(kr + d);
-          float node = fmaf(row_lane_f(qv, (d & 63)), lo_h(kraw.x), 0.0f);
-          node = fmaf(row_lane_f(qv, (d & 63) + 1), hi_h(kraw.x), node);
-          node = fmaf(row_lane_f(qv, (d & 63) + 2), lo_h(kraw.y), node);
-          n[l] = fmaf(row_lane_f(qv, (d & 63) + 3), hi_h(kraw.y), node);
+          const h2_t k01 = as_h2(kraw.x), k23 = as_h2(kraw.y);      // half operands go straight into the FMA
+          float node = fmaf(row_lane_f(qv, (d & 63)), (float)k01.x, 0.0f);
+          node = fmaf(row_lane_f(qv, (d & 63) + 1), (float)k01.y, node);
+          node = fmaf(row_lane_f(qv, (d & 63) + 2), (float)k23.x, node);
+          n[l] = fmaf(row_lane_f(qv, (d & 63) + 3), (float)k23.y, node);
         }
         g[gi] = ((n[0] + n[1]) + (n[2] + n[3])) + ((n[4] + n[5]) + (n[6] + n[7]));
       }
@@ -493,8 +494,9 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       for (int j = 0; j < nk; ++j) {
         const uint32_t vv = *reinterpret_cast<const uint32_t*>(vt + j * 256);
         const float pj = row_lane_f(pmine, j);
-        o0 = fmaf(pj, lo_h(vv), o0);
-        o1 = fmaf(pj, hi_h(vv), o1);
+        const h2_t v01 = as_h2(vv);
+        o0 = fmaf(pj, (float)v01.x, o0);
+        o1 = fmaf(pj, (float)v01.y, o1);
       }
       const int head = kvh * 8 + h;
       stw4(co_rsrc(uni(F.tpo)), ((head * uni(P.max_tiles) + tile) * 128 + 64 * half + lane) * 4, __float_as_uint(o0), __float_as_uint(o1), tcore, tcore);
@@ -533,7 +535,8 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   wload_row<2>(wr.w[0], wr.sb[0], uni(Y.out_w), uni(Y.out_sb), (size_t)(valid ? gw : 0), valid, lane);
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
-  if (!lin && wg == 0) {
+  if (!lin && wg == G - 1) {        // the last workgroup owns a tile unit only in very long contexts, so its
+                                     // waves have no stores of their own to wait for
     // Merge the attention tiles of head `wave` in order with the global max (each wave polls on its own).
     // The round trips are batched: lane i fetches {max, sum} of tile t0+i (64 tiles per load), the per-dim
     // partials of 4 tiles are in flight at a time; the accumulation itself runs in tile order.
