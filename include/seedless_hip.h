@@ -146,6 +146,18 @@ int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out);
 /* chainedStepArgmax (SFV:4413): equals K successive sl_step_argmax of one token each, the
  * output of step k feeding step k+1 on the device. */
 int sl_chained_step_argmax(sl_engine* e, int32_t first_token, int k, int32_t* out);
+/* stepSampleRows (SFV:3954): sampling is outside this build (greedy only).  Always returns
+ * SL_ERR_UNSUPPORTED without touching `out`; Tell then samples on its own side (TellRuntime.swift:424). */
+int sl_step_sample_rows(sl_engine* e, const int32_t* tokens, int m, float temperature, float top_p,
+                        uint64_t seed, int32_t* out);
+/* A further sequence on the weights of `base` (reference: the lanes of SeedlessLaneBatch share one weight
+ * set, SeedlessLaneBatch.swift:876): own caches, scratch and stream; `base` keeps the weights and must be
+ * destroyed after its lanes.  The lane is a full engine: every entry point works on it. */
+int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine** out);
+/* SeedlessLaneBatch.stepArgmaxBatch (SeedlessLaneBatch.swift:876): one token in and one out per lane, per
+ * lane identical to a solo sl_step_argmax of that lane.  The lanes' steps run back to back (each is one
+ * launch of the single-launch step); weights are not shared between the lanes within a step. */
+int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t* out);
 /* forwardRows (SFV:3641): hidden rows in, hidden rows (final_norm=0) or final-normed rows out. */
 int sl_forward_rows(sl_engine* e, const uint16_t* x_f16, int m, int final_norm, uint16_t* out_f16);
 /* Tell.SpecBackend.forward (TellRuntime.swift:84): embed + forwardRows with final norm. */

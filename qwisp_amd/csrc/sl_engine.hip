@@ -310,6 +310,29 @@ bool shape_ok(const sl_q4& q, int n, int k) { return q.w && q.scales && q.biases
 
 extern "C" {
 
+namespace {
+// Per-sequence storage of one layer: conv history and recurrent state (ping-pong), or the KV arena; routing read-back.
+int alloc_layer_state(sl_engine* e, LayerDev& L) {
+  if (L.is_linear) {
+    for (int p = 0; p < 2; ++p) {
+      L.hist[p] = dalloc<uint16_t>(e, HIST_ELEMS, true);
+      L.state[p] = dalloc<float>(e, STATE_ELEMS, true);
+    }
+    if (!L.hist[1] || !L.state[1]) return SL_ERR_DEVICE;
+  } else {
+    e->has_attn = true;
+    L.kcache = dalloc<uint16_t>(e, (size_t)SL_ATT_KV * e->max_seq * SL_ATT_D, true);
+    L.vcache = dalloc<uint16_t>(e, (size_t)SL_ATT_KV * e->max_seq * SL_ATT_D, true);
+    if (!L.kcache || !L.vcache) return SL_ERR_DEVICE;
+  }
+  L.route_inds = dalloc<int32_t>(e, (size_t)e->max_m * 8, true);
+  L.route_scores = dalloc<uint16_t>(e, (size_t)e->max_m * 8, true);
+  if (!L.route_inds || !L.route_scores) return SL_ERR_DEVICE;
+  return SL_OK;
+}
+int alloc_runtime(sl_engine* e);
+}  // namespace
+
 int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** out) {
   if (!d || !out || max_m < 1 || max_seq_len < 1 || d->n_layers < 1 || !d->layers) return SL_ERR_ARG;
   if (d->n_experts < 8 || d->n_experts > SL_MAX_EXPERTS || (d->n_experts % 8) != 0) return SL_ERR_ARG;
@@ -350,13 +373,8 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
       L.a_log = upload<float>(e, g.a_log, SL_GDN_HV, loc);
       L.dt_bias = upload<float>(e, g.dt_bias, SL_GDN_HV, loc);
       L.gdn_norm_w = upload<uint16_t>(e, g.norm_w, SL_GDN_D, loc);
-      for (int p = 0; p < 2; ++p) {
-        L.hist[p] = dalloc<uint16_t>(e, HIST_ELEMS, true);
-        L.state[p] = dalloc<float>(e, STATE_ELEMS, true);
-      }
-      if (!L.conv_w || !L.a_log || !L.dt_bias || !L.gdn_norm_w || !L.hist[1] || !L.state[1]) return SL_ERR_DEVICE;
+      if (!L.conv_w || !L.a_log || !L.dt_bias || !L.gdn_norm_w) return SL_ERR_DEVICE;
     } else {
-      e->has_attn = true;
       const sl_attn_w& a = s.attn;
       if (!alloc_q4(e, L.qkv, SL_ATT_QKV_N, H)) return SL_ERR_DEVICE;
       if (!fill_q4(e, L.qkv, 0, a.q_proj, 8192, H, loc) || !fill_q4(e, L.qkv, 8192, a.k_proj, 512, H, loc) ||
@@ -364,9 +382,7 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
         return SL_ERR_ARG;
       L.q_norm = upload<uint16_t>(e, a.q_norm, SL_ATT_D, loc);
       L.k_norm = upload<uint16_t>(e, a.k_norm, SL_ATT_D, loc);
-      L.kcache = dalloc<uint16_t>(e, (size_t)SL_ATT_KV * max_seq_len * SL_ATT_D, true);
-      L.vcache = dalloc<uint16_t>(e, (size_t)SL_ATT_KV * max_seq_len * SL_ATT_D, true);
-      if (!L.q_norm || !L.k_norm || !L.kcache || !L.vcache) return SL_ERR_DEVICE;
+      if (!L.q_norm || !L.k_norm) return SL_ERR_DEVICE;
     }
     const sl_moe_w& w = s.moe;
     L.router_w = upload<uint16_t>(e, w.router_w, (size_t)E * H, loc);
@@ -376,19 +392,31 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
         !upload_q4(e, L.sw_down, w.sw_down, E * H, SL_MOE_I, loc) || !upload_q4(e, L.sh_gate, w.sh_gate, SL_MOE_I, H, loc) ||
         !upload_q4(e, L.sh_up, w.sh_up, SL_MOE_I, H, loc) || !upload_q4(e, L.sh_down, w.sh_down, H, SL_MOE_I, loc))
       return SL_ERR_ARG;
-    L.route_inds = dalloc<int32_t>(e, (size_t)max_m * 8, true);
-    L.route_scores = dalloc<uint16_t>(e, (size_t)max_m * 8, true);
-    if (!L.route_inds || !L.route_scores) return SL_ERR_DEVICE;
+    { const int r = alloc_layer_state(e, L); if (r) return r; }
   }
   if (has_head) {
     if (!upload_q4(e, e->embed, d->embed, d->vocab, H, loc) || !upload_q4(e, e->lm_head, d->lm_head, d->vocab, H, loc))
       return SL_ERR_ARG;
     e->final_norm = upload<uint16_t>(e, d->final_norm, H, loc);
+    if (!e->final_norm) return SL_ERR_DEVICE;
+  }
+  return alloc_runtime(e);
+}
+
+namespace {
+// Everything an engine needs besides weights and per-layer caches: scratch rows, head buffers, rope table,
+// step state, the single-launch step's parameter blocks, pinned staging.
+int alloc_runtime(sl_engine* e) {
+  const int max_m = e->max_m, max_seq_len = e->max_seq, E = e->n_experts;
+  const bool has_head = e->has_head;
+  struct { int n_layers, vocab; } dd = {e->n_layers, e->vocab};
+  const auto* d = &dd;
+  if (has_head) {
     e->n_cand = d->vocab / 16;
     e->logits = dalloc<uint16_t>(e, (size_t)max_m * d->vocab);
     e->cand_v = dalloc<float>(e, (size_t)max_m * e->n_cand + 1024);
     e->cand_i = dalloc<int32_t>(e, (size_t)max_m * e->n_cand + 1024);
-    if (!e->final_norm || !e->logits || !e->cand_v || !e->cand_i) return SL_ERR_DEVICE;
+    if (!e->logits || !e->cand_v || !e->cand_i) return SL_ERR_DEVICE;
   }
   if (e->has_attn) {
     std::vector<float> c, s;
@@ -476,6 +504,51 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
   SL_TRY(e, hipHostMalloc(&e->pinned, e->pinned_bytes, hipHostMallocDefault));
   SL_TRY(e, hipStreamSynchronize(e->stream));
   return SL_OK;
+}
+}  // namespace
+
+// A further sequence ("lane") on the weights of `base`: own caches, scratch and stream; the weight pointers are
+// shared and stay owned by `base`, which must outlive its lanes.
+int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine** out) {
+  if (!base || !out || max_m < 1 || max_seq_len < 1) return SL_ERR_ARG;
+  if (!base->fault.empty()) return SL_ERR_POISONED;
+  sl_engine* e = new sl_engine();
+  *out = e;
+  e->n_layers = base->n_layers; e->n_experts = base->n_experts; e->vocab = base->vocab;
+  e->max_m = max_m; e->max_seq = max_seq_len; e->max_tiles = (max_seq_len + SDPA_TILE - 1) / SDPA_TILE;
+  e->has_head = base->has_head;
+  e->parity.assign(e->n_layers, 0);
+  SL_TRY(e, hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
+  SL_TRY(e, hipEventCreate(&e->ev0));
+  SL_TRY(e, hipEventCreate(&e->ev1));
+  e->layers = base->layers;                       // weight pointers; the per-sequence ones are replaced below
+  for (LayerDev& L : e->layers) {
+    L.hist[0] = L.hist[1] = nullptr; L.state[0] = L.state[1] = nullptr;
+    L.kcache = L.vcache = nullptr; L.route_inds = nullptr; L.route_scores = nullptr;
+    const int r = alloc_layer_state(e, L); if (r) return r;
+  }
+  e->embed = base->embed; e->lm_head = base->lm_head; e->final_norm = base->final_norm;
+  return alloc_runtime(e);
+}
+
+// One token per lane (reference: SeedlessLaneBatch.stepArgmaxBatch).  Each lane's step is the single-launch
+// step of that lane; the launches are queued back to back and the tokens read afterwards, so per lane the
+// result is that of a solo step by construction.
+int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t* out) {
+  if (!lanes || b < 1 || !tokens || !out) return SL_ERR_ARG;
+  for (int i = 0; i < b; ++i) {
+    if (!lanes[i]) return SL_ERR_ARG;
+    for (int j = 0; j < i; ++j) if (lanes[j] == lanes[i]) return SL_ERR_ARG;
+  }
+  for (int i = 0; i < b; ++i) { const int r = sl_step_argmax(lanes[i], tokens + i, 1, out + i); if (r) return r; }
+  return SL_OK;
+}
+
+// Sampling is outside this build (greedy only); Tell falls back to its own sampler on "unsupported".
+int sl_step_sample_rows(sl_engine* e, const int32_t* tokens, int m, float temperature, float top_p, uint64_t seed, int32_t* out) {
+  (void)tokens; (void)m; (void)temperature; (void)top_p; (void)seed; (void)out;
+  int r = guard(e); if (r) return r;
+  return SL_ERR_UNSUPPORTED;
 }
 
 void sl_destroy(sl_engine* e) {

@@ -39,6 +39,36 @@ class SeedlessFusedForward:
                 self.h = None
             raise _lib.SeedlessError("sl_create", status, fault.decode() if fault else None)
 
+    # -- lanes (SeedlessLaneBatch.swift:876): sequences that share this engine's weights ---------------
+    def new_lane(self, max_m=1, max_seq_len=1024):
+        """A further sequence on this engine's weights.  Close the lanes before this engine."""
+        h = C.c_void_p()
+        status = self.lib.dll.sl_lane_create(self.h, max_m, max_seq_len, C.byref(h))
+        lane = object.__new__(type(self))
+        lane.lib, lane.cfg, lane.h = self.lib, self.cfg, h
+        if status != abi.SL_OK:
+            fault = lane.gpu_fault if h else None
+            lane.close()
+            raise _lib.SeedlessError("sl_lane_create", status, fault)
+        return lane
+
+    @staticmethod
+    def lane_step_argmax(lanes, tokens):
+        """One token in, one out per lane; per lane identical to a solo step."""
+        tok = np.ascontiguousarray(tokens, np.int32)
+        assert len(tok) == len(lanes) > 0
+        out = np.empty(len(tok), np.int32)
+        arr = (C.c_void_p * len(lanes))(*[l.h for l in lanes])
+        if lanes[0].lib.dll.sl_lane_step_argmax(arr, len(lanes), _p(tok), _p(out)) != abi.SL_OK:
+            return None
+        return out
+
+    def step_sample_rows(self, tokens, temperature=1.0, top_p=1.0, seed=0):
+        """Not built (greedy only): returns the status code, SL_ERR_UNSUPPORTED on a healthy engine."""
+        tok = np.ascontiguousarray(tokens, np.int32)
+        out = np.full(len(tok), -1, np.int32)
+        return self.lib.dll.sl_step_sample_rows(self.h, _p(tok), len(tok), float(temperature), float(top_p), int(seed), _p(out)), out
+
     # -- lifetime ---------------------------------------------------------------------------------
     def close(self):
         if getattr(self, "h", None):

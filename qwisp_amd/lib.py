@@ -19,6 +19,9 @@ SIGNATURES = {
     "sl_fault": (C.c_char_p, [_vp]),
     "sl_inject_failure": (None, [_vp]),
     "sl_step_argmax": (_i32, [_vp, _vp, _i32, _vp]),
+    "sl_step_sample_rows": (_i32, [_vp, _vp, _i32, _f32, _f32, _u64, _vp]),
+    "sl_lane_create": (_i32, [_vp, _i32, _i32, _vp]),
+    "sl_lane_step_argmax": (_i32, [_vp, _i32, _vp, _vp]),
     "sl_chained_step_argmax": (_i32, [_vp, _i32, _i32, _vp]),
     "sl_forward_rows": (_i32, [_vp, _vp, _i32, _i32, _vp]),
     "sl_forward_tokens": (_i32, [_vp, _vp, _i32, _vp]),

@@ -236,6 +236,38 @@ def test_persistent_step_long_context(env, small_model):
             assert same_bits(x, y), (li, first_diff(x, y))
 
 
+def test_lanes_share_weights_and_equal_solo(env, small_model):
+    """Lanes (SeedlessLaneBatch.swift:876): sequences on one weight set.  Per lane the token stream is that
+    of a solo engine, whatever the other lanes do; sampling is reported as unsupported."""
+    cfg, dev, host = small_model
+    base = env["Engine"](cfg, dev, max_m=4, max_seq_len=96)
+    lanes = [base.new_lane(max_m=4, max_seq_len=96) for _ in range(3)]
+    solos = [env["Engine"](cfg, dev, max_m=4, max_seq_len=96) for _ in range(3)]
+    prompts = [[5, 6, 7], [900, 11], [42]]
+    cur = []
+    for lane, solo, pr in zip(lanes, solos, prompts):
+        a, b = lane.step_argmax(pr), solo.step_argmax(pr)
+        assert a is not None and b is not None, (lane.gpu_fault, solo.gpu_fault)
+        assert a.tolist() == b.tolist()
+        cur.append(int(a[-1]))
+    for step in range(12):
+        got = type(base).lane_step_argmax(lanes, cur)
+        assert got is not None, [l.gpu_fault for l in lanes]
+        want = [int(solo.step_argmax([t])[0]) for solo, t in zip(solos, cur)]
+        assert got.tolist() == want, step
+        cur = want
+    assert [l.position for l in lanes] == [s.position for s in solos]
+    for lane, solo in zip(lanes, solos):
+        assert same_bits(lane.logits_row(0), solo.logits_row(0))
+    # the base engine is untouched by its lanes and still works
+    assert base.position == 0 and base.step_argmax([1, 2]) is not None
+    status, out = base.step_sample_rows([3], temperature=0.7, top_p=0.9, seed=1)
+    assert status == abi.SL_ERR_UNSUPPORTED and out.tolist() == [-1]
+    assert type(base).lane_step_argmax([lanes[0], lanes[0]], [1, 2]) is None      # the same lane twice
+    for lane in lanes:
+        lane.close()
+
+
 def test_forward_rows_and_head(env, small_model):
     cfg, dev, host = small_model
     eng = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)
