@@ -200,6 +200,8 @@ SL_DEV void flow_prologue(float& h0, float& h1, bool has_r, float r0, float r1, 
 // finish a poll before the write has travelled to memory and back.  All tagged results of a stage are therefore
 // gathered in LDS and written by wave 15 (full 64-byte lines), and wave 15 never takes part in a poll.
 constexpr int PUB_WAVE = DEC_WAVES - 1;
+constexpr int DENSE_WAVE0 = 128 * DEC_WAVES;     // first wave of the router rows (workgroup 128)
+constexpr int PAIR_WAVE0 = 160 * DEC_WAVES;      // first wave of the shared gate/up pairs (workgroups 160..191)
 
 #define FLOW_IDS const int tid = fresh_v(threadIdx.x), lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); \
                  const int wg = fresh_s(blockIdx.x), G = fresh_s(gridDim.x), NW = G * DEC_WAVES, gw = wg * DEC_WAVES + wave; \
@@ -261,6 +263,7 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
     const int row = wg * DEC_WAVES + (lane & 15) + (lane >> 4) * NW;      // four runs of 16 consecutive rows
     if (row < N) stw1(co_rsrc(uni(F.tproj)), row, g_L.pub[lane]);
   }
+ 
  
  
   return true;
@@ -364,6 +367,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
   gh.tnew = f2h(newest);
   __syncthreads();
   if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tycore)), hv * 128 + dvb * 16 + lane, L.pub[lane]);
+ 
  
  
   return true;
@@ -503,6 +507,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
     }
     __syncthreads();
   }
+ 
  
  
   return true;
@@ -686,6 +691,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   }
  
  
+ 
   return true;
 }
 
@@ -693,15 +699,19 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
 SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, float& h0, float& h1) {
   FLOW_IDS;
   const DecodeP& P = F.d;
-  const bool is_dense = gw <= uni(P.E);
-  const bool is_pair = gw >= 512 && gw < 1024;
+  // The router rows, the shared-gate row and the shared gate/up pairs sit on workgroups of the upper half
+  // of the grid: those have no row of the K = 4096 projection, reach this stage early and so have their
+  // rows in registers long before the hand-over arrives (the router logits are what stage B waits for).
+  const int gd = gw - DENSE_WAVE0, gp = gw - PAIR_WAVE0;
+  const bool is_dense = gd >= 0 && gd <= uni(P.E);
+  const bool is_pair = gp >= 0 && gp < 512;
   uint4 dwr[4] = {};                      // dense fp16 row, kept packed until the wait is over
   WRegs<1, 2> wr;
-  const size_t prow = is_pair ? (size_t)(gw - 512) : 0;
+  const size_t prow = is_pair ? (size_t)gp : 0;
   wload_row<1>(wr.w[0], wr.sb[0], uni(Y.shg_w), uni(Y.shg_sb), prow, is_pair, lane);
   wload_row<1>(wr.w[1], wr.sb[1], uni(Y.shu_w), uni(Y.shu_sb), prow, is_pair, lane);
   if (is_dense) {
-    const uint16_t* drow = (gw < uni(P.E) ? uni(Y.router_w) + (size_t)gw * H : uni(Y.sgate_w)) + 32 * lane;
+    const uint16_t* drow = (gd < uni(P.E) ? uni(Y.router_w) + (size_t)gd * H : uni(Y.sgate_w)) + 32 * lane;
 #pragma unroll
     for (int j = 0; j < 4; ++j) dwr[j] = ld16(drow + 8 * j);
   }
@@ -726,19 +736,20 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
     if (lane == 0) g_L.pub[wave] = tagged(swiglu16(f16r(gu.v[0]), f16r(gu.v[1])), ta);
   }
   {
-    const int g0 = wg * DEC_WAVES, E = uni(P.E);
-    if (g0 <= E || (g0 >= 512 && g0 < 1024)) {     // uniform per workgroup: it holds router rows, the gate row or pairs
+    const int d0 = wg * DEC_WAVES - DENSE_WAVE0, p0 = wg * DEC_WAVES - PAIR_WAVE0, E = uni(P.E);
+    if ((d0 >= 0 && d0 <= E) || (p0 >= 0 && p0 < 512)) {     // uniform per workgroup: it holds router rows, the gate row or pairs
       __syncthreads();
       if (wave == PUB_WAVE && lane < 16) {
-        const int g = g0 + lane;
-        if (g < E) stw1(co_rsrc(uni(F.trlog)), g, g_L.pub[lane]);
-        else if (g == E) stw1(co_rsrc(uni(F.tsg)), 0, g_L.pub[lane]);
-        else if (g >= 512 && g < 1024) stw1(co_rsrc(uni(F.tsh)), g - 512, g_L.pub[lane]);
+        if (d0 >= 0 && d0 <= E) {
+          const int g = d0 + lane;
+          if (g < E) stw1(co_rsrc(uni(F.trlog)), g, g_L.pub[lane]);
+          else if (g == E) stw1(co_rsrc(uni(F.tsg)), 0, g_L.pub[lane]);
+        } else {
+          stw1(co_rsrc(uni(F.tsh)), p0 + lane, g_L.pub[lane]);
+        }
       }
     }
   }
- 
- 
   return true;
 }
 
@@ -842,6 +853,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
   if (wave == PUB_WAVE && lane < 16 && wg * DEC_WAVES + lane < 8 * 512) stw1(co_rsrc(uni(F.tact)), wg * DEC_WAVES + lane, L.pub[lane]);
  
  
+ 
   return true;
 }
 
@@ -930,6 +942,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, c
     stw1(co_rsrc(uni(F.tmoe)), quad * 4 + sb4, tagged(f16r(acc + f16r(s * L.dbuf[(ql * 9 + 8) * 4 + sb4])), flow_tag(base, li, FS_C)));
   }
   __syncthreads();
+ 
  
  
   return true;
