@@ -620,9 +620,9 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   // every thread prepares 4 consecutive elements of the 4096-long activation; waves 0..7 fetch them, for
   // themselves and for the wave 8 above (handed over through LDS)
   const int e0 = 256 * wave + 4 * lane;
-  float out[4], z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  float out[4], sz[4] = {0.0f, 0.0f, 0.0f, 0.0f};            // sz: z * sigmoid(z) of the gate values
   {
-    uint4* ystage = reinterpret_cast<uint4*>(g_vt);            // [512] y chunks, [512] z chunks of waves 8..15
+    uint4* ystage = reinterpret_cast<uint4*>(g_vt);            // [512] y chunks, [512] silu(z) quads of waves 8..15
     const uint32_t ty = lin ? tcore : tmerge;
     const rsrc_t ry = co_rsrc(uni(F.tycore)), rz = co_rsrc(uni(F.tproj));
     uint4 a = make_uint4(0, 0, 0, 0), b = make_uint4(0, 0, 0, 0);
@@ -643,7 +643,15 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
           zdone = tag_ok(b.x, tin) && tag_ok(b.y, tin) && tag_ok(b.z, tin) && tag_ok(b.w, tin) &&
                   tag_ok(b2.x, tin) && tag_ok(b2.y, tin) && tag_ok(b2.z, tin) && tag_ok(b2.w, tin);
           ok = ok && zdone;
-          ystage[512 + tid] = b2;
+          if (zdone) {
+            // z * sigmoid(z) does not need the core output: formed while that is still on its way
+            const float z1[4] = {lo_h(b.x), lo_h(b.y), lo_h(b.z), lo_h(b.w)};
+            const float z2[4] = {lo_h(b2.x), lo_h(b2.y), lo_h(b2.z), lo_h(b2.w)};
+            float s2[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { sz[i] = z1[i] * sigmoid32(z1[i]); s2[i] = z2[i] * sigmoid32(z2[i]); }
+            ystage[512 + tid] = make_uint4(__float_as_uint(s2[0]), __float_as_uint(s2[1]), __float_as_uint(s2[2]), __float_as_uint(s2[3]));
+          }
         }
       }
       const int v = flow_round(ok, spins, uni(P.bar) + 32);
@@ -651,10 +659,12 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
       if (v < 0) return false;
     }
     fstamp(P, 7, spins);
-    if (wave >= 8) { a = ystage[tid - 512]; if (lin) b = ystage[tid]; }
+    if (wave >= 8) {
+      a = ystage[tid - 512];
+      if (lin) { b = ystage[tid]; sz[0] = __uint_as_float(b.x); sz[1] = __uint_as_float(b.y); sz[2] = __uint_as_float(b.z); sz[3] = __uint_as_float(b.w); }
+    }
     if (lin) store_hist(Y, li, gh);
     out[0] = lo_h(a.x); out[1] = lo_h(a.y); out[2] = lo_h(a.z); out[3] = lo_h(a.w);
-    z[0] = lo_h(b.x); z[1] = lo_h(b.y); z[2] = lo_h(b.z); z[3] = lo_h(b.w);
   }
   if (lin) {
     float nw[4];
@@ -667,7 +677,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const float nrm = f16r(nw[i] * f16r(out[i] * inv));
-      out[i] = f16r((z[i] * sigmoid32(z[i])) * nrm);
+      out[i] = f16r(sz[i] * nrm);
     }
   }
   {
