@@ -226,8 +226,10 @@ void* sl_stream(sl_engine* e);
  * 0 switches to the kernel-per-stage sequence used for M > 1.  Both give identical results. */
 int sl_set_persistent(sl_engine* e, int enable);
 
-/* Diagnostic: while enabled, workgroup 0 of the persistent kernel records a 100 MHz clock stamp after
- * every grid barrier; the call copies out[0] = number of stamps and out[1..] = stamps of the last step. */
+/* Diagnostic: while enabled, workgroups 0 and 100 of the single-launch step record a 100 MHz clock stamp
+ * before and after every poll; the call copies out[0] = number of stamps of workgroup 0 and out[1..] its
+ * stamps of the last step (clock << 16 | stage id << 8 | poll retries), the same for workgroup 100 from
+ * out[2048]. */
 int sl_debug_stage_clock(sl_engine* e, int enable, unsigned long long* out, int cap);
 
 /* Per-kernel timing in the manner of forwardRowsProfiled (SFV:4352): while enabled, every launch of

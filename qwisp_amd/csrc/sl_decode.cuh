@@ -38,12 +38,11 @@ struct LayerP {
 struct DecodeP {
   int n_layers, E, vocab, max_seq, max_tiles;
   const LayerP* layers;
-  const uint32_t *emb_w, *emb_sb, *lm_w, *lm_sb;
+  const uint32_t *lm_w, *lm_sb;
   const uint16_t* final_norm;
   const float *rope_cos, *rope_sin;
-  uint16_t *hA, *hB, *proj, *ycore, *mix, *rlogits, *sgate, *sh_act, *act, *moe_out, *normed, *logits;
-  float *pm, *pl, *po, *cand_v;
-  int32_t *cand_i, *tok_in, *tok_out, *st;
+  uint16_t *hA, *normed, *logits;     // embedded row in; final-normed row and logits out
+  int32_t *tok_in, *tok_out, *st;     // st: {position, parity of every layer's ping-pong caches}
   unsigned long long* tstamp;   // optional diagnostic clock stamps
   unsigned* bar;   // [16] stage-instance counter (advanced every launch), [32] abort flag
 };

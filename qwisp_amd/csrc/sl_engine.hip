@@ -473,11 +473,9 @@ int alloc_runtime(sl_engine* e) {
       DecodeP P;
       std::memset(&P, 0, sizeof(P));
       P.n_layers = d->n_layers; P.E = E; P.vocab = d->vocab; P.max_seq = max_seq_len; P.max_tiles = e->max_tiles;
-      P.layers = dl; P.emb_w = e->embed.w; P.emb_sb = e->embed.sb; P.lm_w = e->lm_head.w; P.lm_sb = e->lm_head.sb;
+      P.layers = dl; P.lm_w = e->lm_head.w; P.lm_sb = e->lm_head.sb;
       P.final_norm = e->final_norm; P.rope_cos = e->rope_cos; P.rope_sin = e->rope_sin;
-      P.hA = e->hA; P.hB = e->hB; P.proj = e->proj; P.ycore = e->ycore; P.mix = e->mix; P.rlogits = e->rlogits;
-      P.sgate = e->sgate; P.sh_act = e->sh_act; P.act = e->act; P.moe_out = e->moe_out; P.normed = e->normed;
-      P.logits = e->logits; P.pm = e->pm; P.pl = e->pl; P.po = e->po; P.cand_v = e->cand_v; P.cand_i = e->cand_i;
+      P.hA = e->hA; P.normed = e->normed; P.logits = e->logits;
       P.tok_in = e->tok_in; P.tok_out = e->tok_out; P.st = e->st; P.bar = e->dec_bar;
       e->dec_tstamp = dalloc<unsigned long long>(e, 2048 + 16 * 256 * 2, true);
       {
@@ -573,8 +571,9 @@ int sl_set_persistent(sl_engine* e, int enable) {
   e->use_persistent = enable != 0;
   return SL_OK;
 }
-// Test/diagnostic hook: per-barrier clock stamps (100 MHz ticks) of workgroup 0 for the steps run while
-// enabled; out[0] = count, out[1..] = stamps.
+// Test/diagnostic hook: clock stamps (100 MHz ticks) that workgroups 0 and 100 take before and after every poll
+// of the single-launch step while enabled; out[0] = count, out[1..] = (clock << 16 | stage id << 8 | retries),
+// the same for workgroup 100 from out[2048].
 int sl_debug_stage_clock(sl_engine* e, int enable, unsigned long long* out, int cap) {
   int r = guard(e); if (r) return r;
   if (!e->flow_params) return SL_ERR_UNSUPPORTED;

@@ -76,34 +76,6 @@ SL_DEV T uni(const T& r) {
 SL_DEV int fresh_v(int x) { asm volatile("" : "+v"(x)); return x; }
 SL_DEV int fresh_s(int x) { asm volatile("" : "+s"(x)); return x; }
 
-// A touch pulls a line into this XCD's L2 (and its translation into the TLB) one stage ahead.  It is an
-// ordinary load of one dword whose value goes to touch_done() later, at a point where the wave has already
-// waited for younger loads; nothing is done with the value.  (A volatile load would be waited for at once.)
-SL_DEV uint32_t ftouch(const void* p, bool on) {
-  uint32_t v = 0;
-  if (on) v = *reinterpret_cast<const uint32_t*>(p);
-  return v;
-}
-SL_DEV void touch_done(uint32_t v) { asm volatile("" ::"v"(v)); }
-SL_DEV void touch_done(uint2 v) { touch_done(v.x); touch_done(v.y); }
-// Rows of K = 2048*NBLK of a 4-bit matrix: 8*NBLK lines of weights per row (x) and the row's scale line (y).
-template <int NBLK>
-SL_DEV uint2 ftouch_rows(const uint32_t* W, const uint32_t* SB, const size_t* rows, const bool* valid, int nrows, int lane) {
-  constexpr int LPR = 8 * NBLK;
-  const int r = lane / LPR, l = lane % LPR;
-  bool onw = false, ons = false;
-  size_t rw = 0, rs = 0;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    if (j < nrows && r == j && valid[j]) { onw = true; rw = rows[j]; }
-    if (j < nrows && lane == j && valid[j]) { ons = true; rs = rows[j]; }
-  }
-  uint2 t;
-  t.x = ftouch(reinterpret_cast<const char*>(W + rw * (NBLK * 256)) + 128 * l, onw);
-  t.y = ftouch(SB + rs * (NBLK * 32), ons);
-  return t;
-}
-
 enum { FS_IN = 0, FS_CORE = 1, FS_MERGE = 2, FS_OUT = 3, FS_A = 4, FS_B = 5, FS_C = 6 };
 constexpr unsigned FLOW_SPIN_LIMIT = 1u << 19;
 
@@ -771,7 +743,7 @@ SL_DEV uint32_t route_key(uint32_t hbits, int e) {
   u = (u & 0x8000u) ? (~u & 0xffffu) : (u | 0x8000u);
   return (u << 8) | (uint32_t)(255 - e);
 }
-SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, uint32_t* carry /*4*/) {
+SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   Lds& L = g_L;
@@ -836,7 +808,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
     for (int kk = 0; kk < 8; ++kk) L.scores[kk] = f16r(sc[kk] / ss);
     if (wg == 0) for (int kk = 0; kk < 8; ++kk) { uni(Y.route_inds)[kk] = L.inds[kk]; uni(Y.route_scores)[kk] = f2h(L.scores[kk]); }
   }
-  // this wave's gate/up pair (issued as soon as the indices are known), then first touches of its down rows
+  // this wave's gate/up pair, requested as soon as the indices are known
   const int p = gw;
   WRegs<1, 2> wr;
   int k = 0, i = 0;
@@ -846,14 +818,6 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
     const size_t row = (size_t)L.inds[k] * 512 + i;
     wload_row<1>(wr.w[0], wr.sb[0], uni(Y.swg_w), uni(Y.swg_sb), row, true, lane);
     wload_row<1>(wr.w[1], wr.sb[1], uni(Y.swu_w), uni(Y.swu_sb), row, true, lane);
-  }
-#pragma unroll
-  for (int qq = 0; qq < 2; ++qq) {
-    const int un = wave + 16 * qq, ql = un / 9, slot = un % 9;
-    const bool on = ql < 2 && slot < 8;
-    const size_t row = on ? (size_t)L.inds[slot] * 2048 + (size_t)(wg * 2 + ql) * 4 : 0;
-    carry[2 * qq] = ftouch(reinterpret_cast<const char*>(uni(Y.swd_w) + row * 64) + 128 * lane, on && lane < 8);
-    carry[2 * qq + 1] = ftouch(uni(Y.swd_sb) + row * 8, on && lane == 8);
   }
   if (active) {
     const F2 gu = dot_1x2(wr);
@@ -871,8 +835,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base, u
 // Units (quad of 4 outputs, slot): slots 0..7 routed experts, slot 8 shared; 2 quads per workgroup.  The nine
 // activation rows are fetched once per workgroup into LDS (packed pairs, 20-word stride per 32 elements).
 constexpr int XC_STRIDE = 20;
-SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base, const uint32_t* next_w, const uint32_t* next_sb,
-                       int next_n, int next_contig, const uint32_t* carry /*4*/) {
+SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   Lds& L = g_L;
@@ -1082,14 +1045,8 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
       if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh)) return;
     }
     if (!flow_moe_a(F, Y, li, base, h0, h1)) return;
-    uint32_t carry[4];
-    if (!flow_moe_b(F, Y, li, base, carry)) return;
-    {
-      const bool last = li + 1 == nl;
-      const LayerP& Z = g_K.layers[last ? li : li + 1];
-      if (!flow_moe_c(F, Y, li, base, last ? uni(P.lm_w) : uni(Z.in_w), last ? uni(P.lm_sb) : uni(Z.in_sb),
-                      last ? uni(P.vocab) : (uni(Z.is_linear) ? SL_GDN_IN_N : SL_ATT_QKV_N), last ? 1 : 0, carry)) return;
-    }
+    if (!flow_moe_b(F, Y, li, base)) return;
+    if (!flow_moe_c(F, Y, li, base)) return;
   }
   flow_head(F, pos, out_off, feed, base, h0, h1);
   fstamp(P, 18, 0);
