@@ -185,10 +185,10 @@ SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, fl
   uint32_t* rs = reinterpret_cast<uint32_t*>(g_L.part);       // [1024] packed pairs
   const rsrc_t rr = co_rsrc(vec);
   unsigned spins = 0;
+  bool ok = tid >= 512;                         // a thread whose words have arrived does not fetch them again
   fstamp(P, id, 0);
   for (;;) {
-    bool ok = true;
-    if (tid < 512) {
+    if (tid < 512 && !ok) {
       const uint4 b = ldw4(rr, 4 * tid);
       ok = tag_ok(b.x, tag) && tag_ok(b.y, tag) && tag_ok(b.z, tag) && tag_ok(b.w, tag);
       *reinterpret_cast<uint2*>(&rs[2 * tid]) = make_uint2((b.x & 0xffffu) | (b.y << 16), (b.z & 0xffffu) | (b.w << 16));
@@ -598,17 +598,19 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     const uint32_t ty = lin ? tcore : tmerge;
     const rsrc_t ry = co_rsrc(uni(F.tycore)), rz = co_rsrc(uni(F.tproj));
     uint4 a = make_uint4(0, 0, 0, 0), b = make_uint4(0, 0, 0, 0);
-    bool zdone = false;
+    bool zdone = false, y1done = false, y2done = false;   // what has arrived is not fetched again
     unsigned spins = 0;
     fstamp(P, 6, 0);
     for (;;) {
       bool ok = true;
       if (wave < 8) {
-        a = ldw4(ry, e0);
-        const uint4 a2 = ldw4(ry, e0 + 2048);
-        ok = tag_ok(a.x, ty) && tag_ok(a.y, ty) && tag_ok(a.z, ty) && tag_ok(a.w, ty) &&
-             tag_ok(a2.x, ty) && tag_ok(a2.y, ty) && tag_ok(a2.z, ty) && tag_ok(a2.w, ty);
-        ystage[tid] = a2;
+        if (!y1done) { a = ldw4(ry, e0); y1done = tag_ok(a.x, ty) && tag_ok(a.y, ty) && tag_ok(a.z, ty) && tag_ok(a.w, ty); }
+        if (!y2done) {
+          const uint4 a2 = ldw4(ry, e0 + 2048);
+          y2done = tag_ok(a2.x, ty) && tag_ok(a2.y, ty) && tag_ok(a2.z, ty) && tag_ok(a2.w, ty);
+          ystage[tid] = a2;
+        }
+        ok = y1done && y2done;
         if (lin && !zdone) {                      // the gate values were published a stage earlier: fetched once
           b = ldw4(rz, 8192 + e0);
           const uint4 b2 = ldw4(rz, 8192 + e0 + 2048);
@@ -862,17 +864,20 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     // the nine activation rows (8 x 512 routed + 512 shared) are 1152 chunks of 4 tagged words: 3 per thread
     const rsrc_t ra = co_rsrc(uni(F.tact)), rs = co_rsrc(uni(F.tsh)), rg = co_rsrc(uni(F.tsg));
     unsigned spins = 0;
+    bool have[3] = {false, false, false};         // a chunk that has arrived is not fetched again
     fstamp(P, 12, 0);
     for (;;) {
       bool ok = true;
       if (wave < 6) {
 #pragma unroll
         for (int c = 0; c < 3; ++c) {
+          if (have[c]) continue;
           // chunk t holds elements 4(t%128).. of slot t/128 (slot 8 = shared): packed pairs 2(t%128), 2(t%128)+1
           const int t = tid + 384 * c, slot = t >> 7, pi = 2 * (t & 127);
           const uint4 a4 = (slot < 8) ? ldw4(ra, 4 * t) : ldw4(rs, 4 * (t & 127));
           const uint32_t tx = (slot < 8) ? tb : ta;
-          ok = ok && tag_ok(a4.x, tx) && tag_ok(a4.y, tx) && tag_ok(a4.z, tx) && tag_ok(a4.w, tx);
+          have[c] = tag_ok(a4.x, tx) && tag_ok(a4.y, tx) && tag_ok(a4.z, tx) && tag_ok(a4.w, tx);
+          ok = ok && have[c];
           *reinterpret_cast<uint2*>(&xc[(slot * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
               make_uint2((a4.x & 0xffffu) | (a4.y << 16), (a4.z & 0xffffu) | (a4.w << 16));
         }
