@@ -49,6 +49,8 @@ def main():
     ap.add_argument("--chain", type=int, default=8, help="tokens per on-device chain")
     ap.add_argument("--layers", type=int, default=40, help="for quick functional runs only")
     ap.add_argument("--cpu-tokens", type=int, default=4, help="decode tokens timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--lanes", type=int, default=0, metavar="B",
+                    help="also time B lanes stepped as one batch of rows on the same weights (extra object in the JSON line)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run a plain device copy of this many MiB (reference for rocprofv3 FETCH_SIZE/WRITE_SIZE) and exit")
     args = ap.parse_args()
@@ -121,6 +123,34 @@ def main():
     head_gbs = total_b / (head_avg_ms * 1e-3) / 1e9 if head_n else 0.0
     step_gbs = total_b / (ms_step * 1e-3) / 1e9
 
+    lanes_report = None
+    if args.lanes > 1:
+        B = args.lanes
+        lanes = [eng.new_lane(max_m=B, max_seq_len=256) for _ in range(B)]
+        rng = np.random.default_rng(4000)
+        toks = []
+        for i, lane in enumerate(lanes):                 # lanes at different short contexts
+            pr = rng.integers(0, cfg.vocab, 8 + (i * 5) % 40).astype(np.int32)
+            o = None
+            for j in range(0, len(pr), B):
+                o = lane.step_argmax(pr[j:j + B])
+                assert o is not None, lane.gpu_fault
+            toks.append(int(o[-1]))
+        step = type(eng).lane_step_argmax
+        for _ in range(2):
+            toks = step(lanes, toks).tolist()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        n_lane_steps = 8
+        for _ in range(n_lane_steps):
+            toks = step(lanes, toks).tolist()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        lanes_report = {"lanes": B, "ms_per_step": dt * 1e3 / n_lane_steps, "tok_s_aggregate": B * n_lane_steps / dt,
+                        "contexts": "8-56 tokens", "path": "rows of the kernel-per-stage path, one launch sequence for all lanes"}
+        for lane in lanes:
+            lane.close()
+
     cpu = None
     if host is not None:
         from oracle import orc
@@ -150,6 +180,7 @@ def main():
                      "traffic": TRAFFIC_BYTES_PER_LAUNCH, "launches": head_n, "avg_ms": head_avg_ms, "bytes_per_launch": total_b},
         "step_hbm": {"bytes_per_token": total_b, "achieved_GBs": step_gbs, "frac_of_peak": step_gbs / HBM_PEAK_GBS},
         "cpu_baseline": cpu,
+        "lane_batch": lanes_report,
         "setup_s": {"generate": t_gen, "prefill_512": t_prefill},
         "tokens_head": stream[:8],
     }))

@@ -155,8 +155,12 @@ int sl_step_sample_rows(sl_engine* e, const int32_t* tokens, int m, float temper
  * destroyed after its lanes.  The lane is a full engine: every entry point works on it. */
 int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine** out);
 /* SeedlessLaneBatch.stepArgmaxBatch (SeedlessLaneBatch.swift:876): one token in and one out per lane, per
- * lane identical to a solo sl_step_argmax of that lane.  The lanes' steps run back to back (each is one
- * launch of the single-launch step); weights are not shared between the lanes within a step. */
+ * lane identical (bit for bit) to a solo sl_step_argmax of that lane.  With 2 <= b <= max_m of lanes[0], and
+ * lanes of one base and one max_seq_len, the lanes go through the layers together as b rows in the scratch of
+ * lanes[0]: every projection, expert and lm_head kernel is launched once for all lanes, the recurrence and
+ * attention kernels take each row to its lane's caches and position.  Otherwise the lanes' single-launch
+ * steps run back to back.  After a batched step sl_logits_row(lane, 0) and sl_hidden_rows(lane, 1) give that
+ * lane's row.  A device failure poisons every lane of the call. */
 int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t* out);
 /* forwardRows (SFV:3641): hidden rows in, hidden rows (final_norm=0) or final-normed rows out. */
 int sl_forward_rows(sl_engine* e, const uint16_t* x_f16, int m, int final_norm, uint16_t* out_f16);

@@ -5,6 +5,7 @@
 // token ids.  No CPU fallback exists: without a GPU every entry point fails.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -91,6 +92,12 @@ struct sl_engine {
   long head_launches = 0;
   bool use_persistent = true;
   bool inject_failure = false;
+  // lane batch driven from this engine's scratch: device table [n_layers][max_m] of the lanes last stepped together
+  LaneRef* lane_tab = nullptr;
+  std::vector<sl_engine*> lane_set;
+  // where the logits / normed rows of the most recent step live (a lane-batched step leaves them in the driver's rows)
+  const uint16_t* logits_view = nullptr;
+  const uint16_t* normed_view = nullptr;
   std::string fault;
 };
 
@@ -217,43 +224,47 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   c.d_w = L.sw_down.w; c.d_sb = L.sw_down.sb; c.shd_w = L.sh_down.w; c.shd_sb = L.sh_down.sb; c.out = e->moe_out;
   hipLaunchKernelGGL(k_moe_c, dim3(256, M), dim3(128), 0, e->stream, c);
 }
-void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs& ha) {
+// `lanes` (null for rows of one sequence) = this layer's row of the lane table: row b of the batch is lane b's next token.
+void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs& ha, const LaneRef* lanes) {
   hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_GDN_IN_N / 16, M), dim3(256), 0, e->stream, ha, L.in_proj.w, L.in_proj.sb,
                      SL_GDN_IN_N, e->proj, PROJ_STRIDE);
   GdnArgs g{};
   g.proj = e->proj; g.conv_w = L.conv_w; g.a_log = L.a_log; g.dt_bias = L.dt_bias;
   g.hist[0] = L.hist[0]; g.hist[1] = L.hist[1]; g.state[0] = L.state[0]; g.state[1] = L.state[1];
   g.st = e->st + li;       // st[1] of this view = parity of layer li
-  g.ycore = e->ycore; g.M = M;
-  hipLaunchKernelGGL(k_gdn_core, dim3(256), dim3(256), 0, e->stream, g);
+  g.ycore = e->ycore; g.M = M; g.lanes = lanes; g.layer = li;
+  hipLaunchKernelGGL(k_gdn_core, dim3(256, lanes ? M : 1), dim3(256), 0, e->stream, g);
   hipLaunchKernelGGL(k_qmv_gdn_out<2>, dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w,
                      L.out_proj.w, L.out_proj.sb, H, e->mix);
 }
-void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
+void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, const LaneRef* lanes, int lane_tiles) {
   hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_ATT_QKV_N / 16, M), dim3(256), 0, e->stream, ha, L.qkv.w, L.qkv.sb,
                      SL_ATT_QKV_N, e->proj, PROJ_STRIDE);
   AttnPrepArgs p{};
   p.proj = e->proj; p.q_norm = L.q_norm; p.k_norm = L.k_norm; p.rope_cos = e->rope_cos; p.rope_sin = e->rope_sin;
-  p.st = e->st; p.qrot = e->qrot; p.kcache = L.kcache; p.vcache = L.vcache; p.maxSeq = e->max_seq;
+  p.st = e->st; p.qrot = e->qrot; p.kcache = L.kcache; p.vcache = L.vcache; p.maxSeq = e->max_seq; p.lanes = lanes;
   hipLaunchKernelGGL(k_attn_prep, dim3(18, M), dim3(64), 0, e->stream, p);
-  const int tiles = (e->pos + M + SDPA_TILE - 1) / SDPA_TILE;
+  const int tiles = lanes ? lane_tiles : (e->pos + M + SDPA_TILE - 1) / SDPA_TILE;
   SdpaArgs s{};
   s.qrot = e->qrot; s.kcache = L.kcache; s.vcache = L.vcache; s.st = e->st; s.maxSeq = e->max_seq; s.maxTiles = e->max_tiles;
-  s.pm = e->pm; s.pl = e->pl; s.po = e->po;
+  s.pm = e->pm; s.pl = e->pl; s.po = e->po; s.lanes = lanes;
   hipLaunchKernelGGL(k_sdpa_tile, dim3(tiles, SL_ATT_KV, M), dim3(64), 0, e->stream, s);
   SdpaMergeArgs g{};
-  g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore;
+  g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore; g.lanes = lanes;
   hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
   hipLaunchKernelGGL((k_qmv_plain<2, 2>), dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, 4096, L.o_proj.w, L.o_proj.sb,
                      H, e->mix, H);
 }
 // All layers over M rows held in hA.  On return the hidden state is hA + moe_out (residual pending).
-void launch_layers(sl_engine* e, int M) {
+// With `lane_tab` the M rows are one token each of M lanes (caches and positions from the table, the longest
+// lane needing `lane_tiles` key tiles); without, M consecutive rows of this engine's own sequence.
+void launch_layers(sl_engine* e, int M, const LaneRef* lane_tab = nullptr, int lane_tiles = 0) {
   for (int li = 0; li < e->n_layers; ++li) {
     LayerDev& L = e->layers[li];
+    const LaneRef* lanes = lane_tab ? lane_tab + (size_t)li * e->max_m : nullptr;
     HiddenArgs ha{e->hA, li > 0 ? e->moe_out : nullptr, L.input_ln, e->hB, nullptr};
-    if (L.is_linear) launch_gdn_mixer(e, L, li, M, ha);
-    else launch_attn_mixer(e, L, M, ha);
+    if (L.is_linear) launch_gdn_mixer(e, L, li, M, ha, lanes);
+    else launch_attn_mixer(e, L, M, ha, lanes, lane_tiles);
     HiddenArgs hb{e->hB, e->mix, L.post_ln, e->hA, e->xn};
     launch_moe(e, L, M, hb);
   }
@@ -332,6 +343,8 @@ int alloc_layer_state(sl_engine* e, LayerDev& L) {
 }
 int alloc_runtime(sl_engine* e);
 }  // namespace
+static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, const char* what);
+static void time_end(sl_engine* e);
 
 int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** out) {
   if (!d || !out || max_m < 1 || max_seq_len < 1 || d->n_layers < 1 || !d->layers) return SL_ERR_ARG;
@@ -529,16 +542,90 @@ int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine*
   return alloc_runtime(e);
 }
 
-// One token per lane (reference: SeedlessLaneBatch.stepArgmaxBatch).  Each lane's step is the single-launch
-// step of that lane; the launches are queued back to back and the tokens read afterwards, so per lane the
-// result is that of a solo step by construction.
+namespace {
+// Lanes can be stepped as one batch of rows when they share weights and shapes with the driver (lanes[0]),
+// whose scratch rows they then use.
+bool lanes_batchable(sl_engine** lanes, int b) {
+  sl_engine* d = lanes[0];
+  if (b < 2 || b > d->max_m || !d->has_head) return false;
+  for (int i = 0; i < b; ++i) {
+    const sl_engine* l = lanes[i];
+    if (l->n_layers != d->n_layers || l->max_seq != d->max_seq || l->lm_head.w != d->lm_head.w ||
+        l->layers[0].router_w != d->layers[0].router_w) return false;
+  }
+  return true;
+}
+// Device table of the lanes' caches, [n_layers][max_m] in the driver; rebuilt when the set of lanes changes.
+int bind_lanes(sl_engine* d, sl_engine** lanes, int b) {
+  if ((int)d->lane_set.size() == b && std::equal(d->lane_set.begin(), d->lane_set.end(), lanes)) return SL_OK;
+  if (!d->lane_tab) {
+    d->lane_tab = dalloc<LaneRef>(d, (size_t)d->n_layers * d->max_m, true);
+    if (!d->lane_tab) return SL_ERR_DEVICE;
+  }
+  std::vector<LaneRef> tab((size_t)d->n_layers * d->max_m);
+  std::memset(tab.data(), 0, tab.size() * sizeof(LaneRef));
+  for (int li = 0; li < d->n_layers; ++li)
+    for (int i = 0; i < b; ++i) {
+      const LayerDev& L = lanes[i]->layers[li];
+      LaneRef& r = tab[(size_t)li * d->max_m + i];
+      r.hist[0] = L.hist[0]; r.hist[1] = L.hist[1]; r.state[0] = L.state[0]; r.state[1] = L.state[1];
+      r.kcache = L.kcache; r.vcache = L.vcache; r.st = lanes[i]->st; r.max_seq = lanes[i]->max_seq;
+    }
+  int r = copy_sync(d, d->lane_tab, tab.data(), tab.size() * sizeof(LaneRef), hipMemcpyHostToDevice); if (r) return r;
+  d->lane_set.assign(lanes, lanes + b);
+  return SL_OK;
+}
+}  // namespace
+
+// One token per lane (reference: SeedlessLaneBatch.stepArgmaxBatch, SeedlessLaneBatch.swift:876).  When the lanes
+// fit the scratch rows of lanes[0] (b <= its max_m, same weights and max_seq_len) the step runs as b rows through the
+// kernel-per-stage path: every projection, expert and lm_head kernel sees all lanes in one launch, and only the
+// recurrence and attention kernels go to each lane's own caches and position.  The arithmetic per row is that of
+// a solo step, so per lane the result is bit-identical to stepping it alone.  Otherwise the lanes' single-launch
+// steps are queued back to back.
 int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t* out) {
   if (!lanes || b < 1 || !tokens || !out) return SL_ERR_ARG;
   for (int i = 0; i < b; ++i) {
     if (!lanes[i]) return SL_ERR_ARG;
     for (int j = 0; j < i; ++j) if (lanes[j] == lanes[i]) return SL_ERR_ARG;
   }
-  for (int i = 0; i < b; ++i) { const int r = sl_step_argmax(lanes[i], tokens + i, 1, out + i); if (r) return r; }
+  if (!lanes_batchable(lanes, b)) {
+    for (int i = 0; i < b; ++i) { const int r = sl_step_argmax(lanes[i], tokens + i, 1, out + i); if (r) return r; }
+    return SL_OK;
+  }
+  sl_engine* d = lanes[0];
+  int max_pos = 0;
+  for (int i = 0; i < b; ++i) {
+    int r = guard(lanes[i]); if (r) return r;
+    if (tokens[i] < 0 || tokens[i] >= d->vocab) return SL_ERR_ARG;
+    if (lanes[i]->has_attn && lanes[i]->pos + 1 > lanes[i]->max_seq) return SL_ERR_ARG;
+    if (lanes[i]->pos > max_pos) max_pos = lanes[i]->pos;
+  }
+  int r = bind_lanes(d, lanes, b); if (r) return r;
+  // work queued on the other lanes' own streams (none after a completed call) must not overlap this step
+  for (int i = 1; i < b; ++i) SL_TRY(lanes[i], hipStreamSynchronize(lanes[i]->stream));
+  r = to_device(d, d->tok_in, tokens, (size_t)b * 4); if (r) return r;
+  SL_TRY(d, hipEventRecord(d->ev0, d->stream));
+  hipLaunchKernelGGL(k_embed, dim3(H / 256, b), dim3(256), 0, d->stream, d->tok_in, d->embed.w, d->embed.sb, d->hA);
+  launch_layers(d, b, d->lane_tab, (max_pos + 1 + SDPA_TILE - 1) / SDPA_TILE);
+  HiddenArgs ha{d->hA, d->moe_out, d->final_norm, d->hB, d->normed};
+  launch_head(d, b, ha, 0, false);
+  hipLaunchKernelGGL(k_lane_advance, dim3(b), dim3(64), 0, d->stream, d->lane_tab, d->n_layers);
+  SL_TRY(d, hipEventRecord(d->ev1, d->stream));
+  r = read_back(d, out, d->tok_out, (size_t)b * 4, "stepArgmaxBatch");
+  if (r) {   // the lanes' caches were written by the failed step: all of them are unusable
+    for (int i = 1; i < b; ++i) if (lanes[i]->fault.empty()) lanes[i]->fault = d->fault;
+    return r;
+  }
+  time_end(d);
+  for (int i = 0; i < b; ++i) {
+    sl_engine* l = lanes[i];
+    l->pos += 1;
+    for (int j = 0; j < l->n_layers; ++j) if (l->layers[j].is_linear) l->parity[j] ^= 1;
+    l->logits_view = d->logits + (size_t)i * d->vocab;
+    l->normed_view = d->normed + (size_t)i * H;
+    l->last_ms = d->last_ms;
+  }
   return SL_OK;
 }
 
@@ -617,6 +704,7 @@ static void time_end(sl_engine* e) {
 
 int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
   int r = guard(e); if (r) return r;
+  e->logits_view = e->normed_view = nullptr;
   if (!tokens || !out || !e->has_head) return SL_ERR_ARG;
   r = check_rows(e, m); if (r) return r;
   for (int i = 0; i < m; ++i) if (tokens[i] < 0 || tokens[i] >= e->vocab) return SL_ERR_ARG;
@@ -641,6 +729,7 @@ int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
 
 int sl_chained_step_argmax(sl_engine* e, int32_t first, int k, int32_t* out) {
   int r = guard(e); if (r) return r;
+  e->logits_view = e->normed_view = nullptr;
   if (!out || !e->has_head || k < 1 || k > MAX_CHAIN || first < 0 || first >= e->vocab) return SL_ERR_ARG;
   if (e->has_attn && e->pos + k > e->max_seq) return SL_ERR_ARG;
   r = to_device(e, e->tok_in, &first, 4); if (r) return r;
@@ -662,6 +751,7 @@ int sl_chained_step_argmax(sl_engine* e, int32_t first, int k, int32_t* out) {
 }
 
 static int forward_common(sl_engine* e, int m, int final_norm, uint16_t* out, const char* what) {
+  e->logits_view = e->normed_view = nullptr;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   launch_layers(e, m);
   HiddenArgs ha{e->hA, e->moe_out, final_norm ? e->final_norm : nullptr, final_norm ? e->hB : e->rows_out,
@@ -692,12 +782,18 @@ int sl_forward_tokens(sl_engine* e, const int32_t* tokens, int m, uint16_t* out)
 int sl_hidden_rows(sl_engine* e, int m, uint16_t* out) {
   int r = guard(e); if (r) return r;
   if (!out || m < 1 || m > e->max_m) return SL_ERR_ARG;
+  if (e->normed_view) {   // after a lane-batched step: this lane's one row, held by the driver
+    if (m != 1) return SL_ERR_ARG;
+    return read_back(e, out, e->normed_view, (size_t)H * 2, "hiddenRows");
+  }
   return read_back(e, out, e->normed, (size_t)m * H * 2, "hiddenRows");
 }
 int sl_logits_row(sl_engine* e, int m, uint16_t* out) {
   int r = guard(e); if (r) return r;
   if (!out || !e->has_head || m < 0 || m >= e->max_m) return SL_ERR_ARG;
-  r = copy_sync(e, out, e->logits + (size_t)m * e->vocab, (size_t)e->vocab * 2, hipMemcpyDeviceToHost);
+  if (e->logits_view && m != 0) return SL_ERR_ARG;   // after a lane-batched step a lane has one row
+  const uint16_t* src = e->logits_view ? e->logits_view : e->logits + (size_t)m * e->vocab;
+  r = copy_sync(e, out, src, (size_t)e->vocab * 2, hipMemcpyDeviceToHost);
   return r;
 }
 int sl_head_argmax(sl_engine* e, const uint16_t* normed, int m, int32_t* out) {
@@ -902,7 +998,7 @@ int sl_gdn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_
   r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
-  launch_gdn_mixer(e, e->layers[layer], layer, m, ha);
+  launch_gdn_mixer(e, e->layers[layer], layer, m, ha, nullptr);
   SL_TRY(e, hipEventRecord(e->ev1, e->stream));
   r = read_back(e, out, e->mix, (size_t)m * H * 2, "gdnLayerRows"); if (r) return r;
   time_end(e);
@@ -916,7 +1012,7 @@ int sl_attn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16
   r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
-  launch_attn_mixer(e, e->layers[layer], m, ha);
+  launch_attn_mixer(e, e->layers[layer], m, ha, nullptr, 0);
   SL_TRY(e, hipEventRecord(e->ev1, e->stream));
   r = read_back(e, out, e->mix, (size_t)m * H * 2, "attnLayerRows"); if (r) return r;
   time_end(e);

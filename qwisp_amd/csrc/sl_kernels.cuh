@@ -185,6 +185,16 @@ __global__ __launch_bounds__(256) void k_qmv_plain(const uint16_t* __restrict__ 
 // Grid: 32 value heads x 8 slices of 16 state rows; 4 waves, each wave 2 x 2 rows, a row = 32
 // lanes x 4 contiguous dk.  State layout [hv][dv][dk] fp32, ping-pong selected by st[1].
 // -------------------------------------------------------------------------------------------------
+// One sequence ("lane") of a lane-batched step as one layer's kernels see it: row b of the batch belongs to
+// lanes[b], which brings its own caches and its own step state (st[0] = position, st[1 + layer] = parity).
+struct LaneRef {
+  uint16_t* hist[2];         // Gated-DeltaNet layers
+  float* state[2];
+  uint16_t *kcache, *vcache; // attention layers
+  int32_t* st;
+  int max_seq, pad;
+};
+
 struct GdnArgs {
   const uint16_t* proj;      // [M, PROJ_STRIDE]: qkv 8192 | z 4096 | b 32 | a 32
   const float* conv_w;       // [8192, 4]
@@ -195,6 +205,8 @@ struct GdnArgs {
   const int32_t* st;         // st[1] = parity: read side
   uint16_t* ycore;           // [M, 4096]
   int M;
+  const LaneRef* lanes;      // lane batch: blockIdx.y = lane, one row each, caches and parity of that lane
+  int layer;
 };
 SL_DEV float conv_tap(const GdnArgs& a, const uint16_t* hin, int row, int ch) {
   // row of the concatenation [hist(3) | qkv(M)]
@@ -208,6 +220,12 @@ SL_DEV float conv_silu(const GdnArgs& a, const uint16_t* hin, int t, int ch) {
 }
 __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
   __shared__ float s_q[128], s_k[128], s_v[16], s_gb[2];
+  if (a.lanes) {
+    const LaneRef& r = a.lanes[blockIdx.y];
+    a.hist[0] = r.hist[0]; a.hist[1] = r.hist[1]; a.state[0] = r.state[0]; a.state[1] = r.state[1];
+    a.st = r.st + a.layer;
+    a.proj += (size_t)blockIdx.y * PROJ_STRIDE; a.ycore += (size_t)blockIdx.y * 4096; a.M = 1;
+  }
   const int hv = blockIdx.x >> 3, dvb = blockIdx.x & 7, hk = hv >> 1;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
   const int par = a.st[1];
@@ -512,11 +530,16 @@ struct AttnPrepArgs {
   uint16_t* qrot;              // [M, 16, 256]
   uint16_t *kcache, *vcache;   // [2, maxSeq, 256]
   int maxSeq;
+  const LaneRef* lanes;        // lane batch: row m is the next token of lanes[m]
 };
 __global__ __launch_bounds__(64) void k_attn_prep(AttnPrepArgs a) {
   __shared__ float s_n[256];
   const int m = blockIdx.y, hb = blockIdx.x, lane = threadIdx.x;
-  const int pos = a.st[0] + m;
+  int pos = a.st[0] + m;
+  if (a.lanes) {
+    const LaneRef& r = a.lanes[m];
+    pos = r.st[0]; a.kcache = r.kcache; a.vcache = r.vcache; a.maxSeq = r.max_seq;
+  }
   const bool isq = hb < 16;
   const uint16_t* src = a.proj + (size_t)m * PROJ_STRIDE + (isq ? hb * 512 : 8192 + (hb - 16) * 256);
   const uint16_t* nw = isq ? a.q_norm : a.k_norm;
@@ -568,12 +591,17 @@ struct SdpaArgs {
   int maxSeq, maxTiles;
   float *pm, *pl;              // [M, 16, maxTiles]
   float* po;                   // [M, 16, maxTiles, 256]
+  const LaneRef* lanes;        // lane batch: row m attends to the cache of lanes[m]
 };
 __global__ __launch_bounds__(64) void k_sdpa_tile(SdpaArgs a) {
   __shared__ __align__(16) uint16_t s_k[SDPA_TILE * KT_STRIDE];
   __shared__ __align__(16) float s_q[8 * 256];
   const int tile = blockIdx.x, kvh = blockIdx.y, m = blockIdx.z, lane = threadIdx.x;
-  const int N = a.st[0] + m + 1;
+  int N = a.st[0] + m + 1;
+  if (a.lanes) {
+    const LaneRef& r = a.lanes[m];
+    N = r.st[0] + 1; a.kcache = r.kcache; a.vcache = r.vcache; a.maxSeq = r.max_seq;
+  }
   const int j0 = tile * SDPA_TILE;
   if (j0 >= N) return;
   const int nk = min(SDPA_TILE, N - j0);
@@ -655,10 +683,11 @@ struct SdpaMergeArgs {
   const int32_t* st;
   int maxTiles;
   uint16_t* gated;             // [M, 4096]
+  const LaneRef* lanes;
 };
 __global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
   const int h = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;
-  const int N = a.st[0] + m + 1;
+  const int N = a.lanes ? a.lanes[m].st[0] + 1 : a.st[0] + m + 1;
   const int nt = (N + SDPA_TILE - 1) / SDPA_TILE;
   const size_t base = ((size_t)m * 16 + h) * a.maxTiles;
   float Mx = -__int_as_float(0x7f800000);
@@ -759,6 +788,13 @@ __global__ __launch_bounds__(64) void k_final_rows(HiddenArgs ha) {
 __global__ void k_advance(int32_t* st, int M, int n_layers) {
   const int t = threadIdx.x;
   if (t == 0) st[0] += M;
+  for (int i = t; i < n_layers; i += blockDim.x) st[1 + i] ^= 1;
+}
+// The same for every lane of a lane-batched step (one token each); blockIdx.x = lane.
+__global__ void k_lane_advance(const LaneRef* lanes, int n_layers) {
+  int32_t* st = lanes[blockIdx.x].st;
+  const int t = threadIdx.x;
+  if (t == 0) st[0] += 1;
   for (int i = t; i < n_layers; i += blockDim.x) st[1 + i] ^= 1;
 }
 // {scale, bias} interleave: the engine keeps one 32-bit pair per quantisation group.

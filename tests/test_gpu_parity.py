@@ -238,27 +238,39 @@ def test_persistent_step_long_context(env, small_model):
 
 def test_lanes_share_weights_and_equal_solo(env, small_model):
     """Lanes (SeedlessLaneBatch.swift:876): sequences on one weight set.  Per lane the token stream is that
-    of a solo engine, whatever the other lanes do; sampling is reported as unsupported."""
+    of a solo engine, whatever the other lanes do; sampling is reported as unsupported.  Three lanes fit the
+    four scratch rows of the first, so they are stepped as one batch of rows (lanes at different positions,
+    one of them past the first key tile); with five lanes the steps are queued lane by lane."""
     cfg, dev, host = small_model
     base = env["Engine"](cfg, dev, max_m=4, max_seq_len=96)
-    lanes = [base.new_lane(max_m=4, max_seq_len=96) for _ in range(3)]
-    solos = [env["Engine"](cfg, dev, max_m=4, max_seq_len=96) for _ in range(3)]
-    prompts = [[5, 6, 7], [900, 11], [42]]
+    lanes = [base.new_lane(max_m=4, max_seq_len=96) for _ in range(5)]
+    solos = [env["Engine"](cfg, dev, max_m=4, max_seq_len=96) for _ in range(5)]
+    rng = np.random.default_rng(77)
+    prompts = [rng.integers(0, cfg.vocab, size=62).tolist(), [900, 11], [42], [5, 6, 7], [8]]
     cur = []
     for lane, solo, pr in zip(lanes, solos, prompts):
-        a, b = lane.step_argmax(pr), solo.step_argmax(pr)
-        assert a is not None and b is not None, (lane.gpu_fault, solo.gpu_fault)
-        assert a.tolist() == b.tolist()
+        for i in range(0, len(pr), 4):
+            a, b = lane.step_argmax(pr[i:i + 4]), solo.step_argmax(pr[i:i + 4])
+            assert a is not None and b is not None, (lane.gpu_fault, solo.gpu_fault)
+            assert a.tolist() == b.tolist()
         cur.append(int(a[-1]))
     for step in range(12):
-        got = type(base).lane_step_argmax(lanes, cur)
+        n = 3 if step < 8 else 5          # 3 lanes: one batch of rows; 5 lanes: lane by lane
+        got = type(base).lane_step_argmax(lanes[:n], cur[:n])
         assert got is not None, [l.gpu_fault for l in lanes]
-        want = [int(solo.step_argmax([t])[0]) for solo, t in zip(solos, cur)]
+        want = [int(solo.step_argmax([t])[0]) for solo, t in zip(solos[:n], cur[:n])]
         assert got.tolist() == want, step
-        cur = want
+        cur[:n] = want
+        if step == 7:
+            for lane, solo in zip(lanes[:3], solos[:3]):
+                assert same_bits(lane.logits_row(0), solo.logits_row(0))
+                assert same_bits(lane.hidden_rows(1), solo.hidden_rows(1))
     assert [l.position for l in lanes] == [s.position for s in solos]
     for lane, solo in zip(lanes, solos):
         assert same_bits(lane.logits_row(0), solo.logits_row(0))
+    # a lane stepped in a batch goes on alone, and as rows of its own, from the same caches
+    for lane, solo, t in zip(lanes[:3], solos[:3], cur[:3]):
+        assert lane.step_argmax([t, 3, 4]).tolist() == solo.step_argmax([t, 3, 4]).tolist()
     # the base engine is untouched by its lanes and still works
     assert base.position == 0 and base.step_argmax([1, 2]) is not None
     status, out = base.step_sample_rows([3], temperature=0.7, top_p=0.9, seed=1)
