@@ -220,6 +220,53 @@ int sl_debug_scratch(sl_engine* e, int which, uint16_t* out_f16, size_t count);
 int sl_greedy_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_new, int chain_k,
                        int32_t* out);
 
+/* ---- Tell's SuffixSpec loop (host logic above the entry points; no device code of its own) -------------
+ * Tell.suffixDraft (Tell.swift:104-175): the longest suffix of seq[0, n) of length min_match..max_match that
+ * also occurs earlier; every earlier occurrence votes token by token on the continuation (ties go to the
+ * most recent occurrence, occurrences that disagree drop out).  At most min(draft_k, 4 * match length)
+ * tokens are written to `draft`; returns their number (0 = no draft) or SL_ERR_ARG. */
+int sl_suffix_draft(const int32_t* seq, int n, int max_match, int draft_k, int min_match, int32_t* draft);
+/* The mechanical speculation gate (Tell.swift:45-57): break-even threshold of accepted tokens per attempt,
+ * attempts needed before suspending, and the decision on a rolling window of accepted counts (1 / 0). */
+int sl_spec_gate_threshold(int hist_len);
+int sl_spec_gate_window_needed(int hist_len);
+int sl_spec_gate_should_suspend(const int32_t* window, int n, int hist_len);
+
+typedef struct {
+  int32_t max_draft;     /* cap on draft length (maxK); verify rows = 1 + drafts <= max_m */
+  int32_t chain_k;       /* draftless spans run as chains of this many steps (0 = single steps); Tell default 8 */
+  int32_t min_match;     /* QWISP_SUFFIX_MINMATCH, default 4 */
+  int32_t gate;          /* 1 = speculation gate on (QWISP_SPEC_GATE) */
+  int32_t gate_reprobe;  /* emitted tokens before drafting is tried again (QWISP_SPEC_REPROBE, default 256, >= 8) */
+} sl_spec_options;
+typedef struct {
+  int32_t steps, drafted, accepted, draftless, rejects, chain_calls, gate_suspensions, reserved;
+} sl_spec_stats;
+/* Tell.runSpecLoop without its A3 mode (TellRuntime.swift:716-886): prefill, then per step a suffix draft,
+ * one sl_step_argmax over [pending token] + drafts, acceptance of the matching prefix; a reject is undone with
+ * sl_rollback_one_step and the accepted rows are run again with sl_forward_tokens.  The n_new tokens written to
+ * `out` are those of sl_greedy_generate.  max_seq_len must cover n_prompt + n_new + max_draft + chain_k. */
+int sl_spec_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_new, const sl_spec_options* opt,
+                     int32_t* out, sl_spec_stats* stats);
+/* The same loop on a table of callbacks shaped like Tell.SpecBackend (TellRuntime.swift:83-111); every
+ * callback returns 0 or an error that ends the loop.  first_token = argmax of the head on the last row of
+ * the most recent forward_tokens; rollback undoes the one step made since the last snapshot;
+ * chained_step_argmax may be NULL (then draftless spans run as single steps). */
+typedef struct {
+  void* ctx;
+  int32_t max_rows;
+  int (*step_argmax)(void* ctx, const int32_t* tokens, int m, int32_t* out);
+  int (*chained_step_argmax)(void* ctx, int32_t first, int k, int32_t* out);
+  int (*forward_tokens)(void* ctx, const int32_t* tokens, int m);
+  int (*first_token)(void* ctx, int32_t* out);
+  int (*snapshot)(void* ctx);
+  int (*rollback)(void* ctx);
+} sl_spec_backend;
+int sl_spec_generate_backend(const sl_spec_backend* b, const int32_t* prompt, int n_prompt, int n_new,
+                             const sl_spec_options* opt, int32_t* out, sl_spec_stats* stats);
+/* max_m of the engine (rows per call). */
+int sl_max_rows(const sl_engine* e);
+
 /* Timing of the most recent step on the engine's stream, measured with HIP events
  * (profLastGPUMs, SFV:3137). */
 float sl_last_gpu_ms(const sl_engine* e);

@@ -55,6 +55,28 @@ class Snap(C.Structure):
     _fields_ = [("kv_len", C.c_int32), ("reserved", C.c_int32)]
 
 
+class SpecOptions(C.Structure):
+    _fields_ = [("max_draft", C.c_int32), ("chain_k", C.c_int32), ("min_match", C.c_int32), ("gate", C.c_int32),
+                ("gate_reprobe", C.c_int32)]
+
+
+class SpecStats(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("steps", "drafted", "accepted", "draftless", "rejects", "chain_calls",
+                                         "gate_suspensions", "reserved")]
+
+
+STEP_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int32), C.c_int, C.POINTER(C.c_int32))
+CHAIN_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int32, C.c_int, C.POINTER(C.c_int32))
+FORWARD_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int32), C.c_int)
+FIRST_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int32))
+VOID_FN = C.CFUNCTYPE(C.c_int, C.c_void_p)
+
+
+class SpecBackend(C.Structure):
+    _fields_ = [("ctx", C.c_void_p), ("max_rows", C.c_int32), ("step_argmax", STEP_FN), ("chained_step_argmax", CHAIN_FN),
+                ("forward_tokens", FORWARD_FN), ("first_token", FIRST_FN), ("snapshot", VOID_FN), ("rollback", VOID_FN)]
+
+
 def _ptr(t):
     """Address of a numpy array or a torch tensor."""
     if t is None:

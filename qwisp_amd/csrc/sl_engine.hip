@@ -651,6 +651,7 @@ void sl_destroy(sl_engine* e) {
 const char* sl_fault(const sl_engine* e) { return (e && !e->fault.empty()) ? e->fault.c_str() : nullptr; }
 void sl_inject_failure(sl_engine* e) { if (e) e->inject_failure = true; }
 int sl_position(const sl_engine* e) { return e ? e->pos : -1; }
+int sl_max_rows(const sl_engine* e) { return e ? e->max_m : -1; }
 float sl_last_gpu_ms(const sl_engine* e) { return e ? e->last_ms : 0.0f; }
 void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
 int sl_set_persistent(sl_engine* e, int enable) {

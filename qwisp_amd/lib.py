@@ -45,6 +45,14 @@ SIGNATURES = {
     "sl_attn_layer_rows": (_i32, [_vp, _i32, _vp, _i32, _vp]),
     "sl_debug_scratch": (_i32, [_vp, _i32, _vp, _sz]),
     "sl_greedy_generate": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp]),
+    "sl_suffix_draft": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp]),
+    "sl_spec_gate_threshold": (_i32, [_i32]),
+    "sl_spec_gate_window_needed": (_i32, [_i32]),
+    "sl_spec_gate_should_suspend": (_i32, [_vp, _i32, _i32]),
+    "sl_spec_generate": (_i32, [_vp, _vp, _i32, _i32, C.POINTER(abi.SpecOptions), _vp, C.POINTER(abi.SpecStats)]),
+    "sl_spec_generate_backend": (_i32, [C.POINTER(abi.SpecBackend), _vp, _i32, _i32, C.POINTER(abi.SpecOptions), _vp,
+                                        C.POINTER(abi.SpecStats)]),
+    "sl_max_rows": (_i32, [_vp]),
     "sl_last_gpu_ms": (_f32, [_vp]),
     "sl_stream": (_vp, [_vp]),
     "sl_set_persistent": (_i32, [_vp, _i32]),

@@ -280,6 +280,35 @@ def test_lanes_share_weights_and_equal_solo(env, small_model):
         lane.close()
 
 
+def test_spec_loop_stream_equals_greedy_stream(env):
+    """Tell.runSpecLoop on the engine (TellRuntime.swift:716-886): suffix drafts verified as rows of one step,
+    rejects rolled back and rebuilt.  The stream must be the greedy stream token for token (a verify step of M
+    rows is bit-identical to M single steps here), whatever is drafted, accepted or rejected.  A random model
+    rarely repeats itself, so drafts are provoked with a 64-token vocabulary and a match length of 1; most are
+    wrong, which exercises snapshot -> M-row step -> rollback -> rebuild on the device."""
+    cfg = ModelConfig(n_layers=4, n_experts=8, vocab=64)
+    dev, host = device_and_host_model(cfg)
+    rng = np.random.default_rng(5)
+    motif = rng.integers(0, cfg.vocab, 9).tolist()
+    prompt = motif + [17, 18] + motif + [19] + motif[:6]          # repeats: drafts from the first step on
+    n_new = 160
+    ref = env["Engine"](cfg, dev, max_m=8, max_seq_len=256)
+    want = ref.greedy_generate(prompt, n_new, chain_k=8)
+    assert want is not None, ref.gpu_fault
+    for max_draft, chain_k, gate in [(7, 8, False), (3, 0, False), (7, 4, True)]:
+        eng = env["Engine"](cfg, dev, max_m=8, max_seq_len=256)
+        res = eng.spec_generate(prompt, n_new, max_draft=max_draft, chain_k=chain_k, min_match=1, gate=gate, gate_reprobe=8)
+        assert res is not None, eng.gpu_fault
+        got, st = res
+        assert got.tolist() == want.tolist(), (max_draft, chain_k, gate, st)
+        print("spec loop", (max_draft, chain_k, gate), st)
+        assert st["drafted"] > 0 and st["accepted"] <= st["drafted"] and st["steps"] > 0
+        assert st["rejects"] > 0 or st["accepted"] == st["drafted"]
+        assert eng.position >= len(prompt) + n_new - 1
+        eng.close()
+    ref.close()
+
+
 def test_forward_rows_and_head(env, small_model):
     cfg, dev, host = small_model
     eng = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)
