@@ -264,6 +264,49 @@ typedef struct {
 } sl_spec_backend;
 int sl_spec_generate_backend(const sl_spec_backend* b, const int32_t* prompt, int n_prompt, int n_new,
                              const sl_spec_options* opt, int32_t* out, sl_spec_stats* stats);
+/* ---- continuous batching: the scheduler seam (host logic; a device is reached only through the callbacks) ----
+ * BatchSlots (ContinuousBatch.swift:38-66) as a table of callbacks.
+ *   admit_step: advance the prefill of `prompt` in `slot` by at most token_budget tokens but at least one
+ *     chunk (token_budget <= 0: the whole prompt).  The full prompt is passed every call, the slot keeps its own
+ *     resume position.  seq_budget = prompt + 1 + max_tokens, the arena the request needs (0 = unknown).
+ *     Returns 0 when the prompt is done (*first = greedy first token), 1 when paused at a chunk boundary,
+ *     < 0 on failure; *consumed = tokens processed in this call.
+ *   step: one batched decode step; last[b] = token to feed slot b or -1 for an idle slot; next[b] likewise.
+ *   release: the slot's request is over.   can_admit (may be NULL = always): the aggregate memory gate. */
+typedef struct {
+  void* ctx;
+  int32_t slot_count;
+  int (*admit_step)(void* ctx, const int32_t* prompt, int n_prompt, int slot, int token_budget, int seq_budget,
+                    int32_t* first, int32_t* consumed);
+  int (*step)(void* ctx, const int32_t* last, int32_t* next);
+  void (*release)(void* ctx, int slot);
+  int (*can_admit)(void* ctx, int prompt_len, int seq_budget);
+} sl_batch_slots;
+typedef void (*sl_token_fn)(void* user, int job, int32_t token);
+typedef void (*sl_finish_fn)(void* user, int job);
+typedef struct sl_sched sl_sched;
+/* ContinuousScheduler (ContinuousBatch.swift:95-266).  token_budget 0: a request is prefilled whole when a slot
+ * frees up, then all active slots step together; token_budget > 0: per round the running slots' tokens are
+ * reserved first and the rest of the budget drains waiting prefill in submission order, so decode is never
+ * starved by a long prompt.  Stop tokens are not emitted; a request ends at max_tokens.  Runs on the caller's
+ * thread: sl_sched_submit returns the job id (>= 0) reported to the callbacks, sl_sched_round does one
+ * scheduling round and returns the number of requests still queued, prefilling or running (0 = idle) or an
+ * error.  The caller serialises submit and round. */
+int sl_sched_create(const sl_batch_slots* slots, int token_budget, sl_token_fn on_token, sl_finish_fn on_finish,
+                    void* user, sl_sched** out);
+void sl_sched_destroy(sl_sched* s);
+int sl_sched_submit(sl_sched* s, const int32_t* prompt, int n_prompt, int max_tokens, const int32_t* stop, int n_stop);
+int sl_sched_round(sl_sched* s);
+/* LaneBatchSlots (LaneServe.swift:26): n_slots lanes on the weights of `base`; prefill in chunks of chunk_rows
+ * rows, resumable at chunk boundaries (a budget grants whole chunks, rounded up, at least one); decode through
+ * sl_lane_step_argmax; can_admit holds the sum of the admitted requests' seq_budget within kv_budget_tokens
+ * (<= 0: n_slots * max_seq_len).  Fills `table` for sl_sched_create; destroy after the scheduler, before `base`. */
+typedef struct sl_lane_slots sl_lane_slots;
+int sl_lane_slots_create(const sl_engine* base, int n_slots, int chunk_rows, int max_seq_len, long kv_budget_tokens,
+                         sl_lane_slots** out, sl_batch_slots* table);
+void sl_lane_slots_destroy(sl_lane_slots* slots);
+/* Back to the cold state of a new engine: position 0, conv history and recurrent state zero (release of a slot). */
+int sl_reset(sl_engine* e);
 /* max_m of the engine (rows per call). */
 int sl_max_rows(const sl_engine* e);
 

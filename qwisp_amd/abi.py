@@ -77,6 +77,20 @@ class SpecBackend(C.Structure):
                 ("forward_tokens", FORWARD_FN), ("first_token", FIRST_FN), ("snapshot", VOID_FN), ("rollback", VOID_FN)]
 
 
+ADMIT_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int32), C.c_int, C.c_int, C.c_int, C.c_int,
+                       C.POINTER(C.c_int32), C.POINTER(C.c_int32))
+SLOT_STEP_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int32), C.POINTER(C.c_int32))
+RELEASE_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_int)
+CAN_ADMIT_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_int)
+TOKEN_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_int, C.c_int32)
+FINISH_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_int)
+
+
+class BatchSlots(C.Structure):
+    _fields_ = [("ctx", C.c_void_p), ("slot_count", C.c_int32), ("admit_step", ADMIT_FN), ("step", SLOT_STEP_FN),
+                ("release", RELEASE_FN), ("can_admit", CAN_ADMIT_FN)]
+
+
 def _ptr(t):
     """Address of a numpy array or a torch tensor."""
     if t is None:

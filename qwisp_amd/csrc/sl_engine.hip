@@ -819,6 +819,20 @@ int sl_rollback_one_step(sl_engine* e, const sl_snap* s) {
   for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
   return push_state(e);
 }
+int sl_reset(sl_engine* e) {
+  int r = guard(e); if (r) return r;
+  for (LayerDev& L : e->layers) {
+    if (!L.is_linear) continue;
+    for (int p = 0; p < 2; ++p) {
+      SL_TRY(e, hipMemsetAsync(L.hist[p], 0, HIST_ELEMS * sizeof(uint16_t), e->stream));
+      SL_TRY(e, hipMemsetAsync(L.state[p], 0, STATE_ELEMS * sizeof(float), e->stream));
+    }
+  }
+  e->pos = 0;
+  e->parity.assign(e->n_layers, 0);
+  e->logits_view = e->normed_view = nullptr;
+  return push_state(e);
+}
 int sl_full_snapshot(sl_engine* e, sl_full_snap** out) {
   int r = guard(e); if (r) return r;
   if (!out) return SL_ERR_ARG;

@@ -263,3 +263,56 @@ class _FullSnap:
         if self.h:
             self.lib.dll.sl_full_snap_free(self.h)
             self.h = None
+
+
+class LaneScheduler:
+    """ContinuousScheduler over LaneBatchSlots (ContinuousBatch.swift:95, LaneServe.swift:26): requests queue up,
+    free slots admit, all active slots decode in one batched step per round.  Synchronous: `run()` drives rounds
+    until every submitted request has finished and returns the token streams in submission order."""
+
+    def __init__(self, base, slots, chunk_rows=8, max_seq_len=1024, token_budget=0, kv_budget_tokens=0):
+        self.lib, self.base = base.lib, base
+        self.streams, self.finished = [], []
+        self._tok = abi.TOKEN_FN(lambda user, job, t: self.streams[job].append(t))
+        self._fin = abi.FINISH_FN(lambda user, job: self.finished.append(job))
+        self.table = abi.BatchSlots()
+        self.slots = C.c_void_p()
+        self.h = C.c_void_p()
+        r = self.lib.dll.sl_lane_slots_create(base.h, slots, chunk_rows, max_seq_len, kv_budget_tokens, C.byref(self.slots),
+                                              C.byref(self.table))
+        if r != abi.SL_OK:
+            self.close()
+            raise _lib.SeedlessError("sl_lane_slots_create", r)
+        r = self.lib.dll.sl_sched_create(C.byref(self.table), token_budget, self._tok, self._fin, None, C.byref(self.h))
+        if r != abi.SL_OK:
+            self.close()
+            raise _lib.SeedlessError("sl_sched_create", r)
+
+    def submit(self, prompt, max_tokens, stop=()):
+        p = np.ascontiguousarray(prompt, np.int32)
+        s = np.ascontiguousarray(list(stop), np.int32)
+        jid = self.lib.dll.sl_sched_submit(self.h, _p(p), len(p), max_tokens, _p(s) if len(s) else None, len(s))
+        if jid < 0:
+            raise _lib.SeedlessError("sl_sched_submit", jid)
+        self.streams.append([])
+        return jid
+
+    def round(self):
+        return self.lib.dll.sl_sched_round(self.h)
+
+    def run(self, max_rounds=1 << 20):
+        for _ in range(max_rounds):
+            left = self.round()
+            if left < 0:
+                return None
+            if left == 0:
+                return self.streams
+        return None
+
+    def close(self):
+        if self.h:
+            self.lib.dll.sl_sched_destroy(self.h)
+            self.h = C.c_void_p()
+        if self.slots:
+            self.lib.dll.sl_lane_slots_destroy(self.slots)
+            self.slots = C.c_void_p()

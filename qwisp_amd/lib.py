@@ -52,6 +52,13 @@ SIGNATURES = {
     "sl_spec_generate": (_i32, [_vp, _vp, _i32, _i32, C.POINTER(abi.SpecOptions), _vp, C.POINTER(abi.SpecStats)]),
     "sl_spec_generate_backend": (_i32, [C.POINTER(abi.SpecBackend), _vp, _i32, _i32, C.POINTER(abi.SpecOptions), _vp,
                                         C.POINTER(abi.SpecStats)]),
+    "sl_sched_create": (_i32, [C.POINTER(abi.BatchSlots), _i32, abi.TOKEN_FN, abi.FINISH_FN, _vp, C.POINTER(_vp)]),
+    "sl_sched_destroy": (None, [_vp]),
+    "sl_sched_submit": (_i32, [_vp, _vp, _i32, _i32, _vp, _i32]),
+    "sl_sched_round": (_i32, [_vp]),
+    "sl_lane_slots_create": (_i32, [_vp, _i32, _i32, _i32, C.c_long, C.POINTER(_vp), C.POINTER(abi.BatchSlots)]),
+    "sl_lane_slots_destroy": (None, [_vp]),
+    "sl_reset": (_i32, [_vp]),
     "sl_max_rows": (_i32, [_vp]),
     "sl_last_gpu_ms": (_f32, [_vp]),
     "sl_stream": (_vp, [_vp]),

@@ -43,7 +43,7 @@ def test_ctypes_structs_match_the_c_layout(tmp_path):
         int main(void) {
           printf("%zu %zu %zu %zu %zu %zu %zu\\n", sizeof(sl_q4), sizeof(sl_gdn_w), sizeof(sl_attn_w), sizeof(sl_moe_w),
                  sizeof(sl_layer_desc), sizeof(sl_model_desc), sizeof(sl_snap));
-          printf("%zu %zu %zu\\n", sizeof(sl_spec_options), sizeof(sl_spec_stats), sizeof(sl_spec_backend));
+          printf("%zu %zu %zu %zu\\n", sizeof(sl_spec_options), sizeof(sl_spec_stats), sizeof(sl_spec_backend), sizeof(sl_batch_slots));
           printf("%zu %zu %zu %zu\\n", offsetof(sl_layer_desc, gdn), offsetof(sl_layer_desc, attn), offsetof(sl_layer_desc, moe),
                  offsetof(sl_model_desc, embed));
           return 0;
@@ -52,7 +52,7 @@ def test_ctypes_structs_match_the_c_layout(tmp_path):
     subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), "-o", str(exe), str(prog)])
     out = subprocess.check_output([str(exe)]).decode().split()
     sizes = [C.sizeof(t) for t in (abi.Q4, abi.GdnW, abi.AttnW, abi.MoeW, abi.LayerDesc, abi.ModelDesc, abi.Snap,
-                                   abi.SpecOptions, abi.SpecStats, abi.SpecBackend)]
+                                   abi.SpecOptions, abi.SpecStats, abi.SpecBackend, abi.BatchSlots)]
     offs = [abi.LayerDesc.gdn.offset, abi.LayerDesc.attn.offset, abi.LayerDesc.moe.offset, abi.ModelDesc.embed.offset]
     assert [int(x) for x in out] == sizes + offs
 

@@ -309,6 +309,41 @@ def test_spec_loop_stream_equals_greedy_stream(env):
     ref.close()
 
 
+def test_scheduler_over_lane_slots_streams_equal_solo(env, small_model):
+    """ContinuousScheduler + LaneBatchSlots (ContinuousBatch.swift:95, LaneServe.swift:26): six requests on three
+    slots, atomic and token-budgeted (prefill paused and resumed at chunk boundaries, interleaved with decode).
+    Whatever the schedule, each request's stream is the solo greedy stream of its prompt, and stop tokens and
+    length caps are honoured."""
+    from qwisp_amd.engine import LaneScheduler
+    cfg, dev, host = small_model
+    base = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)
+    rng = np.random.default_rng(11)
+    prompts = [rng.integers(0, cfg.vocab, n).tolist() for n in (3, 17, 9, 1, 30, 6)]
+    caps = [6, 4, 9, 5, 3, 7]
+    solo = []
+    for pr in prompts:
+        e = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)
+        solo.append(e.greedy_generate(pr, 9, chain_k=1).tolist())
+        e.close()
+    stop2 = solo[2][4]                                  # request 2 ends at its fifth token, which is not emitted
+    cut2 = solo[2].index(stop2)
+    for budget in (0, 6):
+        sch = LaneScheduler(base, slots=3, chunk_rows=4, max_seq_len=64, token_budget=budget)
+        for i, pr in enumerate(prompts):
+            sch.submit(pr, caps[i], stop=[stop2] if i == 2 else [])
+        streams = sch.run(max_rounds=500)
+        assert streams is not None
+        for i in range(len(prompts)):
+            want = solo[i][:caps[i]]
+            if i == 2:
+                want = solo[2][:min(cut2, caps[2])]
+            assert streams[i] == want, (budget, i)
+        assert sorted(sch.finished) == list(range(len(prompts)))
+        sch.close()
+    assert base.position == 0
+    base.close()
+
+
 def test_forward_rows_and_head(env, small_model):
     cfg, dev, host = small_model
     eng = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)
