@@ -503,16 +503,52 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   wload_row<2>(wr.w[0], wr.sb[0], uni(Y.out_w), uni(Y.out_sb), (size_t)(valid ? gw : 0), valid, lane);
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
-  if (!lin && wg == G - 1) {        // the last workgroup owns a tile unit only in very long contexts, so its
+  if (!lin && wg >= G - 2) {        // the last workgroups own a tile unit only in very long contexts, so their
                                      // waves have no stores of their own to wait for
-    // Merge the attention tiles of head `wave` in order with the global max (each wave polls on its own).
-    // The round trips are batched: lane i fetches {max, sum} of tile t0+i (64 tiles per load), the per-dim
-    // partials of 4 tiles are in flight at a time; the accumulation itself runs in tile order.
-    const int h = wave, slot0 = h * uni(P.max_tiles);
-    const rsrc_t rml = co_rsrc(uni(F.tml)), rpo = co_rsrc(uni(F.tpo));
+    // Merge the attention tiles in order with the global max: 8 heads per workgroup, two waves per head, a lane
+    // owns one 16-byte chunk (2 dims) of the 256; each wave polls on its own.  The round trips are batched:
+    // lane i fetches {max, sum} of tile t0+i (64 tiles per load) and the partials of MB tiles are in flight at
+    // a time; the accumulation itself runs in tile order.
+    const int h = (wg - (G - 2)) * 8 + (wave >> 1), slot0 = h * uni(P.max_tiles), chunk = 64 * (wave & 1) + lane;
+    const rsrc_t rml = co_rsrc(uni(F.tml)), rpo = co_rsrc(uni(F.tpo)), rp = co_rsrc(uni(F.tproj));
     int fail = 0;
     float Mx = NEG;
-    for (int t0 = 0; t0 < nt && !fail; t0 += 64) {
+    // First round trip: {max, sum} of the first 64 tiles, the partials of the first MB tiles and the output gate
+    // (it sits in the q projection of this step) are polled together, each piece until it has arrived; at short
+    // contexts that is everything the merge needs.
+    constexpr int MB = 12;
+    uint4 a[MB];
+    uint4 m0 = make_uint4(0, 0, 0, 0);
+    uint2 g2 = make_uint2(0u, 0u);
+    {
+      const bool mine = lane < nt;
+      const int cnt0 = min(MB, nt);
+      bool mdone = false, gdone = false;
+      unsigned have = 0, spins = 0;
+      for (;;) {
+        if (!mdone) {
+          bool ok = true;
+          if (mine) { m0 = ldw4(rml, (slot0 + lane) * 4); ok = m0.z == tcore32 && m0.w == tcore32; }
+          mdone = __all(ok ? 1 : 0) != 0;
+        }
+        if (!gdone) {
+          g2 = ldw2(rp, h * 512 + 256 + 2 * chunk);
+          gdone = __all((tag_ok(g2.x, tin) && tag_ok(g2.y, tin)) ? 1 : 0) != 0;
+        }
+#pragma unroll
+        for (int u = 0; u < MB; ++u) {
+          if (u < cnt0 && !(have & (1u << u))) {
+            a[u] = ldw4(rpo, ((slot0 + u) * 128 + chunk) * 4);
+            if (__all((a[u].z == tcore32 && a[u].w == tcore32) ? 1 : 0)) have |= 1u << u;
+          }
+        }
+        if (mdone && gdone && have == (1u << cnt0) - 1u) break;
+        if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      Mx = tree_max<64>(mine ? __uint_as_float(m0.x) : NEG);
+    }
+    for (int t0 = 64; t0 < nt && !fail; t0 += 64) {       // maxima of the tiles beyond the first 64
       const bool mine = t0 + lane < nt;
       unsigned spins = 0;
       for (;;) {
@@ -524,57 +560,46 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
         __builtin_amdgcn_s_sleep(1);
       }
     }
-    float Ls = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float Ls = 0.0f, O0 = 0.0f, O1 = 0.0f;
     for (int t0 = 0; t0 < nt && !fail; t0 += 64) {
       float fl = 0.0f, pl = 0.0f;                         // lane i: scale and sum of tile t0+i (tags verified above)
       if (t0 + lane < nt) {
-        const uint4 m = ldw4(rml, (slot0 + t0 + lane) * 4);
+        const uint4 m = t0 == 0 ? m0 : ldw4(rml, (slot0 + t0 + lane) * 4);
         fl = exp_c(__uint_as_float(m.x) - Mx); pl = __uint_as_float(m.y);
       }
       const int cnt = min(64, nt - t0);
-      for (int u0 = 0; u0 < cnt && !fail; u0 += 4) {
-        uint4 a[4], b[4];
-        unsigned spins = 0;
-        for (;;) {
-          bool ok = true;
+      for (int u0 = 0; u0 < cnt && !fail; u0 += MB) {
+        if (t0 + u0 > 0) {                                // the first batch is already here
+          unsigned spins = 0;
+          for (;;) {
+            bool ok = true;
 #pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            if (u0 + u < cnt) {
-              const int t = slot0 + t0 + u0 + u;
-              a[u] = ldw4(rpo, (t * 128 + 2 * lane) * 4); b[u] = ldw4(rpo, (t * 128 + 2 * lane + 1) * 4);
-              ok = ok && a[u].z == tcore32 && a[u].w == tcore32 && b[u].z == tcore32 && b[u].w == tcore32;
+            for (int u = 0; u < MB; ++u) {
+              if (u0 + u < cnt) {
+                a[u] = ldw4(rpo, ((slot0 + t0 + u0 + u) * 128 + chunk) * 4);
+                ok = ok && a[u].z == tcore32 && a[u].w == tcore32;
+              }
             }
+            if (__all(ok ? 1 : 0)) break;
+            if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+            __builtin_amdgcn_s_sleep(1);
           }
-          if (__all(ok ? 1 : 0)) break;
-          if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
-          __builtin_amdgcn_s_sleep(1);
+          if (fail) break;
         }
-        if (fail) break;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < MB; ++u) {
           if (u0 + u < cnt) {
             const float f = row_lane_f(fl, u0 + u), l = row_lane_f(pl, u0 + u);
             Ls = fmaf(l, f, Ls);
-            O[0] = fmaf(__uint_as_float(a[u].x), f, O[0]); O[1] = fmaf(__uint_as_float(a[u].y), f, O[1]);
-            O[2] = fmaf(__uint_as_float(b[u].x), f, O[2]); O[3] = fmaf(__uint_as_float(b[u].y), f, O[3]);
+            O0 = fmaf(__uint_as_float(a[u].x), f, O0); O1 = fmaf(__uint_as_float(a[u].y), f, O1);
           }
         }
       }
     }
-    // the output gate sits in the q projection of this step
-    const rsrc_t rp = co_rsrc(uni(F.tproj));
-    uint4 g4 = make_uint4(0, 0, 0, 0);
-    for (unsigned spins = 0; !fail;) {
-      g4 = ldw4(rp, h * 512 + 256 + 4 * lane);
-      if (__all((tag_ok(g4.x, tin) && tag_ok(g4.y, tin) && tag_ok(g4.z, tin) && tag_ok(g4.w, tin)) ? 1 : 0)) break;
-      if (++spins > FLOW_SPIN_LIMIT) fail = 1;
-    }
     if (fail) st_co32(uni(P.bar) + 32, 1u);
-    const float gt[4] = {lo_h(g4.x), lo_h(g4.y), lo_h(g4.z), lo_h(g4.w)};
-    uint32_t r[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) r[i] = tagged(f16r(f16r(O[i] / Ls) * sigmoid16(gt[i])), tmerge);
-    if (!fail) stw4(co_rsrc(uni(F.tycore)), h * 256 + 4 * lane, r[0], r[1], r[2], r[3]);
+    const uint32_t r0 = tagged(f16r(f16r(O0 / Ls) * sigmoid16(lo_h(g2.x))), tmerge);
+    const uint32_t r1 = tagged(f16r(f16r(O1 / Ls) * sigmoid16(lo_h(g2.y))), tmerge);
+    if (!fail) stw2(co_rsrc(uni(F.tycore)), h * 256 + 2 * chunk, r0, r1);
   }
   if (wg * DEC_WAVES >= H) {                       // no output row here (uniform per workgroup): nothing to fetch
     if (lin) store_hist(Y, li, gh);
