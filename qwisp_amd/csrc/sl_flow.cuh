@@ -476,6 +476,139 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
   return true;
 }
 
+// The same stage at contexts of up to G/8 key tiles: a unit is (tile, kv head, quarter of the group's 8 query
+// heads), so four times as many workgroups share the work and a unit's arithmetic is a quarter.  Wave (head of
+// the pair, slice of 32 dims) scores its slice; waves 0..7 = (head, 64 dims) accumulate the values, one dim per
+// lane.  The partial sums meet in the order of the undivided stage: 32-dim groups pairwise up to the halves of
+// the 256 dims, keys in sequence.  Only quarter 0 writes the new key and value rows to the cache.
+SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base) {
+  FLOW_IDS;
+  const DecodeP& P = F.d;
+  Lds& L = g_L;
+  const float NEG = -__int_as_float(0x7f800000);
+  const int N = pos + 1, nt = (N + SDPA_TILE - 1) / SDPA_TILE;
+  const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag32(base, li, FS_CORE);
+  if (wg >= nt * SL_ATT_KV * 4) return true;
+  const int tile = wg >> 3, kvh = (wg >> 2) & 1, hq = wg & 3;
+  const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
+  const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
+  const uint16_t* kbase = uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + j0) * 256;
+  const uint16_t* vbase = uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + j0) * 256;
+  __syncthreads();                    // the key tile aliases the activation vector the in-projection just read
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int row = it * 32 + (tid >> 5), c8 = (tid & 31) * 8;
+    if (row < nk && j0 + row != pos) {
+      st16(&L.kt[row * KT_STRIDE + c8], ld16(kbase + (size_t)row * 256 + c8));
+      st16(&g_vt[row * 256 + c8], ld16(vbase + (size_t)row * 256 + c8));
+    }
+  }
+  // waves 0,1: the unit's two query heads; wave 8: new key; wave 9: new value -- 4 tagged words per lane
+  const bool fetches = wave < 2 || wave == 8 || wave == 9;
+  const int src = wave < 2 ? (kvh * 8 + hq * 2 + wave) * 512 : (wave == 8 ? 8192 + kvh * 256 : 8192 + 512 + kvh * 256);
+  uint4 w4 = make_uint4(0, 0, 0, 0);
+  {
+    const rsrc_t rp = co_rsrc(uni(F.tproj));
+    unsigned spins = 0;
+    fstamp(P, 4, 0);
+    for (;;) {
+      bool ok = true;
+      if (fetches) { w4 = ldw4(rp, src + 4 * lane); ok = tag_ok(w4.x, tin) && tag_ok(w4.y, tin) && tag_ok(w4.z, tin) && tag_ok(w4.w, tin); }
+      const int v = flow_round(ok, spins, uni(P.bar) + 32);
+      if (v > 0) break;
+      if (v < 0) return false;
+    }
+    fstamp(P, 5, spins);
+  }
+  if (wave < 2 || wave == 8) {
+    const bool isq = wave < 2;
+    const uint16_t* nwp = isq ? uni(Y.q_norm) : uni(Y.k_norm);
+    const float xv[4] = {lo_h(w4.x), lo_h(w4.y), lo_h(w4.z), lo_h(w4.w)};
+    float wv[4];
+    const uint2 wraw = *reinterpret_cast<const uint2*>(nwp + 4 * lane);
+    wv[0] = lo_h(wraw.x); wv[1] = hi_h(wraw.x); wv[2] = lo_h(wraw.y); wv[3] = hi_h(wraw.y);
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ss = fmaf(xv[i], xv[i], ss);
+    ss = tree_sum<64>(ss);
+    const float inv = 1.0f / sqrtf(ss / 256.0f + EPS);
+    float* dst = isq ? &L.sq[wave * 256] : L.knew;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[4 * lane + i] = f16r(wv[i] * f16r(xv[i] * inv));
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = dst[4 * lane + i];
+    if (lane < 16) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = 4 * lane + i, ii = d & 31;
+        const float c = uni(P.rope_cos)[(size_t)pos * 32 + ii], sn = uni(P.rope_sin)[(size_t)pos * 32 + ii];
+        const float x0 = dst[ii], x1 = dst[ii + 32];
+        o[i] = (d < 32) ? f16r(fmaf(-x1, sn, x0 * c)) : f16r(fmaf(x1, c, x0 * sn));
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[4 * lane + i] = isq ? 0.0625f * o[i] : o[i];
+    if (!isq && has_new) {
+      if (hq == 0) st_co_h4(co_rsrc(uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 4 * lane, o);
+      *reinterpret_cast<uint2*>(&L.kt[(pos - j0) * KT_STRIDE + 4 * lane]) = make_uint2(pack2(o[0], o[1]), pack2(o[2], o[3]));
+    }
+  } else if (wave == 9 && has_new) {
+    const uint32_t a = (w4.x & 0xffffu) | (w4.y << 16), b = (w4.z & 0xffffu) | (w4.w << 16);
+    if (hq == 0) stw2(co_rsrc(uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 2 * lane, a, b);
+    *reinterpret_cast<uint2*>(&g_vt[(pos - j0) * 256 + 4 * lane]) = make_uint2(a, b);
+  }
+  __syncthreads();
+  {
+    // scores: wave (head, slice) takes the 8 leaves of its 32 dims, lane j is key j; the 32 query values sit one
+    // per lane (lanes 0..31) and reach the multiply as scalar operands
+    const int hh = wave >> 3, sl = wave & 7;
+    const uint16_t* kr = &L.kt[(lane < nk ? lane : 0) * KT_STRIDE + 32 * sl];
+    const float qv = L.sq[hh * 256 + 32 * sl + (lane & 31)];
+    float n[8];
+#pragma unroll
+    for (int l = 0; l < 8; ++l) {
+      const uint2 kraw = *reinterpret_cast<const uint2*>(kr + 4 * l);
+      const h2_t k01 = as_h2(kraw.x), k23 = as_h2(kraw.y);
+      float node = fmaf(row_lane_f(qv, 4 * l), (float)k01.x, 0.0f);
+      node = fmaf(row_lane_f(qv, 4 * l + 1), (float)k01.y, node);
+      node = fmaf(row_lane_f(qv, 4 * l + 2), (float)k23.x, node);
+      n[l] = fmaf(row_lane_f(qv, 4 * l + 3), (float)k23.y, node);
+    }
+    L.part[wave * 64 + lane] = ((n[0] + n[1]) + (n[2] + n[3])) + ((n[4] + n[5]) + (n[6] + n[7]));
+  }
+  __syncthreads();
+  if ((wave & 7) == 0) {
+    const int hh = wave >> 3;
+    const float* pp = &L.part[hh * 512 + lane];
+    const float lo = (pp[0] + pp[64]) + (pp[128] + pp[192]), hi = (pp[256] + pp[320]) + (pp[384] + pp[448]);
+    const float sc = (lane < nk) ? lo + hi : NEG;
+    const float mx = tree_max<64>(sc);
+    const float p = (lane < nk) ? exp_c(sc - mx) : 0.0f;
+    const float l = tree_sum<64>(p);
+    L.sm[hh * 64 + lane] = p;
+    const int head = kvh * 8 + hq * 2 + hh;
+    if (lane == 0) stw4(co_rsrc(uni(F.tml)), (head * uni(P.max_tiles) + tile) * 4, __float_as_uint(mx), __float_as_uint(l), tcore, tcore);
+  }
+  __syncthreads();
+  if (wave < 8) {
+    // values: wave (head, quarter of the dims), one dim per lane; the weight of key j is handed out by readlane
+    const int hh = wave >> 2, q4 = wave & 3;
+    float o = 0.0f;
+    const uint16_t* vt = &g_vt[64 * q4 + lane];
+    const float pmine = L.sm[hh * 64 + lane];
+    for (int j = 0; j < nk; ++j) o = fmaf(row_lane_f(pmine, j), h2f(vt[j * 256]), o);
+    // a 16-byte chunk carries two dims: the odd lane stores its neighbour's value and its own
+    const float oprev = prev_lane(o);
+    const int head = kvh * 8 + hq * 2 + hh;
+    if (lane & 1)
+      stw4(co_rsrc(uni(F.tpo)), ((head * uni(P.max_tiles) + tile) * 128 + 32 * q4 + (lane >> 1)) * 4, __float_as_uint(oprev),
+           __float_as_uint(o), tcore, tcore);
+  }
+  __syncthreads();
+  return true;
+}
+
 // History shift of a linear-attention layer: rows 1,2 of the old history and the new sample (each channel is
 // written by one workgroup).
 SL_DEV void store_hist(const LayerP& Y, int li, const GdnHist& gh) {
@@ -1053,7 +1186,7 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
       if (!flow_gdn(F, Y, li, base, gh)) return;
       if (!flow_out(F, Y, li, 0, base, gh)) return;
     } else {
-      if (!flow_sdpa(F, Y, li, pos, base)) return;
+      if (((pos + SDPA_TILE) / SDPA_TILE) * SL_ATT_KV * 4 <= (int)gridDim.x ? !flow_sdpa4(F, Y, li, pos, base) : !flow_sdpa(F, Y, li, pos, base)) return;
       if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh)) return;
     }
     if (!flow_moe_a(F, Y, li, base, h0, h1)) return;
