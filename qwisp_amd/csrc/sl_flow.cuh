@@ -507,6 +507,19 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
   const bool fetches = wave < 2 || wave == 8 || wave == 9;
   const int src = wave < 2 ? (kvh * 8 + hq * 2 + wave) * 512 : (wave == 8 ? 8192 + kvh * 256 : 8192 + 512 + kvh * 256);
   uint4 w4 = make_uint4(0, 0, 0, 0);
+  // norm weights and the rope row of this position do not depend on the projection: fetched ahead of the poll
+  uint2 wraw = make_uint2(0, 0);
+  float rc[4] = {1.0f, 1.0f, 1.0f, 1.0f}, rsn[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (wave < 2 || wave == 8) {
+    wraw = *reinterpret_cast<const uint2*>((wave < 2 ? uni(Y.q_norm) : uni(Y.k_norm)) + 4 * lane);
+    if (lane < 16) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ii = (4 * lane + i) & 31;
+        rc[i] = uni(P.rope_cos)[(size_t)pos * 32 + ii]; rsn[i] = uni(P.rope_sin)[(size_t)pos * 32 + ii];
+      }
+    }
+  }
   {
     const rsrc_t rp = co_rsrc(uni(F.tproj));
     unsigned spins = 0;
@@ -522,10 +535,8 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
   }
   if (wave < 2 || wave == 8) {
     const bool isq = wave < 2;
-    const uint16_t* nwp = isq ? uni(Y.q_norm) : uni(Y.k_norm);
     const float xv[4] = {lo_h(w4.x), lo_h(w4.y), lo_h(w4.z), lo_h(w4.w)};
     float wv[4];
-    const uint2 wraw = *reinterpret_cast<const uint2*>(nwp + 4 * lane);
     wv[0] = lo_h(wraw.x); wv[1] = hi_h(wraw.x); wv[2] = lo_h(wraw.y); wv[3] = hi_h(wraw.y);
     float ss = 0.0f;
 #pragma unroll
@@ -542,7 +553,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int d = 4 * lane + i, ii = d & 31;
-        const float c = uni(P.rope_cos)[(size_t)pos * 32 + ii], sn = uni(P.rope_sin)[(size_t)pos * 32 + ii];
+        const float c = rc[i], sn = rsn[i];
         const float x0 = dst[ii], x1 = dst[ii + 32];
         o[i] = (d < 32) ? f16r(fmaf(-x1, sn, x0 * c)) : f16r(fmaf(x1, c, x0 * sn));
       }
