@@ -95,6 +95,17 @@ constexpr int DPP_HALF_MIRROR = 0x141;  // lane i <-> 7-i within 8
 constexpr int DPP_MIRROR = 0x140;       // lane i <-> 15-i within 16
 constexpr int DPP_SHR1 = 0x111;         // lane i takes lane i-1 within its 16-lane row
 SL_DEV float row_lane_f(float v, int lane) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane)); }
+// Values of lanes base..base+7 as scalars.  The empty asm keeps all eight in scalar registers at one point, so the
+// extractions are issued back to back ahead of their uses: a scalar written by the vector unit takes tens of cycles
+// to become readable, and extraction and use strictly alternating on one register pay that for every element.
+SL_DEV void lanes8(float v, int base, float (&out)[8]) {
+  int t[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) t[i] = __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), base + i);
+  asm volatile("" : "+s"(t[0]), "+s"(t[1]), "+s"(t[2]), "+s"(t[3]), "+s"(t[4]), "+s"(t[5]), "+s"(t[6]), "+s"(t[7]));
+#pragma unroll
+  for (int i = 0; i < 8; ++i) out[i] = __builtin_bit_cast(float, t[i]);
+}
 
 template <int WIDTH>
 SL_DEV float tree_sum(float v) {

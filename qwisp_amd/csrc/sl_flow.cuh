@@ -461,7 +461,20 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       float o0 = 0.0f, o1 = 0.0f;
       const uint16_t* vt = &g_vt[128 * half + 2 * lane];
       const float pmine = L.sm[h * 64 + lane];            // weight of key `lane`; handed out by readlane below
-      for (int j = 0; j < nk; ++j) {
+      int j = 0;
+      for (; j + 8 <= nk; j += 8) {            // the eight LDS reads are issued together, then used in key order
+        uint32_t v8[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v8[i] = *reinterpret_cast<const uint32_t*>(vt + (j + i) * 256);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float pj = row_lane_f(pmine, j + i);
+          const h2_t v01 = as_h2(v8[i]);
+          o0 = fmaf(pj, (float)v01.x, o0);
+          o1 = fmaf(pj, (float)v01.y, o1);
+        }
+      }
+      for (; j < nk; ++j) {
         const uint32_t vv = *reinterpret_cast<const uint32_t*>(vt + j * 256);
         const float pj = row_lane_f(pmine, j);
         const h2_t v01 = as_h2(vv);
@@ -478,7 +491,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
 
 // The same stage at contexts of up to G/8 key tiles: a unit is (tile, kv head, quarter of the group's 8 query
 // heads), so four times as many workgroups share the work and a unit's arithmetic is a quarter.  Wave (head of
-// the pair, slice of 32 dims) scores its slice; waves 0..7 = (head, 64 dims) accumulate the values, one dim per
+// the pair, slice of 32 dims) scores its slice; waves 0..3 = (head, half of the dims) accumulate the values, two dims per
 // lane.  The partial sums meet in the order of the undivided stage: 32-dim groups pairwise up to the halves of
 // the 256 dims, keys in sequence.  Only quarter 0 writes the new key and value rows to the cache.
 SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base) {
@@ -602,19 +615,36 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
     if (lane == 0) stw4(co_rsrc(uni(F.tml)), (head * uni(P.max_tiles) + tile) * 4, __float_as_uint(mx), __float_as_uint(l), tcore, tcore);
   }
   __syncthreads();
-  if (wave < 8) {
-    // values: wave (head, quarter of the dims), one dim per lane; the weight of key j is handed out by readlane
-    const int hh = wave >> 2, q4 = wave & 3;
-    float o = 0.0f;
-    const uint16_t* vt = &g_vt[64 * q4 + lane];
+  if (wave < 4) {
+    // values: wave (head, half of the dims), two dims per lane (one LDS word per key); the weight of key j is
+    // handed out by readlane.  Eight LDS reads are issued together, then used in key order.
+    const int hh = wave >> 1, half = wave & 1;
+    float o0 = 0.0f, o1 = 0.0f;
+    const uint16_t* vt = &g_vt[128 * half + 2 * lane];
     const float pmine = L.sm[hh * 64 + lane];
-    for (int j = 0; j < nk; ++j) o = fmaf(row_lane_f(pmine, j), h2f(vt[j * 256]), o);
-    // a 16-byte chunk carries two dims: the odd lane stores its neighbour's value and its own
-    const float oprev = prev_lane(o);
+    int j = 0;
+    for (; j + 8 <= nk; j += 8) {              // eight LDS reads and eight weights at a time, used in key order
+      uint32_t v8[8];
+      float p8[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v8[i] = *reinterpret_cast<const uint32_t*>(vt + (j + i) * 256);
+      lanes8(pmine, j, p8);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const h2_t v01 = as_h2(v8[i]);
+        o0 = fmaf(p8[i], (float)v01.x, o0);
+        o1 = fmaf(p8[i], (float)v01.y, o1);
+      }
+    }
+    for (; j < nk; ++j) {
+      const h2_t v01 = as_h2(*reinterpret_cast<const uint32_t*>(vt + j * 256));
+      const float pj = row_lane_f(pmine, j);
+      o0 = fmaf(pj, (float)v01.x, o0);
+      o1 = fmaf(pj, (float)v01.y, o1);
+    }
     const int head = kvh * 8 + hq * 2 + hh;
-    if (lane & 1)
-      stw4(co_rsrc(uni(F.tpo)), ((head * uni(P.max_tiles) + tile) * 128 + 32 * q4 + (lane >> 1)) * 4, __float_as_uint(oprev),
-           __float_as_uint(o), tcore, tcore);
+    stw4(co_rsrc(uni(F.tpo)), ((head * uni(P.max_tiles) + tile) * 128 + 64 * half + lane) * 4, __float_as_uint(o0), __float_as_uint(o1),
+         tcore, tcore);
   }
   __syncthreads();
   return true;
