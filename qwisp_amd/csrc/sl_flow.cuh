@@ -988,15 +988,8 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     if (lane == 0) L.gb[0] = Z;
   }
   __syncthreads();
-  if (tid == 0) {
-    float sc[8], ss = 0.0f;
-    const float Z = L.gb[0];
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) { sc[kk] = f16r(ex[L.inds[kk]] / Z); ss = f16r(ss + sc[kk]); }
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) L.scores[kk] = f16r(sc[kk] / ss);
-    if (wg == 0) for (int kk = 0; kk < 8; ++kk) { uni(Y.route_inds)[kk] = L.inds[kk]; uni(Y.route_scores)[kk] = f2h(L.scores[kk]); }
-  }
+  // (the renormalised scores are only needed by the combine of the next stage and are formed there, off this
+  // stage's path: exp values, sum and indices stay in LDS)
   // this wave's gate/up pair, requested as soon as the indices are known
   const int p = gw;
   WRegs<1, 2> wr;
@@ -1043,6 +1036,18 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
       wv[qq] = ld16(W + row * 64 + 4 * li16);
       sbv[qq] = SB[row * 8 + (li16 >> 1)];
     }
+  }
+  if (tid == PUB_WAVE * 64) {
+    // scores of the routing done in the stage before: gates = half(exp / Z) of the selected, renormalised in half
+    // (the publisher wave neither polls nor owns a unit, so this costs the stage nothing)
+    const float* ex = L.part + 256;
+    float sc[8], ss = 0.0f;
+    const float Z = L.gb[0];
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) { sc[kk] = f16r(ex[L.inds[kk]] / Z); ss = f16r(ss + sc[kk]); }
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) L.scores[kk] = f16r(sc[kk] / ss);
+    if (wg == 0) for (int kk = 0; kk < 8; ++kk) { uni(Y.route_inds)[kk] = L.inds[kk]; uni(Y.route_scores)[kk] = f2h(L.scores[kk]); }
   }
   {
     // the nine activation rows (8 x 512 routed + 512 shared) are 1152 chunks of 4 tagged words: 3 per thread
