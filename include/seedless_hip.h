@@ -93,6 +93,11 @@ typedef struct {
 typedef struct {
   const uint16_t* router_w;      /* [E, 2048] fp16 gate */
   const uint16_t* shared_gate_w; /* [2048] fp16 shared_expert_gate row */
+  /* The two gates as the released checkpoint stores them: MLX affine 8-bit, group 64, 4 values per little-endian
+   * word (mlp.gate and mlp.shared_expert_gate, SeedlessEngine.swift:93-106; kernel qmm8, SeedlessMetalForward.swift:384).
+   * Used when router_w / shared_gate_w are NULL: w [n, 512], scales and biases [n, 32]; n = E and n = 1. */
+  sl_q4 router_q8;
+  sl_q4 shared_gate_q8;
   sl_q4 sw_gate;                 /* [E*512, 2048]  switch_mlp.gate_proj, expert-major */
   sl_q4 sw_up;                   /* [E*512, 2048]  */
   sl_q4 sw_down;                 /* [E*2048, 512]  */

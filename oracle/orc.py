@@ -54,6 +54,7 @@ def _load():
         "orc_qmv": (None, [vp, vp, vp, vp, i32, i32, vp]),
         "orc_qmv_f32": (None, [vp, vp, vp, vp, i32, i32, vp]),
         "orc_dense_f16": (None, [vp, vp, i32, i32, vp]),
+        "orc_q8_f32": (None, [vp, vp, vp, vp, i32, i32, vp]),
         "orc_rmsnorm": (None, [vp, vp, i32, vp]),
         "orc_route": (None, [vp, i32, vp, vp]),
         "orc_swiglu": (None, [vp, vp, i32, vp]),
@@ -111,6 +112,11 @@ def generate_host(cfg):
             t[name] = synth_f16(shape, seed, mean, sigma)
         else:
             t[name] = synth_f32(shape, seed, mean, sigma)
+    if getattr(cfg, "gate_bits", 16) == 8:      # the two gates re-expressed in 8 bits, as generate_device does
+        from qwisp_amd.synth import quantize_q8
+        for i in range(cfg.n_layers):
+            for nm in (f"layers.{i}.mlp.gate", f"layers.{i}.mlp.shared_expert_gate"):
+                t[nm + ".weight"], t[nm + ".scales"], t[nm + ".biases"] = quantize_q8(t[nm + ".weight"].reshape(-1, 2048))
     return t
 
 

@@ -108,6 +108,28 @@ static float dense_dot(const float* x, const uint16_t* wrow, int K) {
   return tree_sum(p, 64);
 }
 
+// 8-bit affine row dot, group 64 (router gate and shared-expert gate of the released checkpoint; reference
+// kernel qmm8, SeedlessMetalForward.swift:372-428: per 8 values `scale * sum(x*q) + bias * sum(x)`, the sum of x
+// formed sequentially in fp32).  Lane l of 64 owns the 32 contiguous values 32l..32l+31, i.e. half a group and
+// four terms of 8; a term is fmaf(s, chain of fmaf(x, q), b * sx), the lane's partial (t0+t1)+(t2+t3).
+static float q8_dot(const float* x, const uint32_t* wrow, const uint16_t* srow, const uint16_t* brow, int K) {
+  const uint8_t* q = reinterpret_cast<const uint8_t*>(wrow);   // little-endian: value j of a word in bits 8j..8j+7
+  float p[64];
+  for (int l = 0; l < 64; ++l) {
+    const float s = h2f(srow[(32 * l) / 64]), b = h2f(brow[(32 * l) / 64]);
+    float t[4];
+    for (int j = 0; j < 4; ++j) {
+      const int e0 = 32 * l + 8 * j;
+      float dq = 0.0f, sx = 0.0f;
+      for (int i = 0; i < 8; ++i) { dq = std::fmaf(x[e0 + i], (float)q[e0 + i], dq); sx = sx + x[e0 + i]; }
+      t[j] = std::fmaf(s, dq, b * sx);
+    }
+    p[l] = (t[0] + t[1]) + (t[2] + t[3]);
+  }
+  (void)K;
+  return tree_sum(p, 64);
+}
+
 // Sum of squares over D (a multiple of 64) values.
 static float sumsq(const float* x, int D) {
   const int per = D / 64;
@@ -201,7 +223,10 @@ static void moe_block_rows(Engine& e, int li, const float* x, int M, float* out)
   std::vector<float> gl(E), g(I), u(I), act(I), d((size_t)TOPK * H), sg(I), su(I), sact(I), sy(H);
   for (int m = 0; m < M; ++m) {
     const float* xm = x + (size_t)m * H;
-    for (int i = 0; i < E; ++i) gl[i] = f16r(dense_dot(xm, w.router_w + (size_t)i * H, H));
+    for (int i = 0; i < E; ++i)
+      gl[i] = w.router_w ? f16r(dense_dot(xm, w.router_w + (size_t)i * H, H))
+                         : f16r(q8_dot(xm, w.router_q8.w + (size_t)i * (H / 4), w.router_q8.scales + (size_t)i * (H / 64),
+                                       w.router_q8.biases + (size_t)i * (H / 64), H));
     int32_t* inds = &e.routeInds[((size_t)li * e.maxM + m) * TOPK];
     float* sc = &e.routeScores[((size_t)li * e.maxM + m) * TOPK];
     route(gl.data(), E, inds, sc);
@@ -215,7 +240,8 @@ static void moe_block_rows(Engine& e, int li, const float* x, int M, float* out)
     qmv(xm, w.sh_up, 0, I, su.data());
     for (int i = 0; i < I; ++i) sact[i] = swiglu16(sg[i], su[i]);
     qmv(sact.data(), w.sh_down, 0, H, sy.data());
-    const float t = f16r(dense_dot(xm, w.shared_gate_w, H));
+    const float t = w.shared_gate_w ? f16r(dense_dot(xm, w.shared_gate_w, H))
+                                    : f16r(q8_dot(xm, w.shared_gate_q8.w, w.shared_gate_q8.scales, w.shared_gate_q8.biases, H));
     const float s = sigmoid16(t);
     for (int n = 0; n < H; ++n) {
       float acc = 0.0f;
@@ -681,6 +707,12 @@ void orc_dense_f16(const uint16_t* x, const uint16_t* w, int n, int k, uint16_t*
   std::vector<float> xf(k);
   for (int i = 0; i < k; ++i) xf[i] = h2f(x[i]);
   for (int r = 0; r < n; ++r) y[r] = f2h(dense_dot(xf.data(), w + (size_t)r * k, k));
+}
+// 8-bit rows (K = 2048): y = q8_dot before the half rounding, for checks against float64.
+void orc_q8_f32(const uint16_t* x, const uint32_t* w, const uint16_t* s, const uint16_t* b, int n, int k, float* y) {
+  std::vector<float> xf(k);
+  for (int i = 0; i < k; ++i) xf[i] = h2f(x[i]);
+  for (int r = 0; r < n; ++r) y[r] = q8_dot(xf.data(), w + (size_t)r * (k / 4), s + (size_t)r * (k / 64), b + (size_t)r * (k / 64), k);
 }
 void orc_rmsnorm(const uint16_t* x, const uint16_t* w, int D, uint16_t* y) {
   std::vector<float> xf(D), yf(D);

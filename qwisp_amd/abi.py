@@ -35,7 +35,7 @@ class AttnW(C.Structure):
 
 
 class MoeW(C.Structure):
-    _fields_ = [("router_w", C.c_void_p), ("shared_gate_w", C.c_void_p),
+    _fields_ = [("router_w", C.c_void_p), ("shared_gate_w", C.c_void_p), ("router_q8", Q4), ("shared_gate_q8", Q4),
                 ("sw_gate", Q4), ("sw_up", Q4), ("sw_down", Q4),
                 ("sh_gate", Q4), ("sh_up", Q4), ("sh_down", Q4)]
 
@@ -134,7 +134,11 @@ def build_desc(cfg, tensors, location):
                            _q4(tensors, sa + "o_proj", H, ATT_HEADS * ATT_D),
                            _ptr(tensors[sa + "q_norm.weight"]), _ptr(tensors[sa + "k_norm.weight"]))
         mp = p + "mlp."
-        L.moe = MoeW(_ptr(tensors[mp + "gate.weight"]), _ptr(tensors[mp + "shared_expert_gate.weight"]),
+        if mp + "gate.scales" in tensors:      # 8-bit gates, as the released checkpoint stores them
+            gates = (None, None, _q4(tensors, mp + "gate", E, H), _q4(tensors, mp + "shared_expert_gate", 1, H))
+        else:                                  # fp16 gates (the benchmark configuration)
+            gates = (_ptr(tensors[mp + "gate.weight"]), _ptr(tensors[mp + "shared_expert_gate.weight"]), Q4(), Q4())
+        L.moe = MoeW(*gates,
                      _q4(tensors, mp + "switch_mlp.gate_proj", E * MOE_I, H),
                      _q4(tensors, mp + "switch_mlp.up_proj", E * MOE_I, H),
                      _q4(tensors, mp + "switch_mlp.down_proj", E * H, MOE_I),

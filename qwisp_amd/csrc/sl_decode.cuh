@@ -28,7 +28,7 @@ struct LayerP {
   float* state[2];
   const uint16_t *q_norm, *k_norm;
   uint16_t *kcache, *vcache;
-  const uint16_t *router_w, *sgate_w;
+  const uint16_t *router_w, *sgate_w;    // with 8-bit gates: words [E+1, 512] (row E = shared gate) and {scale, bias} [E+1, 32]
   const uint32_t *swg_w, *swg_sb, *swu_w, *swu_sb, *swd_w, *swd_sb;
   const uint32_t *shg_w, *shg_sb, *shu_w, *shu_sb, *shd_w, *shd_sb;
   int32_t* route_inds;

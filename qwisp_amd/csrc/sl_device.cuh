@@ -175,6 +175,26 @@ SL_DEV float word_dot(uint32_t w, const uint32_t* xp /*4 packed pairs*/) {
   return dq;
 }
 // Four consecutive words of one group-half: t_j = fmaf(s, dq_j, b*sx_j); returns (t0+t1)+(t2+t3).
+// 8-bit affine row dot, group 64 (the router gate and shared-expert gate of the released checkpoint; reference
+// kernel qmm8, SeedlessMetalForward.swift:372-428).  Lane l owns the 32 contiguous values 32l..32l+31 = 8 words,
+// half a group.  Per 8 values: t = fmaf(s, chain of fmaf(x, q), b * sx) with sx the sequential fp32 sum of the
+// eight x; the lane's partial is (t0+t1)+(t2+t3).
+SL_DEV float q8_lane(const uint32_t* w8 /*8 words*/, uint32_t sb, const float* x /*32*/) {
+  const float s = lo_h(sb), b = hi_h(sb);
+  float t[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float dq = 0.0f, sx = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float q = (float)((w8[2 * j + (i >> 2)] >> (8 * (i & 3))) & 255u);
+      dq = fmaf(x[8 * j + i], q, dq);
+      sx = sx + x[8 * j + i];
+    }
+    t[j] = fmaf(s, dq, b * sx);
+  }
+  return (t[0] + t[1]) + (t[2] + t[3]);
+}
 SL_DEV float quad_term(uint4 w, uint32_t sb, const uint32_t* xp /*16 packed pairs*/, const float* sx /*4*/) {
   const float s = lo_h(sb) * 16777216.0f, b = hi_h(sb);
   float t0 = fmaf(s, word_dot(w.x, xp), b * sx[0]);

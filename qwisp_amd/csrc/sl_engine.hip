@@ -38,6 +38,7 @@ struct LayerDev {
   uint16_t *q_norm = nullptr, *k_norm = nullptr, *kcache = nullptr, *vcache = nullptr;
   // MoE
   uint16_t *router_w = nullptr, *sgate_w = nullptr;
+  uint32_t *gate8_w = nullptr, *gate8_sb = nullptr;   // 8-bit gates instead: [E+1, 512] words and [E+1, 32] {scale, bias}; row E = shared gate
   DevQ4 sw_gate, sw_up, sw_down, sh_gate, sh_up, sh_down;
   int32_t* route_inds = nullptr;
   uint16_t* route_scores = nullptr;
@@ -58,6 +59,7 @@ struct sl_full_snap {
 struct sl_engine {
   int n_layers = 0, n_experts = 0, vocab = 0, max_m = 0, max_seq = 0, max_tiles = 0;
   bool has_attn = false, has_head = false;
+  bool gate8 = false;              // router / shared gate are 8-bit rows (all layers alike)
   hipStream_t stream = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   std::vector<void*> allocs;
@@ -153,6 +155,19 @@ bool fill_q4(sl_engine* e, DevQ4& dst, int row_off, const sl_q4& src, int n, int
   hipLaunchKernelGGL(k_pack_sb, dim3((unsigned)((gcount + 255) / 256)), dim3(256), 0, e->stream, src.scales, src.biases, out, gcount);
   return ok(e, hipGetLastError(), "k_pack_sb");
 }
+// Rows of an 8-bit matrix (k = 2048: 512 words and 32 groups per row) into rows [row_off, row_off + src.n).
+bool fill_q8(sl_engine* e, uint32_t* dw, uint32_t* dsb, int row_off, const sl_q4& src, int loc) {
+  const size_t wcount = (size_t)src.n * (H / 4), gcount = (size_t)src.n * (H / 64);
+  if (!copy_in(e, dw + (size_t)row_off * (H / 4), src.w, wcount * 4, loc)) return false;
+  uint32_t* out = dsb + (size_t)row_off * (H / 64);
+  if (loc == SL_LOC_HOST) {
+    std::vector<uint32_t> tmp(gcount);
+    for (size_t i = 0; i < gcount; ++i) tmp[i] = (uint32_t)src.scales[i] | ((uint32_t)src.biases[i] << 16);
+    return copy_in(e, out, tmp.data(), gcount * 4, SL_LOC_HOST);
+  }
+  hipLaunchKernelGGL(k_pack_sb, dim3((unsigned)((gcount + 255) / 256)), dim3(256), 0, e->stream, src.scales, src.biases, out, gcount);
+  return ok(e, hipGetLastError(), "k_pack_sb");
+}
 bool upload_q4(sl_engine* e, DevQ4& d, const sl_q4& src, int n, int k, int loc) {
   return alloc_q4(e, d, n, k) && fill_q4(e, d, 0, src, n, k, loc);
 }
@@ -210,7 +225,7 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   MoeAArgs a{};
   a.ha = ha;
   a.shg_w = L.sh_gate.w; a.shg_sb = L.sh_gate.sb; a.shu_w = L.sh_up.w; a.shu_sb = L.sh_up.sb;
-  a.router_w = L.router_w; a.sgate_w = L.sgate_w; a.E = e->n_experts;
+  a.router_w = L.router_w; a.sgate_w = L.sgate_w; a.g8_w = L.gate8_w; a.g8_sb = L.gate8_sb; a.E = e->n_experts;
   a.sh_act = e->sh_act; a.rlogits = e->rlogits; a.sgate = e->sgate;
   const int router_blocks = (e->n_experts + 1 + 15) / 16;
   hipLaunchKernelGGL(k_moe_a, dim3(MOE_A_SHARED_BLOCKS + router_blocks, M), dim3(256), 0, e->stream, a);
@@ -288,7 +303,8 @@ void launch_decode(sl_engine* e, int out_off, bool feed) {
   const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
   hipLaunchKernelGGL(k_embed, dim3(H / 256, 1), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
-  hipLaunchKernelGGL(k_decode_flow, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0);
+  if (e->gate8) hipLaunchKernelGGL(k_decode_flow<true>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0);
+  else hipLaunchKernelGGL(k_decode_flow<false>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0);
   if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
   e->pos += 1;
   for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
@@ -398,9 +414,24 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
       if (!L.q_norm || !L.k_norm) return SL_ERR_DEVICE;
     }
     const sl_moe_w& w = s.moe;
-    L.router_w = upload<uint16_t>(e, w.router_w, (size_t)E * H, loc);
-    L.sgate_w = upload<uint16_t>(e, w.shared_gate_w, H, loc);
-    if (!L.router_w || !L.sgate_w) return SL_ERR_DEVICE;
+    if (w.router_w || w.shared_gate_w) {
+      L.router_w = upload<uint16_t>(e, w.router_w, (size_t)E * H, loc);
+      L.sgate_w = upload<uint16_t>(e, w.shared_gate_w, H, loc);
+      if (!L.router_w || !L.sgate_w) return SL_ERR_DEVICE;
+    } else {
+      // 8-bit gates: router rows and the shared-gate row in one matrix of E + 1 rows
+      if (!shape_ok(w.router_q8, E, H) || !shape_ok(w.shared_gate_q8, 1, H)) {
+        e->fault = "router / shared gate: neither fp16 rows nor 8-bit tensors of the right shape";
+        return SL_ERR_ARG;
+      }
+      L.gate8_w = dalloc<uint32_t>(e, (size_t)(E + 1) * (H / 4));
+      L.gate8_sb = dalloc<uint32_t>(e, (size_t)(E + 1) * (H / 64));
+      if (!L.gate8_w || !L.gate8_sb) return SL_ERR_DEVICE;
+      if (!fill_q8(e, L.gate8_w, L.gate8_sb, 0, w.router_q8, loc) || !fill_q8(e, L.gate8_w, L.gate8_sb, E, w.shared_gate_q8, loc))
+        return SL_ERR_DEVICE;
+    }
+    if (i == 0) e->gate8 = L.gate8_w != nullptr;
+    else if (e->gate8 != (L.gate8_w != nullptr)) { e->fault = "fp16 and 8-bit gates mixed across layers"; return SL_ERR_ARG; }
     if (!upload_q4(e, L.sw_gate, w.sw_gate, E * SL_MOE_I, H, loc) || !upload_q4(e, L.sw_up, w.sw_up, E * SL_MOE_I, H, loc) ||
         !upload_q4(e, L.sw_down, w.sw_down, E * H, SL_MOE_I, loc) || !upload_q4(e, L.sh_gate, w.sh_gate, SL_MOE_I, H, loc) ||
         !upload_q4(e, L.sh_up, w.sh_up, SL_MOE_I, H, loc) || !upload_q4(e, L.sh_down, w.sh_down, H, SL_MOE_I, loc))
@@ -475,6 +506,7 @@ int alloc_runtime(sl_engine* e) {
           q.q_norm = L.q_norm; q.k_norm = L.k_norm; q.kcache = L.kcache; q.vcache = L.vcache;
         }
         q.router_w = L.router_w; q.sgate_w = L.sgate_w;
+        if (L.gate8_w) { q.router_w = reinterpret_cast<const uint16_t*>(L.gate8_w); q.sgate_w = reinterpret_cast<const uint16_t*>(L.gate8_sb); }
         q.swg_w = L.sw_gate.w; q.swg_sb = L.sw_gate.sb; q.swu_w = L.sw_up.w; q.swu_sb = L.sw_up.sb;
         q.swd_w = L.sw_down.w; q.swd_sb = L.sw_down.sb; q.shg_w = L.sh_gate.w; q.shg_sb = L.sh_gate.sb;
         q.shu_w = L.sh_up.w; q.shu_sb = L.sh_up.sb; q.shd_w = L.sh_down.w; q.shd_sb = L.sh_down.sb;
@@ -506,7 +538,8 @@ int alloc_runtime(sl_engine* e) {
         e->flow_host = F;
         e->flow_params = upload<FlowP>(e, &F, 1, SL_LOC_HOST);
         if (!e->flow_params) return SL_ERR_DEVICE;
-        SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
+        SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<false>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
+        SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<true>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
       }
       e->dec_grid = 256;
     }
@@ -538,7 +571,7 @@ int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine*
     L.kcache = L.vcache = nullptr; L.route_inds = nullptr; L.route_scores = nullptr;
     const int r = alloc_layer_state(e, L); if (r) return r;
   }
-  e->embed = base->embed; e->lm_head = base->lm_head; e->final_norm = base->final_norm;
+  e->embed = base->embed; e->lm_head = base->lm_head; e->final_norm = base->final_norm; e->gate8 = base->gate8;
   return alloc_runtime(e);
 }
 
@@ -551,7 +584,7 @@ bool lanes_batchable(sl_engine** lanes, int b) {
   for (int i = 0; i < b; ++i) {
     const sl_engine* l = lanes[i];
     if (l->n_layers != d->n_layers || l->max_seq != d->max_seq || l->lm_head.w != d->lm_head.w ||
-        l->layers[0].router_w != d->layers[0].router_w) return false;
+        l->layers[0].router_w != d->layers[0].router_w || l->layers[0].gate8_w != d->layers[0].gate8_w) return false;
   }
   return true;
 }

@@ -867,6 +867,9 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
 }
 
 // ---- MoE stage A -------------------------------------------------------------------------------------
+// GATE8: the router and shared-gate rows are 8-bit affine rows instead of fp16 (a compile-time variant, so that
+// the fp16 configuration carries none of its registers or branches).
+template <bool GATE8>
 SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, float& h0, float& h1) {
   FLOW_IDS;
   const DecodeP& P = F.d;
@@ -881,10 +884,16 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
   const size_t prow = is_pair ? (size_t)gp : 0;
   wload_row<1>(wr.w[0], wr.sb[0], uni(Y.shg_w), uni(Y.shg_sb), prow, is_pair, lane);
   wload_row<1>(wr.w[1], wr.sb[1], uni(Y.shu_w), uni(Y.shu_sb), prow, is_pair, lane);
-  if (is_dense) {
+  constexpr bool gate8 = GATE8;
+  uint32_t dsb = 0;                       // 8-bit gates: {scale, bias} of this lane's half group
+  if (is_dense && !gate8) {
     const uint16_t* drow = (gd < uni(P.E) ? uni(Y.router_w) + (size_t)gd * H : uni(Y.sgate_w)) + 32 * lane;
 #pragma unroll
     for (int j = 0; j < 4; ++j) dwr[j] = ld16(drow + 8 * j);
+  } else if (is_dense) {
+    const uint32_t* drow = reinterpret_cast<const uint32_t*>(uni(Y.router_w)) + (size_t)gd * 512 + 8 * lane;
+    dwr[0] = ld16(drow); dwr[1] = ld16(drow + 4);
+    dsb = reinterpret_cast<const uint32_t*>(uni(Y.sgate_w))[(size_t)gd * 32 + (lane >> 1)];
   }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.post_ln) + 2 * tid);
   float r0, r1;
@@ -897,8 +906,15 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
     const uint32_t dww[16] = {dwr[0].x, dwr[0].y, dwr[0].z, dwr[0].w, dwr[1].x, dwr[1].y, dwr[1].z, dwr[1].w,
                               dwr[2].x, dwr[2].y, dwr[2].z, dwr[2].w, dwr[3].x, dwr[3].y, dwr[3].z, dwr[3].w};
     float acc = 0.0f;
+    if (!gate8) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { acc = fmaf(lo_h(xp[i]), lo_h(dww[i]), acc); acc = fmaf(hi_h(xp[i]), hi_h(dww[i]), acc); }
+      for (int i = 0; i < 16; ++i) { acc = fmaf(lo_h(xp[i]), lo_h(dww[i]), acc); acc = fmaf(hi_h(xp[i]), hi_h(dww[i]), acc); }
+    } else {
+      float xf[32];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { xf[2 * i] = lo_h(xp[i]); xf[2 * i + 1] = hi_h(xp[i]); }
+      acc = q8_lane(dww, dsb, xf);
+    }
     acc = tree_sum<64>(acc);
     if (lane == 0) g_L.pub[wave] = tagged(acc, ta);
   }
@@ -1199,6 +1215,7 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
 }
 
 // ---- the kernel: hA already holds the embedded token row (k_embed) --------------------------------------
+template <bool GATE8>
 __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __restrict__ Fp, int out_off, int feed) {
   {
     const int tid = threadIdx.x;
@@ -1235,7 +1252,7 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
       if (((pos + SDPA_TILE) / SDPA_TILE) * SL_ATT_KV * 4 <= (int)gridDim.x ? !flow_sdpa4(F, Y, li, pos, base) : !flow_sdpa(F, Y, li, pos, base)) return;
       if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh)) return;
     }
-    if (!flow_moe_a(F, Y, li, base, h0, h1)) return;
+    if (!flow_moe_a<GATE8>(F, Y, li, base, h0, h1)) return;
     if (!flow_moe_b(F, Y, li, base)) return;
     if (!flow_moe_c(F, Y, li, base)) return;
   }

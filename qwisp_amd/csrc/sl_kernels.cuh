@@ -361,6 +361,7 @@ struct MoeAArgs {
   const uint32_t *shg_w, *shg_sb, *shu_w, *shu_sb;   // shared gate_proj / up_proj [512, 2048]
   const uint16_t* router_w;                          // [E, 2048]
   const uint16_t* sgate_w;                           // [2048]
+  const uint32_t *g8_w, *g8_sb;                      // 8-bit gates instead (null: fp16): [E+1, 512] words, [E+1, 32] {scale, bias}; row E = shared gate
   int E;
   uint16_t* sh_act;                                  // [M, 512]
   uint16_t* rlogits;                                 // [M, 256]
@@ -388,13 +389,16 @@ __global__ __launch_bounds__(256) void k_moe_a(MoeAArgs a) {
     const int row0 = ((blockIdx.x - MOE_A_SHARED_BLOCKS) * 4 + wave) * 4;
     for (int r = 0; r < 4; ++r) {
       const int row = row0 + r;
-      if (row < a.E) {
-        const float v = dense_dot(a.router_w + (size_t)row * H, lane, x);
-        if (lane == 0) a.rlogits[(size_t)m * 256 + row] = f2h(v);
-      } else if (row == a.E) {
-        const float v = dense_dot(a.sgate_w, lane, x);
-        if (lane == 0) a.sgate[m] = f2h(v);
+      if (row > a.E) continue;
+      float v;
+      if (a.g8_w) {
+        const uint4 w0 = ld16(a.g8_w + (size_t)row * 512 + 8 * lane), w1 = ld16(a.g8_w + (size_t)row * 512 + 8 * lane + 4);
+        const uint32_t w8[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+        v = tree_sum<64>(q8_lane(w8, a.g8_sb[(size_t)row * 32 + (lane >> 1)], x));
+      } else {
+        v = dense_dot(row < a.E ? a.router_w + (size_t)row * H : a.sgate_w, lane, x);
       }
+      if (lane == 0) { if (row < a.E) a.rlogits[(size_t)m * 256 + row] = f2h(v); else a.sgate[m] = f2h(v); }
     }
   }
 }

@@ -19,6 +19,7 @@ class ModelConfig:
     full_attn_interval: int = 4       # layer i is full attention iff (i+1) % interval == 0
     seed_base: int = 2000
     layer_types: tuple = None         # optional explicit override, e.g. ("gdn",) or ("attn",)
+    gate_bits: int = 16               # 16: fp16 router / shared gate (benchmark configuration); 8: MLX affine 8-bit
 
     def is_linear(self, i):
         if self.layer_types is not None:
@@ -87,6 +88,29 @@ def weight_bytes(cfg):
     return total
 
 
+def quantize_q8(w):
+    """MLX affine quantisation, 8 bits, group 64, of an fp16/fp32 matrix [n, k] (numpy).  Returns packed words
+    uint32 [n, k/4] (value j of a word in bits 8j..8j+7), scales and biases fp16 [n, k/64].  Same rule as the
+    4-bit generator: the group's edge with the larger magnitude is represented exactly."""
+    import numpy as np
+    w = np.asarray(w, np.float32)
+    n, k = w.shape
+    g = w.reshape(n, k // 64, 64)
+    lo, hi = g.min(axis=2), g.max(axis=2)
+    mask = np.abs(lo) > np.abs(hi)
+    scale = np.maximum((hi - lo) / np.float32(255.0), np.float32(1e-7))
+    scale = np.where(mask, scale, -scale)
+    edge = np.where(mask, lo, hi)
+    q0 = np.rint(edge / scale)
+    nz = q0 != 0
+    scale = np.where(nz, edge / np.where(nz, q0, 1), scale).astype(np.float32)
+    bias = np.where(nz, edge, np.float32(0.0)).astype(np.float32)
+    s16, b16 = scale.astype(np.float16), bias.astype(np.float16)
+    q = np.clip(np.rint((g - bias[..., None]) / scale[..., None]), 0, 255).astype(np.uint32).reshape(n, k // 4, 4)
+    words = q[..., 0] | (q[..., 1] << 8) | (q[..., 2] << 16) | (q[..., 3] << 24)
+    return words.astype(np.uint32), s16, b16
+
+
 def generate_device(cfg, lib, device="cuda:0"):
     """Materialise the model in HBM.  Returns dict name -> torch tensor (q4 tensors appear as
     name.weight / name.scales / name.biases)."""
@@ -114,4 +138,13 @@ def generate_device(cfg, lib, device="cuda:0"):
                                            C.c_float(sigma), stream), "sl_synth_f32")
             t[name] = x
     torch.cuda.synchronize(dev)
+    if cfg.gate_bits == 8:
+        # the two gates of every layer re-expressed in 8 bits (quantised on the host: 0.5 M values per layer)
+        for i in range(cfg.n_layers):
+            for nm in (f"layers.{i}.mlp.gate", f"layers.{i}.mlp.shared_expert_gate"):
+                w, s, b = quantize_q8(t[nm + ".weight"].float().cpu().numpy().reshape(-1, abi.H))
+                t[nm + ".weight"] = torch.from_numpy(w.view("int32")).to(dev)
+                t[nm + ".scales"] = torch.from_numpy(s).to(dev)
+                t[nm + ".biases"] = torch.from_numpy(b).to(dev)
+        torch.cuda.synchronize(dev)
     return t

@@ -94,6 +94,59 @@ def test_moe_block_rows(moe_model, m, seed):
     assert np.isfinite(got.astype(np.float32)).all() and np.abs(got.astype(np.float32)).max() > 0
 
 
+def test_moe_block_rows_with_8bit_gates(env):
+    """The released checkpoint stores the router and the shared-expert gate in 8 bits (qmm8,
+    SeedlessMetalForward.swift:384): same block, gates as MLX-affine 8-bit rows."""
+    cfg = ModelConfig(n_layers=1, n_experts=256, vocab=0, layer_types=("gdn",), gate_bits=8)
+    dev, host = device_and_host_model(cfg)
+    assert host["layers.0.mlp.gate.weight"].shape == (256, 512) and host["layers.0.mlp.gate.scales"].shape == (256, 32)
+    eng = env["Engine"](cfg, dev, max_m=4, max_seq_len=16)
+    ora = env["orc"].Oracle(cfg, host, max_m=4, max_seq_len=16)
+    for m, seed in [(1, 1100), (4, 1101)]:
+        x = xrows(m, seed)
+        got, want = eng.moe_block_rows(0, x), ora.moe_block_rows(0, x)
+        assert got is not None, eng.gpu_fault
+        gi, gs = eng.read_route(0, m)
+        wi, ws = ora.read_route(0, m)
+        assert np.array_equal(gi, wi) and same_bits(gs, ws), first_diff(gs, ws)
+        assert same_bits(got, want), first_diff(got, want)
+        assert same_bits(eng.debug_scratch(7, m * 256).reshape(m, 256), ora_logits(ora, env, x, host)), "router logits"
+    eng.close()
+
+
+def ora_logits(ora, env, x, host):
+    """Router logits of the oracle's 8-bit rows for the post-normed rows the oracle's block saw."""
+    import ctypes as C
+    orc = env["orc"]
+    xn = np.ascontiguousarray(x, np.float16)
+    out = np.empty((xn.shape[0], 256), np.float16)
+    w, s, b = host["layers.0.mlp.gate.weight"], host["layers.0.mlp.gate.scales"], host["layers.0.mlp.gate.biases"]
+    for m in range(xn.shape[0]):
+        y = np.empty(256, np.float32)
+        orc.dll.orc_q8_f32(orc.p(xn[m]), orc.p(w), orc.p(s), orc.p(b), 256, 2048, orc.p(y))
+        out[m] = y.astype(np.float16)
+    return out
+
+
+def test_whole_stack_with_8bit_gates(env):
+    """8-bit gates through both execution paths: the greedy stream equals the oracle's, and the single-launch
+    step equals the kernel-per-stage sequence."""
+    cfg = ModelConfig(n_layers=4, n_experts=32, vocab=4096, gate_bits=8)
+    dev, host = device_and_host_model(cfg)
+    prompt = np.random.default_rng(31).integers(0, cfg.vocab, 11)
+    eng = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)
+    ora = env["orc"].Oracle(cfg, host, max_m=4, max_seq_len=64)
+    got = eng.greedy_generate(prompt, 20, chain_k=4)
+    assert got is not None, eng.gpu_fault
+    want = ora.greedy_generate(prompt, 20)
+    assert got.tolist() == want.tolist()
+    rows = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)
+    rows.set_persistent(False)
+    assert rows.greedy_generate(prompt, 20, chain_k=4).tolist() == want.tolist()
+    assert same_bits(eng.logits_row(0), rows.logits_row(0))
+    eng.close(); rows.close()
+
+
 # ---- BASELINE config 1: one GDN layer, sequential steps --------------------------------------------
 def test_gdn_layer_sequence(env):
     cfg = ModelConfig(n_layers=1, n_experts=8, vocab=0, layer_types=("gdn",))

@@ -189,6 +189,70 @@ def test_qmv_zero_codes_give_bias_times_sum():
     assert np.allclose(y, want, rtol=0, atol=2e-5)
 
 
+# ---- 8-bit gate rows (qmm8, SeedlessMetalForward.swift:372-428) ------------------------------------
+def q8_model(n, seed):
+    from qwisp_amd.synth import quantize_q8
+    w = np.random.default_rng(seed).normal(0, 0.02, (n, 2048)).astype(np.float16)
+    return w, quantize_q8(w)
+
+
+def test_q8_quantizer_invariants():
+    """MLX affine rule at 8 bits: 4 values per word, least significant byte first; reconstruction within half a
+    step; codes use the range; the group's edge of larger magnitude is represented exactly (up to fp16 storage)."""
+    w, (words, s, b) = q8_model(6, 5)
+    assert words.shape == (6, 512) and s.shape == b.shape == (6, 32) and s.dtype == b.dtype == np.float16
+    q = ((words[:, :, None] >> (8 * np.arange(4, dtype=np.uint32))[None, None, :]) & 255).reshape(6, 2048)
+    deq = s.astype(np.float64).repeat(64, axis=1) * q + b.astype(np.float64).repeat(64, axis=1)
+    step = np.abs(s.astype(np.float64)).repeat(64, axis=1)
+    slack = 255 * step * 2.0 ** -11 + np.abs(b.astype(np.float64)).repeat(64, axis=1) * 2.0 ** -11 + 1e-9   # fp16 scale and bias
+    err = np.abs(deq - w.astype(np.float64))
+    assert np.all(err[q < 255] <= 0.5 * step[q < 255] + slack[q < 255])
+    # the rule re-derives the step from the edge it pins, so the far end may clip at code 255 by about a step
+    assert np.all(err[q == 255] <= 1.5 * step[q == 255] + slack[q == 255])
+    assert q.min() == 0 and q.max() == 255
+    g = w.astype(np.float64).reshape(6, 32, 64)
+    edge = np.where(np.abs(g.min(axis=2)) > np.abs(g.max(axis=2)), g.min(axis=2), g.max(axis=2))
+    assert np.allclose(b.astype(np.float64), edge, rtol=1e-3, atol=0)
+
+
+def test_q8_dot_against_float64():
+    n = 40
+    w, (words, s, b) = q8_model(n, 6)
+    x = rng.normal(0, 1, 2048).astype(np.float16)
+    y = np.empty(n, np.float32)
+    dll.orc_q8_f32(orc.p(x), orc.p(words), orc.p(s), orc.p(b), n, 2048, orc.p(y))
+    q = ((words[:, :, None] >> (8 * np.arange(4, dtype=np.uint32))[None, None, :]) & 255).reshape(n, 2048)
+    d = s.astype(np.float64).repeat(64, axis=1) * q + b.astype(np.float64).repeat(64, axis=1)
+    want = d @ x.astype(np.float64)
+    # the two parts scale*sum(x q) and bias*sum(x) are large and cancel: bound on their magnitudes
+    mag = np.abs(s.astype(np.float64)).repeat(64, axis=1) * q @ np.abs(x.astype(np.float64)) + np.abs(b.astype(np.float64)).repeat(64, axis=1) @ np.abs(x.astype(np.float64))
+    assert np.all(np.abs(y - want) <= 4e-6 * mag + 1e-7), np.abs(y - want).max()
+    # and close to the unquantised row: the quantisation error of 8 bits is small against the logit scale
+    assert np.abs(want - w.astype(np.float64) @ x.astype(np.float64)).max() < 0.02
+
+
+def test_q8_unit_vectors_and_constant_codes():
+    """x = e_j returns float32(s*q + b) of exactly that value (byte order, word order, group and row indexing);
+    all codes equal c gives (s*c + b) * sum(x) group by group."""
+    n = 5
+    w, (words, s, b) = q8_model(n, 7)
+    q = ((words[:, :, None] >> (8 * np.arange(4, dtype=np.uint32))[None, None, :]) & 255).reshape(n, 2048)
+    for j in list(rng.integers(0, 2048, 24)) + [0, 3, 4, 31, 32, 63, 64, 2047]:
+        x = np.zeros(2048, np.float16)
+        x[j] = 1.0
+        y = np.empty(n, np.float32)
+        dll.orc_q8_f32(orc.p(x), orc.p(words), orc.p(s), orc.p(b), n, 2048, orc.p(y))
+        want = (s[:, j // 64].astype(np.float32) * q[:, j].astype(np.float32) + b[:, j // 64].astype(np.float32))
+        assert np.allclose(y, want, rtol=2e-7, atol=0), j
+    x = rng.normal(0, 1, 2048).astype(np.float16)
+    const = np.full((n, 512), 0x07070707, np.uint32)
+    y = np.empty(n, np.float32)
+    dll.orc_q8_f32(orc.p(x), orc.p(const), orc.p(s), orc.p(b), n, 2048, orc.p(y))
+    gs = x.astype(np.float64).reshape(32, 64).sum(axis=1)
+    want = ((s.astype(np.float64) * 7 + b.astype(np.float64)) * gs[None, :]).sum(axis=1)
+    assert np.allclose(y, want, rtol=0, atol=3e-5)
+
+
 def test_dense_and_rmsnorm_closed_forms():
     k, n = 2048, 12
     W = rng.normal(0, 0.02, (n, k)).astype(np.float16)
@@ -442,6 +506,39 @@ def test_engine_against_float64_graph(small_model):
             assert a.shape == (2, len(toks), 256)
             assert np.allclose(a.astype(np.float64), ref.cache[li]["k"], atol=0.03 * np.abs(ref.cache[li]["k"]).max())
             assert np.allclose(b.astype(np.float64), ref.cache[li]["v"], atol=0.03 * np.abs(ref.cache[li]["v"]).max())
+
+
+def test_eight_bit_gates_against_their_dequantised_fp16_rows():
+    """The 8-bit router / shared gate wired through the whole stack: the same model with the gates given as
+    fp16 rows holding half(s*q + b) differs only by that rounding, so router logits agree closely, nearly all
+    expert sets coincide and the hidden rows stay close; and the 8-bit model is not the unquantised one."""
+    cfg8 = ModelConfig(n_layers=4, n_experts=16, vocab=2048, gate_bits=8)
+    t8 = orc.generate_host(cfg8)
+    t16 = dict(t8)
+    for i in range(4):
+        for nm in (f"layers.{i}.mlp.gate", f"layers.{i}.mlp.shared_expert_gate"):
+            words, s, b = t8[nm + ".weight"], t8[nm + ".scales"], t8[nm + ".biases"]
+            q = ((words[:, :, None] >> (8 * np.arange(4, dtype=np.uint32))[None, None, :]) & 255).reshape(words.shape[0], 2048)
+            d = s.astype(np.float64).repeat(64, axis=1) * q + b.astype(np.float64).repeat(64, axis=1)
+            t16[nm + ".weight"] = d.astype(np.float16).reshape(-1) if words.shape[0] == 1 else d.astype(np.float16)
+            del t16[nm + ".scales"], t16[nm + ".biases"]
+    cfg16 = ModelConfig(n_layers=4, n_experts=16, vocab=2048)
+    o8, o16 = orc.Oracle(cfg8, t8, max_m=4, max_seq_len=32), orc.Oracle(cfg16, t16, max_m=4, max_seq_len=32)
+    toks = [5, 77, 1033, 9, 300, 12]
+    same_sets = total = 0
+    for t in toks:
+        a, b_ = o8.forward_tokens([t]), o16.forward_tokens([t])
+        for li in range(4):
+            i8, s8 = o8.read_route(li, 1)
+            i16, s16 = o16.read_route(li, 1)
+            total += 1
+            same_sets += set(i8[0].tolist()) == set(i16[0].tolist())
+        rel = np.linalg.norm(a.astype(np.float64) - b_.astype(np.float64)) / np.linalg.norm(b_.astype(np.float64))
+        assert rel < 0.05, rel
+    assert same_sets >= total - 2, (same_sets, total)
+    # the quantised gates are really in use: against the unquantised fp16 gates the logits move
+    o_plain = orc.Oracle(cfg16, orc.generate_host(cfg16), max_m=4, max_seq_len=32)
+    assert not np.array_equal(o_plain.forward_tokens([5]), orc.Oracle(cfg8, t8, max_m=4, max_seq_len=32).forward_tokens([5]))
 
 
 def test_rows_equal_single_steps_and_chain(small_model):
