@@ -77,6 +77,10 @@ typedef struct {
   const uint16_t* norm_w;   /* [128] fp16 */
   const float*    a_log;    /* [32] */
   const float*    dt_bias;  /* [32] */
+  /* linear_attn.norm.weight stored in fp32: used instead of norm_w when non-NULL.  The gated norm then forms
+   * w * (y * inv) in fp32 without the two half roundings of the fp16 case (the reference's "promote" variant,
+   * SeedlessFusedVerify.swift:2815 and :811). */
+  const float*    norm_w_f32; /* [128] */
 } sl_gdn_w;
 
 /* Full-attention mixer weights; names as in SeedlessEngine.swift:69-84. */

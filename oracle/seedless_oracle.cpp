@@ -328,7 +328,8 @@ static void gdn_layer_rows(Engine& e, int li, const float* x, int M, float* out)
     for (int hv = 0; hv < HV; ++hv) {
       const float inv = inv_rms(&y[hv * GD], GD);
       for (int i = 0; i < GD; ++i) {
-        const float nrm = f16r(h2f(w.norm_w[i]) * f16r(y[hv * GD + i] * inv));
+        // fp32 weight: w * (y * inv) stays in fp32 (the reference's promote variant, SeedlessFusedVerify.swift:811)
+        const float nrm = w.norm_w_f32 ? w.norm_w_f32[i] * (y[hv * GD + i] * inv) : f16r(h2f(w.norm_w[i]) * f16r(y[hv * GD + i] * inv));
         const float zf = z[(size_t)m * VALDIM + hv * GD + i];
         gated[hv * GD + i] = f16r((zf * sigmoid32(zf)) * nrm);
       }

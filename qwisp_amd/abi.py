@@ -26,7 +26,7 @@ class Q4(C.Structure):
 class GdnW(C.Structure):
     _fields_ = [("in_proj_qkv", Q4), ("in_proj_z", Q4), ("in_proj_b", Q4), ("in_proj_a", Q4),
                 ("out_proj", Q4), ("conv1d_w", C.c_void_p), ("norm_w", C.c_void_p),
-                ("a_log", C.c_void_p), ("dt_bias", C.c_void_p)]
+                ("a_log", C.c_void_p), ("dt_bias", C.c_void_p), ("norm_w_f32", C.c_void_p)]
 
 
 class AttnW(C.Structure):
@@ -100,6 +100,10 @@ def _ptr(t):
     return t.ctypes.data
 
 
+def _is_f32(t):
+    return "float32" in str(t.dtype)
+
+
 def _q4(tensors, name, n, k):
     w, s, b = tensors[name + ".weight"], tensors[name + ".scales"], tensors[name + ".biases"]
     return Q4(_ptr(w), _ptr(s), _ptr(b), n, k)
@@ -124,8 +128,9 @@ def build_desc(cfg, tensors, location):
                          _q4(tensors, la + "in_proj_b", GDN_HV, H),
                          _q4(tensors, la + "in_proj_a", GDN_HV, H),
                          _q4(tensors, la + "out_proj", H, GDN_HV * GDN_D),
-                         _ptr(tensors[la + "conv1d.weight"]), _ptr(tensors[la + "norm.weight"]),
-                         _ptr(tensors[la + "A_log"]), _ptr(tensors[la + "dt_bias"]))
+                         _ptr(tensors[la + "conv1d.weight"]), None if _is_f32(tensors[la + "norm.weight"]) else _ptr(tensors[la + "norm.weight"]),
+                         _ptr(tensors[la + "A_log"]), _ptr(tensors[la + "dt_bias"]),
+                         _ptr(tensors[la + "norm.weight"]) if _is_f32(tensors[la + "norm.weight"]) else None)
         else:
             sa = p + "self_attn."
             L.attn = AttnW(_q4(tensors, sa + "q_proj", ATT_HEADS * 2 * ATT_D, H),

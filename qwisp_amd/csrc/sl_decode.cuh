@@ -23,7 +23,8 @@ struct LayerP {
   const uint32_t *in_w, *in_sb;          // GDN in_proj [12352,2048] or attention q|k|v [9216,2048]
   const uint32_t *out_w, *out_sb;        // GDN out_proj or attention o_proj [2048,4096]
   const float *conv_w, *a_log, *dt_bias;
-  const uint16_t* gdn_norm_w;
+  const float* gdn_norm_w;               // [128] fp32 (an fp16 checkpoint weight converted exactly)
+  int gdn_norm_f32;                      // the checkpoint weight was fp32: gated norm without the half roundings
   uint16_t* hist[2];
   float* state[2];
   const uint16_t *q_norm, *k_norm;

@@ -30,7 +30,8 @@ struct LayerDev {
   // Gated-DeltaNet
   DevQ4 in_proj, out_proj;
   float *conv_w = nullptr, *a_log = nullptr, *dt_bias = nullptr;
-  uint16_t* gdn_norm_w = nullptr;
+  float* gdn_norm_w = nullptr;     // [128] fp32; norm_f32: it came as fp32 (gated norm without the half roundings)
+  int norm_f32 = 0;
   uint16_t* hist[2] = {nullptr, nullptr};
   float* state[2] = {nullptr, nullptr};
   // attention
@@ -172,6 +173,7 @@ bool upload_q4(sl_engine* e, DevQ4& d, const sl_q4& src, int n, int k, int loc) 
   return alloc_q4(e, d, n, k) && fill_q4(e, d, 0, src, n, k, loc);
 }
 
+float half_bits_to_float(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 void build_rope(std::vector<float>& c, std::vector<float>& s, int max_seq) {
   c.resize((size_t)max_seq * 32); s.resize((size_t)max_seq * 32);
   for (int i = 0; i < 32; ++i) {
@@ -249,7 +251,7 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
   g.st = e->st + li;       // st[1] of this view = parity of layer li
   g.ycore = e->ycore; g.M = M; g.lanes = lanes; g.layer = li;
   hipLaunchKernelGGL(k_gdn_core, dim3(256, lanes ? M : 1), dim3(256), 0, e->stream, g);
-  hipLaunchKernelGGL(k_qmv_gdn_out<2>, dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w,
+  hipLaunchKernelGGL(k_qmv_gdn_out<2>, dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32,
                      L.out_proj.w, L.out_proj.sb, H, e->mix);
 }
 void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, const LaneRef* lanes, int lane_tiles) {
@@ -401,7 +403,18 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
       L.conv_w = upload<float>(e, g.conv1d_w, (size_t)SL_CONV_DIM * SL_CONV_K, loc);
       L.a_log = upload<float>(e, g.a_log, SL_GDN_HV, loc);
       L.dt_bias = upload<float>(e, g.dt_bias, SL_GDN_HV, loc);
-      L.gdn_norm_w = upload<uint16_t>(e, g.norm_w, SL_GDN_D, loc);
+      if (g.norm_w_f32) {
+        L.gdn_norm_w = upload<float>(e, g.norm_w_f32, SL_GDN_D, loc);
+        L.norm_f32 = 1;
+      } else if (g.norm_w) {
+        // fp16 weight, kept as fp32 on the device (exact); a device-resident source comes through the host
+        uint16_t hw[SL_GDN_D];
+        float fw[SL_GDN_D];
+        if (loc == SL_LOC_HOST) std::memcpy(hw, g.norm_w, sizeof(hw));
+        else SL_TRY(e, hipMemcpy(hw, g.norm_w, sizeof(hw), hipMemcpyDeviceToHost));
+        for (int j = 0; j < SL_GDN_D; ++j) fw[j] = half_bits_to_float(hw[j]);
+        L.gdn_norm_w = upload<float>(e, fw, SL_GDN_D, SL_LOC_HOST);
+      }
       if (!L.conv_w || !L.a_log || !L.dt_bias || !L.gdn_norm_w) return SL_ERR_DEVICE;
     } else {
       const sl_attn_w& a = s.attn;
@@ -499,7 +512,7 @@ int alloc_runtime(sl_engine* e) {
         q.is_linear = L.is_linear; q.input_ln = L.input_ln; q.post_ln = L.post_ln;
         if (L.is_linear) {
           q.in_w = L.in_proj.w; q.in_sb = L.in_proj.sb; q.out_w = L.out_proj.w; q.out_sb = L.out_proj.sb;
-          q.conv_w = L.conv_w; q.a_log = L.a_log; q.dt_bias = L.dt_bias; q.gdn_norm_w = L.gdn_norm_w;
+          q.conv_w = L.conv_w; q.a_log = L.a_log; q.dt_bias = L.dt_bias; q.gdn_norm_w = L.gdn_norm_w; q.gdn_norm_f32 = L.norm_f32;
           q.hist[0] = L.hist[0]; q.hist[1] = L.hist[1]; q.state[0] = L.state[0]; q.state[1] = L.state[1];
         } else {
           q.in_w = L.qkv.w; q.in_sb = L.qkv.sb; q.out_w = L.o_proj.w; q.out_sb = L.o_proj.sb;

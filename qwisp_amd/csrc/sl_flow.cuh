@@ -831,16 +831,16 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     out[0] = lo_h(a.x); out[1] = lo_h(a.y); out[2] = lo_h(a.z); out[3] = lo_h(a.w);
   }
   if (lin) {
-    float nw[4];
-    const uint2 wraw = *reinterpret_cast<const uint2*>(uni(Y.gdn_norm_w) + (e0 & 127));
-    nw[0] = lo_h(wraw.x); nw[1] = hi_h(wraw.x); nw[2] = lo_h(wraw.y); nw[3] = hi_h(wraw.y);
+    const float4 wraw = *reinterpret_cast<const float4*>(uni(Y.gdn_norm_w) + (e0 & 127));
+    const float nw[4] = {wraw.x, wraw.y, wraw.z, wraw.w};
+    const bool nf32 = uni(Y.gdn_norm_f32) != 0;
     const float la = fmaf(out[1], out[1], fmaf(out[0], out[0], 0.0f));
     const float lb = fmaf(out[3], out[3], fmaf(out[2], out[2], 0.0f));
     const float ss = tree_sum<32>(la + lb);
     const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float nrm = f16r(nw[i] * f16r(out[i] * inv));
+      const float nrm = nf32 ? nw[i] * (out[i] * inv) : f16r(nw[i] * f16r(out[i] * inv));
       out[i] = f16r(sz[i] * nrm);
     }
   }

@@ -303,18 +303,22 @@ __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
 }
 
 // -------------------------------------------------------------------------------------------------
-// GDN out-proj with the gated rmsnorm as prologue: x = half(silu(z) * (w * half(y*inv))) per value
-// head, then the K = 4096 4-bit dot.  Reference: gdn_norm_gate_rows SeedlessFusedVerify.swift:768-812.
+// GDN out-proj with the gated rmsnorm as prologue: x = half(silu(z) * half(w * half(y*inv))) per value
+// head (with an fp32 norm weight: half(silu(z) * (w * (y*inv)))), then the K = 4096 4-bit dot.  Reference: gdn_norm_gate_rows SeedlessFusedVerify.swift:768-812.
 // -------------------------------------------------------------------------------------------------
 template <int R>
 __global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict__ ycore, const uint16_t* __restrict__ proj,
-                                                     const uint16_t* __restrict__ norm_w, const uint32_t* __restrict__ W,
+                                                     const float* __restrict__ norm_w, int norm_f32, const uint32_t* __restrict__ W,
                                                      const uint32_t* __restrict__ SB, int N, uint16_t* __restrict__ y) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float sx[8];
   uint32_t xp[32];
-  float nw[32];
-  load32(norm_w + 32 * (lane & 3), nw);
+  float nw[32];                                  // norm weight as fp32 (exact for an fp16 checkpoint weight)
+#pragma unroll
+  for (int i = 0; i < 32; i += 4) {
+    const float4 v = *reinterpret_cast<const float4*>(norm_w + 32 * (lane & 3) + i);
+    nw[i] = v.x; nw[i + 1] = v.y; nw[i + 2] = v.z; nw[i + 3] = v.w;
+  }
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
     float xb[32];
@@ -332,7 +336,7 @@ __global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict_
     load32(proj + (size_t)m * PROJ_STRIDE + 8192 + b * 2048 + 32 * lane, z);
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
-      const float nrm = f16r(nw[i] * f16r(xb[i] * inv));
+      const float nrm = norm_f32 ? nw[i] * (xb[i] * inv) : f16r(nw[i] * f16r(xb[i] * inv));
       xb[i] = f16r((z[i] * sigmoid32(z[i])) * nrm);
     }
     word_sums(xb, sx + 4 * b);

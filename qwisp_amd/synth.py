@@ -20,6 +20,7 @@ class ModelConfig:
     seed_base: int = 2000
     layer_types: tuple = None         # optional explicit override, e.g. ("gdn",) or ("attn",)
     gate_bits: int = 16               # 16: fp16 router / shared gate (benchmark configuration); 8: MLX affine 8-bit
+    norm_f32: bool = False            # linear_attn.norm.weight in fp32 (the reference's "promote" variant of the gated norm)
 
     def is_linear(self, i):
         if self.layer_types is not None:
@@ -54,7 +55,7 @@ def tensor_specs(cfg):
                     _q4(la + "in_proj_a", abi.GDN_HV, H, s + 13),
                     _q4(la + "out_proj", H, abi.GDN_HV * abi.GDN_D, s + 14),
                     (la + "conv1d.weight", "f32", (abi.CONV_DIM, abi.CONV_K), s + 15, 0.0, 0.5),
-                    (la + "norm.weight", "f16", (abi.GDN_D,), s + 16, 1.0, 0.1),
+                    (la + "norm.weight", "f32" if cfg.norm_f32 else "f16", (abi.GDN_D,), s + 16, 1.0, 0.1),
                     (la + "A_log", "f32", (abi.GDN_HV,), s + 17, 0.0, 1.0),
                     (la + "dt_bias", "f32", (abi.GDN_HV,), s + 18, 0.0, 1.0)]
         else:

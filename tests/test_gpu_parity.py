@@ -128,10 +128,22 @@ def ora_logits(ora, env, x, host):
     return out
 
 
-def test_whole_stack_with_8bit_gates(env):
-    """8-bit gates through both execution paths: the greedy stream equals the oracle's, and the single-launch
-    step equals the kernel-per-stage sequence."""
-    cfg = ModelConfig(n_layers=4, n_experts=32, vocab=4096, gate_bits=8)
+def test_whole_stack_in_the_released_checkpoint_configuration(env):
+    """8-bit gates and an fp32 linear_attn.norm.weight (SeedlessFusedVerify.swift:2815) through both execution
+    paths: the greedy stream equals the oracle's, and the single-launch step equals the kernel-per-stage
+    sequence; one GDN layer's rows equal the oracle's bit for bit."""
+    cfg1 = ModelConfig(n_layers=1, n_experts=8, vocab=0, layer_types=("gdn",), norm_f32=True)
+    dev1, host1 = device_and_host_model(cfg1)
+    assert host1["layers.0.linear_attn.norm.weight"].dtype == np.float32
+    e1 = env["Engine"](cfg1, dev1, max_m=4, max_seq_len=8)
+    o1 = env["orc"].Oracle(cfg1, host1, max_m=4, max_seq_len=8)
+    for m, seed in [(1, 1400), (3, 1401)]:
+        x = xrows(m, seed)
+        got, want = e1.gdn_layer_rows(0, x), o1.gdn_layer_rows(0, x)
+        assert got is not None, e1.gpu_fault
+        assert same_bits(got, want), first_diff(got, want)
+    e1.close()
+    cfg = ModelConfig(n_layers=4, n_experts=32, vocab=4096, gate_bits=8, norm_f32=True)
     dev, host = device_and_host_model(cfg)
     prompt = np.random.default_rng(31).integers(0, cfg.vocab, 11)
     eng = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)

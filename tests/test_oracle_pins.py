@@ -541,6 +541,27 @@ def test_eight_bit_gates_against_their_dequantised_fp16_rows():
     assert not np.array_equal(o_plain.forward_tokens([5]), orc.Oracle(cfg8, t8, max_m=4, max_seq_len=32).forward_tokens([5]))
 
 
+def test_fp32_gated_norm_weight_variant():
+    """linear_attn.norm.weight in fp32 (the reference's promote variant, SeedlessFusedVerify.swift:2815, :811):
+    w * (y * inv) is formed in fp32.  With a weight that is exactly 1 the two variants differ only by the half
+    rounding of y * inv, so the layer outputs agree closely but not bit for bit; with weight 2 the output of the
+    gated norm doubles exactly (a power of two commutes with every rounding), which the out-projection then
+    carries through linearly up to its own rounding."""
+    cfg = ModelConfig(n_layers=1, n_experts=8, vocab=0, layer_types=("gdn",), norm_f32=True)
+    t = orc.generate_host(cfg)
+    assert t["layers.0.linear_attn.norm.weight"].dtype == np.float32
+    x = rng.normal(0, 1, (3, 2048)).astype(np.float16)
+    outs = {}
+    for name, w in (("one32", np.ones(128, np.float32)), ("one16", np.ones(128, np.float16)), ("two32", np.full(128, 2.0, np.float32))):
+        tt = dict(t)
+        tt["layers.0.linear_attn.norm.weight"] = w
+        o = orc.Oracle(cfg, tt, max_m=4, max_seq_len=8)
+        outs[name] = o.gdn_layer_rows(0, x).astype(np.float64)
+    d = np.abs(outs["one32"] - outs["one16"])
+    assert 0 < d.max() < 0.02 * np.abs(outs["one16"]).max()
+    assert np.abs(outs["two32"] - 2 * outs["one32"]).max() < 0.004 * np.abs(outs["two32"]).max()
+
+
 def test_rows_equal_single_steps_and_chain(small_model):
     """M-row forward == M single-row forwards (SeedlessVerifyTests.swift:613), chained == stepped
     (:2445): tokens, logits and every cache bit-for-bit."""
