@@ -159,6 +159,24 @@ def test_whole_stack_in_the_released_checkpoint_configuration(env):
     eng.close(); rows.close()
 
 
+def test_engine_from_a_checkpoint_directory(env, tmp_path):
+    """A model written in the reference's checkpoint layout (shards + index, reference tensor names) and loaded
+    back onto the device gives the stream of the engine built from the generator's tensors directly."""
+    from qwisp_amd import checkpoint
+    cfg = ModelConfig(n_layers=4, n_experts=32, vocab=4096, gate_bits=8, norm_f32=True)
+    dev, host = device_and_host_model(cfg)
+    checkpoint.save_checkpoint(str(tmp_path), host, shard_bytes=16 << 20)
+    cfg2, t2 = checkpoint.load_checkpoint(str(tmp_path), device="cuda:0")
+    assert (cfg2.n_layers, cfg2.n_experts, cfg2.vocab, cfg2.gate_bits, cfg2.norm_f32) == (4, 32, 4096, 8, True)
+    prompt = np.random.default_rng(8).integers(0, cfg.vocab, 9)
+    a = env["Engine"](cfg, dev, max_m=4, max_seq_len=64)
+    b = env["Engine"](cfg2, t2, max_m=4, max_seq_len=64)
+    ga, gb = a.greedy_generate(prompt, 16, chain_k=4), b.greedy_generate(prompt, 16, chain_k=4)
+    assert ga is not None and gb is not None, (a.gpu_fault, b.gpu_fault)
+    assert ga.tolist() == gb.tolist() and same_bits(a.logits_row(0), b.logits_row(0))
+    a.close(); b.close()
+
+
 # ---- BASELINE config 1: one GDN layer, sequential steps --------------------------------------------
 def test_gdn_layer_sequence(env):
     cfg = ModelConfig(n_layers=1, n_experts=8, vocab=0, layer_types=("gdn",))
