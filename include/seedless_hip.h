@@ -328,6 +328,12 @@ void* sl_stream(sl_engine* e);
  * compute units (the reference's counterpart is the one-command-buffer step, SFV:3881-3890);
  * 0 switches to the kernel-per-stage sequence used for M > 1.  Both give identical results. */
 int sl_set_persistent(sl_engine* e, int enable);
+/* forwardRowsHybrid (SeedlessFusedVerify.swift:4240-4247): while enabled, calls with 16 <= m <= 128 rows of one
+ * sequence (prefill chunks) compute the dense mixer projections (GDN in/out, attention q|k|v and o) on the matrix
+ * cores, with weights dequantised to half.  Like the reference's matrix-unit prefill this is not bit-identical to
+ * the GEMV order (tolerance-level agreement) but deterministic and independent of how a prompt is chunked.
+ * Decode steps, verify rows below 16 and lane batches are unaffected. */
+int sl_set_hybrid(sl_engine* e, int enable);
 
 /* Diagnostic: while enabled, workgroups 0 and 100 of the single-launch step record a 100 MHz clock stamp
  * before and after every poll; the call copies out[0] = number of stamps of workgroup 0 and out[1..] its
@@ -356,6 +362,10 @@ int sl_synth_f32(float* dst_dev, int64_t count, uint64_t seed, float mean, float
  * op: 0 exp, 1 log, 2 sigmoid (fp32), 3 sigmoid (half), 4 softplus, 5 round-to-half,
  * 6 1/sqrt(x/128 + 1e-6), 7 half(x*sigmoid(x)), 8 normal quantile. */
 int sl_selftest_math(int op, const float* x_host, float* y_host, int64_t n);
+/* Self-test of the matrix-core GEMM of the hybrid prefill (host arrays in and out): y[m, n] = half(sum_k x[m, k] *
+ * half(s*q + b)) for 4-bit group-64 weights [n, k]; m <= 128, n % 32 == 0, k % 64 == 0. */
+int sl_selftest_qmm4(const uint16_t* x_host, int m, const uint32_t* w_host, const uint16_t* scales_host,
+                     const uint16_t* biases_host, int n, int k, uint16_t* y_host);
 
 #ifdef __cplusplus
 }

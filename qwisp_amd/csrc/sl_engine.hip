@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "sl_flow.cuh"
+#include "sl_mfma.cuh"
 
 using namespace sl;
 
@@ -94,6 +95,11 @@ struct sl_engine {
   double head_ms_sum = 0.0;
   long head_launches = 0;
   bool use_persistent = true;
+  bool hybrid = false;             // prefill chunks: dense projections and grouped experts on the matrix cores (not bit-identical to the GEMV order)
+  // scratch of the hybrid MoE (allocated when hybrid is first enabled): routed gate / up / down results per pair,
+  // shared gate / up / down rows, pairs listed per expert
+  uint16_t *hy_g = nullptr, *hy_u = nullptr, *hy_d = nullptr, *hy_sg = nullptr, *hy_su = nullptr, *hy_sy = nullptr, *hy_lists = nullptr;
+  int32_t* hy_counts = nullptr;
   bool inject_failure = false;
   // lane batch driven from this engine's scratch: device table [n_layers][max_m] of the lanes last stepped together
   LaneRef* lane_tab = nullptr;
@@ -223,6 +229,34 @@ int finish(sl_engine* e, const char* what) {
 }
 
 // ---- launch sequences -------------------------------------------------------------------------------
+// Hybrid prefill: router and shared-gate logits stay on the exact GEMV rows (routing decides which experts run);
+// the shared expert and the routed experts, grouped by expert, go to the matrix cores.
+void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
+  const int E = e->n_experts;
+  MoeAArgs a{};
+  a.ha = ha;
+  a.router_w = L.router_w; a.sgate_w = L.sgate_w; a.g8_w = L.gate8_w; a.g8_sb = L.gate8_sb; a.E = E; a.skip_shared = 1;
+  a.sh_act = e->sh_act; a.rlogits = e->rlogits; a.sgate = e->sgate;
+  const int router_blocks = (E + 1 + 15) / 16;
+  hipLaunchKernelGGL(k_moe_a, dim3(MOE_A_SHARED_BLOCKS + router_blocks, M), dim3(256), 0, e->stream, a);
+  hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, E, L.route_inds, L.route_scores);
+  hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, E, e->hy_lists, e->hy_counts);
+  // routed gate / up by expert, SwiGLU, routed down by expert
+  QmmGroupArgs g{e->xn, H, 0, L.sw_gate.w, L.sw_gate.sb, SL_MOE_I, H, e->hy_lists, e->hy_counts, e->hy_g, SL_MOE_I};
+  hipLaunchKernelGGL(k_qmm4_mfma_grouped, dim3(SL_MOE_I / 128, E), dim3(256), 0, e->stream, g);
+  g.W = L.sw_up.w; g.SB = L.sw_up.sb; g.y = e->hy_u;
+  hipLaunchKernelGGL(k_qmm4_mfma_grouped, dim3(SL_MOE_I / 128, E), dim3(256), 0, e->stream, g);
+  const int tot = M * 8 * SL_MOE_I;
+  hipLaunchKernelGGL(k_swiglu_rows, dim3((tot + 255) / 256), dim3(256), 0, e->stream, e->hy_g, e->hy_u, e->act, tot);
+  QmmGroupArgs d{e->act, SL_MOE_I, 1, L.sw_down.w, L.sw_down.sb, H, SL_MOE_I, e->hy_lists, e->hy_counts, e->hy_d, H};
+  hipLaunchKernelGGL(k_qmm4_mfma_grouped, dim3(H / 128, E), dim3(256), 0, e->stream, d);
+  // shared expert
+  launch_qmm4_mfma(QmmArgs{e->xn, H, L.sh_gate.w, L.sh_gate.sb, M, SL_MOE_I, H, e->hy_sg, SL_MOE_I}, e->stream);
+  launch_qmm4_mfma(QmmArgs{e->xn, H, L.sh_up.w, L.sh_up.sb, M, SL_MOE_I, H, e->hy_su, SL_MOE_I}, e->stream);
+  hipLaunchKernelGGL(k_swiglu_rows, dim3((M * SL_MOE_I + 255) / 256), dim3(256), 0, e->stream, e->hy_sg, e->hy_su, e->sh_act, M * SL_MOE_I);
+  launch_qmm4_mfma(QmmArgs{e->sh_act, SL_MOE_I, L.sh_down.w, L.sh_down.sb, M, H, SL_MOE_I, e->hy_sy, H}, e->stream);
+  hipLaunchKernelGGL(k_moe_combine_rows, dim3(H / 256, M), dim3(256), 0, e->stream, e->hy_d, L.route_scores, e->sgate, e->hy_sy, e->moe_out);
+}
 void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   MoeAArgs a{};
   a.ha = ha;
@@ -241,22 +275,43 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   c.d_w = L.sw_down.w; c.d_sb = L.sw_down.sb; c.shd_w = L.sh_down.w; c.shd_sb = L.sh_down.sb; c.out = e->moe_out;
   hipLaunchKernelGGL(k_moe_c, dim3(256, M), dim3(128), 0, e->stream, c);
 }
+// Hybrid prefill: chunks of at least 16 rows of one sequence take the dense mixer projections to the matrix cores.
+bool use_matrix_cores(const sl_engine* e, int M, const LaneRef* lanes) { return e->hybrid && !lanes && M >= 16 && M <= 128; }
 // `lanes` (null for rows of one sequence) = this layer's row of the lane table: row b of the batch is lane b's next token.
 void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs& ha, const LaneRef* lanes) {
-  hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_GDN_IN_N / 16, M), dim3(256), 0, e->stream, ha, L.in_proj.w, L.in_proj.sb,
-                     SL_GDN_IN_N, e->proj, PROJ_STRIDE);
+  const bool mm = use_matrix_cores(e, M, lanes);
+  if (mm) {
+    HiddenArgs hn = ha; hn.xn_out = e->xn;      // residual + norm rows on their own, then the GEMM
+    hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
+    launch_qmm4_mfma(QmmArgs{e->xn, H, L.in_proj.w, L.in_proj.sb, M, SL_GDN_IN_N, H, e->proj, PROJ_STRIDE}, e->stream);
+  } else {
+    hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_GDN_IN_N / 16, M), dim3(256), 0, e->stream, ha, L.in_proj.w, L.in_proj.sb,
+                       SL_GDN_IN_N, e->proj, PROJ_STRIDE);
+  }
   GdnArgs g{};
   g.proj = e->proj; g.conv_w = L.conv_w; g.a_log = L.a_log; g.dt_bias = L.dt_bias;
   g.hist[0] = L.hist[0]; g.hist[1] = L.hist[1]; g.state[0] = L.state[0]; g.state[1] = L.state[1];
   g.st = e->st + li;       // st[1] of this view = parity of layer li
   g.ycore = e->ycore; g.M = M; g.lanes = lanes; g.layer = li;
   hipLaunchKernelGGL(k_gdn_core, dim3(256, lanes ? M : 1), dim3(256), 0, e->stream, g);
-  hipLaunchKernelGGL(k_qmv_gdn_out<2>, dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32,
-                     L.out_proj.w, L.out_proj.sb, H, e->mix);
+  if (mm) {
+    hipLaunchKernelGGL(k_gdn_gate_rows, dim3(SL_GDN_HV, M), dim3(64), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32);
+    launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.out_proj.w, L.out_proj.sb, M, H, 4096, e->mix, H}, e->stream);
+  } else {
+    hipLaunchKernelGGL(k_qmv_gdn_out<2>, dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32,
+                       L.out_proj.w, L.out_proj.sb, H, e->mix);
+  }
 }
 void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, const LaneRef* lanes, int lane_tiles) {
-  hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_ATT_QKV_N / 16, M), dim3(256), 0, e->stream, ha, L.qkv.w, L.qkv.sb,
-                     SL_ATT_QKV_N, e->proj, PROJ_STRIDE);
+  const bool mm = use_matrix_cores(e, M, lanes);
+  if (mm) {
+    HiddenArgs hn = ha; hn.xn_out = e->xn;
+    hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
+    launch_qmm4_mfma(QmmArgs{e->xn, H, L.qkv.w, L.qkv.sb, M, SL_ATT_QKV_N, H, e->proj, PROJ_STRIDE}, e->stream);
+  } else {
+    hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_ATT_QKV_N / 16, M), dim3(256), 0, e->stream, ha, L.qkv.w, L.qkv.sb,
+                       SL_ATT_QKV_N, e->proj, PROJ_STRIDE);
+  }
   AttnPrepArgs p{};
   p.proj = e->proj; p.q_norm = L.q_norm; p.k_norm = L.k_norm; p.rope_cos = e->rope_cos; p.rope_sin = e->rope_sin;
   p.st = e->st; p.qrot = e->qrot; p.kcache = L.kcache; p.vcache = L.vcache; p.maxSeq = e->max_seq; p.lanes = lanes;
@@ -269,8 +324,9 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
   SdpaMergeArgs g{};
   g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore; g.lanes = lanes;
   hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
-  hipLaunchKernelGGL((k_qmv_plain<2, 2>), dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, 4096, L.o_proj.w, L.o_proj.sb,
-                     H, e->mix, H);
+  if (mm) launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.o_proj.w, L.o_proj.sb, M, H, 4096, e->mix, H}, e->stream);
+  else hipLaunchKernelGGL((k_qmv_plain<2, 2>), dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, 4096, L.o_proj.w, L.o_proj.sb,
+                          H, e->mix, H);
 }
 // All layers over M rows held in hA.  On return the hidden state is hA + moe_out (residual pending).
 // With `lane_tab` the M rows are one token each of M lanes (caches and positions from the table, the longest
@@ -283,7 +339,8 @@ void launch_layers(sl_engine* e, int M, const LaneRef* lane_tab = nullptr, int l
     if (L.is_linear) launch_gdn_mixer(e, L, li, M, ha, lanes);
     else launch_attn_mixer(e, L, M, ha, lanes, lane_tiles);
     HiddenArgs hb{e->hB, e->mix, L.post_ln, e->hA, e->xn};
-    launch_moe(e, L, M, hb);
+    if (use_matrix_cores(e, M, lanes)) launch_moe_hybrid(e, L, M, hb);
+    else launch_moe(e, L, M, hb);
   }
 }
 void advance(sl_engine* e, int M) {
@@ -700,6 +757,22 @@ int sl_position(const sl_engine* e) { return e ? e->pos : -1; }
 int sl_max_rows(const sl_engine* e) { return e ? e->max_m : -1; }
 float sl_last_gpu_ms(const sl_engine* e) { return e ? e->last_ms : 0.0f; }
 void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
+int sl_set_hybrid(sl_engine* e, int enable) {
+  int r = guard(e); if (r) return r;
+  if (enable && !e->hy_g) {
+    const size_t rows = (size_t)(e->max_m < 128 ? e->max_m : 128);
+    e->hy_g = dalloc<uint16_t>(e, rows * 8 * SL_MOE_I); e->hy_u = dalloc<uint16_t>(e, rows * 8 * SL_MOE_I);
+    e->hy_d = dalloc<uint16_t>(e, rows * 8 * H);
+    e->hy_sg = dalloc<uint16_t>(e, rows * SL_MOE_I); e->hy_su = dalloc<uint16_t>(e, rows * SL_MOE_I);
+    e->hy_sy = dalloc<uint16_t>(e, rows * H);
+    e->hy_lists = dalloc<uint16_t>(e, (size_t)SL_MAX_EXPERTS * GROUP_CAP, true);
+    e->hy_counts = dalloc<int32_t>(e, SL_MAX_EXPERTS, true);
+    if (!e->hy_g || !e->hy_u || !e->hy_d || !e->hy_sg || !e->hy_su || !e->hy_sy || !e->hy_lists || !e->hy_counts) return SL_ERR_DEVICE;
+    SL_TRY(e, hipStreamSynchronize(e->stream));
+  }
+  e->hybrid = enable != 0;
+  return SL_OK;
+}
 int sl_set_persistent(sl_engine* e, int enable) {
   int r = guard(e); if (r) return r;
   e->use_persistent = enable != 0;
@@ -1125,3 +1198,27 @@ int sl_greedy_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_
 }
 
 }  // extern "C"
+
+// Self-test of the matrix-core GEMM (sl_mfma.cuh): host arrays in and out, temporary device buffers.
+extern "C" int sl_selftest_qmm4(const uint16_t* x_host, int m, const uint32_t* w_host, const uint16_t* s_host,
+                                const uint16_t* b_host, int n, int k, uint16_t* y_host) {
+  if (!x_host || !w_host || !s_host || !b_host || !y_host || m < 1 || m > 128 || n < 32 || (n % 32) || k < 64 || (k % 64))
+    return SL_ERR_ARG;
+  const size_t xb = (size_t)m * k * 2, wb = (size_t)n * (k / 8) * 4, gb = (size_t)n * (k / 64) * 4, yb = (size_t)m * n * 2;
+  std::vector<uint32_t> sb((size_t)n * (k / 64));
+  for (size_t i = 0; i < sb.size(); ++i) sb[i] = (uint32_t)s_host[i] | ((uint32_t)b_host[i] << 16);
+  uint16_t *dx = nullptr, *dy = nullptr;
+  uint32_t *dw = nullptr, *dsb = nullptr;
+  int rc = SL_ERR_DEVICE;
+  if (hipMalloc((void**)&dx, xb) == hipSuccess && hipMalloc((void**)&dw, wb) == hipSuccess &&
+      hipMalloc((void**)&dsb, gb) == hipSuccess && hipMalloc((void**)&dy, yb) == hipSuccess &&
+      hipMemcpy(dx, x_host, xb, hipMemcpyHostToDevice) == hipSuccess && hipMemcpy(dw, w_host, wb, hipMemcpyHostToDevice) == hipSuccess &&
+      hipMemcpy(dsb, sb.data(), gb, hipMemcpyHostToDevice) == hipSuccess) {
+    QmmArgs a{dx, k, dw, dsb, m, n, k, dy, n};
+    launch_qmm4_mfma(a, nullptr);
+    if (hipGetLastError() == hipSuccess && hipDeviceSynchronize() == hipSuccess &&
+        hipMemcpy(y_host, dy, yb, hipMemcpyDeviceToHost) == hipSuccess) rc = SL_OK;
+  }
+  (void)hipFree(dx); (void)hipFree(dw); (void)hipFree(dsb); (void)hipFree(dy);
+  return rc;
+}

@@ -356,6 +356,26 @@ __global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict_
 }
 
 // -------------------------------------------------------------------------------------------------
+// Gated rmsnorm rows on their own (hybrid prefill: the out-projection then runs on the matrix cores):
+// gated[m, hv, :] = half(silu(z) * norm(y)) in place of y.  One wave per (value head, row); lane l owns the pair
+// 2l, 2l+1, so the sum of squares is the same balanced tree as in the fused kernel above.
+// -------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void k_gdn_gate_rows(uint16_t* __restrict__ ycore, const uint16_t* __restrict__ proj,
+                                                      const float* __restrict__ norm_w, int norm_f32) {
+  const int hv = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;
+  uint16_t* yp = ycore + (size_t)m * 4096 + hv * 128 + 2 * lane;
+  const uint32_t yw = *reinterpret_cast<const uint32_t*>(yp);
+  const uint32_t zw = *reinterpret_cast<const uint32_t*>(proj + (size_t)m * PROJ_STRIDE + 8192 + hv * 128 + 2 * lane);
+  const float y0 = lo_h(yw), y1 = hi_h(yw), z0 = lo_h(zw), z1 = hi_h(zw);
+  const float ss = tree_sum<64>(fmaf(y1, y1, fmaf(y0, y0, 0.0f)));
+  const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
+  const float w0 = norm_w[2 * lane], w1 = norm_w[2 * lane + 1];
+  const float n0 = norm_f32 ? w0 * (y0 * inv) : f16r(w0 * f16r(y0 * inv));
+  const float n1 = norm_f32 ? w1 * (y1 * inv) : f16r(w1 * f16r(y1 * inv));
+  *reinterpret_cast<uint32_t*>(yp) = pack2(f16r((z0 * sigmoid32(z0)) * n0), f16r((z1 * sigmoid32(z1)) * n1));
+}
+
+// -------------------------------------------------------------------------------------------------
 // MoE stage A: residual + post-attention norm, then in one launch the shared expert's gate/up
 // with SwiGLU (64 workgroups), the fp16 router gate rows and the shared-expert gate row.
 // References: MoEBlock.swift:69-97; shared expert SeedlessFusedVerify.swift:1859-1871.
@@ -367,6 +387,7 @@ struct MoeAArgs {
   const uint16_t* sgate_w;                           // [2048]
   const uint32_t *g8_w, *g8_sb;                      // 8-bit gates instead (null: fp16): [E+1, 512] words, [E+1, 32] {scale, bias}; row E = shared gate
   int E;
+  int skip_shared;                                   // hybrid prefill: the shared expert's gate/up run on the matrix cores
   uint16_t* sh_act;                                  // [M, 512]
   uint16_t* rlogits;                                 // [M, 256]
   uint16_t* sgate;                                   // [M]
@@ -377,6 +398,7 @@ __global__ __launch_bounds__(256) void k_moe_a(MoeAArgs a) {
   float x[32], sx[4];
   hidden_prologue(a.ha, m, lane, blockIdx.x == 0 && wave == 0, x);
   if (blockIdx.x < MOE_A_SHARED_BLOCKS) {
+    if (a.skip_shared) return;
     word_sums(x, sx);
     uint32_t xp[16];
     pack_x(x, xp);

@@ -109,3 +109,4 @@ extern "C" int sl_selftest_math(int op, const float* x_host, float* y_host, int6
   (void)hipFree(dx); (void)hipFree(dy);
   return rc;
 }
+

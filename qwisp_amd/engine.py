@@ -101,6 +101,10 @@ class SeedlessFusedForward:
     def last_gpu_ms(self):
         return self.lib.dll.sl_last_gpu_ms(self.h)
 
+    def set_hybrid(self, enable=True):
+        """forwardRowsHybrid (SeedlessFusedVerify.swift:4247): prefill chunks of >= 16 rows on the matrix cores."""
+        self.lib.check(self.lib.dll.sl_set_hybrid(self.h, 1 if enable else 0), "sl_set_hybrid", self.gpu_fault)
+
     def set_persistent(self, enable=True):
         return self.lib.dll.sl_set_persistent(self.h, int(enable)) == abi.SL_OK
 

@@ -63,10 +63,12 @@ SIGNATURES = {
     "sl_last_gpu_ms": (_f32, [_vp]),
     "sl_stream": (_vp, [_vp]),
     "sl_set_persistent": (_i32, [_vp, _i32]),
+    "sl_set_hybrid": (_i32, [_vp, _i32]),
     "sl_debug_stage_clock": (_i32, [_vp, _i32, _vp, _i32]),
     "sl_profile_head": (_i32, [_vp, _i32]),
     "sl_profile_head_read": (_i32, [_vp, C.POINTER(C.c_double), C.POINTER(_i64)]),
     "sl_selftest_math": (_i32, [_i32, _vp, _vp, _i64]),
+    "sl_selftest_qmm4": (_i32, [_vp, _i32, _vp, _vp, _vp, _i32, _i32, _vp]),
     "sl_synth_q4": (_i32, [_vp, _vp, _vp, _i64, _i32, _u64, _f32, _vp]),
     "sl_synth_f16": (_i32, [_vp, _i64, _u64, _f32, _f32, _vp]),
     "sl_synth_f32": (_i32, [_vp, _i64, _u64, _f32, _f32, _vp]),
