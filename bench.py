@@ -51,6 +51,9 @@ def main():
     ap.add_argument("--cpu-tokens", type=int, default=4, help="decode tokens timed on the CPU oracle (0 = skip)")
     ap.add_argument("--lanes", type=int, default=0, metavar="B",
                     help="also time B lanes stepped as one batch of rows on the same weights (extra object in the JSON line)")
+    ap.add_argument("--prefill-chunk", type=int, default=0, metavar="M",
+                    help="also time the 512-token prefill in chunks of M rows, exact rows and hybrid (matrix cores), on lanes "
+                         "of the same weights (extra object in the JSON line)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run a plain device copy of this many MiB (reference for rocprofv3 FETCH_SIZE/WRITE_SIZE) and exit")
     args = ap.parse_args()
@@ -151,6 +154,23 @@ def main():
         for lane in lanes:
             lane.close()
 
+    prefill_report = None
+    if args.prefill_chunk > 0:
+        prefill_report = {"prompt": PROMPT_LEN, "chunk_rows": args.prefill_chunk}
+        for name, hyb in (("exact_rows", False), ("hybrid_matrix_cores", True)):
+            times = []
+            for rep in range(2):                           # the first pass warms code and caches
+                lane = eng.new_lane(max_m=args.prefill_chunk, max_seq_len=PROMPT_LEN + 8)
+                lane.set_hybrid(hyb)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                o = lane.greedy_generate(prompt, 1, chain_k=1)
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                assert o is not None, lane.gpu_fault
+                lane.close()
+            prefill_report[name] = {"ms": times[-1] * 1e3, "tok_s": PROMPT_LEN / times[-1]}
+
     cpu = None
     if host is not None:
         from oracle import orc
@@ -181,6 +201,7 @@ def main():
         "step_hbm": {"bytes_per_token": total_b, "achieved_GBs": step_gbs, "frac_of_peak": step_gbs / HBM_PEAK_GBS},
         "cpu_baseline": cpu,
         "lane_batch": lanes_report,
+        "prefill": prefill_report,
         "setup_s": {"generate": t_gen, "prefill_512": t_prefill},
         "tokens_head": stream[:8],
     }))

@@ -328,9 +328,10 @@ void* sl_stream(sl_engine* e);
  * compute units (the reference's counterpart is the one-command-buffer step, SFV:3881-3890);
  * 0 switches to the kernel-per-stage sequence used for M > 1.  Both give identical results. */
 int sl_set_persistent(sl_engine* e, int enable);
-/* forwardRowsHybrid (SeedlessFusedVerify.swift:4240-4247): while enabled, calls with 16 <= m <= 128 rows of one
+/* forwardRowsHybrid (SeedlessFusedVerify.swift:4240-4247): while enabled, calls with 16 <= m <= 512 rows of one
  * sequence (prefill chunks) compute the dense mixer projections (GDN in/out, attention q|k|v and o) on the matrix
- * cores, with weights dequantised to half.  Like the reference's matrix-unit prefill this is not bit-identical to
+ * cores, and the routed experts grouped by expert (steelMoEGather, SeedlessFusedVerify.swift:4174), with weights
+ * dequantised to half.  Like the reference's matrix-unit prefill this is not bit-identical to
  * the GEMV order (tolerance-level agreement) but deterministic and independent of how a prompt is chunked.
  * Decode steps, verify rows below 16 and lane batches are unaffected. */
 int sl_set_hybrid(sl_engine* e, int enable);
@@ -363,7 +364,7 @@ int sl_synth_f32(float* dst_dev, int64_t count, uint64_t seed, float mean, float
  * 6 1/sqrt(x/128 + 1e-6), 7 half(x*sigmoid(x)), 8 normal quantile. */
 int sl_selftest_math(int op, const float* x_host, float* y_host, int64_t n);
 /* Self-test of the matrix-core GEMM of the hybrid prefill (host arrays in and out): y[m, n] = half(sum_k x[m, k] *
- * half(s*q + b)) for 4-bit group-64 weights [n, k]; m <= 128, n % 32 == 0, k % 64 == 0. */
+ * half(s*q + b)) for 4-bit group-64 weights [n, k]; m <= 512, n % 32 == 0, k % 64 == 0. */
 int sl_selftest_qmm4(const uint16_t* x_host, int m, const uint32_t* w_host, const uint16_t* scales_host,
                      const uint16_t* biases_host, int n, int k, uint16_t* y_host);
 

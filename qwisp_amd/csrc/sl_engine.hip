@@ -276,7 +276,7 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   hipLaunchKernelGGL(k_moe_c, dim3(256, M), dim3(128), 0, e->stream, c);
 }
 // Hybrid prefill: chunks of at least 16 rows of one sequence take the dense mixer projections to the matrix cores.
-bool use_matrix_cores(const sl_engine* e, int M, const LaneRef* lanes) { return e->hybrid && !lanes && M >= 16 && M <= 128; }
+bool use_matrix_cores(const sl_engine* e, int M, const LaneRef* lanes) { return e->hybrid && !lanes && M >= 16 && M <= GROUP_CAP; }
 // `lanes` (null for rows of one sequence) = this layer's row of the lane table: row b of the batch is lane b's next token.
 void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs& ha, const LaneRef* lanes) {
   const bool mm = use_matrix_cores(e, M, lanes);
@@ -760,7 +760,7 @@ void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
 int sl_set_hybrid(sl_engine* e, int enable) {
   int r = guard(e); if (r) return r;
   if (enable && !e->hy_g) {
-    const size_t rows = (size_t)(e->max_m < 128 ? e->max_m : 128);
+    const size_t rows = (size_t)(e->max_m < GROUP_CAP ? e->max_m : GROUP_CAP);
     e->hy_g = dalloc<uint16_t>(e, rows * 8 * SL_MOE_I); e->hy_u = dalloc<uint16_t>(e, rows * 8 * SL_MOE_I);
     e->hy_d = dalloc<uint16_t>(e, rows * 8 * H);
     e->hy_sg = dalloc<uint16_t>(e, rows * SL_MOE_I); e->hy_su = dalloc<uint16_t>(e, rows * SL_MOE_I);
@@ -1202,7 +1202,7 @@ int sl_greedy_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_
 // Self-test of the matrix-core GEMM (sl_mfma.cuh): host arrays in and out, temporary device buffers.
 extern "C" int sl_selftest_qmm4(const uint16_t* x_host, int m, const uint32_t* w_host, const uint16_t* s_host,
                                 const uint16_t* b_host, int n, int k, uint16_t* y_host) {
-  if (!x_host || !w_host || !s_host || !b_host || !y_host || m < 1 || m > 128 || n < 32 || (n % 32) || k < 64 || (k % 64))
+  if (!x_host || !w_host || !s_host || !b_host || !y_host || m < 1 || m > 512 || n < 32 || (n % 32) || k < 64 || (k % 64))
     return SL_ERR_ARG;
   const size_t xb = (size_t)m * k * 2, wb = (size_t)n * (k / 8) * 4, gb = (size_t)n * (k / 64) * 4, yb = (size_t)m * n * 2;
   std::vector<uint32_t> sb((size_t)n * (k / 64));

@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma(QmmArgs a) {
 // SeedlessFusedVerify.swift:4174): the (row, slot) pairs that chose expert e are gathered, multiplied with that
 // expert's matrix once, and scattered back by pair.  Workgroup = (strip block, expert); experts nobody chose exit.
 // -------------------------------------------------------------------------------------------------
-constexpr int GROUP_CAP = 128;          // pairs per expert: an expert is chosen at most once per row, M <= 128
+constexpr int GROUP_CAP = 512;          // pairs per expert: an expert is chosen at most once per row, M <= 512
 
 struct QmmGroupArgs {
   const uint16_t* x;     // source rows, fp16
@@ -127,89 +127,92 @@ struct QmmGroupArgs {
 };
 
 __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
-  constexpr int MT = GROUP_CAP / 32;
+  constexpr int MT = 4;                                  // 32-row tiles per pass (an expert with more than 128 rows takes several passes)
   __shared__ __align__(16) uint16_t xs[2][MT * 32 * QMM_XS];
   const int e = blockIdx.y;
-  const int cnt = min(a.counts[e], GROUP_CAP);
-  if (cnt == 0) return;                                  // uniform for the workgroup
+  const int cnt_all = min(a.counts[e], GROUP_CAP);
+  if (cnt_all == 0) return;                              // uniform for the workgroup
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, hh = lane >> 5;
   const int n0 = (blockIdx.x * 4 + wave) * 32;
   const bool live = n0 < a.NE;
   const size_t wrow = (size_t)e * a.NE + (live ? n0 + col : 0);
   const int chunks = a.K / 64;
-  const int tiles = (cnt + 31) >> 5;
-  // the rows this thread stages (one per 32-row tile) and the pairs this lane's results belong to
-  int src[MT];
-#pragma unroll
-  for (int p = 0; p < MT; ++p) {
-    const int row = p * 32 + (tid >> 3);
-    src[p] = -1;
-    if (row < cnt) { const int pr = a.lists[e * GROUP_CAP + row]; src[p] = a.x_by_pair ? pr : (pr >> 3); }
-  }
-  mf_f16v acc[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
-  uint4 xr[MT];
-  auto fetch = [&](int c) {
+  for (int r0 = 0; r0 < cnt_all; r0 += MT * 32) {
+    const int cnt = min(cnt_all - r0, MT * 32);
+    const int tiles = (cnt + 31) >> 5;
+    const uint16_t* list = a.lists + (size_t)e * GROUP_CAP + r0;
+    // the rows this thread stages (one per 32-row tile)
+    int src[MT];
 #pragma unroll
     for (int p = 0; p < MT; ++p) {
-      xr[p] = make_uint4(0, 0, 0, 0);
-      if (p < tiles && src[p] >= 0) xr[p] = ld16(a.x + (size_t)src[p] * a.x_stride + c * 64 + (tid & 7) * 8);
+      const int row = p * 32 + (tid >> 3);
+      src[p] = -1;
+      if (row < cnt) { const int pr = list[row]; src[p] = a.x_by_pair ? pr : (pr >> 3); }
     }
-  };
-  auto put = [&](int buf) {
+    mf_f16v acc[MT];
 #pragma unroll
-    for (int p = 0; p < MT; ++p)
-      if (p < tiles) st16(&xs[buf][(p * 32 + (tid >> 3)) * QMM_XS + (tid & 7) * 8], xr[p]);
-  };
-  fetch(0);
-  put(0);
-  if (chunks > 1) fetch(1);
-  uint4 nw0 = make_uint4(0, 0, 0, 0), nw1 = make_uint4(0, 0, 0, 0);
-  uint32_t nsb = 0;
-  if (live) { nw0 = ld16(a.W + wrow * (a.K / 8)); nw1 = ld16(a.W + wrow * (a.K / 8) + 4); nsb = a.SB[wrow * (a.K / 64)]; }
-  for (int c = 0; c < chunks; ++c) {
-    const int buf = c & 1;
-    const uint4 w0 = nw0, w1 = nw1;
-    const uint32_t sb = nsb;
-    if (live && c + 1 < chunks) {
-      nw0 = ld16(a.W + wrow * (a.K / 8) + (c + 1) * 8);
-      nw1 = ld16(a.W + wrow * (a.K / 8) + (c + 1) * 8 + 4);
-      nsb = a.SB[wrow * (a.K / 64) + c + 1];
-    }
-    __syncthreads();
-    if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
-    const float s = lo_h(sb), b = hi_h(sb);
-    const uint32_t words[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+    for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int st = 0; st < 8; ++st) {
-      const uint32_t q4 = words[st] >> (16 * hh);
-      mf_h4 bw;
+      for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
+    uint4 xr[MT];
+    auto fetch = [&](int c) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) bw[i] = (_Float16)fmaf(s, (float)((q4 >> (4 * i)) & 15u), b);
+      for (int p = 0; p < MT; ++p) {
+        xr[p] = make_uint4(0, 0, 0, 0);
+        if (p < tiles && src[p] >= 0) xr[p] = ld16(a.x + (size_t)src[p] * a.x_stride + c * 64 + (tid & 7) * 8);
+      }
+    };
+    auto put = [&](int buf) {
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        if (t < tiles) {
-          const mf_h4 ax = *reinterpret_cast<const mf_h4*>(&xs[buf][(t * 32 + col) * QMM_XS + 8 * st + 4 * hh]);
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x8f16(ax, bw, acc[t], 0, 0, 0);
+      for (int p = 0; p < MT; ++p)
+        if (p < tiles) st16(&xs[buf][(p * 32 + (tid >> 3)) * QMM_XS + (tid & 7) * 8], xr[p]);
+    };
+    __syncthreads();                                     // the pass before has finished reading the staging buffers
+    fetch(0);
+    put(0);
+    if (chunks > 1) fetch(1);
+    uint4 nw0 = make_uint4(0, 0, 0, 0), nw1 = make_uint4(0, 0, 0, 0);
+    uint32_t nsb = 0;
+    if (live) { nw0 = ld16(a.W + wrow * (a.K / 8)); nw1 = ld16(a.W + wrow * (a.K / 8) + 4); nsb = a.SB[wrow * (a.K / 64)]; }
+    for (int c = 0; c < chunks; ++c) {
+      const int buf = c & 1;
+      const uint4 w0 = nw0, w1 = nw1;
+      const uint32_t sb = nsb;
+      if (live && c + 1 < chunks) {
+        nw0 = ld16(a.W + wrow * (a.K / 8) + (c + 1) * 8);
+        nw1 = ld16(a.W + wrow * (a.K / 8) + (c + 1) * 8 + 4);
+        nsb = a.SB[wrow * (a.K / 64) + c + 1];
+      }
+      __syncthreads();
+      if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
+      const float s = lo_h(sb), b = hi_h(sb);
+      const uint32_t words[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+      for (int st = 0; st < 8; ++st) {
+        const uint32_t q4 = words[st] >> (16 * hh);
+        mf_h4 bw;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bw[i] = (_Float16)fmaf(s, (float)((q4 >> (4 * i)) & 15u), b);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          if (t < tiles) {
+            const mf_h4 ax = *reinterpret_cast<const mf_h4*>(&xs[buf][(t * 32 + col) * QMM_XS + 8 * st + 4 * hh]);
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x8f16(ax, bw, acc[t], 0, 0, 0);
+          }
         }
       }
     }
-  }
-  if (!live) return;
+    if (live) {
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
+      for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-      if (row < cnt) {
-        const int pr = a.lists[e * GROUP_CAP + row];
-        a.y[(size_t)pr * a.y_stride + n0 + col] = f2h(acc[t][r]);
-      }
+        for (int r = 0; r < 16; ++r) {
+          const int row = t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+          if (row < cnt) a.y[(size_t)list[row] * a.y_stride + n0 + col] = f2h(acc[t][r]);
+        }
     }
+  }
 }
 
 // Routing of M rows on its own (the GEMV path routes inside its gate/up kernel): one wave per row.
@@ -222,15 +225,14 @@ __global__ __launch_bounds__(64) void k_route_rows(const uint16_t* __restrict__ 
   __syncthreads();
   if (lane < 8) { inds[m * 8 + lane] = s_inds[lane]; scores[m * 8 + lane] = f2h(s_sc[lane]); }
 }
-// Pairs (row, slot) listed per expert: one thread per pair (M * 8 <= 1024), places handed out by LDS counters.
+// Pairs (row, slot) listed per expert (M * 8 <= 4096 pairs over 1024 threads), places handed out by LDS counters.
 // The order within a list varies from run to run; results do not depend on it (they are scattered back by pair).
 __global__ __launch_bounds__(1024) void k_group_pairs(const int32_t* __restrict__ inds, int M, int E, uint16_t* __restrict__ lists,
                                                       int32_t* __restrict__ counts) {
   __shared__ int s_cnt[SL_MAX_EXPERTS];
-  const int p = threadIdx.x;
-  if (p < SL_MAX_EXPERTS) s_cnt[p] = 0;
+  if (threadIdx.x < SL_MAX_EXPERTS) s_cnt[threadIdx.x] = 0;
   __syncthreads();
-  if (p < M * 8) {
+  for (int p = threadIdx.x; p < M * 8; p += 1024) {
     const int e = inds[p];
     if (e >= 0 && e < E) {
       const int pos = atomicAdd(&s_cnt[e], 1);
@@ -238,7 +240,7 @@ __global__ __launch_bounds__(1024) void k_group_pairs(const int32_t* __restrict_
     }
   }
   __syncthreads();
-  if (p < E) counts[p] = s_cnt[p];
+  if ((int)threadIdx.x < E) counts[threadIdx.x] = s_cnt[threadIdx.x];
 }
 // act = half(silu(g) * u) in half arithmetic, elementwise over [rows, 512] (same rule as the GEMV kernels).
 __global__ __launch_bounds__(256) void k_swiglu_rows(const uint16_t* __restrict__ g, const uint16_t* __restrict__ u,
@@ -259,13 +261,19 @@ __global__ __launch_bounds__(256) void k_moe_combine_rows(const uint16_t* __rest
   out[(size_t)m * H + n] = f2h(f16r(acc + f16r(s * h2f(sy[(size_t)m * H + n]))));
 }
 
-// Host-side launch: picks the row-tile count for M (<= 128 rows per launch).
-inline void launch_qmm4_mfma(const QmmArgs& a, hipStream_t stream) {
-  const int strips = a.N / 32;
+// Host-side launch: picks the row-tile count per block of up to 128 rows.
+inline void launch_qmm4_mfma(const QmmArgs& all, hipStream_t stream) {
+  const int strips = all.N / 32;
   const dim3 block(256);
-  if (a.M <= 32) hipLaunchKernelGGL(k_qmm4_mfma<1>, dim3((unsigned)((strips + 3) / 4)), block, 0, stream, a);
-  else if (a.M <= 64) hipLaunchKernelGGL(k_qmm4_mfma<2>, dim3((unsigned)((strips + 1) / 2)), block, 0, stream, a);
-  else hipLaunchKernelGGL(k_qmm4_mfma<4>, dim3((unsigned)strips), block, 0, stream, a);
+  for (int r0 = 0; r0 < all.M; r0 += 128) {             // the kernel takes up to 128 rows: longer chunks go in blocks
+    QmmArgs a = all;
+    a.x = all.x + (size_t)r0 * all.x_stride;
+    a.y = all.y + (size_t)r0 * all.y_stride;
+    a.M = all.M - r0 < 128 ? all.M - r0 : 128;
+    if (a.M <= 32) hipLaunchKernelGGL(k_qmm4_mfma<1>, dim3((unsigned)((strips + 3) / 4)), block, 0, stream, a);
+    else if (a.M <= 64) hipLaunchKernelGGL(k_qmm4_mfma<2>, dim3((unsigned)((strips + 1) / 2)), block, 0, stream, a);
+    else hipLaunchKernelGGL(k_qmm4_mfma<4>, dim3((unsigned)strips), block, 0, stream, a);
+  }
 }
 
 }  // namespace sl

@@ -71,7 +71,7 @@ def test_generator_device_equals_host(env):
 
 # ---- matrix-core GEMM of the hybrid prefill ---------------------------------------------------------
 @pytest.mark.gpu
-@pytest.mark.parametrize("m,n,k", [(1, 32, 64), (5, 96, 512), (32, 128, 2048), (33, 160, 2048), (64, 2048, 4096), (100, 64, 512)])
+@pytest.mark.parametrize("m,n,k", [(1, 32, 64), (5, 96, 512), (32, 128, 2048), (33, 160, 2048), (64, 2048, 4096), (100, 64, 512), (300, 96, 512)])
 def test_mfma_qmm4_against_the_oracle_rows(env, m, n, k):
     """Y = X W^T with 4-bit weights on the matrix cores.  Not bit-identical to the GEMV order (the reference
     says the same of its matrix-unit prefill, SeedlessFusedVerify.swift:4244): within the error of weights
@@ -124,6 +124,18 @@ def test_hybrid_prefill_agrees_with_the_exact_rows(env, small_model):
     # chunking does not change a row: 48 rows at once against 16 + 32
     c1 = hyb2.forward_tokens(toks[:16]); c2 = hyb2.forward_tokens(toks[16:])
     assert same_bits(np.concatenate([c1, c2]), b)
+    # a chunk longer than 128 rows (several row blocks per GEMM, experts with many rows) gives the same rows again
+    big = env["Engine"](cfg, dev, max_m=192, max_seq_len=256)
+    big.set_hybrid(True)
+    toks2 = np.concatenate([toks, np.random.default_rng(13).integers(0, cfg.vocab, 112).astype(np.int32)])
+    d1 = big.forward_tokens(toks2)
+    assert d1 is not None, big.gpu_fault
+    assert same_bits(d1[:48], b)
+    ex2 = env["Engine"](cfg, dev, max_m=192, max_seq_len=256)
+    d0 = ex2.forward_tokens(toks2)
+    rel2 = np.linalg.norm(d0.astype(np.float64) - d1.astype(np.float64), axis=1) / np.linalg.norm(d0.astype(np.float64), axis=1)
+    assert np.median(rel2) < 0.02 and rel2.max() < 0.15, (np.median(rel2), rel2.max())
+    big.close(); ex2.close()
     # decode goes on from the hybrid caches (single-launch step), close to the exact stream's logits
     t0 = int(exact.head_argmax(a[-1:])[0])
     sa, sb = exact.step_argmax([t0]), hyb.step_argmax([t0])
