@@ -74,6 +74,8 @@ struct sl_engine {
   uint16_t *rlogits = nullptr, *sgate = nullptr, *sh_act = nullptr, *act = nullptr, *moe_out = nullptr, *normed = nullptr;
   uint16_t *logits = nullptr, *rows_out = nullptr;
   float *pm = nullptr, *pl = nullptr, *po = nullptr, *cand_v = nullptr;
+  uint16_t *gdn_qn = nullptr, *gdn_kn = nullptr, *gdn_vc = nullptr;   // per-row inputs of the GDN scan (M >= 2 rows)
+  float* gdn_gb = nullptr;
   int32_t *cand_i = nullptr, *tok_in = nullptr, *tok_out = nullptr, *st = nullptr;
   int n_cand = 0;
   // persistent single-token kernel
@@ -293,7 +295,14 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
   g.hist[0] = L.hist[0]; g.hist[1] = L.hist[1]; g.state[0] = L.state[0]; g.state[1] = L.state[1];
   g.st = e->st + li;       // st[1] of this view = parity of layer li
   g.ycore = e->ycore; g.M = M; g.lanes = lanes; g.layer = li;
-  hipLaunchKernelGGL(k_gdn_core, dim3(256, lanes ? M : 1), dim3(256), 0, e->stream, g);
+  if (!lanes && M >= 2) {
+    // rows of one sequence: the state-independent part for all rows at once, then the scan without barriers
+    GdnPrepArgs pa{g, e->gdn_qn, e->gdn_kn, e->gdn_vc, e->gdn_gb};
+    hipLaunchKernelGGL(k_gdn_prep_rows, dim3(65, M), dim3(64), 0, e->stream, pa);
+    hipLaunchKernelGGL(k_gdn_scan_rows, dim3(256), dim3(256), 0, e->stream, pa);
+  } else {
+    hipLaunchKernelGGL(k_gdn_core, dim3(256, lanes ? M : 1), dim3(256), 0, e->stream, g);
+  }
   if (mm) {
     hipLaunchKernelGGL(k_gdn_gate_rows, dim3(SL_GDN_HV, M), dim3(64), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32);
     launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.out_proj.w, L.out_proj.sb, M, H, 4096, e->mix, H}, e->stream);
@@ -552,6 +561,9 @@ int alloc_runtime(sl_engine* e) {
   e->sh_act = dalloc<uint16_t>(e, (size_t)max_m * 512, true); e->act = dalloc<uint16_t>(e, (size_t)max_m * 8 * 512, true);
   e->moe_out = dalloc<uint16_t>(e, MH, true); e->normed = dalloc<uint16_t>(e, MH, true);
   e->rows_out = dalloc<uint16_t>(e, MH, true);
+  e->gdn_qn = dalloc<uint16_t>(e, MH, true); e->gdn_kn = dalloc<uint16_t>(e, MH, true);
+  e->gdn_vc = dalloc<uint16_t>(e, (size_t)max_m * 4096, true); e->gdn_gb = dalloc<float>(e, (size_t)max_m * 64, true);
+  if (!e->gdn_qn || !e->gdn_kn || !e->gdn_vc || !e->gdn_gb) return SL_ERR_DEVICE;
   e->tok_in = dalloc<int32_t>(e, max_m, true);
   e->tok_out = dalloc<int32_t>(e, max_m > MAX_CHAIN ? max_m : MAX_CHAIN, true);
   e->st = dalloc<int32_t>(e, 1 + d->n_layers, true);

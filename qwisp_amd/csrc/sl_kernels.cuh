@@ -303,6 +303,114 @@ __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
 }
 
 // -------------------------------------------------------------------------------------------------
+// The same layer for M >= 2 rows in two kernels with the same arithmetic.  Everything that does not depend on the
+// recurrent state (conv + silu, q/k norms, decay and beta) is formed for all rows at once (k_gdn_prep_rows);
+// the recurrence itself then streams through the rows without a barrier (k_gdn_scan_rows), the next row's inputs
+// being requested while the current row is worked on.
+// -------------------------------------------------------------------------------------------------
+struct GdnPrepArgs {
+  GdnArgs g;                 // proj, conv_w, a_log, dt_bias, hist, st, M as above
+  uint16_t *qn, *kn;         // [M, 2048] normed, scaled query / key (half values)
+  uint16_t* vc;              // [M, 4096] conv + silu of the value channels
+  float* gb;                 // [M, 64]: decay g of the 32 value heads, then beta
+};
+// One wave per (unit, row): units 0..15 query heads, 16..31 key heads, 32..63 value heads, 64 decay / beta.
+__global__ __launch_bounds__(64) void k_gdn_prep_rows(GdnPrepArgs p) {
+  const GdnArgs& a = p.g;
+  const int u = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+  const uint16_t* hin = a.hist[a.st[1]];
+  if (u < 32) {
+    const bool isk = u >= 16;
+    const int ch = (isk ? 2048 : 0) + (u & 15) * 128 + 2 * lane;
+    const float x0 = conv_silu(a, hin, t, ch), x1 = conv_silu(a, hin, t, ch + 1);
+    float ss = fmaf(x1, x1, fmaf(x0, x0, 0.0f));
+    ss = tree_sum<64>(ss);
+    const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
+    const float sc = isk ? f16r(0.08838834764831845f) : f16r(0.0078125f);
+    const float y0 = f16r(sc * f16r(x0 * inv)), y1 = f16r(sc * f16r(x1 * inv));
+    *reinterpret_cast<uint32_t*>((isk ? p.kn : p.qn) + (size_t)t * 2048 + (u & 15) * 128 + 2 * lane) = pack2(y0, y1);
+  } else if (u < 64) {
+    const int ch = 4096 + (u - 32) * 128 + 2 * lane;
+    *reinterpret_cast<uint32_t*>(p.vc + (size_t)t * 4096 + (u - 32) * 128 + 2 * lane) =
+        pack2(conv_silu(a, hin, t, ch), conv_silu(a, hin, t, ch + 1));
+  } else {
+    const int hv = lane & 31;
+    if (lane < 32) {
+      const float aP = h2f(a.proj[(size_t)t * PROJ_STRIDE + 12320 + hv]);
+      p.gb[(size_t)t * 64 + hv] = exp_c(-(exp_c(a.a_log[hv]) * softplus_c(aP + a.dt_bias[hv])));
+    } else {
+      p.gb[(size_t)t * 64 + 32 + hv] = sigmoid16(h2f(a.proj[(size_t)t * PROJ_STRIDE + 12288 + hv]));
+    }
+  }
+}
+// The recurrence over the rows: workgroup = (value head, block of 16 dv), thread layout and arithmetic of
+// k_gdn_core.  Also shifts the conv history.
+__global__ __launch_bounds__(256) void k_gdn_scan_rows(GdnPrepArgs p) {
+  const GdnArgs& a = p.g;
+  const int hv = blockIdx.x >> 3, dvb = blockIdx.x & 7, hk = hv >> 1;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+  const int par = a.st[1];
+  const uint16_t* hin = a.hist[par];
+  uint16_t* hout = a.hist[par ^ 1];
+  const float* sin_ = a.state[par];
+  float* sout = a.state[par ^ 1];
+  float s[2][4];
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int dv = dvb * 16 + wave * 4 + it * 2 + half;
+    const float4 v = *reinterpret_cast<const float4*>(sin_ + ((size_t)hv * 128 + dv) * 128 + 4 * l32);
+    s[it][0] = v.x; s[it][1] = v.y; s[it][2] = v.z; s[it][3] = v.w;
+  }
+  struct Row { uint2 k, q; uint16_t v[2]; float g, beta; };
+  auto fetch = [&](int t) {
+    Row r;
+    r.k = *reinterpret_cast<const uint2*>(p.kn + (size_t)t * 2048 + hk * 128 + 4 * l32);
+    r.q = *reinterpret_cast<const uint2*>(p.qn + (size_t)t * 2048 + hk * 128 + 4 * l32);
+#pragma unroll
+    for (int it = 0; it < 2; ++it) r.v[it] = p.vc[(size_t)t * 4096 + hv * 128 + dvb * 16 + wave * 4 + it * 2 + half];
+    r.g = p.gb[(size_t)t * 64 + hv]; r.beta = p.gb[(size_t)t * 64 + 32 + hv];
+    return r;
+  };
+  Row nxt = fetch(0);
+  for (int t = 0; t < a.M; ++t) {
+    const Row cur = nxt;
+    if (t + 1 < a.M) nxt = fetch(t + 1);
+    const float kk[4] = {lo_h(cur.k.x), hi_h(cur.k.x), lo_h(cur.k.y), hi_h(cur.k.y)};
+    const float qq[4] = {lo_h(cur.q.x), hi_h(cur.q.x), lo_h(cur.q.y), hi_h(cur.q.y)};
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int dvl = wave * 4 + it * 2 + half;
+      float acc = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { s[it][i] = s[it][i] * cur.g; acc = fmaf(s[it][i], kk[i], acc); }
+      const float kv = tree_sum<32>(acc);
+      const float delta = (h2f(cur.v[it]) - kv) * cur.beta;
+      acc = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { s[it][i] = fmaf(kk[i], delta, s[it][i]); acc = fmaf(s[it][i], qq[i], acc); }
+      const float y = tree_sum<32>(acc);
+      if (l32 == 0) a.ycore[(size_t)t * 4096 + hv * 128 + dvb * 16 + dvl] = f2h(y);
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int dv = dvb * 16 + wave * 4 + it * 2 + half;
+    *reinterpret_cast<float4*>(sout + ((size_t)hv * 128 + dv) * 128 + 4 * l32) = make_float4(s[it][0], s[it][1], s[it][2], s[it][3]);
+  }
+  // history shift: rows M..M+2 of [hist | qkv]; each channel written by exactly one workgroup
+  const int qk_ch = (tid < 128) ? (hk * 128 + tid) : (2048 + hk * 128 + (tid - 128));
+  const int v_ch = 4096 + hv * 128 + dvb * 16 + (tid & 15);
+  if ((hv & 1) == 0 && dvb == 0) {
+#pragma unroll
+    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + qk_ch] = f2h(conv_tap(a, hin, a.M + j, qk_ch));
+  }
+  if (tid < 16) {
+#pragma unroll
+    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + v_ch] = f2h(conv_tap(a, hin, a.M + j, v_ch));
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
 // GDN out-proj with the gated rmsnorm as prologue: x = half(silu(z) * half(w * half(y*inv))) per value
 // head (with an fp32 norm weight: half(silu(z) * (w * (y*inv)))), then the K = 4096 4-bit dot.  Reference: gdn_norm_gate_rows SeedlessFusedVerify.swift:768-812.
 // -------------------------------------------------------------------------------------------------
