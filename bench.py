@@ -23,7 +23,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 PROMPT_LEN = 512
 # HBM bytes per k_decode_flow launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/), or None until measured
-TRAFFIC_BYTES_PER_LAUNCH = 1936707441   # 2 x FETCH_SIZE (copy-calibrated) + WRITE_SIZE, in bytes, at context ~525
+TRAFFIC_BYTES_PER_LAUNCH = 1936711864   # 2 x FETCH_SIZE (copy-calibrated) + WRITE_SIZE, in bytes, at context ~525
 
 
 def step_bytes(cfg, ctx):
