@@ -396,6 +396,29 @@ def test_persistent_step_long_context(env, small_model):
             assert same_bits(x, y), (li, first_diff(x, y))
 
 
+def test_persistent_step_across_the_attention_split_boundary(env, small_model):
+    """Up to 2048 tokens of context an attention tile unit is split four ways over the query heads, beyond that
+    it is not; the merge polls 12 tiles per round trip.  Steps that cross position 2048 (and the 13th tile at
+    768) on the single-launch path equal the kernel-per-stage sequence."""
+    cfg, dev, host = small_model
+    for n_prefill in (760, 2040):
+        a = env["Engine"](cfg, dev, max_m=64, max_seq_len=2200)
+        b = env["Engine"](cfg, dev, max_m=64, max_seq_len=2200)
+        assert b.set_persistent(False)
+        toks = np.random.default_rng(78).integers(0, cfg.vocab, n_prefill).astype(np.int32)
+        for eng in (a, b):
+            for i in range(0, len(toks), 64):
+                assert eng.step_argmax(toks[i:i + 64]) is not None, eng.gpu_fault
+        ta, tb = a.chained_step_argmax(5, 16), b.chained_step_argmax(5, 16)
+        assert ta is not None and tb is not None, (a.gpu_fault, b.gpu_fault)
+        assert ta.tolist() == tb.tolist(), n_prefill
+        assert same_bits(a.logits_row(0), b.logits_row(0))
+        for li in range(cfg.n_layers):
+            for x, y in zip(a.read_layer_cache(li), b.read_layer_cache(li)):
+                assert same_bits(x, y), (n_prefill, li, first_diff(x, y))
+        a.close(); b.close()
+
+
 def test_lanes_share_weights_and_equal_solo(env, small_model):
     """Lanes (SeedlessLaneBatch.swift:876): sequences on one weight set.  Per lane the token stream is that
     of a solo engine, whatever the other lanes do; sampling is reported as unsupported.  Three lanes fit the
