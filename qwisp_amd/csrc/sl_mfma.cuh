@@ -3,7 +3,7 @@
 // SeedlessFusedVerify.swift:4240-4247).
 //
 //   Y[m, n] = half( sum_k X[m, k] * half(s * q + b) ),  X fp16 [M, K], W MLX-affine 4-bit group 64 [N, K],
-//   fp32 accumulation in v_mfma_f32_32x32x8_f16.
+//   the weight formed in half arithmetic (one fused multiply-add), fp32 accumulation in v_mfma_f32_32x32x8_f16.
 //
 // A wave owns a 32x32 tile of Y (32 rows of X against 32 weight rows): it walks K in chunks of 64 (one
 // quantisation group), dequantises its 4 weights per MFMA step in registers and feeds them as the B operand;
@@ -20,6 +20,27 @@ namespace sl {
 
 typedef _Float16 mf_h4 __attribute__((ext_vector_type(4)));
 typedef float mf_f16v __attribute__((ext_vector_type(16)));
+typedef _Float16 mf_h2 __attribute__((ext_vector_type(2)));
+
+// Dequantisation of a lane's 4 weights of an MFMA step in packed half arithmetic.  `wsh` holds two nibble pairs
+// (bits 0-7 and 16-23).  or-ing a nibble into the mantissa of 1024.0 gives 1024 + q exactly, subtracting 1024
+// gives q exactly, and half(q * s + b) is one fused multiply-add per pair.  The four results belong to the
+// nibbles {a, a+4, a+1, a+5} of the word (a = 0 or 2), which is the order the X chunk is staged in.
+SL_DEV mf_h4 dequant4(uint32_t wsh, mf_h2 s2, mf_h2 b2) {
+  const mf_h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+  const mf_h2 q0 = __builtin_bit_cast(mf_h2, (wsh & 0x000F000Fu) | 0x64006400u) - k1024;
+  const mf_h2 q1 = __builtin_bit_cast(mf_h2, ((wsh >> 4) & 0x000F000Fu) | 0x64006400u) - k1024;
+  const mf_h2 w0 = __builtin_elementwise_fma(q0, s2, b2), w1 = __builtin_elementwise_fma(q1, s2, b2);
+  mf_h4 r;
+  r[0] = w0[0]; r[1] = w0[1]; r[2] = w1[0]; r[3] = w1[1];
+  return r;
+}
+// The 8 halves of a staged 16-byte piece (k = 8j .. 8j+7) in the order {0,4,1,5, 2,6,3,7}: positions 0-3 are read
+// by the lanes of the lower half-wave, 4-7 by the upper, matching dequant4.
+SL_DEV uint4 permute8(uint4 v) {
+  return make_uint4((v.x & 0xffffu) | (v.z << 16), (v.x >> 16) | (v.z & 0xffff0000u),
+                    (v.y & 0xffffu) | (v.w << 16), (v.y >> 16) | (v.w & 0xffff0000u));
+}
 
 struct QmmArgs {
   const uint16_t* x;     // [M, x_stride] fp16
@@ -63,7 +84,7 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma(QmmArgs a) {
   };
   auto put = [&](int buf) {
 #pragma unroll
-    for (int p = 0; p < WM; ++p) st16(&xs[buf][(p * 32 + (tid >> 3)) * QMM_XS + (tid & 7) * 8], xr[p]);
+    for (int p = 0; p < WM; ++p) st16(&xs[buf][(p * 32 + (tid >> 3)) * QMM_XS + (tid & 7) * 8], permute8(xr[p]));
   };
   fetch(0);
   put(0);
@@ -84,15 +105,12 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma(QmmArgs a) {
     __syncthreads();                                     // chunk c is staged; chunk c-1 is no longer read
     if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
     if (!live) continue;
-    const float s = lo_h(sb), b = hi_h(sb);
+    const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb >> 16) * 0x10001u);
     const uint32_t words[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
     for (int st = 0; st < 8; ++st) {
-      // this lane's 4 weights of the step: nibbles 4*hh .. 4*hh+3 of word st, k = 8*st + 4*hh + i
-      const uint32_t q4 = words[st] >> (16 * hh);
-      mf_h4 bw;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) bw[i] = (_Float16)fmaf(s, (float)((q4 >> (4 * i)) & 15u), b);
+      // this lane's 4 weights of the step: nibbles {a, a+4, a+1, a+5} of word st with a = 2*hh
+      const mf_h4 bw = dequant4(words[st] >> (8 * hh), s2, b2);
       const mf_h4 ax = *reinterpret_cast<const mf_h4*>(&xs[buf][(mt * 32 + col) * QMM_XS + 8 * st + 4 * hh]);
       acc = __builtin_amdgcn_mfma_f32_32x32x8f16(ax, bw, acc, 0, 0, 0);
     }
@@ -127,8 +145,9 @@ struct QmmGroupArgs {
 };
 
 __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
-  constexpr int MT = 4;                                  // 32-row tiles per pass (an expert with more than 128 rows takes several passes)
-  __shared__ __align__(16) uint16_t xs[2][MT * 32 * QMM_XS];
+  // One 32-row tile per pass and one accumulator per wave (most experts have fewer than 32 rows in a chunk; an
+  // expert with more takes several passes over its weights, which then come from cache).
+  __shared__ __align__(16) uint16_t xs[2][32 * QMM_XS];
   const int e = blockIdx.y;
   const int cnt_all = min(a.counts[e], GROUP_CAP);
   if (cnt_all == 0) return;                              // uniform for the workgroup
@@ -138,36 +157,21 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
   const bool live = n0 < a.NE;
   const size_t wrow = (size_t)e * a.NE + (live ? n0 + col : 0);
   const int chunks = a.K / 64;
-  for (int r0 = 0; r0 < cnt_all; r0 += MT * 32) {
-    const int cnt = min(cnt_all - r0, MT * 32);
-    const int tiles = (cnt + 31) >> 5;
+  for (int r0 = 0; r0 < cnt_all; r0 += 32) {
+    const int cnt = min(cnt_all - r0, 32);
     const uint16_t* list = a.lists + (size_t)e * GROUP_CAP + r0;
-    // the rows this thread stages (one per 32-row tile)
-    int src[MT];
+    // the row this thread stages
+    int src = -1;
+    if ((tid >> 3) < cnt) { const int pr = list[tid >> 3]; src = a.x_by_pair ? pr : (pr >> 3); }
+    mf_f16v acc;
 #pragma unroll
-    for (int p = 0; p < MT; ++p) {
-      const int row = p * 32 + (tid >> 3);
-      src[p] = -1;
-      if (row < cnt) { const int pr = list[row]; src[p] = a.x_by_pair ? pr : (pr >> 3); }
-    }
-    mf_f16v acc[MT];
-#pragma unroll
-    for (int t = 0; t < MT; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
-    uint4 xr[MT];
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    uint4 xr = make_uint4(0, 0, 0, 0);
     auto fetch = [&](int c) {
-#pragma unroll
-      for (int p = 0; p < MT; ++p) {
-        xr[p] = make_uint4(0, 0, 0, 0);
-        if (p < tiles && src[p] >= 0) xr[p] = ld16(a.x + (size_t)src[p] * a.x_stride + c * 64 + (tid & 7) * 8);
-      }
+      xr = make_uint4(0, 0, 0, 0);
+      if (src >= 0) xr = ld16(a.x + (size_t)src * a.x_stride + c * 64 + (tid & 7) * 8);
     };
-    auto put = [&](int buf) {
-#pragma unroll
-      for (int p = 0; p < MT; ++p)
-        if (p < tiles) st16(&xs[buf][(p * 32 + (tid >> 3)) * QMM_XS + (tid & 7) * 8], xr[p]);
-    };
+    auto put = [&](int buf) { st16(&xs[buf][(tid >> 3) * QMM_XS + (tid & 7) * 8], permute8(xr)); };
     __syncthreads();                                     // the pass before has finished reading the staging buffers
     fetch(0);
     put(0);
@@ -186,31 +190,21 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
       }
       __syncthreads();
       if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
-      const float s = lo_h(sb), b = hi_h(sb);
+      const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb >> 16) * 0x10001u);
       const uint32_t words[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
       for (int st = 0; st < 8; ++st) {
-        const uint32_t q4 = words[st] >> (16 * hh);
-        mf_h4 bw;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) bw[i] = (_Float16)fmaf(s, (float)((q4 >> (4 * i)) & 15u), b);
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-          if (t < tiles) {
-            const mf_h4 ax = *reinterpret_cast<const mf_h4*>(&xs[buf][(t * 32 + col) * QMM_XS + 8 * st + 4 * hh]);
-            acc[t] = __builtin_amdgcn_mfma_f32_32x32x8f16(ax, bw, acc[t], 0, 0, 0);
-          }
-        }
+        const mf_h4 bw = dequant4(words[st] >> (8 * hh), s2, b2);
+        const mf_h4 ax = *reinterpret_cast<const mf_h4*>(&xs[buf][col * QMM_XS + 8 * st + 4 * hh]);
+        acc = __builtin_amdgcn_mfma_f32_32x32x8f16(ax, bw, acc, 0, 0, 0);
       }
     }
     if (live) {
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-          if (row < cnt) a.y[(size_t)list[row] * a.y_stride + n0 + col] = f2h(acc[t][r]);
-        }
+      for (int r = 0; r < 16; ++r) {
+        const int row = 8 * (r >> 2) + 4 * hh + (r & 3);
+        if (row < cnt) a.y[(size_t)list[row] * a.y_stride + n0 + col] = f2h(acc[r]);
+      }
     }
   }
 }
