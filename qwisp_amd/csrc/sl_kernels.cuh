@@ -495,7 +495,7 @@ struct MoeAArgs {
   const uint16_t* sgate_w;                           // [2048]
   const uint32_t *g8_w, *g8_sb;                      // 8-bit gates instead (null: fp16): [E+1, 512] words, [E+1, 32] {scale, bias}; row E = shared gate
   int E;
-  int skip_shared;                                   // hybrid prefill: the shared expert's gate/up run on the matrix cores
+  int skip_shared;                                   // hybrid prefill: the shared expert's gate/up run on the matrix cores; grid.x = router blocks only
   uint16_t* sh_act;                                  // [M, 512]
   uint16_t* rlogits;                                 // [M, 256]
   uint16_t* sgate;                                   // [M]
@@ -505,12 +505,13 @@ __global__ __launch_bounds__(256) void k_moe_a(MoeAArgs a) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float x[32], sx[4];
   hidden_prologue(a.ha, m, lane, blockIdx.x == 0 && wave == 0, x);
-  if (blockIdx.x < MOE_A_SHARED_BLOCKS) {
-    if (a.skip_shared) return;
+  // skip_shared: the grid holds the router blocks only
+  const int bx = a.skip_shared ? (int)blockIdx.x + MOE_A_SHARED_BLOCKS : (int)blockIdx.x;
+  if (bx < MOE_A_SHARED_BLOCKS) {
     word_sums(x, sx);
     uint32_t xp[16];
     pack_x(x, xp);
-    const size_t i0 = ((size_t)blockIdx.x * 4 + wave) * 2;
+    const size_t i0 = ((size_t)bx * 4 + wave) * 2;
     const size_t rows[2] = {i0, i0 + 1};
     float g[2], u[2];
     qdot_rows<1, 2>(a.shg_w, a.shg_sb, rows, lane, xp, sx, g);
@@ -520,7 +521,7 @@ __global__ __launch_bounds__(256) void k_moe_a(MoeAArgs a) {
       for (int r = 0; r < 2; ++r) a.sh_act[(size_t)m * 512 + i0 + r] = f2h(swiglu16(f16r(g[r]), f16r(u[r])));
     }
   } else {
-    const int row0 = ((blockIdx.x - MOE_A_SHARED_BLOCKS) * 4 + wave) * 4;
+    const int row0 = ((bx - MOE_A_SHARED_BLOCKS) * 4 + wave) * 4;
     for (int r = 0; r < 4; ++r) {
       const int row = row0 + r;
       if (row > a.E) continue;
