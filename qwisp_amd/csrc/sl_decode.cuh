@@ -40,9 +40,10 @@ struct DecodeP {
   int n_layers, E, vocab, max_seq, max_tiles;
   const LayerP* layers;
   const uint32_t *lm_w, *lm_sb;
+  const uint32_t *emb_w, *emb_sb;     // token embedding [vocab, 2048] 4-bit
   const uint16_t* final_norm;
   const float *rope_cos, *rope_sin;
-  uint16_t *hA, *normed, *logits;     // embedded row in; final-normed row and logits out
+  uint16_t *hA, *normed, *logits;     // (hA: unused by the step kernel) final-normed row and logits out
   int32_t *tok_in, *tok_out, *st;     // st: {position, parity of every layer's ping-pong caches}
   unsigned long long* tstamp;   // optional diagnostic clock stamps
   unsigned* bar;   // [16] stage-instance counter (advanced every launch), [32] abort flag

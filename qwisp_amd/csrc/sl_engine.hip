@@ -370,7 +370,6 @@ void launch_head(sl_engine* e, int M, const HiddenArgs& ha, int out_off, bool fe
 void launch_decode(sl_engine* e, int out_off, bool feed) {
   const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
-  hipLaunchKernelGGL(k_embed, dim3(H / 256, 1), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
   if (e->gate8) hipLaunchKernelGGL(k_decode_flow<true>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0);
   else hipLaunchKernelGGL(k_decode_flow<false>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0);
   if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
@@ -600,7 +599,7 @@ int alloc_runtime(sl_engine* e) {
       DecodeP P;
       std::memset(&P, 0, sizeof(P));
       P.n_layers = d->n_layers; P.E = E; P.vocab = d->vocab; P.max_seq = max_seq_len; P.max_tiles = e->max_tiles;
-      P.layers = dl; P.lm_w = e->lm_head.w; P.lm_sb = e->lm_head.sb;
+      P.layers = dl; P.lm_w = e->lm_head.w; P.lm_sb = e->lm_head.sb; P.emb_w = e->embed.w; P.emb_sb = e->embed.sb;
       P.final_norm = e->final_norm; P.rope_cos = e->rope_cos; P.rope_sin = e->rope_sin;
       P.hA = e->hA; P.normed = e->normed; P.logits = e->logits;
       P.tok_in = e->tok_in; P.tok_out = e->tok_out; P.st = e->st; P.bar = e->dec_bar;

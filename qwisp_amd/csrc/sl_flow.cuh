@@ -218,8 +218,14 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   // first touches of the next stage: this workgroup's recurrent-state rows, or its key/value tile
   float r0 = 0.0f, r1 = 0.0f;
   if (li == 0) {
-    const uint32_t w = *reinterpret_cast<const uint32_t*>(uni(P.hA) + 2 * tid);   // embedded row from k_embed
-    h0 = lo_h(w); h1 = hi_h(w);
+    // the token's embedding row, dequantised in half arithmetic: half(half(s * q) + b) (embed_rows_q4,
+    // SeedlessFusedVerify.swift:556-569); thread t owns elements 2t, 2t+1
+    const size_t tok = (size_t)uni(P.tok_in)[0];
+    const uint32_t w = uni(P.emb_w)[tok * 256 + (tid >> 2)];
+    const uint32_t sb = uni(P.emb_sb)[tok * 32 + (tid >> 5)];
+    const float q0 = (float)((w >> (8 * (tid & 3))) & 15u), q1 = (float)((w >> (8 * (tid & 3) + 4)) & 15u);
+    h0 = f16r(f16r(lo_h(sb) * q0) + hi_h(sb));
+    h1 = f16r(f16r(lo_h(sb) * q1) + hi_h(sb));
   } else {
     if (!poll_vec2048(P, uni(F.tmoe), flow_tag(base, li - 1, FS_C), r0, r1, 0)) return false;
   }

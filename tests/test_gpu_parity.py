@@ -146,7 +146,7 @@ def test_hybrid_prefill_agrees_with_the_exact_rows(env, small_model):
         e.close()
 
 
-# ---- BASELINE config 0: one MoE block, batch 1 (and M rows) ---------------------------------------
+# ---- benchmark configuration 0: one MoE block, batch 1 (and M rows) ---------------------------------------
 @pytest.fixture(scope="module")
 def moe_model(env):
     cfg = ModelConfig(n_layers=1, n_experts=256, vocab=0, layer_types=("gdn",))
@@ -254,7 +254,7 @@ def test_engine_from_a_checkpoint_directory(env, tmp_path):
     a.close(); b.close()
 
 
-# ---- BASELINE config 1: one GDN layer, sequential steps --------------------------------------------
+# ---- benchmark configuration 1: one GDN layer, sequential steps --------------------------------------------
 def test_gdn_layer_sequence(env):
     cfg = ModelConfig(n_layers=1, n_experts=8, vocab=0, layer_types=("gdn",))
     dev, host = device_and_host_model(cfg)
@@ -277,7 +277,7 @@ def test_gdn_layer_sequence(env):
     assert np.abs(gs).max() > 0
 
 
-# ---- BASELINE config 2: one attention layer over a pre-filled KV arena ------------------------------
+# ---- benchmark configuration 2: one attention layer over a pre-filled KV arena ------------------------------
 @pytest.mark.parametrize("S", [0, 1, 63, 64, 200, 4096])
 def test_attention_layer_decode(env, S):
     cfg = ModelConfig(n_layers=1, n_experts=8, vocab=0, layer_types=("attn",))
@@ -300,7 +300,7 @@ def test_attention_layer_decode(env, S):
     assert same_bits(gk, wk) and same_bits(gv, wv)
 
 
-# ---- BASELINE config 3, reduced: the whole hybrid stack --------------------------------------------
+# ---- benchmark configuration 3, reduced: the whole hybrid stack --------------------------------------------
 @pytest.fixture(scope="module")
 def small_model(env):
     cfg = ModelConfig(n_layers=8, n_experts=32, vocab=8192)
@@ -589,7 +589,7 @@ def test_argument_errors_and_fault_firewall(env, small_model):
     assert eng.snapshot() is None
 
 
-# ---- BASELINE config 3 at full size: 40 layers, 256 experts, vocab 248320 ---------------------------
+# ---- benchmark configuration 3 at full size: 40 layers, 256 experts, vocab 248320 ---------------------------
 def test_full_size_model_short_stream(env):
     """The 19.5 GB model: a short prompt and a few greedy tokens against the oracle (which runs at
     a fraction of a token per second), plus the size-independent properties: chain == steps, and a
