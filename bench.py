@@ -7,8 +7,10 @@ before the timed region; tokens feed back on the device in chains, as the refere
 decode does (chainedStepArgmax, K = 8).
 
 Prints one JSON line: throughput, the roofline of the dominant kernel (the persistent step kernel
-k_decode_flow, which runs a whole token; timed with HIP events on the engine's stream), and the CPU
-baseline (the oracle, timed on this host's cores on a bounded sample of the same workload).
+k_decode_flow: one launch runs a chain of `--chain` tokens, each fed back on the device; launches are
+timed with HIP events on the engine's stream, and roofline.avg_ms is launch duration / tokens per
+launch), and the CPU baseline (the oracle, timed on this host's cores on a bounded sample of the same
+workload).
 """
 import argparse
 import json
@@ -197,7 +199,8 @@ def main():
                    "chain_k": args.chain, "context": [PROMPT_LEN + args.warmup, PROMPT_LEN + args.warmup + args.steps]},
         "roofline": {"bound": "hbm", "kernel": "k_decode_flow (persistent batch-1 step: 40 layers + lm_head + argmax)",
                      "achieved": head_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head_gbs / HBM_PEAK_GBS,
-                     "traffic": TRAFFIC_BYTES_PER_LAUNCH, "launches": head_n, "avg_ms": head_avg_ms, "bytes_per_launch": total_b},
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH, "launches": head_n, "avg_ms": head_avg_ms, "bytes_per_launch": total_b,
+                     "note": f"a launch runs {args.chain} tokens; launches, avg_ms, traffic and bytes_per_launch are per token"},
         "step_hbm": {"bytes_per_token": total_b, "achieved_GBs": step_gbs, "frac_of_peak": step_gbs / HBM_PEAK_GBS},
         "cpu_baseline": cpu,
         "lane_batch": lanes_report,

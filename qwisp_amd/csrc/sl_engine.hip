@@ -94,6 +94,7 @@ struct sl_engine {
   bool profile_head = false;
   std::vector<hipEvent_t> head_ev;      // 2 * MAX_CHAIN
   int head_pending = 0;
+  int head_steps[256] = {0};       // tokens of each timed launch
   double head_ms_sum = 0.0;
   long head_launches = 0;
   bool use_persistent = true;
@@ -366,15 +367,16 @@ void launch_head(sl_engine* e, int M, const HiddenArgs& ha, int out_off, bool fe
   hipLaunchKernelGGL(k_argmax_final, dim3(M), dim3(256), 0, e->stream, e->cand_v, e->cand_i, e->n_cand, e->tok_out, out_off,
                      feed ? e->tok_in : (int32_t*)nullptr);
 }
-// One batch-1 step in a single persistent launch; host mirrors advance as the kernel's own update does.
-void launch_decode(sl_engine* e, int out_off, bool feed) {
+// `steps` batch-1 steps in a single persistent launch (each token fed back on the device); host mirrors advance
+// as the kernel's own update does.
+void launch_decode(sl_engine* e, int out_off, bool feed, int steps) {
   const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
-  if (e->gate8) hipLaunchKernelGGL(k_decode_flow<true>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0);
-  else hipLaunchKernelGGL(k_decode_flow<false>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0);
-  if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
-  e->pos += 1;
-  for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
+  if (e->gate8) hipLaunchKernelGGL(k_decode_flow<true>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0, steps);
+  else hipLaunchKernelGGL(k_decode_flow<false>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0, steps);
+  if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_steps[e->head_pending] = steps; e->head_pending++; }
+  e->pos += steps;
+  if (steps & 1) for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
 }
 // After a persistent step: a workgroup that gave up waiting leaves the abort word set.
 int check_decode_abort(sl_engine* e) {
@@ -614,8 +616,9 @@ int alloc_runtime(sl_engine* e) {
         F.tml = dalloc<uint4>(e, (size_t)SL_ATT_HEADS * e->max_tiles, true);
         F.tpo = dalloc<uint4>(e, (size_t)SL_ATT_HEADS * e->max_tiles * 128, true);
         F.tcand = dalloc<uint4>(e, 256, true);
+        F.ttok = dalloc<uint4>(e, 4, true);
         if (!F.tproj || !F.tycore || !F.tmix || !F.trlog || !F.tsg || !F.tsh || !F.tact || !F.tmoe ||
-            !F.tml || !F.tpo || !F.tcand) return SL_ERR_DEVICE;
+            !F.tml || !F.tpo || !F.tcand || !F.ttok) return SL_ERR_DEVICE;
         e->flow_host = F;
         e->flow_params = upload<FlowP>(e, &F, 1, SL_LOC_HOST);
         if (!e->flow_params) return SL_ERR_DEVICE;
@@ -829,7 +832,7 @@ static void time_end(sl_engine* e) {
   float ms = 0.0f;
   if (hipEventElapsedTime(&ms, e->ev0, e->ev1) == hipSuccess) e->last_ms = ms;
   for (int i = 0; i < e->head_pending; ++i)
-    if (hipEventElapsedTime(&ms, e->head_ev[2 * i], e->head_ev[2 * i + 1]) == hipSuccess) { e->head_ms_sum += ms; e->head_launches++; }
+    if (hipEventElapsedTime(&ms, e->head_ev[2 * i], e->head_ev[2 * i + 1]) == hipSuccess) { e->head_ms_sum += ms; e->head_launches += e->head_steps[i] > 0 ? e->head_steps[i] : 1; }
   e->head_pending = 0;
 }
 
@@ -843,7 +846,7 @@ int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   const bool persistent = (m == 1 && e->dec_grid > 0 && e->use_persistent);
   if (persistent) {
-    launch_decode(e, 0, false);
+    launch_decode(e, 0, false, 1);
   } else {
     hipLaunchKernelGGL(k_embed, dim3(H / 256, m), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
     launch_layers(e, m);
@@ -866,8 +869,8 @@ int sl_chained_step_argmax(sl_engine* e, int32_t first, int k, int32_t* out) {
   r = to_device(e, e->tok_in, &first, 4); if (r) return r;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   const bool persistent = (e->dec_grid > 0 && e->use_persistent);
-  for (int s = 0; s < k; ++s) {
-    if (persistent) { launch_decode(e, s, true); continue; }
+  if (persistent) launch_decode(e, 0, true, k);        // the whole chain in one launch
+  for (int s = 0; s < k && !persistent; ++s) {
     hipLaunchKernelGGL(k_embed, dim3(H / 256, 1), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
     launch_layers(e, 1);
     HiddenArgs ha{e->hA, e->moe_out, e->final_norm, e->hB, e->normed};

@@ -32,6 +32,7 @@ struct FlowP {
   uint4 *tml;           // attention {max, sum, tag, tag}  [16][max_tiles]
   uint4 *tpo;           // attention {o[2c], o[2c+1], tag, tag}  [16][max_tiles][128]
   uint4 *tcand;         // {value, index, tag, tag}        [256]
+  uint4 *ttok;          // {token, token, tag, tag}: the token a step of a multi-step launch hands to the next [1]
 };
 
 // Parameters live in LDS for the whole launch.  Reading them there (ds_read + readfirstlane) does not
@@ -42,8 +43,10 @@ struct FlowLds {
   FlowP F;
   LayerP layers[FLOW_MAX_LAYERS];
   unsigned long long parity;      // bit l = which copy of layer l's recurrent state / history is current
+  unsigned long long linmask;     // bit l = layer l is a linear-attention layer (its parity flips every step)
   int pos;
   uint32_t base;
+  int tok;                        // token of the current step when it came from the step before in the same launch
 };
 __shared__ FlowLds g_K;
 
@@ -203,7 +206,7 @@ SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, fl
 }
 
 // ---- stage 1: input norm + in-projection ------------------------------------------------------------
-SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base, float& h0, float& h1) {
+SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base, float& h0, float& h1, int step) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   const int N = uni(Y.is_linear) ? SL_GDN_IN_N : SL_ATT_QKV_N;
@@ -220,7 +223,24 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   if (li == 0) {
     // the token's embedding row, dequantised in half arithmetic: half(half(s * q) + b) (embed_rows_q4,
     // SeedlessFusedVerify.swift:556-569); thread t owns elements 2t, 2t+1
-    const size_t tok = (size_t)uni(P.tok_in)[0];
+    if (step > 0) {
+      // the token comes from the step before of this launch: workgroup 0 published it with this step's tag
+      const uint32_t ttag = flow_tag32(base, 0, 7);
+      const rsrc_t rt = co_rsrc(uni(F.ttok));
+      unsigned spins = 0;
+      for (;;) {
+        bool ok = true;
+        if (wave == 1) {                 // not wave 0: in workgroup 0 that one has just stored the step's results
+          const uint4 c = ldw4(rt, 0);
+          ok = c.z == ttag && c.w == ttag;
+          if (ok && lane == 0) g_K.tok = (int)c.x;
+        }
+        const int v = flow_round(ok, spins, uni(P.bar) + 32);
+        if (v > 0) break;
+        if (v < 0) return false;
+      }
+    }
+    const size_t tok = (size_t)(step > 0 ? uni(g_K.tok) : uni(P.tok_in)[0]);
     const uint32_t w = uni(P.emb_w)[tok * 256 + (tid >> 2)];
     const uint32_t sb = uni(P.emb_sb)[tok * 32 + (tid >> 5)];
     const float q0 = (float)((w >> (8 * (tid & 3))) & 15u), q1 = (float)((w >> (8 * (tid & 3) + 4)) & 15u);
@@ -1135,7 +1155,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
 }
 
 // ---- head -------------------------------------------------------------------------------------------
-SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t base, float h0, float h1) {
+SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t base, float h0, float h1, bool hand_on) {
   FLOW_IDS;
   const DecodeP& P = F.d;
   Lds& L = g_L;
@@ -1214,15 +1234,19 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
     uni(P.tok_out)[out_off] = i;
     if (feed) uni(P.tok_in)[0] = i;
     uni(P.st)[0] = pos + 1;
-    st_co32(uni(P.bar) + 16, base + (uint32_t)(nl + 1) * 8u);
+    const uint32_t nbase = base + (uint32_t)(nl + 1) * 8u;
+    st_co32(uni(P.bar) + 16, nbase);
+    if (hand_on) { const uint32_t ttag = flow_tag32(nbase, 0, 7); stw4(co_rsrc(uni(F.ttok)), 0, (uint32_t)i, (uint32_t)i, ttag, ttag); }
   }
   for (int l = tid; l < nl; l += DEC_THREADS) uni(P.st)[1 + l] ^= 1;
   return true;
 }
 
 // ---- the kernel: hA already holds the embedded token row (k_embed) --------------------------------------
+// `steps` tokens per launch (a chain feeds each token back on the device): between two steps workgroup 0 hands the
+// new token to everybody as a tagged word, which costs one hand-over instead of a kernel boundary.
 template <bool GATE8>
-__global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __restrict__ Fp, int out_off, int feed) {
+__global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __restrict__ Fp, int out_off, int feed, int steps) {
   {
     const int tid = threadIdx.x;
     const uint32_t* src = reinterpret_cast<const uint32_t*>(Fp);
@@ -1235,34 +1259,42 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
     if (tid < 64) {
       const int bit = (tid < nl) ? (Fp->d.st[1 + tid] & 1) : 0;
       const unsigned long long m = __ballot(bit);
-      if (tid == 0) { g_K.parity = m; g_K.pos = Fp->d.st[0]; g_K.base = ld_co32(Fp->d.bar + 16); g_L.bar.nts = 0; }
+      const unsigned long long lm = __ballot((tid < nl) ? (Fp->d.layers[tid].is_linear != 0) : 0);
+      if (tid == 0) { g_K.parity = m; g_K.linmask = lm; g_K.pos = Fp->d.st[0]; g_K.base = ld_co32(Fp->d.bar + 16); g_K.tok = 0; g_L.bar.nts = 0; }
       if (tid < 4) g_L.pf[tid] = 0;
     }
     __syncthreads();
   }
   const FlowP& F = g_K.F;
   const DecodeP& P = F.d;
-  const uint32_t base = uni(g_K.base);
-  const int pos = uni(g_K.pos);
   const int nl = uni(P.n_layers);
-  float h0 = 0.0f, h1 = 0.0f;          // this thread's two elements of the residual stream
-  for (int li = 0; li < nl; ++li) {
-    const LayerP& Y = g_K.layers[li];
-    const int is_linear = uni(Y.is_linear);
-    if (!flow_in(F, Y, li, pos, base, h0, h1)) return;
-    GdnHist gh = {0u, 0u};
-    if (is_linear) {
-      if (!flow_gdn(F, Y, li, base, gh)) return;
-      if (!flow_out(F, Y, li, 0, base, gh)) return;
-    } else {
-      if (((pos + SDPA_TILE) / SDPA_TILE) * SL_ATT_KV * 4 <= (int)gridDim.x ? !flow_sdpa4(F, Y, li, pos, base) : !flow_sdpa(F, Y, li, pos, base)) return;
-      if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh)) return;
+  for (int step = 0; step < steps; ++step) {
+    const uint32_t base = uni(g_K.base);
+    const int pos = uni(g_K.pos);
+    float h0 = 0.0f, h1 = 0.0f;          // this thread's two elements of the residual stream
+    for (int li = 0; li < nl; ++li) {
+      const LayerP& Y = g_K.layers[li];
+      const int is_linear = uni(Y.is_linear);
+      if (!flow_in(F, Y, li, pos, base, h0, h1, step)) return;
+      GdnHist gh = {0u, 0u};
+      if (is_linear) {
+        if (!flow_gdn(F, Y, li, base, gh)) return;
+        if (!flow_out(F, Y, li, 0, base, gh)) return;
+      } else {
+        if (((pos + SDPA_TILE) / SDPA_TILE) * SL_ATT_KV * 4 <= (int)gridDim.x ? !flow_sdpa4(F, Y, li, pos, base) : !flow_sdpa(F, Y, li, pos, base)) return;
+        if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh)) return;
+      }
+      if (!flow_moe_a<GATE8>(F, Y, li, base, h0, h1)) return;
+      if (!flow_moe_b(F, Y, li, base)) return;
+      if (!flow_moe_c(F, Y, li, base)) return;
     }
-    if (!flow_moe_a<GATE8>(F, Y, li, base, h0, h1)) return;
-    if (!flow_moe_b(F, Y, li, base)) return;
-    if (!flow_moe_c(F, Y, li, base)) return;
+    if (!flow_head(F, pos, out_off + step, feed, base, h0, h1, step + 1 < steps)) return;
+    if (step + 1 < steps) {
+      __syncthreads();                   // everybody has read this step's position, tag base and parities
+      if (threadIdx.x == 0) { g_K.pos = pos + 1; g_K.base = base + (uint32_t)(nl + 1) * 8u; g_K.parity ^= g_K.linmask; }
+      __syncthreads();
+    }
   }
-  flow_head(F, pos, out_off, feed, base, h0, h1);
   fstamp(P, 18, 0);
   if (uni(P.tstamp) && threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == 100))
     uni(P.tstamp)[blockIdx.x ? 2048 : 0] = (unsigned long long)g_L.bar.nts;
