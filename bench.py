@@ -8,8 +8,8 @@ decode does (chainedStepArgmax, K = 8).
 
 Prints one JSON line: throughput, the roofline of the dominant kernel (the persistent step kernel
 k_decode_flow: one launch runs a chain of `--chain` tokens, each fed back on the device; launches are
-timed with HIP events on the engine's stream, and roofline.avg_ms is launch duration / tokens per
-launch), and the CPU baseline (the oracle, timed on this host's cores on a bounded sample of the same
+timed with HIP events on the engine's stream; roofline.avg_ms and bytes_per_launch are those of one
+launch = `--chain` tokens), and the CPU baseline (the oracle, timed on this host's cores on a bounded sample of the same
 workload).
 """
 import argparse
@@ -24,8 +24,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 PROMPT_LEN = 512
-# HBM bytes per k_decode_flow launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/), or None until measured
-TRAFFIC_BYTES_PER_LAUNCH = 1936711864   # 2 x FETCH_SIZE (copy-calibrated) + WRITE_SIZE, in bytes, at context ~525
+# HBM bytes per decoded token: rocprofv3 FETCH_SIZE + WRITE_SIZE of a k_decode_flow launch (profiles/) / its 8 tokens
+TRAFFIC_BYTES_PER_TOKEN = 1936470412   # 2 x FETCH_SIZE (copy-calibrated) + WRITE_SIZE, in bytes, at context ~525
 
 
 def step_bytes(cfg, ctx):
@@ -124,8 +124,10 @@ def main():
     total_b, head_b = step_bytes(cfg, ctx_mid)
     ms_step = elapsed * 1e3 / args.steps
     tok_s = args.steps / elapsed
+    tok_per_launch = args.steps / max(head_n, 1)          # a launch of k_decode_flow runs a whole chain
     head_avg_ms = head_ms / max(head_n, 1)
-    head_gbs = total_b / (head_avg_ms * 1e-3) / 1e9 if head_n else 0.0
+    launch_b = int(total_b * tok_per_launch)
+    head_gbs = launch_b / (head_avg_ms * 1e-3) / 1e9 if head_n else 0.0
     step_gbs = total_b / (ms_step * 1e-3) / 1e9
 
     lanes_report = None
@@ -199,8 +201,9 @@ def main():
                    "chain_k": args.chain, "context": [PROMPT_LEN + args.warmup, PROMPT_LEN + args.warmup + args.steps]},
         "roofline": {"bound": "hbm", "kernel": "k_decode_flow (persistent batch-1 step: 40 layers + lm_head + argmax)",
                      "achieved": head_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head_gbs / HBM_PEAK_GBS,
-                     "traffic": TRAFFIC_BYTES_PER_LAUNCH, "launches": head_n, "avg_ms": head_avg_ms, "bytes_per_launch": total_b,
-                     "note": f"a launch runs {args.chain} tokens; launches, avg_ms, traffic and bytes_per_launch are per token"},
+                     "traffic": int(TRAFFIC_BYTES_PER_TOKEN * tok_per_launch), "launches": head_n, "avg_ms": head_avg_ms,
+                     "bytes_per_launch": launch_b, "tokens_per_launch": tok_per_launch, "bytes_per_token": total_b,
+                     "avg_ms_per_token": head_avg_ms / tok_per_launch},
         "step_hbm": {"bytes_per_token": total_b, "achieved_GBs": step_gbs, "frac_of_peak": step_gbs / HBM_PEAK_GBS},
         "cpu_baseline": cpu,
         "lane_batch": lanes_report,

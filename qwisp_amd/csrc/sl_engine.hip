@@ -94,7 +94,6 @@ struct sl_engine {
   bool profile_head = false;
   std::vector<hipEvent_t> head_ev;      // 2 * MAX_CHAIN
   int head_pending = 0;
-  int head_steps[256] = {0};       // tokens of each timed launch
   double head_ms_sum = 0.0;
   long head_launches = 0;
   bool use_persistent = true;
@@ -374,7 +373,7 @@ void launch_decode(sl_engine* e, int out_off, bool feed, int steps) {
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
   if (e->gate8) hipLaunchKernelGGL(k_decode_flow<true>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0, steps);
   else hipLaunchKernelGGL(k_decode_flow<false>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0, steps);
-  if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_steps[e->head_pending] = steps; e->head_pending++; }
+  if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
   e->pos += steps;
   if (steps & 1) for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
 }
@@ -832,7 +831,7 @@ static void time_end(sl_engine* e) {
   float ms = 0.0f;
   if (hipEventElapsedTime(&ms, e->ev0, e->ev1) == hipSuccess) e->last_ms = ms;
   for (int i = 0; i < e->head_pending; ++i)
-    if (hipEventElapsedTime(&ms, e->head_ev[2 * i], e->head_ev[2 * i + 1]) == hipSuccess) { e->head_ms_sum += ms; e->head_launches += e->head_steps[i] > 0 ? e->head_steps[i] : 1; }
+    if (hipEventElapsedTime(&ms, e->head_ev[2 * i], e->head_ev[2 * i + 1]) == hipSuccess) { e->head_ms_sum += ms; e->head_launches += 1; }
   e->head_pending = 0;
 }
 
