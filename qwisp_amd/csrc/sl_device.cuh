@@ -158,6 +158,25 @@ SL_DEV uint4 pack8(const float* f) {
 // operands into v_fma_mix_f32.  The 2^24 is returned to the scale: t = fmaf(s*2^24, dq', b*sx).
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 SL_DEV h2_t as_h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
+// The four masked forms of a word: mk[j] holds the nibbles j (low half) and j+4 (high half).
+SL_DEV void word_masks(uint32_t w, h2_t* mk /*4*/) {
+  mk[0] = as_h2(w & 0x000F000Fu); mk[1] = as_h2((w >> 4) & 0x000F000Fu);
+  mk[2] = as_h2((w >> 8) & 0x000F000Fu); mk[3] = as_h2((w >> 12) & 0x000F000Fu);
+}
+// word_dot with the masked forms prepared by the caller: the same chain
+SL_DEV float word_dot_masked(const h2_t* mk /*4*/, const uint32_t* xp /*4 packed pairs*/) {
+  const h2_t x0 = as_h2(xp[0]), x1 = as_h2(xp[1]), x2 = as_h2(xp[2]), x3 = as_h2(xp[3]);
+  float dq = 0.0f;
+  dq = fmaf((float)x0.x, (float)mk[0].x, dq);
+  dq = fmaf((float)x0.y, (float)mk[1].x, dq);
+  dq = fmaf((float)x1.x, (float)mk[2].x, dq);
+  dq = fmaf((float)x1.y, (float)mk[3].x, dq);
+  dq = fmaf((float)x2.x, (float)mk[0].y, dq);
+  dq = fmaf((float)x2.y, (float)mk[1].y, dq);
+  dq = fmaf((float)x3.x, (float)mk[2].y, dq);
+  dq = fmaf((float)x3.y, (float)mk[3].y, dq);
+  return dq;
+}
 // dq' = 2^-24 * (fmaf chain over the 8 nibbles, least significant first)
 SL_DEV float word_dot(uint32_t w, const uint32_t* xp /*4 packed pairs*/) {
   const h2_t m0 = as_h2(w & 0x000F000Fu), m1 = as_h2((w >> 4) & 0x000F000Fu);
@@ -201,6 +220,15 @@ SL_DEV float quad_term(uint4 w, uint32_t sb, const uint32_t* xp /*16 packed pair
   float t1 = fmaf(s, word_dot(w.y, xp + 4), b * sx[1]);
   float t2 = fmaf(s, word_dot(w.z, xp + 8), b * sx[2]);
   float t3 = fmaf(s, word_dot(w.w, xp + 12), b * sx[3]);
+  return (t0 + t1) + (t2 + t3);
+}
+// quad_term with the 16 masked forms of the four words prepared by the caller (reused over several activation rows)
+SL_DEV float quad_term_masked(const h2_t* mk /*16*/, uint32_t sb, const uint32_t* xp, const float* sx) {
+  const float s = lo_h(sb) * 16777216.0f, b = hi_h(sb);
+  float t0 = fmaf(s, word_dot_masked(mk, xp), b * sx[0]);
+  float t1 = fmaf(s, word_dot_masked(mk + 4, xp + 4), b * sx[1]);
+  float t2 = fmaf(s, word_dot_masked(mk + 8, xp + 8), b * sx[2]);
+  float t3 = fmaf(s, word_dot_masked(mk + 12, xp + 12), b * sx[3]);
   return (t0 + t1) + (t2 + t3);
 }
 // 32 half-valued floats -> 16 packed pairs (exact)

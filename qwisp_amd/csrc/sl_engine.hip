@@ -267,15 +267,15 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   a.sh_act = e->sh_act; a.rlogits = e->rlogits; a.sgate = e->sgate;
   const int router_blocks = (e->n_experts + 1 + 15) / 16;
   hipLaunchKernelGGL(k_moe_a, dim3(MOE_A_SHARED_BLOCKS + router_blocks, M), dim3(256), 0, e->stream, a);
+  hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, e->n_experts, L.route_inds, L.route_scores);
   MoeBArgs b{};
-  b.xn = e->xn; b.rlogits = e->rlogits; b.E = e->n_experts;
-  b.g_w = L.sw_gate.w; b.g_sb = L.sw_gate.sb; b.u_w = L.sw_up.w; b.u_sb = L.sw_up.sb;
-  b.act = e->act; b.inds = L.route_inds; b.scores = L.route_scores;
-  hipLaunchKernelGGL(k_moe_b, dim3(512, M), dim3(256), 0, e->stream, b);
+  b.xn = e->xn; b.g_w = L.sw_gate.w; b.g_sb = L.sw_gate.sb; b.u_w = L.sw_up.w; b.u_sb = L.sw_up.sb;
+  b.act = e->act; b.inds = L.route_inds;
+  hipLaunchKernelGGL(k_moe_b, dim3(256, M), dim3(256), 0, e->stream, b);
   MoeCArgs c{};
   c.act = e->act; c.sh_act = e->sh_act; c.inds = L.route_inds; c.scores = L.route_scores; c.sgate = e->sgate;
   c.d_w = L.sw_down.w; c.d_sb = L.sw_down.sb; c.shd_w = L.sh_down.w; c.shd_sb = L.sh_down.sb; c.out = e->moe_out;
-  hipLaunchKernelGGL(k_moe_c, dim3(256, M), dim3(128), 0, e->stream, c);
+  hipLaunchKernelGGL(k_moe_c, dim3(128, M), dim3(256), 0, e->stream, c);
 }
 // Hybrid prefill: chunks of at least 16 rows of one sequence take the dense mixer projections to the matrix cores.
 bool use_matrix_cores(const sl_engine* e, int M, const LaneRef* lanes) { return e->hybrid && !lanes && M >= 16 && M <= GROUP_CAP; }
@@ -286,6 +286,9 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
     HiddenArgs hn = ha; hn.xn_out = e->xn;      // residual + norm rows on their own, then the GEMM
     hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
     launch_qmm4_mfma(QmmArgs{e->xn, H, L.in_proj.w, L.in_proj.sb, M, SL_GDN_IN_N, H, e->proj, PROJ_STRIDE}, e->stream);
+  } else if (M >= 2) {
+    hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, true>), dim3(SL_GDN_IN_N / 32, (M + 7) / 8), dim3(512), 0, e->stream, ha, (const uint16_t*)nullptr, 0,
+                       L.in_proj.w, L.in_proj.sb, SL_GDN_IN_N, e->proj, PROJ_STRIDE, M);
   } else {
     hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_GDN_IN_N / 16, M), dim3(256), 0, e->stream, ha, L.in_proj.w, L.in_proj.sb,
                        SL_GDN_IN_N, e->proj, PROJ_STRIDE);
@@ -306,6 +309,11 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
   if (mm) {
     hipLaunchKernelGGL(k_gdn_gate_rows, dim3(SL_GDN_HV, M), dim3(64), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32);
     launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.out_proj.w, L.out_proj.sb, M, H, 4096, e->mix, H}, e->stream);
+  } else if (M >= 2) {
+    // the gated norm once per row, then the row-tiled projection (same bits as the fused kernel below)
+    hipLaunchKernelGGL(k_gdn_gate_rows, dim3(SL_GDN_HV, M), dim3(64), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32);
+    hipLaunchKernelGGL((k_qmv_tile<2, 2, 4, false>), dim3(H / 8, (M + 3) / 4), dim3(256), 0, e->stream, HiddenArgs{}, e->ycore, 4096,
+                       L.out_proj.w, L.out_proj.sb, H, e->mix, H, M);
   } else {
     hipLaunchKernelGGL(k_qmv_gdn_out<2>, dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32,
                        L.out_proj.w, L.out_proj.sb, H, e->mix);
@@ -317,6 +325,9 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
     HiddenArgs hn = ha; hn.xn_out = e->xn;
     hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
     launch_qmm4_mfma(QmmArgs{e->xn, H, L.qkv.w, L.qkv.sb, M, SL_ATT_QKV_N, H, e->proj, PROJ_STRIDE}, e->stream);
+  } else if (M >= 2) {
+    hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, true>), dim3(SL_ATT_QKV_N / 32, (M + 7) / 8), dim3(512), 0, e->stream, ha, (const uint16_t*)nullptr, 0,
+                       L.qkv.w, L.qkv.sb, SL_ATT_QKV_N, e->proj, PROJ_STRIDE, M);
   } else {
     hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_ATT_QKV_N / 16, M), dim3(256), 0, e->stream, ha, L.qkv.w, L.qkv.sb,
                        SL_ATT_QKV_N, e->proj, PROJ_STRIDE);
@@ -329,11 +340,13 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
   SdpaArgs s{};
   s.qrot = e->qrot; s.kcache = L.kcache; s.vcache = L.vcache; s.st = e->st; s.maxSeq = e->max_seq; s.maxTiles = e->max_tiles;
   s.pm = e->pm; s.pl = e->pl; s.po = e->po; s.lanes = lanes;
-  hipLaunchKernelGGL(k_sdpa_tile, dim3(tiles, SL_ATT_KV, M), dim3(64), 0, e->stream, s);
+  hipLaunchKernelGGL(k_sdpa_tile, dim3(tiles, SL_ATT_KV, M), dim3(256), 0, e->stream, s);
   SdpaMergeArgs g{};
   g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore; g.lanes = lanes;
   hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
   if (mm) launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.o_proj.w, L.o_proj.sb, M, H, 4096, e->mix, H}, e->stream);
+  else if (M >= 2) hipLaunchKernelGGL((k_qmv_tile<2, 2, 4, false>), dim3(H / 8, (M + 3) / 4), dim3(256), 0, e->stream, HiddenArgs{}, e->ycore, 4096,
+                                      L.o_proj.w, L.o_proj.sb, H, e->mix, H, M);
   else hipLaunchKernelGGL((k_qmv_plain<2, 2>), dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, 4096, L.o_proj.w, L.o_proj.sb,
                           H, e->mix, H);
 }
@@ -360,8 +373,21 @@ void advance(sl_engine* e, int M) {
 void launch_head(sl_engine* e, int M, const HiddenArgs& ha, int out_off, bool feed) {
   const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
-  hipLaunchKernelGGL(k_head, dim3(e->n_cand, M), dim3(256), 0, e->stream, ha, e->lm_head.w, e->lm_head.sb, e->vocab,
-                     e->logits, e->cand_v, e->cand_i);
+  if (M >= 2) {
+    // residual + final norm once per row, then the row-tiled lm_head (weights streamed once per 8 rows)
+    const uint16_t* xin = ha.h_in;
+    if (ha.r_in || ha.lnw) {
+      HiddenArgs hn = ha;
+      if (!hn.xn_out) hn.xn_out = e->xn;
+      hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
+      xin = hn.xn_out;
+    }
+    hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, false, true>), dim3(e->n_cand, (M + 7) / 8), dim3(256), 0, e->stream, HiddenArgs{}, xin, H,
+                       e->lm_head.w, e->lm_head.sb, e->vocab, e->logits, e->vocab, M, e->cand_v, e->cand_i);
+  } else {
+    hipLaunchKernelGGL(k_head, dim3(e->n_cand, M), dim3(256), 0, e->stream, ha, e->lm_head.w, e->lm_head.sb, e->vocab,
+                       e->logits, e->cand_v, e->cand_i);
+  }
   if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
   hipLaunchKernelGGL(k_argmax_final, dim3(M), dim3(256), 0, e->stream, e->cand_v, e->cand_i, e->n_cand, e->tok_out, out_off,
                      feed ? e->tok_in : (int32_t*)nullptr);

@@ -178,6 +178,125 @@ __global__ __launch_bounds__(256) void k_qmv_plain(const uint16_t* __restrict__ 
 }
 
 // -------------------------------------------------------------------------------------------------
+// The same projections for a tile of MT activation rows at a time (verify rows, lane batches, exact prefill
+// chunks): a wave fetches and masks its R weight rows once and runs every activation row of the tile against
+// them, so the weight stream and the nibble unpacking are shared; per activation row the arithmetic is that of
+// k_qmv_hidden / k_qmv_plain.  The tile's activation rows are prepared once per workgroup (residual, norm,
+// packing: wave w takes rows w, w + waves, ...) and parked in LDS, 20 words per lane (16 packed pairs, 4 sums)
+// so that a lane reads back its own 80 bytes with five 16-byte reads free of bank conflicts.
+// HIDDEN: x comes from the hidden prologue (K = 2048); otherwise from the fp16 buffer xin (K = 2048*NBLK).
+// Grid (ceil(N / (waves*R)), ceil(M / MT)), any multiple of 64 threads up to 512.
+// -------------------------------------------------------------------------------------------------
+// ARGMAX (lm_head, R = 4, 4 waves): y is the logits matrix and every workgroup also leaves one (value, index)
+// candidate per activation row, the first maximum of its 16 rounded logits, for k_argmax_final.
+template <int NBLK, int R, int MT, bool HIDDEN, bool ARGMAX = false>
+__global__ __launch_bounds__(512) void k_qmv_tile(HiddenArgs ha, const uint16_t* __restrict__ xin, int x_stride,
+                                                  const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB,
+                                                  int N, uint16_t* __restrict__ y, int y_stride, int M,
+                                                  float* __restrict__ cand_v = nullptr, int32_t* __restrict__ cand_i = nullptr) {
+  static_assert(!HIDDEN || NBLK == 1, "the hidden row is one block of 2048");
+  static_assert(!ARGMAX || R == 4, "candidates are formed over four rows per wave");
+  constexpr int WPR = NBLK * 256, GPR = NBLK * 32;
+  __shared__ uint4 xs[MT * NBLK * 64 * 5];
+  __shared__ float s_v[ARGMAX ? MT * 8 : 1];
+  __shared__ int s_i[ARGMAX ? MT * 8 : 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const int m0 = blockIdx.y * MT, mc = min(MT, M - m0);
+  const size_t row0 = ((size_t)blockIdx.x * waves + wave) * R;
+  const bool live = row0 < (size_t)N;
+  // weights first: their latency hides behind the preparation of the activation rows
+  uint4 wv[R][NBLK];
+  uint32_t sb[R][NBLK];
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int b = 0; b < NBLK; ++b) {
+        wv[r][b] = ld16(W + (row0 + r) * WPR + b * 256 + 4 * lane);
+        sb[r][b] = SB[(row0 + r) * GPR + b * 32 + (lane >> 1)];
+      }
+  }
+  for (int m = wave; m < mc; m += waves) {
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b) {
+      float x[32], sx[4];
+      if constexpr (HIDDEN) hidden_prologue(ha, m0 + m, lane, blockIdx.x == 0, x);
+      else load32(xin + (size_t)(m0 + m) * x_stride + b * 2048 + 32 * lane, x);
+      word_sums(x, sx);
+      uint32_t xp[16];
+      pack_x(x, xp);
+      uint4* dst = xs + ((m * NBLK + b) * 64 + lane) * 5;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dst[j] = make_uint4(xp[4 * j], xp[4 * j + 1], xp[4 * j + 2], xp[4 * j + 3]);
+      dst[4] = make_uint4(__float_as_uint(sx[0]), __float_as_uint(sx[1]), __float_as_uint(sx[2]), __float_as_uint(sx[3]));
+    }
+  }
+  __syncthreads();
+  if (!live) {
+    if constexpr (ARGMAX) {
+      if (lane == 0) for (int m = 0; m < mc; ++m) { s_v[m * 8 + wave] = -__int_as_float(0x7f800000); s_i[m * 8 + wave] = 0x7fffffff; }
+      __syncthreads();
+    }
+    return;
+  }
+  h2_t mk[R][NBLK][16];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b) {
+      word_masks(wv[r][b].x, mk[r][b]); word_masks(wv[r][b].y, mk[r][b] + 4);
+      word_masks(wv[r][b].z, mk[r][b] + 8); word_masks(wv[r][b].w, mk[r][b] + 12);
+    }
+  for (int m = 0; m < mc; ++m) {
+    float acc[R];
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b) {
+      const uint4* src = xs + ((m * NBLK + b) * 64 + lane) * 5;
+      uint32_t xp[16];
+      float sx[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { const uint4 v = src[j]; xp[4 * j] = v.x; xp[4 * j + 1] = v.y; xp[4 * j + 2] = v.z; xp[4 * j + 3] = v.w; }
+      { const uint4 v = src[4]; sx[0] = __uint_as_float(v.x); sx[1] = __uint_as_float(v.y); sx[2] = __uint_as_float(v.z); sx[3] = __uint_as_float(v.w); }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const float t = quad_term_masked(mk[r][b], sb[r][b], xp, sx);
+        acc[r] = (b == 0) ? t : acc[r] + t;
+      }
+    }
+    float out[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) out[r] = tree_sum<64>(acc[r]);
+    if constexpr (ARGMAX) {
+      if (lane == 0) {
+        float bv = -__int_as_float(0x7f800000);
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float v = f16r(out[r]);
+          if (v > bv) { bv = v; bi = (int)(row0 + r); }
+        }
+        s_v[m * 8 + wave] = bv; s_i[m * 8 + wave] = bi;
+        *reinterpret_cast<uint2*>(y + (size_t)(m0 + m) * y_stride + row0) = make_uint2(pack2(out[0], out[1]), pack2(out[2], out[3]));
+      }
+    } else if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) y[(size_t)(m0 + m) * y_stride + row0 + r] = f2h(out[r]);
+    }
+  }
+  if constexpr (ARGMAX) {
+    __syncthreads();
+    if ((int)threadIdx.x < mc) {
+      const int m = threadIdx.x;
+      float bv = s_v[m * 8];
+      int bi = s_i[m * 8];
+      for (int w = 1; w < waves; ++w) if (s_v[m * 8 + w] > bv) { bv = s_v[m * 8 + w]; bi = s_i[m * 8 + w]; }
+      cand_v[(size_t)(m0 + m) * gridDim.x + blockIdx.x] = bv;
+      cand_i[(size_t)(m0 + m) * gridDim.x + blockIdx.x] = bi;
+    }
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
 // Gated-DeltaNet core: causal conv(4)+SiLU+history shift, q/k head norms and scales, beta and
 // decay, and the gated delta rule with the fp32 state in registers, M rows in sequence.
 // References: conv_shift_fused_rows SeedlessFusedVerify.swift:634-663; gdn_prep_rows :839-938;
@@ -543,80 +662,102 @@ __global__ __launch_bounds__(256) void k_moe_a(MoeAArgs a) {
 // (ties to the lower index), half renormalisation.  One wave; lane l owns experts 4l..4l+3.
 // Reference: route_top8_rows SeedlessFusedVerify.swift:191-213.
 // -------------------------------------------------------------------------------------------------
+// Order key of a router logit: larger logit first, lower expert index first on ties (+0 and -0 tie).
+SL_DEV uint32_t route_order_key(uint32_t hbits, int e) {
+  uint32_t u = hbits & 0xffffu;
+  if ((u & 0x7fffu) == 0) u = 0;
+  u = (u & 0x8000u) ? (~u & 0xffffu) : (u | 0x8000u);
+  return (u << 8) | (uint32_t)(255 - e);
+}
 SL_DEV void route_wave(const uint16_t* __restrict__ logits, int E, int lane, int* inds /*LDS [8]*/, float* scores /*LDS [8]*/) {
   const float NEG = -__int_as_float(0x7f800000);
   float lg[4], ex[4];
+  uint32_t key[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) lg[i] = (4 * lane + i < E) ? h2f(logits[4 * lane + i]) : NEG;
+  for (int i = 0; i < 4; ++i) {
+    const bool in = 4 * lane + i < E;
+    const uint32_t bits = in ? logits[4 * lane + i] : 0u;
+    lg[i] = in ? h2f((uint16_t)bits) : NEG;
+    key[i] = in ? route_order_key(bits, 4 * lane + i) : 0u;
+  }
   const float mx = tree_max<64>(fmaxf(fmaxf(lg[0], lg[1]), fmaxf(lg[2], lg[3])));
 #pragma unroll
   for (int i = 0; i < 4; ++i) ex[i] = (4 * lane + i < E) ? exp_c(lg[i] - mx) : 0.0f;
   const float Z = tree_sum<64>(((ex[0] + ex[1]) + ex[2]) + ex[3]);
-#pragma unroll 1
+  // eight times: the largest remaining key (one value to reduce; the index rides in its low byte), then remove it
+  float sc[8];
+#pragma unroll
   for (int k = 0; k < 8; ++k) {
-    float bv = lg[0]; int bi = 4 * lane;
+    uint32_t m = max(max(key[0], key[1]), max(key[2], key[3]));
+    m = max(m, dpp_u<DPP_XOR1>(m));
+    m = max(m, dpp_u<DPP_XOR2>(m));
+    m = max(m, dpp_u<DPP_HALF_MIRROR>(m));
+    m = max(m, dpp_u<DPP_MIRROR>(m));
+    const uint32_t top = max(max((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
+                             max((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
 #pragma unroll
-    for (int i = 1; i < 4; ++i) if (lg[i] > bv) { bv = lg[i]; bi = 4 * lane + i; }
-#pragma unroll
-    for (int msk = 1; msk < 64; msk <<= 1) {
-      const float ov = __shfl_xor(bv, msk, 64);
-      const int oi = __shfl_xor(bi, msk, 64);
-      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
-    const int sub = bi & 3;
+    for (int i = 0; i < 4; ++i) key[i] = (key[i] == top) ? 0u : key[i];
+    const int bi = min(255 - (int)(top & 255u), E - 1), sub = bi & 3;
     const float mine = (sub == 0) ? ex[0] : (sub == 1) ? ex[1] : (sub == 2) ? ex[2] : ex[3];
-    const float e = __shfl(mine, bi >> 2, 64);
-    if (lane == 0) { inds[k] = bi; scores[k] = f16r(e / Z); }
-    if ((bi >> 2) == lane) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) if (i == sub) lg[i] = NEG;
-    }
+    const float e = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(mine), bi >> 2));
+    sc[k] = f16r(e / Z);
+    if (lane == 0) inds[k] = bi;
   }
   if (lane == 0) {
     float ss = 0.0f;
-    for (int k = 0; k < 8; ++k) ss = f16r(ss + scores[k]);
-    for (int k = 0; k < 8; ++k) scores[k] = f16r(scores[k] / ss);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) ss = f16r(ss + sc[k]);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) scores[k] = f16r(sc[k] / ss);
   }
 }
 
-// MoE stage B: routing + the 8 routed experts' gate/up with SwiGLU.
+// Routing of M rows: one wave per row (softmax, top-8, renormalise; MoEBlock.swift:69-97).
+__global__ __launch_bounds__(64) void k_route_rows(const uint16_t* __restrict__ rlogits, int E, int32_t* __restrict__ inds,
+                                                   uint16_t* __restrict__ scores) {
+  __shared__ int s_inds[8];
+  __shared__ float s_sc[8];
+  const int m = blockIdx.x, lane = threadIdx.x;
+  route_wave(rlogits + (size_t)m * 256, E, lane, s_inds, s_sc);
+  __syncthreads();
+  if (lane < 8) { inds[m * 8 + lane] = s_inds[lane]; scores[m * 8 + lane] = f2h(s_sc[lane]); }
+}
+
+// MoE stage B: the 8 routed experts' gate/up with SwiGLU, after k_route_rows.  A wave owns four consecutive rows of
+// one expert (gate and up); all eight weight loads are in flight before the first dot.  Grid (256, M).
 // Reference: gqmm4_swiglu_rows SeedlessMetalForward.swift:1419-1460.
 struct MoeBArgs {
   const uint16_t* xn;          // [M, 2048] post-normed rows
-  const uint16_t* rlogits;     // [M, 256]
-  int E;
   const uint32_t *g_w, *g_sb, *u_w, *u_sb;   // [E*512, 2048]
   uint16_t* act;               // [M, 8, 512]
-  int32_t* inds;               // [M, 8]
-  uint16_t* scores;            // [M, 8]
+  const int32_t* inds;         // [M, 8]
 };
 __global__ __launch_bounds__(256) void k_moe_b(MoeBArgs a) {
-  __shared__ int s_inds[8];
-  __shared__ float s_sc[8];
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (wave == 0) {
-    route_wave(a.rlogits + (size_t)m * 256, a.E, lane, s_inds, s_sc);
-    if (lane == 0 && blockIdx.x == 0) {
-      for (int k = 0; k < 8; ++k) { a.inds[m * 8 + k] = s_inds[k]; a.scores[m * 8 + k] = f2h(s_sc[k]); }
-    }
+  const int p0 = (blockIdx.x * 4 + wave) * 4;          // row index in [0, 8*512)
+  const int k = p0 >> 9, i0 = p0 & 511;
+  const size_t base = (size_t)a.inds[m * 8 + k] * 512 + i0;
+  uint4 gw[4], uw[4];
+  uint32_t gs[4], us[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    gw[r] = ld16(a.g_w + (base + r) * 256 + 4 * lane); gs[r] = a.g_sb[(base + r) * 32 + (lane >> 1)];
+    uw[r] = ld16(a.u_w + (base + r) * 256 + 4 * lane); us[r] = a.u_sb[(base + r) * 32 + (lane >> 1)];
   }
   float x[32], sx[4];
   load32(a.xn + (size_t)m * H + 32 * lane, x);
   word_sums(x, sx);
   uint32_t xp[16];
   pack_x(x, xp);
-  __syncthreads();
-  const int p0 = (blockIdx.x * 4 + wave) * 2;          // pair index in [0, 8*512)
-  const int k = p0 >> 9, i0 = p0 & 511;
-  const size_t base = (size_t)s_inds[k] * 512 + i0;
-  const size_t rows[2] = {base, base + 1};
-  float g[2], u[2];
-  qdot_rows<1, 2>(a.g_w, a.g_sb, rows, lane, xp, sx, g);
-  qdot_rows<1, 2>(a.u_w, a.u_sb, rows, lane, xp, sx, u);
-  if (lane == 0) {
+  float o[4];
 #pragma unroll
-    for (int r = 0; r < 2; ++r) a.act[((size_t)m * 8 + k) * 512 + i0 + r] = f2h(swiglu16(f16r(g[r]), f16r(u[r])));
+  for (int r = 0; r < 4; ++r) {
+    const float g = tree_sum<64>(quad_term(gw[r], gs[r], xp, sx));
+    const float u = tree_sum<64>(quad_term(uw[r], us[r], xp, sx));
+    o[r] = swiglu16(f16r(g), f16r(u));
   }
+  if (lane == 0)
+    *reinterpret_cast<uint2*>(a.act + ((size_t)m * 8 + k) * 512 + i0) = make_uint2(pack2(o[0], o[1]), pack2(o[2], o[3]));
 }
 
 // MoE stage C: routed down-proj, half-precision combine in routing order, shared down-proj and the
@@ -632,26 +773,47 @@ struct MoeCArgs {
   const uint32_t *shd_w, *shd_sb;   // [2048, 512]
   uint16_t* out;               // [M, 2048]
 };
-__global__ __launch_bounds__(128) void k_moe_c(MoeCArgs a) {
-  const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+// Grid (128, M), four waves: 16 lanes per output row, 16 rows per workgroup.  The word sums of the nine activation
+// rows are formed once per workgroup (LDS); the packed activations are the stored halves as they are.
+__global__ __launch_bounds__(256) void k_moe_c(MoeCArgs a) {
+  __shared__ __align__(16) float s_sx[9 * 16 * 4];
+  const int m = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int sub = lane >> 4, li = lane & 15;
-  const int n = (blockIdx.x * 2 + wave) * 4 + sub;
-  float acc = 0.0f;
-  float x[32], sx[4];
-  uint32_t xp[16];
-#pragma unroll 1
+  const int n = (blockIdx.x * 4 + wave) * 4 + sub;
+  // every load of the eight experts and of the shared expert is issued before the first dot
+  uint4 wv[9];
+  uint32_t sb[9];
+  float sc[8];
+#pragma unroll
   for (int k = 0; k < 8; ++k) {
-    load32(a.act + ((size_t)m * 8 + k) * 512 + 32 * li, x);
-    word_sums(x, sx);
-    pack_x(x, xp);
     const size_t row = (size_t)a.inds[m * 8 + k] * 2048 + n;
-    const float d = f16r(qdot512(a.d_w, a.d_sb, row, li, xp, sx));
-    acc = f16r(acc + f16r(d * h2f(a.scores[m * 8 + k])));
+    wv[k] = ld16(a.d_w + row * 64 + 4 * li);
+    sb[k] = a.d_sb[row * 8 + (li >> 1)];
+    sc[k] = h2f(a.scores[m * 8 + k]);
   }
-  load32(a.sh_act + (size_t)m * 512 + 32 * li, x);
-  word_sums(x, sx);
-  pack_x(x, xp);
-  const float sy = f16r(qdot512(a.shd_w, a.shd_sb, (size_t)n, li, xp, sx));
+  wv[8] = ld16(a.shd_w + (size_t)n * 64 + 4 * li);
+  sb[8] = a.shd_sb[(size_t)n * 8 + (li >> 1)];
+  if (tid < 9 * 16) {
+    const int k = tid >> 4, l = tid & 15;
+    float x[32], sx[4];
+    load32((k < 8 ? a.act + ((size_t)m * 8 + k) * 512 : a.sh_act + (size_t)m * 512) + 32 * l, x);
+    word_sums(x, sx);
+    *reinterpret_cast<float4*>(&s_sx[tid * 4]) = make_float4(sx[0], sx[1], sx[2], sx[3]);
+  }
+  __syncthreads();
+  float acc = 0.0f, sy = 0.0f;
+#pragma unroll
+  for (int k = 0; k < 9; ++k) {
+    const uint16_t* src = (k < 8 ? a.act + ((size_t)m * 8 + k) * 512 : a.sh_act + (size_t)m * 512) + 32 * li;
+    uint32_t xp[16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { const uint4 v = ld16(src + 8 * j); xp[4 * j] = v.x; xp[4 * j + 1] = v.y; xp[4 * j + 2] = v.z; xp[4 * j + 3] = v.w; }
+    const float4 s4 = *reinterpret_cast<const float4*>(&s_sx[(k * 16 + li) * 4]);
+    const float sx[4] = {s4.x, s4.y, s4.z, s4.w};
+    const float d = f16r(tree_sum<16>(quad_term(wv[k], sb[k], xp, sx)));
+    if (k < 8) acc = f16r(acc + f16r(d * sc[k]));
+    else sy = d;
+  }
   const float s = sigmoid16(h2f(a.sgate[m]));
   if (li == 0) a.out[(size_t)m * H + n] = f2h(f16r(acc + f16r(s * sy)));
 }
@@ -717,8 +879,9 @@ __global__ __launch_bounds__(64) void k_attn_prep(AttnPrepArgs a) {
 }
 
 // -------------------------------------------------------------------------------------------------
-// Decode attention, tile pass: one wave per (key tile of 64, kv head, row).  The tile's keys are
-// staged in LDS; lane j scores key j against the 8 query heads of the group (a balanced tree over
+// Decode attention, tile pass: one workgroup of four waves per (key tile of 64, kv head, row), a wave per pair of
+// query heads.  The tile's keys are
+// staged in LDS; lane j scores key j against the query heads of its wave (a balanced tree over
 // 64 leaves of 4 dims), then p = exp(s - tile max), l = butterfly sum of p, o = fmaf chain over
 // the tile's keys with V rows read coalesced.  Reference semantics: sdpa_rows
 // SeedlessMetalForward.swift:4922-4989 (q scaled by 1/16, fp32 softmax).
@@ -732,10 +895,10 @@ struct SdpaArgs {
   float* po;                   // [M, 16, maxTiles, 256]
   const LaneRef* lanes;        // lane batch: row m attends to the cache of lanes[m]
 };
-__global__ __launch_bounds__(64) void k_sdpa_tile(SdpaArgs a) {
+__global__ __launch_bounds__(256) void k_sdpa_tile(SdpaArgs a) {
   __shared__ __align__(16) uint16_t s_k[SDPA_TILE * KT_STRIDE];
   __shared__ __align__(16) float s_q[8 * 256];
-  const int tile = blockIdx.x, kvh = blockIdx.y, m = blockIdx.z, lane = threadIdx.x;
+  const int tile = blockIdx.x, kvh = blockIdx.y, m = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int N = a.st[0] + m + 1;
   if (a.lanes) {
     const LaneRef& r = a.lanes[m];
@@ -746,13 +909,13 @@ __global__ __launch_bounds__(64) void k_sdpa_tile(SdpaArgs a) {
   const int nk = min(SDPA_TILE, N - j0);
   const uint16_t* kbase = a.kcache + ((size_t)kvh * a.maxSeq + j0) * 256;
   const uint16_t* vbase = a.vcache + ((size_t)kvh * a.maxSeq + j0) * 256;
-  // stage keys (rows >= nk are never read) and the group's 8 scaled queries
-  for (int it = 0; it < 32; ++it) {
-    const int row = it * 2 + (lane >> 5), c8 = (lane & 31) * 8;
+  // stage keys (rows >= nk are never read) and the group's 8 scaled queries; wave w then owns heads 2w, 2w+1
+  for (int it = 0; it < 8; ++it) {
+    const int row = it * 8 + (tid >> 5), c8 = (tid & 31) * 8;
     if (row < nk) st16(&s_k[row * KT_STRIDE + c8], ld16(kbase + (size_t)row * 256 + c8));
   }
-  for (int it = 0; it < 4; ++it) {
-    const int idx = (it * 64 + lane) * 8;            // 0..2047 step 8
+  {
+    const int idx = tid * 8;                         // 0..2047 step 8
     float f[8];
     unpack8(ld16(a.qrot + ((size_t)m * 16 + kvh * 8) * 256 + idx), f);
 #pragma unroll
@@ -760,55 +923,67 @@ __global__ __launch_bounds__(64) void k_sdpa_tile(SdpaArgs a) {
   }
   __syncthreads();
   const float NEG = -__int_as_float(0x7f800000);
-  float sc[8];
+  const int h0 = 2 * wave;
+  // scores: a balanced tree over 64 leaves of 4 dims, eight leaves (one sub-tree) at a time so that the staged
+  // key row is read in step with its use
+  float sc[2];
   {
-    float stk[8][7];
+    float grp[2][8];
     const uint16_t* kr = &s_k[(lane < nk ? lane : 0) * KT_STRIDE];
 #pragma unroll
-    for (int leaf = 0; leaf < 64; ++leaf) {
-      const uint2 kraw = *reinterpret_cast<const uint2*>(kr + 4 * leaf);
-      const float kf[4] = {lo_h(kraw.x), hi_h(kraw.x), lo_h(kraw.y), hi_h(kraw.y)};
+    for (int g = 0; g < 8; ++g) {
+      float n[2][8];
 #pragma unroll
-      for (int h = 0; h < 8; ++h) {
-        const float4 q4 = *reinterpret_cast<const float4*>(&s_q[h * 256 + 4 * leaf]);
-        float node = fmaf(q4.x, kf[0], 0.0f);
-        node = fmaf(q4.y, kf[1], node);
-        node = fmaf(q4.z, kf[2], node);
-        node = fmaf(q4.w, kf[3], node);
-        int c = leaf, lvl = 0;
-        while (c & 1) { node = stk[h][lvl] + node; c >>= 1; ++lvl; }
-        stk[h][lvl] = node;
+      for (int l = 0; l < 8; ++l) {
+        const int leaf = 8 * g + l;
+        const uint2 kraw = *reinterpret_cast<const uint2*>(kr + 4 * leaf);
+        const float kf[4] = {lo_h(kraw.x), hi_h(kraw.x), lo_h(kraw.y), hi_h(kraw.y)};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const float4 q4 = *reinterpret_cast<const float4*>(&s_q[(h0 + h) * 256 + 4 * leaf]);
+          float node = fmaf(q4.x, kf[0], 0.0f);
+          node = fmaf(q4.y, kf[1], node);
+          node = fmaf(q4.z, kf[2], node);
+          n[h][l] = fmaf(q4.w, kf[3], node);
+        }
       }
+#pragma unroll
+      for (int h = 0; h < 2; ++h) grp[h][g] = ((n[h][0] + n[h][1]) + (n[h][2] + n[h][3])) + ((n[h][4] + n[h][5]) + (n[h][6] + n[h][7]));
+      asm volatile("" : "+v"(grp[0][g]), "+v"(grp[1][g]) : : "memory");   // both heads' sub-trees end here: nothing is carried along
     }
 #pragma unroll
-    for (int h = 0; h < 8; ++h) sc[h] = (lane < nk) ? stk[h][6] : NEG;
+    for (int h = 0; h < 2; ++h) {
+      const float t = ((grp[h][0] + grp[h][1]) + (grp[h][2] + grp[h][3])) + ((grp[h][4] + grp[h][5]) + (grp[h][6] + grp[h][7]));
+      sc[h] = (lane < nk) ? t : NEG;
+    }
   }
-  float p[8], o[8][4];
+  float p[2], o[2][4];
 #pragma unroll
-  for (int h = 0; h < 8; ++h) {
+  for (int h = 0; h < 2; ++h) {
     const float mx = tree_max<64>(sc[h]);
     p[h] = (lane < nk) ? exp_c(sc[h] - mx) : 0.0f;
     const float l = tree_sum<64>(p[h]);
     if (lane == 0) {
-      const size_t pi = ((size_t)m * 16 + kvh * 8 + h) * a.maxTiles + tile;
+      const size_t pi = ((size_t)m * 16 + kvh * 8 + h0 + h) * a.maxTiles + tile;
       a.pm[pi] = mx; a.pl[pi] = l;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) o[h][i] = 0.0f;
   }
+#pragma unroll 8
   for (int j = 0; j < nk; ++j) {
     const uint2 vraw = *reinterpret_cast<const uint2*>(vbase + (size_t)j * 256 + 4 * lane);
     const float vf[4] = {lo_h(vraw.x), hi_h(vraw.x), lo_h(vraw.y), hi_h(vraw.y)};
 #pragma unroll
-    for (int h = 0; h < 8; ++h) {
+    for (int h = 0; h < 2; ++h) {
       const float pj = __shfl(p[h], j, 64);
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[h][i] = fmaf(pj, vf[i], o[h][i]);
     }
   }
 #pragma unroll
-  for (int h = 0; h < 8; ++h) {
-    const size_t pi = ((size_t)m * 16 + kvh * 8 + h) * a.maxTiles + tile;
+  for (int h = 0; h < 2; ++h) {
+    const size_t pi = ((size_t)m * 16 + kvh * 8 + h0 + h) * a.maxTiles + tile;
     *reinterpret_cast<float4*>(a.po + pi * 256 + 4 * lane) = make_float4(o[h][0], o[h][1], o[h][2], o[h][3]);
   }
 }

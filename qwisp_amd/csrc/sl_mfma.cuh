@@ -209,16 +209,6 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
   }
 }
 
-// Routing of M rows on its own (the GEMV path routes inside its gate/up kernel): one wave per row.
-__global__ __launch_bounds__(64) void k_route_rows(const uint16_t* __restrict__ rlogits, int E, int32_t* __restrict__ inds,
-                                                   uint16_t* __restrict__ scores) {
-  __shared__ int s_inds[8];
-  __shared__ float s_sc[8];
-  const int m = blockIdx.x, lane = threadIdx.x;
-  route_wave(rlogits + (size_t)m * 256, E, lane, s_inds, s_sc);
-  __syncthreads();
-  if (lane < 8) { inds[m * 8 + lane] = s_inds[lane]; scores[m * 8 + lane] = f2h(s_sc[lane]); }
-}
 // Pairs (row, slot) listed per expert (M * 8 <= 4096 pairs over 1024 threads), places handed out by LDS counters.
 // The order within a list varies from run to run; results do not depend on it (they are scattered back by pair).
 __global__ __launch_bounds__(1024) void k_group_pairs(const int32_t* __restrict__ inds, int M, int E, uint16_t* __restrict__ lists,
