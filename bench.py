@@ -56,6 +56,11 @@ def main():
     ap.add_argument("--prefill-chunk", type=int, default=0, metavar="M",
                     help="also time the 512-token prefill in chunks of M rows, exact rows and hybrid (matrix cores), on lanes "
                          "of the same weights (extra object in the JSON line)")
+    ap.add_argument("--prefill-tokens", type=int, default=PROMPT_LEN, metavar="N",
+                    help="prompt length of the --prefill-chunk measurement (the reference's batched configuration uses 2048)")
+    ap.add_argument("--verify-rows", type=int, default=0, metavar="R",
+                    help="also time verify steps of R rows ([token] + R-1 drafts through stepArgmax) at the decode context "
+                         "(extra object in the JSON line)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run a plain device copy of this many MiB (reference for rocprofv3 FETCH_SIZE/WRITE_SIZE) and exit")
     args = ap.parse_args()
@@ -83,7 +88,7 @@ def main():
     t0 = time.time()
     dev = synth.generate_device(cfg, lib.get())
     t_gen = time.time() - t0
-    max_seq = PROMPT_LEN + args.warmup + args.steps + 16
+    max_seq = PROMPT_LEN + args.warmup + args.steps + 16 + 24 * max(args.verify_rows, 0)
     eng = SeedlessFusedForward(cfg, dev, max_m=64, max_seq_len=max_seq)
     host = None
     if args.cpu_tokens > 0:
@@ -158,22 +163,43 @@ def main():
         for lane in lanes:
             lane.close()
 
+    verify_report = None
+    if args.verify_rows > 1:
+        R = args.verify_rows
+        rng = np.random.default_rng(5000)
+        reps = 16
+        rows = [np.concatenate([[cur], rng.integers(0, cfg.vocab, R - 1)]).astype(np.int32) for _ in range(reps + 4)]
+        for r in rows[:4]:
+            assert eng.step_argmax(r) is not None, eng.gpu_fault
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for r in rows[4:]:
+            o = eng.step_argmax(r)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert o is not None, eng.gpu_fault
+        verify_report = {"rows": R, "ms_per_step": dt * 1e3 / reps, "ms_per_row": dt * 1e3 / reps / R,
+                         "context": PROMPT_LEN + args.warmup + args.steps + 4 * R,
+                         "path": "rows of the kernel-per-stage path; every row accepted (the context advances R per step)"}
+
     prefill_report = None
     if args.prefill_chunk > 0:
-        prefill_report = {"prompt": PROMPT_LEN, "chunk_rows": args.prefill_chunk}
+        PF = args.prefill_tokens
+        pf_prompt = np.random.default_rng(3000).integers(0, cfg.vocab, PF).astype(np.int32)
+        prefill_report = {"prompt": PF, "chunk_rows": args.prefill_chunk}
         for name, hyb in (("exact_rows", False), ("hybrid_matrix_cores", True)):
             times = []
             for rep in range(2):                           # the first pass warms code and caches
-                lane = eng.new_lane(max_m=args.prefill_chunk, max_seq_len=PROMPT_LEN + 8)
+                lane = eng.new_lane(max_m=args.prefill_chunk, max_seq_len=PF + 8)
                 lane.set_hybrid(hyb)
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
-                o = lane.greedy_generate(prompt, 1, chain_k=1)
+                o = lane.greedy_generate(pf_prompt, 1, chain_k=1)
                 torch.cuda.synchronize()
                 times.append(time.perf_counter() - t0)
                 assert o is not None, lane.gpu_fault
                 lane.close()
-            prefill_report[name] = {"ms": times[-1] * 1e3, "tok_s": PROMPT_LEN / times[-1]}
+            prefill_report[name] = {"ms": times[-1] * 1e3, "tok_s": PF / times[-1]}
 
     cpu = None
     if host is not None:
@@ -208,6 +234,7 @@ def main():
         "cpu_baseline": cpu,
         "lane_batch": lanes_report,
         "prefill": prefill_report,
+        "verify": verify_report,
         "setup_s": {"generate": t_gen, "prefill_512": t_prefill},
         "tokens_head": stream[:8],
     }))

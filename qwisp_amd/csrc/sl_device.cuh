@@ -150,6 +150,11 @@ SL_DEV uint4 pack8(const float* f) {
   return make_uint4(pack2(f[0], f[1]), pack2(f[2], f[3]), pack2(f[4], f[5]), pack2(f[6], f[7]));
 }
 
+// A pointer read from device memory (a table of per-sequence buffers) is device memory itself: saying so lets the
+// compiler use global instead of generic ("flat") accesses through it.
+template <class T>
+SL_DEV T* as_global(T* p) { return (T*)(T __attribute__((address_space(1)))*)(unsigned long long)p; }
+
 // ---- one packed word against 8 activations ---------------------------------------------------------
 // The 8 activations arrive as 4 packed half pairs.  Masking the word with 0x000F000F leaves two
 // halves whose bit patterns are the nibbles j and j+4: as (subnormal) half values they equal

@@ -327,31 +327,54 @@ struct GdnArgs {
   const LaneRef* lanes;      // lane batch: blockIdx.y = lane, one row each, caches and parity of that lane
   int layer;
 };
-SL_DEV float conv_tap(const GdnArgs& a, const uint16_t* hin, int row, int ch) {
+SL_DEV float conv_tap(const uint16_t* proj, const uint16_t* hin, int row, int ch) {
   // row of the concatenation [hist(3) | qkv(M)]
-  return (row < 3) ? h2f(hin[row * SL_CONV_DIM + ch]) : h2f(a.proj[(size_t)(row - 3) * PROJ_STRIDE + ch]);
+  return (row < 3) ? h2f(hin[row * SL_CONV_DIM + ch]) : h2f(proj[(size_t)(row - 3) * PROJ_STRIDE + ch]);
 }
-SL_DEV float conv_silu(const GdnArgs& a, const uint16_t* hin, int t, int ch) {
+SL_DEV float conv_silu(const uint16_t* proj, const float* conv_w, const uint16_t* hin, int t, int ch) {
   float acc = 0.0f;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) acc = fmaf(conv_tap(a, hin, t + k, ch), a.conv_w[ch * 4 + k], acc);
+  for (int k = 0; k < 4; ++k) acc = fmaf(conv_tap(proj, hin, t + k, ch), conv_w[ch * 4 + k], acc);
   return f16r(acc * sigmoid32(acc));
+}
+// The ping-pong sides of the conv history and the recurrent state, and the rows a workgroup works on: of the
+// engine's own sequence, or (lane batch) of lane blockIdx.y.  Plain selects: the argument struct is never indexed
+// with a run-time value nor written, so it stays in scalar registers.
+struct GdnView {
+  const uint16_t* hin; uint16_t* hout;
+  const float* sin_; float* sout;
+  const uint16_t* proj; uint16_t* ycore;
+  int M;
+};
+SL_DEV GdnView gdn_view(const GdnArgs& a, int lane_row) {
+  GdnView v;
+  const uint16_t *h0 = a.hist[0], *h1 = a.hist[1];
+  const float *s0 = a.state[0], *s1 = a.state[1];
+  const int32_t* st = a.st;
+  v.proj = a.proj; v.ycore = a.ycore; v.M = a.M;
+  if (a.lanes) {
+    const LaneRef& r = a.lanes[lane_row];
+    h0 = as_global(r.hist[0]); h1 = as_global(r.hist[1]); s0 = as_global(r.state[0]); s1 = as_global(r.state[1]);
+    st = as_global(r.st) + a.layer;
+    v.proj += (size_t)lane_row * PROJ_STRIDE; v.ycore += (size_t)lane_row * 4096; v.M = 1;
+  }
+  const bool par = st[1] != 0;
+  v.hin = par ? h1 : h0; v.hout = const_cast<uint16_t*>(par ? h0 : h1);
+  v.sin_ = par ? s1 : s0; v.sout = const_cast<float*>(par ? s0 : s1);
+  return v;
 }
 __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
   __shared__ float s_q[128], s_k[128], s_v[16], s_gb[2];
-  if (a.lanes) {
-    const LaneRef& r = a.lanes[blockIdx.y];
-    a.hist[0] = r.hist[0]; a.hist[1] = r.hist[1]; a.state[0] = r.state[0]; a.state[1] = r.state[1];
-    a.st = r.st + a.layer;
-    a.proj += (size_t)blockIdx.y * PROJ_STRIDE; a.ycore += (size_t)blockIdx.y * 4096; a.M = 1;
-  }
+  const GdnView vw = gdn_view(a, blockIdx.y);
+  const uint16_t* hin = vw.hin;
+  uint16_t* hout = vw.hout;
+  const float* sin_ = vw.sin_;
+  float* sout = vw.sout;
+  const uint16_t* proj = vw.proj;
+  uint16_t* ycore = vw.ycore;
+  const int M = vw.M;
   const int hv = blockIdx.x >> 3, dvb = blockIdx.x & 7, hk = hv >> 1;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
-  const int par = a.st[1];
-  const uint16_t* hin = a.hist[par];
-  uint16_t* hout = a.hist[par ^ 1];
-  const float* sin_ = a.state[par];
-  float* sout = a.state[par ^ 1];
 
   float s[2][4];
 #pragma unroll
@@ -363,10 +386,10 @@ __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
   const int qk_ch = (tid < 128) ? (hk * 128 + tid) : (2048 + hk * 128 + (tid - 128));
   const int v_ch = 4096 + hv * 128 + dvb * 16 + (tid & 15);
 
-  for (int t = 0; t < a.M; ++t) {
-    const float c = conv_silu(a, hin, t, qk_ch);
+  for (int t = 0; t < M; ++t) {
+    const float c = conv_silu(proj, a.conv_w, hin, t, qk_ch);
     if (tid < 128) s_q[tid] = c; else s_k[tid - 128] = c;
-    if (tid < 16) s_v[tid] = conv_silu(a, hin, t, v_ch);
+    if (tid < 16) s_v[tid] = conv_silu(proj, a.conv_w, hin, t, v_ch);
     __syncthreads();
     if (wave < 2) {
       // weightless rmsnorm over 128, then the key/query scale, both rounded to half
@@ -379,8 +402,8 @@ __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
       const float y0 = f16r(sc * f16r(x0 * inv)), y1 = f16r(sc * f16r(x1 * inv));
       buf[2 * lane] = y0; buf[2 * lane + 1] = y1;
     } else if (tid == 128) {
-      const float bP = h2f(a.proj[(size_t)t * PROJ_STRIDE + 12288 + hv]);
-      const float aP = h2f(a.proj[(size_t)t * PROJ_STRIDE + 12320 + hv]);
+      const float bP = h2f(proj[(size_t)t * PROJ_STRIDE + 12288 + hv]);
+      const float aP = h2f(proj[(size_t)t * PROJ_STRIDE + 12320 + hv]);
       s_gb[0] = exp_c(-(exp_c(a.a_log[hv]) * softplus_c(aP + a.dt_bias[hv])));
       s_gb[1] = sigmoid16(bP);
     }
@@ -401,7 +424,7 @@ __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) { s[it][i] = fmaf(kk[i], delta, s[it][i]); acc = fmaf(s[it][i], qq[i], acc); }
       const float y = tree_sum<32>(acc);
-      if (l32 == 0) a.ycore[(size_t)t * 4096 + hv * 128 + dvb * 16 + dvl] = f2h(y);
+      if (l32 == 0) ycore[(size_t)t * 4096 + hv * 128 + dvb * 16 + dvl] = f2h(y);
     }
     __syncthreads();
   }
@@ -413,11 +436,11 @@ __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
   // history shift: rows M..M+2 of [hist | qkv]; each channel written by exactly one workgroup
   if ((hv & 1) == 0 && dvb == 0) {
 #pragma unroll
-    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + qk_ch] = f2h(conv_tap(a, hin, a.M + j, qk_ch));
+    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + qk_ch] = f2h(conv_tap(proj, hin, M + j, qk_ch));
   }
   if (tid < 16) {
 #pragma unroll
-    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + v_ch] = f2h(conv_tap(a, hin, a.M + j, v_ch));
+    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + v_ch] = f2h(conv_tap(proj, hin, M + j, v_ch));
   }
 }
 
@@ -437,11 +460,11 @@ struct GdnPrepArgs {
 __global__ __launch_bounds__(64) void k_gdn_prep_rows(GdnPrepArgs p) {
   const GdnArgs& a = p.g;
   const int u = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
-  const uint16_t* hin = a.hist[a.st[1]];
+  const uint16_t* hin = a.st[1] ? a.hist[1] : a.hist[0];
   if (u < 32) {
     const bool isk = u >= 16;
     const int ch = (isk ? 2048 : 0) + (u & 15) * 128 + 2 * lane;
-    const float x0 = conv_silu(a, hin, t, ch), x1 = conv_silu(a, hin, t, ch + 1);
+    const float x0 = conv_silu(a.proj, a.conv_w, hin, t, ch), x1 = conv_silu(a.proj, a.conv_w, hin, t, ch + 1);
     float ss = fmaf(x1, x1, fmaf(x0, x0, 0.0f));
     ss = tree_sum<64>(ss);
     const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
@@ -451,7 +474,7 @@ __global__ __launch_bounds__(64) void k_gdn_prep_rows(GdnPrepArgs p) {
   } else if (u < 64) {
     const int ch = 4096 + (u - 32) * 128 + 2 * lane;
     *reinterpret_cast<uint32_t*>(p.vc + (size_t)t * 4096 + (u - 32) * 128 + 2 * lane) =
-        pack2(conv_silu(a, hin, t, ch), conv_silu(a, hin, t, ch + 1));
+        pack2(conv_silu(a.proj, a.conv_w, hin, t, ch), conv_silu(a.proj, a.conv_w, hin, t, ch + 1));
   } else {
     const int hv = lane & 31;
     if (lane < 32) {
@@ -468,11 +491,11 @@ __global__ __launch_bounds__(256) void k_gdn_scan_rows(GdnPrepArgs p) {
   const GdnArgs& a = p.g;
   const int hv = blockIdx.x >> 3, dvb = blockIdx.x & 7, hk = hv >> 1;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
-  const int par = a.st[1];
-  const uint16_t* hin = a.hist[par];
-  uint16_t* hout = a.hist[par ^ 1];
-  const float* sin_ = a.state[par];
-  float* sout = a.state[par ^ 1];
+  const bool par = a.st[1] != 0;
+  const uint16_t* hin = par ? a.hist[1] : a.hist[0];
+  uint16_t* hout = par ? a.hist[0] : a.hist[1];
+  const float* sin_ = par ? a.state[1] : a.state[0];
+  float* sout = par ? a.state[0] : a.state[1];
   float s[2][4];
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
@@ -521,11 +544,11 @@ __global__ __launch_bounds__(256) void k_gdn_scan_rows(GdnPrepArgs p) {
   const int v_ch = 4096 + hv * 128 + dvb * 16 + (tid & 15);
   if ((hv & 1) == 0 && dvb == 0) {
 #pragma unroll
-    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + qk_ch] = f2h(conv_tap(a, hin, a.M + j, qk_ch));
+    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + qk_ch] = f2h(conv_tap(a.proj, hin, a.M + j, qk_ch));
   }
   if (tid < 16) {
 #pragma unroll
-    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + v_ch] = f2h(conv_tap(a, hin, a.M + j, v_ch));
+    for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + v_ch] = f2h(conv_tap(a.proj, hin, a.M + j, v_ch));
   }
 }
 
