@@ -277,6 +277,21 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   c.d_w = L.sw_down.w; c.d_sb = L.sw_down.sb; c.shd_w = L.sh_down.w; c.shd_sb = L.sh_down.sb; c.out = e->moe_out;
   hipLaunchKernelGGL(k_moe_c, dim3(128, M), dim3(256), 0, e->stream, c);
 }
+// In-projection of M >= 2 rows: residual + norm once per row, then the row-tiled projection into e->proj.  Workgroups
+// of 16 weight rows, three to a compute unit: when the count is just over a multiple of the machine's 768 places the
+// surplus rows go one each to the first workgroups instead of opening another round.
+void launch_hidden_tile(sl_engine* e, const HiddenArgs& ha, const uint32_t* w, const uint32_t* sb, int N, int M) {
+  HiddenArgs hn = ha;
+  hn.xn_out = e->xn;
+  hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
+  constexpr int PLACES = 768;
+  int G = N / 16;
+  const int over = G % PLACES;
+  if (G > PLACES && over <= 16) G -= over;
+  if (G * 16 + G < N) G = (N + 15) / 16;          // (not with the shapes of this model)
+  hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, false>), dim3(G, (M + 7) / 8), dim3(256), 0, e->stream, HiddenArgs{}, e->xn, H,
+                     w, sb, N, e->proj, PROJ_STRIDE, M);
+}
 // Hybrid prefill: chunks of at least 16 rows of one sequence take the dense mixer projections to the matrix cores.
 bool use_matrix_cores(const sl_engine* e, int M, const LaneRef* lanes) { return e->hybrid && !lanes && M >= 16 && M <= GROUP_CAP; }
 // `lanes` (null for rows of one sequence) = this layer's row of the lane table: row b of the batch is lane b's next token.
@@ -287,8 +302,7 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
     hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
     launch_qmm4_mfma(QmmArgs{e->xn, H, L.in_proj.w, L.in_proj.sb, M, SL_GDN_IN_N, H, e->proj, PROJ_STRIDE}, e->stream);
   } else if (M >= 2) {
-    hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, true>), dim3(SL_GDN_IN_N / 32, (M + 7) / 8), dim3(512), 0, e->stream, ha, (const uint16_t*)nullptr, 0,
-                       L.in_proj.w, L.in_proj.sb, SL_GDN_IN_N, e->proj, PROJ_STRIDE, M);
+    launch_hidden_tile(e, ha, L.in_proj.w, L.in_proj.sb, SL_GDN_IN_N, M);
   } else {
     hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_GDN_IN_N / 16, M), dim3(256), 0, e->stream, ha, L.in_proj.w, L.in_proj.sb,
                        SL_GDN_IN_N, e->proj, PROJ_STRIDE);
@@ -326,8 +340,7 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
     hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
     launch_qmm4_mfma(QmmArgs{e->xn, H, L.qkv.w, L.qkv.sb, M, SL_ATT_QKV_N, H, e->proj, PROJ_STRIDE}, e->stream);
   } else if (M >= 2) {
-    hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, true>), dim3(SL_ATT_QKV_N / 32, (M + 7) / 8), dim3(512), 0, e->stream, ha, (const uint16_t*)nullptr, 0,
-                       L.qkv.w, L.qkv.sb, SL_ATT_QKV_N, e->proj, PROJ_STRIDE, M);
+    launch_hidden_tile(e, ha, L.qkv.w, L.qkv.sb, SL_ATT_QKV_N, M);
   } else {
     hipLaunchKernelGGL(k_qmv_hidden<4>, dim3(SL_ATT_QKV_N / 16, M), dim3(256), 0, e->stream, ha, L.qkv.w, L.qkv.sb,
                        SL_ATT_QKV_N, e->proj, PROJ_STRIDE);

@@ -185,12 +185,15 @@ __global__ __launch_bounds__(256) void k_qmv_plain(const uint16_t* __restrict__ 
 // packing: wave w takes rows w, w + waves, ...) and parked in LDS, 20 words per lane (16 packed pairs, 4 sums)
 // so that a lane reads back its own 80 bytes with five 16-byte reads free of bank conflicts.
 // HIDDEN: x comes from the hidden prologue (K = 2048); otherwise from the fp16 buffer xin (K = 2048*NBLK).
-// Grid (ceil(N / (waves*R)), ceil(M / MT)), any multiple of 64 threads up to 512.
+// Grid (G, ceil(M / MT)); up to 8 waves with the hidden prologue, 4 without (three workgroups share a compute
+// unit).  G workgroups cover G*waves*R rows; rows beyond that (fewer than G) are taken one each by wave 0 of the
+// first workgroups, so that G can be chosen to fill the machine exactly once (12352 rows: 768 workgroups of 16
+// rows + 64 single rows, instead of 772 workgroups on 768 places).
 // -------------------------------------------------------------------------------------------------
 // ARGMAX (lm_head, R = 4, 4 waves): y is the logits matrix and every workgroup also leaves one (value, index)
 // candidate per activation row, the first maximum of its 16 rounded logits, for k_argmax_final.
 template <int NBLK, int R, int MT, bool HIDDEN, bool ARGMAX = false>
-__global__ __launch_bounds__(512) void k_qmv_tile(HiddenArgs ha, const uint16_t* __restrict__ xin, int x_stride,
+__global__ __launch_bounds__(HIDDEN ? 512 : 256, HIDDEN ? 2 : 3) void k_qmv_tile(HiddenArgs ha, const uint16_t* __restrict__ xin, int x_stride,
                                                   const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB,
                                                   int N, uint16_t* __restrict__ y, int y_stride, int M,
                                                   float* __restrict__ cand_v = nullptr, int32_t* __restrict__ cand_i = nullptr) {
@@ -216,6 +219,8 @@ __global__ __launch_bounds__(512) void k_qmv_tile(HiddenArgs ha, const uint16_t*
         sb[r][b] = SB[(row0 + r) * GPR + b * 32 + (lane >> 1)];
       }
   }
+  const size_t xrow = (size_t)gridDim.x * waves * R + blockIdx.x;      // this workgroup's single row beyond the grid's cover
+  const bool extra = !ARGMAX && wave == 0 && xrow < (size_t)N;
   for (int m = wave; m < mc; m += waves) {
 #pragma unroll
     for (int b = 0; b < NBLK; ++b) {
@@ -281,6 +286,33 @@ __global__ __launch_bounds__(512) void k_qmv_tile(HiddenArgs ha, const uint16_t*
     } else if (lane == 0) {
 #pragma unroll
       for (int r = 0; r < R; ++r) y[(size_t)(m0 + m) * y_stride + row0 + r] = f2h(out[r]);
+    }
+  }
+  if (extra) {
+    uint4 wx[NBLK];
+    uint32_t sbx[NBLK];
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b) { wx[b] = ld16(W + xrow * WPR + b * 256 + 4 * lane); sbx[b] = SB[xrow * GPR + b * 32 + (lane >> 1)]; }
+    h2_t mx[NBLK][16];
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b) {
+      word_masks(wx[b].x, mx[b]); word_masks(wx[b].y, mx[b] + 4); word_masks(wx[b].z, mx[b] + 8); word_masks(wx[b].w, mx[b] + 12);
+    }
+    for (int m = 0; m < mc; ++m) {
+      float acc = 0.0f;
+#pragma unroll
+      for (int b = 0; b < NBLK; ++b) {
+        const uint4* src = xs + ((m * NBLK + b) * 64 + lane) * 5;
+        uint32_t xp[16];
+        float sx[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { const uint4 v = src[j]; xp[4 * j] = v.x; xp[4 * j + 1] = v.y; xp[4 * j + 2] = v.z; xp[4 * j + 3] = v.w; }
+        { const uint4 v = src[4]; sx[0] = __uint_as_float(v.x); sx[1] = __uint_as_float(v.y); sx[2] = __uint_as_float(v.z); sx[3] = __uint_as_float(v.w); }
+        const float t = quad_term_masked(mx[b], sbx[b], xp, sx);
+        acc = (b == 0) ? t : acc + t;
+      }
+      const float o = tree_sum<64>(acc);
+      if (lane == 0) y[(size_t)(m0 + m) * y_stride + xrow] = f2h(o);
     }
   }
   if constexpr (ARGMAX) {
