@@ -3,11 +3,11 @@
 // SeedlessFusedVerify.swift:4240-4247).
 //
 //   Y[m, n] = half( sum_k X[m, k] * half(s * q + b) ),  X fp16 [M, K], W MLX-affine 4-bit group 64 [N, K],
-//   the weight formed in half arithmetic (one fused multiply-add), fp32 accumulation in v_mfma_f32_32x32x8_f16.
+//   the weight formed in half arithmetic (one fused multiply-add), fp32 accumulation in v_mfma_f32_32x32x16_f16.
 //
-// A wave owns a 32x32 tile of Y (32 rows of X against 32 weight rows): it walks K in chunks of 64 (one
-// quantisation group), dequantises its 4 weights per MFMA step in registers and feeds them as the B operand;
-// the X chunk [M, 64] is staged in LDS by the whole workgroup (double-buffered, one barrier per chunk) and
+// A wave owns 32x32 tiles of Y (32 rows of X against a strip of 32 weight rows): it walks K in chunks of 64 (one
+// quantisation group), dequantises its 8 weights per MFMA step in registers and feeds them as the B operand;
+// the X chunk [rows, 64] is staged in LDS by the whole workgroup (double-buffered, one barrier per chunk) and
 // read as the A operand.  A row's result depends only on that row of X and on W, and K is walked in a fixed
 // order, so the result is independent of M and of the chunking of a prompt.
 #pragma once
@@ -18,25 +18,11 @@
 
 namespace sl {
 
-typedef _Float16 mf_h4 __attribute__((ext_vector_type(4)));
 typedef float mf_f16v __attribute__((ext_vector_type(16)));
 typedef _Float16 mf_h2 __attribute__((ext_vector_type(2)));
 
-// Dequantisation of a lane's 4 weights of an MFMA step in packed half arithmetic.  `wsh` holds two nibble pairs
-// (bits 0-7 and 16-23).  or-ing a nibble into the mantissa of 1024.0 gives 1024 + q exactly, subtracting 1024
-// gives q exactly, and half(q * s + b) is one fused multiply-add per pair.  The four results belong to the
-// nibbles {a, a+4, a+1, a+5} of the word (a = 0 or 2), which is the order the X chunk is staged in.
-SL_DEV mf_h4 dequant4(uint32_t wsh, mf_h2 s2, mf_h2 b2) {
-  const mf_h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
-  const mf_h2 q0 = __builtin_bit_cast(mf_h2, (wsh & 0x000F000Fu) | 0x64006400u) - k1024;
-  const mf_h2 q1 = __builtin_bit_cast(mf_h2, ((wsh >> 4) & 0x000F000Fu) | 0x64006400u) - k1024;
-  const mf_h2 w0 = __builtin_elementwise_fma(q0, s2, b2), w1 = __builtin_elementwise_fma(q1, s2, b2);
-  mf_h4 r;
-  r[0] = w0[0]; r[1] = w0[1]; r[2] = w1[0]; r[3] = w1[1];
-  return r;
-}
-// The 8 halves of a staged 16-byte piece (k = 8j .. 8j+7) in the order {0,4,1,5, 2,6,3,7}: positions 0-3 are read
-// by the lanes of the lower half-wave, 4-7 by the upper, matching dequant4.
+// The 8 halves of a staged 16-byte piece (k = 8j .. 8j+7) in the order {0,4,1,5, 2,6,3,7}, the order in which
+// dequant8 delivers the 8 nibbles of a packed word.
 SL_DEV uint4 permute8(uint4 v) {
   return make_uint4((v.x & 0xffffu) | (v.z << 16), (v.x >> 16) | (v.z & 0xffff0000u),
                     (v.y & 0xffffu) | (v.w << 16), (v.y >> 16) | (v.w & 0xffff0000u));
@@ -47,81 +33,124 @@ struct QmmArgs {
   int x_stride;
   const uint32_t* W;     // [N, K/8] packed
   const uint32_t* SB;    // [N, K/64] {scale, bias}
-  int M, N, K;           // N % 32 == 0, K % 64 == 0, M <= 128
+  int M, N, K;           // N % 32 == 0, K % 64 == 0
   uint16_t* y;           // [M, y_stride] fp16
   int y_stride;
 };
 
-constexpr int QMM_XS = 72;   // halves per staged X row: 64 + 8 pad (rows 144 bytes apart spread over the LDS banks)
 
-// WM = number of 32-row tiles of X, spread over the waves of a workgroup: wave = (strip of the workgroup, row
-// tile), 4 / WM strips per workgroup.  Every wave holds one 32x32 accumulator; the waves of a strip read the same
-// weights (from cache) and dequantise them again, which costs less than the latency of a lone wave per SIMD.
-template <int WM>
-__global__ __launch_bounds__(256) void k_qmm4_mfma(QmmArgs a) {
-  __shared__ __align__(16) uint16_t xs[2][WM * 32 * QMM_XS];
+// -------------------------------------------------------------------------------------------------
+// The dense projections of a chunk: v_mfma_f32_32x32x16_f16, RT row tiles per wave.  A wave owns a strip of 32
+// weight rows and RT x 32 rows of X (RT accumulators): it dequantises the 8 weights of a step once and feeds them
+// to RT matrix instructions, so the unpacking is shared by up to 128 rows of X; the four waves of a workgroup take
+// four neighbouring strips and read the same staged X chunk.  Grid (ceil(N / 128), ceil(M / (32*RT))).
+// Operands of a step (16 values of k): lane (col, hh) brings k = 8*hh .. 8*hh+7 of its row (A) / weight row (B),
+// i.e. one packed word of the weight row; the order within the eight is {0,4,1,5,2,6,3,7} on both sides.
+// -------------------------------------------------------------------------------------------------
+// Dequantisation of a packed word (8 weights) in packed half arithmetic: masking with 0x000F000F leaves the nibbles
+// j and j+4; or-ing a nibble into the mantissa of 1024.0 gives 1024 + q exactly, subtracting 1024 gives q exactly,
+// and half(q * s + b) is one fused multiply-add per pair.
+typedef _Float16 mf_h8 __attribute__((ext_vector_type(8)));
+SL_DEV mf_h8 dequant8(uint32_t w, mf_h2 s2, mf_h2 b2) {
+  const mf_h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+  mf_h8 r;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const mf_h2 q = __builtin_bit_cast(mf_h2, ((w >> (4 * j)) & 0x000F000Fu) | 0x64006400u) - k1024;
+    const mf_h2 v = __builtin_elementwise_fma(q, s2, b2);
+    r[2 * j] = v[0]; r[2 * j + 1] = v[1];
+  }
+  return r;
+}
+template <int RT, int G>      // G quantisation groups (64 k) per staged chunk and barrier; K % (64*G) == 0
+__global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
+  constexpr int XS = 64 * G + 8;                         // halves per staged row (rows 16 bytes off a multiple of 128)
+  __shared__ __align__(16) uint16_t xs[2][RT * 32 * XS];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, hh = lane >> 5;
-  const int mt = wave % WM;
-  const int n0 = (blockIdx.x * (4 / WM) + wave / WM) * 32;
-  const bool live = n0 < a.N && mt * 32 < a.M;          // a workgroup's last waves may have no strip or no rows
-  const size_t wrow = (size_t)(n0 < a.N ? n0 + col : 0);
-  const int chunks = a.K / 64;
-  mf_f16v acc;
+  const int n0 = (blockIdx.x * 4 + wave) * 32;
+  const int m0 = blockIdx.y * RT * 32;
+  const bool live = n0 < a.N;                            // the last workgroup's waves may have no strip
+  const size_t wrow = (size_t)(live ? n0 + col : 0);
+  const int chunks = a.K / (64 * G);
+  const uint32_t* wp = a.W + wrow * (a.K / 8);
+  const uint32_t* sp = a.SB + wrow * (a.K / 64);
+  mf_f16v acc[RT];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-
-  // X chunks travel global -> registers -> LDS one iteration apart, so that no iteration waits for a load it
-  // has just issued: 32*WM rows x 128 bytes, one 16-byte piece per thread and pass; rows beyond M are zero
-  uint4 xr[WM];
+  for (int t = 0; t < RT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
+  // X chunks travel global -> registers -> LDS one iteration apart: 32*RT rows x 128*G bytes, one 16-byte piece per
+  // thread and pass; rows beyond M are zero
+  uint4 xr[RT * G];
   auto fetch = [&](int c) {
 #pragma unroll
-    for (int p = 0; p < WM; ++p) {
-      const int row = p * 32 + (tid >> 3);
-      xr[p] = make_uint4(0, 0, 0, 0);
-      if (row < a.M) xr[p] = ld16(a.x + (size_t)row * a.x_stride + c * 64 + (tid & 7) * 8);
-    }
+    for (int p = 0; p < RT; ++p)
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const int row = m0 + p * 32 + (tid >> 3);
+        xr[p * G + g] = make_uint4(0, 0, 0, 0);
+        if (row < a.M) xr[p * G + g] = ld16(a.x + (size_t)row * a.x_stride + (c * G + g) * 64 + (tid & 7) * 8);
+      }
   };
   auto put = [&](int buf) {
 #pragma unroll
-    for (int p = 0; p < WM; ++p) st16(&xs[buf][(p * 32 + (tid >> 3)) * QMM_XS + (tid & 7) * 8], permute8(xr[p]));
+    for (int p = 0; p < RT; ++p)
+#pragma unroll
+      for (int g = 0; g < G; ++g) st16(&xs[buf][(p * 32 + (tid >> 3)) * XS + g * 64 + (tid & 7) * 8], permute8(xr[p * G + g]));
+  };
+  uint4 nw[2 * G];
+  uint32_t nsb[G];
+  auto wfetch = [&](int c) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      nw[2 * g] = ld16(wp + (c * G + g) * 8);
+      nw[2 * g + 1] = ld16(wp + (c * G + g) * 8 + 4);
+      nsb[g] = sp[c * G + g];
+    }
   };
   fetch(0);
   put(0);
   if (chunks > 1) fetch(1);
-  // the weights of chunk c+1 are requested before chunk c is consumed
-  uint4 nw0 = make_uint4(0, 0, 0, 0), nw1 = make_uint4(0, 0, 0, 0);
-  uint32_t nsb = 0;
-  if (live) { nw0 = ld16(a.W + wrow * (a.K / 8)); nw1 = ld16(a.W + wrow * (a.K / 8) + 4); nsb = a.SB[wrow * (a.K / 64)]; }
+#pragma unroll
+  for (int g = 0; g < G; ++g) { nw[2 * g] = nw[2 * g + 1] = make_uint4(0, 0, 0, 0); nsb[g] = 0; }
+  if (live) wfetch(0);
   for (int c = 0; c < chunks; ++c) {
     const int buf = c & 1;
-    const uint4 w0 = nw0, w1 = nw1;
-    const uint32_t sb = nsb;
-    if (live && c + 1 < chunks) {
-      nw0 = ld16(a.W + wrow * (a.K / 8) + (c + 1) * 8);
-      nw1 = ld16(a.W + wrow * (a.K / 8) + (c + 1) * 8 + 4);
-      nsb = a.SB[wrow * (a.K / 64) + c + 1];
-    }
+    uint4 w[2 * G];
+    uint32_t sb[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) { w[2 * g] = nw[2 * g]; w[2 * g + 1] = nw[2 * g + 1]; sb[g] = nsb[g]; }
+    if (live && c + 1 < chunks) wfetch(c + 1);           // the weights of the next chunk are requested before this one is consumed
     __syncthreads();                                     // chunk c is staged; chunk c-1 is no longer read
     if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
     if (!live) continue;
-    const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb >> 16) * 0x10001u);
-    const uint32_t words[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
-    for (int st = 0; st < 8; ++st) {
-      // this lane's 4 weights of the step: nibbles {a, a+4, a+1, a+5} of word st with a = 2*hh
-      const mf_h4 bw = dequant4(words[st] >> (8 * hh), s2, b2);
-      const mf_h4 ax = *reinterpret_cast<const mf_h4*>(&xs[buf][(mt * 32 + col) * QMM_XS + 8 * st + 4 * hh]);
-      acc = __builtin_amdgcn_mfma_f32_32x32x8f16(ax, bw, acc, 0, 0, 0);
+    for (int g = 0; g < G; ++g) {
+      const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[g] >> 16) * 0x10001u);
+      const uint4 w0 = w[2 * g], w1 = w[2 * g + 1];
+      // this lane's word of each step: word 2*st + hh of the group
+      const uint32_t wsel[4] = {hh ? w0.y : w0.x, hh ? w0.w : w0.z, hh ? w1.y : w1.x, hh ? w1.w : w1.z};
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const mf_h8 bw = dequant8(wsel[st], s2, b2);
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+          const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][(t * 32 + col) * XS + g * 64 + 16 * st + 8 * hh]);
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax, bw, acc[t], 0, 0, 0);
+        }
+      }
     }
   }
   if (!live) return;
-  // D layout of the 32x32 tile: register r of lane (col, hh) holds row 8*(r/4) + 4*hh + r%4, column col
+  // D layout of a 32x32 tile: register r of lane (col, hh) holds row 8*(r/4) + 4*hh + r%4, column col
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int m = mt * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-    if (m < a.M) a.y[(size_t)m * a.y_stride + n0 + col] = f2h(acc[r]);
-  }
+  for (int t = 0; t < RT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = m0 + t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+      if (m < a.M) a.y[(size_t)m * a.y_stride + n0 + col] = f2h(acc[t][r]);
+    }
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -144,10 +173,12 @@ struct QmmGroupArgs {
   int y_stride;
 };
 
+constexpr int GQ_G = 4;                       // quantisation groups (64 k) per staged chunk: one barrier per 256 k
+constexpr int GQ_XS = 64 * GQ_G + 8;          // halves per staged row
 __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
   // One 32-row tile per pass and one accumulator per wave (most experts have fewer than 32 rows in a chunk; an
-  // expert with more takes several passes over its weights, which then come from cache).
-  __shared__ __align__(16) uint16_t xs[2][32 * QMM_XS];
+  // expert with more takes several passes over its weights, which then come from cache).  K % 256 == 0.
+  __shared__ __align__(16) uint16_t xs[2][32 * GQ_XS];
   const int e = blockIdx.y;
   const int cnt_all = min(a.counts[e], GROUP_CAP);
   if (cnt_all == 0) return;                              // uniform for the workgroup
@@ -156,47 +187,67 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
   const int n0 = (blockIdx.x * 4 + wave) * 32;
   const bool live = n0 < a.NE;
   const size_t wrow = (size_t)e * a.NE + (live ? n0 + col : 0);
-  const int chunks = a.K / 64;
+  const int chunks = a.K / (64 * GQ_G);
+  const uint32_t* wp = a.W + wrow * (a.K / 8);
+  const uint32_t* sp = a.SB + wrow * (a.K / 64);
   for (int r0 = 0; r0 < cnt_all; r0 += 32) {
     const int cnt = min(cnt_all - r0, 32);
     const uint16_t* list = a.lists + (size_t)e * GROUP_CAP + r0;
-    // the row this thread stages
+    // the row this thread stages: 32 rows x GQ_G x 8 pieces of 16 bytes, GQ_G pieces per thread
     int src = -1;
     if ((tid >> 3) < cnt) { const int pr = list[tid >> 3]; src = a.x_by_pair ? pr : (pr >> 3); }
     mf_f16v acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-    uint4 xr = make_uint4(0, 0, 0, 0);
+    uint4 xr[GQ_G];
     auto fetch = [&](int c) {
-      xr = make_uint4(0, 0, 0, 0);
-      if (src >= 0) xr = ld16(a.x + (size_t)src * a.x_stride + c * 64 + (tid & 7) * 8);
+#pragma unroll
+      for (int g = 0; g < GQ_G; ++g) {
+        xr[g] = make_uint4(0, 0, 0, 0);
+        if (src >= 0) xr[g] = ld16(a.x + (size_t)src * a.x_stride + (c * GQ_G + g) * 64 + (tid & 7) * 8);
+      }
     };
-    auto put = [&](int buf) { st16(&xs[buf][(tid >> 3) * QMM_XS + (tid & 7) * 8], permute8(xr)); };
+    auto put = [&](int buf) {
+#pragma unroll
+      for (int g = 0; g < GQ_G; ++g) st16(&xs[buf][(tid >> 3) * GQ_XS + g * 64 + (tid & 7) * 8], permute8(xr[g]));
+    };
+    uint4 nw[2 * GQ_G];
+    uint32_t nsb[GQ_G];
+    auto wfetch = [&](int c) {
+#pragma unroll
+      for (int g = 0; g < GQ_G; ++g) {
+        nw[2 * g] = ld16(wp + (c * GQ_G + g) * 8);
+        nw[2 * g + 1] = ld16(wp + (c * GQ_G + g) * 8 + 4);
+        nsb[g] = sp[c * GQ_G + g];
+      }
+    };
     __syncthreads();                                     // the pass before has finished reading the staging buffers
     fetch(0);
     put(0);
     if (chunks > 1) fetch(1);
-    uint4 nw0 = make_uint4(0, 0, 0, 0), nw1 = make_uint4(0, 0, 0, 0);
-    uint32_t nsb = 0;
-    if (live) { nw0 = ld16(a.W + wrow * (a.K / 8)); nw1 = ld16(a.W + wrow * (a.K / 8) + 4); nsb = a.SB[wrow * (a.K / 64)]; }
+#pragma unroll
+    for (int g = 0; g < GQ_G; ++g) { nw[2 * g] = nw[2 * g + 1] = make_uint4(0, 0, 0, 0); nsb[g] = 0; }
+    if (live) wfetch(0);
     for (int c = 0; c < chunks; ++c) {
       const int buf = c & 1;
-      const uint4 w0 = nw0, w1 = nw1;
-      const uint32_t sb = nsb;
-      if (live && c + 1 < chunks) {
-        nw0 = ld16(a.W + wrow * (a.K / 8) + (c + 1) * 8);
-        nw1 = ld16(a.W + wrow * (a.K / 8) + (c + 1) * 8 + 4);
-        nsb = a.SB[wrow * (a.K / 64) + c + 1];
-      }
+      uint4 w[2 * GQ_G];
+      uint32_t sb[GQ_G];
+#pragma unroll
+      for (int g = 0; g < GQ_G; ++g) { w[2 * g] = nw[2 * g]; w[2 * g + 1] = nw[2 * g + 1]; sb[g] = nsb[g]; }
+      if (live && c + 1 < chunks) wfetch(c + 1);
       __syncthreads();
       if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
-      const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb >> 16) * 0x10001u);
-      const uint32_t words[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
-      for (int st = 0; st < 8; ++st) {
-        const mf_h4 bw = dequant4(words[st] >> (8 * hh), s2, b2);
-        const mf_h4 ax = *reinterpret_cast<const mf_h4*>(&xs[buf][col * QMM_XS + 8 * st + 4 * hh]);
-        acc = __builtin_amdgcn_mfma_f32_32x32x8f16(ax, bw, acc, 0, 0, 0);
+      for (int g = 0; g < GQ_G; ++g) {
+        const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[g] >> 16) * 0x10001u);
+        const uint4 w0 = w[2 * g], w1 = w[2 * g + 1];
+        const uint32_t wsel[4] = {hh ? w0.y : w0.x, hh ? w0.w : w0.z, hh ? w1.y : w1.x, hh ? w1.w : w1.z};
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+          const mf_h8 bw = dequant8(wsel[st], s2, b2);
+          const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][col * GQ_XS + g * 64 + 16 * st + 8 * hh]);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax, bw, acc, 0, 0, 0);
+        }
       }
     }
     if (live) {
@@ -245,19 +296,22 @@ __global__ __launch_bounds__(256) void k_moe_combine_rows(const uint16_t* __rest
   out[(size_t)m * H + n] = f2h(f16r(acc + f16r(s * h2f(sy[(size_t)m * H + n]))));
 }
 
-// Host-side launch: picks the row-tile count per block of up to 128 rows.
-inline void launch_qmm4_mfma(const QmmArgs& all, hipStream_t stream) {
-  const int strips = all.N / 32;
+// Host-side launch: row tiles per wave chosen so that there are about as many wave tasks as SIMDs (1024): wide
+// projections share the unpacking over 128 rows, narrow ones spread their rows over more waves instead.
+template <int RT>
+inline void launch_qmm4_rt(const QmmArgs& a, dim3 grid, hipStream_t stream) {
   const dim3 block(256);
-  for (int r0 = 0; r0 < all.M; r0 += 128) {             // the kernel takes up to 128 rows: longer chunks go in blocks
-    QmmArgs a = all;
-    a.x = all.x + (size_t)r0 * all.x_stride;
-    a.y = all.y + (size_t)r0 * all.y_stride;
-    a.M = all.M - r0 < 128 ? all.M - r0 : 128;
-    if (a.M <= 32) hipLaunchKernelGGL(k_qmm4_mfma<1>, dim3((unsigned)((strips + 3) / 4)), block, 0, stream, a);
-    else if (a.M <= 64) hipLaunchKernelGGL(k_qmm4_mfma<2>, dim3((unsigned)((strips + 1) / 2)), block, 0, stream, a);
-    else hipLaunchKernelGGL(k_qmm4_mfma<4>, dim3((unsigned)strips), block, 0, stream, a);
-  }
+  constexpr int GMAX = RT == 1 ? 4 : 2;                  // staging buffers of at most ~70 KB
+  if (GMAX == 4 && a.K % 256 == 0) hipLaunchKernelGGL((k_qmm4_mfma16<RT, GMAX>), grid, block, 0, stream, a);
+  else if (a.K % 128 == 0) hipLaunchKernelGGL((k_qmm4_mfma16<RT, 2>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((k_qmm4_mfma16<RT, 1>), grid, block, 0, stream, a);
+}
+inline void launch_qmm4_mfma(const QmmArgs& a, hipStream_t stream) {
+  const int strips = a.N / 32, tiles = (a.M + 31) / 32;
+  const unsigned gx = (unsigned)((strips + 3) / 4);
+  if (tiles >= 4 && strips * (tiles / 4) >= 768) launch_qmm4_rt<4>(a, dim3(gx, (unsigned)((tiles + 3) / 4)), stream);
+  else if (tiles >= 2 && strips * (tiles / 2) >= 768) launch_qmm4_rt<2>(a, dim3(gx, (unsigned)((tiles + 1) / 2)), stream);
+  else launch_qmm4_rt<1>(a, dim3(gx, (unsigned)tiles), stream);
 }
 
 }  // namespace sl
