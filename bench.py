@@ -9,8 +9,12 @@ decode does (chainedStepArgmax, K = 8).
 Prints one JSON line: throughput, the roofline of the dominant kernel (the persistent step kernel
 k_decode_flow: one launch runs a chain of `--chain` tokens, each fed back on the device; launches are
 timed with HIP events on the engine's stream; roofline.avg_ms and bytes_per_launch are those of one
-launch = `--chain` tokens), and the CPU baseline (the oracle, timed on this host's cores on a bounded sample of the same
-workload).
+launch = `--chain` tokens), and the CPU baseline (the oracle, timed on this host's cores on a bounded
+sample of the same workload).  After the timed decode region the same engine also times the batched
+paths on the same weights and reports them as extra objects of the line: `lane_batch` (32 sequences
+stepped together), `verify` (4-row verify steps) and `prefill` (a 2048-token prompt in chunks of 512
+rows, exact rows and hybrid on the matrix cores); `--lanes 0 --verify-rows 0 --prefill-chunk 0`
+skips them.
 """
 import argparse
 import json
@@ -51,16 +55,16 @@ def main():
     ap.add_argument("--chain", type=int, default=8, help="tokens per on-device chain")
     ap.add_argument("--layers", type=int, default=40, help="for quick functional runs only")
     ap.add_argument("--cpu-tokens", type=int, default=4, help="decode tokens timed on the CPU oracle (0 = skip)")
-    ap.add_argument("--lanes", type=int, default=0, metavar="B",
-                    help="also time B lanes stepped as one batch of rows on the same weights (extra object in the JSON line)")
-    ap.add_argument("--prefill-chunk", type=int, default=0, metavar="M",
-                    help="also time the 512-token prefill in chunks of M rows, exact rows and hybrid (matrix cores), on lanes "
-                         "of the same weights (extra object in the JSON line)")
-    ap.add_argument("--prefill-tokens", type=int, default=PROMPT_LEN, metavar="N",
+    ap.add_argument("--lanes", type=int, default=32, metavar="B",
+                    help="also time B lanes stepped as one batch of rows on the same weights (extra object in the JSON line; 0 = skip)")
+    ap.add_argument("--prefill-chunk", type=int, default=512, metavar="M",
+                    help="also time a prefill in chunks of M rows, exact rows and hybrid (matrix cores), on lanes "
+                         "of the same weights (extra object in the JSON line; 0 = skip)")
+    ap.add_argument("--prefill-tokens", type=int, default=2048, metavar="N",
                     help="prompt length of the --prefill-chunk measurement (the reference's batched configuration uses 2048)")
-    ap.add_argument("--verify-rows", type=int, default=0, metavar="R",
+    ap.add_argument("--verify-rows", type=int, default=4, metavar="R",
                     help="also time verify steps of R rows ([token] + R-1 drafts through stepArgmax) at the decode context "
-                         "(extra object in the JSON line)")
+                         "(extra object in the JSON line; 0 = skip)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run a plain device copy of this many MiB (reference for rocprofv3 FETCH_SIZE/WRITE_SIZE) and exit")
     args = ap.parse_args()

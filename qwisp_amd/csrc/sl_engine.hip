@@ -240,6 +240,8 @@ void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   a.router_w = L.router_w; a.sgate_w = L.sgate_w; a.g8_w = L.gate8_w; a.g8_sb = L.gate8_sb; a.E = E; a.skip_shared = 1;
   a.sh_act = e->sh_act; a.rlogits = e->rlogits; a.sgate = e->sgate;
   const int router_blocks = (E + 1 + 15) / 16;
+  hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, ha);     // residual + norm once per row
+  a.xn_in = ha.xn_out;
   hipLaunchKernelGGL(k_moe_a, dim3(router_blocks, M), dim3(256), 0, e->stream, a);
   hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, E, L.route_inds, L.route_scores);
   hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, E, e->hy_lists, e->hy_counts);
@@ -266,6 +268,10 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   a.router_w = L.router_w; a.sgate_w = L.sgate_w; a.g8_w = L.gate8_w; a.g8_sb = L.gate8_sb; a.E = e->n_experts;
   a.sh_act = e->sh_act; a.rlogits = e->rlogits; a.sgate = e->sgate;
   const int router_blocks = (e->n_experts + 1 + 15) / 16;
+  if (M >= 2) {                                         // residual + norm once per row instead of once per wave
+    hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, ha);
+    a.xn_in = ha.xn_out;
+  }
   hipLaunchKernelGGL(k_moe_a, dim3(MOE_A_SHARED_BLOCKS + router_blocks, M), dim3(256), 0, e->stream, a);
   hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, e->n_experts, L.route_inds, L.route_scores);
   MoeBArgs b{};

@@ -670,6 +670,7 @@ struct MoeAArgs {
   const uint32_t *g8_w, *g8_sb;                      // 8-bit gates instead (null: fp16): [E+1, 512] words, [E+1, 32] {scale, bias}; row E = shared gate
   int E;
   int skip_shared;                                   // hybrid prefill: the shared expert's gate/up run on the matrix cores; grid.x = router blocks only
+  const uint16_t* xn_in;                             // rows already normed by k_final_rows (M >= 2), or null: hidden prologue here
   uint16_t* sh_act;                                  // [M, 512]
   uint16_t* rlogits;                                 // [M, 256]
   uint16_t* sgate;                                   // [M]
@@ -678,7 +679,8 @@ constexpr int MOE_A_SHARED_BLOCKS = 64;
 __global__ __launch_bounds__(256) void k_moe_a(MoeAArgs a) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float x[32], sx[4];
-  hidden_prologue(a.ha, m, lane, blockIdx.x == 0 && wave == 0, x);
+  if (a.xn_in) load32(a.xn_in + (size_t)m * H + 32 * lane, x);
+  else hidden_prologue(a.ha, m, lane, blockIdx.x == 0 && wave == 0, x);
   // skip_shared: the grid holds the router blocks only
   const int bx = a.skip_shared ? (int)blockIdx.x + MOE_A_SHARED_BLOCKS : (int)blockIdx.x;
   if (bx < MOE_A_SHARED_BLOCKS) {
