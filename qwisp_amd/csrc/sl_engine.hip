@@ -245,15 +245,11 @@ void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   hipLaunchKernelGGL(k_moe_a, dim3(router_blocks, M), dim3(256), 0, e->stream, a);
   hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, E, L.route_inds, L.route_scores);
   hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, E, e->hy_lists, e->hy_counts);
-  // routed gate / up by expert, SwiGLU, routed down by expert
-  QmmGroupArgs g{e->xn, H, 0, L.sw_gate.w, L.sw_gate.sb, SL_MOE_I, H, e->hy_lists, e->hy_counts, e->hy_g, SL_MOE_I};
-  hipLaunchKernelGGL(k_qmm4_mfma_grouped, dim3(SL_MOE_I / 128, E), dim3(256), 0, e->stream, g);
-  g.W = L.sw_up.w; g.SB = L.sw_up.sb; g.y = e->hy_u;
-  hipLaunchKernelGGL(k_qmm4_mfma_grouped, dim3(SL_MOE_I / 128, E), dim3(256), 0, e->stream, g);
-  const int tot = M * 8 * SL_MOE_I;
-  hipLaunchKernelGGL(k_swiglu_rows, dim3((tot + 255) / 256), dim3(256), 0, e->stream, e->hy_g, e->hy_u, e->act, tot);
-  QmmGroupArgs d{e->act, SL_MOE_I, 1, L.sw_down.w, L.sw_down.sb, H, SL_MOE_I, e->hy_lists, e->hy_counts, e->hy_d, H};
-  hipLaunchKernelGGL(k_qmm4_mfma_grouped, dim3(H / 128, E), dim3(256), 0, e->stream, d);
+  // routed gate and up by expert in one pass with SwiGLU, then routed down by expert
+  QmmGroupArgs g{e->xn, H, 0, L.sw_gate.w, L.sw_gate.sb, L.sw_up.w, L.sw_up.sb, SL_MOE_I, H, e->hy_lists, e->hy_counts, e->act, SL_MOE_I};
+  hipLaunchKernelGGL(k_qmm4_mfma_grouped<true>, dim3(SL_MOE_I / 128, E), dim3(256), 0, e->stream, g);
+  QmmGroupArgs d{e->act, SL_MOE_I, 1, L.sw_down.w, L.sw_down.sb, nullptr, nullptr, H, SL_MOE_I, e->hy_lists, e->hy_counts, e->hy_d, H};
+  hipLaunchKernelGGL(k_qmm4_mfma_grouped<false>, dim3(H / 128, E), dim3(256), 0, e->stream, d);
   // shared expert
   launch_qmm4_mfma(QmmArgs{e->xn, H, L.sh_gate.w, L.sh_gate.sb, M, SL_MOE_I, H, e->hy_sg, SL_MOE_I}, e->stream);
   launch_qmm4_mfma(QmmArgs{e->xn, H, L.sh_up.w, L.sh_up.sb, M, SL_MOE_I, H, e->hy_su, SL_MOE_I}, e->stream);

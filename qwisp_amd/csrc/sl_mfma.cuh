@@ -166,6 +166,7 @@ struct QmmGroupArgs {
   int x_by_pair;         // 0: source row = token row (pair >> 3); 1: source row = pair index (m * 8 + slot)
   const uint32_t* W;     // [E * NE, K/8]: expert e owns rows e*NE .. e*NE + NE - 1
   const uint32_t* SB;    // [E * NE, K/64]
+  const uint32_t *W2, *SB2;  // second matrix of the dual form (else unused)
   int NE, K;
   const uint16_t* lists; // [E, GROUP_CAP] pair indices
   const int32_t* counts; // [E]
@@ -175,9 +176,14 @@ struct QmmGroupArgs {
 
 constexpr int GQ_G = 4;                       // quantisation groups (64 k) per staged chunk: one barrier per 256 k
 constexpr int GQ_XS = 64 * GQ_G + 8;          // halves per staged row
+// DUAL: two weight matrices of the same shape against the same rows (the experts' gate_proj and up_proj): one
+// staging of X, two weight streams in flight per wave, and y = half(silu(g) * u) of the two rounded results
+// written directly (the SwiGLU of the GEMV path, swiglu16).
+template <bool DUAL>
 __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
-  // One 32-row tile per pass and one accumulator per wave (most experts have fewer than 32 rows in a chunk; an
-  // expert with more takes several passes over its weights, which then come from cache).  K % 256 == 0.
+  // One 32-row tile per pass and one accumulator per wave and matrix (most experts have fewer than 32 rows in a
+  // chunk; an expert with more takes several passes over its weights, which then come from cache).  K % 256 == 0.
+  constexpr int NW = DUAL ? 2 : 1;
   __shared__ __align__(16) uint16_t xs[2][32 * GQ_XS];
   const int e = blockIdx.y;
   const int cnt_all = min(a.counts[e], GROUP_CAP);
@@ -188,17 +194,19 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
   const bool live = n0 < a.NE;
   const size_t wrow = (size_t)e * a.NE + (live ? n0 + col : 0);
   const int chunks = a.K / (64 * GQ_G);
-  const uint32_t* wp = a.W + wrow * (a.K / 8);
-  const uint32_t* sp = a.SB + wrow * (a.K / 64);
+  const uint32_t* wp[2] = {a.W + wrow * (a.K / 8), DUAL ? a.W2 + wrow * (a.K / 8) : nullptr};
+  const uint32_t* sp[2] = {a.SB + wrow * (a.K / 64), DUAL ? a.SB2 + wrow * (a.K / 64) : nullptr};
   for (int r0 = 0; r0 < cnt_all; r0 += 32) {
     const int cnt = min(cnt_all - r0, 32);
     const uint16_t* list = a.lists + (size_t)e * GROUP_CAP + r0;
     // the row this thread stages: 32 rows x GQ_G x 8 pieces of 16 bytes, GQ_G pieces per thread
     int src = -1;
     if ((tid >> 3) < cnt) { const int pr = list[tid >> 3]; src = a.x_by_pair ? pr : (pr >> 3); }
-    mf_f16v acc;
+    mf_f16v acc[NW];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    for (int q = 0; q < NW; ++q)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[q][r] = 0.0f;
     uint4 xr[GQ_G];
     auto fetch = [&](int c) {
 #pragma unroll
@@ -211,42 +219,50 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
 #pragma unroll
       for (int g = 0; g < GQ_G; ++g) st16(&xs[buf][(tid >> 3) * GQ_XS + g * 64 + (tid & 7) * 8], permute8(xr[g]));
     };
-    uint4 nw[2 * GQ_G];
-    uint32_t nsb[GQ_G];
+    uint4 nw[NW][2 * GQ_G];
+    uint32_t nsb[NW][GQ_G];
     auto wfetch = [&](int c) {
 #pragma unroll
-      for (int g = 0; g < GQ_G; ++g) {
-        nw[2 * g] = ld16(wp + (c * GQ_G + g) * 8);
-        nw[2 * g + 1] = ld16(wp + (c * GQ_G + g) * 8 + 4);
-        nsb[g] = sp[c * GQ_G + g];
-      }
+      for (int q = 0; q < NW; ++q)
+#pragma unroll
+        for (int g = 0; g < GQ_G; ++g) {
+          nw[q][2 * g] = ld16(wp[q] + (c * GQ_G + g) * 8);
+          nw[q][2 * g + 1] = ld16(wp[q] + (c * GQ_G + g) * 8 + 4);
+          nsb[q][g] = sp[q][c * GQ_G + g];
+        }
     };
     __syncthreads();                                     // the pass before has finished reading the staging buffers
     fetch(0);
     put(0);
     if (chunks > 1) fetch(1);
 #pragma unroll
-    for (int g = 0; g < GQ_G; ++g) { nw[2 * g] = nw[2 * g + 1] = make_uint4(0, 0, 0, 0); nsb[g] = 0; }
+    for (int q = 0; q < NW; ++q)
+#pragma unroll
+      for (int g = 0; g < GQ_G; ++g) { nw[q][2 * g] = nw[q][2 * g + 1] = make_uint4(0, 0, 0, 0); nsb[q][g] = 0; }
     if (live) wfetch(0);
     for (int c = 0; c < chunks; ++c) {
       const int buf = c & 1;
-      uint4 w[2 * GQ_G];
-      uint32_t sb[GQ_G];
+      uint4 w[NW][2 * GQ_G];
+      uint32_t sb[NW][GQ_G];
 #pragma unroll
-      for (int g = 0; g < GQ_G; ++g) { w[2 * g] = nw[2 * g]; w[2 * g + 1] = nw[2 * g + 1]; sb[g] = nsb[g]; }
+      for (int q = 0; q < NW; ++q)
+#pragma unroll
+        for (int g = 0; g < GQ_G; ++g) { w[q][2 * g] = nw[q][2 * g]; w[q][2 * g + 1] = nw[q][2 * g + 1]; sb[q][g] = nsb[q][g]; }
       if (live && c + 1 < chunks) wfetch(c + 1);
       __syncthreads();
       if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
 #pragma unroll
       for (int g = 0; g < GQ_G; ++g) {
-        const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[g] >> 16) * 0x10001u);
-        const uint4 w0 = w[2 * g], w1 = w[2 * g + 1];
-        const uint32_t wsel[4] = {hh ? w0.y : w0.x, hh ? w0.w : w0.z, hh ? w1.y : w1.x, hh ? w1.w : w1.z};
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
-          const mf_h8 bw = dequant8(wsel[st], s2, b2);
           const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][col * GQ_XS + g * 64 + 16 * st + 8 * hh]);
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax, bw, acc, 0, 0, 0);
+#pragma unroll
+          for (int q = 0; q < NW; ++q) {
+            const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[q][g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[q][g] >> 16) * 0x10001u);
+            const uint4 w0 = w[q][2 * g], w1 = w[q][2 * g + 1];
+            const uint32_t wsel = st == 0 ? (hh ? w0.y : w0.x) : st == 1 ? (hh ? w0.w : w0.z) : st == 2 ? (hh ? w1.y : w1.x) : (hh ? w1.w : w1.z);
+            acc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax, dequant8(wsel, s2, b2), acc[q], 0, 0, 0);
+          }
         }
       }
     }
@@ -254,7 +270,11 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = 8 * (r >> 2) + 4 * hh + (r & 3);
-        if (row < cnt) a.y[(size_t)list[row] * a.y_stride + n0 + col] = f2h(acc[r]);
+        if (row < cnt) {
+          float v = f16r(acc[0][r]);
+          if constexpr (DUAL) v = swiglu16(v, f16r(acc[1][r]));
+          a.y[(size_t)list[row] * a.y_stride + n0 + col] = f2h(v);
+        }
       }
     }
   }
