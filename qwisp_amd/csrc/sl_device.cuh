@@ -107,6 +107,20 @@ SL_DEV void lanes8(float v, int base, float (&out)[8]) {
   for (int i = 0; i < 8; ++i) out[i] = __builtin_bit_cast(float, t[i]);
 }
 
+#ifndef SL_SWAP_REDUCE
+#define SL_SWAP_REDUCE 1
+#endif
+// {row0, row1, row2, row3} -> {row0+row1, row0+row1, row2+row3, row2+row3} (rows of 16 lanes), and lower + upper half.
+SL_DEV float swap16_sum(float v) {
+  const unsigned u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+SL_DEV float swap32_sum(float v) {
+  const unsigned u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 template <int WIDTH>
 SL_DEV float tree_sum(float v) {
   static_assert(WIDTH == 4 || WIDTH == 8 || WIDTH == 16 || WIDTH == 32 || WIDTH == 64, "group sizes used by the kernels");
@@ -117,10 +131,18 @@ SL_DEV float tree_sum(float v) {
   if constexpr (WIDTH == 8) return v;
   v = v + dpp_f<DPP_MIRROR>(v);
   if constexpr (WIDTH == 16) return v;
+#if SL_SWAP_REDUCE
+  // rows 0|1 and 2|3, then halves: v_permlane16_swap / v_permlane32_swap of a value with its own copy hand every
+  // lane its partner group's value (no trip through scalar registers); a + b == b + a bit for bit
+  v = swap16_sum(v);
+  if constexpr (WIDTH == 32) return v;
+  return swap32_sum(v);
+#else
   const float r0 = row_lane_f(v, 0), r1 = row_lane_f(v, 16), r2 = row_lane_f(v, 32), r3 = row_lane_f(v, 48);
   const float lo = r0 + r1, hi = r2 + r3;
   if constexpr (WIDTH == 32) return (__lane_id() < 32) ? lo : hi;
   return lo + hi;
+#endif
 }
 template <int WIDTH>
 SL_DEV float tree_max(float v) {
@@ -129,8 +151,19 @@ SL_DEV float tree_max(float v) {
   v = fmaxf(v, dpp_f<DPP_XOR2>(v));
   v = fmaxf(v, dpp_f<DPP_HALF_MIRROR>(v));
   v = fmaxf(v, dpp_f<DPP_MIRROR>(v));
+#if SL_SWAP_REDUCE
+  {
+    const unsigned u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    const unsigned w = __float_as_uint(v);
+    const auto q = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
+  }
+#else
   const float r0 = row_lane_f(v, 0), r1 = row_lane_f(v, 16), r2 = row_lane_f(v, 32), r3 = row_lane_f(v, 48);
   return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+#endif
 }
 // Value of the previous lane (lanes 0, 16, 32, 48 get 0): for left-to-right chains inside a 16-lane row.
 SL_DEV float prev_lane(float v) { return dpp_f<DPP_SHR1>(v); }
