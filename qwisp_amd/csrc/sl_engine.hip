@@ -318,7 +318,7 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
     // rows of one sequence: the state-independent part for all rows at once, then the scan without barriers
     GdnPrepArgs pa{g, e->gdn_qn, e->gdn_kn, e->gdn_vc, e->gdn_gb};
     hipLaunchKernelGGL(k_gdn_prep_rows, dim3(65, M), dim3(64), 0, e->stream, pa);
-    hipLaunchKernelGGL(k_gdn_scan_rows, dim3(256), dim3(256), 0, e->stream, pa);
+    hipLaunchKernelGGL(k_gdn_scan_rows, dim3(512), dim3(256), 0, e->stream, pa);
   } else {
     hipLaunchKernelGGL(k_gdn_core, dim3(256, lanes ? M : 1), dim3(256), 0, e->stream, g);
   }

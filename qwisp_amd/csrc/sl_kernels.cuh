@@ -517,68 +517,69 @@ __global__ __launch_bounds__(64) void k_gdn_prep_rows(GdnPrepArgs p) {
     }
   }
 }
-// The recurrence over the rows: workgroup = (value head, block of 16 dv), thread layout and arithmetic of
-// k_gdn_core.  Also shifts the conv history.
+// The recurrence over the rows: workgroup = (value head, block of 8 dv), arithmetic of k_gdn_core.  Also shifts the conv history.
 __global__ __launch_bounds__(256) void k_gdn_scan_rows(GdnPrepArgs p) {
   const GdnArgs& a = p.g;
-  const int hv = blockIdx.x >> 3, dvb = blockIdx.x & 7, hk = hv >> 1;
+  const int hv = blockIdx.x >> 4, dvb = blockIdx.x & 15, hk = hv >> 1;   // 16 slices of 8 state rows per value head
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
   const bool par = a.st[1] != 0;
   const uint16_t* hin = par ? a.hist[1] : a.hist[0];
   uint16_t* hout = par ? a.hist[0] : a.hist[1];
   const float* sin_ = par ? a.state[1] : a.state[0];
   float* sout = par ? a.state[0] : a.state[1];
-  float s[2][4];
-#pragma unroll
-  for (int it = 0; it < 2; ++it) {
-    const int dv = dvb * 16 + wave * 4 + it * 2 + half;
+  // a wave owns two state rows (one per half-wave): twice the waves of k_gdn_core, because here a wave's step is a
+  // chain of dependent instructions and a SIMD with one wave idles between them
+  const int dv = dvb * 8 + wave * 2 + half;
+  float s[4];
+  {
     const float4 v = *reinterpret_cast<const float4*>(sin_ + ((size_t)hv * 128 + dv) * 128 + 4 * l32);
-    s[it][0] = v.x; s[it][1] = v.y; s[it][2] = v.z; s[it][3] = v.w;
+    s[0] = v.x; s[1] = v.y; s[2] = v.z; s[3] = v.w;
   }
-  struct Row { uint2 k, q; uint16_t v[2]; float g, beta; };
+  struct Row { uint2 k, q; uint16_t v; float g, beta; };
   auto fetch = [&](int t) {
     Row r;
     r.k = *reinterpret_cast<const uint2*>(p.kn + (size_t)t * 2048 + hk * 128 + 4 * l32);
     r.q = *reinterpret_cast<const uint2*>(p.qn + (size_t)t * 2048 + hk * 128 + 4 * l32);
-#pragma unroll
-    for (int it = 0; it < 2; ++it) r.v[it] = p.vc[(size_t)t * 4096 + hv * 128 + dvb * 16 + wave * 4 + it * 2 + half];
+    r.v = p.vc[(size_t)t * 4096 + hv * 128 + dv];
     r.g = p.gb[(size_t)t * 64 + hv]; r.beta = p.gb[(size_t)t * 64 + 32 + hv];
     return r;
   };
-  Row nxt = fetch(0);
-  for (int t = 0; t < a.M; ++t) {
-    const Row cur = nxt;
-    if (t + 1 < a.M) nxt = fetch(t + 1);
-    const float kk[4] = {lo_h(cur.k.x), hi_h(cur.k.x), lo_h(cur.k.y), hi_h(cur.k.y)};
-    const float qq[4] = {lo_h(cur.q.x), hi_h(cur.q.x), lo_h(cur.q.y), hi_h(cur.q.y)};
+  // the inputs of the next SCAN_AHEAD rows are in flight while a row is worked on (a row's step is far shorter than
+  // a trip to memory); the ring is indexed with constants only, so it stays in registers
+  constexpr int SCAN_AHEAD = 8;
+  Row ring[SCAN_AHEAD];
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int dvl = wave * 4 + it * 2 + half;
+  for (int j = 0; j < SCAN_AHEAD; ++j) if (j < a.M) ring[j] = fetch(j);
+  for (int t0 = 0; t0 < a.M; t0 += SCAN_AHEAD) {
+#pragma unroll
+    for (int j = 0; j < SCAN_AHEAD; ++j) {
+      const int t = t0 + j;
+      if (t >= a.M) break;
+      const Row cur = ring[j];
+      if (t + SCAN_AHEAD < a.M) ring[j] = fetch(t + SCAN_AHEAD);
+      const float kk[4] = {lo_h(cur.k.x), hi_h(cur.k.x), lo_h(cur.k.y), hi_h(cur.k.y)};
+      const float qq[4] = {lo_h(cur.q.x), hi_h(cur.q.x), lo_h(cur.q.y), hi_h(cur.q.y)};
       float acc = 0.0f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { s[it][i] = s[it][i] * cur.g; acc = fmaf(s[it][i], kk[i], acc); }
+      for (int i = 0; i < 4; ++i) { s[i] = s[i] * cur.g; acc = fmaf(s[i], kk[i], acc); }
       const float kv = tree_sum<32>(acc);
-      const float delta = (h2f(cur.v[it]) - kv) * cur.beta;
+      const float delta = (h2f(cur.v) - kv) * cur.beta;
       acc = 0.0f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { s[it][i] = fmaf(kk[i], delta, s[it][i]); acc = fmaf(s[it][i], qq[i], acc); }
+      for (int i = 0; i < 4; ++i) { s[i] = fmaf(kk[i], delta, s[i]); acc = fmaf(s[i], qq[i], acc); }
       const float y = tree_sum<32>(acc);
-      if (l32 == 0) a.ycore[(size_t)t * 4096 + hv * 128 + dvb * 16 + dvl] = f2h(y);
+      if (l32 == 0) a.ycore[(size_t)t * 4096 + hv * 128 + dv] = f2h(y);
     }
   }
-#pragma unroll
-  for (int it = 0; it < 2; ++it) {
-    const int dv = dvb * 16 + wave * 4 + it * 2 + half;
-    *reinterpret_cast<float4*>(sout + ((size_t)hv * 128 + dv) * 128 + 4 * l32) = make_float4(s[it][0], s[it][1], s[it][2], s[it][3]);
-  }
+  *reinterpret_cast<float4*>(sout + ((size_t)hv * 128 + dv) * 128 + 4 * l32) = make_float4(s[0], s[1], s[2], s[3]);
   // history shift: rows M..M+2 of [hist | qkv]; each channel written by exactly one workgroup
   const int qk_ch = (tid < 128) ? (hk * 128 + tid) : (2048 + hk * 128 + (tid - 128));
-  const int v_ch = 4096 + hv * 128 + dvb * 16 + (tid & 15);
+  const int v_ch = 4096 + hv * 128 + dvb * 8 + (tid & 7);
   if ((hv & 1) == 0 && dvb == 0) {
 #pragma unroll
     for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + qk_ch] = f2h(conv_tap(a.proj, hin, a.M + j, qk_ch));
   }
-  if (tid < 16) {
+  if (tid < 8) {
 #pragma unroll
     for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + v_ch] = f2h(conv_tap(a.proj, hin, a.M + j, v_ch));
   }
