@@ -70,6 +70,64 @@ def test_generator_device_equals_host(env):
 
 
 # ---- matrix-core GEMM of the hybrid prefill ---------------------------------------------------------
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m", [2, 5, 8, 9, 13, 17, 32])
+def test_row_tiles_of_any_count_equal_single_steps(env, small_model, m):
+    """The row kernels take activation rows in tiles of 8 (in-projection, lm_head) and 4 (out-projection): full
+    tiles, ragged last tiles and several tiles give, row by row, the bits of single steps (SeedlessVerifyTests.swift:613)."""
+    cfg, dev, host = small_model
+    a = env["Engine"](cfg, dev, max_m=32, max_seq_len=96)
+    b = env["Engine"](cfg, dev, max_m=32, max_seq_len=96)
+    rng = np.random.default_rng(500 + m)
+    pre = rng.integers(0, cfg.vocab, 7).tolist()
+    assert a.step_argmax(pre).tolist() == b.step_argmax(pre).tolist()
+    toks = rng.integers(0, cfg.vocab, m).tolist()
+    ta = a.step_argmax(toks)
+    assert ta is not None, a.gpu_fault
+    tb = []
+    for r, t in enumerate(toks):
+        tb.append(int(b.step_argmax([t])[0]))
+        assert same_bits(a.logits_row(r), b.logits_row(0)), r
+    assert ta.tolist() == tb
+    assert a.position == b.position == 7 + m
+    for li in range(cfg.n_layers):
+        for x, y in zip(a.read_layer_cache(li), b.read_layer_cache(li)):
+            assert same_bits(x, y), li
+    assert a.chained_step_argmax(int(ta[-1]), 3).tolist() == b.chained_step_argmax(tb[-1], 3).tolist()
+
+
+@pytest.mark.gpu
+def test_eleven_lanes_in_one_batch_equal_solo(env, small_model):
+    """A lane batch that is not a multiple of the row tiles (11 rows: tiles of 8 + 3 and 4 + 4 + 3), lanes at
+    different positions (SeedlessLaneBatch.swift:876)."""
+    cfg, dev, host = small_model
+    B = 11
+    base = env["Engine"](cfg, dev, max_m=B, max_seq_len=96)
+    lanes = [base.new_lane(max_m=B, max_seq_len=96) for _ in range(B)]
+    solos = [env["Engine"](cfg, dev, max_m=B, max_seq_len=96) for _ in range(B)]
+    rng = np.random.default_rng(78)
+    cur = []
+    for i, (lane, solo) in enumerate(zip(lanes, solos)):
+        pr = rng.integers(0, cfg.vocab, 1 + (7 * i) % 10).tolist()
+        ta, tb = lane.step_argmax(pr), solo.step_argmax(pr)
+        assert ta.tolist() == tb.tolist()
+        cur.append(int(ta[-1]))
+    for step in range(4):
+        got = type(base).lane_step_argmax(lanes, cur)
+        assert got is not None, [l.gpu_fault for l in lanes]
+        want = [int(solo.step_argmax([t])[0]) for solo, t in zip(solos, cur)]
+        assert got.tolist() == want, step
+        cur = want
+    for lane, solo in zip(lanes, solos):
+        assert same_bits(lane.logits_row(0), solo.logits_row(0))
+        for li in range(cfg.n_layers):
+            for x, y in zip(lane.read_layer_cache(li), solo.read_layer_cache(li)):
+                assert same_bits(x, y), li
+    for lane in lanes:
+        lane.close()
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("m,n,k", [(1, 32, 64), (5, 96, 512), (32, 128, 2048), (33, 160, 2048), (64, 2048, 4096), (100, 64, 512), (300, 96, 512)])
 def test_mfma_qmm4_against_the_oracle_rows(env, m, n, k):
