@@ -44,8 +44,9 @@ struct QmmArgs {
 // weight rows and RT x 32 rows of X (RT accumulators): it dequantises the 8 weights of a step once and feeds them
 // to RT matrix instructions, so the unpacking is shared by up to 128 rows of X; the four waves of a workgroup take
 // four neighbouring strips and read the same staged X chunk.  Grid (ceil(N / 128), ceil(M / (32*RT))).
-// Operands of a step (16 values of k): lane (col, hh) brings k = 8*hh .. 8*hh+7 of its row (A) / weight row (B),
-// i.e. one packed word of the weight row; the order within the eight is {0,4,1,5,2,6,3,7} on both sides.
+// Operands of a step (16 values of k): lane (col, hh) brings the 8 values of one packed word of its row (A) / weight
+// row (B) -- word st of the 64-k group on the lower half-wave, word 4+st on the upper, so that a lane fetches its four
+// words of a group with one 16-byte load; the order within the eight is {0,4,1,5,2,6,3,7} on both sides.
 // -------------------------------------------------------------------------------------------------
 // Dequantisation of a packed word (8 weights) in packed half arithmetic: masking with 0x000F000F leaves the nibbles
 // j and j+4; or-ing a nibble into the mantissa of 1024.0 gives 1024 + q exactly, subtracting 1024 gives q exactly,
@@ -99,13 +100,14 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
 #pragma unroll
       for (int g = 0; g < G; ++g) st16(&xs[buf][(p * 32 + (tid >> 3)) * XS + g * 64 + (tid & 7) * 8], permute8(xr[p * G + g]));
   };
-  uint4 nw[2 * G];
+  // of a group's 8 packed words the lower half-wave takes words 0..3 and the upper 4..7 (one 16-byte load each):
+  // step st multiplies the k of word st (lower) and of word 4+st (upper), on the A side as well
+  uint4 nw[G];
   uint32_t nsb[G];
   auto wfetch = [&](int c) {
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      nw[2 * g] = ld16(wp + (c * G + g) * 8);
-      nw[2 * g + 1] = ld16(wp + (c * G + g) * 8 + 4);
+      nw[g] = ld16(wp + (c * G + g) * 8 + 4 * hh);
       nsb[g] = sp[c * G + g];
     }
   };
@@ -113,14 +115,14 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
   put(0);
   if (chunks > 1) fetch(1);
 #pragma unroll
-  for (int g = 0; g < G; ++g) { nw[2 * g] = nw[2 * g + 1] = make_uint4(0, 0, 0, 0); nsb[g] = 0; }
+  for (int g = 0; g < G; ++g) { nw[g] = make_uint4(0, 0, 0, 0); nsb[g] = 0; }
   if (live) wfetch(0);
   for (int c = 0; c < chunks; ++c) {
     const int buf = c & 1;
-    uint4 w[2 * G];
+    uint4 w[G];
     uint32_t sb[G];
 #pragma unroll
-    for (int g = 0; g < G; ++g) { w[2 * g] = nw[2 * g]; w[2 * g + 1] = nw[2 * g + 1]; sb[g] = nsb[g]; }
+    for (int g = 0; g < G; ++g) { w[g] = nw[g]; sb[g] = nsb[g]; }
     if (live && c + 1 < chunks) wfetch(c + 1);           // the weights of the next chunk are requested before this one is consumed
     __syncthreads();                                     // chunk c is staged; chunk c-1 is no longer read
     if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
@@ -128,15 +130,13 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[g] >> 16) * 0x10001u);
-      const uint4 w0 = w[2 * g], w1 = w[2 * g + 1];
-      // this lane's word of each step: word 2*st + hh of the group
-      const uint32_t wsel[4] = {hh ? w0.y : w0.x, hh ? w0.w : w0.z, hh ? w1.y : w1.x, hh ? w1.w : w1.z};
+      const uint32_t wsel[4] = {w[g].x, w[g].y, w[g].z, w[g].w};
 #pragma unroll
       for (int st = 0; st < 4; ++st) {
         const mf_h8 bw = dequant8(wsel[st], s2, b2);
 #pragma unroll
         for (int t = 0; t < RT; ++t) {
-          const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][(t * 32 + col) * XS + g * 64 + 16 * st + 8 * hh]);
+          const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][(t * 32 + col) * XS + g * 64 + 32 * hh + 8 * st]);
           acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax, bw, acc[t], 0, 0, 0);
         }
       }
@@ -219,15 +219,14 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
 #pragma unroll
       for (int g = 0; g < GQ_G; ++g) st16(&xs[buf][(tid >> 3) * GQ_XS + g * 64 + (tid & 7) * 8], permute8(xr[g]));
     };
-    uint4 nw[NW][2 * GQ_G];
+    uint4 nw[NW][GQ_G];                                  // words 4*hh .. 4*hh+3 of each group (see k_qmm4_mfma16)
     uint32_t nsb[NW][GQ_G];
     auto wfetch = [&](int c) {
 #pragma unroll
       for (int q = 0; q < NW; ++q)
 #pragma unroll
         for (int g = 0; g < GQ_G; ++g) {
-          nw[q][2 * g] = ld16(wp[q] + (c * GQ_G + g) * 8);
-          nw[q][2 * g + 1] = ld16(wp[q] + (c * GQ_G + g) * 8 + 4);
+          nw[q][g] = ld16(wp[q] + (c * GQ_G + g) * 8 + 4 * hh);
           nsb[q][g] = sp[q][c * GQ_G + g];
         }
     };
@@ -238,16 +237,16 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
 #pragma unroll
     for (int q = 0; q < NW; ++q)
 #pragma unroll
-      for (int g = 0; g < GQ_G; ++g) { nw[q][2 * g] = nw[q][2 * g + 1] = make_uint4(0, 0, 0, 0); nsb[q][g] = 0; }
+      for (int g = 0; g < GQ_G; ++g) { nw[q][g] = make_uint4(0, 0, 0, 0); nsb[q][g] = 0; }
     if (live) wfetch(0);
     for (int c = 0; c < chunks; ++c) {
       const int buf = c & 1;
-      uint4 w[NW][2 * GQ_G];
+      uint4 w[NW][GQ_G];
       uint32_t sb[NW][GQ_G];
 #pragma unroll
       for (int q = 0; q < NW; ++q)
 #pragma unroll
-        for (int g = 0; g < GQ_G; ++g) { w[q][2 * g] = nw[q][2 * g]; w[q][2 * g + 1] = nw[q][2 * g + 1]; sb[q][g] = nsb[q][g]; }
+        for (int g = 0; g < GQ_G; ++g) { w[q][g] = nw[q][g]; sb[q][g] = nsb[q][g]; }
       if (live && c + 1 < chunks) wfetch(c + 1);
       __syncthreads();
       if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
@@ -255,12 +254,12 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
       for (int g = 0; g < GQ_G; ++g) {
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
-          const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][col * GQ_XS + g * 64 + 16 * st + 8 * hh]);
+          const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][col * GQ_XS + g * 64 + 32 * hh + 8 * st]);
 #pragma unroll
           for (int q = 0; q < NW; ++q) {
             const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[q][g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[q][g] >> 16) * 0x10001u);
-            const uint4 w0 = w[q][2 * g], w1 = w[q][2 * g + 1];
-            const uint32_t wsel = st == 0 ? (hh ? w0.y : w0.x) : st == 1 ? (hh ? w0.w : w0.z) : st == 2 ? (hh ? w1.y : w1.x) : (hh ? w1.w : w1.z);
+            const uint4 w0 = w[q][g];
+            const uint32_t wsel = st == 0 ? w0.x : st == 1 ? w0.y : st == 2 ? w0.z : w0.w;
             acc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax, dequant8(wsel, s2, b2), acc[q], 0, 0, 0);
           }
         }
