@@ -251,8 +251,7 @@ void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   QmmGroupArgs d{e->act, SL_MOE_I, 1, L.sw_down.w, L.sw_down.sb, nullptr, nullptr, H, SL_MOE_I, e->hy_lists, e->hy_counts, e->hy_d, H};
   hipLaunchKernelGGL(k_qmm4_mfma_grouped<false>, dim3(H / 128, E), dim3(256), 0, e->stream, d);
   // shared expert
-  launch_qmm4_mfma(QmmArgs{e->xn, H, L.sh_gate.w, L.sh_gate.sb, M, SL_MOE_I, H, e->hy_sg, SL_MOE_I}, e->stream);
-  launch_qmm4_mfma(QmmArgs{e->xn, H, L.sh_up.w, L.sh_up.sb, M, SL_MOE_I, H, e->hy_su, SL_MOE_I}, e->stream);
+  launch_qmm4_mfma(QmmArgs{e->xn, H, L.sh_gate.w, L.sh_gate.sb, M, SL_MOE_I, H, e->hy_sg, SL_MOE_I, L.sh_up.w, L.sh_up.sb, e->hy_su}, e->stream);
   hipLaunchKernelGGL(k_swiglu_rows, dim3((M * SL_MOE_I + 255) / 256), dim3(256), 0, e->stream, e->hy_sg, e->hy_su, e->sh_act, M * SL_MOE_I);
   launch_qmm4_mfma(QmmArgs{e->sh_act, SL_MOE_I, L.sh_down.w, L.sh_down.sb, M, H, SL_MOE_I, e->hy_sy, H}, e->stream);
   hipLaunchKernelGGL(k_moe_combine_rows, dim3(H / 256, M), dim3(256), 0, e->stream, e->hy_d, L.route_scores, e->sgate, e->hy_sy, e->moe_out);

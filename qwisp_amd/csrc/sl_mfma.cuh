@@ -36,6 +36,11 @@ struct QmmArgs {
   int M, N, K;           // N % 32 == 0, K % 64 == 0
   uint16_t* y;           // [M, y_stride] fp16
   int y_stride;
+  // optional second matrix of the same shape against the same X (grid.z = 2: blockIdx.z picks the matrix), e.g. the
+  // shared expert's gate_proj and up_proj, which alone would fill a quarter of the machine each
+  const uint32_t* W2 = nullptr;
+  const uint32_t* SB2 = nullptr;
+  uint16_t* y2 = nullptr;
 };
 
 
@@ -74,8 +79,10 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
   const bool live = n0 < a.N;                            // the last workgroup's waves may have no strip
   const size_t wrow = (size_t)(live ? n0 + col : 0);
   const int chunks = a.K / (64 * G);
-  const uint32_t* wp = a.W + wrow * (a.K / 8);
-  const uint32_t* sp = a.SB + wrow * (a.K / 64);
+  const bool second = blockIdx.z != 0;
+  const uint32_t* wp = (second ? a.W2 : a.W) + wrow * (a.K / 8);
+  const uint32_t* sp = (second ? a.SB2 : a.SB) + wrow * (a.K / 64);
+  uint16_t* yout = second ? a.y2 : a.y;
   mf_f16v acc[RT];
 #pragma unroll
   for (int t = 0; t < RT; ++t)
@@ -149,7 +156,7 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int m = m0 + t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-      if (m < a.M) a.y[(size_t)m * a.y_stride + n0 + col] = f2h(acc[t][r]);
+      if (m < a.M) yout[(size_t)m * a.y_stride + n0 + col] = f2h(acc[t][r]);
     }
 }
 
@@ -326,11 +333,12 @@ inline void launch_qmm4_rt(const QmmArgs& a, dim3 grid, hipStream_t stream) {
   else hipLaunchKernelGGL((k_qmm4_mfma16<RT, 1>), grid, block, 0, stream, a);
 }
 inline void launch_qmm4_mfma(const QmmArgs& a, hipStream_t stream) {
-  const int strips = a.N / 32, tiles = (a.M + 31) / 32;
-  const unsigned gx = (unsigned)((strips + 3) / 4);
-  if (tiles >= 4 && strips * (tiles / 4) >= 768) launch_qmm4_rt<4>(a, dim3(gx, (unsigned)((tiles + 3) / 4)), stream);
-  else if (tiles >= 2 && strips * (tiles / 2) >= 768) launch_qmm4_rt<2>(a, dim3(gx, (unsigned)((tiles + 1) / 2)), stream);
-  else launch_qmm4_rt<1>(a, dim3(gx, (unsigned)tiles), stream);
+  const unsigned nz = a.W2 ? 2 : 1;
+  const int strips = a.N / 32 * (int)nz, tiles = (a.M + 31) / 32;
+  const unsigned gx = (unsigned)((a.N / 32 + 3) / 4);
+  if (tiles >= 4 && strips * (tiles / 4) >= 768) launch_qmm4_rt<4>(a, dim3(gx, (unsigned)((tiles + 3) / 4), nz), stream);
+  else if (tiles >= 2 && strips * (tiles / 2) >= 768) launch_qmm4_rt<2>(a, dim3(gx, (unsigned)((tiles + 1) / 2), nz), stream);
+  else launch_qmm4_rt<1>(a, dim3(gx, (unsigned)tiles, nz), stream);
 }
 
 }  // namespace sl
