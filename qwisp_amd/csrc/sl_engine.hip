@@ -100,7 +100,7 @@ struct sl_engine {
   bool hybrid = false;             // prefill chunks: dense projections and grouped experts on the matrix cores (not bit-identical to the GEMV order)
   // scratch of the hybrid MoE (allocated when hybrid is first enabled): routed gate / up / down results per pair,
   // shared gate / up / down rows, pairs listed per expert
-  uint16_t *hy_g = nullptr, *hy_u = nullptr, *hy_d = nullptr, *hy_sg = nullptr, *hy_su = nullptr, *hy_sy = nullptr, *hy_lists = nullptr;
+  uint16_t *hy_d = nullptr, *hy_sg = nullptr, *hy_su = nullptr, *hy_sy = nullptr, *hy_lists = nullptr;
   int32_t* hy_counts = nullptr;
   bool inject_failure = false;
   // lane batch driven from this engine's scratch: device table [n_layers][max_m] of the lanes last stepped together
@@ -812,15 +812,14 @@ float sl_last_gpu_ms(const sl_engine* e) { return e ? e->last_ms : 0.0f; }
 void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
 int sl_set_hybrid(sl_engine* e, int enable) {
   int r = guard(e); if (r) return r;
-  if (enable && !e->hy_g) {
+  if (enable && !e->hy_d) {
     const size_t rows = (size_t)(e->max_m < GROUP_CAP ? e->max_m : GROUP_CAP);
-    e->hy_g = dalloc<uint16_t>(e, rows * 8 * SL_MOE_I); e->hy_u = dalloc<uint16_t>(e, rows * 8 * SL_MOE_I);
     e->hy_d = dalloc<uint16_t>(e, rows * 8 * H);
     e->hy_sg = dalloc<uint16_t>(e, rows * SL_MOE_I); e->hy_su = dalloc<uint16_t>(e, rows * SL_MOE_I);
     e->hy_sy = dalloc<uint16_t>(e, rows * H);
     e->hy_lists = dalloc<uint16_t>(e, (size_t)SL_MAX_EXPERTS * GROUP_CAP, true);
     e->hy_counts = dalloc<int32_t>(e, SL_MAX_EXPERTS, true);
-    if (!e->hy_g || !e->hy_u || !e->hy_d || !e->hy_sg || !e->hy_su || !e->hy_sy || !e->hy_lists || !e->hy_counts) return SL_ERR_DEVICE;
+    if (!e->hy_d || !e->hy_sg || !e->hy_su || !e->hy_sy || !e->hy_lists || !e->hy_counts) return SL_ERR_DEVICE;
     SL_TRY(e, hipStreamSynchronize(e->stream));
   }
   e->hybrid = enable != 0;
