@@ -12,7 +12,7 @@ timed with HIP events on the engine's stream; roofline.avg_ms and bytes_per_laun
 launch = `--chain` tokens), and the CPU baseline (the oracle, timed on this host's cores on a bounded
 sample of the same workload).  After the timed decode region the same engine also times the batched
 paths on the same weights and reports them as extra objects of the line: `lane_batch` (32 sequences
-stepped together), `verify` (4-row verify steps) and `prefill` (a 2048-token prompt in chunks of 512
+stepped together), `verify` (4-row verify steps) and `prefill` (a 2048-token prompt in chunks of 1024
 rows, exact rows and hybrid on the matrix cores); `--lanes 0 --verify-rows 0 --prefill-chunk 0`
 skips them.
 """
@@ -57,7 +57,7 @@ def main():
     ap.add_argument("--cpu-tokens", type=int, default=4, help="decode tokens timed on the CPU oracle (0 = skip)")
     ap.add_argument("--lanes", type=int, default=32, metavar="B",
                     help="also time B lanes stepped as one batch of rows on the same weights (extra object in the JSON line; 0 = skip)")
-    ap.add_argument("--prefill-chunk", type=int, default=512, metavar="M",
+    ap.add_argument("--prefill-chunk", type=int, default=1024, metavar="M",
                     help="also time a prefill in chunks of M rows, exact rows and hybrid (matrix cores), on lanes "
                          "of the same weights (extra object in the JSON line; 0 = skip)")
     ap.add_argument("--prefill-tokens", type=int, default=2048, metavar="N",

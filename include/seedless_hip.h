@@ -328,7 +328,7 @@ void* sl_stream(sl_engine* e);
  * compute units (the reference's counterpart is the one-command-buffer step, SFV:3881-3890);
  * 0 switches to the kernel-per-stage sequence used for M > 1.  Both give identical results. */
 int sl_set_persistent(sl_engine* e, int enable);
-/* forwardRowsHybrid (SeedlessFusedVerify.swift:4240-4247): while enabled, calls with 16 <= m <= 512 rows of one
+/* forwardRowsHybrid (SeedlessFusedVerify.swift:4240-4247): while enabled, calls with 16 <= m <= 2048 rows of one
  * sequence (prefill chunks) compute the dense mixer projections (GDN in/out, attention q|k|v and o) on the matrix
  * cores, and the routed experts grouped by expert (steelMoEGather, SeedlessFusedVerify.swift:4174), with weights
  * dequantised to half.  Like the reference's matrix-unit prefill this is not bit-identical to

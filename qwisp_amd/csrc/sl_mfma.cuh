@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
 // SeedlessFusedVerify.swift:4174): the (row, slot) pairs that chose expert e are gathered, multiplied with that
 // expert's matrix once, and scattered back by pair.  Workgroup = (strip block, expert); experts nobody chose exit.
 // -------------------------------------------------------------------------------------------------
-constexpr int GROUP_CAP = 512;          // pairs per expert: an expert is chosen at most once per row, M <= 512
+constexpr int GROUP_CAP = 2048;         // pairs per expert: an expert is chosen at most once per row, M <= 2048
 
 struct QmmGroupArgs {
   const uint16_t* x;     // source rows, fp16

@@ -182,14 +182,14 @@ def test_hybrid_prefill_agrees_with_the_exact_rows(env, small_model):
     # chunking does not change a row: 48 rows at once against 16 + 32
     c1 = hyb2.forward_tokens(toks[:16]); c2 = hyb2.forward_tokens(toks[16:])
     assert same_bits(np.concatenate([c1, c2]), b)
-    # a chunk longer than 128 rows (several row blocks per GEMM, experts with many rows) gives the same rows again
-    big = env["Engine"](cfg, dev, max_m=192, max_seq_len=256)
+    # a chunk of 640 rows (several row blocks per GEMM, experts with several passes of rows) gives the same rows again
+    big = env["Engine"](cfg, dev, max_m=768, max_seq_len=800)
     big.set_hybrid(True)
-    toks2 = np.concatenate([toks, np.random.default_rng(13).integers(0, cfg.vocab, 112).astype(np.int32)])
+    toks2 = np.concatenate([toks, np.random.default_rng(13).integers(0, cfg.vocab, 592).astype(np.int32)])
     d1 = big.forward_tokens(toks2)
     assert d1 is not None, big.gpu_fault
     assert same_bits(d1[:48], b)
-    ex2 = env["Engine"](cfg, dev, max_m=192, max_seq_len=256)
+    ex2 = env["Engine"](cfg, dev, max_m=768, max_seq_len=800)
     d0 = ex2.forward_tokens(toks2)
     rel2 = np.linalg.norm(d0.astype(np.float64) - d1.astype(np.float64), axis=1) / np.linalg.norm(d0.astype(np.float64), axis=1)
     assert np.median(rel2) < 0.02 and rel2.max() < 0.15, (np.median(rel2), rel2.max())
