@@ -164,6 +164,18 @@ def main():
         dt = time.perf_counter() - t0
         lanes_report = {"lanes": B, "ms_per_step": dt * 1e3 / n_lane_steps, "tok_s_aggregate": B * n_lane_steps / dt,
                         "contexts": "8-56 tokens", "path": "rows of the kernel-per-stage path, one launch sequence for all lanes"}
+        if B >= 16:                                     # the same batch with projections, experts and lm_head on the matrix cores
+            lanes[0].set_hybrid(True)
+            for _ in range(2):
+                toks = step(lanes, toks).tolist()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n_lane_steps):
+                toks = step(lanes, toks).tolist()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            lanes_report["hybrid_matrix_cores"] = {"ms_per_step": dt * 1e3 / n_lane_steps, "tok_s_aggregate": B * n_lane_steps / dt}
+            lanes[0].set_hybrid(False)
         for lane in lanes:
             lane.close()
 

@@ -333,7 +333,9 @@ int sl_set_persistent(sl_engine* e, int enable);
  * cores, and the routed experts grouped by expert (steelMoEGather, SeedlessFusedVerify.swift:4174), with weights
  * dequantised to half.  Like the reference's matrix-unit prefill this is not bit-identical to
  * the GEMV order (tolerance-level agreement) but deterministic and independent of how a prompt is chunked.
- * Decode steps, verify rows below 16 and lane batches are unaffected. */
+ * Enabled on the engine that drives a lane batch (lanes[0] of sl_lane_step_argmax), batches of 16 or more lanes take
+ * the same projections and lm_head to the matrix cores (the experts too from 64 lanes on); recurrent state, caches
+ * and attention stay on the exact kernels.  Decode steps and steps of fewer than 16 rows are unaffected. */
 int sl_set_hybrid(sl_engine* e, int enable);
 
 /* Diagnostic: while enabled, workgroups 0 and 100 of the single-launch step record a 100 MHz clock stamp

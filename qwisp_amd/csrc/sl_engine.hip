@@ -293,8 +293,9 @@ void launch_hidden_tile(sl_engine* e, const HiddenArgs& ha, const uint32_t* w, c
   hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, false>), dim3(G, (M + 7) / 8), dim3(256), 0, e->stream, HiddenArgs{}, e->xn, H,
                      w, sb, N, e->proj, PROJ_STRIDE, M);
 }
-// Hybrid prefill: chunks of at least 16 rows of one sequence take the dense mixer projections to the matrix cores.
-bool use_matrix_cores(const sl_engine* e, int M, const LaneRef* lanes) { return e->hybrid && !lanes && M >= 16 && M <= GROUP_CAP; }
+// Hybrid mode: steps of at least 16 rows (prefill chunks, lane batches) take the dense projections to the matrix cores.
+// (Rows of one sequence or one row each of a batch of lanes: the projections and the experts do not care.)
+bool use_matrix_cores(const sl_engine* e, int M, const LaneRef* lanes) { (void)lanes; return e->hybrid && M >= 16 && M <= GROUP_CAP; }
 // `lanes` (null for rows of one sequence) = this layer's row of the lane table: row b of the batch is lane b's next token.
 void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs& ha, const LaneRef* lanes) {
   const bool mm = use_matrix_cores(e, M, lanes);
@@ -375,7 +376,10 @@ void launch_layers(sl_engine* e, int M, const LaneRef* lane_tab = nullptr, int l
     if (L.is_linear) launch_gdn_mixer(e, L, li, M, ha, lanes);
     else launch_attn_mixer(e, L, M, ha, lanes, lane_tiles);
     HiddenArgs hb{e->hB, e->mix, L.post_ln, e->hA, e->xn};
-    if (use_matrix_cores(e, M, lanes)) launch_moe_hybrid(e, L, M, hb);
+    // grouping by expert pays once an expert sees several rows; a batch of fewer than 64 lanes leaves most experts
+    // with one row or none, and the per-row expert kernels stream the same weights with less overhead (rows of one
+    // sequence always take the grouped path, so that a row's result does not depend on the size of its chunk)
+    if (use_matrix_cores(e, M, lanes) && (!lanes || M >= 64)) launch_moe_hybrid(e, L, M, hb);
     else launch_moe(e, L, M, hb);
   }
 }
@@ -387,6 +391,7 @@ void advance(sl_engine* e, int M) {
 void launch_head(sl_engine* e, int M, const HiddenArgs& ha, int out_off, bool feed) {
   const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
+  bool have_tokens = false;
   if (M >= 2) {
     // residual + final norm once per row, then the row-tiled lm_head (weights streamed once per 8 rows)
     const uint16_t* xin = ha.h_in;
@@ -396,15 +401,23 @@ void launch_head(sl_engine* e, int M, const HiddenArgs& ha, int out_off, bool fe
       hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
       xin = hn.xn_out;
     }
-    hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, false, true>), dim3(e->n_cand, (M + 7) / 8), dim3(256), 0, e->stream, HiddenArgs{}, xin, H,
-                       e->lm_head.w, e->lm_head.sb, e->vocab, e->logits, e->vocab, M, e->cand_v, e->cand_i);
+    if (use_matrix_cores(e, M, nullptr) && e->vocab % 32 == 0) {
+      // hybrid mode: lm_head on the matrix cores, arg-max of the rounded logits rows
+      launch_qmm4_mfma(QmmArgs{xin, H, e->lm_head.w, e->lm_head.sb, M, e->vocab, H, e->logits, e->vocab}, e->stream);
+      hipLaunchKernelGGL(k_argmax_logits, dim3(M), dim3(1024), 0, e->stream, e->logits, e->vocab, e->tok_out, out_off);
+      have_tokens = true;
+    } else {
+      hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, false, true>), dim3(e->n_cand, (M + 7) / 8), dim3(256), 0, e->stream, HiddenArgs{}, xin, H,
+                         e->lm_head.w, e->lm_head.sb, e->vocab, e->logits, e->vocab, M, e->cand_v, e->cand_i);
+    }
   } else {
     hipLaunchKernelGGL(k_head, dim3(e->n_cand, M), dim3(256), 0, e->stream, ha, e->lm_head.w, e->lm_head.sb, e->vocab,
                        e->logits, e->cand_v, e->cand_i);
   }
   if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
-  hipLaunchKernelGGL(k_argmax_final, dim3(M), dim3(256), 0, e->stream, e->cand_v, e->cand_i, e->n_cand, e->tok_out, out_off,
-                     feed ? e->tok_in : (int32_t*)nullptr);
+  if (!have_tokens)
+    hipLaunchKernelGGL(k_argmax_final, dim3(M), dim3(256), 0, e->stream, e->cand_v, e->cand_i, e->n_cand, e->tok_out, out_off,
+                       feed ? e->tok_in : (int32_t*)nullptr);
 }
 // `steps` batch-1 steps in a single persistent launch (each token fed back on the device); host mirrors advance
 // as the kernel's own update does.

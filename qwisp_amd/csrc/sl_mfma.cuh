@@ -324,6 +324,33 @@ __global__ __launch_bounds__(256) void k_moe_combine_rows(const uint16_t* __rest
 
 // Host-side launch: row tiles per wave chosen so that there are about as many wave tasks as SIMDs (1024): wide
 // projections share the unpacking over 128 rows, narrow ones spread their rows over more waves instead.
+// Arg-max of rows of logits (first maximum, i.e. the lowest index on ties, of the half values): one workgroup per row.
+__global__ __launch_bounds__(1024) void k_argmax_logits(const uint16_t* __restrict__ logits, int V, int32_t* __restrict__ tok_out,
+                                                        int out_off) {
+  __shared__ float s_v[1024];
+  __shared__ int s_i[1024];
+  const int m = blockIdx.x, tid = threadIdx.x;
+  const uint16_t* row = logits + (size_t)m * V;
+  float bv = -__int_as_float(0x7f800000);
+  int bi = 0x7fffffff;
+  for (int c = tid * 8; c < V; c += 1024 * 8) {          // V % 8 == 0
+    float f[8];
+    unpack8(ld16(row + c), f);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) if (f[i] > bv) { bv = f[i]; bi = c + i; }
+  }
+  s_v[tid] = bv; s_i[tid] = bi;
+  __syncthreads();
+  for (int s = 512; s > 0; s >>= 1) {
+    if (tid < s) {
+      const float ov = s_v[tid + s]; const int oi = s_i[tid + s];
+      if (ov > s_v[tid] || (ov == s_v[tid] && oi < s_i[tid])) { s_v[tid] = ov; s_i[tid] = oi; }
+    }
+    __syncthreads();
+  }
+  if (tid == 0) tok_out[out_off + m] = s_i[0];
+}
+
 template <int RT>
 inline void launch_qmm4_rt(const QmmArgs& a, dim3 grid, hipStream_t stream) {
   const dim3 block(256);

@@ -129,6 +129,52 @@ def test_eleven_lanes_in_one_batch_equal_solo(env, small_model):
 
 
 @pytest.mark.gpu
+def test_lane_batch_on_the_matrix_cores_stays_close_to_solo(env, small_model):
+    """Hybrid mode on the engine that drives a lane batch: with 16 or more lanes the projections, the grouped experts
+    and lm_head of the batched step run on the matrix cores (tolerance-level, like the hybrid prefill); the lanes'
+    recurrent state, caches and attention stay on the exact kernels.  Logits stay within a few per cent of solo
+    engines on the exact path and most tokens agree; switching hybrid off returns to the exact bits."""
+    cfg, dev, host = small_model
+    B = 16
+    base = env["Engine"](cfg, dev, max_m=B, max_seq_len=64)
+    lanes = [base.new_lane(max_m=B, max_seq_len=64) for _ in range(B)]
+    solos = [env["Engine"](cfg, dev, max_m=B, max_seq_len=64) for _ in range(B)]
+    rng = np.random.default_rng(79)
+    cur = []
+    for i, (lane, solo) in enumerate(zip(lanes, solos)):
+        pr = rng.integers(0, cfg.vocab, 2 + (5 * i) % 9).tolist()
+        ta, tb = lane.step_argmax(pr), solo.step_argmax(pr)
+        assert ta.tolist() == tb.tolist()
+        cur.append(int(ta[-1]))
+    lanes[0].set_hybrid(True)
+    got = type(base).lane_step_argmax(lanes, cur)
+    assert got is not None, [l.gpu_fault for l in lanes]
+    want = [int(solo.step_argmax([t])[0]) for solo, t in zip(solos, cur)]
+    agree = sum(int(a) == b for a, b in zip(got.tolist(), want))
+    rels = []
+    for lane, solo in zip(lanes, solos):
+        la, lb = lane.logits_row(0).astype(np.float64), solo.logits_row(0).astype(np.float64)
+        rels.append(np.linalg.norm(la - lb) / np.linalg.norm(lb))
+    assert max(rels) < 0.05 and agree >= B - 2, (max(rels), agree)
+    assert any(not same_bits(lane.logits_row(0), solo.logits_row(0)) for lane, solo in zip(lanes, solos))
+    # exact again: feed both sides the solo tokens and compare bits of a step from (slightly different) caches is not
+    # meaningful, so rebuild: fresh lanes, same prompts, hybrid off -> the exact bits
+    lanes[0].set_hybrid(False)
+    for lane in lanes:
+        lane.close()
+    lanes = [base.new_lane(max_m=B, max_seq_len=64) for _ in range(B)]
+    rng = np.random.default_rng(79)
+    cur = []
+    for i, lane in enumerate(lanes):
+        pr = rng.integers(0, cfg.vocab, 2 + (5 * i) % 9).tolist()
+        cur.append(int(lane.step_argmax(pr)[-1]))
+    got = type(base).lane_step_argmax(lanes, cur)
+    assert got.tolist() == want
+    for lane in lanes:
+        lane.close()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("m,n,k", [(1, 32, 64), (5, 96, 512), (32, 128, 2048), (33, 160, 2048), (64, 2048, 4096), (100, 64, 512), (300, 96, 512)])
 def test_mfma_qmm4_against_the_oracle_rows(env, m, n, k):
     """Y = X W^T with 4-bit weights on the matrix cores.  Not bit-identical to the GEMV order (the reference
