@@ -330,8 +330,8 @@ void* sl_stream(sl_engine* e);
 int sl_set_persistent(sl_engine* e, int enable);
 /* forwardRowsHybrid (SeedlessFusedVerify.swift:4240-4247): while enabled, calls with 16 <= m <= 2048 rows of one
  * sequence (prefill chunks) compute the dense mixer projections (GDN in/out, attention q|k|v and o) on the matrix
- * cores, and the routed experts grouped by expert (steelMoEGather, SeedlessFusedVerify.swift:4174), with weights
- * dequantised to half.  Like the reference's matrix-unit prefill this is not bit-identical to
+ * cores, the routed experts grouped by expert (steelMoEGather, SeedlessFusedVerify.swift:4174) with weights
+ * dequantised to half, and the attention tile pass (scores, probabilities in half, values).  Like the reference's matrix-unit prefill this is not bit-identical to
  * the GEMV order (tolerance-level agreement) but deterministic and independent of how a prompt is chunked.
  * Enabled on the engine that drives a lane batch (lanes[0] of sl_lane_step_argmax), batches of 16 or more lanes take
  * the same projections and lm_head to the matrix cores (the experts too from 64 lanes on); recurrent state, caches

@@ -355,7 +355,8 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
   SdpaArgs s{};
   s.qrot = e->qrot; s.kcache = L.kcache; s.vcache = L.vcache; s.st = e->st; s.maxSeq = e->max_seq; s.maxTiles = e->max_tiles;
   s.pm = e->pm; s.pl = e->pl; s.po = e->po; s.lanes = lanes;
-  hipLaunchKernelGGL(k_sdpa_tile, dim3(tiles, SL_ATT_KV, M), dim3(256), 0, e->stream, s);
+  if (mm && !lanes) hipLaunchKernelGGL(k_sdpa_tile_mfma, dim3(tiles, SL_ATT_KV, (M + 31) / 32), dim3(256), 0, e->stream, SdpaMmArgs{s, M});
+  else hipLaunchKernelGGL(k_sdpa_tile, dim3(tiles, SL_ATT_KV, M), dim3(256), 0, e->stream, s);
   SdpaMergeArgs g{};
   g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore; g.lanes = lanes;
   hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);

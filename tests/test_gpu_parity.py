@@ -404,6 +404,41 @@ def test_attention_layer_decode(env, S):
     assert same_bits(gk, wk) and same_bits(gv, wv)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("S,m", [(0, 16), (0, 100), (37, 33), (200, 64), (1000, 130)])
+def test_attention_layer_chunk_on_the_matrix_cores(env, S, m):
+    """Hybrid mode, one attention layer: a chunk of m rows over S cached tokens (masks inside the first tile, ragged
+    row blocks, several key tiles) against the exact kernels of the same engine class -- the same K and V rows in
+    the cache bit for bit (they are written by the exact prep kernel from projections that only differ by the GEMM),
+    outputs within the tolerance of half-precision probabilities."""
+    cfg = ModelConfig(n_layers=1, n_experts=8, vocab=0, layer_types=("attn",))
+    dev, host = device_and_host_model(cfg)
+    ex = env["Engine"](cfg, dev, max_m=m, max_seq_len=S + m + 8)
+    hy = env["Engine"](cfg, dev, max_m=m, max_seq_len=S + m + 8)
+    hy.set_hybrid(True)
+    if S:
+        k = env["orc"].synth_f16((abi.ATT_KV, S, abi.ATT_D), 1410, 0.0, 1.0)
+        v = env["orc"].synth_f16((abi.ATT_KV, S, abi.ATT_D), 1411, 0.0, 1.0)
+        assert ex.load_layer_cache(0, k, v) and hy.load_layer_cache(0, k, v)
+    x = xrows(m, 1420 + m)
+    a, b = ex.attn_layer_rows(0, x), hy.attn_layer_rows(0, x)
+    assert a is not None and b is not None, (ex.gpu_fault, hy.gpu_fault)
+    af, bf = a.astype(np.float64), b.astype(np.float64)
+    assert np.all(np.isfinite(bf))
+    rel = np.linalg.norm(af - bf, axis=1) / np.linalg.norm(af, axis=1)
+    assert rel.max() < 0.02 and not same_bits(a, b), rel.max()
+    # a row does not depend on the rows that share its chunk: the last 16 rows again, on their own
+    if m >= 32:
+        hy2 = env["Engine"](cfg, dev, max_m=m, max_seq_len=S + m + 8)
+        hy2.set_hybrid(True)
+        if S:
+            assert hy2.load_layer_cache(0, k, v)
+        b1 = hy2.attn_layer_rows(0, x[:m - 16]); b2 = hy2.attn_layer_rows(0, x[m - 16:])
+        assert same_bits(np.concatenate([b1, b2]), b)
+        hy2.close()
+    ex.close(); hy.close()
+
+
 # ---- benchmark configuration 3, reduced: the whole hybrid stack --------------------------------------------
 @pytest.fixture(scope="module")
 def small_model(env):
