@@ -13,8 +13,8 @@ launch = `--chain` tokens), and the CPU baseline (the oracle, timed on this host
 sample of the same workload).  After the timed decode region the same engine also times the batched
 paths on the same weights and reports them as extra objects of the line: `lane_batch` (32 sequences
 stepped together), `verify` (4-row verify steps) and `prefill` (a 2048-token prompt in chunks of 1024
-rows, exact rows and hybrid on the matrix cores); `--lanes 0 --verify-rows 0 --prefill-chunk 0`
-skips them.
+rows, exact rows and hybrid on the matrix cores) and `context_sweep` (decode after 4K and 16K prompts);
+`--lanes 0 --verify-rows 0 --prefill-chunk 0 --context-sweep ''` skips them.
 """
 import argparse
 import json
@@ -65,6 +65,9 @@ def main():
     ap.add_argument("--verify-rows", type=int, default=4, metavar="R",
                     help="also time verify steps of R rows ([token] + R-1 drafts through stepArgmax) at the decode context "
                          "(extra object in the JSON line; 0 = skip)")
+    ap.add_argument("--context-sweep", type=str, default="4096,16384", metavar="S1,S2",
+                    help="also time batch-1 decode after prompts of these lengths (hybrid prefill in chunks of 1024; extra "
+                         "object in the JSON line; empty = skip)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run a plain device copy of this many MiB (reference for rocprofv3 FETCH_SIZE/WRITE_SIZE) and exit")
     args = ap.parse_args()
@@ -217,6 +220,32 @@ def main():
                 lane.close()
             prefill_report[name] = {"ms": times[-1] * 1e3, "tok_s": PF / times[-1]}
 
+    sweep_report = None
+    if args.context_sweep:
+        sweep_report = []
+        for S in [int(x) for x in args.context_sweep.split(",") if x]:
+            lane = eng.new_lane(max_m=1024, max_seq_len=S + 128)
+            lane.set_hybrid(True)
+            pr = np.random.default_rng(6000 + S).integers(0, cfg.vocab, S).astype(np.int32)
+            o = lane.greedy_generate(pr, 1, chain_k=args.chain)
+            assert o is not None, lane.gpu_fault
+            t = int(o[0])
+            o = lane.chained_step_argmax(t, args.chain)          # warm-up chain
+            t = int(o[-1])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            n_tok = 8 * args.chain
+            for _ in range(8):
+                o = lane.chained_step_argmax(t, args.chain)
+                t = int(o[-1])
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            assert o is not None, lane.gpu_fault
+            b_tok, _ = step_bytes(cfg, S + args.chain + n_tok // 2)
+            sweep_report.append({"context": S, "ms_per_token": dt * 1e3 / n_tok, "tok_s": n_tok / dt, "bytes_per_token": b_tok,
+                                 "frac_of_peak": b_tok / (dt / n_tok) / 1e9 / HBM_PEAK_GBS})
+            lane.close()
+
     cpu = None
     if host is not None:
         from oracle import orc
@@ -253,6 +282,7 @@ def main():
         "lane_batch": lanes_report,
         "prefill": prefill_report,
         "verify": verify_report,
+        "context_sweep": sweep_report,
         "setup_s": {"generate": t_gen, "prefill_512": t_prefill},
         "tokens_head": stream[:8],
     }))

@@ -693,6 +693,7 @@ SL_DEV void store_hist(const LayerP& Y, int li, const GdnHist& gh) {
 }
 
 // ---- K = 4096 projection (GDN out_proj with gated rmsnorm prologue / attention merge + o_proj) ---------
+constexpr int FLOW_MERGE_WGS = 16;     // = query heads
 SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t base, const GdnHist& gh) {
   FLOW_IDS;
   const DecodeP& P = F.d;
@@ -703,13 +704,14 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   wload_row<2>(wr.w[0], wr.sb[0], uni(Y.out_w), uni(Y.out_sb), (size_t)(valid ? gw : 0), valid, lane);
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
-  if (!lin && wg >= G - 2) {        // the last workgroups own a tile unit only in very long contexts, so their
-                                     // waves have no stores of their own to wait for
-    // Merge the attention tiles in order with the global max: 8 heads per workgroup, two waves per head, a lane
-    // owns one 16-byte chunk (2 dims) of the 256; each wave polls on its own.  The round trips are batched:
-    // lane i fetches {max, sum} of tile t0+i (64 tiles per load) and the partials of MB tiles are in flight at
-    // a time; the accumulation itself runs in tile order.
-    const int h = (wg - (G - 2)) * 8 + (wave >> 1), slot0 = h * uni(P.max_tiles), chunk = 64 * (wave & 1) + lane;
+  if (!lin && wg >= G - FLOW_MERGE_WGS && wave < 2) {
+    // Merge the attention tiles in order with the global max: one head per workgroup on the last 16 workgroups (they
+    // own a tile unit only at contexts of several thousand tokens, so their waves normally have no stores of their own
+    // to wait for; a long context's partials, a megabyte per four heads, then come in over 16 compute units), two
+    // waves per head, a lane owns one 16-byte chunk (2 dims) of the 256; each wave polls on its own.  The round
+    // trips are batched: lane i fetches {max, sum} of tile t0+i (64 tiles per load) and the partials of MB tiles
+    // are in flight at a time; the accumulation itself runs in tile order.
+    const int h = wg - (G - FLOW_MERGE_WGS), slot0 = h * uni(P.max_tiles), chunk = 64 * wave + lane;
     const rsrc_t rml = co_rsrc(uni(F.tml)), rpo = co_rsrc(uni(F.tpo)), rp = co_rsrc(uni(F.tproj));
     int fail = 0;
     float Mx = NEG;
