@@ -693,7 +693,7 @@ SL_DEV void store_hist(const LayerP& Y, int li, const GdnHist& gh) {
 }
 
 // ---- K = 4096 projection (GDN out_proj with gated rmsnorm prologue / attention merge + o_proj) ---------
-constexpr int FLOW_MERGE_WGS = 16;     // = query heads
+constexpr int FLOW_MERGE_WGS = 32;     // two per query head
 SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t base, const GdnHist& gh) {
   FLOW_IDS;
   const DecodeP& P = F.d;
@@ -704,104 +704,124 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   wload_row<2>(wr.w[0], wr.sb[0], uni(Y.out_w), uni(Y.out_sb), (size_t)(valid ? gw : 0), valid, lane);
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
-  if (!lin && wg >= G - FLOW_MERGE_WGS && wave < 2) {
-    // Merge the attention tiles in order with the global max: one head per workgroup on the last 16 workgroups (they
-    // own a tile unit only at contexts of several thousand tokens, so their waves normally have no stores of their own
-    // to wait for; a long context's partials, a megabyte per four heads, then come in over 16 compute units), two
-    // waves per head, a lane owns one 16-byte chunk (2 dims) of the 256; each wave polls on its own.  The round
-    // trips are batched: lane i fetches {max, sum} of tile t0+i (64 tiles per load) and the partials of MB tiles
-    // are in flight at a time; the accumulation itself runs in tile order.
-    const int h = wg - (G - FLOW_MERGE_WGS), slot0 = h * uni(P.max_tiles), chunk = 64 * wave + lane;
+  if (!lin && wg >= G - FLOW_MERGE_WGS) {
+    // Merge the attention tiles in order with the global max: the last 32 workgroups take half a head each (they own
+    // a tile unit only at contexts of several thousand tokens, so their waves normally have no stores of their own
+    // to wait for).  Wave 0 is the merging wave: a lane owns one 16-byte chunk (2 dims) of its 128 dims.
+    // First round trip: {max, sum} of the first 64 tiles (lane i fetches tile i), the partials of the first MB tiles
+    // and the output gate (it sits in the q projection of this step) are polled together, each piece until it has
+    // arrived; at contexts of up to MB tiles that is everything the merge needs.  Beyond that a round trip per MB
+    // tiles would dominate (about 3 us each, whatever its size), so all 16 waves fetch: per block of 64 tiles wave w
+    // polls tiles 4w .. 4w+3 and parks their values in LDS (the value tile's space), and wave 0 then adds the block
+    // up from LDS.  The accumulation always runs in tile order.
+    const int mi = wg - (G - FLOW_MERGE_WGS), h = mi >> 1, slot0 = h * uni(P.max_tiles), chunk = 64 * (mi & 1) + lane;
     const rsrc_t rml = co_rsrc(uni(F.tml)), rpo = co_rsrc(uni(F.tpo)), rp = co_rsrc(uni(F.tproj));
-    int fail = 0;
-    float Mx = NEG;
-    // First round trip: {max, sum} of the first 64 tiles, the partials of the first MB tiles and the output gate
-    // (it sits in the q projection of this step) are polled together, each piece until it has arrived; at short
-    // contexts that is everything the merge needs.
     constexpr int MB = 12;
-    uint4 a[MB];
+    int fail = 0;
+    float Mx = NEG, Ls = 0.0f, O0 = 0.0f, O1 = 0.0f;
     uint4 m0 = make_uint4(0, 0, 0, 0);
     uint2 g2 = make_uint2(0u, 0u);
-    {
-      const bool mine = lane < nt;
-      const int cnt0 = min(MB, nt);
-      bool mdone = false, gdone = false;
-      unsigned have = 0, spins = 0;
-      for (;;) {
-        if (!mdone) {
-          bool ok = true;
-          if (mine) { m0 = ldw4(rml, (slot0 + lane) * 4); ok = m0.z == tcore32 && m0.w == tcore32; }
-          mdone = __all(ok ? 1 : 0) != 0;
-        }
-        if (!gdone) {
-          g2 = ldw2(rp, h * 512 + 256 + 2 * chunk);
-          gdone = __all((tag_ok(g2.x, tin) && tag_ok(g2.y, tin)) ? 1 : 0) != 0;
-        }
-#pragma unroll
-        for (int u = 0; u < MB; ++u) {
-          if (u < cnt0 && !(have & (1u << u))) {
-            a[u] = ldw4(rpo, ((slot0 + u) * 128 + chunk) * 4);
-            if (__all((a[u].z == tcore32 && a[u].w == tcore32) ? 1 : 0)) have |= 1u << u;
-          }
-        }
-        if (mdone && gdone && have == (1u << cnt0) - 1u) break;
-        if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
-        __builtin_amdgcn_s_sleep(1);
-      }
-      Mx = tree_max<64>(mine ? __uint_as_float(m0.x) : NEG);
-    }
-    for (int t0 = 64; t0 < nt && !fail; t0 += 64) {       // maxima of the tiles beyond the first 64
-      const bool mine = t0 + lane < nt;
-      unsigned spins = 0;
-      for (;;) {
-        bool ok = true;
-        float pm = NEG;
-        if (mine) { const uint4 m = ldw4(rml, (slot0 + t0 + lane) * 4); ok = m.z == tcore32 && m.w == tcore32; pm = __uint_as_float(m.x); }
-        if (__all(ok ? 1 : 0)) { Mx = fmaxf(Mx, tree_max<64>(pm)); break; }
-        if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
-        __builtin_amdgcn_s_sleep(1);
-      }
-    }
-    float Ls = 0.0f, O0 = 0.0f, O1 = 0.0f;
-    for (int t0 = 0; t0 < nt && !fail; t0 += 64) {
-      float fl = 0.0f, pl = 0.0f;                         // lane i: scale and sum of tile t0+i (tags verified above)
-      if (t0 + lane < nt) {
-        const uint4 m = t0 == 0 ? m0 : ldw4(rml, (slot0 + t0 + lane) * 4);
-        fl = exp_c(__uint_as_float(m.x) - Mx); pl = __uint_as_float(m.y);
-      }
-      const int cnt = min(64, nt - t0);
-      for (int u0 = 0; u0 < cnt && !fail; u0 += MB) {
-        if (t0 + u0 > 0) {                                // the first batch is already here
-          unsigned spins = 0;
-          for (;;) {
+    if (wave == 0) {
+      uint4 a[MB];
+      {
+        const bool mine = lane < nt;
+        const int cnt0 = min(MB, nt);
+        bool mdone = false, gdone = false;
+        unsigned have = 0, spins = 0;
+        for (;;) {
+          if (!mdone) {
             bool ok = true;
-#pragma unroll
-            for (int u = 0; u < MB; ++u) {
-              if (u0 + u < cnt) {
-                a[u] = ldw4(rpo, ((slot0 + t0 + u0 + u) * 128 + chunk) * 4);
-                ok = ok && a[u].z == tcore32 && a[u].w == tcore32;
-              }
-            }
-            if (__all(ok ? 1 : 0)) break;
-            if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
-            __builtin_amdgcn_s_sleep(1);
+            if (mine) { m0 = ldw4(rml, (slot0 + lane) * 4); ok = m0.z == tcore32 && m0.w == tcore32; }
+            mdone = __all(ok ? 1 : 0) != 0;
           }
-          if (fail) break;
+          if (!gdone) {
+            g2 = ldw2(rp, h * 512 + 256 + 2 * chunk);
+            gdone = __all((tag_ok(g2.x, tin) && tag_ok(g2.y, tin)) ? 1 : 0) != 0;
+          }
+#pragma unroll
+          for (int u = 0; u < MB; ++u) {
+            if (u < cnt0 && !(have & (1u << u))) {
+              a[u] = ldw4(rpo, ((slot0 + u) * 128 + chunk) * 4);
+              if (__all((a[u].z == tcore32 && a[u].w == tcore32) ? 1 : 0)) have |= 1u << u;
+            }
+          }
+          if (mdone && gdone && have == (1u << cnt0) - 1u) break;
+          if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+          __builtin_amdgcn_s_sleep(1);
         }
+        Mx = tree_max<64>(mine ? __uint_as_float(m0.x) : NEG);
+      }
+      for (int t0 = 64; t0 < nt && !fail; t0 += 64) {       // maxima of the tiles beyond the first 64
+        const bool mine = t0 + lane < nt;
+        unsigned spins = 0;
+        for (;;) {
+          bool ok = true;
+          float pm = NEG;
+          if (mine) { const uint4 m = ldw4(rml, (slot0 + t0 + lane) * 4); ok = m.z == tcore32 && m.w == tcore32; pm = __uint_as_float(m.x); }
+          if (__all(ok ? 1 : 0)) { Mx = fmaxf(Mx, tree_max<64>(pm)); break; }
+          if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+          __builtin_amdgcn_s_sleep(1);
+        }
+      }
+      if (!fail) {                                          // the first batch is already here
+        float fl = 0.0f, pl = 0.0f;
+        if (lane < nt) { fl = exp_c(__uint_as_float(m0.x) - Mx); pl = __uint_as_float(m0.y); }
 #pragma unroll
         for (int u = 0; u < MB; ++u) {
-          if (u0 + u < cnt) {
-            const float f = row_lane_f(fl, u0 + u), l = row_lane_f(pl, u0 + u);
+          if (u < nt) {
+            const float f = row_lane_f(fl, u), l = row_lane_f(pl, u);
             Ls = fmaf(l, f, Ls);
             O0 = fmaf(__uint_as_float(a[u].x), f, O0); O1 = fmaf(__uint_as_float(a[u].y), f, O1);
           }
         }
       }
     }
+    if (nt > MB) {                                          // uniform for the grid
+      uint2* park = reinterpret_cast<uint2*>(g_vt);         // [64 tiles][64 lanes] {o0, o1}
+      __syncthreads();                                      // this workgroup's own tile units are done with the value tile
+      for (int t0 = 0; t0 < nt; t0 += 64) {
+        uint4 q[4];
+        unsigned spins = 0;
+        for (;;) {
+          bool ok = true;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int t = t0 + 4 * wave + j;
+            if (t >= MB && t < nt) { q[j] = ldw4(rpo, ((slot0 + t) * 128 + chunk) * 4); ok = ok && q[j].z == tcore32 && q[j].w == tcore32; }
+          }
+          if (__all(ok ? 1 : 0)) break;
+          if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+          __builtin_amdgcn_s_sleep(1);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int t = t0 + 4 * wave + j;
+          if (t >= MB && t < nt) park[(4 * wave + j) * 64 + lane] = make_uint2(q[j].x, q[j].y);
+        }
+        __syncthreads();
+        if (wave == 0 && !fail) {
+          float fl = 0.0f, pl = 0.0f;                       // lane i: scale and sum of tile t0+i (tags verified above)
+          if (t0 + lane < nt) {
+            const uint4 m = t0 == 0 ? m0 : ldw4(rml, (slot0 + t0 + lane) * 4);
+            fl = exp_c(__uint_as_float(m.x) - Mx); pl = __uint_as_float(m.y);
+          }
+          const int lo = t0 == 0 ? MB : 0, hi = min(64, nt - t0);
+          for (int u = lo; u < hi; ++u) {
+            const uint2 v = park[u * 64 + lane];
+            const float f = row_lane_f(fl, u), l = row_lane_f(pl, u);
+            Ls = fmaf(l, f, Ls);
+            O0 = fmaf(__uint_as_float(v.x), f, O0); O1 = fmaf(__uint_as_float(v.y), f, O1);
+          }
+        }
+        __syncthreads();                                    // the block is consumed before the next one is parked
+      }
+    }
     if (fail) st_co32(uni(P.bar) + 32, 1u);
-    const uint32_t r0 = tagged(f16r(f16r(O0 / Ls) * sigmoid16(lo_h(g2.x))), tmerge);
-    const uint32_t r1 = tagged(f16r(f16r(O1 / Ls) * sigmoid16(lo_h(g2.y))), tmerge);
-    if (!fail) stw2(co_rsrc(uni(F.tycore)), h * 256 + 2 * chunk, r0, r1);
+    if (wave == 0 && !fail) {
+      const uint32_t r0 = tagged(f16r(f16r(O0 / Ls) * sigmoid16(lo_h(g2.x))), tmerge);
+      const uint32_t r1 = tagged(f16r(f16r(O1 / Ls) * sigmoid16(lo_h(g2.y))), tmerge);
+      stw2(co_rsrc(uni(F.tycore)), h * 256 + 2 * chunk, r0, r1);
+    }
   }
   if (wg * DEC_WAVES >= H) {                       // no output row here (uniform per workgroup): nothing to fetch
     if (lin) store_hist(Y, li, gh);
