@@ -806,11 +806,20 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
             fl = exp_c(__uint_as_float(m.x) - Mx); pl = __uint_as_float(m.y);
           }
           const int lo = t0 == 0 ? MB : 0, hi = min(64, nt - t0);
-          for (int u = lo; u < hi; ++u) {
-            const uint2 v = park[u * 64 + lane];
-            const float f = row_lane_f(fl, u), l = row_lane_f(pl, u);
-            Ls = fmaf(l, f, Ls);
-            O0 = fmaf(__uint_as_float(v.x), f, O0); O1 = fmaf(__uint_as_float(v.y), f, O1);
+          for (int u0 = lo; u0 < hi; u0 += 8) {             // eight LDS reads and sixteen lane reads at a time, used in tile order
+            uint2 v[8];
+            float f[8], l[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = park[min(u0 + i, 63) * 64 + lane];
+            lanes8(fl, u0, f);
+            lanes8(pl, u0, l);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              if (u0 + i < hi) {
+                Ls = fmaf(l[i], f[i], Ls);
+                O0 = fmaf(__uint_as_float(v[i].x), f[i], O0); O1 = fmaf(__uint_as_float(v[i].y), f[i], O1);
+              }
+            }
           }
         }
         __syncthreads();                                    // the block is consumed before the next one is parked
