@@ -29,7 +29,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 PROMPT_LEN = 512
 # HBM bytes per decoded token: rocprofv3 FETCH_SIZE + WRITE_SIZE of a k_decode_flow launch (profiles/) / its 8 tokens
-TRAFFIC_BYTES_PER_TOKEN = 1935870906   # 2 x FETCH_SIZE (copy-calibrated) + WRITE_SIZE, in bytes, at context ~525
+TRAFFIC_BYTES_PER_TOKEN = 1936080204   # 2 x FETCH_SIZE (copy-calibrated) + WRITE_SIZE, in bytes, at context ~525
 
 
 def step_bytes(cfg, ctx):
