@@ -535,6 +535,30 @@ def test_persistent_step_long_context(env, small_model):
             assert same_bits(x, y), (li, first_diff(x, y))
 
 
+def test_persistent_step_with_several_tile_units_per_workgroup(env, small_model):
+    """Beyond 8192 tokens of context there are more (key tile, kv head) units than workgroups: some workgroups take
+    two units in turn, the merge runs over three blocks of 64 tiles.  Same tokens, logits and caches as the
+    kernel-per-stage sequence."""
+    cfg, dev, host = small_model
+    a = env["Engine"](cfg, dev, max_m=256, max_seq_len=8704)
+    b = env["Engine"](cfg, dev, max_m=256, max_seq_len=8704)
+    assert b.set_persistent(False)
+    toks = np.random.default_rng(79).integers(0, cfg.vocab, 8500).astype(np.int32)
+    for eng in (a, b):
+        for i in range(0, len(toks), 256):
+            assert eng.step_argmax(toks[i:i + 256]) is not None, eng.gpu_fault
+    ta = a.chained_step_argmax(11, 12)
+    tb = b.chained_step_argmax(11, 12)
+    assert ta is not None and tb is not None, (a.gpu_fault, b.gpu_fault)
+    assert ta.tolist() == tb.tolist()
+    assert same_bits(a.logits_row(0), b.logits_row(0))
+    for li in range(cfg.n_layers):
+        for x, y in zip(a.read_layer_cache(li), b.read_layer_cache(li)):
+            assert same_bits(x, y), (li, first_diff(x, y))
+    a.close(); b.close()
+
+
+
 def test_persistent_step_across_the_attention_split_boundary(env, small_model):
     """Up to 2048 tokens of context an attention tile unit is split four ways over the query heads, beyond that
     it is not; the merge polls 12 tiles per round trip.  Steps that cross position 2048 (and the 13th tile at
