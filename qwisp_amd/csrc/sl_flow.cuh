@@ -373,6 +373,10 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
   const float NEG = -__int_as_float(0x7f800000);
   const int N = pos + 1, nt = (N + SDPA_TILE - 1) / SDPA_TILE;
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag32(base, li, FS_CORE);
+  // The queries of the kv head's group and the new key and value row are the same for every unit of a workgroup
+  // (with an even grid a workgroup stays with one kv head): polled, normed and rotated for its first unit only.
+  uint4 w4 = make_uint4(0, 0, 0, 0);
+  int prep_kvh = -1;
   for (int u = wg; u < nt * SL_ATT_KV; u += G) {
     const int tile = u >> 1, kvh = u & 1;
     const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
@@ -390,7 +394,8 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
     }
     // waves 0..7: query heads of the group; wave 8: new key; wave 9: new value -- 4 tagged words per lane
     const int src = wave < 8 ? (kvh * 8 + wave) * 512 : (wave == 8 ? 8192 + kvh * 256 : 8192 + 512 + kvh * 256);
-    uint4 w4 = make_uint4(0, 0, 0, 0);
+    if (kvh != prep_kvh) {
+    prep_kvh = kvh;
     {
       const rsrc_t rp = co_rsrc(uni(F.tproj));
       unsigned spins = 0;
@@ -433,14 +438,20 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) dst[4 * lane + i] = isq ? 0.0625f * o[i] : o[i];
-      if (!isq && has_new) {
+    }
+    }
+    if (has_new) {                      // the unit whose tile holds the new position: its key and value row
+      if (wave == 8) {
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = L.knew[4 * lane + i];
         st_co_h4(co_rsrc(uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 4 * lane, o);
         *reinterpret_cast<uint2*>(&L.kt[(pos - j0) * KT_STRIDE + 4 * lane]) = make_uint2(pack2(o[0], o[1]), pack2(o[2], o[3]));
+      } else if (wave == 9) {
+        const uint32_t a = (w4.x & 0xffffu) | (w4.y << 16), b = (w4.z & 0xffffu) | (w4.w << 16);
+        stw2(co_rsrc(uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 2 * lane, a, b);
+        *reinterpret_cast<uint2*>(&g_vt[(pos - j0) * 256 + 4 * lane]) = make_uint2(a, b);
       }
-    } else if (wave == 9 && has_new) {
-      const uint32_t a = (w4.x & 0xffffu) | (w4.y << 16), b = (w4.z & 0xffffu) | (w4.w << 16);
-      stw2(co_rsrc(uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 2 * lane, a, b);
-      *reinterpret_cast<uint2*>(&g_vt[(pos - j0) * 256 + 4 * lane]) = make_uint2(a, b);
     }
     __syncthreads();
     {
