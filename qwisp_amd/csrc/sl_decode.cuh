@@ -122,8 +122,10 @@ struct Lds {
   StampState bar;
 };
 __shared__ Lds g_L;
-extern __shared__ __align__(16) uint16_t g_vt[];   // dynamic: staged value tile [64][256] halves
-constexpr int DEC_DYN_LDS = SDPA_TILE * 256 * 2;
+extern __shared__ __align__(16) uint16_t g_vt[];   // dynamic: staged value tile [64][256] halves, then the softmax
+                                                   // weights of up to SDPA_ROUND (tile, kv head) units [8 heads][64 keys]
+constexpr int SDPA_ROUND = 20;
+constexpr int DEC_DYN_LDS = SDPA_TILE * 256 * 2 + SDPA_ROUND * 8 * 64 * 4;
 
 SL_DEV void lds_put_x(int b, int lane, const float* x) {
 #pragma unroll

@@ -8,6 +8,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -256,6 +257,7 @@ void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   launch_qmm4_mfma(QmmArgs{e->sh_act, SL_MOE_I, L.sh_down.w, L.sh_down.sb, M, H, SL_MOE_I, e->hy_sy, H}, e->stream);
   hipLaunchKernelGGL(k_moe_combine_rows, dim3(H / 256, M), dim3(256), 0, e->stream, e->hy_d, L.route_scores, e->sgate, e->hy_sy, e->moe_out);
 }
+constexpr int MOE_GROUP_MIN_ROWS = 128;   // below, most experts are chosen by one row and the extra launches cost more
 void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   MoeAArgs a{};
   a.ha = ha;
@@ -272,7 +274,13 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   MoeBArgs b{};
   b.xn = e->xn; b.g_w = L.sw_gate.w; b.g_sb = L.sw_gate.sb; b.u_w = L.sw_up.w; b.u_sb = L.sw_up.sb;
   b.act = e->act; b.inds = L.route_inds;
-  hipLaunchKernelGGL(k_moe_b, dim3(256, M), dim3(256), 0, e->stream, b);
+  if (M >= MOE_GROUP_MIN_ROWS && M <= GROUP_CAP) {      // weights of an expert fetched once for all rows that chose it
+    hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, e->n_experts, e->hy_lists, e->hy_counts);
+    MoeBGroupArgs g{e->xn, b.g_w, b.g_sb, b.u_w, b.u_sb, e->act, e->hy_lists, e->hy_counts};
+    hipLaunchKernelGGL(k_moe_b_grouped, dim3(64, e->n_experts), dim3(256), 0, e->stream, g);
+  } else {
+    hipLaunchKernelGGL(k_moe_b, dim3(256, M), dim3(256), 0, e->stream, b);
+  }
   MoeCArgs c{};
   c.act = e->act; c.sh_act = e->sh_act; c.inds = L.route_inds; c.scores = L.route_scores; c.sgate = e->sgate;
   c.d_w = L.sw_down.w; c.d_sb = L.sw_down.sb; c.shd_w = L.sh_down.w; c.shd_sb = L.sh_down.sb; c.out = e->moe_out;
@@ -613,6 +621,8 @@ int alloc_runtime(sl_engine* e) {
   e->mix = dalloc<uint16_t>(e, MH, true); e->xn = dalloc<uint16_t>(e, MH, true);
   e->rlogits = dalloc<uint16_t>(e, (size_t)max_m * 256, true); e->sgate = dalloc<uint16_t>(e, max_m, true);
   e->sh_act = dalloc<uint16_t>(e, (size_t)max_m * 512, true); e->act = dalloc<uint16_t>(e, (size_t)max_m * 8 * 512, true);
+  e->hy_lists = dalloc<uint16_t>(e, (size_t)SL_MAX_EXPERTS * GROUP_CAP, true);
+  e->hy_counts = dalloc<int32_t>(e, SL_MAX_EXPERTS, true);
   e->moe_out = dalloc<uint16_t>(e, MH, true); e->normed = dalloc<uint16_t>(e, MH, true);
   e->rows_out = dalloc<uint16_t>(e, MH, true);
   e->gdn_qn = dalloc<uint16_t>(e, MH, true); e->gdn_kn = dalloc<uint16_t>(e, MH, true);
@@ -621,7 +631,7 @@ int alloc_runtime(sl_engine* e) {
   e->tok_in = dalloc<int32_t>(e, max_m, true);
   e->tok_out = dalloc<int32_t>(e, max_m > MAX_CHAIN ? max_m : MAX_CHAIN, true);
   e->st = dalloc<int32_t>(e, 1 + d->n_layers, true);
-  if (!e->hA || !e->hB || !e->proj || !e->ycore || !e->mix || !e->xn || !e->rlogits || !e->sgate || !e->sh_act || !e->act ||
+  if (!e->hA || !e->hB || !e->proj || !e->ycore || !e->mix || !e->xn || !e->rlogits || !e->sgate || !e->sh_act || !e->act || !e->hy_lists || !e->hy_counts ||
       !e->moe_out || !e->normed || !e->rows_out || !e->tok_in || !e->tok_out || !e->st) return SL_ERR_DEVICE;
   if (has_head) {
     int ncu = 0;
@@ -670,6 +680,11 @@ int alloc_runtime(sl_engine* e) {
         F.tpo = dalloc<uint4>(e, (size_t)SL_ATT_HEADS * e->max_tiles * 128, true);
         F.tcand = dalloc<uint4>(e, 256, true);
         F.ttok = dalloc<uint4>(e, 4, true);
+        F.sdpa_round = SDPA_ROUND;
+        if (const char* s = std::getenv("QWISP_SDPA_ROUND")) {      // smaller rounds, for tests of the round loop
+          const int v = std::atoi(s);
+          if (v >= 1 && v <= SDPA_ROUND) F.sdpa_round = v;
+        }
         if (!F.tproj || !F.tycore || !F.tmix || !F.trlog || !F.tsg || !F.tsh || !F.tact || !F.tmoe ||
             !F.tml || !F.tpo || !F.tcand || !F.ttok) return SL_ERR_DEVICE;
         e->flow_host = F;
@@ -831,9 +846,7 @@ int sl_set_hybrid(sl_engine* e, int enable) {
     e->hy_d = dalloc<uint16_t>(e, rows * 8 * H);
     e->hy_sg = dalloc<uint16_t>(e, rows * SL_MOE_I); e->hy_su = dalloc<uint16_t>(e, rows * SL_MOE_I);
     e->hy_sy = dalloc<uint16_t>(e, rows * H);
-    e->hy_lists = dalloc<uint16_t>(e, (size_t)SL_MAX_EXPERTS * GROUP_CAP, true);
-    e->hy_counts = dalloc<int32_t>(e, SL_MAX_EXPERTS, true);
-    if (!e->hy_d || !e->hy_sg || !e->hy_su || !e->hy_sy || !e->hy_lists || !e->hy_counts) return SL_ERR_DEVICE;
+    if (!e->hy_d || !e->hy_sg || !e->hy_su || !e->hy_sy) return SL_ERR_DEVICE;
     SL_TRY(e, hipStreamSynchronize(e->stream));
   }
   e->hybrid = enable != 0;

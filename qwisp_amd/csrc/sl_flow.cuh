@@ -33,6 +33,7 @@ struct FlowP {
   uint4 *tpo;           // attention {o[2c], o[2c+1], tag, tag}  [16][max_tiles][128]
   uint4 *tcand;         // {value, index, tag, tag}        [256]
   uint4 *ttok;          // {token, token, tag, tag}: the token a step of a multi-step launch hands to the next [1]
+  int sdpa_round;       // long contexts: (tile, kv head) units a workgroup scores before it turns to their values
 };
 
 // Parameters live in LDS for the whole launch.  Reading them there (ds_read + readfirstlane) does not
@@ -366,6 +367,14 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
 }
 
 // ---- attention stage 2: q/k prep, KV append, tile pass ---------------------------------------------------
+// A unit is (key tile of 64 positions, kv head); the workgroups take their units in two passes: scores, softmax
+// weights (kept in LDS) and the published {max, sum} of every unit first, then the weighted value sums in the same
+// order.  With several units per workgroup (contexts beyond about 7000 tokens) the merge knows the global maximum
+// after the first pass and adds the tiles up while the second pass runs.
+#ifndef SL_MERGE_WGS
+#define SL_MERGE_WGS 32
+#endif
+constexpr int FLOW_MERGE_WGS = SL_MERGE_WGS;     // workgroups that merge the attention tiles: two or four per query head
 SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base) {
   FLOW_IDS;
   const DecodeP& P = F.d;
@@ -373,131 +382,167 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
   const float NEG = -__int_as_float(0x7f800000);
   const int N = pos + 1, nt = (N + SDPA_TILE - 1) / SDPA_TILE;
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag32(base, li, FS_CORE);
+  // The workgroups that merge the tiles take no units: they start polling at once, see every tile's maximum after
+  // the first pass below and add up the tiles' value sums while the second pass is still producing them.
+  const int GU = G > 2 * FLOW_MERGE_WGS ? G - FLOW_MERGE_WGS : G;
+  if (wg >= GU) return true;
+  const int U = nt * SL_ATT_KV, RND = uni(F.sdpa_round);
+  float* const ps = reinterpret_cast<float*>(g_vt + SDPA_TILE * 256);      // [SDPA_ROUND][8 heads][64 keys]
+  uint32_t* const vn = reinterpret_cast<uint32_t*>(L.vnew);                // [kv head][128 words]: the new value row
   // The queries of the kv head's group and the new key and value row are the same for every unit of a workgroup
-  // (with an even grid a workgroup stays with one kv head): polled, normed and rotated for its first unit only.
+  // (with an even count of unit workgroups a workgroup stays with one kv head): polled, normed and rotated for its
+  // first unit only.
   uint4 w4 = make_uint4(0, 0, 0, 0);
   int prep_kvh = -1;
-  for (int u = wg; u < nt * SL_ATT_KV; u += G) {
-    const int tile = u >> 1, kvh = u & 1;
-    const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
-    const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
-    const uint16_t* kbase = uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + j0) * 256;
-    const uint16_t* vbase = uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + j0) * 256;
-    __syncthreads();                    // the key tile aliases the activation vector the in-projection just read
+  // A thread stages two 16-byte pieces of a unit's key and value tiles: rows srow and srow + 32 (the row of the new
+  // position comes from this step's projection instead).
+  const int srow = tid >> 5, c8 = (tid & 31) * 8;
+  auto stage = [&](bool keys, bool values, int u) {
+    const int j0 = (u >> 1) * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
+    const size_t off = ((size_t)(u & 1) * uni(P.max_seq) + j0) * 256 + c8;
+    uint4 kq[2], vq[2];
+    bool on[2];
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
-      const int row = it * 32 + (tid >> 5), c8 = (tid & 31) * 8;
-      if (row < nk && j0 + row != pos) {
-        st16(&L.kt[row * KT_STRIDE + c8], ld16(kbase + (size_t)row * 256 + c8));
-        st16(&g_vt[row * 256 + c8], ld16(vbase + (size_t)row * 256 + c8));
-      }
+      const int row = it * 32 + srow;
+      on[it] = row < nk && j0 + row != pos;
+      if (on[it] && keys) kq[it] = ld16(uni(Y.kcache) + off + (size_t)row * 256);
+      if (on[it] && values) vq[it] = ld16(uni(Y.vcache) + off + (size_t)row * 256);
     }
-    // waves 0..7: query heads of the group; wave 8: new key; wave 9: new value -- 4 tagged words per lane
-    const int src = wave < 8 ? (kvh * 8 + wave) * 512 : (wave == 8 ? 8192 + kvh * 256 : 8192 + 512 + kvh * 256);
-    if (kvh != prep_kvh) {
-    prep_kvh = kvh;
-    {
-      const rsrc_t rp = co_rsrc(uni(F.tproj));
-      unsigned spins = 0;
-    fstamp(P, 4, 0);
-      for (;;) {
-        bool ok = true;
-        if (wave < 10) { w4 = ldw4(rp, src + 4 * lane); ok = tag_ok(w4.x, tin) && tag_ok(w4.y, tin) && tag_ok(w4.z, tin) && tag_ok(w4.w, tin); }
-        const int v = flow_round(ok, spins, uni(P.bar) + 32);
-        if (v > 0) break;
-        if (v < 0) return false;
-      }
-      fstamp(P, 5, spins);
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int row = it * 32 + srow;
+      if (on[it] && keys) st16(&L.kt[row * KT_STRIDE + c8], kq[it]);
+      if (on[it] && values) st16(&g_vt[row * 256 + c8], vq[it]);
     }
-      if (wave < 9) {
-      const bool isq = wave < 8;
-      const uint16_t* nwp = isq ? uni(Y.q_norm) : uni(Y.k_norm);
-      const float xv[4] = {lo_h(w4.x), lo_h(w4.y), lo_h(w4.z), lo_h(w4.w)};
-      float wv[4];
-      const uint2 wraw = *reinterpret_cast<const uint2*>(nwp + 4 * lane);
-      wv[0] = lo_h(wraw.x); wv[1] = hi_h(wraw.x); wv[2] = lo_h(wraw.y); wv[3] = hi_h(wraw.y);
-      float ss = 0.0f;
+  };
+  for (int ub = wg; ub < U; ub += GU * RND) {
+    const int nr = min(RND, (U - ub + GU - 1) / GU);       // units of this round
+    // pass 1, keys: scores and softmax weights of every unit of the round; maxima and sums published per tile.
+    // The value tile of the round's first unit is staged here as well (its space is free during this pass).
+    for (int r = 0; r < nr; ++r) {
+      const int u = ub + r * GU;
+      const int tile = u >> 1, kvh = u & 1;
+      const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
+      const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
+      __syncthreads();                    // the key tile aliases the activation vector the in-projection just read
+      stage(true, r == 0, u);
+      // waves 0..7: query heads of the group; wave 8: new key; wave 9: new value -- 4 tagged words per lane
+      const int src = wave < 8 ? (kvh * 8 + wave) * 512 : (wave == 8 ? 8192 + kvh * 256 : 8192 + 512 + kvh * 256);
+      if (kvh != prep_kvh) {
+        prep_kvh = kvh;
+        {
+          const rsrc_t rp = co_rsrc(uni(F.tproj));
+          unsigned spins = 0;
+          fstamp(P, 4, 0);
+          for (;;) {
+            bool ok = true;
+            if (wave < 10) { w4 = ldw4(rp, src + 4 * lane); ok = tag_ok(w4.x, tin) && tag_ok(w4.y, tin) && tag_ok(w4.z, tin) && tag_ok(w4.w, tin); }
+            const int v = flow_round(ok, spins, uni(P.bar) + 32);
+            if (v > 0) break;
+            if (v < 0) return false;
+          }
+          fstamp(P, 5, spins);
+        }
+        if (wave < 9) {
+          const bool isq = wave < 8;
+          const uint16_t* nwp = isq ? uni(Y.q_norm) : uni(Y.k_norm);
+          const float xv[4] = {lo_h(w4.x), lo_h(w4.y), lo_h(w4.z), lo_h(w4.w)};
+          float wv[4];
+          const uint2 wraw = *reinterpret_cast<const uint2*>(nwp + 4 * lane);
+          wv[0] = lo_h(wraw.x); wv[1] = hi_h(wraw.x); wv[2] = lo_h(wraw.y); wv[3] = hi_h(wraw.y);
+          float ss = 0.0f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) ss = fmaf(xv[i], xv[i], ss);
-      ss = tree_sum<64>(ss);
-      const float inv = 1.0f / sqrtf(ss / 256.0f + EPS);
-      float* dst = isq ? &L.sq[wave * 256] : L.knew;
+          for (int i = 0; i < 4; ++i) ss = fmaf(xv[i], xv[i], ss);
+          ss = tree_sum<64>(ss);
+          const float inv = 1.0f / sqrtf(ss / 256.0f + EPS);
+          float* dst = isq ? &L.sq[wave * 256] : L.knew;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dst[4 * lane + i] = f16r(wv[i] * f16r(xv[i] * inv));
-      float o[4];
+          for (int i = 0; i < 4; ++i) dst[4 * lane + i] = f16r(wv[i] * f16r(xv[i] * inv));
+          float o[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] = dst[4 * lane + i];
-      if (lane < 16) {
+          for (int i = 0; i < 4; ++i) o[i] = dst[4 * lane + i];
+          if (lane < 16) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int d = 4 * lane + i, ii = d & 31;
-          const float c = uni(P.rope_cos)[(size_t)pos * 32 + ii], sn = uni(P.rope_sin)[(size_t)pos * 32 + ii];
-          const float x0 = dst[ii], x1 = dst[ii + 32];
-          o[i] = (d < 32) ? f16r(fmaf(-x1, sn, x0 * c)) : f16r(fmaf(x1, c, x0 * sn));
+            for (int i = 0; i < 4; ++i) {
+              const int d = 4 * lane + i, ii = d & 31;
+              const float c = uni(P.rope_cos)[(size_t)pos * 32 + ii], sn = uni(P.rope_sin)[(size_t)pos * 32 + ii];
+              const float x0 = dst[ii], x1 = dst[ii + 32];
+              o[i] = (d < 32) ? f16r(fmaf(-x1, sn, x0 * c)) : f16r(fmaf(x1, c, x0 * sn));
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dst[4 * lane + i] = isq ? 0.0625f * o[i] : o[i];
+        } else if (wave == 9) {             // the new value row waits in LDS for the second pass
+          vn[kvh * 128 + 2 * lane] = (w4.x & 0xffffu) | (w4.y << 16);
+          vn[kvh * 128 + 2 * lane + 1] = (w4.z & 0xffffu) | (w4.w << 16);
         }
       }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) dst[4 * lane + i] = isq ? 0.0625f * o[i] : o[i];
-    }
-    }
-    if (has_new) {                      // the unit whose tile holds the new position: its key and value row
-      if (wave == 8) {
+      if (has_new && wave == 8) {         // the unit whose tile holds the new position: its key row
         float o[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[i] = L.knew[4 * lane + i];
         st_co_h4(co_rsrc(uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 4 * lane, o);
         *reinterpret_cast<uint2*>(&L.kt[(pos - j0) * KT_STRIDE + 4 * lane]) = make_uint2(pack2(o[0], o[1]), pack2(o[2], o[3]));
-      } else if (wave == 9) {
-        const uint32_t a = (w4.x & 0xffffu) | (w4.y << 16), b = (w4.z & 0xffffu) | (w4.w << 16);
+      }
+      __syncthreads();
+      {
+        // scores: wave (head, half) takes the 32 leaves of its half of the 256 dims, lane j is key j.  The 128
+        // query values sit two per lane and reach the multiply as scalar operands (readlane), so LDS only
+        // serves the key rows.
+        const int h = wave >> 1, half = wave & 1;
+        const uint16_t* kr = &L.kt[(lane < nk ? lane : 0) * KT_STRIDE + 128 * half];
+        const float qa = L.sq[h * 256 + 128 * half + lane], qb = L.sq[h * 256 + 128 * half + 64 + lane];
+        float g[4];
+#pragma unroll
+        for (int gi = 0; gi < 4; ++gi) {
+          float n[8];
+#pragma unroll
+          for (int l = 0; l < 8; ++l) {
+            const int d = 32 * gi + 4 * l;                 // first dim of the leaf within the half
+            const float qv = d < 64 ? qa : qb;
+            const uint2 kraw = *reinterpret_cast<const uint2*>(kr + d);
+            const h2_t k01 = as_h2(kraw.x), k23 = as_h2(kraw.y);      // half operands go straight into the FMA
+            float node = fmaf(row_lane_f(qv, (d & 63)), (float)k01.x, 0.0f);
+            node = fmaf(row_lane_f(qv, (d & 63) + 1), (float)k01.y, node);
+            node = fmaf(row_lane_f(qv, (d & 63) + 2), (float)k23.x, node);
+            n[l] = fmaf(row_lane_f(qv, (d & 63) + 3), (float)k23.y, node);
+          }
+          g[gi] = ((n[0] + n[1]) + (n[2] + n[3])) + ((n[4] + n[5]) + (n[6] + n[7]));
+        }
+        L.part[wave * 64 + lane] = (g[0] + g[1]) + (g[2] + g[3]);
+      }
+      __syncthreads();
+      if ((wave & 1) == 0) {
+        const int h = wave >> 1;
+        const float dotv = L.part[wave * 64 + lane] + L.part[(wave + 1) * 64 + lane];
+        const float sc = (lane < nk) ? dotv : NEG;
+        const float mx = tree_max<64>(sc);
+        const float p = (lane < nk) ? exp_c(sc - mx) : 0.0f;
+        const float l = tree_sum<64>(p);
+        ps[(r * 8 + h) * 64 + lane] = p;
+        const int head = kvh * 8 + h;
+        if (lane == 0) stw4(co_rsrc(uni(F.tml)), (head * uni(P.max_tiles) + tile) * 4, __float_as_uint(mx), __float_as_uint(l), tcore, tcore);
+      }
+    }
+    // pass 2, values: the weighted value sums of the same units, in the same order
+    for (int r = 0; r < nr; ++r) {
+      const int u = ub + r * GU;
+      const int tile = u >> 1, kvh = u & 1;
+      const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
+      const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
+      __syncthreads();                    // the previous unit's value tile has been read; the weights are in place
+      if (r > 0) stage(false, true, u);
+      if (has_new && wave == 9) {
+        const uint32_t a = vn[kvh * 128 + 2 * lane], b = vn[kvh * 128 + 2 * lane + 1];
         stw2(co_rsrc(uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 2 * lane, a, b);
         *reinterpret_cast<uint2*>(&g_vt[(pos - j0) * 256 + 4 * lane]) = make_uint2(a, b);
       }
-    }
-    __syncthreads();
-    {
-      // scores: wave (head, half) takes the 32 leaves of its half of the 256 dims, lane j is key j.  The 128
-      // query values sit two per lane and reach the multiply as scalar operands (readlane), so LDS only
-      // serves the key rows.
-      const int h = wave >> 1, half = wave & 1;
-      const uint16_t* kr = &L.kt[(lane < nk ? lane : 0) * KT_STRIDE + 128 * half];
-      const float qa = L.sq[h * 256 + 128 * half + lane], qb = L.sq[h * 256 + 128 * half + 64 + lane];
-      float g[4];
-#pragma unroll
-      for (int gi = 0; gi < 4; ++gi) {
-        float n[8];
-#pragma unroll
-        for (int l = 0; l < 8; ++l) {
-          const int d = 32 * gi + 4 * l;                 // first dim of the leaf within the half
-          const float qv = d < 64 ? qa : qb;
-          const uint2 kraw = *reinterpret_cast<const uint2*>(kr + d);
-          const h2_t k01 = as_h2(kraw.x), k23 = as_h2(kraw.y);      // half operands go straight into the FMA
-          float node = fmaf(row_lane_f(qv, (d & 63)), (float)k01.x, 0.0f);
-          node = fmaf(row_lane_f(qv, (d & 63) + 1), (float)k01.y, node);
-          node = fmaf(row_lane_f(qv, (d & 63) + 2), (float)k23.x, node);
-          n[l] = fmaf(row_lane_f(qv, (d & 63) + 3), (float)k23.y, node);
-        }
-        g[gi] = ((n[0] + n[1]) + (n[2] + n[3])) + ((n[4] + n[5]) + (n[6] + n[7]));
-      }
-      L.part[wave * 64 + lane] = (g[0] + g[1]) + (g[2] + g[3]);
-    }
-    __syncthreads();
-    if ((wave & 1) == 0) {
-      const int h = wave >> 1;
-      const float dotv = L.part[wave * 64 + lane] + L.part[(wave + 1) * 64 + lane];
-      const float sc = (lane < nk) ? dotv : NEG;
-      const float mx = tree_max<64>(sc);
-      const float p = (lane < nk) ? exp_c(sc - mx) : 0.0f;
-      const float l = tree_sum<64>(p);
-      L.sm[h * 64 + lane] = p;
-      const int head = kvh * 8 + h;
-      if (lane == 0) stw4(co_rsrc(uni(F.tml)), (head * uni(P.max_tiles) + tile) * 4, __float_as_uint(mx), __float_as_uint(l), tcore, tcore);
-    }
-    __syncthreads();
-    {
+      __syncthreads();
       const int h = wave >> 1, half = wave & 1;
       float o0 = 0.0f, o1 = 0.0f;
       const uint16_t* vt = &g_vt[128 * half + 2 * lane];
-      const float pmine = L.sm[h * 64 + lane];            // weight of key `lane`; handed out by readlane below
+      const float pmine = ps[(r * 8 + h) * 64 + lane];     // weight of key `lane`; handed out by readlane below
       int j = 0;
       for (; j + 8 <= nk; j += 8) {            // the eight LDS reads are issued together, then used in key order
         uint32_t v8[8];
@@ -704,7 +749,6 @@ SL_DEV void store_hist(const LayerP& Y, int li, const GdnHist& gh) {
 }
 
 // ---- K = 4096 projection (GDN out_proj with gated rmsnorm prologue / attention merge + o_proj) ---------
-constexpr int FLOW_MERGE_WGS = 32;     // two per query head
 SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t base, const GdnHist& gh) {
   FLOW_IDS;
   const DecodeP& P = F.d;
@@ -717,15 +761,18 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
   if (!lin && wg >= G - FLOW_MERGE_WGS) {
     // Merge the attention tiles in order with the global max: the last 32 workgroups take half a head each (they own
-    // a tile unit only at contexts of several thousand tokens, so their waves normally have no stores of their own
-    // to wait for).  Wave 0 is the merging wave: a lane owns one 16-byte chunk (2 dims) of its 128 dims.
+    // no tile units, so their waves have no stores of their own to wait for and poll from the start of the
+    // stage).  Wave 0 is the merging wave: a lane owns one 16-byte chunk (2 dims) of its 128 dims.
     // First round trip: {max, sum} of the first 64 tiles (lane i fetches tile i), the partials of the first MB tiles
     // and the output gate (it sits in the q projection of this step) are polled together, each piece until it has
     // arrived; at contexts of up to MB tiles that is everything the merge needs.  Beyond that a round trip per MB
     // tiles would dominate (about 3 us each, whatever its size), so all 16 waves fetch: per block of 64 tiles wave w
     // polls tiles 4w .. 4w+3 and parks their values in LDS (the value tile's space), and wave 0 then adds the block
-    // up from LDS.  The accumulation always runs in tile order.
-    const int mi = wg - (G - FLOW_MERGE_WGS), h = mi >> 1, slot0 = h * uni(P.max_tiles), chunk = 64 * (mi & 1) + lane;
+    // up from LDS (its {max, sum} words fetched during the poll).  The accumulation always runs in tile order.
+    constexpr int MPH = FLOW_MERGE_WGS / SL_ATT_HEADS, LPW = 128 / MPH;      // workgroups per head, chunks (lanes) per workgroup
+    const int mi = wg - (G - FLOW_MERGE_WGS), h = mi / MPH, slot0 = h * uni(P.max_tiles);
+    const bool act = lane < LPW;
+    const int chunk = LPW * (mi % MPH) + (act ? lane : 0);      // (idle lanes of a narrower workgroup fetch and store nothing)
     const rsrc_t rml = co_rsrc(uni(F.tml)), rpo = co_rsrc(uni(F.tpo)), rp = co_rsrc(uni(F.tproj));
     constexpr int MB = 12;
     int fail = 0;
@@ -746,14 +793,14 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
             mdone = __all(ok ? 1 : 0) != 0;
           }
           if (!gdone) {
-            g2 = ldw2(rp, h * 512 + 256 + 2 * chunk);
-            gdone = __all((tag_ok(g2.x, tin) && tag_ok(g2.y, tin)) ? 1 : 0) != 0;
+            if (act) g2 = ldw2(rp, h * 512 + 256 + 2 * chunk);
+            gdone = __all((!act || (tag_ok(g2.x, tin) && tag_ok(g2.y, tin))) ? 1 : 0) != 0;
           }
 #pragma unroll
           for (int u = 0; u < MB; ++u) {
             if (u < cnt0 && !(have & (1u << u))) {
-              a[u] = ldw4(rpo, ((slot0 + u) * 128 + chunk) * 4);
-              if (__all((a[u].z == tcore32 && a[u].w == tcore32) ? 1 : 0)) have |= 1u << u;
+              if (act) a[u] = ldw4(rpo, ((slot0 + u) * 128 + chunk) * 4);
+              if (__all((!act || (a[u].z == tcore32 && a[u].w == tcore32)) ? 1 : 0)) have |= 1u << u;
             }
           }
           if (mdone && gdone && have == (1u << cnt0) - 1u) break;
@@ -789,16 +836,19 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     }
     if (nt > MB) {                                          // uniform for the grid
       uint2* park = reinterpret_cast<uint2*>(g_vt);         // [64 tiles][64 lanes] {o0, o1}
-      __syncthreads();                                      // this workgroup's own tile units are done with the value tile
+      __syncthreads();                                      // tile units this workgroup may have had are done with the space
       for (int t0 = 0; t0 < nt; t0 += 64) {
         uint4 q[4];
+        // wave 0, lane i: {max, sum} of tile t0 + i (its tags were verified above), fetched in the shadow of the poll
+        uint4 ma = m0;
+        if (wave == 0 && t0 > 0 && t0 + lane < nt) ma = ldw4(rml, (slot0 + t0 + lane) * 4);
         unsigned spins = 0;
         for (;;) {
           bool ok = true;
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const int t = t0 + 4 * wave + j;
-            if (t >= MB && t < nt) { q[j] = ldw4(rpo, ((slot0 + t) * 128 + chunk) * 4); ok = ok && q[j].z == tcore32 && q[j].w == tcore32; }
+            if (t >= MB && t < nt && act) { q[j] = ldw4(rpo, ((slot0 + t) * 128 + chunk) * 4); ok = ok && q[j].z == tcore32 && q[j].w == tcore32; }
           }
           if (__all(ok ? 1 : 0)) break;
           if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
@@ -807,15 +857,12 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int t = t0 + 4 * wave + j;
-          if (t >= MB && t < nt) park[(4 * wave + j) * 64 + lane] = make_uint2(q[j].x, q[j].y);
+          if (t >= MB && t < nt && act) park[(4 * wave + j) * 64 + lane] = make_uint2(q[j].x, q[j].y);
         }
         __syncthreads();
         if (wave == 0 && !fail) {
-          float fl = 0.0f, pl = 0.0f;                       // lane i: scale and sum of tile t0+i (tags verified above)
-          if (t0 + lane < nt) {
-            const uint4 m = t0 == 0 ? m0 : ldw4(rml, (slot0 + t0 + lane) * 4);
-            fl = exp_c(__uint_as_float(m.x) - Mx); pl = __uint_as_float(m.y);
-          }
+          float fl = 0.0f, pl = 0.0f;                       // lane i: scale and sum of tile t0+i
+          if (t0 + lane < nt) { fl = exp_c(__uint_as_float(ma.x) - Mx); pl = __uint_as_float(ma.y); }
           const int lo = t0 == 0 ? MB : 0, hi = min(64, nt - t0);
           for (int u0 = lo; u0 < hi; u0 += 8) {             // eight LDS reads and sixteen lane reads at a time, used in tile order
             uint2 v[8];
@@ -837,7 +884,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
       }
     }
     if (fail) st_co32(uni(P.bar) + 32, 1u);
-    if (wave == 0 && !fail) {
+    if (wave == 0 && !fail && act) {
       const uint32_t r0 = tagged(f16r(f16r(O0 / Ls) * sigmoid16(lo_h(g2.x))), tmerge);
       const uint32_t r1 = tagged(f16r(f16r(O1 / Ls) * sigmoid16(lo_h(g2.y))), tmerge);
       stw2(co_rsrc(uni(F.tycore)), h * 256 + 2 * chunk, r0, r1);

@@ -790,6 +790,92 @@ struct MoeBArgs {
   uint16_t* act;               // [M, 8, 512]
   const int32_t* inds;         // [M, 8]
 };
+constexpr int GROUP_CAP = 2048;         // pairs per expert: an expert is chosen at most once per row, M <= 2048
+// Pairs (row, slot) listed per expert (M * 8 pairs walked by 1024 threads), places handed out by LDS counters.
+// The order within a list varies from run to run; results do not depend on it (they are scattered back by pair).
+__global__ __launch_bounds__(1024) void k_group_pairs(const int32_t* __restrict__ inds, int M, int E, uint16_t* __restrict__ lists,
+                                                      int32_t* __restrict__ counts) {
+  __shared__ int s_cnt[SL_MAX_EXPERTS];
+  if (threadIdx.x < SL_MAX_EXPERTS) s_cnt[threadIdx.x] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < M * 8; p += 1024) {
+    const int e = inds[p];
+    if (e >= 0 && e < E) {
+      const int pos = atomicAdd(&s_cnt[e], 1);
+      if (pos < GROUP_CAP) lists[e * GROUP_CAP + pos] = (uint16_t)p;
+    }
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < E) counts[threadIdx.x] = s_cnt[threadIdx.x];
+}
+// Stage B by expert (steps of many rows): grid (64, E).  A workgroup holds eight gate/up row pairs of one expert
+// (two pairs per wave, unpacked into masks once) and walks the expert's list of (row, slot) pairs in tiles of
+// MOEB_MT activation rows parked in LDS as in k_qmv_tile, so the expert's weights are fetched and unpacked once
+// per step instead of once per row that chose it.  Same arithmetic per (pair, weight row) as k_moe_b.
+struct MoeBGroupArgs {
+  const uint16_t* xn;          // [M, 2048]
+  const uint32_t *g_w, *g_sb, *u_w, *u_sb;   // [E*512, 2048]
+  uint16_t* act;               // [M, 8, 512]
+  const uint16_t* lists;       // [E, GROUP_CAP] pair indices row*8 + slot
+  const int32_t* counts;       // [E]
+};
+constexpr int MOEB_MT = 8;
+__global__ __launch_bounds__(256, 3) void k_moe_b_grouped(MoeBGroupArgs a) {
+  __shared__ uint4 xs[MOEB_MT * 64 * 5];
+  __shared__ int s_pair[MOEB_MT];
+  const int e = blockIdx.y, cnt = min(a.counts[e], GROUP_CAP);
+  if (cnt == 0) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i0 = (blockIdx.x * 4 + wave) * 2;
+  const size_t base = (size_t)e * 512 + i0;
+  uint4 wv[4];
+  uint32_t sb[4];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    wv[r] = ld16(a.g_w + (base + r) * 256 + 4 * lane); sb[r] = a.g_sb[(base + r) * 32 + (lane >> 1)];
+    wv[2 + r] = ld16(a.u_w + (base + r) * 256 + 4 * lane); sb[2 + r] = a.u_sb[(base + r) * 32 + (lane >> 1)];
+  }
+  h2_t mk[4][16];
+  for (int t0 = 0; t0 < cnt; t0 += MOEB_MT) {
+    const int mc = min(MOEB_MT, cnt - t0);
+    if (t0) __syncthreads();                             // the previous tile has been read
+    for (int j = wave; j < mc; j += 4) {
+      const int p = a.lists[(size_t)e * GROUP_CAP + t0 + j];
+      if (lane == 0) s_pair[j] = p;
+      float x[32], sx[4];
+      load32(a.xn + (size_t)(p >> 3) * H + 32 * lane, x);
+      word_sums(x, sx);
+      uint32_t xp[16];
+      pack_x(x, xp);
+      uint4* dst = xs + (j * 64 + lane) * 5;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) dst[q] = make_uint4(xp[4 * q], xp[4 * q + 1], xp[4 * q + 2], xp[4 * q + 3]);
+      dst[4] = make_uint4(__float_as_uint(sx[0]), __float_as_uint(sx[1]), __float_as_uint(sx[2]), __float_as_uint(sx[3]));
+    }
+    __syncthreads();
+    if (t0 == 0) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        word_masks(wv[r].x, mk[r]); word_masks(wv[r].y, mk[r] + 4);
+        word_masks(wv[r].z, mk[r] + 8); word_masks(wv[r].w, mk[r] + 12);
+      }
+    }
+    for (int j = 0; j < mc; ++j) {
+      const uint4* src = xs + (j * 64 + lane) * 5;
+      uint32_t xp[16];
+      float sx[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) { const uint4 v = src[q]; xp[4 * q] = v.x; xp[4 * q + 1] = v.y; xp[4 * q + 2] = v.z; xp[4 * q + 3] = v.w; }
+      { const uint4 v = src[4]; sx[0] = __uint_as_float(v.x); sx[1] = __uint_as_float(v.y); sx[2] = __uint_as_float(v.z); sx[3] = __uint_as_float(v.w); }
+      float o[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[r] = tree_sum<64>(quad_term_masked(mk[r], sb[r], xp, sx));
+      if (lane == 0)
+        *reinterpret_cast<uint32_t*>(a.act + (size_t)s_pair[j] * 512 + i0) =
+            pack2(swiglu16(f16r(o[0]), f16r(o[2])), swiglu16(f16r(o[1]), f16r(o[3])));
+    }
+  }
+}
 __global__ __launch_bounds__(256) void k_moe_b(MoeBArgs a) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int p0 = (blockIdx.x * 4 + wave) * 4;          // row index in [0, 8*512)

@@ -165,7 +165,6 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
 // SeedlessFusedVerify.swift:4174): the (row, slot) pairs that chose expert e are gathered, multiplied with that
 // expert's matrix once, and scattered back by pair.  Workgroup = (strip block, expert); experts nobody chose exit.
 // -------------------------------------------------------------------------------------------------
-constexpr int GROUP_CAP = 2048;         // pairs per expert: an expert is chosen at most once per row, M <= 2048
 
 struct QmmGroupArgs {
   const uint16_t* x;     // source rows, fp16
@@ -286,23 +285,6 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
   }
 }
 
-// Pairs (row, slot) listed per expert (M * 8 <= 4096 pairs over 1024 threads), places handed out by LDS counters.
-// The order within a list varies from run to run; results do not depend on it (they are scattered back by pair).
-__global__ __launch_bounds__(1024) void k_group_pairs(const int32_t* __restrict__ inds, int M, int E, uint16_t* __restrict__ lists,
-                                                      int32_t* __restrict__ counts) {
-  __shared__ int s_cnt[SL_MAX_EXPERTS];
-  if (threadIdx.x < SL_MAX_EXPERTS) s_cnt[threadIdx.x] = 0;
-  __syncthreads();
-  for (int p = threadIdx.x; p < M * 8; p += 1024) {
-    const int e = inds[p];
-    if (e >= 0 && e < E) {
-      const int pos = atomicAdd(&s_cnt[e], 1);
-      if (pos < GROUP_CAP) lists[e * GROUP_CAP + pos] = (uint16_t)p;
-    }
-  }
-  __syncthreads();
-  if ((int)threadIdx.x < E) counts[threadIdx.x] = s_cnt[threadIdx.x];
-}
 // act = half(silu(g) * u) in half arithmetic, elementwise over [rows, 512] (same rule as the GEMV kernels).
 __global__ __launch_bounds__(256) void k_swiglu_rows(const uint16_t* __restrict__ g, const uint16_t* __restrict__ u,
                                                      uint16_t* __restrict__ act, int total) {

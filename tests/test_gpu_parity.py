@@ -237,6 +237,7 @@ def test_hybrid_prefill_agrees_with_the_exact_rows(env, small_model):
     assert same_bits(d1[:48], b)
     ex2 = env["Engine"](cfg, dev, max_m=768, max_seq_len=800)
     d0 = ex2.forward_tokens(toks2)
+    assert same_bits(d0[:48], a)       # exact rows: the expert-grouped gate/up stage of large chunks changes no bit
     rel2 = np.linalg.norm(d0.astype(np.float64) - d1.astype(np.float64), axis=1) / np.linalg.norm(d0.astype(np.float64), axis=1)
     assert np.median(rel2) < 0.02 and rel2.max() < 0.15, (np.median(rel2), rel2.max())
     big.close(); ex2.close()
@@ -535,12 +536,18 @@ def test_persistent_step_long_context(env, small_model):
             assert same_bits(x, y), (li, first_diff(x, y))
 
 
-def test_persistent_step_with_several_tile_units_per_workgroup(env, small_model):
-    """Beyond 8192 tokens of context there are more (key tile, kv head) units than workgroups: some workgroups take
-    two units in turn, the merge runs over three blocks of 64 tiles.  Same tokens, logits and caches as the
-    kernel-per-stage sequence."""
+@pytest.mark.parametrize("round_units", [None, 1])
+def test_persistent_step_with_several_tile_units_per_workgroup(env, small_model, monkeypatch, round_units):
+    """Beyond 7168 tokens of context there are more (key tile, kv head) units than the workgroups that take them
+    (all but the 32 that merge): some take two units in turn, first the keys of both, then the values; the merge
+    runs over two blocks of 128 tiles.  Same tokens, logits and caches as the kernel-per-stage sequence.  With a
+    round of one unit (QWISP_SDPA_ROUND, read when the engine is created) the same step runs several rounds of the
+    two passes, as contexts beyond 140k tokens do with the default round of 20."""
     cfg, dev, host = small_model
+    if round_units is not None:
+        monkeypatch.setenv("QWISP_SDPA_ROUND", str(round_units))
     a = env["Engine"](cfg, dev, max_m=256, max_seq_len=8704)
+    monkeypatch.delenv("QWISP_SDPA_ROUND", raising=False)
     b = env["Engine"](cfg, dev, max_m=256, max_seq_len=8704)
     assert b.set_persistent(False)
     toks = np.random.default_rng(79).integers(0, cfg.vocab, 8500).astype(np.int32)
