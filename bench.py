@@ -57,6 +57,9 @@ def main():
     ap.add_argument("--cpu-tokens", type=int, default=256, help="decode tokens timed on the CPU oracle (0 = skip)")
     ap.add_argument("--lanes", type=int, default=32, metavar="B",
                     help="also time B lanes stepped as one batch of rows on the same weights (extra object in the JSON line; 0 = skip)")
+    ap.add_argument("--lane-contexts", choices=("mixed", "short"), default="mixed",
+                    help="contexts of the --lanes sequences: mixed = 1K to 16K tokens spread evenly over the lanes (prefilled "
+                         "on the matrix cores first), short = 8 to 56 tokens")
     ap.add_argument("--prefill-chunk", type=int, default=1024, metavar="M",
                     help="also time a prefill in chunks of M rows, exact rows and hybrid (matrix cores), on lanes "
                          "of the same weights (extra object in the JSON line; 0 = skip)")
@@ -145,16 +148,30 @@ def main():
     lanes_report = None
     if args.lanes > 1:
         B = args.lanes
-        lanes = [eng.new_lane(max_m=B, max_seq_len=256) for _ in range(B)]
+        # the batched configuration of the reference: concurrent sequences at mixed contexts of 1K to 16K tokens
+        # (spread evenly over the lanes; --lane-contexts short keeps them at 8-56 tokens for quick runs)
+        mixed = args.lane_contexts == "mixed"
+        ctxs = [1024 + (15 * 1024 * i) // max(B - 1, 1) for i in range(B)] if mixed else [8 + (i * 5) % 40 for i in range(B)]
+        lane_m = max(B, 256) if mixed else B
+        lanes = [eng.new_lane(max_m=lane_m, max_seq_len=(max(ctxs) + 64 if mixed else 256)) for _ in range(B)]
         rng = np.random.default_rng(4000)
         toks = []
-        for i, lane in enumerate(lanes):                 # lanes at different short contexts
-            pr = rng.integers(0, cfg.vocab, 8 + (i * 5) % 40).astype(np.int32)
-            o = None
-            for j in range(0, len(pr), B):
-                o = lane.step_argmax(pr[j:j + B])
+        t_fill = time.time()
+        for i, lane in enumerate(lanes):
+            pr = rng.integers(0, cfg.vocab, ctxs[i]).astype(np.int32)
+            if mixed:                                    # prompts through the hybrid prefill in chunks of lane_m rows
+                lane.set_hybrid(True)
+                o = lane.greedy_generate(pr, 1, chain_k=1)
                 assert o is not None, lane.gpu_fault
-            toks.append(int(o[-1]))
+                lane.set_hybrid(False)
+                toks.append(int(o[0]))
+            else:
+                o = None
+                for j in range(0, len(pr), B):
+                    o = lane.step_argmax(pr[j:j + B])
+                    assert o is not None, lane.gpu_fault
+                toks.append(int(o[-1]))
+        t_fill = time.time() - t_fill
         step = type(eng).lane_step_argmax
         for _ in range(2):
             toks = step(lanes, toks).tolist()
@@ -166,7 +183,7 @@ def main():
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         lanes_report = {"lanes": B, "ms_per_step": dt * 1e3 / n_lane_steps, "tok_s_aggregate": B * n_lane_steps / dt,
-                        "contexts": "8-56 tokens", "path": "rows of the kernel-per-stage path, one launch sequence for all lanes"}
+                        "contexts": f"{min(ctxs)}-{max(ctxs)} tokens, mean {sum(ctxs) // B}", "fill_s": t_fill, "path": "rows of the kernel-per-stage path, one launch sequence for all lanes"}
         if B >= 16:                                     # the same batch with projections, experts and lm_head on the matrix cores
             lanes[0].set_hybrid(True)
             for _ in range(2):

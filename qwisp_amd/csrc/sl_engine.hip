@@ -363,11 +363,16 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
   SdpaArgs s{};
   s.qrot = e->qrot; s.kcache = L.kcache; s.vcache = L.vcache; s.st = e->st; s.maxSeq = e->max_seq; s.maxTiles = e->max_tiles;
   s.pm = e->pm; s.pl = e->pl; s.po = e->po; s.lanes = lanes;
-  if (mm && !lanes) hipLaunchKernelGGL(k_sdpa_tile_mfma, dim3(tiles, SL_ATT_KV, (M + 31) / 32), dim3(256), 0, e->stream, SdpaMmArgs{s, M});
+  if (mm && lanes) {
+    const int T = tiles >= 32 ? 4 : (tiles >= 8 ? 2 : 1);
+    hipLaunchKernelGGL(k_sdpa_lane_mfma, dim3((tiles + T - 1) / T, SL_ATT_KV, M), dim3(256), 0, e->stream, SdpaLaneArgs{s, T});
+  }
+  else if (mm) hipLaunchKernelGGL(k_sdpa_tile_mfma, dim3(tiles, SL_ATT_KV, (M + 31) / 32), dim3(256), 0, e->stream, SdpaMmArgs{s, M});
   else hipLaunchKernelGGL(k_sdpa_tile, dim3(tiles, SL_ATT_KV, M), dim3(256), 0, e->stream, s);
   SdpaMergeArgs g{};
   g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore; g.lanes = lanes;
-  hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
+  if (mm) hipLaunchKernelGGL(k_sdpa_merge_par, dim3(SL_ATT_HEADS, M), dim3(256), 0, e->stream, g);
+  else hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
   if (mm) launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.o_proj.w, L.o_proj.sb, M, H, 4096, e->mix, H}, e->stream);
   else if (M >= 2) hipLaunchKernelGGL((k_qmv_tile<2, 2, 4, false>), dim3(H / 8, (M + 3) / 4), dim3(256), 0, e->stream, HiddenArgs{}, e->ycore, 4096,
                                       L.o_proj.w, L.o_proj.sb, H, e->mix, H, M);

@@ -432,6 +432,192 @@ __global__ __launch_bounds__(256) void k_sdpa_tile_mfma(SdpaMmArgs a) {
   }
 }
 
+// -------------------------------------------------------------------------------------------------
+// Decode attention of a lane batch on the matrix cores (hybrid mode): every row is one new token of its own
+// sequence, so a key tile is shared only by the 8 query heads of a kv group.  Workgroup = (key tile of 64, kv head,
+// lane); the heads take rows 0..7 of a 32-row matrix operand (rows 8..31 carry nothing and their results are never
+// read).  Waves 0 and 1 form S = Q K^T for 32 keys each (16 matrix instructions), every wave then turns two heads'
+// scores into softmax pieces (fp32, hardware exp2; P rounded to half), and wave w forms dims 64w .. 64w+63 of
+// O = P V (8 matrix instructions).  A workgroup walks T consecutive tiles with the keys and values of
+// the next two tiles on their way while it works on the current one.  Same per-tile partials as k_sdpa_tile; k_sdpa_merge_par adds them up.
+// -------------------------------------------------------------------------------------------------
+struct SdpaLaneArgs {
+  SdpaArgs s;
+  int T;                       // consecutive key tiles per workgroup
+};
+// Workgroup barrier that waits for the wave's LDS traffic only: global loads issued before it stay in flight across it
+// (__syncthreads would wait for them as well).
+SL_DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+__global__ __launch_bounds__(256) void k_sdpa_lane_mfma(SdpaLaneArgs la) {
+  __shared__ __align__(16) uint16_t s_k[SDPA_TILE * KT_STRIDE];
+  __shared__ __align__(16) uint16_t s_vt[256 * VT_STRIDE];
+  __shared__ __align__(16) uint16_t s_p[8 * VT_STRIDE];
+  __shared__ __align__(16) uint16_t s_q[8 * KT_STRIDE];
+  __shared__ float s_s[8 * SDPA_TILE];
+  const SdpaArgs& a = la.s;
+  const int kvh = blockIdx.y, m = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, hh = lane >> 5;
+  const LaneRef& ref = a.lanes[m];
+  const int N = ref.st[0] + 1;                           // keys visible to the lane's new token, itself included
+  const int nt = (N + SDPA_TILE - 1) / SDPA_TILE;
+  const int t_begin = blockIdx.x * la.T, t_end = min(t_begin + la.T, nt);
+  if (t_begin >= nt) return;                             // uniform for the workgroup
+  const uint16_t* kbase = ref.kcache + (size_t)kvh * ref.max_seq * 256;
+  const uint16_t* vbase = ref.vcache + (size_t)kvh * ref.max_seq * 256;
+  // A tile's keys and values (a row on 32 neighbouring lanes each) as they are fetched;
+  // rows at or beyond N are zero.  The next tile's pieces are requested while the current tile is worked on.
+  struct Piece { uint4 k[8], v[8]; };
+  Piece pa, pb;
+  auto fetch = [&](Piece& pc, int t) {
+    const int j0 = t * SDPA_TILE;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int row = it * 8 + (tid >> 5), c8 = (tid & 31) * 8;
+      pc.k[it] = make_uint4(0, 0, 0, 0);
+      if (j0 + row < N) pc.k[it] = ld16(kbase + (size_t)(j0 + row) * 256 + c8);
+    }
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int row = it * 8 + (tid >> 5), c8 = (tid & 31) * 8;
+      pc.v[it] = make_uint4(0, 0, 0, 0);
+      if (j0 + row < N) pc.v[it] = ld16(vbase + (size_t)(j0 + row) * 256 + c8);
+    }
+  };
+  fetch(pa, t_begin);
+  if (t_begin + 1 < t_end) fetch(pb, t_begin + 1);
+  // the group's 8 query rows wait in LDS (first read after the first tile's barrier)
+  st16(&s_q[(tid >> 5) * KT_STRIDE + (tid & 31) * 8], ld16(a.qrot + ((size_t)m * 16 + kvh * 8 + (tid >> 5)) * 256 + (tid & 31) * 8));
+  const float NEG = -__int_as_float(0x7f800000);
+  // one tile from the piece that holds it; the piece is then free for the tile after the next, requested at once so
+  // that two tiles are in flight while this one is worked on
+  auto work = [&](Piece& pc, int tile) {
+    const int j0 = tile * SDPA_TILE;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) st16(&s_k[(it * 8 + (tid >> 5)) * KT_STRIDE + (tid & 31) * 8], pc.k[it]);
+    // values transposed [dim][key]; the eight-key blocks of a dim's row are permuted by (dim / 8) % 8, so that the 32
+    // lanes that hold one key (dims 8 apart, 1152 bytes in LDS) do not all write to the same two banks
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int c = tid & 31, kpos = ((it ^ (c & 7)) << 3) | (tid >> 5);       // key it*8 + (tid >> 5)
+      const uint32_t w[4] = {pc.v[it].x, pc.v[it].y, pc.v[it].z, pc.v[it].w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s_vt[(8 * c + i) * VT_STRIDE + kpos] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
+    }
+    lds_barrier();
+    if (tile + 2 < t_end) fetch(pc, tile + 2);
+    if (wave < 2) {
+      mf_f16v S;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S[r] = 0.0f;
+#pragma unroll
+      for (int st = 0; st < 16; ++st) {
+        // A: lane (col, hh) brings dims 16*st + 8*hh .. +7 of head col (rows 8..31 carry no head)
+        mf_h8 aq = *reinterpret_cast<const mf_h8*>(&s_q[(col & 7) * KT_STRIDE + 16 * st + 8 * hh]);
+        if (col >= 8) aq = __builtin_bit_cast(mf_h8, make_uint4(0, 0, 0, 0));
+        const mf_h8 bk = *reinterpret_cast<const mf_h8*>(&s_k[(32 * wave + col) * KT_STRIDE + 16 * st + 8 * hh]);
+        S = __builtin_amdgcn_mfma_f32_32x32x16_f16(aq, bk, S, 0, 0, 0);
+      }
+      // registers 0..3 of lane (col, hh) are heads 4*hh .. 4*hh+3 against key 32*wave + col
+      const int key = 32 * wave + col;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s_s[(4 * hh + r) * SDPA_TILE + key] = (j0 + key < N) ? 0.0625f * S[r] : NEG;
+    }
+    lds_barrier();
+#pragma unroll
+    for (int hq = 0; hq < 2; ++hq) {
+      const int h8 = 2 * wave + hq;
+      const float sv = s_s[h8 * SDPA_TILE + lane];
+      const float mx = tree_max<64>(sv);                 // the tile's first key is always visible: finite
+      const float p = (sv == NEG) ? 0.0f : __builtin_amdgcn_exp2f((sv - mx) * 1.44269504f);
+      const float l = tree_sum<64>(p);
+      if (lane == 0) {
+        const size_t pi = ((size_t)m * 16 + kvh * 8 + h8) * a.maxTiles + tile;
+        a.pm[pi] = mx; a.pl[pi] = l;
+      }
+      s_p[h8 * VT_STRIDE + lane] = f2h(p);
+    }
+    lds_barrier();
+    mf_f16v O[2];
+#pragma unroll
+    for (int d = 0; d < 2; ++d)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) O[d][r] = 0.0f;
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      mf_h8 ap = *reinterpret_cast<const mf_h8*>(&s_p[(col & 7) * VT_STRIDE + 16 * st + 8 * hh]);
+      if (col >= 8) ap = __builtin_bit_cast(mf_h8, make_uint4(0, 0, 0, 0));      // rows without a head
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        const int dim = 32 * (2 * wave + d) + col;
+        const mf_h8 bv = *reinterpret_cast<const mf_h8*>(&s_vt[dim * VT_STRIDE + (((2 * st + hh) ^ ((dim >> 3) & 7)) << 3)]);
+        O[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ap, bv, O[d], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float* po = a.po + (((size_t)m * 16 + kvh * 8 + 4 * hh + r) * a.maxTiles + tile) * 256 + col;
+#pragma unroll
+      for (int d = 0; d < 2; ++d) po[32 * (2 * wave + d)] = O[d][r];
+    }
+    lds_barrier();                                       // the tile's LDS is read out before the next one is written
+  };
+  for (int tile = t_begin; tile < t_end; tile += 2) {
+    work(pa, tile);
+    if (tile + 1 < t_end) work(pb, tile + 1);
+  }
+}
+
+// Merge of the tile partials on four waves (hybrid mode; tolerance-level: the tiles are not added up in tile order):
+// workgroup = (head, row); the global maximum first, then wave w takes tiles w, w+4, ... with four loads in flight,
+// and wave 0 adds the four partial sums and applies the output gate like k_sdpa_merge.
+__global__ __launch_bounds__(256) void k_sdpa_merge_par(SdpaMergeArgs a) {
+  __shared__ float s_mx[4], s_l[4];
+  __shared__ __align__(16) float s_o[4][256];
+  const int h = blockIdx.x, m = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int N = a.lanes ? a.lanes[m].st[0] + 1 : a.st[0] + m + 1;
+  const int nt = (N + SDPA_TILE - 1) / SDPA_TILE;
+  const size_t base = ((size_t)m * 16 + h) * a.maxTiles;
+  const float NEG = -__int_as_float(0x7f800000);
+  float mx = NEG;
+  for (int t = tid; t < nt; t += 256) mx = fmaxf(mx, a.pm[base + t]);
+  mx = tree_max<64>(mx);
+  if (lane == 0) s_mx[wave] = mx;
+  __syncthreads();
+  const float Mx = fmaxf(fmaxf(s_mx[0], s_mx[1]), fmaxf(s_mx[2], s_mx[3]));
+  float L = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int t0 = wave; t0 < nt; t0 += 16) {
+    float4 o[4]; float f[4], l[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = t0 + 4 * i;
+      const bool ok = t < nt;
+      const size_t pi = base + (ok ? t : t0);
+      o[i] = *reinterpret_cast<const float4*>(a.po + pi * 256 + 4 * lane);
+      f[i] = ok ? exp_c(a.pm[pi] - Mx) : 0.0f;
+      l[i] = a.pl[pi];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      L = fmaf(l[i], f[i], L);
+      O[0] = fmaf(o[i].x, f[i], O[0]); O[1] = fmaf(o[i].y, f[i], O[1]); O[2] = fmaf(o[i].z, f[i], O[2]); O[3] = fmaf(o[i].w, f[i], O[3]);
+    }
+  }
+  if (lane == 0) s_l[wave] = L;
+  *reinterpret_cast<float4*>(&s_o[wave][4 * lane]) = make_float4(O[0], O[1], O[2], O[3]);
+  __syncthreads();
+  if (wave != 0) return;
+  const float Ls = (s_l[0] + s_l[1]) + (s_l[2] + s_l[3]);
+  const uint2 graw = *reinterpret_cast<const uint2*>(a.proj + (size_t)m * PROJ_STRIDE + h * 512 + 256 + 4 * lane);
+  const float gt[4] = {lo_h(graw.x), hi_h(graw.x), lo_h(graw.y), hi_h(graw.y)};
+  float r[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float Oi = (s_o[0][4 * lane + i] + s_o[1][4 * lane + i]) + (s_o[2][4 * lane + i] + s_o[3][4 * lane + i]);
+    r[i] = f16r(f16r(Oi / Ls) * sigmoid16(gt[i]));
+  }
+  *reinterpret_cast<uint2*>(a.gated + (size_t)m * 4096 + h * 256 + 4 * lane) = make_uint2(pack2(r[0], r[1]), pack2(r[2], r[3]));
+}
+
 // Arg-max of rows of logits (first maximum, i.e. the lowest index on ties, of the half values): one workgroup per row.
 __global__ __launch_bounds__(1024) void k_argmax_logits(const uint16_t* __restrict__ logits, int V, int32_t* __restrict__ tok_out,
                                                         int out_off) {
