@@ -917,10 +917,13 @@ struct MoeCArgs {
   const uint32_t *shd_w, *shd_sb;   // [2048, 512]
   uint16_t* out;               // [M, 2048]
 };
-// Grid (128, M), four waves: 16 lanes per output row, 16 rows per workgroup.  The word sums of the nine activation
-// rows are formed once per workgroup (LDS); the packed activations are the stored halves as they are.
+// Grid (128, M), four waves: 16 lanes per output row, 16 rows per workgroup.  The nine activation rows (the stored
+// halves as they are) are parked in LDS once per workgroup, 64 bytes per lane at an 80-byte pitch so that the 16 lanes
+// of a row read them without bank conflicts, and their word sums are formed once per workgroup.
 __global__ __launch_bounds__(256) void k_moe_c(MoeCArgs a) {
+  constexpr int XP = 20;                                  // words per lane slot: 16 + 4 pad
   __shared__ __align__(16) float s_sx[9 * 16 * 4];
+  __shared__ __align__(16) uint32_t s_x[9 * 16 * XP];
   const int m = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int sub = lane >> 4, li = lane & 15;
   const int n = (blockIdx.x * 4 + wave) * 4 + sub;
@@ -937,10 +940,16 @@ __global__ __launch_bounds__(256) void k_moe_c(MoeCArgs a) {
   }
   wv[8] = ld16(a.shd_w + (size_t)n * 64 + 4 * li);
   sb[8] = a.shd_sb[(size_t)n * 8 + (li >> 1)];
+  for (int c = tid; c < 9 * 64; c += 256) {              // 16-byte pieces: row k, lane slot l, quarter j
+    const int k = c >> 6, l = (c >> 2) & 15, j = c & 3;
+    const uint16_t* src = (k < 8 ? a.act + ((size_t)m * 8 + k) * 512 : a.sh_act + (size_t)m * 512) + 32 * l + 8 * j;
+    st16(&s_x[(k * 16 + l) * XP + 4 * j], ld16(src));
+  }
+  __syncthreads();
   if (tid < 9 * 16) {
-    const int k = tid >> 4, l = tid & 15;
     float x[32], sx[4];
-    load32((k < 8 ? a.act + ((size_t)m * 8 + k) * 512 : a.sh_act + (size_t)m * 512) + 32 * l, x);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) unpack8(ld16(&s_x[tid * XP + 4 * j]), x + 8 * j);
     word_sums(x, sx);
     *reinterpret_cast<float4*>(&s_sx[tid * 4]) = make_float4(sx[0], sx[1], sx[2], sx[3]);
   }
@@ -948,10 +957,9 @@ __global__ __launch_bounds__(256) void k_moe_c(MoeCArgs a) {
   float acc = 0.0f, sy = 0.0f;
 #pragma unroll
   for (int k = 0; k < 9; ++k) {
-    const uint16_t* src = (k < 8 ? a.act + ((size_t)m * 8 + k) * 512 : a.sh_act + (size_t)m * 512) + 32 * li;
     uint32_t xp[16];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) { const uint4 v = ld16(src + 8 * j); xp[4 * j] = v.x; xp[4 * j + 1] = v.y; xp[4 * j + 2] = v.z; xp[4 * j + 3] = v.w; }
+    for (int j = 0; j < 4; ++j) { const uint4 v = ld16(&s_x[(k * 16 + li) * XP + 4 * j]); xp[4 * j] = v.x; xp[4 * j + 1] = v.y; xp[4 * j + 2] = v.z; xp[4 * j + 3] = v.w; }
     const float4 s4 = *reinterpret_cast<const float4*>(&s_sx[(k * 16 + li) * 4]);
     const float sx[4] = {s4.x, s4.y, s4.z, s4.w};
     const float d = f16r(tree_sum<16>(quad_term(wv[k], sb[k], xp, sx)));
