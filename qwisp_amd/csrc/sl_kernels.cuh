@@ -1035,7 +1035,7 @@ __global__ __launch_bounds__(64) void k_attn_prep(AttnPrepArgs a) {
 // query heads.  The tile's keys are
 // staged in LDS; lane j scores key j against the query heads of its wave (a balanced tree over
 // 64 leaves of 4 dims), then p = exp(s - tile max), l = butterfly sum of p, o = fmaf chain over
-// the tile's keys with V rows read coalesced.  Reference semantics: sdpa_rows
+// the tile's keys with the value tile parked in LDS (fetched once per workgroup).  Reference semantics: sdpa_rows
 // SeedlessMetalForward.swift:4922-4989 (q scaled by 1/16, fp32 softmax).
 // -------------------------------------------------------------------------------------------------
 struct SdpaArgs {
@@ -1062,9 +1062,14 @@ __global__ __launch_bounds__(256) void k_sdpa_tile(SdpaArgs a) {
   const uint16_t* kbase = a.kcache + ((size_t)kvh * a.maxSeq + j0) * 256;
   const uint16_t* vbase = a.vcache + ((size_t)kvh * a.maxSeq + j0) * 256;
   // stage keys (rows >= nk are never read) and the group's 8 scaled queries; wave w then owns heads 2w, 2w+1
+  // the value tile is requested now and parked in the key tile's space once the scores are done (rows >= nk: zero)
+  uint4 vr[8];
+#pragma unroll
   for (int it = 0; it < 8; ++it) {
     const int row = it * 8 + (tid >> 5), c8 = (tid & 31) * 8;
     if (row < nk) st16(&s_k[row * KT_STRIDE + c8], ld16(kbase + (size_t)row * 256 + c8));
+    vr[it] = make_uint4(0, 0, 0, 0);
+    if (row < nk) vr[it] = ld16(vbase + (size_t)row * 256 + c8);
   }
   {
     const int idx = tid * 8;                         // 0..2047 step 8
@@ -1122,15 +1127,31 @@ __global__ __launch_bounds__(256) void k_sdpa_tile(SdpaArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) o[h][i] = 0.0f;
   }
-#pragma unroll 8
-  for (int j = 0; j < nk; ++j) {
-    const uint2 vraw = *reinterpret_cast<const uint2*>(vbase + (size_t)j * 256 + 4 * lane);
-    const float vf[4] = {lo_h(vraw.x), hi_h(vraw.x), lo_h(vraw.y), hi_h(vraw.y)};
+  // Weighted value sums: the chain of fmaf over the tile's keys in order.  All 64 keys are walked: beyond nk the weight
+  // and the parked value are zero, and fmaf(0, 0, o) returns o as it is.  Eight keys at a time: their weights come
+  // over as scalars (lane reads), their value pieces from LDS.
+  __syncthreads();                                   // every wave is done with the keys
+  uint16_t* s_v = s_k;                               // [64][256] halves
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const float pj = __shfl(p[h], j, 64);
+  for (int it = 0; it < 8; ++it) st16(&s_v[(it * 8 + (tid >> 5)) * 256 + (tid & 31) * 8], vr[it]);
+  __syncthreads();
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[h][i] = fmaf(pj, vf[i], o[h][i]);
+  for (int j0v = 0; j0v < SDPA_TILE; j0v += 8) {
+    uint2 vraw[8];
+    float pj[2][8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) vraw[u] = *reinterpret_cast<const uint2*>(&s_v[(j0v + u) * 256 + 4 * lane]);
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int u = 0; u < 8; ++u) pj[h][u] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(p[h]), j0v + u));
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float vf[4] = {lo_h(vraw[u].x), hi_h(vraw[u].x), lo_h(vraw[u].y), hi_h(vraw[u].y)};
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[h][i] = fmaf(pj[h][u], vf[i], o[h][i]);
     }
   }
 #pragma unroll
@@ -1157,13 +1178,27 @@ __global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
   const int nt = (N + SDPA_TILE - 1) / SDPA_TILE;
   const size_t base = ((size_t)m * 16 + h) * a.maxTiles;
   float Mx = -__int_as_float(0x7f800000);
-  for (int t = 0; t < nt; ++t) Mx = fmaxf(Mx, a.pm[base + t]);
+  for (int t = lane; t < nt; t += 64) Mx = fmaxf(Mx, a.pm[base + t]);
+  Mx = tree_max<64>(Mx);
+  // tiles are added up in order; eight tiles' partials are requested together (one memory round trip per eight tiles)
   float L = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int t = 0; t < nt; ++t) {
-    const float f = exp_c(a.pm[base + t] - Mx);
-    L = fmaf(a.pl[base + t], f, L);
-    const float4 o = *reinterpret_cast<const float4*>(a.po + (base + t) * 256 + 4 * lane);
-    O[0] = fmaf(o.x, f, O[0]); O[1] = fmaf(o.y, f, O[1]); O[2] = fmaf(o.z, f, O[2]); O[3] = fmaf(o.w, f, O[3]);
+  for (int t0 = 0; t0 < nt; t0 += 8) {
+    float4 o[8];
+    float pmv[8], plv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const size_t pi = base + min(t0 + u, nt - 1);
+      o[u] = *reinterpret_cast<const float4*>(a.po + pi * 256 + 4 * lane);
+      pmv[u] = a.pm[pi]; plv[u] = a.pl[pi];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (t0 + u < nt) {
+        const float f = exp_c(pmv[u] - Mx);
+        L = fmaf(plv[u], f, L);
+        O[0] = fmaf(o[u].x, f, O[0]); O[1] = fmaf(o[u].y, f, O[1]); O[2] = fmaf(o[u].z, f, O[2]); O[3] = fmaf(o[u].w, f, O[3]);
+      }
+    }
   }
   const uint2 graw = *reinterpret_cast<const uint2*>(a.proj + (size_t)m * PROJ_STRIDE + h * 512 + 256 + 4 * lane);
   const float gt[4] = {lo_h(graw.x), hi_h(graw.x), lo_h(graw.y), hi_h(graw.y)};
