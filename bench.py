@@ -11,7 +11,7 @@ k_decode_flow: one launch runs a chain of `--chain` tokens, each fed back on the
 timed with HIP events on the engine's stream; roofline.avg_ms and bytes_per_launch are those of one
 launch = `--chain` tokens), and the CPU baseline (the oracle, timed on this host's cores on a bounded
 sample of the same workload).  After the timed decode region the same engine also times the batched
-paths on the same weights and reports them as extra objects of the line: `lane_batch` (32 sequences
+paths on the same weights and reports them as extra objects of the line: `lane_batch` (32 sequences at mixed contexts of 1K-16K tokens
 stepped together), `verify` (4-row verify steps) and `prefill` (a 2048-token prompt in chunks of 1024
 rows, exact rows and hybrid on the matrix cores) and `context_sweep` (decode after 4K and 16K prompts);
 `--lanes 0 --verify-rows 0 --prefill-chunk 0 --context-sweep ''` skips them.
@@ -29,7 +29,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 PROMPT_LEN = 512
 # HBM bytes per decoded token: rocprofv3 FETCH_SIZE + WRITE_SIZE of a k_decode_flow launch (profiles/) / its 8 tokens
-TRAFFIC_BYTES_PER_TOKEN = 1936080204   # 2 x FETCH_SIZE (copy-calibrated) + WRITE_SIZE, in bytes, at context ~525
+TRAFFIC_BYTES_PER_TOKEN = 1936024336   # 2 x FETCH_SIZE (copy-calibrated) + WRITE_SIZE, in bytes, at context ~525
 
 
 def step_bytes(cfg, ctx):

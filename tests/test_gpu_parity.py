@@ -131,8 +131,8 @@ def test_eleven_lanes_in_one_batch_equal_solo(env, small_model):
 @pytest.mark.gpu
 def test_lane_batch_on_the_matrix_cores_stays_close_to_solo(env, small_model):
     """Hybrid mode on the engine that drives a lane batch: with 16 or more lanes the projections, the grouped experts
-    and lm_head of the batched step run on the matrix cores (tolerance-level, like the hybrid prefill); the lanes'
-    recurrent state, caches and attention stay on the exact kernels.  Logits stay within a few per cent of solo
+    lm_head and the decode attention of the batched step run on the matrix cores (tolerance-level, like the hybrid
+    prefill); the lanes' recurrent state and the cache appends stay on the exact kernels.  Logits stay within a few per cent of solo
     engines on the exact path and most tokens agree; switching hybrid off returns to the exact bits."""
     cfg, dev, host = small_model
     B = 16
