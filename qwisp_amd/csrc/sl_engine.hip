@@ -303,6 +303,10 @@ void launch_hidden_tile(sl_engine* e, const HiddenArgs& ha, const uint32_t* w, c
 }
 // Hybrid mode: steps of at least 16 rows (prefill chunks, lane batches) take the dense projections to the matrix cores.
 // (Rows of one sequence or one row each of a batch of lanes: the projections and the experts do not care.)
+// The K = 4096 projections have 2048 outputs = 16 workgroups per 32-row tile on the matrix cores: a lane batch of
+// fewer than 64 rows keeps the row-tiled exact kernel for them (256 workgroups per 4 rows; 32 rows: 21 against 28 us).
+// Prefill chunks do not switch, so that a row's result does not depend on the chunking.
+constexpr int MM_OUT_ROWS = 64;
 bool use_matrix_cores(const sl_engine* e, int M, const LaneRef* lanes) { (void)lanes; return e->hybrid && M >= 16 && M <= GROUP_CAP; }
 // `lanes` (null for rows of one sequence) = this layer's row of the lane table: row b of the batch is lane b's next token.
 void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs& ha, const LaneRef* lanes) {
@@ -330,7 +334,7 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
   } else {
     hipLaunchKernelGGL(k_gdn_core, dim3(256, lanes ? M : 1), dim3(256), 0, e->stream, g);
   }
-  if (mm) {
+  if (mm && !(lanes && M < MM_OUT_ROWS)) {
     hipLaunchKernelGGL(k_gdn_gate_rows, dim3(SL_GDN_HV, M), dim3(64), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32);
     launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.out_proj.w, L.out_proj.sb, M, H, 4096, e->mix, H}, e->stream);
   } else if (M >= 2) {
@@ -373,7 +377,7 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
   g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore; g.lanes = lanes;
   if (mm) hipLaunchKernelGGL(k_sdpa_merge_par, dim3(SL_ATT_HEADS, M), dim3(256), 0, e->stream, g);
   else hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
-  if (mm) launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.o_proj.w, L.o_proj.sb, M, H, 4096, e->mix, H}, e->stream);
+  if (mm && !(lanes && M < MM_OUT_ROWS)) launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.o_proj.w, L.o_proj.sb, M, H, 4096, e->mix, H}, e->stream);
   else if (M >= 2) hipLaunchKernelGGL((k_qmv_tile<2, 2, 4, false>), dim3(H / 8, (M + 3) / 4), dim3(256), 0, e->stream, HiddenArgs{}, e->ycore, 4096,
                                       L.o_proj.w, L.o_proj.sb, H, e->mix, H, M);
   else hipLaunchKernelGGL((k_qmv_plain<2, 2>), dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, 4096, L.o_proj.w, L.o_proj.sb,

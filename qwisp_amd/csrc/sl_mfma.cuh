@@ -568,7 +568,7 @@ __global__ __launch_bounds__(256) void k_sdpa_lane_mfma(SdpaLaneArgs la) {
 }
 
 // Merge of the tile partials on four waves (hybrid mode; tolerance-level: the tiles are not added up in tile order):
-// workgroup = (head, row); the global maximum first, then wave w takes tiles w, w+4, ... with four loads in flight,
+// workgroup = (head, row); the global maximum first, then wave w takes tiles w, w+4, ... with eight loads in flight,
 // and wave 0 adds the four partial sums and applies the output gate like k_sdpa_merge.
 __global__ __launch_bounds__(256) void k_sdpa_merge_par(SdpaMergeArgs a) {
   __shared__ float s_mx[4], s_l[4];
@@ -585,10 +585,10 @@ __global__ __launch_bounds__(256) void k_sdpa_merge_par(SdpaMergeArgs a) {
   __syncthreads();
   const float Mx = fmaxf(fmaxf(s_mx[0], s_mx[1]), fmaxf(s_mx[2], s_mx[3]));
   float L = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int t0 = wave; t0 < nt; t0 += 16) {
-    float4 o[4]; float f[4], l[4];
+  for (int t0 = wave; t0 < nt; t0 += 32) {
+    float4 o[8]; float f[8], l[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 8; ++i) {
       const int t = t0 + 4 * i;
       const bool ok = t < nt;
       const size_t pi = base + (ok ? t : t0);
@@ -597,7 +597,7 @@ __global__ __launch_bounds__(256) void k_sdpa_merge_par(SdpaMergeArgs a) {
       l[i] = a.pl[pi];
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 8; ++i) {
       L = fmaf(l[i], f[i], L);
       O[0] = fmaf(o[i].x, f[i], O[0]); O[1] = fmaf(o[i].y, f[i], O[1]); O[2] = fmaf(o[i].z, f[i], O[2]); O[3] = fmaf(o[i].w, f[i], O[3]);
     }
