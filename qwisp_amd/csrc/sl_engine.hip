@@ -332,7 +332,8 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
     hipLaunchKernelGGL(k_gdn_prep_rows, dim3(65, M), dim3(64), 0, e->stream, pa);
     hipLaunchKernelGGL(k_gdn_scan_rows, dim3(512), dim3(256), 0, e->stream, pa);
   } else {
-    hipLaunchKernelGGL(k_gdn_core, dim3(256, lanes ? M : 1), dim3(256), 0, e->stream, g);
+    if (lanes) hipLaunchKernelGGL(k_gdn_core<4>, dim3(128, M), dim3(256), 0, e->stream, g);
+    else hipLaunchKernelGGL(k_gdn_core<2>, dim3(256, 1), dim3(256), 0, e->stream, g);
   }
   if (mm && !(lanes && M < MM_OUT_ROWS)) {
     hipLaunchKernelGGL(k_gdn_gate_rows, dim3(SL_GDN_HV, M), dim3(64), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32);

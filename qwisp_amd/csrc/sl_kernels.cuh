@@ -395,8 +395,13 @@ SL_DEV GdnView gdn_view(const GdnArgs& a, int lane_row) {
   v.sin_ = par ? s1 : s0; v.sout = const_cast<float*>(par ? s0 : s1);
   return v;
 }
+// NIT pairs of value rows per wave: a workgroup owns 8 * NIT value dims of one head (grid.x = 32 heads * 16 / NIT).
+// Lane batches use NIT = 4 (half the workgroups, twice the state bytes in flight per workgroup); the arithmetic per
+// value row is the same.
+template <int NIT>
 __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
-  __shared__ float s_q[128], s_k[128], s_v[16], s_gb[2];
+  constexpr int DVW = 8 * NIT, NB = 128 / DVW;          // value dims per workgroup, workgroups per head
+  __shared__ float s_q[128], s_k[128], s_v[DVW], s_gb[2];
   const GdnView vw = gdn_view(a, blockIdx.y);
   const uint16_t* hin = vw.hin;
   uint16_t* hout = vw.hout;
@@ -405,23 +410,23 @@ __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
   const uint16_t* proj = vw.proj;
   uint16_t* ycore = vw.ycore;
   const int M = vw.M;
-  const int hv = blockIdx.x >> 3, dvb = blockIdx.x & 7, hk = hv >> 1;
+  const int hv = blockIdx.x / NB, dvb = blockIdx.x % NB, hk = hv >> 1;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
 
-  float s[2][4];
+  float s[NIT][4];
 #pragma unroll
-  for (int it = 0; it < 2; ++it) {
-    const int dv = dvb * 16 + wave * 4 + it * 2 + half;
+  for (int it = 0; it < NIT; ++it) {
+    const int dv = dvb * DVW + wave * 2 * NIT + it * 2 + half;
     const float4 v = *reinterpret_cast<const float4*>(sin_ + ((size_t)hv * 128 + dv) * 128 + 4 * l32);
     s[it][0] = v.x; s[it][1] = v.y; s[it][2] = v.z; s[it][3] = v.w;
   }
   const int qk_ch = (tid < 128) ? (hk * 128 + tid) : (2048 + hk * 128 + (tid - 128));
-  const int v_ch = 4096 + hv * 128 + dvb * 16 + (tid & 15);
+  const int v_ch = 4096 + hv * 128 + dvb * DVW + (tid & (DVW - 1));
 
   for (int t = 0; t < M; ++t) {
     const float c = conv_silu(proj, a.conv_w, hin, t, qk_ch);
     if (tid < 128) s_q[tid] = c; else s_k[tid - 128] = c;
-    if (tid < 16) s_v[tid] = conv_silu(proj, a.conv_w, hin, t, v_ch);
+    if (tid < DVW) s_v[tid] = conv_silu(proj, a.conv_w, hin, t, v_ch);
     __syncthreads();
     if (wave < 2) {
       // weightless rmsnorm over 128, then the key/query scale, both rounded to half
@@ -445,8 +450,8 @@ __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
     const float4 q4 = *reinterpret_cast<const float4*>(&s_q[4 * l32]);
     const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, qq[4] = {q4.x, q4.y, q4.z, q4.w};
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int dvl = wave * 4 + it * 2 + half;
+    for (int it = 0; it < NIT; ++it) {
+      const int dvl = wave * 2 * NIT + it * 2 + half;
       float acc = 0.0f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) { s[it][i] = s[it][i] * g; acc = fmaf(s[it][i], kk[i], acc); }
@@ -456,13 +461,13 @@ __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) { s[it][i] = fmaf(kk[i], delta, s[it][i]); acc = fmaf(s[it][i], qq[i], acc); }
       const float y = tree_sum<32>(acc);
-      if (l32 == 0) ycore[(size_t)t * 4096 + hv * 128 + dvb * 16 + dvl] = f2h(y);
+      if (l32 == 0) ycore[(size_t)t * 4096 + hv * 128 + dvb * DVW + dvl] = f2h(y);
     }
     __syncthreads();
   }
 #pragma unroll
-  for (int it = 0; it < 2; ++it) {
-    const int dv = dvb * 16 + wave * 4 + it * 2 + half;
+  for (int it = 0; it < NIT; ++it) {
+    const int dv = dvb * DVW + wave * 2 * NIT + it * 2 + half;
     *reinterpret_cast<float4*>(sout + ((size_t)hv * 128 + dv) * 128 + 4 * l32) = make_float4(s[it][0], s[it][1], s[it][2], s[it][3]);
   }
   // history shift: rows M..M+2 of [hist | qkv]; each channel written by exactly one workgroup
@@ -470,7 +475,7 @@ __global__ __launch_bounds__(256) void k_gdn_core(GdnArgs a) {
 #pragma unroll
     for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + qk_ch] = f2h(conv_tap(proj, hin, M + j, qk_ch));
   }
-  if (tid < 16) {
+  if (tid < DVW) {
 #pragma unroll
     for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + v_ch] = f2h(conv_tap(proj, hin, M + j, v_ch));
   }
