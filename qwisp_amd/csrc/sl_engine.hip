@@ -376,7 +376,8 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
   else hipLaunchKernelGGL(k_sdpa_tile, dim3(tiles, SL_ATT_KV, M), dim3(256), 0, e->stream, s);
   SdpaMergeArgs g{};
   g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore; g.lanes = lanes;
-  if (mm) hipLaunchKernelGGL(k_sdpa_merge_par, dim3(SL_ATT_HEADS, M), dim3(256), 0, e->stream, g);
+  if (mm && lanes) hipLaunchKernelGGL(k_sdpa_merge_par<16>, dim3(SL_ATT_HEADS, M), dim3(1024), 0, e->stream, g);
+  else if (mm) hipLaunchKernelGGL(k_sdpa_merge_par<4>, dim3(SL_ATT_HEADS, M), dim3(256), 0, e->stream, g);
   else hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
   if (mm && !(lanes && M < MM_OUT_ROWS)) launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.o_proj.w, L.o_proj.sb, M, H, 4096, e->mix, H}, e->stream);
   else if (M >= 2) hipLaunchKernelGGL((k_qmv_tile<2, 2, 4, false>), dim3(H / 8, (M + 3) / 4), dim3(256), 0, e->stream, HiddenArgs{}, e->ycore, 4096,

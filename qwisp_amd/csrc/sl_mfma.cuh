@@ -567,29 +567,34 @@ __global__ __launch_bounds__(256) void k_sdpa_lane_mfma(SdpaLaneArgs la) {
   }
 }
 
-// Merge of the tile partials on four waves (hybrid mode; tolerance-level: the tiles are not added up in tile order):
-// workgroup = (head, row); the global maximum first, then wave w takes tiles w, w+4, ... with eight loads in flight,
-// and wave 0 adds the four partial sums and applies the output gate like k_sdpa_merge.
-__global__ __launch_bounds__(256) void k_sdpa_merge_par(SdpaMergeArgs a) {
-  __shared__ float s_mx[4], s_l[4];
-  __shared__ __align__(16) float s_o[4][256];
+// Merge of the tile partials on several waves (hybrid mode; tolerance-level: the tiles are not added up in tile order):
+// workgroup = (head, row); the global maximum first, then wave w takes tiles w, w + MERGE_WAVES, ... with eight loads in
+// flight, and wave 0 adds the waves' partial sums and applies the output gate like k_sdpa_merge.  Sixteen waves for a
+// lane batch (few rows, each with up to hundreds of tiles), four for the rows of a prefill chunk (thousands of
+// workgroups: bound by the bytes, and slower with large workgroups).
+template <int MERGE_WAVES>
+__global__ __launch_bounds__(64 * MERGE_WAVES) void k_sdpa_merge_par(SdpaMergeArgs a) {
+  __shared__ float s_mx[MERGE_WAVES], s_l[MERGE_WAVES];
+  __shared__ __align__(16) float s_o[MERGE_WAVES][256];
   const int h = blockIdx.x, m = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int N = a.lanes ? a.lanes[m].st[0] + 1 : a.st[0] + m + 1;
   const int nt = (N + SDPA_TILE - 1) / SDPA_TILE;
   const size_t base = ((size_t)m * 16 + h) * a.maxTiles;
   const float NEG = -__int_as_float(0x7f800000);
   float mx = NEG;
-  for (int t = tid; t < nt; t += 256) mx = fmaxf(mx, a.pm[base + t]);
+  for (int t = tid; t < nt; t += 64 * MERGE_WAVES) mx = fmaxf(mx, a.pm[base + t]);
   mx = tree_max<64>(mx);
   if (lane == 0) s_mx[wave] = mx;
   __syncthreads();
-  const float Mx = fmaxf(fmaxf(s_mx[0], s_mx[1]), fmaxf(s_mx[2], s_mx[3]));
+  float Mx = s_mx[0];
+#pragma unroll
+  for (int w = 1; w < MERGE_WAVES; ++w) Mx = fmaxf(Mx, s_mx[w]);
   float L = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int t0 = wave; t0 < nt; t0 += 32) {
+  for (int t0 = wave; t0 < nt; t0 += 8 * MERGE_WAVES) {
     float4 o[8]; float f[8], l[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int t = t0 + 4 * i;
+      const int t = t0 + MERGE_WAVES * i;
       const bool ok = t < nt;
       const size_t pi = base + (ok ? t : t0);
       o[i] = *reinterpret_cast<const float4*>(a.po + pi * 256 + 4 * lane);
@@ -606,15 +611,18 @@ __global__ __launch_bounds__(256) void k_sdpa_merge_par(SdpaMergeArgs a) {
   *reinterpret_cast<float4*>(&s_o[wave][4 * lane]) = make_float4(O[0], O[1], O[2], O[3]);
   __syncthreads();
   if (wave != 0) return;
-  const float Ls = (s_l[0] + s_l[1]) + (s_l[2] + s_l[3]);
+  float Ls = 0.0f, Os[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int w = 0; w < MERGE_WAVES; ++w) {
+    Ls += s_l[w];
+    const float4 v = *reinterpret_cast<const float4*>(&s_o[w][4 * lane]);
+    Os[0] += v.x; Os[1] += v.y; Os[2] += v.z; Os[3] += v.w;
+  }
   const uint2 graw = *reinterpret_cast<const uint2*>(a.proj + (size_t)m * PROJ_STRIDE + h * 512 + 256 + 4 * lane);
   const float gt[4] = {lo_h(graw.x), hi_h(graw.x), lo_h(graw.y), hi_h(graw.y)};
   float r[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float Oi = (s_o[0][4 * lane + i] + s_o[1][4 * lane + i]) + (s_o[2][4 * lane + i] + s_o[3][4 * lane + i]);
-    r[i] = f16r(f16r(Oi / Ls) * sigmoid16(gt[i]));
-  }
+  for (int i = 0; i < 4; ++i) r[i] = f16r(f16r(Os[i] / Ls) * sigmoid16(gt[i]));
   *reinterpret_cast<uint2*>(a.gated + (size_t)m * 4096 + h * 256 + 4 * lane) = make_uint2(pack2(r[0], r[1]), pack2(r[2], r[3]));
 }
 
