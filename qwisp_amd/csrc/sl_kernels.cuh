@@ -1185,19 +1185,19 @@ __global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
   float Mx = -__int_as_float(0x7f800000);
   for (int t = lane; t < nt; t += 64) Mx = fmaxf(Mx, a.pm[base + t]);
   Mx = tree_max<64>(Mx);
-  // tiles are added up in order; eight tiles' partials are requested together (one memory round trip per eight tiles)
+  // tiles are added up in order; sixteen tiles' partials are requested together (one memory round trip per sixteen tiles)
   float L = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int t0 = 0; t0 < nt; t0 += 8) {
-    float4 o[8];
-    float pmv[8], plv[8];
+  for (int t0 = 0; t0 < nt; t0 += 16) {
+    float4 o[16];
+    float pmv[16], plv[16];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < 16; ++u) {
       const size_t pi = base + min(t0 + u, nt - 1);
       o[u] = *reinterpret_cast<const float4*>(a.po + pi * 256 + 4 * lane);
       pmv[u] = a.pm[pi]; plv[u] = a.pl[pi];
     }
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < 16; ++u) {
       if (t0 + u < nt) {
         const float f = exp_c(pmv[u] - Mx);
         L = fmaf(plv[u], f, L);
