@@ -338,11 +338,16 @@ int sl_set_persistent(sl_engine* e, int enable);
  * and attention stay on the exact kernels.  Decode steps and steps of fewer than 16 rows are unaffected. */
 int sl_set_hybrid(sl_engine* e, int enable);
 
-/* Diagnostic: while enabled, workgroups 0 and 100 of the single-launch step record a 100 MHz clock stamp
- * before and after every poll; the call copies out[0] = number of stamps of workgroup 0 and out[1..] its
- * stamps of the last step (clock << 16 | stage id << 8 | poll retries), the same for workgroup 100 from
- * out[2048]. */
-int sl_debug_stage_clock(sl_engine* e, int enable, unsigned long long* out, int cap);
+/* Diagnostic in the manner of forwardRowsProfiled (SFV:4352), at the grain of one stage of the single-launch step:
+ * while enabled, batch-1 steps run a variant of that kernel in which every workgroup records 100 MHz clock stamps of
+ * the last step of a launch (kept on chip until the launch ends, so they do not disturb what they time).  The call
+ * copies the stamps of the most recent launch out, then sets the mode:
+ * out[wg * sl_stage_clock_words() + (layer * 8 + stage) * 8 + kind], 0 = not reached; stage 0 in-projection, 1 recurrence
+ * or attention tiles, 2 attention merge, 3 K = 4096 projection, 4 router and shared gate/up, 5 routed gate/up, 6 down and
+ * combine; layer n_layers = head (stage 0 lm_head, 1 final arg-max); kind 0 stage entered, 1 inputs arrived,
+ * 2 preparation done, 3 arithmetic done, 4 results stored. */
+int sl_debug_stage_clock(sl_engine* e, int enable, uint32_t* out, int cap_words);
+int sl_stage_clock_words(void);
 
 /* Per-kernel timing in the manner of forwardRowsProfiled (SFV:4352): while enabled, every launch of
  * the dominant kernel (the persistent step kernel, or lm_head in the kernel-per-stage sequence) is bracketed by HIP events on the engine's stream; the read call returns the

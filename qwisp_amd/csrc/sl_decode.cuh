@@ -45,7 +45,7 @@ struct DecodeP {
   const float *rope_cos, *rope_sin;
   uint16_t *hA, *normed, *logits;     // (hA: unused by the step kernel) final-normed row and logits out
   int32_t *tok_in, *tok_out, *st;     // st: {position, parity of every layer's ping-pong caches}
-  unsigned long long* tstamp;   // optional diagnostic clock stamps
+  uint32_t* tstamp;             // diagnostic clock stamps of the stamping kernel variant: [workgroups][STAMP_WORDS]
   unsigned* bar;   // [16] stage-instance counter (advanced every launch), [32] abort flag
 };
 
@@ -98,7 +98,6 @@ SL_DEV void st_co_h4(rsrc_t r, int idx, const float* x) {
   __builtin_amdgcn_raw_buffer_store_b64(v, r, idx * 2, 0, CO_SC1);
 }
 
-struct StampState { int nts, kbar; };      // diagnostic stamp bookkeeping
 // ---- activation vector in LDS ------------------------------------------------------------------------
 // Packed pair i (elements 2i, 2i+1) of lane l of block b lives at xs[(16*b + i)*64 + l]; word sums at
 // sxs[(4*b + j)*64 + l].
@@ -119,7 +118,6 @@ struct Lds {
   float knew[256], vnew[256];
   float sm[8 * 64];                         // attention: per head softmax weights of the tile
   float part[16 * 64];                      // attention: half-tree score partials; router: logits and exps
-  StampState bar;
 };
 __shared__ Lds g_L;
 extern __shared__ __align__(16) uint16_t g_vt[];   // dynamic: staged value tile [64][256] halves, then the softmax

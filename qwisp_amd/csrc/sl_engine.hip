@@ -80,7 +80,8 @@ struct sl_engine {
   int32_t *cand_i = nullptr, *tok_in = nullptr, *tok_out = nullptr, *st = nullptr;
   int n_cand = 0;
   // persistent single-token kernel
-  unsigned long long* dec_tstamp = nullptr;
+  uint32_t* dec_tstamp = nullptr;  // stage clock stamps [dec_grid][STAMP_WORDS], written by the stamping kernel variant
+  bool stage_clock = false;
   unsigned* dec_bar = nullptr;
   int dec_grid = 0;                // 0 = not available (fewer than 256 compute units)
   FlowP* flow_params = nullptr;    // device copy of the single-launch step's parameters
@@ -444,8 +445,9 @@ void launch_head(sl_engine* e, int M, const HiddenArgs& ha, int out_off, bool fe
 void launch_decode(sl_engine* e, int out_off, bool feed, int steps) {
   const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
-  if (e->gate8) hipLaunchKernelGGL(k_decode_flow<true>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0, steps);
-  else hipLaunchKernelGGL(k_decode_flow<false>, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0, steps);
+  auto kern = e->gate8 ? (e->stage_clock ? k_decode_flow<true, true> : k_decode_flow<true, false>)
+                       : (e->stage_clock ? k_decode_flow<false, true> : k_decode_flow<false, false>);
+  hipLaunchKernelGGL(kern, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, out_off, feed ? 1 : 0, steps);
   if (prof) { (void)hipEventRecord(e->head_ev[2 * e->head_pending + 1], e->stream); e->head_pending++; }
   e->pos += steps;
   if (steps & 1) for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
@@ -679,7 +681,9 @@ int alloc_runtime(sl_engine* e) {
       P.final_norm = e->final_norm; P.rope_cos = e->rope_cos; P.rope_sin = e->rope_sin;
       P.hA = e->hA; P.normed = e->normed; P.logits = e->logits;
       P.tok_in = e->tok_in; P.tok_out = e->tok_out; P.st = e->st; P.bar = e->dec_bar;
-      e->dec_tstamp = dalloc<unsigned long long>(e, 2048 + 16 * 256 * 2, true);
+      e->dec_tstamp = dalloc<uint32_t>(e, (size_t)256 * STAMP_WORDS, true);
+      if (!e->dec_tstamp) return SL_ERR_DEVICE;
+      P.tstamp = e->dec_tstamp;
       {
         FlowP F;
         std::memset(&F, 0, sizeof(F));
@@ -701,8 +705,10 @@ int alloc_runtime(sl_engine* e) {
         e->flow_host = F;
         e->flow_params = upload<FlowP>(e, &F, 1, SL_LOC_HOST);
         if (!e->flow_params) return SL_ERR_DEVICE;
-        SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<false>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
-        SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<true>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
+        SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
+        SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
+        SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
+        SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
       }
       e->dec_grid = 256;
     }
@@ -868,18 +874,20 @@ int sl_set_persistent(sl_engine* e, int enable) {
   e->use_persistent = enable != 0;
   return SL_OK;
 }
-// Test/diagnostic hook: clock stamps (100 MHz ticks) that workgroups 0 and 100 take before and after every poll
-// of the single-launch step while enabled; out[0] = count, out[1..] = (clock << 16 | stage id << 8 | retries),
-// the same for workgroup 100 from out[2048].
-int sl_debug_stage_clock(sl_engine* e, int enable, unsigned long long* out, int cap) {
+// Diagnostic hook: while enabled, batch-1 steps run the stamping variant of the single-launch kernel, in which every
+// workgroup records 100 MHz clock stamps of the last step of a launch; the call copies them out,
+// out[wg * sl_stage_clock_words() + (layer * 8 + stage) * 8 + kind] (0 = not reached).
+int sl_debug_stage_clock(sl_engine* e, int enable, uint32_t* out, int cap_words) {
   int r = guard(e); if (r) return r;
   if (!e->flow_params) return SL_ERR_UNSUPPORTED;
-  if (out && cap > 0) {
-    r = copy_sync(e, out, e->dec_tstamp, (size_t)(cap < 2048 + 8192 ? cap : 2048 + 8192) * 8, hipMemcpyDeviceToHost); if (r) return r;
+  if (out && cap_words > 0) {
+    const size_t n = std::min<size_t>((size_t)cap_words, (size_t)e->dec_grid * STAMP_WORDS);
+    r = copy_sync(e, out, e->dec_tstamp, n * 4, hipMemcpyDeviceToHost); if (r) return r;
   }
-  e->flow_host.d.tstamp = enable ? e->dec_tstamp : nullptr;
-  return copy_sync(e, e->flow_params, &e->flow_host, sizeof(FlowP), hipMemcpyHostToDevice);
+  e->stage_clock = enable != 0;
+  return SL_OK;
 }
+int sl_stage_clock_words(void) { return STAMP_WORDS; }
 int sl_profile_head(sl_engine* e, int enable) {
   int r = guard(e); if (r) return r;
   if (enable && e->head_ev.empty()) {

@@ -104,11 +104,19 @@ SL_DEV void stw4(rsrc_t r, int idx, uint32_t a, uint32_t b, uint32_t c, uint32_t
   __builtin_amdgcn_raw_buffer_store_b128(v, r, idx * 4, 0, CO_SC1);
 }
 
-// Diagnostic clock stamps (100 MHz) of workgroups 0 and 100: (clock << 16) | id << 8 | min(v, 255).
-SL_DEV void fstamp(const DecodeP& P, unsigned id, unsigned v) {
-  if (uni(P.tstamp) && threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == 100)) {
-    const int n = g_L.bar.nts;
-    if (n < 2040) { uni(P.tstamp)[(blockIdx.x ? 2048 : 0) + 1 + n] = ((unsigned long long)wall_clock64() << 16) | (id << 8) | (v > 255u ? 255u : v); g_L.bar.nts = n + 1; }
+// Diagnostic stage clock (kernel variant ST only): every workgroup keeps 100 MHz clock stamps of the last step
+// it ran in LDS, word (layer * 8 + stage) * STAMP_KINDS + kind, and copies them out when the launch ends.  Nothing
+// is stored to memory while the step runs, so the stamps do not disturb the polls they time.
+//   kind 0 stage entered, 1 poll satisfied, 2 prologue / preparation done, 3 arithmetic done (wave 0),
+//   4 results handed to the publishing wave's store, 5..7 stage specific.
+constexpr int STAMP_KINDS = 8;
+constexpr int STAMP_LAYERS = 41;                      // 40 layers and the head
+constexpr int STAMP_WORDS = STAMP_LAYERS * 8 * STAMP_KINDS;
+__shared__ uint32_t g_stamps[STAMP_WORDS];
+template <bool ST>
+SL_DEV void fstamp(int layer, int stage, int kind, bool who) {
+  if constexpr (ST) {
+    if (who && layer < STAMP_LAYERS) g_stamps[(layer * 8 + stage) * STAMP_KINDS + kind] = (uint32_t)wall_clock64();
   }
 }
 // One polling round's verdict for the whole workgroup: 1 = all tags present, 0 = retry, -1 = give up (spin
@@ -184,13 +192,13 @@ constexpr int PAIR_WAVE0 = 160 * DEC_WAVES;      // first wave of the shared gat
                  (void)tid; (void)lane; (void)wave; (void)wg; (void)G; (void)NW; (void)gw
 
 // Waves 0..7 poll a 2048-long tagged vector (4 words per thread); every thread then takes the pair it owns.
-SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, float& r0, float& r1, unsigned id) {
+template <bool ST>
+SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, float& r0, float& r1, int sl, int ss) {
   const int tid = fresh_v(threadIdx.x);
   uint32_t* rs = reinterpret_cast<uint32_t*>(g_L.part);       // [1024] packed pairs
   const rsrc_t rr = co_rsrc(vec);
   unsigned spins = 0;
   bool ok = tid >= 512;                         // a thread whose words have arrived does not fetch them again
-  fstamp(P, id, 0);
   for (;;) {
     if (tid < 512 && !ok) {
       const uint4 b = ldw4(rr, 4 * tid);
@@ -201,14 +209,17 @@ SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, fl
     if (v > 0) break;
     if (v < 0) return false;
   }
+  fstamp<ST>(sl, ss, 1, tid == 0);
   const uint32_t w = rs[tid];
   r0 = lo_h(w); r1 = hi_h(w);
   return true;
 }
 
 // ---- stage 1: input norm + in-projection ------------------------------------------------------------
+template <bool ST>
 SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base, float& h0, float& h1, int step) {
   FLOW_IDS;
+  fstamp<ST>(li, FS_IN, 0, tid == 0);
   const DecodeP& P = F.d;
   const int N = uni(Y.is_linear) ? SL_GDN_IN_N : SL_ATT_QKV_N;
   WRegs<1, 4> wr;
@@ -248,11 +259,13 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
     h0 = f16r(f16r(lo_h(sb) * q0) + hi_h(sb));
     h1 = f16r(f16r(lo_h(sb) * q1) + hi_h(sb));
   } else {
-    if (!poll_vec2048(P, uni(F.tmoe), flow_tag(base, li - 1, FS_C), r0, r1, 0)) return false;
+    if (!poll_vec2048<ST>(P, uni(F.tmoe), flow_tag(base, li - 1, FS_C), r0, r1, li, FS_IN)) return false;
   }
   const uint32_t tin = flow_tag(base, li, FS_IN);
   flow_prologue(h0, h1, li > 0, r0, r1, lnw, nullptr);
+  fstamp<ST>(li, FS_IN, 2, tid == 0);
   const F4 o = dot_1x4(wr);
+  fstamp<ST>(li, FS_IN, 3, tid == 0);
   if (lane == 0) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) g_L.pub[j * 16 + wave] = tagged(o.v[j], tin);
@@ -262,6 +275,7 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
     const int row = wg * DEC_WAVES + (lane & 15) + (lane >> 4) * NW;      // four runs of 16 consecutive rows
     if (row < N) stw1(co_rsrc(uni(F.tproj)), row, g_L.pub[lane]);
   }
+  fstamp<ST>(li, FS_IN, 4, tid == PUB_WAVE * 64);
   return true;
 }
 
@@ -269,8 +283,10 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
 // New conv-history samples of a thread's channel; written to memory by the next stage once its poll is over
 // (a store issued here would hold up that poll until it is acknowledged).
 struct GdnHist { uint32_t t12; uint32_t tnew; };
+template <bool ST>
 SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, GdnHist& gh) {
   FLOW_IDS;
+  fstamp<ST>(li, FS_CORE, 0, tid == 0);
   const DecodeP& P = F.d;
   Lds& L = g_L;
   if (wg >= 256) return true;
@@ -305,7 +321,6 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
     const uint32_t tin = flow_tag(base, li, FS_IN);
     const rsrc_t rp = co_rsrc(uni(F.tproj));
     unsigned spins = 0;
-    fstamp(P, 2, 0);
     for (;;) {
       bool ok = true;
       if (ch >= 0) { const uint32_t w = ldw1(rp, ch); ok = tag_ok(w, tin); newest = lo_h(w); }
@@ -313,7 +328,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
       if (v > 0) break;
       if (v < 0) return false;
     }
-    fstamp(P, 3, spins);
+    fstamp<ST>(li, FS_CORE, 1, tid == 0);
   }
   const float tap[3] = {h2f(traw[0]), h2f(traw[1]), h2f(traw[2])};
   if (tid < 272) {
@@ -340,6 +355,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
     buf[2 * lane] = y0; buf[2 * lane + 1] = y1;
   }
   __syncthreads();
+  fstamp<ST>(li, FS_CORE, 2, tid == 0);
   if (wave >= 8) {
     const float g = L.gb[0], beta = L.gb[1];
     const int dvl = (wave - 8) * 2 + half;
@@ -361,8 +377,10 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
   }
   gh.t12 = (uint32_t)traw[1] | ((uint32_t)traw[2] << 16);
   gh.tnew = f2h(newest);
+  fstamp<ST>(li, FS_CORE, 3, tid == 8 * 64);
   __syncthreads();
   if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tycore)), hv * 128 + dvb * 16 + lane, L.pub[lane]);
+  fstamp<ST>(li, FS_CORE, 4, tid == PUB_WAVE * 64);
   return true;
 }
 
@@ -375,8 +393,10 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
 #define SL_MERGE_WGS 32
 #endif
 constexpr int FLOW_MERGE_WGS = SL_MERGE_WGS;     // workgroups that merge the attention tiles: two or four per query head
+template <bool ST>
 SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base) {
   FLOW_IDS;
+  fstamp<ST>(li, FS_CORE, 0, tid == 0);
   const DecodeP& P = F.d;
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
@@ -434,7 +454,6 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
         {
           const rsrc_t rp = co_rsrc(uni(F.tproj));
           unsigned spins = 0;
-          fstamp(P, 4, 0);
           for (;;) {
             bool ok = true;
             if (wave < 10) { w4 = ldw4(rp, src + 4 * lane); ok = tag_ok(w4.x, tin) && tag_ok(w4.y, tin) && tag_ok(w4.z, tin) && tag_ok(w4.w, tin); }
@@ -442,7 +461,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
             if (v > 0) break;
             if (v < 0) return false;
           }
-          fstamp(P, 5, spins);
+          fstamp<ST>(li, FS_CORE, 1, tid == 0);
         }
         if (wave < 9) {
           const bool isq = wave < 8;
@@ -568,6 +587,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
     }
     __syncthreads();
   }
+  fstamp<ST>(li, FS_CORE, 4, tid == 0);
   return true;
 }
 
@@ -576,8 +596,10 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
 // the pair, slice of 32 dims) scores its slice; waves 0..3 = (head, half of the dims) accumulate the values, two dims per
 // lane.  The partial sums meet in the order of the undivided stage: 32-dim groups pairwise up to the halves of
 // the 256 dims, keys in sequence.  Only quarter 0 writes the new key and value rows to the cache.
+template <bool ST>
 SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base) {
   FLOW_IDS;
+  fstamp<ST>(li, FS_CORE, 0, tid == 0);
   const DecodeP& P = F.d;
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
@@ -618,7 +640,6 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
   {
     const rsrc_t rp = co_rsrc(uni(F.tproj));
     unsigned spins = 0;
-    fstamp(P, 4, 0);
     for (;;) {
       bool ok = true;
       if (fetches) { w4 = ldw4(rp, src + 4 * lane); ok = tag_ok(w4.x, tin) && tag_ok(w4.y, tin) && tag_ok(w4.z, tin) && tag_ok(w4.w, tin); }
@@ -626,7 +647,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
       if (v > 0) break;
       if (v < 0) return false;
     }
-    fstamp(P, 5, spins);
+    fstamp<ST>(li, FS_CORE, 1, tid == 0);
   }
   if (wave < 2 || wave == 8) {
     const bool isq = wave < 2;
@@ -728,6 +749,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
     stw4(co_rsrc(uni(F.tpo)), ((head * uni(P.max_tiles) + tile) * 128 + 64 * half + lane) * 4, __float_as_uint(o0), __float_as_uint(o1),
          tcore, tcore);
   }
+  fstamp<ST>(li, FS_CORE, 4, tid == 0);
   __syncthreads();
   return true;
 }
@@ -749,8 +771,10 @@ SL_DEV void store_hist(const LayerP& Y, int li, const GdnHist& gh) {
 }
 
 // ---- K = 4096 projection (GDN out_proj with gated rmsnorm prologue / attention merge + o_proj) ---------
+template <bool ST>
 SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t base, const GdnHist& gh) {
   FLOW_IDS;
+  fstamp<ST>(li, FS_OUT, 0, tid == 0);
   const DecodeP& P = F.d;
   const bool lin = uni(Y.is_linear) != 0;
   const float NEG = -__int_as_float(0x7f800000);
@@ -889,6 +913,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
       const uint32_t r1 = tagged(f16r(f16r(O1 / Ls) * sigmoid16(lo_h(g2.y))), tmerge);
       stw2(co_rsrc(uni(F.tycore)), h * 256 + 2 * chunk, r0, r1);
     }
+    fstamp<ST>(li, FS_MERGE, 4, tid == 0);
   }
   if (wg * DEC_WAVES >= H) {                       // no output row here (uniform per workgroup): nothing to fetch
     if (lin) store_hist(Y, li, gh);
@@ -905,7 +930,6 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     uint4 a = make_uint4(0, 0, 0, 0), b = make_uint4(0, 0, 0, 0);
     bool zdone = false, y1done = false, y2done = false;   // what has arrived is not fetched again
     unsigned spins = 0;
-    fstamp(P, 6, 0);
     for (;;) {
       bool ok = true;
       if (wave < 8) {
@@ -937,7 +961,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
       if (v > 0) break;
       if (v < 0) return false;
     }
-    fstamp(P, 7, spins);
+    fstamp<ST>(li, FS_OUT, 1, tid == 0);
     if (wave >= 8) {
       a = ystage[tid - 512];
       if (lin) { b = ystage[tid]; sz[0] = __uint_as_float(b.x); sz[1] = __uint_as_float(b.y); sz[2] = __uint_as_float(b.z); sz[3] = __uint_as_float(b.w); }
@@ -972,11 +996,14 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     if (lane & 1) g_L.sxs[(4 * b + (i0 >> 3)) * 64 + lo] = srest;
   }
   __syncthreads();
+  fstamp<ST>(li, FS_OUT, 2, tid == 0);
   const float o = dot_2x1(wr);
+  fstamp<ST>(li, FS_OUT, 3, tid == 0);
   if (wg * DEC_WAVES < H) {                       // uniform per workgroup
     if (lane == 0) g_L.pub[wave] = tagged(o, flow_tag(base, li, FS_OUT));
     __syncthreads();
     if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tmix)), wg * DEC_WAVES + lane, g_L.pub[lane]);
+    fstamp<ST>(li, FS_OUT, 4, tid == PUB_WAVE * 64);
   }
   return true;
 }
@@ -984,9 +1011,10 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
 // ---- MoE stage A -------------------------------------------------------------------------------------
 // GATE8: the router and shared-gate rows are 8-bit affine rows instead of fp16 (a compile-time variant, so that
 // the fp16 configuration carries none of its registers or branches).
-template <bool GATE8>
+template <bool GATE8, bool ST>
 SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, float& h0, float& h1) {
   FLOW_IDS;
+  fstamp<ST>(li, FS_A, 0, tid == 0);
   const DecodeP& P = F.d;
   // The router rows, the shared-gate row and the shared gate/up pairs sit on workgroups of the upper half
   // of the grid: those have no row of the K = 4096 projection, reach this stage early and so have their
@@ -1012,9 +1040,10 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
   }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.post_ln) + 2 * tid);
   float r0, r1;
-  if (!poll_vec2048(P, uni(F.tmix), flow_tag(base, li, FS_OUT), r0, r1, 8)) return false;
+  if (!poll_vec2048<ST>(P, uni(F.tmix), flow_tag(base, li, FS_OUT), r0, r1, li, FS_A)) return false;
   const uint32_t ta = flow_tag(base, li, FS_A);
   flow_prologue(h0, h1, true, r0, r1, lnw, nullptr);
+  fstamp<ST>(li, FS_A, 2, tid == 0);
   if (is_dense) {
     uint32_t xp[16]; float sx[4];
     lds_get_x(0, lane, xp, sx);
@@ -1050,6 +1079,7 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
           stw1(co_rsrc(uni(F.tsh)), p0 + lane, g_L.pub[lane]);
         }
       }
+      fstamp<ST>(li, FS_A, 4, tid == PUB_WAVE * 64);
     }
   }
   return true;
@@ -1063,8 +1093,10 @@ SL_DEV uint32_t route_key(uint32_t hbits, int e) {
   u = (u & 0x8000u) ? (~u & 0xffffu) : (u | 0x8000u);
   return (u << 8) | (uint32_t)(255 - e);
 }
+template <bool ST>
 SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   FLOW_IDS;
+  fstamp<ST>(li, FS_B, 0, tid == 0);
   const DecodeP& P = F.d;
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
@@ -1076,7 +1108,6 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     const rsrc_t rl = co_rsrc(uni(F.trlog));
     const int E = uni(P.E);
     unsigned spins = 0;
-    fstamp(P, 10, 0);
     for (;;) {
       bool ok = true;
       float v0 = NEG;
@@ -1087,7 +1118,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
       if (v > 0) break;
       if (v < 0) return false;
     }
-    fstamp(P, 11, spins);
+    fstamp<ST>(li, FS_B, 1, tid == 0);
   }
   // Wave 0 picks the 8 largest keys in order (max, remove, repeat; the wave-wide max is a DPP reduction plus
   // one lane per row); wave 1 forms the softmax sums meanwhile.
@@ -1119,6 +1150,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     if (lane == 0) L.gb[0] = Z;
   }
   __syncthreads();
+  fstamp<ST>(li, FS_B, 2, tid == 0);
   // (the renormalised scores are only needed by the combine of the next stage and are formed there, off this
   // stage's path: exp values, sum and indices stay in LDS)
   // this wave's gate/up pair, requested as soon as the indices are known
@@ -1134,10 +1166,12 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   }
   if (active) {
     const F2 gu = dot_1x2(wr);
+    fstamp<ST>(li, FS_B, 3, tid == 0);
     if (lane == 0) L.pub[wave] = tagged(swiglu16(f16r(gu.v[0]), f16r(gu.v[1])), flow_tag(base, li, FS_B));
   }
   __syncthreads();
   if (wave == PUB_WAVE && lane < 16 && wg * DEC_WAVES + lane < 8 * 512) stw1(co_rsrc(uni(F.tact)), wg * DEC_WAVES + lane, L.pub[lane]);
+  fstamp<ST>(li, FS_B, 4, tid == PUB_WAVE * 64);
   return true;
 }
 
@@ -1145,8 +1179,10 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
 // Units (quad of 4 outputs, slot): slots 0..7 routed experts, slot 8 shared; 2 quads per workgroup.  The nine
 // activation rows are fetched once per workgroup into LDS (packed pairs, 20-word stride per 32 elements).
 constexpr int XC_STRIDE = 20;
+template <bool ST>
 SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   FLOW_IDS;
+  fstamp<ST>(li, FS_C, 0, tid == 0);
   const DecodeP& P = F.d;
   Lds& L = g_L;
   uint32_t* xc = reinterpret_cast<uint32_t*>(g_vt);      // [9][16][XC_STRIDE]
@@ -1185,7 +1221,6 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     const rsrc_t ra = co_rsrc(uni(F.tact)), rs = co_rsrc(uni(F.tsh)), rg = co_rsrc(uni(F.tsg));
     unsigned spins = 0;
     bool have[3] = {false, false, false};         // a chunk that has arrived is not fetched again
-    fstamp(P, 12, 0);
     for (;;) {
       bool ok = true;
       if (wave < 6) {
@@ -1207,7 +1242,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
       if (v > 0) break;
       if (v < 0) return false;
     }
-    fstamp(P, 13, spins);
+    fstamp<ST>(li, FS_C, 1, tid == 0);
   }
 #pragma unroll
   for (int qq = 0; qq < 2; ++qq) {
@@ -1229,6 +1264,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
       if (li16 == 0) L.dbuf[(ql * 9 + slot) * 4 + sub] = f16r(d);
     }
   }
+  fstamp<ST>(li, FS_C, 3, tid == 6 * 64);
   __syncthreads();
   if (wave == PUB_WAVE && lane < 8) {
     const int ql = lane >> 2, sb4 = lane & 3;
@@ -1239,11 +1275,13 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     const float s = sigmoid16(L.gb[1]);
     stw1(co_rsrc(uni(F.tmoe)), quad * 4 + sb4, tagged(f16r(acc + f16r(s * L.dbuf[(ql * 9 + 8) * 4 + sb4])), flow_tag(base, li, FS_C)));
   }
+  fstamp<ST>(li, FS_C, 4, tid == PUB_WAVE * 64);
   __syncthreads();
   return true;
 }
 
 // ---- head -------------------------------------------------------------------------------------------
+template <bool ST>
 SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t base, float h0, float h1, bool hand_on) {
   FLOW_IDS;
   const DecodeP& P = F.d;
@@ -1264,7 +1302,8 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
   load_group(cur, gw, 0);
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(P.final_norm) + 2 * tid);
   float r0, r1;
-  if (!poll_vec2048(P, uni(F.tmoe), flow_tag(base, nl - 1, FS_C), r0, r1, 14)) return false;
+  fstamp<ST>(nl, 0, 0, tid == 0);
+  if (!poll_vec2048<ST>(P, uni(F.tmoe), flow_tag(base, nl - 1, FS_C), r0, r1, nl, 0)) return false;
   const uint32_t thd32 = flow_tag32(base, nl, 0);
   flow_prologue(h0, h1, true, r0, r1, lnw, wg == 0 ? uni(P.normed) : nullptr);
   for (int chunk = gw; chunk < nchunks; chunk += NW) {
@@ -1286,6 +1325,7 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
       cur = nxt;
     }
   }
+  fstamp<ST>(nl, 0, 3, tid == 0);
   if (lane == 0) { L.red[wave] = bv; L.ired[wave] = bi; }
   __syncthreads();
   if (wave == PUB_WAVE && lane == 0) {
@@ -1299,7 +1339,6 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
   {
     const rsrc_t rc = co_rsrc(uni(F.tcand));
     unsigned spins = 0;
-    fstamp(P, 16, 0);
     for (;;) {
       bool ok = true;
       if (tid < G) { const uint4 c = ldw4(rc, tid * 4); ok = c.z == thd32 && c.w == thd32; v = __uint_as_float(c.x); i = (int)c.y; }
@@ -1307,7 +1346,7 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
       if (r > 0) break;
       if (r < 0) return false;
     }
-    fstamp(P, 17, spins);
+    fstamp<ST>(nl, 1, 1, tid == 0);
   }
 #pragma unroll
   for (int msk = 1; msk < 64; msk <<= 1) {
@@ -1326,6 +1365,7 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
     const uint32_t nbase = base + (uint32_t)(nl + 1) * 8u;
     st_co32(uni(P.bar) + 16, nbase);
     if (hand_on) { const uint32_t ttag = flow_tag32(nbase, 0, 7); stw4(co_rsrc(uni(F.ttok)), 0, (uint32_t)i, (uint32_t)i, ttag, ttag); }
+    fstamp<ST>(nl, 1, 4, true);
   }
   for (int l = tid; l < nl; l += DEC_THREADS) uni(P.st)[1 + l] ^= 1;
   return true;
@@ -1334,7 +1374,7 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
 // ---- the kernel: hA already holds the embedded token row (k_embed) --------------------------------------
 // `steps` tokens per launch (a chain feeds each token back on the device): between two steps workgroup 0 hands the
 // new token to everybody as a tagged word, which costs one hand-over instead of a kernel boundary.
-template <bool GATE8>
+template <bool GATE8, bool ST>
 __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __restrict__ Fp, int out_off, int feed, int steps) {
   {
     const int tid = threadIdx.x;
@@ -1349,9 +1389,10 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
       const int bit = (tid < nl) ? (Fp->d.st[1 + tid] & 1) : 0;
       const unsigned long long m = __ballot(bit);
       const unsigned long long lm = __ballot((tid < nl) ? (Fp->d.layers[tid].is_linear != 0) : 0);
-      if (tid == 0) { g_K.parity = m; g_K.linmask = lm; g_K.pos = Fp->d.st[0]; g_K.base = ld_co32(Fp->d.bar + 16); g_K.tok = 0; g_L.bar.nts = 0; }
+      if (tid == 0) { g_K.parity = m; g_K.linmask = lm; g_K.pos = Fp->d.st[0]; g_K.base = ld_co32(Fp->d.bar + 16); g_K.tok = 0; }
       if (tid < 4) g_L.pf[tid] = 0;
     }
+    if constexpr (ST) for (int i = tid; i < STAMP_WORDS; i += DEC_THREADS) g_stamps[i] = 0;
     __syncthreads();
   }
   const FlowP& F = g_K.F;
@@ -1364,29 +1405,31 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
     for (int li = 0; li < nl; ++li) {
       const LayerP& Y = g_K.layers[li];
       const int is_linear = uni(Y.is_linear);
-      if (!flow_in(F, Y, li, pos, base, h0, h1, step)) return;
+      if (!flow_in<ST>(F, Y, li, pos, base, h0, h1, step)) return;
       GdnHist gh = {0u, 0u};
       if (is_linear) {
-        if (!flow_gdn(F, Y, li, base, gh)) return;
-        if (!flow_out(F, Y, li, 0, base, gh)) return;
+        if (!flow_gdn<ST>(F, Y, li, base, gh)) return;
+        if (!flow_out<ST>(F, Y, li, 0, base, gh)) return;
       } else {
-        if (((pos + SDPA_TILE) / SDPA_TILE) * SL_ATT_KV * 4 <= (int)gridDim.x ? !flow_sdpa4(F, Y, li, pos, base) : !flow_sdpa(F, Y, li, pos, base)) return;
-        if (!flow_out(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh)) return;
+        if (((pos + SDPA_TILE) / SDPA_TILE) * SL_ATT_KV * 4 <= (int)gridDim.x ? !flow_sdpa4<ST>(F, Y, li, pos, base) : !flow_sdpa<ST>(F, Y, li, pos, base)) return;
+        if (!flow_out<ST>(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh)) return;
       }
-      if (!flow_moe_a<GATE8>(F, Y, li, base, h0, h1)) return;
-      if (!flow_moe_b(F, Y, li, base)) return;
-      if (!flow_moe_c(F, Y, li, base)) return;
+      if (!flow_moe_a<GATE8, ST>(F, Y, li, base, h0, h1)) return;
+      if (!flow_moe_b<ST>(F, Y, li, base)) return;
+      if (!flow_moe_c<ST>(F, Y, li, base)) return;
     }
-    if (!flow_head(F, pos, out_off + step, feed, base, h0, h1, step + 1 < steps)) return;
+    if (!flow_head<ST>(F, pos, out_off + step, feed, base, h0, h1, step + 1 < steps)) return;
     if (step + 1 < steps) {
       __syncthreads();                   // everybody has read this step's position, tag base and parities
       if (threadIdx.x == 0) { g_K.pos = pos + 1; g_K.base = base + (uint32_t)(nl + 1) * 8u; g_K.parity ^= g_K.linmask; }
       __syncthreads();
     }
   }
-  fstamp(P, 18, 0);
-  if (uni(P.tstamp) && threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == 100))
-    uni(P.tstamp)[blockIdx.x ? 2048 : 0] = (unsigned long long)g_L.bar.nts;
+  if constexpr (ST) {
+    __syncthreads();
+    uint32_t* dst = uni(P.tstamp) + (size_t)blockIdx.x * STAMP_WORDS;
+    for (int i = threadIdx.x; i < STAMP_WORDS; i += DEC_THREADS) dst[i] = g_stamps[i];
+  }
 }
 
 }  // namespace sl
