@@ -168,6 +168,10 @@ SL_DEV float tree_max(float v) {
 // Value of the previous lane (lanes 0, 16, 32, 48 get 0): for left-to-right chains inside a 16-lane row.
 SL_DEV float prev_lane(float v) { return dpp_f<DPP_SHR1>(v); }
 
+// Workgroup barrier for data exchanged through LDS: waits for the wave's LDS operations only.  __syncthreads() also
+// waits for every vector-memory load in flight, which would drain weight rows requested ahead of their use.
+SL_DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // ---- 16-byte vector access -------------------------------------------------------------------------
 SL_DEV uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
 SL_DEV void st16(void* p, uint4 v) { *reinterpret_cast<uint4*>(p) = v; }

@@ -131,7 +131,7 @@ SL_DEV int flow_round(bool ok, unsigned& spins, unsigned* abort_word) {
     st_co32(abort_word, 1u);
     g_L.pf[3] = 1;
   }
-  __syncthreads();
+  lds_barrier();
   const int failed = g_L.pf[slot], dead = g_L.pf[3];
   if (threadIdx.x == 0) g_L.pf[(spins + 2u) % 3u] = 0;
   if (dead) return -1;
@@ -150,7 +150,7 @@ SL_DEV void flow_prologue(float& h0, float& h1, bool has_r, float r0, float r1, 
   uint32_t* hs = reinterpret_cast<uint32_t*>(g_L.sq);          // 1024 words of scratch (attention's query area)
   if (has_r) { h0 = f16r(h0 + r0); h1 = f16r(h1 + r1); }
   hs[tid + (tid >> 4)] = pack2(h0, h1);       // 17-word lane stride: conflict-free for the chain below
-  __syncthreads();
+  lds_barrier();
   if (wave == 0) {
     float ss = 0.0f;
 #pragma unroll
@@ -163,7 +163,7 @@ SL_DEV void flow_prologue(float& h0, float& h1, bool has_r, float r0, float r1, 
     ss = tree_sum<64>(ss);
     if (lane == 0) g_L.gb[0] = 1.0f / sqrtf(ss / 2048.0f + EPS);
   }
-  __syncthreads();
+  lds_barrier();
   const float inv = g_L.gb[0];
   const float y0 = f16r(lo_h(lnw_pair) * f16r(h0 * inv)), y1 = f16r(hi_h(lnw_pair) * f16r(h1 * inv));
   g_L.xs[(tid & 15) * 64 + (tid >> 4)] = pack2(y0, y1);
@@ -177,7 +177,7 @@ SL_DEV void flow_prologue(float& h0, float& h1, bool has_r, float r0, float r1, 
   }
   if (q == 3) g_L.sxs[((tid & 15) >> 2) * 64 + (tid >> 4)] = s;
   if (xn_plain) *reinterpret_cast<uint32_t*>(xn_plain + 2 * tid) = pack2(y0, y1);
-  __syncthreads();
+  lds_barrier();
 }
 
 // Stores of a wave are acknowledged in order with its loads, so a wave that has just published results cannot
@@ -216,21 +216,44 @@ SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, fl
 }
 
 // ---- stage 1: input norm + in-projection ------------------------------------------------------------
+// The rows of the in-projection are not equally urgent.  What the next stage waits for (GDN: q, k, v and the
+// two gate logits rows, 8256 of 12352; attention: the query halves, k and v, 5120 of 9216) is computed and
+// published first; the rows that are only read a stage later (GDN: z; attention: the output gates; 4096 either
+// way, one per wave) follow while the first batch is on its way to its consumers, and their weights are only
+// requested once this stage's own inputs have arrived, so they stream during the arithmetic.
+//   GDN: workgroup wg owns rows 32 wg .. 32 wg + 31 (wave w: two of them) and every fourth workgroup one of the
+//        64 b / a rows (wave 0); deferred row 8192 + 16 wg + w.
+//   attention: urgent index c = 20 wg + slot, slot = 2w, 2w + 1 on waves 0..3 and 4 + w on the others;
+//        c < 4096 is query element c % 256 of head c / 256, then k and v; deferred: gate element of the same numbering.
+struct InRows { int crit[3]; int ncrit; int def; };
+SL_DEV int attn_urgent_row(int c) { return c < 4096 ? ((c >> 8) * 512 + (c & 255)) : (8192 + (c - 4096)); }
+SL_DEV int attn_gate_row(int zi) { return (zi >> 8) * 512 + 256 + (zi & 255); }
+SL_DEV InRows in_rows(bool lin, int wg, int wave) {
+  InRows r;
+  if (lin) {
+    const bool extra = wave == 0 && (wg & 3) == 0;
+    r.crit[0] = wg * 32 + wave * 2; r.crit[1] = r.crit[0] + 1; r.crit[2] = extra ? 12288 + (wg >> 2) : 0;
+    r.ncrit = extra ? 3 : 2;
+    r.def = 8192 + wg * 16 + wave;
+  } else {
+    const int c0 = wg * 20 + (wave < 4 ? 2 * wave : 4 + wave);
+    r.ncrit = wave < 4 ? 2 : 1;
+    r.crit[0] = attn_urgent_row(c0); r.crit[1] = wave < 4 ? attn_urgent_row(c0 + 1) : 0; r.crit[2] = 0;
+    r.def = attn_gate_row(wg * 16 + wave);
+  }
+  return r;
+}
 template <bool ST>
 SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base, float& h0, float& h1, int step) {
   FLOW_IDS;
   fstamp<ST>(li, FS_IN, 0, tid == 0);
   const DecodeP& P = F.d;
-  const int N = uni(Y.is_linear) ? SL_GDN_IN_N : SL_ATT_QKV_N;
-  WRegs<1, 4> wr;
-  bool valid[4];
+  const bool lin = uni(Y.is_linear) != 0;
+  const InRows rows = in_rows(lin, wg, wave);
+  WRegs<1, 3> wr;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    valid[j] = gw + j * NW < N;
-    wload_row<1>(wr.w[j], wr.sb[j], uni(Y.in_w), uni(Y.in_sb), (size_t)(valid[j] ? gw + j * NW : 0), valid[j], lane);
-  }
+  for (int j = 0; j < 3; ++j) wload_row<1>(wr.w[j], wr.sb[j], uni(Y.in_w), uni(Y.in_sb), (size_t)rows.crit[j], j < rows.ncrit, lane);
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.input_ln) + 2 * tid);
-  // first touches of the next stage: this workgroup's recurrent-state rows, or its key/value tile
   float r0 = 0.0f, r1 = 0.0f;
   if (li == 0) {
     // the token's embedding row, dequantised in half arithmetic: half(half(s * q) + b) (embed_rows_q4,
@@ -261,21 +284,50 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   } else {
     if (!poll_vec2048<ST>(P, uni(F.tmoe), flow_tag(base, li - 1, FS_C), r0, r1, li, FS_IN)) return false;
   }
+  // the deferred row (no branch around the load: the waits that follow stay exact)
+  uint4 wd; uint32_t sbd;
+  wload_row<1>(&wd, &sbd, uni(Y.in_w), uni(Y.in_sb), (size_t)rows.def, true, lane);
   const uint32_t tin = flow_tag(base, li, FS_IN);
   flow_prologue(h0, h1, li > 0, r0, r1, lnw, nullptr);
   fstamp<ST>(li, FS_IN, 2, tid == 0);
-  const F4 o = dot_1x4(wr);
-  fstamp<ST>(li, FS_IN, 3, tid == 0);
-  if (lane == 0) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) g_L.pub[j * 16 + wave] = tagged(o.v[j], tin);
+  uint32_t x[16]; float sx[4];
+  lds_get_x(0, lane, x, sx);
+  {
+    // urgent rows: slot of row j = first slot of the wave + j (the extra b / a row: slot 32)
+    const int slot0 = lin ? 2 * wave : (wave < 4 ? 2 * wave : 4 + wave);
+    const float o0 = tree_sum<64>(quad_term(wr.w[0][0], wr.sb[0][0], x, sx));
+    if (lane == 0) g_L.pub[slot0] = tagged(o0, tin);
+    if (rows.ncrit >= 2) {                // wave-uniform
+      const float o1 = tree_sum<64>(quad_term(wr.w[1][0], wr.sb[1][0], x, sx));
+      if (lane == 0) g_L.pub[slot0 + 1] = tagged(o1, tin);
+    }
+    if (rows.ncrit >= 3) {
+      const float o2 = tree_sum<64>(quad_term(wr.w[2][0], wr.sb[2][0], x, sx));
+      if (lane == 0) g_L.pub[32] = tagged(o2, tin);
+    }
   }
-  __syncthreads();
+  fstamp<ST>(li, FS_IN, 3, tid == 0);
+  lds_barrier();
   if (wave == PUB_WAVE) {
-    const int row = wg * DEC_WAVES + (lane & 15) + (lane >> 4) * NW;      // four runs of 16 consecutive rows
-    if (row < N) stw1(co_rsrc(uni(F.tproj)), row, g_L.pub[lane]);
+    const rsrc_t rp = co_rsrc(uni(F.tproj));
+    if (lin) {
+      if (lane < 32) stw1(rp, wg * 32 + lane, g_L.pub[lane]);
+      else if (lane == 32 && (wg & 3) == 0) stw1(rp, 12288 + (wg >> 2), g_L.pub[32]);
+    } else if (lane < 20) {
+      stw1(rp, attn_urgent_row(wg * 20 + lane), g_L.pub[lane]);
+    }
   }
   fstamp<ST>(li, FS_IN, 4, tid == PUB_WAVE * 64);
+  {
+    const float od = tree_sum<64>(quad_term(wd, sbd, x, sx));
+    if (lane == 0) g_L.pub[40 + wave] = tagged(od, tin);
+  }
+  lds_barrier();
+  if (wave == PUB_WAVE && lane < 16) {
+    const int zi = wg * 16 + lane;
+    stw1(co_rsrc(uni(F.tproj)), lin ? 8192 + zi : attn_gate_row(zi), g_L.pub[40 + lane]);
+  }
+  fstamp<ST>(li, FS_IN, 5, tid == PUB_WAVE * 64);
   return true;
 }
 
@@ -343,7 +395,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
   } else if (tid == 273) {
     L.gb[0] = exp_c(-(exp_c(uni(Y.a_log)[hv]) * softplus_c(newest + uni(Y.dt_bias)[hv])));
   }
-  __syncthreads();
+  lds_barrier();
   if (wave < 2) {
     float* buf = wave ? L.k : L.q;
     const float x0 = buf[2 * lane], x1 = buf[2 * lane + 1];
@@ -354,7 +406,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
     const float y0 = f16r(sc * f16r(x0 * inv)), y1 = f16r(sc * f16r(x1 * inv));
     buf[2 * lane] = y0; buf[2 * lane + 1] = y1;
   }
-  __syncthreads();
+  lds_barrier();
   fstamp<ST>(li, FS_CORE, 2, tid == 0);
   if (wave >= 8) {
     const float g = L.gb[0], beta = L.gb[1];
@@ -378,7 +430,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
   gh.t12 = (uint32_t)traw[1] | ((uint32_t)traw[2] << 16);
   gh.tnew = f2h(newest);
   fstamp<ST>(li, FS_CORE, 3, tid == 8 * 64);
-  __syncthreads();
+  lds_barrier();
   if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tycore)), hv * 128 + dvb * 16 + lane, L.pub[lane]);
   fstamp<ST>(li, FS_CORE, 4, tid == PUB_WAVE * 64);
   return true;
@@ -445,7 +497,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       const int tile = u >> 1, kvh = u & 1;
       const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
       const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
-      __syncthreads();                    // the key tile aliases the activation vector the in-projection just read
+      lds_barrier();                    // the key tile aliases the activation vector the in-projection just read
       stage(true, r == 0, u);
       // waves 0..7: query heads of the group; wave 8: new key; wave 9: new value -- 4 tagged words per lane
       const int src = wave < 8 ? (kvh * 8 + wave) * 512 : (wave == 8 ? 8192 + kvh * 256 : 8192 + 512 + kvh * 256);
@@ -504,7 +556,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
         st_co_h4(co_rsrc(uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 4 * lane, o);
         *reinterpret_cast<uint2*>(&L.kt[(pos - j0) * KT_STRIDE + 4 * lane]) = make_uint2(pack2(o[0], o[1]), pack2(o[2], o[3]));
       }
-      __syncthreads();
+      lds_barrier();
       {
         // scores: wave (head, half) takes the 32 leaves of its half of the 256 dims, lane j is key j.  The 128
         // query values sit two per lane and reach the multiply as scalar operands (readlane), so LDS only
@@ -531,7 +583,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
         }
         L.part[wave * 64 + lane] = (g[0] + g[1]) + (g[2] + g[3]);
       }
-      __syncthreads();
+      lds_barrier();
       if ((wave & 1) == 0) {
         const int h = wave >> 1;
         const float dotv = L.part[wave * 64 + lane] + L.part[(wave + 1) * 64 + lane];
@@ -550,14 +602,14 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       const int tile = u >> 1, kvh = u & 1;
       const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
       const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
-      __syncthreads();                    // the previous unit's value tile has been read; the weights are in place
+      lds_barrier();                    // the previous unit's value tile has been read; the weights are in place
       if (r > 0) stage(false, true, u);
       if (has_new && wave == 9) {
         const uint32_t a = vn[kvh * 128 + 2 * lane], b = vn[kvh * 128 + 2 * lane + 1];
         stw2(co_rsrc(uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 2 * lane, a, b);
         *reinterpret_cast<uint2*>(&g_vt[(pos - j0) * 256 + 4 * lane]) = make_uint2(a, b);
       }
-      __syncthreads();
+      lds_barrier();
       const int h = wave >> 1, half = wave & 1;
       float o0 = 0.0f, o1 = 0.0f;
       const uint16_t* vt = &g_vt[128 * half + 2 * lane];
@@ -585,7 +637,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       const int head = kvh * 8 + h;
       stw4(co_rsrc(uni(F.tpo)), ((head * uni(P.max_tiles) + tile) * 128 + 64 * half + lane) * 4, __float_as_uint(o0), __float_as_uint(o1), tcore, tcore);
     }
-    __syncthreads();
+    lds_barrier();
   }
   fstamp<ST>(li, FS_CORE, 4, tid == 0);
   return true;
@@ -611,7 +663,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
   const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
   const uint16_t* kbase = uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + j0) * 256;
   const uint16_t* vbase = uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + j0) * 256;
-  __syncthreads();                    // the key tile aliases the activation vector the in-projection just read
+  lds_barrier();                    // the key tile aliases the activation vector the in-projection just read
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
     const int row = it * 32 + (tid >> 5), c8 = (tid & 31) * 8;
@@ -685,7 +737,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
     if (hq == 0) stw2(co_rsrc(uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 2 * lane, a, b);
     *reinterpret_cast<uint2*>(&g_vt[(pos - j0) * 256 + 4 * lane]) = make_uint2(a, b);
   }
-  __syncthreads();
+  lds_barrier();
   {
     // scores: wave (head, slice) takes the 8 leaves of its 32 dims, lane j is key j; the 32 query values sit one
     // per lane (lanes 0..31) and reach the multiply as scalar operands
@@ -704,7 +756,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
     }
     L.part[wave * 64 + lane] = ((n[0] + n[1]) + (n[2] + n[3])) + ((n[4] + n[5]) + (n[6] + n[7]));
   }
-  __syncthreads();
+  lds_barrier();
   if ((wave & 7) == 0) {
     const int hh = wave >> 3;
     const float* pp = &L.part[hh * 512 + lane];
@@ -717,7 +769,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
     const int head = kvh * 8 + hq * 2 + hh;
     if (lane == 0) stw4(co_rsrc(uni(F.tml)), (head * uni(P.max_tiles) + tile) * 4, __float_as_uint(mx), __float_as_uint(l), tcore, tcore);
   }
-  __syncthreads();
+  lds_barrier();
   if (wave < 4) {
     // values: wave (head, half of the dims), two dims per lane (one LDS word per key); the weight of key j is
     // handed out by readlane.  Eight LDS reads are issued together, then used in key order.
@@ -750,7 +802,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
          tcore, tcore);
   }
   fstamp<ST>(li, FS_CORE, 4, tid == 0);
-  __syncthreads();
+  lds_barrier();
   return true;
 }
 
@@ -860,7 +912,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     }
     if (nt > MB) {                                          // uniform for the grid
       uint2* park = reinterpret_cast<uint2*>(g_vt);         // [64 tiles][64 lanes] {o0, o1}
-      __syncthreads();                                      // tile units this workgroup may have had are done with the space
+      lds_barrier();                                      // tile units this workgroup may have had are done with the space
       for (int t0 = 0; t0 < nt; t0 += 64) {
         uint4 q[4];
         // wave 0, lane i: {max, sum} of tile t0 + i (its tags were verified above), fetched in the shadow of the poll
@@ -883,7 +935,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
           const int t = t0 + 4 * wave + j;
           if (t >= MB && t < nt && act) park[(4 * wave + j) * 64 + lane] = make_uint2(q[j].x, q[j].y);
         }
-        __syncthreads();
+        lds_barrier();
         if (wave == 0 && !fail) {
           float fl = 0.0f, pl = 0.0f;                       // lane i: scale and sum of tile t0+i
           if (t0 + lane < nt) { fl = exp_c(__uint_as_float(ma.x) - Mx); pl = __uint_as_float(ma.y); }
@@ -904,7 +956,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
             }
           }
         }
-        __syncthreads();                                    // the block is consumed before the next one is parked
+        lds_barrier();                                    // the block is consumed before the next one is parked
       }
     }
     if (fail) st_co32(uni(P.bar) + 32, 1u);
@@ -995,13 +1047,13 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     for (int i = 0; i < 4; ++i) srest = srest + out[i];
     if (lane & 1) g_L.sxs[(4 * b + (i0 >> 3)) * 64 + lo] = srest;
   }
-  __syncthreads();
+  lds_barrier();
   fstamp<ST>(li, FS_OUT, 2, tid == 0);
   const float o = dot_2x1(wr);
   fstamp<ST>(li, FS_OUT, 3, tid == 0);
   if (wg * DEC_WAVES < H) {                       // uniform per workgroup
     if (lane == 0) g_L.pub[wave] = tagged(o, flow_tag(base, li, FS_OUT));
-    __syncthreads();
+    lds_barrier();
     if (wave == PUB_WAVE && lane < 16) stw1(co_rsrc(uni(F.tmix)), wg * DEC_WAVES + lane, g_L.pub[lane]);
     fstamp<ST>(li, FS_OUT, 4, tid == PUB_WAVE * 64);
   }
@@ -1069,7 +1121,7 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
   {
     const int d0 = wg * DEC_WAVES - DENSE_WAVE0, p0 = wg * DEC_WAVES - PAIR_WAVE0, E = uni(P.E);
     if ((d0 >= 0 && d0 <= E) || (p0 >= 0 && p0 < 512)) {     // uniform per workgroup: it holds router rows, the gate row or pairs
-      __syncthreads();
+      lds_barrier();
       if (wave == PUB_WAVE && lane < 16) {
         if (d0 >= 0 && d0 <= E) {
           const int g = d0 + lane;
@@ -1149,7 +1201,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     const float Z = tree_sum<64>(((x4[0] + x4[1]) + x4[2]) + x4[3]);
     if (lane == 0) L.gb[0] = Z;
   }
-  __syncthreads();
+  lds_barrier();
   fstamp<ST>(li, FS_B, 2, tid == 0);
   // (the renormalised scores are only needed by the combine of the next stage and are formed there, off this
   // stage's path: exp values, sum and indices stay in LDS)
@@ -1169,7 +1221,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     fstamp<ST>(li, FS_B, 3, tid == 0);
     if (lane == 0) L.pub[wave] = tagged(swiglu16(f16r(gu.v[0]), f16r(gu.v[1])), flow_tag(base, li, FS_B));
   }
-  __syncthreads();
+  lds_barrier();
   if (wave == PUB_WAVE && lane < 16 && wg * DEC_WAVES + lane < 8 * 512) stw1(co_rsrc(uni(F.tact)), wg * DEC_WAVES + lane, L.pub[lane]);
   fstamp<ST>(li, FS_B, 4, tid == PUB_WAVE * 64);
   return true;
@@ -1265,7 +1317,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     }
   }
   fstamp<ST>(li, FS_C, 3, tid == 6 * 64);
-  __syncthreads();
+  lds_barrier();
   if (wave == PUB_WAVE && lane < 8) {
     const int ql = lane >> 2, sb4 = lane & 3;
     const int quad = wg * 2 + ql;
@@ -1276,7 +1328,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     stw1(co_rsrc(uni(F.tmoe)), quad * 4 + sb4, tagged(f16r(acc + f16r(s * L.dbuf[(ql * 9 + 8) * 4 + sb4])), flow_tag(base, li, FS_C)));
   }
   fstamp<ST>(li, FS_C, 4, tid == PUB_WAVE * 64);
-  __syncthreads();
+  lds_barrier();
   return true;
 }
 
@@ -1327,7 +1379,7 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
   }
   fstamp<ST>(nl, 0, 3, tid == 0);
   if (lane == 0) { L.red[wave] = bv; L.ired[wave] = bi; }
-  __syncthreads();
+  lds_barrier();
   if (wave == PUB_WAVE && lane == 0) {
     bv = L.red[0]; bi = L.ired[0];
     for (int w = 1; w < DEC_WAVES; ++w)
@@ -1353,9 +1405,9 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
     const float ov = __shfl_xor(v, msk, 64); const int oi = __shfl_xor(i, msk, 64);
     if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
   }
-  __syncthreads();
+  lds_barrier();
   if (lane == 0) { L.red[wave] = v; L.ired[wave] = i; }
-  __syncthreads();
+  lds_barrier();
   if (tid == 0) {
     for (int w = 1; w < DEC_WAVES; ++w)
       if (L.red[w] > v || (L.red[w] == v && L.ired[w] < i)) { v = L.red[w]; i = L.ired[w]; }
@@ -1420,9 +1472,9 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
     }
     if (!flow_head<ST>(F, pos, out_off + step, feed, base, h0, h1, step + 1 < steps)) return;
     if (step + 1 < steps) {
-      __syncthreads();                   // everybody has read this step's position, tag base and parities
+      lds_barrier();                     // everybody has read this step's position, tag base and parities
       if (threadIdx.x == 0) { g_K.pos = pos + 1; g_K.base = base + (uint32_t)(nl + 1) * 8u; g_K.parity ^= g_K.linmask; }
-      __syncthreads();
+      lds_barrier();
     }
   }
   if constexpr (ST) {

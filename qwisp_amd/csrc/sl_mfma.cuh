@@ -447,7 +447,6 @@ struct SdpaLaneArgs {
 };
 // Workgroup barrier that waits for the wave's LDS traffic only: global loads issued before it stay in flight across it
 // (__syncthreads would wait for them as well).
-SL_DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 __global__ __launch_bounds__(256) void k_sdpa_lane_mfma(SdpaLaneArgs la) {
   __shared__ __align__(16) uint16_t s_k[SDPA_TILE * KT_STRIDE];
   __shared__ __align__(16) uint16_t s_vt[256 * VT_STRIDE];
