@@ -600,3 +600,35 @@ def test_layer_pattern_and_rollback(small_model):
     after = [o.read_layer_cache(li) for li in range(cfg.n_layers)]
     for (a0, b0), (a1, b1) in zip(before, after):
         assert np.array_equal(a0, a1) and np.array_equal(b0, b1)
+
+
+# ---- arg-max: the first of several equal maxima (argmax_rows, SeedlessFusedVerify.swift:583-590; the reference
+#      tests a deliberate tie against MLX's argMax, SeedlessVerifyTests.swift:1179-1186) -----------------------
+def test_head_argmax_takes_the_lowest_index_among_equal_maxima():
+    cfg = ModelConfig(n_layers=1, n_experts=8, vocab=512, layer_types=("gdn",))
+    host = orc.generate_host(cfg)
+    normed = rng.normal(0, 1, (1, 2048)).astype(np.float16)
+    o = orc.Oracle(cfg, host, max_m=2, max_seq_len=8)
+    a = int(o.head_argmax(normed)[0])
+    lg = o.logits_row(0).astype(np.float32)
+    assert a == int(np.argmax(lg)) and np.sum(lg == lg[a]) == 1          # numpy's argmax is first-index too
+    o.close()
+
+    def planted(rows):
+        t = dict(host)
+        for suf in (".weight", ".scales", ".biases"):
+            x = host["lm_head" + suf].copy()
+            for r in rows:
+                x[r] = x[a]
+            t["lm_head" + suf] = x
+        o2 = orc.Oracle(cfg, t, max_m=2, max_seq_len=8)
+        got = int(o2.head_argmax(normed)[0])
+        l2 = o2.logits_row(0)
+        o2.close()
+        assert all(l2[r].view(np.uint16) == l2[a].view(np.uint16) for r in rows)   # equal bits: a real tie
+        return got
+
+    lo, hi = (a - 7) % cfg.vocab, (a + 11) % cfg.vocab
+    lo, hi = min(lo, hi, a - 1 if a else a + 1), max(lo, hi)
+    for rows in ([hi], [lo], [lo, hi], [0, cfg.vocab - 1]):                 # the maximum at two and at three indices
+        assert planted(rows) == min(rows + [a]), rows
