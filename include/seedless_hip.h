@@ -13,7 +13,9 @@
  *    of an engine is sticky: sl_fault() returns its message and every later call on that engine
  *    returns SL_ERR_POISONED without touching its outputs (SFV:388-401, TellRuntime.swift:193).
  *  - One thread inside one engine at a time (the reference serialises callers with a semaphore,
- *    LLMBackend.swift:129).
+ *    LLMBackend.swift:129).  Different engines and lanes may be driven from different threads: batch-1 steps, which
+ *    occupy the whole GPU with one launch, are serialised inside the library (the reference treats the GPU as
+ *    exclusive, AGENTS.md:95).
  *  - Weights are MLX-affine 4-bit, group 64 along K: w = scale*q + bias, q packed 8 per
  *    little-endian uint32, nibble j of a word is (word >> 4*j) & 15 (SeedlessMetalForward.swift
  *    :171-174); scales/biases are fp16 [N, K/64].
@@ -160,8 +162,9 @@ int sl_chained_step_argmax(sl_engine* e, int32_t first_token, int k, int32_t* ou
 int sl_step_sample_rows(sl_engine* e, const int32_t* tokens, int m, float temperature, float top_p,
                         uint64_t seed, int32_t* out);
 /* A further sequence on the weights of `base` (reference: the lanes of SeedlessLaneBatch share one weight
- * set, SeedlessLaneBatch.swift:876): own caches, scratch and stream; `base` keeps the weights and must be
- * destroyed after its lanes.  The lane is a full engine: every entry point works on it. */
+ * set, SeedlessLaneBatch.swift:876): own caches, scratch and stream; `base` keeps the weights.  A base destroyed
+ * before its lanes stops answering calls (sticky fault) and its memory is released with the last lane.  The lane is a
+ * full engine: every entry point works on it. */
 int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine** out);
 /* SeedlessLaneBatch.stepArgmaxBatch (SeedlessLaneBatch.swift:876): one token in and one out per lane, per
  * lane identical (bit for bit) to a solo sl_step_argmax of that lane.  With 2 <= b <= max_m of lanes[0], and
@@ -348,6 +351,11 @@ int sl_set_hybrid(sl_engine* e, int enable);
  * 2 preparation done, 3 arithmetic done, 4 results stored. */
 int sl_debug_stage_clock(sl_engine* e, int enable, uint32_t* out, int cap_words);
 int sl_stage_clock_words(void);
+/* Test hook beside injectCBFailure (SFV:404) for the single-launch step's own failure path: after `rounds` unanswered
+ * polling rounds a workgroup stops waiting and raises an abort word, every other workgroup leaves at its next wait,
+ * the kernel ends normally and the step returns SL_ERR_DEVICE (sticky).  The engine's default is 2^19 rounds, about
+ * half a second; 0 makes the first unanswered poll give up.  No kernel is made to fault or hang. */
+int sl_debug_set_spin_limit(sl_engine* e, unsigned rounds);
 
 /* Per-kernel timing in the manner of forwardRowsProfiled (SFV:4352): while enabled, every launch of
  * the dominant kernel (the persistent step kernel, or lm_head in the kernel-per-stage sequence) is bracketed by HIP events on the engine's stream; the read call returns the

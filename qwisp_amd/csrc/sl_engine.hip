@@ -9,7 +9,9 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <atomic>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -51,6 +53,13 @@ constexpr size_t HIST_ELEMS = (size_t)(SL_CONV_K - 1) * SL_CONV_DIM;
 constexpr size_t STATE_ELEMS = (size_t)SL_GDN_HV * SL_GDN_D * SL_GDN_D;
 constexpr int MAX_CHAIN = 256;
 
+// The single-launch step is a grid of workgroups that wait for each other's results without a grid barrier: it
+// only makes progress when all of them are resident at once.  One such launch fills the machine, so two of them
+// (two engines or lanes driven from two host threads) must never overlap: from launch to read-back a step holds
+// this process-wide lock.
+std::mutex g_flow_mutex;
+std::atomic<uint64_t> g_engine_uid{1};
+
 }  // namespace
 
 struct sl_full_snap {
@@ -60,6 +69,11 @@ struct sl_full_snap {
 };
 
 struct sl_engine {
+  uint64_t uid = g_engine_uid.fetch_add(1);   // never reused: identifies an engine in another engine's lane table
+  // lanes keep their base alive: a base destroyed while lanes exist is only marked, and goes with its last lane
+  sl_engine* base_of = nullptr;
+  int lane_refs = 0;
+  bool destroy_pending = false;
   int n_layers = 0, n_experts = 0, vocab = 0, max_m = 0, max_seq = 0, max_tiles = 0;
   bool has_attn = false, has_head = false;
   bool gate8 = false;              // router / shared gate are 8-bit rows (all layers alike)
@@ -107,7 +121,7 @@ struct sl_engine {
   bool inject_failure = false;
   // lane batch driven from this engine's scratch: device table [n_layers][max_m] of the lanes last stepped together
   LaneRef* lane_tab = nullptr;
-  std::vector<sl_engine*> lane_set;
+  std::vector<uint64_t> lane_set;              // uids of the lanes the table was built for
   // where the logits / normed rows of the most recent step live (a lane-batched step leaves them in the driver's rows)
   const uint16_t* logits_view = nullptr;
   const uint16_t* normed_view = nullptr;
@@ -696,6 +710,7 @@ int alloc_runtime(sl_engine* e) {
         F.tcand = dalloc<uint4>(e, 256, true);
         F.ttok = dalloc<uint4>(e, 4, true);
         F.sdpa_round = SDPA_ROUND;
+        F.spin_limit = FLOW_SPIN_LIMIT;
         if (const char* s = std::getenv("QWISP_SDPA_ROUND")) {      // smaller rounds, for tests of the round loop
           const int v = std::atoi(s);
           if (v >= 1 && v <= SDPA_ROUND) F.sdpa_round = v;
@@ -710,7 +725,10 @@ int alloc_runtime(sl_engine* e) {
         SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
         SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
       }
-      e->dec_grid = 256;
+      // every workgroup of the grid must be resident at once: one per compute unit
+      int per_cu = 0;
+      SL_TRY(e, hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k_decode_flow<false, false>, DEC_THREADS, DEC_DYN_LDS));
+      if (per_cu >= 1) e->dec_grid = 256;
     }
   }
   e->pinned_bytes = MH * 2 + 4096 + (size_t)d->n_layers * 4 + (size_t)MAX_CHAIN * 4;
@@ -741,6 +759,9 @@ int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine*
     const int r = alloc_layer_state(e, L); if (r) return r;
   }
   e->embed = base->embed; e->lm_head = base->lm_head; e->final_norm = base->final_norm; e->gate8 = base->gate8;
+  sl_engine* root = const_cast<sl_engine*>(base->base_of ? base->base_of : base);   // a lane of a lane shares the root's weights
+  e->base_of = root;
+  root->lane_refs += 1;
   return alloc_runtime(e);
 }
 
@@ -759,7 +780,8 @@ bool lanes_batchable(sl_engine** lanes, int b) {
 }
 // Device table of the lanes' caches, [n_layers][max_m] in the driver; rebuilt when the set of lanes changes.
 int bind_lanes(sl_engine* d, sl_engine** lanes, int b) {
-  if ((int)d->lane_set.size() == b && std::equal(d->lane_set.begin(), d->lane_set.end(), lanes)) return SL_OK;
+  if ((int)d->lane_set.size() == b &&
+      std::equal(d->lane_set.begin(), d->lane_set.end(), lanes, [](uint64_t u, const sl_engine* l) { return u == l->uid; })) return SL_OK;
   if (!d->lane_tab) {
     d->lane_tab = dalloc<LaneRef>(d, (size_t)d->n_layers * d->max_m, true);
     if (!d->lane_tab) return SL_ERR_DEVICE;
@@ -774,7 +796,8 @@ int bind_lanes(sl_engine* d, sl_engine** lanes, int b) {
       r.kcache = L.kcache; r.vcache = L.vcache; r.st = lanes[i]->st; r.max_seq = lanes[i]->max_seq;
     }
   int r = copy_sync(d, d->lane_tab, tab.data(), tab.size() * sizeof(LaneRef), hipMemcpyHostToDevice); if (r) return r;
-  d->lane_set.assign(lanes, lanes + b);
+  d->lane_set.clear();
+  for (int i = 0; i < b; ++i) d->lane_set.push_back(lanes[i]->uid);
   return SL_OK;
 }
 }  // namespace
@@ -840,6 +863,13 @@ int sl_step_sample_rows(sl_engine* e, const int32_t* tokens, int m, float temper
 
 void sl_destroy(sl_engine* e) {
   if (!e) return;
+  if (e->lane_refs > 0) {            // lanes still read these weights: the memory goes with the last of them
+    if (e->stream) (void)hipStreamSynchronize(e->stream);
+    e->destroy_pending = true;
+    if (e->fault.empty()) e->fault = "engine destroyed (kept alive by its lanes)";
+    return;
+  }
+  sl_engine* root = e->base_of;
   if (e->stream) (void)hipStreamSynchronize(e->stream);
   for (void* p : e->allocs) (void)hipFree(p);
   if (e->pinned) (void)hipHostFree(e->pinned);
@@ -848,6 +878,7 @@ void sl_destroy(sl_engine* e) {
   if (e->ev1) (void)hipEventDestroy(e->ev1);
   if (e->stream) (void)hipStreamDestroy(e->stream);
   delete e;
+  if (root && --root->lane_refs == 0 && root->destroy_pending) sl_destroy(root);
 }
 
 const char* sl_fault(const sl_engine* e) { return (e && !e->fault.empty()) ? e->fault.c_str() : nullptr; }
@@ -888,6 +919,15 @@ int sl_debug_stage_clock(sl_engine* e, int enable, uint32_t* out, int cap_words)
   return SL_OK;
 }
 int sl_stage_clock_words(void) { return STAMP_WORDS; }
+// Test hook in the manner of injectCBFailure (SFV:404): the number of polling rounds after which a workgroup of the
+// single-launch step stops waiting, raises the abort word and leaves (every workgroup then does the same at its next
+// wait, so the kernel ends normally).  0 makes the first unanswered poll give up.
+int sl_debug_set_spin_limit(sl_engine* e, unsigned rounds) {
+  int r = guard(e); if (r) return r;
+  if (!e->flow_params) return SL_ERR_UNSUPPORTED;
+  e->flow_host.spin_limit = rounds;
+  return copy_sync(e, e->flow_params, &e->flow_host, sizeof(FlowP), hipMemcpyHostToDevice);
+}
 int sl_profile_head(sl_engine* e, int enable) {
   int r = guard(e); if (r) return r;
   if (enable && e->head_ev.empty()) {
@@ -927,8 +967,10 @@ int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
   r = check_rows(e, m); if (r) return r;
   for (int i = 0; i < m; ++i) if (tokens[i] < 0 || tokens[i] >= e->vocab) return SL_ERR_ARG;
   r = to_device(e, e->tok_in, tokens, (size_t)m * 4); if (r) return r;
-  SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   const bool persistent = (m == 1 && e->dec_grid > 0 && e->use_persistent);
+  std::unique_lock<std::mutex> flow_lock(g_flow_mutex, std::defer_lock);
+  if (persistent) flow_lock.lock();
+  SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   if (persistent) {
     launch_decode(e, 0, false, 1);
   } else {
@@ -951,8 +993,10 @@ int sl_chained_step_argmax(sl_engine* e, int32_t first, int k, int32_t* out) {
   if (!out || !e->has_head || k < 1 || k > MAX_CHAIN || first < 0 || first >= e->vocab) return SL_ERR_ARG;
   if (e->has_attn && e->pos + k > e->max_seq) return SL_ERR_ARG;
   r = to_device(e, e->tok_in, &first, 4); if (r) return r;
-  SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   const bool persistent = (e->dec_grid > 0 && e->use_persistent);
+  std::unique_lock<std::mutex> flow_lock(g_flow_mutex, std::defer_lock);
+  if (persistent) flow_lock.lock();
+  SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   if (persistent) launch_decode(e, 0, true, k);        // the whole chain in one launch
   for (int s = 0; s < k && !persistent; ++s) {
     hipLaunchKernelGGL(k_embed, dim3(H / 256, 1), dim3(256), 0, e->stream, e->tok_in, e->embed.w, e->embed.sb, e->hA);
@@ -1017,6 +1061,7 @@ int sl_logits_row(sl_engine* e, int m, uint16_t* out) {
 int sl_head_argmax(sl_engine* e, const uint16_t* normed, int m, int32_t* out) {
   int r = guard(e); if (r) return r;
   if (!normed || !out || !e->has_head || m < 1 || m > e->max_m) return SL_ERR_ARG;
+  e->logits_view = e->normed_view = nullptr;      // the logits this call leaves are the engine's own rows
   r = to_device(e, e->xn, normed, (size_t)m * H * 2); if (r) return r;
   HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
   launch_head(e, m, ha, 0, false);

@@ -34,6 +34,7 @@ struct FlowP {
   uint4 *tcand;         // {value, index, tag, tag}        [256]
   uint4 *ttok;          // {token, token, tag, tag}: the token a step of a multi-step launch hands to the next [1]
   int sdpa_round;       // long contexts: (tile, kv head) units a workgroup scores before it turns to their values
+  unsigned spin_limit;  // polling rounds after which a workgroup gives up and raises the abort word (FLOW_SPIN_LIMIT; tests: 0)
 };
 
 // Parameters live in LDS for the whole launch.  Reading them there (ds_read + readfirstlane) does not
@@ -127,7 +128,7 @@ SL_DEV void fstamp(int layer, int stage, int kind, bool who) {
 SL_DEV int flow_round(bool ok, unsigned& spins, unsigned* abort_word) {
   const unsigned slot = spins % 3u;
   if (!__all(ok ? 1 : 0) && (threadIdx.x & 63) == 0) g_L.pf[slot] = 1;
-  if (threadIdx.x == 0 && (spins > FLOW_SPIN_LIMIT || ((spins & 63u) == 63u && ld_co32(abort_word) != 0))) {
+  if (threadIdx.x == 0 && (spins > g_K.F.spin_limit || ((spins & 63u) == 63u && ld_co32(abort_word) != 0))) {
     st_co32(abort_word, 1u);
     g_L.pf[3] = 1;
   }
@@ -880,7 +881,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
             }
           }
           if (mdone && gdone && have == (1u << cnt0) - 1u) break;
-          if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+          if (++spins > uni(F.spin_limit)) { fail = 1; break; }
           __builtin_amdgcn_s_sleep(1);
         }
         Mx = tree_max<64>(mine ? __uint_as_float(m0.x) : NEG);
@@ -893,7 +894,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
           float pm = NEG;
           if (mine) { const uint4 m = ldw4(rml, (slot0 + t0 + lane) * 4); ok = m.z == tcore32 && m.w == tcore32; pm = __uint_as_float(m.x); }
           if (__all(ok ? 1 : 0)) { Mx = fmaxf(Mx, tree_max<64>(pm)); break; }
-          if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+          if (++spins > uni(F.spin_limit)) { fail = 1; break; }
           __builtin_amdgcn_s_sleep(1);
         }
       }
@@ -927,7 +928,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
             if (t >= MB && t < nt && act) { q[j] = ldw4(rpo, ((slot0 + t) * 128 + chunk) * 4); ok = ok && q[j].z == tcore32 && q[j].w == tcore32; }
           }
           if (__all(ok ? 1 : 0)) break;
-          if (++spins > FLOW_SPIN_LIMIT) { fail = 1; break; }
+          if (++spins > uni(F.spin_limit)) { fail = 1; break; }
           __builtin_amdgcn_s_sleep(1);
         }
 #pragma unroll

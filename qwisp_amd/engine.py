@@ -46,6 +46,8 @@ class SeedlessFusedForward:
         status = self.lib.dll.sl_lane_create(self.h, max_m, max_seq_len, C.byref(h))
         lane = object.__new__(type(self))
         lane.lib, lane.cfg, lane.h = self.lib, self.cfg, h
+        lane.max_m, lane.max_seq_len = max_m, max_seq_len
+        lane._base = self                      # the weights live in the base: keep it referenced while the lane exists
         if status != abi.SL_OK:
             fault = lane.gpu_fault if h else None
             lane.close()

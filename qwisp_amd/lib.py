@@ -66,6 +66,7 @@ SIGNATURES = {
     "sl_set_hybrid": (_i32, [_vp, _i32]),
     "sl_debug_stage_clock": (_i32, [_vp, _i32, _vp, _i32]),
     "sl_stage_clock_words": (_i32, []),
+    "sl_debug_set_spin_limit": (_i32, [_vp, C.c_uint32]),
     "sl_profile_head": (_i32, [_vp, _i32]),
     "sl_profile_head_read": (_i32, [_vp, C.POINTER(C.c_double), C.POINTER(_i64)]),
     "sl_selftest_math": (_i32, [_i32, _vp, _vp, _i64]),

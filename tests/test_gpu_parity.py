@@ -827,3 +827,63 @@ def test_full_size_model_short_stream(env):
     assert eng.rollback_one_step(snap)
     b = eng.chained_step_argmax(int(got[-1]), 3).tolist()
     assert a[0] == b[0]
+
+
+# ---- failure path and lifetimes of the single-launch step ---------------------------------------------------
+def test_single_launch_step_gives_up_reports_and_poisons(env, small_model):
+    """The failure firewall of the step kernel itself (reference: GPUFaultState, SeedlessFusedVerify.swift:388-416,
+    exercised by SeedlessVerifyTests.swift:6246 through injectCBFailure).  With the bounded wait cut to nothing by the
+    host, the first unanswered poll makes its workgroup raise the abort word, every workgroup leaves at its next
+    wait, the kernel ends normally, the call reports a device failure and the engine stays poisoned; the GPU and
+    other engines are unaffected."""
+    cfg, dev, host = small_model
+    eng = env["Engine"](cfg, dev, max_m=2, max_seq_len=32)
+    good = eng.step_argmax([7])
+    assert good is not None
+    assert env["lib"].dll.sl_debug_set_spin_limit(eng.h, 0) == abi.SL_OK
+    assert eng.step_argmax([int(good[0])]) is None
+    assert "timed out" in eng.gpu_fault
+    assert eng.step_argmax([1]) is None and eng.chained_step_argmax(1, 2) is None and eng.forward_tokens([1]) is None
+    other = env["Engine"](cfg, dev, max_m=2, max_seq_len=32)
+    again = other.step_argmax([7])
+    assert again is not None and again.tolist() == good.tolist()
+    eng.close(); other.close()
+
+
+def test_lanes_outlive_their_base_and_two_threads_drive_two_engines(env, small_model):
+    import threading
+    cfg, dev, host = small_model
+    base = env["Engine"](cfg, dev, max_m=4, max_seq_len=96)
+    lane = base.new_lane(max_m=4, max_seq_len=96)
+    solo = env["Engine"](cfg, dev, max_m=4, max_seq_len=96)
+    assert lane.max_m == 4 and lane.max_seq_len == 96
+    base.close()                                  # the weights stay until the last lane is gone
+    prompt = [3, 1415, 926, 535]
+    a, b = lane.greedy_generate(prompt, 6), solo.greedy_generate(prompt, 6)
+    assert a is not None and a.tolist() == b.tolist()
+    # two engines stepped from two host threads at once: their single-launch steps take turns inside the library
+    e1, e2 = env["Engine"](cfg, dev, max_m=1, max_seq_len=160), env["Engine"](cfg, dev, max_m=1, max_seq_len=160)
+    out = {}
+
+    def run(name, e, first):
+        toks, cur = [], first
+        for _ in range(12):
+            o = e.chained_step_argmax(cur, 8)
+            if o is None:
+                out[name] = e.gpu_fault
+                return
+            toks += o.tolist(); cur = int(o[-1])
+        out[name] = toks
+    th = [threading.Thread(target=run, args=("a", e1, 11)), threading.Thread(target=run, args=("b", e2, 12))]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    ref = env["Engine"](cfg, dev, max_m=1, max_seq_len=160)
+    want, cur = [], 11
+    for _ in range(12):
+        o = ref.chained_step_argmax(cur, 8); want += o.tolist(); cur = int(o[-1])
+    assert out["a"] == want, out["a"]
+    assert isinstance(out["b"], list) and len(out["b"]) == 96
+    for e in (lane, solo, e1, e2, ref):
+        e.close()
