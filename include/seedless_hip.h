@@ -53,7 +53,8 @@ typedef enum {
   SL_ERR_POISONED = -2,   /* engine has a sticky fault */
   SL_ERR_DEVICE = -3,     /* a HIP call failed; message in sl_fault() */
   SL_ERR_UNSUPPORTED = -4,
-  SL_ERR_FORMAT = -5      /* persisted-state blob does not match this engine */
+  SL_ERR_FORMAT = -5,     /* persisted-state blob does not match this engine */
+  SL_ERR_TOO_LARGE = -6   /* the request exceeds a fixed capacity of the entry point (sl_head_argmax_noalloc) */
 } sl_status;
 
 /* Where the tensors named by a model description live. */
@@ -185,6 +186,16 @@ int sl_logits_row(sl_engine* e, int m, uint16_t* out_f16 /* [vocab] */);
 /* engine.logits (SeedlessEngine.swift:180): lm_head + argmax over already-normed rows; used for
  * the first token after prefill (TellRuntime.swift:724-727). */
 int sl_head_argmax(sl_engine* e, const uint16_t* normed_f16, int m, int32_t* out);
+
+/* No counterpart in the reference.  sl_head_argmax for callers that cannot allocate device memory or synchronise:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid allocation.  `normed_dev` [m, 2048] fp16
+ * and `out_dev` [m] are device pointers, the kernels are queued on `stream` (a hipStream_t; NULL = the default
+ * stream) and the call returns without waiting.  It allocates nothing, copies nothing and frees nothing: logits and
+ * arg-max candidates go to a fixed 5 MiB array inside the library's device image (one copy per GPU, held until
+ * the process ends).  Limits: m <= 8 rows and a vocabulary of at most 262144, beyond that SL_ERR_TOO_LARGE.  All
+ * calls on one GPU share that array, so calls that overlap on a GPU (different streams or engines) race; calls
+ * queued on one stream are safe.  Results equal sl_head_argmax's. */
+int sl_head_argmax_noalloc(sl_engine* e, const uint16_t* normed_dev, int m, int32_t* out_dev, void* stream);
 
 /* snapshot / rollbackOneStep (SFV:4039-4047): undo exactly one forward made after the snapshot. */
 int sl_snapshot(sl_engine* e, sl_snap* s);

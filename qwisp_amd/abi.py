@@ -14,7 +14,7 @@ ATT_HEADS, ATT_KV, ATT_D = 16, 2, 256
 GDN_HK, GDN_HV, GDN_D = 16, 32, 128
 CONV_K, CONV_DIM = 4, 8192
 
-SL_OK, SL_ERR_ARG, SL_ERR_POISONED, SL_ERR_DEVICE, SL_ERR_UNSUPPORTED, SL_ERR_FORMAT = 0, -1, -2, -3, -4, -5
+SL_OK, SL_ERR_ARG, SL_ERR_POISONED, SL_ERR_DEVICE, SL_ERR_UNSUPPORTED, SL_ERR_FORMAT, SL_ERR_TOO_LARGE = 0, -1, -2, -3, -4, -5, -6
 SL_LOC_HOST, SL_LOC_DEVICE = 0, 1
 
 

@@ -60,6 +60,34 @@ constexpr int MAX_CHAIN = 256;
 std::mutex g_flow_mutex;
 std::atomic<uint64_t> g_engine_uid{1};
 
+// ---- scratch of the entry point that allocates nothing (sl_head_argmax_noalloc) --------------------------------
+// lm_head + arg-max needs room for the logits rows and for one (value, index) candidate per 16 vocabulary rows and
+// activation row.  For callers that must not allocate, that room is a fixed array in the library's device image:
+// every GPU the library runs on holds its own copy at its own address until the process ends.  The array's name is
+// only a host-side handle; the address kernels can use comes from hipGetSymbolAddress, once per device.
+constexpr int NA_MAX_ROWS = 8;
+constexpr int NA_MAX_VOCAB = 262144;
+constexpr size_t NA_LOGITS_BYTES = (size_t)NA_MAX_ROWS * NA_MAX_VOCAB * sizeof(uint16_t);          // 4 MiB
+constexpr size_t NA_CAND = (size_t)NA_MAX_ROWS * (NA_MAX_VOCAB / 16);                               // 131072 candidates
+constexpr size_t NA_SCRATCH_BYTES = NA_LOGITS_BYTES + NA_CAND * (sizeof(float) + sizeof(int32_t));  // 5 MiB
+static __device__ __align__(256) unsigned char scratch[NA_SCRATCH_BYTES];
+constexpr int NA_MAX_DEVICES = 64;
+void* g_scratch_ptr[NA_MAX_DEVICES] = {};
+std::mutex g_scratch_mutex;
+// Address of this device's copy of `scratch`; resolved on the first call per device (with that device current).
+hipError_t scratch_address(int device, void** out) {
+  if (device < 0 || device >= NA_MAX_DEVICES) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    const hipError_t r = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (r != hipSuccess) return r;
+    g_scratch_ptr[device] = p;
+  }
+  *out = g_scratch_ptr[device];
+  return hipSuccess;
+}
+
 }  // namespace
 
 struct sl_full_snap {
@@ -76,6 +104,8 @@ struct sl_engine {
   bool destroy_pending = false;
   int n_layers = 0, n_experts = 0, vocab = 0, max_m = 0, max_seq = 0, max_tiles = 0;
   bool has_attn = false, has_head = false;
+  int device = 0;                  // the device that was current when the engine was created
+  void* na_scratch = nullptr;      // this device's copy of the no-allocation scratch array
   bool gate8 = false;              // router / shared gate are 8-bit rows (all layers alike)
   hipStream_t stream = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -535,6 +565,8 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
   e->max_m = max_m; e->max_seq = max_seq_len; e->max_tiles = (max_seq_len + SDPA_TILE - 1) / SDPA_TILE;
   e->has_head = has_head;
   e->parity.assign(d->n_layers, 0);
+  SL_TRY(e, hipGetDevice(&e->device));
+  SL_TRY(e, scratch_address(e->device, &e->na_scratch));
   SL_TRY(e, hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
   SL_TRY(e, hipEventCreate(&e->ev0));
   SL_TRY(e, hipEventCreate(&e->ev1));
@@ -749,6 +781,7 @@ int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine*
   e->max_m = max_m; e->max_seq = max_seq_len; e->max_tiles = (max_seq_len + SDPA_TILE - 1) / SDPA_TILE;
   e->has_head = base->has_head;
   e->parity.assign(e->n_layers, 0);
+  e->device = base->device; e->na_scratch = base->na_scratch;
   SL_TRY(e, hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
   SL_TRY(e, hipEventCreate(&e->ev0));
   SL_TRY(e, hipEventCreate(&e->ev1));
@@ -1066,6 +1099,32 @@ int sl_head_argmax(sl_engine* e, const uint16_t* normed, int m, int32_t* out) {
   HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
   launch_head(e, m, ha, 0, false);
   return read_back(e, out, e->tok_out, (size_t)m * 4, "headArgmax");
+}
+
+// lm_head + arg-max for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that
+// forbid it): device pointers in and out, the caller's stream, no allocation, copy or synchronisation.  The logits
+// rows and arg-max candidates live in this device's copy of the fixed `scratch` array, which every call on the
+// device shares: calls that overlap on one GPU race.  Every word the reduction reads is written by the same call,
+// so nothing has to be cleared.
+int sl_head_argmax_noalloc(sl_engine* e, const uint16_t* normed_dev, int m, int32_t* out_dev, void* stream) {
+  int r = guard(e); if (r) return r;
+  if (!normed_dev || !out_dev || !e->has_head || m < 1) return SL_ERR_ARG;
+  if (m > NA_MAX_ROWS || e->vocab > NA_MAX_VOCAB) return SL_ERR_TOO_LARGE;
+  if (!e->na_scratch) return SL_ERR_DEVICE;
+  hipStream_t st = (hipStream_t)stream;
+  uint16_t* logits = reinterpret_cast<uint16_t*>(e->na_scratch);
+  float* cand_v = reinterpret_cast<float*>(static_cast<unsigned char*>(e->na_scratch) + NA_LOGITS_BYTES);
+  int32_t* cand_i = reinterpret_cast<int32_t*>(cand_v + NA_CAND);
+  const int n_cand = e->vocab / 16;
+  if (m >= 2) {
+    hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, false, true>), dim3(n_cand, (m + 7) / 8), dim3(256), 0, st, HiddenArgs{}, normed_dev, H,
+                       e->lm_head.w, e->lm_head.sb, e->vocab, logits, e->vocab, m, cand_v, cand_i);
+  } else {
+    HiddenArgs ha{normed_dev, nullptr, nullptr, nullptr, nullptr};
+    hipLaunchKernelGGL(k_head, dim3(n_cand, 1), dim3(256), 0, st, ha, e->lm_head.w, e->lm_head.sb, e->vocab, logits, cand_v, cand_i);
+  }
+  hipLaunchKernelGGL(k_argmax_final, dim3(m), dim3(256), 0, st, cand_v, cand_i, n_cand, out_dev, 0, (int32_t*)nullptr);
+  return hipGetLastError() == hipSuccess ? SL_OK : SL_ERR_DEVICE;
 }
 
 int sl_snapshot(sl_engine* e, sl_snap* s) {

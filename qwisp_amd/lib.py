@@ -28,6 +28,7 @@ SIGNATURES = {
     "sl_hidden_rows": (_i32, [_vp, _i32, _vp]),
     "sl_logits_row": (_i32, [_vp, _i32, _vp]),
     "sl_head_argmax": (_i32, [_vp, _vp, _i32, _vp]),
+    "sl_head_argmax_noalloc": (_i32, [_vp, _vp, _i32, _vp, _vp]),
     "sl_snapshot": (_i32, [_vp, C.POINTER(abi.Snap)]),
     "sl_rollback_one_step": (_i32, [_vp, C.POINTER(abi.Snap)]),
     "sl_full_snapshot": (_i32, [_vp, C.POINTER(_vp)]),
