@@ -28,8 +28,20 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 PROMPT_LEN = 512
-# HBM bytes per decoded token: rocprofv3 FETCH_SIZE + WRITE_SIZE of a k_decode_flow launch (profiles/) / its 8 tokens
-TRAFFIC_BYTES_PER_TOKEN = 1936024336   # 2 x FETCH_SIZE (copy-calibrated) + WRITE_SIZE, in bytes, at context ~525
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "k_decode_flow_decode_b1_40layer_hbm_traffic_pmc.txt")
+
+
+def traffic_bytes_per_token():
+    """HBM bytes per decoded token as the counters saw them: the tracked rocprofv3 FETCH_SIZE / WRITE_SIZE summary of
+    the k_decode_flow launches of this same command (copy-calibrated; the file names the commands).  None when the
+    summary is missing, so the figure can never outlive the profile it came from."""
+    import re
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            m = re.search(r"traffic = (\d+) bytes per launch of (\d+) tokens", f.read())
+        return int(m.group(1)) // int(m.group(2)) if m else None
+    except OSError:
+        return None
 
 
 def step_bytes(cfg, ctx):
@@ -47,6 +59,57 @@ def step_bytes(cfg, ctx):
     return cfg.n_layers * moe + n_gdn * gdn + n_attn * attn + head + norms, head
 
 
+def block_benchmarks(eng, cfg, np, torch):
+    """Benchmark configurations 0-2: one MoE block, one GDN layer, one attention layer over 4K / 8K / 32K keys, batch 1,
+    through the block entry points (the kernel-per-stage sequence: 3 kernels per MoE block, 3 per GDN layer, 5 per
+    attention layer), timed with HIP events around each call's kernels.  "cold": successive calls go to different
+    layers of the model (40 / 30 / 10 distinct weight sets, 0.7 / 0.7 / 0.15-0.8 GB, more than the 256 MB last-level
+    cache), so weights come from HBM; "hot": the same layer every time.  The method follows the reference's kernel
+    micro-benchmarks (PrefixCachePoC.swift:111-162).  Inside the single-launch decode step the same blocks cost what
+    the stage timeline reports."""
+    H = 2048
+    q4 = lambda n, k: n * k // 2 + n * k // 16
+    moe_b = cfg.n_experts * H * 2 + 9 * (2 * q4(512, H) + q4(H, 512)) + H * 2
+    gdn_b = q4(12352, H) + q4(H, 4096) + 8192 * 4 * 4 + 2 * 3 * 8192 * 2 + 2 * 32 * 128 * 128 * 4
+    att_w = q4(9216, H) + q4(H, 4096)
+    lin = [i for i in range(cfg.n_layers) if cfg.is_linear(i)]
+    att = [i for i in range(cfg.n_layers) if not cfg.is_linear(i)]
+    rng = np.random.default_rng(1000)
+    xs = [rng.normal(0, 1, (1, H)).astype(np.float16) for _ in range(8)]
+    REPS, DROP = 30, 5                                    # the reference's 30 repetitions with the first 5 dropped
+
+    def timed(e, fn, layers, nbytes):
+        out = {}
+        for name, seq in (("cold", [layers[i % len(layers)] for i in range(REPS)]), ("hot", [layers[0]] * REPS)):
+            ms = []
+            for i, li in enumerate(seq):
+                y = fn(e, li, xs[i % len(xs)])
+                assert y is not None, e.gpu_fault
+                ms.append(e.last_gpu_ms)
+            us = float(np.median(ms[DROP:])) * 1e3
+            out[name] = {"us": us, "GBs": nbytes / us / 1e3, "frac_of_peak": nbytes / us / 1e3 / HBM_PEAK_GBS}
+        out["bytes"] = nbytes
+        out["roofline_us"] = nbytes / HBM_PEAK_GBS / 1e3
+        return out
+
+    rep = {"method": f"block entry points, kernel-per-stage sequence, batch 1, HIP events, median of {REPS - DROP} calls"}
+    lane = eng.new_lane(max_m=1, max_seq_len=64)
+    rep["moe_block"] = timed(lane, lambda e, li, x: e.moe_block_rows(li, x), list(range(cfg.n_layers)), moe_b)
+    if lin:
+        rep["gdn_layer"] = timed(lane, lambda e, li, x: e.gdn_layer_rows(li, x), lin, gdn_b)
+    lane.close()
+    if att:
+        rep["attention_layer"] = {}
+        for S in (4096, 8192, 32768):
+            lane = eng.new_lane(max_m=1, max_seq_len=S + 2 * REPS + 8)
+            kv = np.random.default_rng(1310).normal(0, 1, (2, S, 256)).astype(np.float16)
+            for li in att:
+                assert lane.load_layer_cache(li, kv, kv)
+            rep["attention_layer"][str(S)] = timed(lane, lambda e, li, x: e.attn_layer_rows(li, x), att, att_w + 2048 * S)
+            lane.close()
+    return rep
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -54,7 +117,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--chain", type=int, default=8, help="tokens per on-device chain")
     ap.add_argument("--layers", type=int, default=40, help="for quick functional runs only")
-    ap.add_argument("--cpu-tokens", type=int, default=256, help="decode tokens timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--cpu-tokens", type=int, default=96,
+                    help="decode tokens the CPU oracle generates after the same 512-token prompt: timed as the CPU baseline and "
+                         "compared with the GPU stream token by token (0 = skip)")
+    ap.add_argument("--blocks", type=int, default=1,
+                    help="also time the single blocks (MoE block, GDN layer, attention layer at 4K / 8K / 32K keys) through their "
+                         "block entry points, weights cold (rotating over the model's layers) and hot (0 = skip)")
+    ap.add_argument("--stage-timeline", type=int, default=1,
+                    help="also run one chain with the stage clock on and report where a step's time goes (0 = skip)")
     ap.add_argument("--lanes", type=int, default=32, metavar="B",
                     help="also time B lanes stepped as one batch of rows on the same weights (extra object in the JSON line; 0 = skip)")
     ap.add_argument("--lane-contexts", choices=("mixed", "short"), default="mixed",
@@ -68,7 +138,7 @@ def main():
     ap.add_argument("--verify-rows", type=int, default=4, metavar="R",
                     help="also time verify steps of R rows ([token] + R-1 drafts through stepArgmax) at the decode context "
                          "(extra object in the JSON line; 0 = skip)")
-    ap.add_argument("--context-sweep", type=str, default="4096,16384", metavar="S1,S2",
+    ap.add_argument("--context-sweep", type=str, default="4096,8192,32768", metavar="S1,S2",
                     help="also time batch-1 decode after prompts of these lengths (hybrid prefill in chunks of 1024; extra "
                          "object in the JSON line; empty = skip)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
@@ -263,23 +333,50 @@ def main():
                                  "frac_of_peak": b_tok / (dt / n_tok) / 1e9 / HBM_PEAK_GBS})
             lane.close()
 
+    blocks_report = None
+    if args.blocks:
+        blocks_report = block_benchmarks(eng, cfg, np, torch)
+
+    timeline_report = None
+    if args.stage_timeline:
+        from qwisp_amd import stage_timeline
+        lib.get().dll.sl_debug_stage_clock(eng.h, 1, None, 0)
+        out = eng.chained_step_argmax(cur, args.chain)            # warms the stamping variant's code
+        out = eng.chained_step_argmax(int(out[-1]), args.chain)
+        assert out is not None, eng.gpu_fault
+        tl = stage_timeline.collect(eng)
+        lib.get().dll.sl_debug_stage_clock(eng.h, 0, None, 0)
+        print(tl.table(), file=sys.stderr)
+        timeline_report = tl.summary()
+
     cpu = None
+    stream_check = None
     if host is not None:
+        # the oracle on the same workload: the same 512-token prompt (untimed), then `--cpu-tokens` greedy tokens, timed
+        # as the CPU baseline and compared with the stream the GPU produced above, token by token
         from oracle import orc
-        CPU_PROMPT = 32
-        ora = orc.Oracle(cfg, host, max_m=4, max_seq_len=CPU_PROMPT + args.cpu_tokens + 8)
-        for i in range(0, CPU_PROMPT, 4):               # a short prompt; also pages the weights in
-            ora.forward_tokens(prompt[i:i + 4])
-        tcur = 17
+        ora = orc.Oracle(cfg, host, max_m=64, max_seq_len=PROMPT_LEN + args.cpu_tokens + 8)
+        t0 = time.perf_counter()
+        nr = None
+        for i in range(0, PROMPT_LEN, 64):
+            nr = ora.forward_tokens(prompt[i:i + 64])
+        cpu_prefill = time.perf_counter() - t0
+        ocur = int(ora.head_argmax(nr[-1:])[0])
+        ostream = [ocur]
         t0 = time.perf_counter()
         for _ in range(args.cpu_tokens):
-            tcur = int(ora.step_argmax([tcur])[0])
+            ocur = int(ora.step_argmax([ocur])[0])
+            ostream.append(ocur)
         cpu_elapsed = time.perf_counter() - t0
+        n_cmp = min(len(ostream), len(stream))
+        bad = [i for i in range(n_cmp) if ostream[i] != stream[i]]
+        assert not bad, f"GPU stream leaves the oracle's at token {bad[0]}: {stream[bad[0]]} vs {ostream[bad[0]]}"
+        stream_check = {"tokens_compared": n_cmp, "equal": True}
         cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
         cpu = {"value": args.cpu_tokens / cpu_elapsed, "unit": "tok/s", "cores": min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))),
                "kind": "port",
-               "sample": f"{args.cpu_tokens} decode tokens after a {CPU_PROMPT}-token prompt, the same {cfg.n_layers}-layer model and weights "
-                         f"(oracle, g++ -O3 OpenMP; {cpu_elapsed:.1f} s)"}
+               "sample": f"{args.cpu_tokens} decode tokens after the same {PROMPT_LEN}-token prompt, the same {cfg.n_layers}-layer model and "
+                         f"weights (oracle, g++ -O3 OpenMP; decode {cpu_elapsed:.1f} s, prompt {cpu_prefill:.1f} s untimed)"}
 
     print(json.dumps({
         "metric": "batch-1 decode tok/s (35B-A3B shape, 4-bit) + achieved HBM GB/s as % of peak",
@@ -291,11 +388,15 @@ def main():
                    "chain_k": args.chain, "context": [PROMPT_LEN + args.warmup, PROMPT_LEN + args.warmup + args.steps]},
         "roofline": {"bound": "hbm", "kernel": "k_decode_flow (persistent batch-1 step: 40 layers + lm_head + argmax)",
                      "achieved": head_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head_gbs / HBM_PEAK_GBS,
-                     "traffic": int(TRAFFIC_BYTES_PER_TOKEN * tok_per_launch), "launches": head_n, "avg_ms": head_avg_ms,
+                     "traffic": (int(traffic_bytes_per_token() * tok_per_launch) if traffic_bytes_per_token() else None),
+                     "launches": head_n, "avg_ms": head_avg_ms,
                      "bytes_per_launch": launch_b, "tokens_per_launch": tok_per_launch, "bytes_per_token": total_b,
                      "avg_ms_per_token": head_avg_ms / tok_per_launch},
         "step_hbm": {"bytes_per_token": total_b, "achieved_GBs": step_gbs, "frac_of_peak": step_gbs / HBM_PEAK_GBS},
         "cpu_baseline": cpu,
+        "stream_vs_oracle": stream_check,
+        "blocks": blocks_report,
+        "stage_timeline": timeline_report,
         "lane_batch": lanes_report,
         "prefill": prefill_report,
         "verify": verify_report,

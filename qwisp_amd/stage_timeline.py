@@ -130,6 +130,29 @@ class Timeline:
         return "\n".join(out)
 
 
+    def summary(self):
+        """Averages per layer type in microseconds, for a report line."""
+        out = {}
+        for name, want_lin in (("gdn_layer", True), ("attention_layer", False)):
+            layers = [l for l in range(1, self.n_layers) if bool(self.lin[l]) == want_lin]
+            if not layers:
+                continue
+            per = [self.stage_rows(l) for l in layers]
+            lt = [x for x in (self.layer_time(l) for l in layers) if x is not None]
+            d = {"us": float(np.mean(lt)) if lt else None}
+            for si in range(6):
+                tot = [p[si]["total"] for p in per if p[si]["total"] is not None]
+                ho = [p[si]["handover_last"] for p in per if p[si]["handover_last"] is not None]
+                d[per[0][si]["stage"]] = {"total_us": float(np.mean(tot)) if tot else None,
+                                          "handover_us": float(np.mean(ho)) if ho else None}
+            mix = [sum(p[si]["total"] or 0.0 for si in (0, 1, 2)) for p in per]
+            moe = [sum(p[si]["total"] or 0.0 for si in (3, 4, 5)) for p in per]
+            d["mixer_us"], d["moe_block_us"] = float(np.mean(mix)), float(np.mean(moe))
+            out[name] = d
+        out["head_us"] = self.head_time()
+        return out
+
+
 def collect(engine):
     """Stamps of the engine's most recent stamped launch as a Timeline."""
     import ctypes as C
