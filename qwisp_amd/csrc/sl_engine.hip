@@ -43,6 +43,7 @@ struct LayerDev {
   uint16_t *q_norm = nullptr, *k_norm = nullptr, *kcache = nullptr, *vcache = nullptr;
   // MoE
   uint16_t *router_w = nullptr, *sgate_w = nullptr;
+  uint16_t* router_pad = nullptr;   // fp16 gates as one matrix [288, 2048] for the matrix-core router of hybrid chunks: rows 0..E-1, row 256 = shared gate
   uint32_t *gate8_w = nullptr, *gate8_sb = nullptr;   // 8-bit gates instead: [E+1, 512] words and [E+1, 32] {scale, bias}; row E = shared gate
   DevQ4 sw_gate, sw_up, sw_down, sh_gate, sh_up, sh_down;
   int32_t* route_inds = nullptr;
@@ -52,6 +53,7 @@ struct LayerDev {
 constexpr size_t HIST_ELEMS = (size_t)(SL_CONV_K - 1) * SL_CONV_DIM;
 constexpr size_t STATE_ELEMS = (size_t)SL_GDN_HV * SL_GDN_D * SL_GDN_D;
 constexpr int MAX_CHAIN = 256;
+constexpr int ROUTER_PAD_ROWS = 288;
 
 // The single-launch step is a grid of workgroups that wait for each other's results without a grid barrier: it
 // only makes progress when all of them are resident at once.  One such launch fills the machine, so two of them
@@ -288,7 +290,11 @@ void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   const int router_blocks = (E + 1 + 15) / 16;
   hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, ha);     // residual + norm once per row
   a.xn_in = ha.xn_out;
-  hipLaunchKernelGGL(k_moe_a, dim3(router_blocks, M), dim3(256), 0, e->stream, a);
+  if (L.router_pad)      // fp16 gates: router and shared-gate logits of all rows as one small GEMM on the matrix cores
+    hipLaunchKernelGGL(k_router_mfma, dim3((ROUTER_PAD_ROWS / 32 + 3) / 4, (M + 31) / 32), dim3(256), 0, e->stream,
+                       RouterMmArgs{ha.xn_out, L.router_pad, M, ROUTER_PAD_ROWS, e->rlogits, e->sgate});
+  else
+    hipLaunchKernelGGL(k_moe_a, dim3(router_blocks, M), dim3(256), 0, e->stream, a);
   hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, E, L.route_inds, L.route_scores);
   hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, E, e->hy_lists, e->hy_counts);
   // routed gate and up by expert in one pass with SwiGLU, then routed down by expert
@@ -617,7 +623,10 @@ int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** ou
     if (w.router_w || w.shared_gate_w) {
       L.router_w = upload<uint16_t>(e, w.router_w, (size_t)E * H, loc);
       L.sgate_w = upload<uint16_t>(e, w.shared_gate_w, H, loc);
-      if (!L.router_w || !L.sgate_w) return SL_ERR_DEVICE;
+      L.router_pad = dalloc<uint16_t>(e, (size_t)ROUTER_PAD_ROWS * H, true);
+      if (!L.router_w || !L.sgate_w || !L.router_pad) return SL_ERR_DEVICE;
+      SL_TRY(e, hipMemcpyAsync(L.router_pad, L.router_w, (size_t)E * H * 2, hipMemcpyDeviceToDevice, e->stream));
+      SL_TRY(e, hipMemcpyAsync(L.router_pad + (size_t)256 * H, L.sgate_w, (size_t)H * 2, hipMemcpyDeviceToDevice, e->stream));
     } else {
       // 8-bit gates: router rows and the shared-gate row in one matrix of E + 1 rows
       if (!shape_ok(w.router_q8, E, H) || !shape_ok(w.shared_gate_q8, 1, H)) {

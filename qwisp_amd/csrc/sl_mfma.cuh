@@ -161,6 +161,93 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
 }
 
 // -------------------------------------------------------------------------------------------------
+// Router and shared-gate logits of a prefill chunk (hybrid mode): Y[m, n] = half(sum_k X[m, k] * W[n, k]) with fp16
+// weights [N, K] (the router's 256 rows, row 256 = the shared expert's gate row, zero rows up to a multiple of 32).
+// Same tiling and operand order as k_qmm4_mfma16 with one row tile per wave; the B operand is eight halves of the
+// weight row itself.  Columns below 256 go to the router logits [M, 256], column 256 to the gate logits [M].
+// -------------------------------------------------------------------------------------------------
+struct RouterMmArgs {
+  const uint16_t* x;     // [M, 2048] fp16 normed rows
+  const uint16_t* W;     // [N, 2048] fp16, N % 32 == 0
+  int M, N;
+  uint16_t* rlogits;     // [M, 256]
+  uint16_t* sgate;       // [M]
+};
+__global__ __launch_bounds__(256) void k_router_mfma(RouterMmArgs a) {
+  constexpr int G = 2, XS = 64 * G + 8, K = 2048;
+  __shared__ __align__(16) uint16_t xs[2][32 * XS];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, hh = lane >> 5;
+  const int n0 = (blockIdx.x * 4 + wave) * 32;
+  const int m0 = blockIdx.y * 32;
+  const bool live = n0 < a.N;
+  const uint16_t* wp = a.W + (size_t)(live ? n0 + col : 0) * K;
+  constexpr int chunks = K / (64 * G);
+  mf_f16v acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  uint4 xr[G];
+  auto fetch = [&](int c) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int row = m0 + (tid >> 3);
+      xr[g] = make_uint4(0, 0, 0, 0);
+      if (row < a.M) xr[g] = ld16(a.x + (size_t)row * K + (c * G + g) * 64 + (tid & 7) * 8);
+    }
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) st16(&xs[buf][(tid >> 3) * XS + g * 64 + (tid & 7) * 8], permute8(xr[g]));
+  };
+  // a lane's weights of a 64-k group: the four 16-byte pieces k = 32 hh + 8 st .. + 7 (st = 0..3), the k order of the A side
+  uint4 nw[G][4];
+  auto wfetch = [&](int c) {
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int st = 0; st < 4; ++st) nw[g][st] = ld16(wp + (c * G + g) * 64 + 32 * hh + 8 * st);
+  };
+  fetch(0);
+  put(0);
+  if (chunks > 1) fetch(1);
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int st = 0; st < 4; ++st) nw[g][st] = make_uint4(0, 0, 0, 0);
+  if (live) wfetch(0);
+  for (int c = 0; c < chunks; ++c) {
+    const int buf = c & 1;
+    uint4 w[G][4];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int st = 0; st < 4; ++st) w[g][st] = nw[g][st];
+    if (live && c + 1 < chunks) wfetch(c + 1);
+    __syncthreads();
+    if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
+    if (!live) continue;
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][col * XS + g * 64 + 32 * hh + 8 * st]);
+        const mf_h8 bw = __builtin_bit_cast(mf_h8, permute8(w[g][st]));
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax, bw, acc, 0, 0, 0);
+      }
+  }
+  if (!live) return;
+  const int n = n0 + col;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int m = m0 + 8 * (r >> 2) + 4 * hh + (r & 3);
+    if (m < a.M) {
+      if (n < 256) a.rlogits[(size_t)m * 256 + n] = f2h(acc[r]);
+      else if (n == 256) a.sgate[m] = f2h(acc[r]);
+    }
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
 // Routed experts of a prefill chunk, grouped by expert (reference: steelMoEGather,
 // SeedlessFusedVerify.swift:4174): the (row, slot) pairs that chose expert e are gathered, multiplied with that
 // expert's matrix once, and scattered back by pair.  Workgroup = (strip block, expert); experts nobody chose exit.
