@@ -346,7 +346,10 @@ int sl_set_persistent(sl_engine* e, int enable);
  * sequence (prefill chunks) compute the dense mixer projections (GDN in/out, attention q|k|v and o) on the matrix
  * cores, the routed experts grouped by expert (steelMoEGather, SeedlessFusedVerify.swift:4174) with weights
  * dequantised to half, and the attention tile pass (scores, probabilities in half, values).  Like the reference's matrix-unit prefill this is not bit-identical to
- * the GEMV order (tolerance-level agreement) but deterministic and independent of how a prompt is chunked.
+ * the GEMV order (tolerance-level agreement) but deterministic.  Calls whose row count and start position are multiples
+ * of 64 also run the recurrence of the GDN layers block-wise on the matrix cores (the chunked form of the delta rule);
+ * a prompt's rows do not depend on how it is cut into such calls, nor on how it is cut into other calls, but the two
+ * kinds agree to tolerance only.
  * Enabled on the engine that drives a lane batch (lanes[0] of sl_lane_step_argmax), batches of 16 or more lanes take
  * the same projections and lm_head to the matrix cores (the experts too from 64 lanes on); recurrent state, caches
  * and attention stay on the exact kernels.  Decode steps and steps of fewer than 16 rows are unaffected. */

@@ -17,6 +17,7 @@
 
 #include "sl_flow.cuh"
 #include "sl_mfma.cuh"
+#include "sl_gdn_chunk.cuh"
 
 using namespace sl;
 
@@ -150,6 +151,7 @@ struct sl_engine {
   // shared gate / up / down rows, pairs listed per expert
   uint16_t *hy_d = nullptr, *hy_sg = nullptr, *hy_su = nullptr, *hy_sy = nullptr, *hy_lists = nullptr;
   int32_t* hy_counts = nullptr;
+  unsigned char* gc_scratch = nullptr;   // chunked gated-delta scan of hybrid chunks: [max_m / 64][32][GC_UNIT_BYTES]
   bool inject_failure = false;
   // lane batch driven from this engine's scratch: device table [n_layers][max_m] of the lanes last stepped together
   LaneRef* lane_tab = nullptr;
@@ -381,7 +383,15 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
     // rows of one sequence: the state-independent part for all rows at once, then the scan without barriers
     GdnPrepArgs pa{g, e->gdn_qn, e->gdn_kn, e->gdn_vc, e->gdn_gb};
     hipLaunchKernelGGL(k_gdn_prep_rows, dim3(65, M), dim3(64), 0, e->stream, pa);
-    hipLaunchKernelGGL(k_gdn_scan_rows, dim3(512), dim3(256), 0, e->stream, pa);
+    if (mm && e->gc_scratch && M % GC == 0 && e->pos % GC == 0) {
+      // hybrid chunks cut at multiples of 64 rows: the delta rule in its chunked form on the matrix cores
+      GdnChunkArgs ca{e->gdn_qn, e->gdn_kn, e->gdn_vc, e->gdn_gb, e->gc_scratch, {L.state[0], L.state[1]}, {L.hist[0], L.hist[1]},
+                      e->proj, e->st + li, e->ycore, M};
+      hipLaunchKernelGGL(k_gdn_chunk_prep, dim3(M / GC, SL_GDN_HV), dim3(256), 0, e->stream, ca);
+      hipLaunchKernelGGL(k_gdn_chunk_scan, dim3(SL_GDN_HV), dim3(256), GC_SCAN_LDS, e->stream, ca);
+    } else {
+      hipLaunchKernelGGL(k_gdn_scan_rows, dim3(512), dim3(256), 0, e->stream, pa);
+    }
   } else {
     if (lanes) hipLaunchKernelGGL(k_gdn_core<4>, dim3(128, M), dim3(256), 0, e->stream, g);
     else hipLaunchKernelGGL(k_gdn_core<2>, dim3(256, 1), dim3(256), 0, e->stream, g);
@@ -937,6 +947,11 @@ int sl_set_hybrid(sl_engine* e, int enable) {
     e->hy_sg = dalloc<uint16_t>(e, rows * SL_MOE_I); e->hy_su = dalloc<uint16_t>(e, rows * SL_MOE_I);
     e->hy_sy = dalloc<uint16_t>(e, rows * H);
     if (!e->hy_d || !e->hy_sg || !e->hy_su || !e->hy_sy) return SL_ERR_DEVICE;
+    if (rows >= GC) {
+      e->gc_scratch = dalloc<unsigned char>(e, (rows / GC) * SL_GDN_HV * GC_UNIT_BYTES);
+      if (!e->gc_scratch) return SL_ERR_DEVICE;
+      SL_TRY(e, hipFuncSetAttribute((const void*)k_gdn_chunk_scan, hipFuncAttributeMaxDynamicSharedMemorySize, GC_SCAN_LDS));
+    }
     SL_TRY(e, hipStreamSynchronize(e->stream));
   }
   e->hybrid = enable != 0;

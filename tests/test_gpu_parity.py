@@ -244,7 +244,8 @@ def test_mfma_qmm4_against_the_oracle_rows(env, m, n, k):
 def test_hybrid_prefill_agrees_with_the_exact_rows(env, small_model):
     """forwardRowsHybrid (SeedlessFusedVerify.swift:4240-4247): prefill chunks with the dense projections and the
     experts, grouped by expert, on the matrix cores.  Tolerance-level agreement with the exact path (normed hidden rows within 2 % rms at the median,
-    the same experts almost everywhere), independent of the chunking, and decode continues from its caches."""
+    the same experts almost everywhere), independent of the chunking (ragged chunks among themselves, chunks of multiples of 64
+    rows among themselves), and decode continues from its caches."""
     cfg, dev, host = small_model
     toks = np.random.default_rng(12).integers(0, cfg.vocab, 48).astype(np.int32)
     exact = env["Engine"](cfg, dev, max_m=64, max_seq_len=128)
@@ -273,7 +274,15 @@ def test_hybrid_prefill_agrees_with_the_exact_rows(env, small_model):
     toks2 = np.concatenate([toks, np.random.default_rng(13).integers(0, cfg.vocab, 592).astype(np.int32)])
     d1 = big.forward_tokens(toks2)
     assert d1 is not None, big.gpu_fault
-    assert same_bits(d1[:48], b)
+    # a call of a multiple of 64 rows runs the recurrence of the GDN layers block-wise (the chunked form of the delta
+    # rule), a ragged one row by row: the two agree to tolerance, and calls cut at multiples of 64 agree bit for bit
+    relb = np.linalg.norm(d1[:48].astype(np.float64) - bf, axis=1) / np.linalg.norm(bf, axis=1)
+    assert np.median(relb) < 0.02 and relb.max() < 0.1, (np.median(relb), relb.max())
+    big2 = env["Engine"](cfg, dev, max_m=768, max_seq_len=800)
+    big2.set_hybrid(True)
+    d2 = np.concatenate([big2.forward_tokens(toks2[:128]), big2.forward_tokens(toks2[128:])])
+    assert same_bits(d2, d1)
+    big2.close()
     ex2 = env["Engine"](cfg, dev, max_m=768, max_seq_len=800)
     d0 = ex2.forward_tokens(toks2)
     assert same_bits(d0[:48], a)       # exact rows: the expert-grouped gate/up stage of large chunks changes no bit
