@@ -267,109 +267,135 @@ struct QmmGroupArgs {
   int y_stride;
 };
 
-constexpr int GQ_G = 4;                       // quantisation groups (64 k) per staged chunk: one barrier per 256 k
-constexpr int GQ_XS = 64 * GQ_G + 8;          // halves per staged row
 // DUAL: two weight matrices of the same shape against the same rows (the experts' gate_proj and up_proj): one
 // staging of X, two weight streams in flight per wave, and y = half(silu(g) * u) of the two rounded results
 // written directly (the SwiGLU of the GEMV path, swiglu16).
-template <bool DUAL>
-__global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
-  // One 32-row tile per pass and one accumulator per wave and matrix (most experts have fewer than 32 rows in a
-  // chunk; an expert with more takes several passes over its weights, which then come from cache).  K % 256 == 0.
+// A pass multiplies RT tiles of 32 gathered rows with the expert's weights: an expert with up to 32 rows takes one
+// pass of one tile (256 k per staged chunk), one with more takes passes of two tiles (128 k per chunk, the same LDS),
+// so that a dequantised operand feeds two matrix instructions and the expert's weights are streamed half as often.
+constexpr int GQ_LDS_HALVES = 2 * 64 * (64 * 2 + 8);      // two staging buffers of 64 rows x 128 k (or 32 rows x 256 k)
+template <bool DUAL, int RT, int G>
+SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* list, int cnt, const uint32_t* const (&wp)[2],
+                         const uint32_t* const (&sp)[2], bool live, int n0) {
   constexpr int NW = DUAL ? 2 : 1;
-  __shared__ __align__(16) uint16_t xs[2][32 * GQ_XS];
-  const int e = blockIdx.y;
-  const int cnt_all = min(a.counts[e], GROUP_CAP);
-  if (cnt_all == 0) return;                              // uniform for the workgroup
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int XS = 64 * G + 8;                         // halves per staged row
+  constexpr int BUF = RT * 32 * XS;                      // halves per staging buffer
+  const int tid = threadIdx.x, lane = tid & 63;
   const int col = lane & 31, hh = lane >> 5;
-  const int n0 = (blockIdx.x * 4 + wave) * 32;
-  const bool live = n0 < a.NE;
-  const size_t wrow = (size_t)e * a.NE + (live ? n0 + col : 0);
-  const int chunks = a.K / (64 * GQ_G);
-  const uint32_t* wp[2] = {a.W + wrow * (a.K / 8), DUAL ? a.W2 + wrow * (a.K / 8) : nullptr};
-  const uint32_t* sp[2] = {a.SB + wrow * (a.K / 64), DUAL ? a.SB2 + wrow * (a.K / 64) : nullptr};
-  for (int r0 = 0; r0 < cnt_all; r0 += 32) {
-    const int cnt = min(cnt_all - r0, 32);
-    const uint16_t* list = a.lists + (size_t)e * GROUP_CAP + r0;
-    // the row this thread stages: 32 rows x GQ_G x 8 pieces of 16 bytes, GQ_G pieces per thread
-    int src = -1;
-    if ((tid >> 3) < cnt) { const int pr = list[tid >> 3]; src = a.x_by_pair ? pr : (pr >> 3); }
-    mf_f16v acc[NW];
+  const int chunks = a.K / (64 * G);
+  // the rows this thread stages: RT x 32 rows x G x 8 pieces of 16 bytes, RT x G pieces per thread
+  int src[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    src[t] = -1;
+    const int row = t * 32 + (tid >> 3);
+    if (row < cnt) { const int pr = list[row]; src[t] = a.x_by_pair ? pr : (pr >> 3); }
+  }
+  mf_f16v acc[RT][NW];
+#pragma unroll
+  for (int t = 0; t < RT; ++t)
 #pragma unroll
     for (int q = 0; q < NW; ++q)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[q][r] = 0.0f;
-    uint4 xr[GQ_G];
-    auto fetch = [&](int c) {
+      for (int r = 0; r < 16; ++r) acc[t][q][r] = 0.0f;
+  uint4 xr[RT][G];
+  auto fetch = [&](int c) {
 #pragma unroll
-      for (int g = 0; g < GQ_G; ++g) {
-        xr[g] = make_uint4(0, 0, 0, 0);
-        if (src >= 0) xr[g] = ld16(a.x + (size_t)src * a.x_stride + (c * GQ_G + g) * 64 + (tid & 7) * 8);
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        xr[t][g] = make_uint4(0, 0, 0, 0);
+        if (src[t] >= 0) xr[t][g] = ld16(a.x + (size_t)src[t] * a.x_stride + (c * G + g) * 64 + (tid & 7) * 8);
       }
-    };
-    auto put = [&](int buf) {
+  };
+  auto put = [&](int buf) {
 #pragma unroll
-      for (int g = 0; g < GQ_G; ++g) st16(&xs[buf][(tid >> 3) * GQ_XS + g * 64 + (tid & 7) * 8], permute8(xr[g]));
-    };
-    uint4 nw[NW][GQ_G];                                  // words 4*hh .. 4*hh+3 of each group (see k_qmm4_mfma16)
-    uint32_t nsb[NW][GQ_G];
-    auto wfetch = [&](int c) {
+    for (int t = 0; t < RT; ++t)
 #pragma unroll
-      for (int q = 0; q < NW; ++q)
-#pragma unroll
-        for (int g = 0; g < GQ_G; ++g) {
-          nw[q][g] = ld16(wp[q] + (c * GQ_G + g) * 8 + 4 * hh);
-          nsb[q][g] = sp[q][c * GQ_G + g];
-        }
-    };
-    __syncthreads();                                     // the pass before has finished reading the staging buffers
-    fetch(0);
-    put(0);
-    if (chunks > 1) fetch(1);
+      for (int g = 0; g < G; ++g) st16(&xsb[buf * BUF + (t * 32 + (tid >> 3)) * XS + g * 64 + (tid & 7) * 8], permute8(xr[t][g]));
+  };
+  uint4 nw[NW][G];                                       // words 4*hh .. 4*hh+3 of each group (see k_qmm4_mfma16)
+  uint32_t nsb[NW][G];
+  auto wfetch = [&](int c) {
 #pragma unroll
     for (int q = 0; q < NW; ++q)
 #pragma unroll
-      for (int g = 0; g < GQ_G; ++g) { nw[q][g] = make_uint4(0, 0, 0, 0); nsb[q][g] = 0; }
-    if (live) wfetch(0);
-    for (int c = 0; c < chunks; ++c) {
-      const int buf = c & 1;
-      uint4 w[NW][GQ_G];
-      uint32_t sb[NW][GQ_G];
-#pragma unroll
-      for (int q = 0; q < NW; ++q)
-#pragma unroll
-        for (int g = 0; g < GQ_G; ++g) { w[q][g] = nw[q][g]; sb[q][g] = nsb[q][g]; }
-      if (live && c + 1 < chunks) wfetch(c + 1);
-      __syncthreads();
-      if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
-#pragma unroll
-      for (int g = 0; g < GQ_G; ++g) {
-#pragma unroll
-        for (int st = 0; st < 4; ++st) {
-          const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][col * GQ_XS + g * 64 + 32 * hh + 8 * st]);
-#pragma unroll
-          for (int q = 0; q < NW; ++q) {
-            const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[q][g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[q][g] >> 16) * 0x10001u);
-            const uint4 w0 = w[q][g];
-            const uint32_t wsel = st == 0 ? w0.x : st == 1 ? w0.y : st == 2 ? w0.z : w0.w;
-            acc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax, dequant8(wsel, s2, b2), acc[q], 0, 0, 0);
-          }
-        }
+      for (int g = 0; g < G; ++g) {
+        nw[q][g] = ld16(wp[q] + (c * G + g) * 8 + 4 * hh);
+        nsb[q][g] = sp[q][c * G + g];
       }
-    }
-    if (live) {
+  };
+  __syncthreads();                                       // the pass before has finished reading the staging buffers
+  fetch(0);
+  put(0);
+  if (chunks > 1) fetch(1);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = 8 * (r >> 2) + 4 * hh + (r & 3);
-        if (row < cnt) {
-          float v = f16r(acc[0][r]);
-          if constexpr (DUAL) v = swiglu16(v, f16r(acc[1][r]));
-          a.y[(size_t)list[row] * a.y_stride + n0 + col] = f2h(v);
+  for (int q = 0; q < NW; ++q)
+#pragma unroll
+    for (int g = 0; g < G; ++g) { nw[q][g] = make_uint4(0, 0, 0, 0); nsb[q][g] = 0; }
+  if (live) wfetch(0);
+  for (int c = 0; c < chunks; ++c) {
+    const int buf = c & 1;
+    uint4 w[NW][G];
+    uint32_t sb[NW][G];
+#pragma unroll
+    for (int q = 0; q < NW; ++q)
+#pragma unroll
+      for (int g = 0; g < G; ++g) { w[q][g] = nw[q][g]; sb[q][g] = nsb[q][g]; }
+    if (live && c + 1 < chunks) wfetch(c + 1);
+    __syncthreads();
+    if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        mf_h8 ax[RT];
+#pragma unroll
+        for (int t = 0; t < RT; ++t) ax[t] = *reinterpret_cast<const mf_h8*>(&xsb[buf * BUF + (t * 32 + col) * XS + g * 64 + 32 * hh + 8 * st]);
+#pragma unroll
+        for (int q = 0; q < NW; ++q) {
+          const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[q][g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[q][g] >> 16) * 0x10001u);
+          const uint4 w0 = w[q][g];
+          const uint32_t wsel = st == 0 ? w0.x : st == 1 ? w0.y : st == 2 ? w0.z : w0.w;
+          const mf_h8 bw = dequant8(wsel, s2, b2);
+#pragma unroll
+          for (int t = 0; t < RT; ++t) acc[t][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax[t], bw, acc[t][q], 0, 0, 0);
         }
       }
     }
   }
+  if (live) {
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+        if (row < cnt) {
+          float v = f16r(acc[t][0][r]);
+          if constexpr (DUAL) v = swiglu16(v, f16r(acc[t][1][r]));
+          a.y[(size_t)list[row] * a.y_stride + n0 + col] = f2h(v);
+        }
+      }
+  }
+}
+template <bool DUAL>
+__global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
+  __shared__ __align__(16) uint16_t xs[GQ_LDS_HALVES];
+  const int e = blockIdx.y;
+  const int cnt_all = min(a.counts[e], GROUP_CAP);
+  if (cnt_all == 0) return;                              // uniform for the workgroup
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 31;
+  const int n0 = (blockIdx.x * 4 + wave) * 32;
+  const bool live = n0 < a.NE;
+  const size_t wrow = (size_t)e * a.NE + (live ? n0 + col : 0);
+  const uint32_t* const wp[2] = {a.W + wrow * (a.K / 8), DUAL ? a.W2 + wrow * (a.K / 8) : nullptr};
+  const uint32_t* const sp[2] = {a.SB + wrow * (a.K / 64), DUAL ? a.SB2 + wrow * (a.K / 64) : nullptr};
+  const uint16_t* lists = a.lists + (size_t)e * GROUP_CAP;
+  int r0 = 0;
+  for (; cnt_all - r0 > 32; r0 += 64)                    // K % 256 == 0 for both shapes
+    grouped_pass<DUAL, 2, 2>(a, xs, lists + r0, min(cnt_all - r0, 64), wp, sp, live, n0);
+  if (r0 < cnt_all) grouped_pass<DUAL, 1, 4>(a, xs, lists + r0, cnt_all - r0, wp, sp, live, n0);
 }
 
 // act = half(silu(g) * u) in half arithmetic, elementwise over [rows, 512] (same rule as the GEMV kernels).
