@@ -24,8 +24,9 @@ typedef _Float16 mf_h2 __attribute__((ext_vector_type(2)));
 // The 8 halves of a staged 16-byte piece (k = 8j .. 8j+7) in the order {0,4,1,5, 2,6,3,7}, the order in which
 // dequant8 delivers the 8 nibbles of a packed word.
 SL_DEV uint4 permute8(uint4 v) {
-  return make_uint4((v.x & 0xffffu) | (v.z << 16), (v.x >> 16) | (v.z & 0xffff0000u),
-                    (v.y & 0xffffu) | (v.w << 16), (v.y >> 16) | (v.w & 0xffff0000u));
+  // v_perm_b32 picks bytes out of {first operand: bytes 4..7, second operand: bytes 0..3}
+  return make_uint4(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
+                    __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));
 }
 
 struct QmmArgs {
@@ -89,17 +90,17 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
   // X chunks travel global -> registers -> LDS one iteration apart: 32*RT rows x 128*G bytes, one 16-byte piece per
-  // thread and pass; rows beyond M are zero
+  // thread and pass.  Rows beyond M repeat row M-1: a row of Y depends on its own row of X only and those rows of Y
+  // are never stored, so the loads need no bounds branch.
   uint4 xr[RT * G];
+  uint32_t xoff[RT];
+#pragma unroll
+  for (int p = 0; p < RT; ++p) xoff[p] = (uint32_t)min(m0 + p * 32 + (tid >> 3), a.M - 1) * (uint32_t)a.x_stride + (tid & 7) * 8;
   auto fetch = [&](int c) {
 #pragma unroll
     for (int p = 0; p < RT; ++p)
 #pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const int row = m0 + p * 32 + (tid >> 3);
-        xr[p * G + g] = make_uint4(0, 0, 0, 0);
-        if (row < a.M) xr[p * G + g] = ld16(a.x + (size_t)row * a.x_stride + (c * G + g) * 64 + (tid & 7) * 8);
-      }
+      for (int g = 0; g < G; ++g) xr[p * G + g] = ld16(a.x + (size_t)(xoff[p] + (uint32_t)((c * G + g) * 64)));
   };
   auto put = [&](int buf) {
 #pragma unroll
@@ -121,19 +122,16 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
   fetch(0);
   put(0);
   if (chunks > 1) fetch(1);
-#pragma unroll
-  for (int g = 0; g < G; ++g) { nw[g] = make_uint4(0, 0, 0, 0); nsb[g] = 0; }
-  if (live) wfetch(0);
+  wfetch(0);                                             // (a wave without a strip works on strip 0 and stores nothing)
   for (int c = 0; c < chunks; ++c) {
     const int buf = c & 1;
     uint4 w[G];
     uint32_t sb[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) { w[g] = nw[g]; sb[g] = nsb[g]; }
-    if (live && c + 1 < chunks) wfetch(c + 1);           // the weights of the next chunk are requested before this one is consumed
+    if (c + 1 < chunks) wfetch(c + 1);                   // the weights of the next chunk are requested before this one is consumed
     __syncthreads();                                     // chunk c is staged; chunk c-1 is no longer read
     if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
-    if (!live) continue;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[g] >> 16) * 0x10001u);
