@@ -56,14 +56,20 @@ struct QmmArgs {
 // -------------------------------------------------------------------------------------------------
 // Dequantisation of a packed word (8 weights) in packed half arithmetic: masking with 0x000F000F leaves the nibbles
 // j and j+4; or-ing a nibble into the mantissa of 1024.0 gives 1024 + q exactly, subtracting 1024 gives q exactly,
-// and half(q * s + b) is one fused multiply-add per pair.
+// and half(q * s + b) is one fused multiply-add per pair.  `k1024` is the pattern 0x64006400 held in a vector
+// register, so that mask and or are one instruction (v_and_or_b32 takes one literal).
 typedef _Float16 mf_h8 __attribute__((ext_vector_type(8)));
-SL_DEV mf_h8 dequant8(uint32_t w, mf_h2 s2, mf_h2 b2) {
-  const mf_h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+SL_DEV uint32_t dequant_k1024() {
+  uint32_t k = 0x64006400u;
+  asm volatile("" : "+v"(k));
+  return k;
+}
+SL_DEV mf_h8 dequant8(uint32_t w, mf_h2 s2, mf_h2 b2, uint32_t k1024) {
+  const mf_h2 f1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
   mf_h8 r;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const mf_h2 q = __builtin_bit_cast(mf_h2, ((w >> (4 * j)) & 0x000F000Fu) | 0x64006400u) - k1024;
+    const mf_h2 q = __builtin_bit_cast(mf_h2, ((w >> (4 * j)) & 0x000F000Fu) | k1024) - f1024;
     const mf_h2 v = __builtin_elementwise_fma(q, s2, b2);
     r[2 * j] = v[0]; r[2 * j + 1] = v[1];
   }
@@ -123,6 +129,7 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
   put(0);
   if (chunks > 1) fetch(1);
   wfetch(0);                                             // (a wave without a strip works on strip 0 and stores nothing)
+  const uint32_t k1024 = dequant_k1024();
   for (int c = 0; c < chunks; ++c) {
     const int buf = c & 1;
     uint4 w[G];
@@ -138,7 +145,7 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
       const uint32_t wsel[4] = {w[g].x, w[g].y, w[g].z, w[g].w};
 #pragma unroll
       for (int st = 0; st < 4; ++st) {
-        const mf_h8 bw = dequant8(wsel[st], s2, b2);
+        const mf_h8 bw = dequant8(wsel[st], s2, b2, k1024);
 #pragma unroll
         for (int t = 0; t < RT; ++t) {
           const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][(t * 32 + col) * XS + g * 64 + 32 * hh + 8 * st]);
@@ -268,26 +275,35 @@ struct QmmGroupArgs {
 // DUAL: two weight matrices of the same shape against the same rows (the experts' gate_proj and up_proj): one
 // staging of X, two weight streams in flight per wave, and y = half(silu(g) * u) of the two rounded results
 // written directly (the SwiGLU of the GEMV path, swiglu16).
-// A pass multiplies RT tiles of 32 gathered rows with the expert's weights: an expert with up to 32 rows takes one
-// pass of one tile (256 k per staged chunk), one with more takes passes of two tiles (128 k per chunk, the same LDS),
-// so that a dequantised operand feeds two matrix instructions and the expert's weights are streamed half as often.
-constexpr int GQ_LDS_HALVES = 2 * 64 * (64 * 2 + 8);      // two staging buffers of 64 rows x 128 k (or 32 rows x 256 k)
+// A pass multiplies RT tiles of 32 gathered rows with the expert's weights, so that a dequantised operand feeds RT
+// matrix instructions and the expert's weights are streamed once per pass: an expert with up to 128 rows takes one
+// pass of ceil(rows / 32) tiles, a larger one passes of four tiles first.  The staged chunk is G quantisation
+// groups wide, narrower for more tiles (the same LDS).  Rows of a tile beyond the expert's count repeat its last
+// row and are not stored; a wave without a strip works on strip 0 and stores nothing.
+// SwiGLU of the matrix-core path: the rounding points of swiglu16 (sigmoid, g * sigmoid and the product with u each
+// rounded to half) with the sigmoid from the hardware exponential and reciprocal, a tenth of the instructions of the
+// bit-exact form (this path is tolerance-level anyway).
+SL_DEV float swiglu_mm(float g, float u) {
+  const float sg = f16r(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g)));
+  return f16r(f16r(g * sg) * u);
+}
+constexpr int GQ_LDS_HALVES = 2 * 128 * (64 + 8);         // two staging buffers of 128 rows x 64 k (the largest shape)
 template <bool DUAL, int RT, int G>
 SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* list, int cnt, const uint32_t* const (&wp)[2],
                          const uint32_t* const (&sp)[2], bool live, int n0) {
   constexpr int NW = DUAL ? 2 : 1;
   constexpr int XS = 64 * G + 8;                         // halves per staged row
   constexpr int BUF = RT * 32 * XS;                      // halves per staging buffer
+  static_assert(2 * BUF <= GQ_LDS_HALVES, "staging buffers exceed the workgroup's LDS");
   const int tid = threadIdx.x, lane = tid & 63;
   const int col = lane & 31, hh = lane >> 5;
   const int chunks = a.K / (64 * G);
   // the rows this thread stages: RT x 32 rows x G x 8 pieces of 16 bytes, RT x G pieces per thread
-  int src[RT];
+  uint32_t xoff[RT];
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
-    src[t] = -1;
-    const int row = t * 32 + (tid >> 3);
-    if (row < cnt) { const int pr = list[row]; src[t] = a.x_by_pair ? pr : (pr >> 3); }
+    const int pr = list[min(t * 32 + (tid >> 3), cnt - 1)];
+    xoff[t] = (uint32_t)(a.x_by_pair ? pr : (pr >> 3)) * (uint32_t)a.x_stride + (tid & 7) * 8;
   }
   mf_f16v acc[RT][NW];
 #pragma unroll
@@ -301,10 +317,7 @@ SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* l
 #pragma unroll
     for (int t = 0; t < RT; ++t)
 #pragma unroll
-      for (int g = 0; g < G; ++g) {
-        xr[t][g] = make_uint4(0, 0, 0, 0);
-        if (src[t] >= 0) xr[t][g] = ld16(a.x + (size_t)src[t] * a.x_stride + (c * G + g) * 64 + (tid & 7) * 8);
-      }
+      for (int g = 0; g < G; ++g) xr[t][g] = ld16(a.x + (size_t)(xoff[t] + (uint32_t)((c * G + g) * 64)));
   };
   auto put = [&](int buf) {
 #pragma unroll
@@ -327,11 +340,8 @@ SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* l
   fetch(0);
   put(0);
   if (chunks > 1) fetch(1);
-#pragma unroll
-  for (int q = 0; q < NW; ++q)
-#pragma unroll
-    for (int g = 0; g < G; ++g) { nw[q][g] = make_uint4(0, 0, 0, 0); nsb[q][g] = 0; }
-  if (live) wfetch(0);
+  wfetch(0);
+  const uint32_t k1024 = dequant_k1024();
   for (int c = 0; c < chunks; ++c) {
     const int buf = c & 1;
     uint4 w[NW][G];
@@ -340,11 +350,17 @@ SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* l
     for (int q = 0; q < NW; ++q)
 #pragma unroll
       for (int g = 0; g < G; ++g) { w[q][g] = nw[q][g]; sb[q][g] = nsb[q][g]; }
-    if (live && c + 1 < chunks) wfetch(c + 1);
+    if (c + 1 < chunks) wfetch(c + 1);
     __syncthreads();
     if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
 #pragma unroll
     for (int g = 0; g < G; ++g) {
+      mf_h2 s2[NW], b2[NW];
+#pragma unroll
+      for (int q = 0; q < NW; ++q) {
+        s2[q] = __builtin_bit_cast(mf_h2, (sb[q][g] & 0xffffu) * 0x10001u);
+        b2[q] = __builtin_bit_cast(mf_h2, (sb[q][g] >> 16) * 0x10001u);
+      }
 #pragma unroll
       for (int st = 0; st < 4; ++st) {
         mf_h8 ax[RT];
@@ -352,10 +368,9 @@ SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* l
         for (int t = 0; t < RT; ++t) ax[t] = *reinterpret_cast<const mf_h8*>(&xsb[buf * BUF + (t * 32 + col) * XS + g * 64 + 32 * hh + 8 * st]);
 #pragma unroll
         for (int q = 0; q < NW; ++q) {
-          const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[q][g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[q][g] >> 16) * 0x10001u);
           const uint4 w0 = w[q][g];
           const uint32_t wsel = st == 0 ? w0.x : st == 1 ? w0.y : st == 2 ? w0.z : w0.w;
-          const mf_h8 bw = dequant8(wsel, s2, b2);
+          const mf_h8 bw = dequant8(wsel, s2[q], b2[q], k1024);
 #pragma unroll
           for (int t = 0; t < RT; ++t) acc[t][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax[t], bw, acc[t][q], 0, 0, 0);
         }
@@ -370,7 +385,7 @@ SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* l
         const int row = t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
         if (row < cnt) {
           float v = f16r(acc[t][0][r]);
-          if constexpr (DUAL) v = swiglu16(v, f16r(acc[t][1][r]));
+          if constexpr (DUAL) v = swiglu_mm(v, f16r(acc[t][1][r]));
           a.y[(size_t)list[row] * a.y_stride + n0 + col] = f2h(v);
         }
       }
@@ -391,9 +406,12 @@ __global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
   const uint32_t* const sp[2] = {a.SB + wrow * (a.K / 64), DUAL ? a.SB2 + wrow * (a.K / 64) : nullptr};
   const uint16_t* lists = a.lists + (size_t)e * GROUP_CAP;
   int r0 = 0;
-  for (; cnt_all - r0 > 32; r0 += 64)                    // K % 256 == 0 for both shapes
-    grouped_pass<DUAL, 2, 2>(a, xs, lists + r0, min(cnt_all - r0, 64), wp, sp, live, n0);
-  if (r0 < cnt_all) grouped_pass<DUAL, 1, 4>(a, xs, lists + r0, cnt_all - r0, wp, sp, live, n0);
+  for (; cnt_all - r0 > 128; r0 += 128) grouped_pass<DUAL, 4, 1>(a, xs, lists + r0, 128, wp, sp, live, n0);
+  const int rest = cnt_all - r0;                         // 1 .. 128; K % 256 == 0 for both shapes
+  if (rest > 96) grouped_pass<DUAL, 4, 1>(a, xs, lists + r0, rest, wp, sp, live, n0);
+  else if (rest > 64) grouped_pass<DUAL, 3, 1>(a, xs, lists + r0, rest, wp, sp, live, n0);
+  else if (rest > 32) grouped_pass<DUAL, 2, 2>(a, xs, lists + r0, rest, wp, sp, live, n0);
+  else grouped_pass<DUAL, 1, 4>(a, xs, lists + r0, rest, wp, sp, live, n0);
 }
 
 // act = half(silu(g) * u) in half arithmetic, elementwise over [rows, 512] (same rule as the GEMV kernels).
