@@ -42,7 +42,36 @@ struct QmmArgs {
   const uint32_t* W2 = nullptr;
   const uint32_t* SB2 = nullptr;
   uint16_t* y2 = nullptr;
+  int col_blocks = 0, row_blocks = 0;   // tiles of the launch (set by launch_qmm4_mfma), see xcd_tile
 };
+
+// Which tile a workgroup takes.  Workgroups go to the 8 XCDs in turn (workgroup n runs on XCD n % 8) and every XCD has
+// an L2 of its own, so the tiles are dealt out by XCD: an XCD owns the row blocks x, x + 8, ... and sweeps the column
+// blocks with them, innermost over its row blocks.  The X rows of its few row blocks then stay in that L2 for the
+// whole sweep and a strip of weights is used by all its row blocks while it is hot, instead of every XCD pulling
+// every block of X through its own L2.  With fewer than 8 row blocks the XCDs that share a row block split the
+// column blocks among them.
+struct TileId { int col_block, row_block; bool valid; };
+SL_DEV TileId xcd_tile(int n, int col_blocks, int row_blocks) {
+  const int x = n & 7, s = n >> 3;
+  TileId t;
+  if (row_blocks >= 8) {
+    const int per = (row_blocks + 7) >> 3;
+    t.row_block = x + 8 * (s % per);
+    t.col_block = s / per;
+  } else {
+    t.row_block = x % row_blocks;
+    const int part = x / row_blocks, sharers = (8 - t.row_block + row_blocks - 1) / row_blocks;
+    t.col_block = s * sharers + part;
+  }
+  t.valid = t.row_block < row_blocks && t.col_block < col_blocks;
+  return t;
+}
+inline unsigned xcd_tile_grid(int col_blocks, int row_blocks) {   // workgroups to launch for xcd_tile
+  if (row_blocks >= 8) return 8u * (unsigned)(((row_blocks + 7) / 8) * col_blocks);
+  const int sharers_min = 8 / row_blocks;
+  return 8u * (unsigned)((col_blocks + sharers_min - 1) / sharers_min);
+}
 
 
 // -------------------------------------------------------------------------------------------------
@@ -64,6 +93,11 @@ SL_DEV uint32_t dequant_k1024() {
   asm volatile("" : "+v"(k));
   return k;
 }
+SL_DEV mf_h2 dequant_pair(uint32_t w, int j, mf_h2 s2, mf_h2 b2, uint32_t k1024) {   // nibbles j and j+4
+  const mf_h2 f1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+  const mf_h2 q = __builtin_bit_cast(mf_h2, ((w >> (4 * j)) & 0x000F000Fu) | k1024) - f1024;
+  return __builtin_elementwise_fma(q, s2, b2);
+}
 SL_DEV mf_h8 dequant8(uint32_t w, mf_h2 s2, mf_h2 b2, uint32_t k1024) {
   const mf_h2 f1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
   mf_h8 r;
@@ -75,94 +109,161 @@ SL_DEV mf_h8 dequant8(uint32_t w, mf_h2 s2, mf_h2 b2, uint32_t k1024) {
   }
   return r;
 }
-template <int RT, int G>      // G quantisation groups (64 k) per staged chunk and barrier; K % (64*G) == 0
-__global__ __launch_bounds__(256) void k_qmm4_mfma16(QmmArgs a) {
-  constexpr int XS = 64 * G + 8;                         // halves per staged row (rows 16 bytes off a multiple of 128)
+// The rows of a chunk on their way global -> registers -> LDS: ROWS rows x G groups x 8 pieces of 16 bytes, dealt out
+// to the NT threads of the workgroup in passes (piece index = pass * NT + thread; pieces past the end repeat the
+// last one, harmlessly).  `row_offset(row)` gives the element offset of a row of the tile in X.
+template <int ROWS, int G, int NT>
+struct RowStager {
+  static constexpr int XS = 64 * G + 8;                  // halves per staged row (rows 16 bytes off a multiple of 128)
+  static constexpr int TOTAL = ROWS * G * 8, PASSES = (TOTAL + NT - 1) / NT;
+  uint32_t src[PASSES];                                  // element offset in X of the thread's piece within chunk 0
+  uint32_t dst[PASSES];                                  // halves offset in a staging buffer
+  uint4 r[PASSES];
+  template <typename F>
+  SL_DEV void init(int tid, F row_offset) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int idx = min(p * NT + tid, TOTAL - 1);
+      const int piece = idx & 7, row = (idx >> 3) % ROWS, g = (idx >> 3) / ROWS;
+      src[p] = row_offset(row) + (uint32_t)(g * 64 + piece * 8);
+      dst[p] = (uint32_t)(row * XS + g * 64 + piece * 8);
+    }
+  }
+  SL_DEV void fetch(const uint16_t* x, int c) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) r[p] = ld16(x + (size_t)(src[p] + (uint32_t)(c * G * 64)));
+  }
+  SL_DEV void put(uint16_t* buf) const {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) st16(buf + dst[p], permute8(r[p]));
+  }
+};
+
+// A SIMD issues one instruction at a time: unpacking, LDS reads and staging all take issue slots next to the matrix
+// instructions instead of hiding behind them, so the kernel's speed is set by the instructions per matrix
+// instruction.  A wave therefore owns NS strips of 32 weight rows and RT x 32 rows of X (RT x NS accumulators): a row
+// operand read from LDS feeds NS matrix instructions, an unpacked weight operand RT, and the staged rows are shared
+// by the WPB waves of the workgroup.
+template <int RT, int NS, int G, int WPB>      // G quantisation groups (64 k) per staged chunk and barrier; K % (64*G) == 0
+__global__ __launch_bounds__(64 * WPB) void k_qmm4_mfma16(QmmArgs a) {
+  constexpr int NT = 64 * WPB;
+  using Stage = RowStager<RT * 32, G, NT>;
+  constexpr int XS = Stage::XS;
   __shared__ __align__(16) uint16_t xs[2][RT * 32 * XS];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, hh = lane >> 5;
-  const int n0 = (blockIdx.x * 4 + wave) * 32;
-  const int m0 = blockIdx.y * RT * 32;
-  const bool live = n0 < a.N;                            // the last workgroup's waves may have no strip
-  const size_t wrow = (size_t)(live ? n0 + col : 0);
+  const TileId tile = xcd_tile((int)blockIdx.x, a.col_blocks, a.row_blocks);
+  if (!tile.valid) return;                               // uniform for the workgroup
+  const int n0 = (tile.col_block * WPB + wave) * NS * 32;  // first of the wave's NS neighbouring strips
+  const int m0 = tile.row_block * RT * 32;
   const int chunks = a.K / (64 * G);
   const bool second = blockIdx.z != 0;
-  const uint32_t* wp = (second ? a.W2 : a.W) + wrow * (a.K / 8);
-  const uint32_t* sp = (second ? a.SB2 : a.SB) + wrow * (a.K / 64);
+  const uint32_t* wp[NS];
+  const uint32_t* sp[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {                         // (a strip beyond N works on strip 0 and stores nothing)
+    const size_t wrow = (size_t)(n0 + 32 * s < a.N ? n0 + 32 * s + col : 0);
+    wp[s] = (second ? a.W2 : a.W) + wrow * (a.K / 8);
+    sp[s] = (second ? a.SB2 : a.SB) + wrow * (a.K / 64);
+  }
   uint16_t* yout = second ? a.y2 : a.y;
-  mf_f16v acc[RT];
+  mf_f16v acc[RT][NS];
 #pragma unroll
   for (int t = 0; t < RT; ++t)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
-  // X chunks travel global -> registers -> LDS one iteration apart: 32*RT rows x 128*G bytes, one 16-byte piece per
-  // thread and pass.  Rows beyond M repeat row M-1: a row of Y depends on its own row of X only and those rows of Y
-  // are never stored, so the loads need no bounds branch.
-  uint4 xr[RT * G];
-  uint32_t xoff[RT];
+    for (int s = 0; s < NS; ++s)
 #pragma unroll
-  for (int p = 0; p < RT; ++p) xoff[p] = (uint32_t)min(m0 + p * 32 + (tid >> 3), a.M - 1) * (uint32_t)a.x_stride + (tid & 7) * 8;
-  auto fetch = [&](int c) {
-#pragma unroll
-    for (int p = 0; p < RT; ++p)
-#pragma unroll
-      for (int g = 0; g < G; ++g) xr[p * G + g] = ld16(a.x + (size_t)(xoff[p] + (uint32_t)((c * G + g) * 64)));
-  };
-  auto put = [&](int buf) {
-#pragma unroll
-    for (int p = 0; p < RT; ++p)
-#pragma unroll
-      for (int g = 0; g < G; ++g) st16(&xs[buf][(p * 32 + (tid >> 3)) * XS + g * 64 + (tid & 7) * 8], permute8(xr[p * G + g]));
-  };
+      for (int r = 0; r < 16; ++r) acc[t][s][r] = 0.0f;
+  // Rows beyond M repeat row M-1: a row of Y depends on its own row of X only and those rows of Y are never stored,
+  // so the loads need no bounds branch.
+  Stage stage;
+  stage.init(tid, [&](int row) { return (uint32_t)min(m0 + row, a.M - 1) * (uint32_t)a.x_stride; });
   // of a group's 8 packed words the lower half-wave takes words 0..3 and the upper 4..7 (one 16-byte load each):
   // step st multiplies the k of word st (lower) and of word 4+st (upper), on the A side as well
-  uint4 nw[G];
-  uint32_t nsb[G];
+  uint4 nw[NS][G];
+  uint32_t nsb[NS][G];
   auto wfetch = [&](int c) {
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      nw[g] = ld16(wp + (c * G + g) * 8 + 4 * hh);
-      nsb[g] = sp[c * G + g];
-    }
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        nw[s][g] = ld16(wp[s] + (c * G + g) * 8 + 4 * hh);
+        nsb[s][g] = sp[s][c * G + g];
+      }
   };
-  fetch(0);
-  put(0);
-  if (chunks > 1) fetch(1);
-  wfetch(0);                                             // (a wave without a strip works on strip 0 and stores nothing)
+  stage.fetch(a.x, 0);
+  stage.put(xs[0]);
+  if (chunks > 1) stage.fetch(a.x, 1);
+  wfetch(0);
   const uint32_t k1024 = dequant_k1024();
   for (int c = 0; c < chunks; ++c) {
     const int buf = c & 1;
-    uint4 w[G];
-    uint32_t sb[G];
+    uint4 w[NS][G];
+    uint32_t sb[NS][G];
 #pragma unroll
-    for (int g = 0; g < G; ++g) { w[g] = nw[g]; sb[g] = nsb[g]; }
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+      for (int g = 0; g < G; ++g) { w[s][g] = nw[s][g]; sb[s][g] = nsb[s][g]; }
     if (c + 1 < chunks) wfetch(c + 1);                   // the weights of the next chunk are requested before this one is consumed
     __syncthreads();                                     // chunk c is staged; chunk c-1 is no longer read
-    if (c + 1 < chunks) { put(buf ^ 1); if (c + 2 < chunks) fetch(c + 2); }
+    if (c + 1 < chunks) { stage.put(xs[buf ^ 1]); if (c + 2 < chunks) stage.fetch(a.x, c + 2); }
+    // The chunk's G x 4 steps in one software pipeline: the pairs of the next step's weights are unpacked between
+    // this step's matrix instructions (the scheduling fences keep that order) and the next step's rows are read from
+    // LDS at the start of the step.
+    constexpr int S = G * 4;
+    auto word = [&](int s, int st) { const uint4 v = w[s][st >> 2]; return (st & 3) == 0 ? v.x : (st & 3) == 1 ? v.y : (st & 3) == 2 ? v.z : v.w; };
+    auto scale = [&](int s, int st) { return __builtin_bit_cast(mf_h2, (sb[s][st >> 2] & 0xffffu) * 0x10001u); };
+    auto bias = [&](int s, int st) { return __builtin_bit_cast(mf_h2, (sb[s][st >> 2] >> 16) * 0x10001u); };
+    auto rows = [&](int st, int t) {
+      return *reinterpret_cast<const mf_h8*>(&xs[buf][(t * 32 + col) * XS + (st >> 2) * 64 + 32 * hh + 8 * (st & 3)]);
+    };
+    mf_h8 bw[NS], ax[RT];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const mf_h2 s2 = __builtin_bit_cast(mf_h2, (sb[g] & 0xffffu) * 0x10001u), b2 = __builtin_bit_cast(mf_h2, (sb[g] >> 16) * 0x10001u);
-      const uint32_t wsel[4] = {w[g].x, w[g].y, w[g].z, w[g].w};
+    for (int s = 0; s < NS; ++s) bw[s] = dequant8(word(s, 0), scale(s, 0), bias(s, 0), k1024);
 #pragma unroll
-      for (int st = 0; st < 4; ++st) {
-        const mf_h8 bw = dequant8(wsel[st], s2, b2, k1024);
+    for (int t = 0; t < RT; ++t) ax[t] = rows(0, t);
+#pragma unroll
+    for (int st = 0; st < S; ++st) {
+      mf_h8 axn[RT], bwn[NS];
+      if (st + 1 < S) {
+#pragma unroll
+        for (int t = 0; t < RT; ++t) axn[t] = rows(st + 1, t);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
 #pragma unroll
         for (int t = 0; t < RT; ++t) {
-          const mf_h8 ax = *reinterpret_cast<const mf_h8*>(&xs[buf][(t * 32 + col) * XS + g * 64 + 32 * hh + 8 * st]);
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax, bw, acc[t], 0, 0, 0);
+          acc[t][s] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax[t], bw[s], acc[t][s], 0, 0, 0);
+          if (st + 1 < S) {                              // strip s's next word is unpacked behind strip s's products
+#pragma unroll
+            for (int j = 4 * t / RT; j < 4 * (t + 1) / RT; ++j) {
+              const mf_h2 v = dequant_pair(word(s, st + 1), j, scale(s, st + 1), bias(s, st + 1), k1024);
+              bwn[s][2 * j] = v[0]; bwn[s][2 * j + 1] = v[1];
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
+      if (st + 1 < S) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) bw[s] = bwn[s];
+#pragma unroll
+        for (int t = 0; t < RT; ++t) ax[t] = axn[t];
       }
     }
   }
-  if (!live) return;
   // D layout of a 32x32 tile: register r of lane (col, hh) holds row 8*(r/4) + 4*hh + r%4, column col
 #pragma unroll
-  for (int t = 0; t < RT; ++t)
+  for (int s = 0; s < NS; ++s) {
+    if (n0 + 32 * s >= a.N) continue;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int m = m0 + t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-      if (m < a.M) yout[(size_t)m * a.y_stride + n0 + col] = f2h(acc[t][r]);
-    }
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+        if (m < a.M) yout[(size_t)m * a.y_stride + n0 + 32 * s + col] = f2h(acc[t][s][r]);
+      }
+  }
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -392,7 +493,7 @@ SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* l
   }
 }
 template <bool DUAL>
-__global__ __launch_bounds__(256) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
+__global__ __launch_bounds__(256, 2) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
   __shared__ __align__(16) uint16_t xs[GQ_LDS_HALVES];
   const int e = blockIdx.y;
   const int cnt_all = min(a.counts[e], GROUP_CAP);
@@ -433,8 +534,6 @@ __global__ __launch_bounds__(256) void k_moe_combine_rows(const uint16_t* __rest
   out[(size_t)m * H + n] = f2h(f16r(acc + f16r(s * h2f(sy[(size_t)m * H + n]))));
 }
 
-// Host-side launch: row tiles per wave chosen so that there are about as many wave tasks as SIMDs (1024): wide
-// projections share the unpacking over 128 rows, narrow ones spread their rows over more waves instead.
 // -------------------------------------------------------------------------------------------------
 // Attention of a prefill chunk on the matrix cores (hybrid mode): the tile pass of k_sdpa_tile for 32 query rows of
 // one sequence at a time.  Workgroup = (key tile of 64, kv head, block of 32 rows); the tile's keys [key][dim] and
@@ -781,21 +880,28 @@ __global__ __launch_bounds__(1024) void k_argmax_logits(const uint16_t* __restri
   if (tid == 0) tok_out[out_off + m] = s_i[0];
 }
 
-template <int RT>
-inline void launch_qmm4_rt(const QmmArgs& a, dim3 grid, hipStream_t stream) {
-  const dim3 block(256);
-  constexpr int GMAX = RT == 1 ? 4 : 2;                  // staging buffers of at most ~70 KB
-  if (GMAX == 4 && a.K % 256 == 0) hipLaunchKernelGGL((k_qmm4_mfma16<RT, GMAX>), grid, block, 0, stream, a);
-  else if (a.K % 128 == 0) hipLaunchKernelGGL((k_qmm4_mfma16<RT, 2>), grid, block, 0, stream, a);
-  else hipLaunchKernelGGL((k_qmm4_mfma16<RT, 1>), grid, block, 0, stream, a);
+template <int RT, int NS, int WPB>
+inline void launch_qmm4_rt(QmmArgs a, int row_blocks, unsigned nz, hipStream_t stream) {
+  const dim3 block(64 * WPB);
+  a.col_blocks = (a.N / 32 + WPB * NS - 1) / (WPB * NS);
+  a.row_blocks = row_blocks;
+  const dim3 grid(xcd_tile_grid(a.col_blocks, a.row_blocks), 1, nz);
+  constexpr int GMAX = RT == 1 ? 4 : NS == 2 ? 1 : 2;    // staging buffers of at most ~70 KB; two strips per wave leave registers for one group
+  if (GMAX == 4 && a.K % 256 == 0) hipLaunchKernelGGL((k_qmm4_mfma16<RT, NS, GMAX, WPB>), grid, block, 0, stream, a);
+  else if (GMAX >= 2 && a.K % 128 == 0) hipLaunchKernelGGL((k_qmm4_mfma16<RT, NS, 2, WPB>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((k_qmm4_mfma16<RT, NS, 1, WPB>), grid, block, 0, stream, a);
 }
+// Host-side launch: row tiles per wave chosen so that there are at least about as many wave tasks as SIMDs (1024):
+// wide projections of many rows share the unpacking over 128 rows, narrow ones spread over more waves instead.
+// (Two strips per wave, NS = 2, halve the LDS reads and the staging per matrix instruction but measured slower on
+// the 2048 x 12352 x 2048 projection, 136-146 us against 129 us: 784 workgroups of one per compute unit leave a
+// fourth round of 16, and one wave per SIMD has nothing to run while it waits at the chunk barrier.)
 inline void launch_qmm4_mfma(const QmmArgs& a, hipStream_t stream) {
   const unsigned nz = a.W2 ? 2 : 1;
   const int strips = a.N / 32 * (int)nz, tiles = (a.M + 31) / 32;
-  const unsigned gx = (unsigned)((a.N / 32 + 3) / 4);
-  if (tiles >= 4 && strips * (tiles / 4) >= 768) launch_qmm4_rt<4>(a, dim3(gx, (unsigned)((tiles + 3) / 4), nz), stream);
-  else if (tiles >= 2 && strips * (tiles / 2) >= 768) launch_qmm4_rt<2>(a, dim3(gx, (unsigned)((tiles + 1) / 2), nz), stream);
-  else launch_qmm4_rt<1>(a, dim3(gx, (unsigned)tiles, nz), stream);
+  if (tiles >= 4 && strips * (tiles / 4) >= 768) launch_qmm4_rt<4, 1, 4>(a, (tiles + 3) / 4, nz, stream);
+  else if (tiles >= 2 && strips * (tiles / 2) >= 768) launch_qmm4_rt<2, 1, 4>(a, (tiles + 1) / 2, nz, stream);
+  else launch_qmm4_rt<1, 1, 4>(a, tiles, nz, stream);
 }
 
 }  // namespace sl
