@@ -382,7 +382,7 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
   if (!lanes && M >= 2) {
     // rows of one sequence: the state-independent part for all rows at once, then the scan without barriers
     GdnPrepArgs pa{g, e->gdn_qn, e->gdn_kn, e->gdn_vc, e->gdn_gb};
-    hipLaunchKernelGGL(k_gdn_prep_rows, dim3(65, M), dim3(64), 0, e->stream, pa);
+    hipLaunchKernelGGL(k_gdn_prep_rows, dim3(65, (M + GDN_PREP_ROWS - 1) / GDN_PREP_ROWS), dim3(64), 0, e->stream, pa);
     if (mm && e->gc_scratch && M % GC == 0 && e->pos % GC == 0) {
       // hybrid chunks cut at multiples of 64 rows: the delta rule in its chunked form on the matrix cores
       GdnChunkArgs ca{e->gdn_qn, e->gdn_kn, e->gdn_vc, e->gdn_gb, e->gc_scratch, {L.state[0], L.state[1]}, {L.hist[0], L.hist[1]},

@@ -493,32 +493,60 @@ struct GdnPrepArgs {
   uint16_t* vc;              // [M, 4096] conv + silu of the value channels
   float* gb;                 // [M, 64]: decay g of the 32 value heads, then beta
 };
-// One wave per (unit, row): units 0..15 query heads, 16..31 key heads, 32..63 value heads, 64 decay / beta.
+// One wave per (unit, block of GDN_PREP_ROWS rows): units 0..15 query heads, 16..31 key heads, 32..63 value heads,
+// 64 decay / beta.  A wave walks its rows with the conv window in registers (a row's four taps are the three rows
+// before it and itself: every row of the projection is loaded once, all loads of the block up front), which also
+// keeps the number of waves of a 2048-row chunk at 8320 instead of one per row and unit.  The arithmetic per row is
+// that of conv_silu.
+constexpr int GDN_PREP_ROWS = 16;
 __global__ __launch_bounds__(64) void k_gdn_prep_rows(GdnPrepArgs p) {
   const GdnArgs& a = p.g;
-  const int u = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+  const int u = blockIdx.x, t0 = blockIdx.y * GDN_PREP_ROWS, lane = threadIdx.x;
+  const int rows = min(GDN_PREP_ROWS, a.M - t0);
   const uint16_t* hin = a.st[1] ? a.hist[1] : a.hist[0];
-  if (u < 32) {
-    const bool isk = u >= 16;
-    const int ch = (isk ? 2048 : 0) + (u & 15) * 128 + 2 * lane;
-    const float x0 = conv_silu(a.proj, a.conv_w, hin, t, ch), x1 = conv_silu(a.proj, a.conv_w, hin, t, ch + 1);
-    float ss = fmaf(x1, x1, fmaf(x0, x0, 0.0f));
-    ss = tree_sum<64>(ss);
-    const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
+  if (u < 64) {
+    const bool isq = u < 16, isk = u >= 16 && u < 32;
+    const int ch = u < 32 ? (isk ? 2048 : 0) + (u & 15) * 128 + 2 * lane : 4096 + (u - 32) * 128 + 2 * lane;
+    // rows t0 .. t0 + rows + 2 of the concatenation [hist(3) | qkv(M)], two neighbouring channels per lane
+    uint32_t win[GDN_PREP_ROWS + 3];
+#pragma unroll
+    for (int j = 0; j < GDN_PREP_ROWS + 3; ++j) {
+      const int row = min(t0 + j, t0 + rows + 2);
+      win[j] = (row < 3) ? *reinterpret_cast<const uint32_t*>(hin + row * SL_CONV_DIM + ch)
+                         : *reinterpret_cast<const uint32_t*>(a.proj + (size_t)(row - 3) * PROJ_STRIDE + ch);
+    }
+    float w0[4], w1[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { w0[k] = a.conv_w[ch * 4 + k]; w1[k] = a.conv_w[(ch + 1) * 4 + k]; }
     const float sc = isk ? f16r(0.08838834764831845f) : f16r(0.0078125f);
-    const float y0 = f16r(sc * f16r(x0 * inv)), y1 = f16r(sc * f16r(x1 * inv));
-    *reinterpret_cast<uint32_t*>((isk ? p.kn : p.qn) + (size_t)t * 2048 + (u & 15) * 128 + 2 * lane) = pack2(y0, y1);
-  } else if (u < 64) {
-    const int ch = 4096 + (u - 32) * 128 + 2 * lane;
-    *reinterpret_cast<uint32_t*>(p.vc + (size_t)t * 4096 + (u - 32) * 128 + 2 * lane) =
-        pack2(conv_silu(a.proj, a.conv_w, hin, t, ch), conv_silu(a.proj, a.conv_w, hin, t, ch + 1));
+#pragma unroll
+    for (int j = 0; j < GDN_PREP_ROWS; ++j) {
+      if (j >= rows) break;
+      const int t = t0 + j;
+      float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) { a0 = fmaf(lo_h(win[j + k]), w0[k], a0); a1 = fmaf(hi_h(win[j + k]), w1[k], a1); }
+      const float x0 = f16r(a0 * sigmoid32(a0)), x1 = f16r(a1 * sigmoid32(a1));
+      if (isq || isk) {
+        float ss = fmaf(x1, x1, fmaf(x0, x0, 0.0f));
+        ss = tree_sum<64>(ss);
+        const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
+        const float y0 = f16r(sc * f16r(x0 * inv)), y1 = f16r(sc * f16r(x1 * inv));
+        *reinterpret_cast<uint32_t*>((isk ? p.kn : p.qn) + (size_t)t * 2048 + (u & 15) * 128 + 2 * lane) = pack2(y0, y1);
+      } else {
+        *reinterpret_cast<uint32_t*>(p.vc + (size_t)t * 4096 + (u - 32) * 128 + 2 * lane) = pack2(x0, x1);
+      }
+    }
   } else {
     const int hv = lane & 31;
-    if (lane < 32) {
-      const float aP = h2f(a.proj[(size_t)t * PROJ_STRIDE + 12320 + hv]);
-      p.gb[(size_t)t * 64 + hv] = exp_c(-(exp_c(a.a_log[hv]) * softplus_c(aP + a.dt_bias[hv])));
-    } else {
-      p.gb[(size_t)t * 64 + 32 + hv] = sigmoid16(h2f(a.proj[(size_t)t * PROJ_STRIDE + 12288 + hv]));
+    for (int j = 0; j < rows; ++j) {
+      const int t = t0 + j;
+      if (lane < 32) {
+        const float aP = h2f(a.proj[(size_t)t * PROJ_STRIDE + 12320 + hv]);
+        p.gb[(size_t)t * 64 + hv] = exp_c(-(exp_c(a.a_log[hv]) * softplus_c(aP + a.dt_bias[hv])));
+      } else {
+        p.gb[(size_t)t * 64 + 32 + hv] = sigmoid16(h2f(a.proj[(size_t)t * PROJ_STRIDE + 12288 + hv]));
+      }
     }
   }
 }
