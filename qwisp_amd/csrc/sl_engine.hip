@@ -298,11 +298,11 @@ void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   else
     hipLaunchKernelGGL(k_moe_a, dim3(router_blocks, M), dim3(256), 0, e->stream, a);
   hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, E, L.route_inds, L.route_scores);
-  hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, E, e->hy_lists, e->hy_counts);
+  hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, E, e->hy_lists, e->hy_counts, e->hy_counts + SL_MAX_EXPERTS);
   // routed gate and up by expert in one pass with SwiGLU, then routed down by expert
-  QmmGroupArgs g{e->xn, H, 0, L.sw_gate.w, L.sw_gate.sb, L.sw_up.w, L.sw_up.sb, SL_MOE_I, H, e->hy_lists, e->hy_counts, e->act, SL_MOE_I};
+  QmmGroupArgs g{e->xn, H, 0, L.sw_gate.w, L.sw_gate.sb, L.sw_up.w, L.sw_up.sb, SL_MOE_I, H, e->hy_lists, e->hy_counts, e->hy_counts + SL_MAX_EXPERTS, e->act, SL_MOE_I};
   hipLaunchKernelGGL(k_qmm4_mfma_grouped<true>, dim3(SL_MOE_I / 128, E), dim3(256), 0, e->stream, g);
-  QmmGroupArgs d{e->act, SL_MOE_I, 1, L.sw_down.w, L.sw_down.sb, nullptr, nullptr, H, SL_MOE_I, e->hy_lists, e->hy_counts, e->hy_d, H};
+  QmmGroupArgs d{e->act, SL_MOE_I, 1, L.sw_down.w, L.sw_down.sb, nullptr, nullptr, H, SL_MOE_I, e->hy_lists, e->hy_counts, e->hy_counts + SL_MAX_EXPERTS, e->hy_d, H};
   hipLaunchKernelGGL(k_qmm4_mfma_grouped<false>, dim3(H / 128, E), dim3(256), 0, e->stream, d);
   // shared expert
   launch_qmm4_mfma(QmmArgs{e->xn, H, L.sh_gate.w, L.sh_gate.sb, M, SL_MOE_I, H, e->hy_sg, SL_MOE_I, L.sh_up.w, L.sh_up.sb, e->hy_su}, e->stream);
@@ -328,7 +328,7 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   b.xn = e->xn; b.g_w = L.sw_gate.w; b.g_sb = L.sw_gate.sb; b.u_w = L.sw_up.w; b.u_sb = L.sw_up.sb;
   b.act = e->act; b.inds = L.route_inds;
   if (M >= MOE_GROUP_MIN_ROWS && M <= GROUP_CAP) {      // weights of an expert fetched once for all rows that chose it
-    hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, e->n_experts, e->hy_lists, e->hy_counts);
+    hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, e->n_experts, e->hy_lists, e->hy_counts, (int32_t*)nullptr);
     MoeBGroupArgs g{e->xn, b.g_w, b.g_sb, b.u_w, b.u_sb, e->act, e->hy_lists, e->hy_counts};
     hipLaunchKernelGGL(k_moe_b_grouped, dim3(64, e->n_experts), dim3(256), 0, e->stream, g);
   } else {
@@ -700,7 +700,7 @@ int alloc_runtime(sl_engine* e) {
   e->rlogits = dalloc<uint16_t>(e, (size_t)max_m * 256, true); e->sgate = dalloc<uint16_t>(e, max_m, true);
   e->sh_act = dalloc<uint16_t>(e, (size_t)max_m * 512, true); e->act = dalloc<uint16_t>(e, (size_t)max_m * 8 * 512, true);
   e->hy_lists = dalloc<uint16_t>(e, (size_t)SL_MAX_EXPERTS * GROUP_CAP, true);
-  e->hy_counts = dalloc<int32_t>(e, SL_MAX_EXPERTS, true);
+  e->hy_counts = dalloc<int32_t>(e, 2 * SL_MAX_EXPERTS, true);    // counts, then the experts ordered by falling count
   e->moe_out = dalloc<uint16_t>(e, MH, true); e->normed = dalloc<uint16_t>(e, MH, true);
   e->rows_out = dalloc<uint16_t>(e, MH, true);
   e->gdn_qn = dalloc<uint16_t>(e, MH, true); e->gdn_kn = dalloc<uint16_t>(e, MH, true);

@@ -826,8 +826,10 @@ struct MoeBArgs {
 constexpr int GROUP_CAP = 2048;         // pairs per expert: an expert is chosen at most once per row, M <= 2048
 // Pairs (row, slot) listed per expert (M * 8 pairs walked by 1024 threads), places handed out by LDS counters.
 // The order within a list varies from run to run; results do not depend on it (they are scattered back by pair).
+// `order` (optional) receives the experts sorted by falling count, ties by index: kernels whose workgroups are
+// dealt out by expert start the long ones first, which shortens the tail of the launch.
 __global__ __launch_bounds__(1024) void k_group_pairs(const int32_t* __restrict__ inds, int M, int E, uint16_t* __restrict__ lists,
-                                                      int32_t* __restrict__ counts) {
+                                                      int32_t* __restrict__ counts, int32_t* __restrict__ order) {
   __shared__ int s_cnt[SL_MAX_EXPERTS];
   if (threadIdx.x < SL_MAX_EXPERTS) s_cnt[threadIdx.x] = 0;
   __syncthreads();
@@ -839,7 +841,15 @@ __global__ __launch_bounds__(1024) void k_group_pairs(const int32_t* __restrict_
     }
   }
   __syncthreads();
-  if ((int)threadIdx.x < E) counts[threadIdx.x] = s_cnt[threadIdx.x];
+  if ((int)threadIdx.x < E) {
+    const int e = threadIdx.x, c = s_cnt[e];
+    counts[e] = c;
+    if (order) {
+      int rank = 0;
+      for (int j = 0; j < E; ++j) rank += (s_cnt[j] > c || (s_cnt[j] == c && j < e)) ? 1 : 0;
+      order[rank] = e;
+    }
+  }
 }
 // Stage B by expert (steps of many rows): grid (64, E).  A workgroup holds eight gate/up row pairs of one expert
 // (two pairs per wave, unpacked into masks once) and walks the expert's list of (row, slot) pairs in tiles of

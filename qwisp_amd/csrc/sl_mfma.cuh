@@ -369,6 +369,7 @@ struct QmmGroupArgs {
   int NE, K;
   const uint16_t* lists; // [E, GROUP_CAP] pair indices
   const int32_t* counts; // [E]
+  const int32_t* order;  // [E] experts by falling count: blockIdx.y walks this order
   uint16_t* y;           // [pairs, y_stride]
   int y_stride;
 };
@@ -495,7 +496,7 @@ SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* l
 template <bool DUAL>
 __global__ __launch_bounds__(256, 2) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
   __shared__ __align__(16) uint16_t xs[GQ_LDS_HALVES];
-  const int e = blockIdx.y;
+  const int e = a.order[blockIdx.y];
   const int cnt_all = min(a.counts[e], GROUP_CAP);
   if (cnt_all == 0) return;                              // uniform for the workgroup
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
