@@ -130,9 +130,12 @@ def main():
     ap.add_argument("--lane-contexts", choices=("mixed", "short"), default="mixed",
                     help="contexts of the --lanes sequences: mixed = 1K to 16K tokens spread evenly over the lanes (prefilled "
                          "on the matrix cores first), short = 8 to 56 tokens")
-    ap.add_argument("--prefill-chunk", type=int, default=1024, metavar="M",
+    ap.add_argument("--prefill-chunk", type=int, default=2048, metavar="M",
                     help="also time a prefill in chunks of M rows, exact rows and hybrid (matrix cores), on lanes "
-                         "of the same weights (extra object in the JSON line; 0 = skip)")
+                         "of the same weights (extra object in the JSON line; 0 = skip); 2048 is the chunk of the "
+                         "reference's batched configuration")
+    ap.add_argument("--prefill-also", default="1024", metavar="M,M",
+                    help="further chunk sizes timed in hybrid mode only (the reference's own default chunk is 1024)")
     ap.add_argument("--prefill-tokens", type=int, default=2048, metavar="N",
                     help="prompt length of the --prefill-chunk measurement (the reference's batched configuration uses 2048)")
     ap.add_argument("--verify-rows", type=int, default=4, metavar="R",
@@ -306,6 +309,19 @@ def main():
                 assert o is not None, lane.gpu_fault
                 lane.close()
             prefill_report[name] = {"ms": times[-1] * 1e3, "tok_s": PF / times[-1]}
+        for m in [int(x) for x in args.prefill_also.split(",") if x]:
+            times = []
+            for rep in range(2):
+                lane = eng.new_lane(max_m=m, max_seq_len=PF + 8)
+                lane.set_hybrid(True)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                o = lane.greedy_generate(pf_prompt, 1, chain_k=1)
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                assert o is not None, lane.gpu_fault
+                lane.close()
+            prefill_report.setdefault("hybrid_other_chunks", {})[str(m)] = {"ms": times[-1] * 1e3, "tok_s": PF / times[-1]}
 
     sweep_report = None
     if args.context_sweep:
