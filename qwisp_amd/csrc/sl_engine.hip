@@ -433,10 +433,19 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
     const int T = tiles >= 32 ? 4 : (tiles >= 8 ? 2 : 1);
     hipLaunchKernelGGL(k_sdpa_lane_mfma, dim3((tiles + T - 1) / T, SL_ATT_KV, M), dim3(256), 0, e->stream, SdpaLaneArgs{s, T});
   }
-  else if (mm) hipLaunchKernelGGL(k_sdpa_tile_mfma, dim3(tiles, SL_ATT_KV, (M + 31) / 32), dim3(256), 0, e->stream, SdpaMmArgs{s, M});
-  else hipLaunchKernelGGL(k_sdpa_tile, dim3(tiles, SL_ATT_KV, M), dim3(256), 0, e->stream, s);
+  int tiles_per_part = 0;
+  if (mm && !lanes) {
+    // parts of SDPA_FLASH_TILES key tiles at fixed positions: a row's tiles are then added up in the same grouping
+    // whatever the chunking of the prompt, so the result of a row does not depend on it
+    const int row_blocks = (M + 31) / 32;
+    tiles_per_part = SDPA_FLASH_TILES;
+    const int parts = (tiles + tiles_per_part - 1) / tiles_per_part;
+    hipLaunchKernelGGL(k_sdpa_flash_mfma, dim3(parts, SL_ATT_KV, row_blocks), dim3(512), 0, e->stream, SdpaFlashArgs{s, M, tiles_per_part});
+  }
+  else if (!mm) hipLaunchKernelGGL(k_sdpa_tile, dim3(tiles, SL_ATT_KV, M), dim3(256), 0, e->stream, s);
   SdpaMergeArgs g{};
   g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore; g.lanes = lanes;
+  g.group = tiles_per_part;
   if (mm && lanes) hipLaunchKernelGGL(k_sdpa_merge_par<16>, dim3(SL_ATT_HEADS, M), dim3(1024), 0, e->stream, g);
   else if (mm) hipLaunchKernelGGL(k_sdpa_merge_par<4>, dim3(SL_ATT_HEADS, M), dim3(256), 0, e->stream, g);
   else hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);

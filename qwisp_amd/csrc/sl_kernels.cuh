@@ -1214,6 +1214,7 @@ struct SdpaMergeArgs {
   int maxTiles;
   uint16_t* gated;             // [M, 4096]
   const LaneRef* lanes;
+  int group = 0;               // > 1: one partial per `group` key tiles at index tile / group (k_sdpa_merge_par only)
 };
 __global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
   const int h = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;

@@ -662,6 +662,164 @@ __global__ __launch_bounds__(256) void k_sdpa_tile_mfma(SdpaMmArgs a) {
 }
 
 // -------------------------------------------------------------------------------------------------
+// Attention of a prefill chunk with running softmax sums (hybrid mode): workgroup = (part of the key range, kv head,
+// block of 32 query rows), eight waves = the eight query heads of the group.  The workgroup walks its key tiles:
+// keys [key][dim] and values transposed [dim][key] staged in LDS once for the eight heads (the next tile's pieces on
+// their way in registers).  Both products are formed transposed, S^T = K Q^T and O^T = V^T P^T, so that a lane owns
+// one query row: its 32 of the tile's 64 scores sit in its own registers (the other 32 in the lane 32 further), the
+// row's running maximum and sum are one value per lane, and the accumulated output of the lane's row is rescaled by
+// the lane's own factor when the maximum moved -- no cross-lane reductions apart from one exchange between the
+// half-waves.  The softmax weights go from the score registers straight into the operand of the second product: the
+// k slots of a matrix step are any eight keys as long as both operands agree, so a step takes the eight keys a lane
+// already holds and the transposed value tile is stored with its keys in that order (key_slot below).  One partial
+// (max, sum, unnormalised output) per part and row goes to the arrays of the per-tile kernels at index `part`;
+// k_sdpa_merge_par finishes it with `group` = SDPA_FLASH_TILES.  Tolerance-level.
+// -------------------------------------------------------------------------------------------------
+constexpr int SDPA_FLASH_TILES = 8;   // key tiles per part (fixed: see the launch)
+struct SdpaFlashArgs {
+  SdpaArgs s;
+  int M;
+  int TP;                      // key tiles per part
+};
+// position of key (0..63) of a tile in a row of the transposed value tile: S^T register r of half-wave hh and 32-key
+// block c holds key 32c + 8(r/4) + 4hh + r%4; step st = 2c + (r/8) of the second product takes registers 8(st%2) .. +7
+SL_DEV int key_slot(int key) {
+  const int c = key >> 5, g = (key >> 3) & 3, h = (key >> 2) & 1, i = key & 3;
+  return 16 * (2 * c + (g >> 1)) + 8 * h + 4 * (g & 1) + i;
+}
+__global__ __launch_bounds__(512, 2) void k_sdpa_flash_mfma(SdpaFlashArgs a) {
+  __shared__ __align__(16) uint16_t s_k[SDPA_TILE * KT_STRIDE];
+  __shared__ __align__(16) uint16_t s_vt[256 * VT_STRIDE];
+  const int part = blockIdx.x, kvh = blockIdx.y, m0 = blockIdx.z * 32;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, hh = lane >> 5;
+  const int pos0 = a.s.st[0];
+  const int rows = min(32, a.M - m0);
+  const int nmax = pos0 + m0 + rows;                     // keys visible to the block's last row
+  const int nt = (nmax + SDPA_TILE - 1) / SDPA_TILE;
+  const int t_begin = part * a.TP, t_end = min(t_begin + a.TP, nt);
+  if (t_begin >= nt) return;                             // uniform for the workgroup
+  const uint16_t* kbase = a.s.kcache + (size_t)kvh * a.s.maxSeq * 256;
+  const uint16_t* vbase = a.s.vcache + (size_t)kvh * a.s.maxSeq * 256;
+  // a tile's pieces: keys 4 rows of 16 per thread (a row on 32 neighbouring lanes), values key tid & 63, eight dims
+  // each; keys beyond the visible range repeat the last visible one (masked below, their values meet a weight of zero)
+  uint4 pk[4], pv[4];
+  auto fetch = [&](int t) {
+    const int j0 = t * SDPA_TILE;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int row = min(j0 + it * 16 + (tid >> 5), nmax - 1), key = min(j0 + (tid & 63), nmax - 1);
+      pk[it] = ld16(kbase + (size_t)row * 256 + (tid & 31) * 8);
+      pv[it] = ld16(vbase + (size_t)key * 256 + ((tid >> 6) + 8 * it) * 8);
+    }
+  };
+  const float NEG = -__int_as_float(0x7f800000);
+  const float C = 0.0625f * 1.44269504f;                 // scale 1/16 and log2(e) in one factor: weights are 2^(C s - max)
+  const int head = kvh * 8 + wave;
+  const int qrow = m0 + col;                             // this lane's query row
+  const bool live = qrow < a.M;
+  const uint16_t* qp = a.s.qrot + ((size_t)min(qrow, a.M - 1) * 16 + head) * 256 + 8 * hh;
+  const int vslot = key_slot(tid & 63);
+  float mrun = NEG, lrun = 0.0f;                         // of the lane's row, in units of log2: running max of C s, sum of 2^(C s - max)
+  mf_f16v O[8];                                          // O^T: register r of block d is dim 32d + 8(r/4) + 4hh + r%4 of the lane's row
+#pragma unroll
+  for (int d = 0; d < 8; ++d)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) O[d][r] = 0.0f;
+  fetch(t_begin);
+  for (int t = t_begin; t < t_end; ++t) {
+    const int j0 = t * SDPA_TILE;
+    __syncthreads();                                     // the tile before is no longer read
+#pragma unroll
+    for (int it = 0; it < 4; ++it) st16(&s_k[(it * 16 + (tid >> 5)) * KT_STRIDE + (tid & 31) * 8], pk[it]);
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int c8 = ((tid >> 6) + 8 * it) * 8;
+      const uint32_t w[4] = {pv[it].x, pv[it].y, pv[it].z, pv[it].w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s_vt[(c8 + i) * VT_STRIDE + vslot] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
+    }
+    fetch(min(t + 1, t_end - 1));
+    __syncthreads();
+    // S^T = K Q^T: lane (col, hh) brings dims 16*st + 8*hh .. +7 of key 32*c + col / of its query row
+    mf_f16v S[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S[c][r] = 0.0f;
+#pragma unroll
+    for (int st = 0; st < 16; ++st) {
+      const mf_h8 bq = __builtin_bit_cast(mf_h8, ld16(qp + 16 * st));
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const mf_h8 ak = *reinterpret_cast<const mf_h8*>(&s_k[(32 * c + col) * KT_STRIDE + 16 * st + 8 * hh]);
+        S[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ak, bq, S[c], 0, 0, 0);
+      }
+    }
+    // register r of block c is key j0 + 32c + 8(r/4) + 4hh + r%4 against the lane's row; the row sees keys up to
+    // pos0 + qrow
+    const int lim = live ? pos0 + qrow - j0 - 4 * hh : -1;   // largest visible value of 32c + 8(r/4) + r%4
+    float mx = NEG;
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        S[c][r] = (32 * c + 8 * (r >> 2) + (r & 3) <= lim) ? C * S[c][r] : NEG;
+        mx = fmaxf(mx, S[c][r]);
+      }
+    {
+      const unsigned u = __float_as_uint(mx);
+      const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+      mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    }
+    const float mn = fmaxf(mrun, mx);
+    const float alpha = (mn == mrun) ? 1.0f : __builtin_amdgcn_exp2f(mrun - mn);   // (mrun = -inf, mn finite: 0)
+    float sum = 0.0f;
+    mf_h8 ap[4];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = (S[c][r] == NEG) ? 0.0f : __builtin_amdgcn_exp2f(S[c][r] - mn);
+        sum += p;
+        ap[2 * c + (r >> 3)][r & 7] = (_Float16)p;
+      }
+    {
+      const unsigned u = __float_as_uint(sum);
+      const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+      sum = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+    }
+    lrun = fmaf(lrun, alpha, sum);
+    mrun = mn;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {   // some row's maximum moved: what it has accumulated shrinks with it
+#pragma unroll
+      for (int d = 0; d < 8; ++d)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) O[d][r] *= alpha;
+    }
+    // O^T += V^T P^T: lane (col, hh) brings key slots 16*st + 8*hh .. +7 of dim 32*d + col / of its row of P
+#pragma unroll
+    for (int st = 0; st < 4; ++st)
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {
+        const mf_h8 av = *reinterpret_cast<const mf_h8*>(&s_vt[(32 * d + col) * VT_STRIDE + 16 * st + 8 * hh]);
+        O[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, ap[st], O[d], 0, 0, 0);
+      }
+  }
+  if (live) {
+    const size_t pi = ((size_t)qrow * 16 + head) * a.s.maxTiles + part;
+    // the merge works with natural logarithms: max back from log2 units
+    if (hh == 0) { a.s.pm[pi] = (mrun == NEG) ? NEG : mrun * 0.6931471805599453f; a.s.pl[pi] = lrun; }
+    float* po = a.s.po + pi * 256 + 4 * hh;
+#pragma unroll
+    for (int d = 0; d < 8; ++d)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<float4*>(po + 32 * d + 8 * g) = make_float4(O[d][4 * g], O[d][4 * g + 1], O[d][4 * g + 2], O[d][4 * g + 3]);
+  }
+}
+
+
+// -------------------------------------------------------------------------------------------------
 // Decode attention of a lane batch on the matrix cores (hybrid mode): every row is one new token of its own
 // sequence, so a key tile is shared only by the 8 query heads of a kv group.  Workgroup = (key tile of 64, kv head,
 // lane); the heads take rows 0..7 of a 32-row matrix operand (rows 8..31 carry nothing and their results are never
@@ -806,7 +964,8 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void k_sdpa_merge_par(SdpaMergeAr
   __shared__ __align__(16) float s_o[MERGE_WAVES][256];
   const int h = blockIdx.x, m = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int N = a.lanes ? a.lanes[m].st[0] + 1 : a.st[0] + m + 1;
-  const int nt = (N + SDPA_TILE - 1) / SDPA_TILE;
+  int nt = (N + SDPA_TILE - 1) / SDPA_TILE;
+  if (a.group > 1) nt = (nt + a.group - 1) / a.group;    // partials per part of `group` tiles (k_sdpa_flash_mfma)
   const size_t base = ((size_t)m * 16 + h) * a.maxTiles;
   const float NEG = -__int_as_float(0x7f800000);
   float mx = NEG;
