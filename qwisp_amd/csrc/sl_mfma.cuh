@@ -535,131 +535,7 @@ __global__ __launch_bounds__(256) void k_moe_combine_rows(const uint16_t* __rest
   out[(size_t)m * H + n] = f2h(f16r(acc + f16r(s * h2f(sy[(size_t)m * H + n]))));
 }
 
-// -------------------------------------------------------------------------------------------------
-// Attention of a prefill chunk on the matrix cores (hybrid mode): the tile pass of k_sdpa_tile for 32 query rows of
-// one sequence at a time.  Workgroup = (key tile of 64, kv head, block of 32 rows); the tile's keys [key][dim] and
-// values transposed [dim][key] are staged in LDS once for the 8 query heads of the group and the 32 rows; wave w
-// takes heads 2w, 2w+1 in turn:  S = Q K^T (32 x 64, 32 matrix instructions), causal mask, scale 1/16, row max and
-// exponentials in fp32, P rounded to half through a wave-private LDS patch into operand order, O = P V (32 x 256,
-// 32 matrix instructions).  It writes the same per-tile partials (max, sum, unnormalised output) as the exact tile
-// kernel, so k_sdpa_merge finishes both.  Tolerance-level (P and the products in half, hardware exp2).
-// -------------------------------------------------------------------------------------------------
-struct SdpaMmArgs {
-  SdpaArgs s;
-  int M;
-};
-constexpr int VT_STRIDE = 72;     // halves per row of the transposed value tile and of the P patch: 64 + 8 pad
-SL_DEV float half_wave_max(float v) {          // over the 32 lanes of a half-wave
-  v = fmaxf(v, dpp_f<DPP_XOR1>(v));
-  v = fmaxf(v, dpp_f<DPP_XOR2>(v));
-  v = fmaxf(v, dpp_f<DPP_HALF_MIRROR>(v));
-  v = fmaxf(v, dpp_f<DPP_MIRROR>(v));
-  const unsigned u = __float_as_uint(v);
-  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__global__ __launch_bounds__(256) void k_sdpa_tile_mfma(SdpaMmArgs a) {
-  __shared__ __align__(16) uint16_t s_k[SDPA_TILE * KT_STRIDE];
-  __shared__ __align__(16) uint16_t s_vt[256 * VT_STRIDE];
-  __shared__ __align__(16) uint16_t s_p[4][32 * VT_STRIDE];
-  const int tile = blockIdx.x, kvh = blockIdx.y, m0 = blockIdx.z * 32;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, hh = lane >> 5;
-  const int pos0 = a.s.st[0];
-  const int rows = min(32, a.M - m0);
-  const int nmax = pos0 + m0 + rows;                     // keys visible to the block's last row
-  const int j0 = tile * SDPA_TILE;
-  if (j0 >= nmax) return;                                // uniform for the workgroup
-  const uint16_t* kbase = a.s.kcache + ((size_t)kvh * a.s.maxSeq + j0) * 256;
-  const uint16_t* vbase = a.s.vcache + ((size_t)kvh * a.s.maxSeq + j0) * 256;
-  // keys: 64 rows x 32 pieces of 16 bytes, a row on 32 neighbouring lanes; rows at or beyond nmax are zero
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int row = it * 8 + (tid >> 5), c8 = (tid & 31) * 8;
-    uint4 kv = make_uint4(0, 0, 0, 0);
-    if (j0 + row < nmax) kv = ld16(kbase + (size_t)row * 256 + c8);
-    st16(&s_k[row * KT_STRIDE + c8], kv);
-  }
-  // values transposed: a lane takes key (tid & 63) and eight dims, so that the 64 lanes of a wave write 64 neighbouring
-  // halves of each of the eight rows of the transposed tile
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int key = tid & 63, c8 = ((tid >> 6) + 4 * it) * 8;
-    uint4 vv = make_uint4(0, 0, 0, 0);
-    if (j0 + key < nmax) vv = ld16(vbase + (size_t)key * 256 + c8);
-    const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
-#pragma unroll
-    for (int i = 0; i < 8; ++i) s_vt[(c8 + i) * VT_STRIDE + key] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
-  }
-  __syncthreads();
-  const float NEG = -__int_as_float(0x7f800000);
-  const int qrow = m0 + col;                             // this lane's row as the A operand
-  for (int hq = 0; hq < 2; ++hq) {
-    const int head = kvh * 8 + 2 * wave + hq;
-    // S = Q K^T: lane (col, hh) brings dims 16*st + 8*hh .. +7 of its query row / of key 32*c + col
-    mf_f16v S[2];
-#pragma unroll
-    for (int c = 0; c < 2; ++c)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) S[c][r] = 0.0f;
-    const uint16_t* qp = a.s.qrot + ((size_t)(qrow < a.M ? qrow : 0) * 16 + head) * 256 + 8 * hh;
-#pragma unroll
-    for (int st = 0; st < 16; ++st) {
-      uint4 qv = ld16(qp + 16 * st);
-      if (qrow >= a.M) qv = make_uint4(0, 0, 0, 0);
-      const mf_h8 aq = __builtin_bit_cast(mf_h8, qv);
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const mf_h8 bk = *reinterpret_cast<const mf_h8*>(&s_k[(32 * c + col) * KT_STRIDE + 16 * st + 8 * hh]);
-        S[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aq, bk, S[c], 0, 0, 0);
-      }
-    }
-    // register r of lane (col, hh) is row 8*(r/4) + 4*hh + r%4, key 32*c + col: mask, scale, softmax pieces per row
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = 8 * (r >> 2) + 4 * hh + (r & 3);
-      const int last = pos0 + m0 + row;                  // the last key this row may see
-      const bool live = m0 + row < a.M;
-      float sv[2];
-#pragma unroll
-      for (int c = 0; c < 2; ++c) sv[c] = (live && j0 + 32 * c + col <= last) ? 0.0625f * S[c][r] : NEG;
-      const float mx = half_wave_max(fmaxf(sv[0], sv[1]));
-      float p[2];
-#pragma unroll
-      for (int c = 0; c < 2; ++c) p[c] = (sv[c] == NEG) ? 0.0f : __builtin_amdgcn_exp2f((sv[c] - mx) * 1.44269504f);
-      const float l = tree_sum<32>(p[0] + p[1]);
-      if (col == 0 && live) {
-        const size_t pi = ((size_t)(m0 + row) * 16 + head) * a.s.maxTiles + tile;
-        a.s.pm[pi] = mx; a.s.pl[pi] = l;
-      }
-#pragma unroll
-      for (int c = 0; c < 2; ++c) s_p[wave][row * VT_STRIDE + 32 * c + col] = f2h(p[c]);
-    }
-    // O = P V: lane (col, hh) brings keys 16*st + 8*hh .. +7 of its row of P / of dim 32*d + col of V^T
-    mf_f16v O[8];
-#pragma unroll
-    for (int d = 0; d < 8; ++d)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) O[d][r] = 0.0f;
-#pragma unroll
-    for (int st = 0; st < 4; ++st) {
-      const mf_h8 ap = *reinterpret_cast<const mf_h8*>(&s_p[wave][col * VT_STRIDE + 16 * st + 8 * hh]);
-#pragma unroll
-      for (int d = 0; d < 8; ++d) {
-        const mf_h8 bv = *reinterpret_cast<const mf_h8*>(&s_vt[(32 * d + col) * VT_STRIDE + 16 * st + 8 * hh]);
-        O[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ap, bv, O[d], 0, 0, 0);
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = 8 * (r >> 2) + 4 * hh + (r & 3);
-      if (m0 + row < a.M) {
-        float* po = a.s.po + (((size_t)(m0 + row) * 16 + head) * a.s.maxTiles + tile) * 256 + col;
-#pragma unroll
-        for (int d = 0; d < 8; ++d) po[32 * d] = O[d][r];
-      }
-    }
-  }
-}
+constexpr int VT_STRIDE = 72;     // halves per row of a transposed value tile (and of the lane kernel's P patch): 64 + 8 pad
 
 // -------------------------------------------------------------------------------------------------
 // Attention of a prefill chunk with running softmax sums (hybrid mode): workgroup = (part of the key range, kv head,
