@@ -389,14 +389,18 @@ SL_DEV float swiglu_mm(float g, float u) {
   const float sg = f16r(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g)));
   return f16r(f16r(g * sg) * u);
 }
-constexpr int GQ_LDS_HALVES = 2 * 128 * (64 + 8);         // two staging buffers of 128 rows x 64 k (the largest shape)
+// two staging buffers of 128 rows x GW groups (the largest shape of a pass): gate|up walks K = 2048 with two groups
+// per barrier, the down projection (K = 512, four times the workgroups) with one, which leaves room for three workgroups
+// per compute unit
+template <bool DUAL> constexpr int GQ_WIDE = DUAL ? 2 : 1;
+template <bool DUAL> constexpr int GQ_LDS_HALVES = 2 * 128 * (64 * GQ_WIDE<DUAL> + 8);
 template <bool DUAL, int RT, int G>
 SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* list, int cnt, const uint32_t* const (&wp)[2],
                          const uint32_t* const (&sp)[2], bool live, int n0) {
   constexpr int NW = DUAL ? 2 : 1;
   constexpr int XS = 64 * G + 8;                         // halves per staged row
   constexpr int BUF = RT * 32 * XS;                      // halves per staging buffer
-  static_assert(2 * BUF <= GQ_LDS_HALVES, "staging buffers exceed the workgroup's LDS");
+  static_assert(2 * BUF <= GQ_LDS_HALVES<DUAL>, "staging buffers exceed the workgroup's LDS");
   const int tid = threadIdx.x, lane = tid & 63;
   const int col = lane & 31, hh = lane >> 5;
   const int chunks = a.K / (64 * G);
@@ -495,7 +499,8 @@ SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* l
 }
 template <bool DUAL>
 __global__ __launch_bounds__(256, 2) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
-  __shared__ __align__(16) uint16_t xs[GQ_LDS_HALVES];
+  __shared__ __align__(16) uint16_t xs[GQ_LDS_HALVES<DUAL>];
+  constexpr int GW = GQ_WIDE<DUAL>;
   const int e = a.order[blockIdx.y];
   const int cnt_all = min(a.counts[e], GROUP_CAP);
   if (cnt_all == 0) return;                              // uniform for the workgroup
@@ -508,10 +513,10 @@ __global__ __launch_bounds__(256, 2) void k_qmm4_mfma_grouped(QmmGroupArgs a) {
   const uint32_t* const sp[2] = {a.SB + wrow * (a.K / 64), DUAL ? a.SB2 + wrow * (a.K / 64) : nullptr};
   const uint16_t* lists = a.lists + (size_t)e * GROUP_CAP;
   int r0 = 0;
-  for (; cnt_all - r0 > 128; r0 += 128) grouped_pass<DUAL, 4, 1>(a, xs, lists + r0, 128, wp, sp, live, n0);
+  for (; cnt_all - r0 > 128; r0 += 128) grouped_pass<DUAL, 4, GW>(a, xs, lists + r0, 128, wp, sp, live, n0);
   const int rest = cnt_all - r0;                         // 1 .. 128; K % 256 == 0 for both shapes
-  if (rest > 96) grouped_pass<DUAL, 4, 1>(a, xs, lists + r0, rest, wp, sp, live, n0);
-  else if (rest > 64) grouped_pass<DUAL, 3, 1>(a, xs, lists + r0, rest, wp, sp, live, n0);
+  if (rest > 96) grouped_pass<DUAL, 4, GW>(a, xs, lists + r0, rest, wp, sp, live, n0);
+  else if (rest > 64) grouped_pass<DUAL, 3, GW>(a, xs, lists + r0, rest, wp, sp, live, n0);
   else if (rest > 32) grouped_pass<DUAL, 2, 2>(a, xs, lists + r0, rest, wp, sp, live, n0);
   else grouped_pass<DUAL, 1, 4>(a, xs, lists + r0, rest, wp, sp, live, n0);
 }
