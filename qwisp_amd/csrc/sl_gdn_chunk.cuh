@@ -192,39 +192,63 @@ __global__ __launch_bounds__(256) void k_gdn_chunk_prep(GdnChunkArgs a) {
 }
 
 // ---- the blocks of a value head in order: grid 32, 256 threads; wave w owns value dims 32 w .. 32 w + 31 ------------
+// Everything the wave carries from product to product stays in registers.  The state slice is kept transposed, as four
+// result tiles T[c] of S^T (rows = 32 key dims, columns = the wave's 32 value dims): a lane then holds, for its
+// value dim, sixteen key dims of each tile, and since the k slots of a matrix step may be any eight indices as long
+// as both operands agree, those registers -- rounded to half -- are the right-hand operand of the products that
+// contract over the key dim (U = UV - Wm S_0^T and Q_g S_0^T), the result tiles U (rows = block rows, columns = value
+// dims) are in turn the right-hand operand of the products that contract over the block row (P U and the state update
+// Kd^T U), and the state update delivers S^T tiles again.  The left-hand operands come from LDS, staged with the
+// contraction index of each 32-block in the matching order (kslot32).  Two sets of staging buffers: one barrier per
+// block; the block after the next is on its way from memory meanwhile.
+// position of contraction index k in a staged row: matrix step st (0, 1) of 32-block c takes, on half-wave hh, the
+// eight indices that registers 8 st .. 8 st + 7 of a result tile hold there: 32 c + 8 (2 st + j / 4) + 4 hh + j % 4
+SL_DEV int kslot32(int k) {
+  const int g = (k >> 3) & 3, h = (k >> 2) & 1, i = k & 3;
+  return (k & ~31) + 16 * (g >> 1) + 8 * h + 4 * (g & 1) + i;
+}
+// a 16-byte piece (eight consecutive indices from k0, a multiple of 8) into its two places of a staged row
+SL_DEV void stage_piece(uint16_t* row, int k0, uint4 v) {
+  uint16_t* p = row + kslot32(k0);
+  *reinterpret_cast<uint2*>(p) = make_uint2(v.x, v.y);
+  *reinterpret_cast<uint2*>(p + 8) = make_uint2(v.z, v.w);
+}
+// registers 8 st .. 8 st + 7 of a result tile as a matrix operand
+SL_DEV mf_h8 tile_operand(const mf_f16v& t, int st) {
+  mf_h8 o;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) o[j] = (_Float16)t[8 * st + j];
+  return o;
+}
+constexpr int GC_SCAN_BUF = 2 * GC * GC_KS + 128 * GC_CS + GC * GC_CS;   // halves per set: Wm, Qg, KdT, P
+constexpr int GC_SCAN_LDS = 2 * GC_SCAN_BUF * 2;
 __global__ __launch_bounds__(256) void k_gdn_chunk_scan(GdnChunkArgs a) {
   extern __shared__ __align__(16) uint16_t gcs[];
-  uint16_t* Wm = gcs;                          // [64][GC_KS]
-  uint16_t* Qg = Wm + GC * GC_KS;              // [64][GC_KS]
-  uint16_t* KdT = Qg + GC * GC_KS;             // [128][GC_CS]
-  uint16_t* P = KdT + 128 * GC_CS;             // [64][GC_CS]
-  uint16_t* S16 = P + GC * GC_CS;              // [128 dv][GC_KS]
-  uint16_t* UT = S16 + 128 * GC_KS;            // [128 dv][GC_CS]
   const int hv = blockIdx.x, hk = hv >> 1;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, hh = lane >> 5;
   const bool par = a.st[1] != 0;
   const float* sin_ = par ? a.state[1] : a.state[0];
   float* sout = par ? a.state[0] : a.state[1];
   const int dv0 = wave * 32;
-  // the state slice as four result tiles: S[dv0 + row][32 j + col]
-  mf_f16v S[4];
+  // T[c][r] = S[dv0 + col][32 c + acc_row(r)]
+  mf_f16v T[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int c = 0; c < 4; ++c)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) S[j][r] = sin_[((size_t)hv * 128 + dv0 + acc_row(r, lane)) * 128 + 32 * j + col];
+    for (int g = 0; g < 4; ++g) {
+      const float4 v = *reinterpret_cast<const float4*>(sin_ + ((size_t)hv * 128 + dv0 + col) * 128 + 32 * c + 8 * g + 4 * hh);
+      T[c][4 * g] = v.x; T[c][4 * g + 1] = v.y; T[c][4 * g + 2] = v.z; T[c][4 * g + 3] = v.w;
+    }
   const int nblk = a.M / GC;
-  // A block's matrices travel global -> registers -> LDS one block ahead: the loads of block b + 1 are in flight
-  // while block b is multiplied (a block's arithmetic is shorter than a trip to memory).
   uint4 pw[4], pq[4], pk[4], pp[2];
-  float uvr[2][16];
-  float gcd_next = 0.0f;
-  auto prefetch = [&](int blk) {
-    const unsigned char* unit = a.scratch + ((size_t)blk * 32 + hv) * GC_UNIT_BYTES;
+  float uvn[2][16];                            // UV of the block after the current one (start value of its U)
+  float gcn = 0.0f;
+  auto fetch = [&](int blk) {
+    const unsigned char* unit = a.scratch + ((size_t)min(blk, nblk - 1) * 32 + hv) * GC_UNIT_BYTES;
     const uint16_t* gWm = reinterpret_cast<const uint16_t*>(unit + GC_OFF_WM);
     const uint16_t* gQg = reinterpret_cast<const uint16_t*>(unit + GC_OFF_QG);
     const uint16_t* gKd = reinterpret_cast<const uint16_t*>(unit + GC_OFF_KDT);
     const uint16_t* gP = reinterpret_cast<const uint16_t*>(unit + GC_OFF_P);
-    const float* UV = reinterpret_cast<const float*>(unit + GC_OFF_UV);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int i = tid + 256 * j;
@@ -237,69 +261,131 @@ __global__ __launch_bounds__(256) void k_gdn_chunk_scan(GdnChunkArgs a) {
       const int i = tid + 256 * j;
       pp[j] = ld16(gP + (i >> 3) * 64 + 8 * (i & 7));
     }
+  };
+  auto fetch_uv = [&](int blk) {
+    const unsigned char* unit = a.scratch + ((size_t)min(blk, nblk - 1) * 32 + hv) * GC_UNIT_BYTES;
+    const float* UV = reinterpret_cast<const float*>(unit + GC_OFF_UV);
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) uvr[rt][r] = UV[(rt * 32 + acc_row(r, lane)) * 128 + dv0 + col];
-    gcd_next = *reinterpret_cast<const float*>(unit + GC_OFF_GC);
+      for (int r = 0; r < 16; ++r) uvn[rt][r] = UV[(rt * 32 + acc_row(r, lane)) * 128 + dv0 + col];
+    gcn = *reinterpret_cast<const float*>(unit + GC_OFF_GC);
   };
-  if (nblk > 0) prefetch(0);
-  for (int blk = 0; blk < nblk; ++blk) {
-    __syncthreads();                           // the block before is done with the staged matrices
+  auto stage = [&](int set) {                  // the fetched block into staging set `set`; its UV and G_C become current
+    uint16_t* Wm = gcs + set * GC_SCAN_BUF;
+    uint16_t* Qg = Wm + GC * GC_KS;
+    uint16_t* KdT = Qg + GC * GC_KS;
+    uint16_t* P = KdT + 128 * GC_CS;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int i = tid + 256 * j;
-      st16(&Wm[(i >> 4) * GC_KS + 8 * (i & 15)], pw[j]);
-      st16(&Qg[(i >> 4) * GC_KS + 8 * (i & 15)], pq[j]);
-      st16(&KdT[(i >> 3) * GC_CS + 8 * (i & 7)], pk[j]);
+      stage_piece(Wm + (i >> 4) * GC_KS, 8 * (i & 15), pw[j]);
+      stage_piece(Qg + (i >> 4) * GC_KS, 8 * (i & 15), pq[j]);
+      stage_piece(KdT + (i >> 3) * GC_CS, 8 * (i & 7), pk[j]);
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int i = tid + 256 * j;
-      st16(&P[(i >> 3) * GC_CS + 8 * (i & 7)], pp[j]);
+      stage_piece(P + (i >> 3) * GC_CS, 8 * (i & 7), pp[j]);
     }
-    // the state in half as the right-hand operand of the products with S_0^T
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) S16[(dv0 + acc_row(r, lane)) * GC_KS + 32 * j + col] = f2h(S[j][r]);
-    const float GCd = gcd_next;
+  };
+  if (nblk > 0) { fetch(0); stage(0); fetch_uv(0); }
+  if (nblk > 1) fetch(1);
+  for (int blk = 0; blk < nblk; ++blk) {
+    const int set = blk & 1;
+    lds_barrier();                             // set `set` is staged; the other set is no longer read (loads stay in flight)
+    const uint16_t* Wm = gcs + set * GC_SCAN_BUF;
+    const uint16_t* Qg = Wm + GC * GC_KS;
+    const uint16_t* KdT = Qg + GC * GC_KS;
+    const uint16_t* P = KdT + 128 * GC_CS;
+    // this block's accumulator start and decay; then the next block goes to the other set and the one after it is requested
     mf_f16v U[2];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) U[rt][r] = uvr[rt][r];
-    __syncthreads();
-    if (blk + 1 < nblk) prefetch(blk + 1);
-    // U = UV - Wm S_0^T for this wave's value dims (rows t, columns dv0 + col), kept transposed in half for what follows
+      for (int r = 0; r < 16; ++r) U[rt][r] = uvn[rt][r];
+    const float GCd = gcn;
+    if (blk + 1 < nblk) {
+      stage(set ^ 1);
+      fetch(blk + 2);
+      fetch_uv(blk + 1);
+    }
+    // the state in half as the right-hand operand of the products that contract over the key dim
+    mf_h8 Th[4][2];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int st = 0; st < 2; ++st) Th[c][st] = tile_operand(T[c], st);
+    // U = UV - Wm S_0^T and Y = Qg S_0^T for this wave's value dims (rows = block rows, columns = value dims).  The
+    // left-hand operands of a group of products are read from LDS together, ahead of the matrix instructions (the
+    // fences keep it that way: a read waited for in front of every matrix instruction costs its full latency each time).
     mf_f16v Y[2];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
-      mma_tile(U[rt], Wm + rt * 32 * GC_KS, GC_KS, S16 + dv0 * GC_KS, GC_KS, 128, lane);
+      mf_h8 aw[8], aq[8];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) UT[(dv0 + col) * GC_CS + rt * 32 + acc_row(r, lane)] = f2h(U[rt][r]);
+      for (int i = 0; i < 8; ++i) {
+        const int off = (rt * 32 + col) * GC_KS + 16 * i + 8 * hh;
+        aw[i] = *reinterpret_cast<const mf_h8*>(Wm + off);
+        aq[i] = *reinterpret_cast<const mf_h8*>(Qg + off);
+      }
       acc_zero(Y[rt]);
-      mma_tile(Y[rt], Qg + rt * 32 * GC_KS, GC_KS, S16 + dv0 * GC_KS, GC_KS, 128, lane);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        U[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aw[i], Th[i >> 1][i & 1], U[rt], 0, 0, 0);
+        Y[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aq[i], Th[i >> 1][i & 1], Y[rt], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    mf_h8 Uh[2][2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int st = 0; st < 2; ++st) Uh[sb][st] = tile_operand(U[sb], st);
+    // S^T = G_C S^T + Kd^T U first (the next block waits for it), then Y += P U
+    {
+      mf_h8 ak[16];
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ak[4 * c + i] = *reinterpret_cast<const mf_h8*>(KdT + (32 * c + col) * GC_CS + 16 * i + 8 * hh);
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) T[c][r] *= GCd;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) T[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ak[4 * c + i], Uh[i >> 1][i & 1], T[c], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    {
+      mf_h8 ap[8];
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ap[4 * rt + i] = *reinterpret_cast<const mf_h8*>(P + (rt * 32 + col) * GC_CS + 16 * i + 8 * hh);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) Y[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ap[4 * rt + i], Uh[i >> 1][i & 1], Y[rt], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-      mma_tile(Y[rt], P + rt * 32 * GC_CS, GC_CS, UT + dv0 * GC_CS, GC_CS, 64, lane);
+    for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         a.ycore[(size_t)(blk * GC + rt * 32 + acc_row(r, lane)) * 4096 + hv * 128 + dv0 + col] = f2h(Y[rt][r]);
-    }
-    // S = G_C S + U^T Kd
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) S[j][r] *= GCd;
-      mma_tile(S[j], UT + dv0 * GC_CS, GC_CS, KdT + 32 * j * GC_CS, GC_CS, 64, lane);
-    }
   }
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int c = 0; c < 4; ++c)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) sout[((size_t)hv * 128 + dv0 + acc_row(r, lane)) * 128 + 32 * j + col] = S[j][r];
+    for (int g = 0; g < 4; ++g)
+      *reinterpret_cast<float4*>(sout + ((size_t)hv * 128 + dv0 + col) * 128 + 32 * c + 8 * g + 4 * hh) =
+          make_float4(T[c][4 * g], T[c][4 * g + 1], T[c][4 * g + 2], T[c][4 * g + 3]);
   // conv-history shift: rows M .. M+2 of [hist | qkv]; q and k channels by the even heads, value channels by every head
   const uint16_t* hin = par ? a.hist[1] : a.hist[0];
   uint16_t* hout = par ? a.hist[0] : a.hist[1];
@@ -314,6 +400,5 @@ __global__ __launch_bounds__(256) void k_gdn_chunk_scan(GdnChunkArgs a) {
     for (int j = 0; j < 3; ++j) hout[j * SL_CONV_DIM + v_ch] = f2h(conv_tap(a.proj, hin, a.M + j, v_ch));
   }
 }
-constexpr int GC_SCAN_LDS = (2 * GC * GC_KS + 128 * GC_CS + GC * GC_CS + 128 * GC_KS + 128 * GC_CS) * 2;
 
 }  // namespace sl
