@@ -62,34 +62,40 @@ SL_DEV int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r
 
 // ---- state-independent part: grid (blocks, 32 value heads), 256 threads ---------------------------------
 __global__ __launch_bounds__(256) void k_gdn_chunk_prep(GdnChunkArgs a) {
-  __shared__ __align__(16) uint16_t Ks[GC * GC_KS], Qs[GC * GC_KS];      // [t][d]
-  __shared__ __align__(16) uint16_t KT[128 * GC_CS], VT[128 * GC_CS];    // [d][t]
-  __shared__ __align__(16) uint16_t T1[GC * GC_CS], T2[GC * GC_CS];      // T diag(beta G) negated, T diag(beta): [t][i]
-  __shared__ __align__(16) float Am[GC * GC_AS];                          // A, strictly lower triangle used
-  __shared__ float Tl[GC * GC];                                           // T, rows as they are solved
+  // 73 KB of LDS, so that two workgroups share a compute unit and one's triangular solve (a chain on a single wave)
+  // runs beside the other's matrix products.  Three areas are used twice: K and Q rows are dead once K K^T, Q K^T, Qg
+  // and KdT are formed, and make room for T and its two scaled half copies; the value tile is staged only after the
+  // solve, into the space of A.
+  __shared__ __align__(16) uint16_t area_k[GC * GC_KS], area_q[2 * GC * GC_CS];
+  __shared__ __align__(16) uint16_t KT[128 * GC_CS];                     // [d][t]
+  __shared__ __align__(16) float area_a[128 * GC_CS / 2];                // A [64][GC_AS] floats, later V^T [128][GC_CS] halves
   __shared__ float Lg[GC], Bt[GC], Eg[GC], Ec[GC];                        // log-decays, betas, G_t, G_C / G_t
+  static_assert(GC * GC_AS <= 128 * GC_CS / 2 && GC * GC * 4 <= GC * GC_KS * 2 && GC * GC_KS <= 2 * GC * GC_CS, "aliased areas");
+  uint16_t* Ks = area_k;                                                  // [t][d]
+  uint16_t* Qs = area_q;
+  float* Tl = reinterpret_cast<float*>(area_k);                           // T, rows as they are solved (after Ks is dead)
+  uint16_t* T1 = area_q;                                                  // T diag(beta G) negated, T diag(beta): [t][i] (after Qs is dead)
+  uint16_t* T2 = area_q + GC * GC_CS;
+  float* Am = area_a;                                                     // A, strictly lower triangle used
+  uint16_t* VT = reinterpret_cast<uint16_t*>(area_a);                     // [d][t], staged after the solve
   const int blk = blockIdx.x, hv = blockIdx.y, hk = hv >> 1;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int row0 = blk * GC;
   unsigned char* unit = a.scratch + ((size_t)blk * 32 + hv) * GC_UNIT_BYTES;
-  // stage K, Q (rows) and K, V transposed
+  // stage K, Q (rows) and K transposed
   for (int i = tid; i < GC * 16; i += 256) {
     const int t = i >> 4, p = i & 15;                       // 16 pieces of 8 halves per row
     const uint4 kq = ld16(a.kn + (size_t)(row0 + t) * 2048 + hk * 128 + 8 * p);
     const uint4 qq = ld16(a.qn + (size_t)(row0 + t) * 2048 + hk * 128 + 8 * p);
-    const uint4 vq = ld16(a.vc + (size_t)(row0 + t) * 4096 + hv * 128 + 8 * p);
     st16(&Ks[t * GC_KS + 8 * p], kq);
     st16(&Qs[t * GC_KS + 8 * p], qq);
-    const uint32_t kw[4] = {kq.x, kq.y, kq.z, kq.w}, vw[4] = {vq.x, vq.y, vq.z, vq.w};
+    const uint32_t kw[4] = {kq.x, kq.y, kq.z, kq.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       KT[(8 * p + 2 * j) * GC_CS + t] = (uint16_t)(kw[j] & 0xffffu);
       KT[(8 * p + 2 * j + 1) * GC_CS + t] = (uint16_t)(kw[j] >> 16);
-      VT[(8 * p + 2 * j) * GC_CS + t] = (uint16_t)(vw[j] & 0xffffu);
-      VT[(8 * p + 2 * j + 1) * GC_CS + t] = (uint16_t)(vw[j] >> 16);
     }
   }
-  for (int i = tid; i < GC * GC; i += 256) Tl[i] = 0.0f;      // rows not solved yet are read (times a zero of A): keep them finite
   if (tid < GC) {
     const float g = a.gb[(size_t)(row0 + tid) * 64 + hv];
     Lg[tid] = fmaxf(log_c(fmaxf(g, 1e-37f)), -80.0f);      // a decay of zero: as good as e^-80
@@ -117,6 +123,28 @@ __global__ __launch_bounds__(256) void k_gdn_chunk_prep(GdnChunkArgs a) {
       Am[t * GC_AS + i] = (i < t) ? Bt[t] * dec * kk[r] : 0.0f;
       P[t * 64 + i] = f2h(dec * qk[r]);
     }
+  }
+  __syncthreads();                                            // G_t and G_C / G_t are written, the products have read K and Q
+  // Qg = diag(G) Q and KdT = (diag(G_C / G) K)^T (all waves; the last readers of the Q rows)
+  {
+    uint16_t* Qg = reinterpret_cast<uint16_t*>(unit + GC_OFF_QG);
+    uint16_t* KdT = reinterpret_cast<uint16_t*>(unit + GC_OFF_KDT);
+    for (int i = tid; i < GC * 128; i += 256) {
+      const int t = i >> 7, d = i & 127;
+      Qg[t * 128 + d] = f2h(Eg[t] * h2f(Qs[t * GC_KS + d]));
+      const int d2 = i >> 6, t2 = i & 63;
+      KdT[d2 * 64 + t2] = f2h(Ec[t2] * h2f(KT[d2 * GC_CS + t2]));
+    }
+    if (tid == 64) *reinterpret_cast<float*>(unit + GC_OFF_GC) = Eg[GC - 1];
+  }
+  __syncthreads();                                            // K and Q rows are dead, A is complete
+  for (int i = tid; i < GC * GC; i += 256) Tl[i] = 0.0f;      // rows not solved yet are read (times a zero of A): keep them finite
+  // the value rows of the block, requested now and staged once A is no longer needed
+  uint4 vq[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = tid + 256 * j, t = i >> 4, p = i & 15;
+    vq[j] = ld16(a.vc + (size_t)(row0 + t) * 4096 + hv * 128 + 8 * p);
   }
   __syncthreads();
   // T = (I + A)^-1 by forward substitution, lane j = column j (wave 0); rows in registers
@@ -157,17 +185,17 @@ __global__ __launch_bounds__(256) void k_gdn_chunk_prep(GdnChunkArgs a) {
       T1[t * GC_CS + lane] = f2h(-(tv * bj * gj));
       T2[t * GC_CS + lane] = f2h(tv * bj);
     }
-  } else {
-    // meanwhile: Qg = diag(G) Q and KdT = (diag(G_C / G) K)^T
-    uint16_t* Qg = reinterpret_cast<uint16_t*>(unit + GC_OFF_QG);
-    uint16_t* KdT = reinterpret_cast<uint16_t*>(unit + GC_OFF_KDT);
-    for (int i = tid - 64; i < GC * 128; i += 192) {
-      const int t = i >> 7, d = i & 127;
-      Qg[t * 128 + d] = f2h(Eg[t] * h2f(Qs[t * GC_KS + d]));
-      const int d2 = i >> 6, t2 = i & 63;
-      KdT[d2 * 64 + t2] = f2h(Ec[t2] * h2f(KT[d2 * GC_CS + t2]));
+  }
+  __syncthreads();                                            // A is dead: the value tile takes its place
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = tid + 256 * j, t = i >> 4, p = i & 15;
+    const uint32_t vw[4] = {vq[j].x, vq[j].y, vq[j].z, vq[j].w};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      VT[(8 * p + 2 * q) * GC_CS + t] = (uint16_t)(vw[q] & 0xffffu);
+      VT[(8 * p + 2 * q + 1) * GC_CS + t] = (uint16_t)(vw[q] >> 16);
     }
-    if (tid == 64) *reinterpret_cast<float*>(unit + GC_OFF_GC) = Eg[GC - 1];
   }
   __syncthreads();
   // -Wm = T1 K and UV = T2 V: 2 x 4 tiles each; wave w takes column tile w of both row tiles
