@@ -157,8 +157,7 @@ SL_DEV bool flow_poll(bool polls, Attempt attempt, unsigned* abort_word) {
         if ((threadIdx.x & 63) == 0) { st_co32(abort_word, 1u); g_L.pf[3] = 1; }
         break;
       }
-      __builtin_amdgcn_s_sleep(1);
-    }
+    }                                                   // (no back-off between attempts: a sleep of 64 clocks measured 0.3 % slower)
   }
   lds_barrier();
   return g_L.pf[3] == 0;
