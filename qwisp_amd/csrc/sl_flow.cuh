@@ -1106,7 +1106,11 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
     float acc = 0.0f;
     if (!gate8) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) { acc = fmaf(lo_h(xp[i]), lo_h(dww[i]), acc); acc = fmaf(hi_h(xp[i]), hi_h(dww[i]), acc); }
+      for (int i = 0; i < 16; ++i) {               // (half operands straight into the mixed-precision multiply-add)
+        const h2_t xv = as_h2(xp[i]), wv = as_h2(dww[i]);
+        acc = fmaf((float)xv.x, (float)wv.x, acc);
+        acc = fmaf((float)xv.y, (float)wv.y, acc);
+      }
     } else {
       float xf[32];
 #pragma unroll
