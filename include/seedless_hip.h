@@ -177,7 +177,9 @@ int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine*
 int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t* out);
 /* forwardRows (SFV:3641): hidden rows in, hidden rows (final_norm=0) or final-normed rows out. */
 int sl_forward_rows(sl_engine* e, const uint16_t* x_f16, int m, int final_norm, uint16_t* out_f16);
-/* Tell.SpecBackend.forward (TellRuntime.swift:84): embed + forwardRows with final norm. */
+/* Tell.SpecBackend.forward (TellRuntime.swift:84): embed + forwardRows with final norm.  out_f16 may be NULL: the rows
+ * then stay on the device, as the reference's forward leaves them in a device array (a prefill only looks at the last
+ * row of its last chunk, TellRuntime.swift:724); sl_hidden_rows and sl_head_argmax_rows read them afterwards. */
 int sl_forward_tokens(sl_engine* e, const int32_t* tokens, int m, uint16_t* out_f16);
 /* hiddenRows (SFV:4392): the normed rows the last step left behind (volatile). */
 int sl_hidden_rows(sl_engine* e, int m, uint16_t* out_f16);
@@ -186,6 +188,10 @@ int sl_logits_row(sl_engine* e, int m, uint16_t* out_f16 /* [vocab] */);
 /* engine.logits (SeedlessEngine.swift:180): lm_head + argmax over already-normed rows; used for
  * the first token after prefill (TellRuntime.swift:724-727). */
 int sl_head_argmax(sl_engine* e, const uint16_t* normed_f16, int m, int32_t* out);
+/* The same over rows first .. first + m - 1 of the final-normed rows that the last sl_forward_tokens / sl_forward_rows
+ * left on the device (engine.logits on a slice of forward's result, TellRuntime.swift:724-727): the first token after
+ * a prefill without the rows' trip to the host and back.  SL_ERR_ARG when those rows are gone (a step ran since). */
+int sl_head_argmax_rows(sl_engine* e, int first, int m, int32_t* out);
 
 /* No counterpart in the reference.  sl_head_argmax for callers that cannot allocate device memory or synchronise:
  * code under HIP graph capture, tight serving loops, harnesses that forbid allocation.  `normed_dev` [m, 2048] fp16

@@ -106,6 +106,7 @@ struct sl_engine {
   int lane_refs = 0;
   bool destroy_pending = false;
   int n_layers = 0, n_experts = 0, vocab = 0, max_m = 0, max_seq = 0, max_tiles = 0;
+  int normed_rows = 0;             // final-normed rows of the last forward still held in `normed` (0 after a step)
   bool has_attn = false, has_head = false;
   int device = 0;                  // the device that was current when the engine was created
   void* na_scratch = nullptr;      // this device's copy of the no-allocation scratch array
@@ -875,6 +876,7 @@ int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t
     if (!lanes[i]) return SL_ERR_ARG;
     for (int j = 0; j < i; ++j) if (lanes[j] == lanes[i]) return SL_ERR_ARG;
   }
+  for (int i = 0; i < b; ++i) lanes[i]->normed_rows = 0;
   if (!lanes_batchable(lanes, b)) {
     for (int i = 0; i < b; ++i) { const int r = sl_step_argmax(lanes[i], tokens + i, 1, out + i); if (r) return r; }
     return SL_OK;
@@ -1028,8 +1030,9 @@ static void time_end(sl_engine* e) {
 
 int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
   int r = guard(e); if (r) return r;
+  e->normed_rows = 0;
   e->logits_view = e->normed_view = nullptr;
-  if (!tokens || !out || !e->has_head) return SL_ERR_ARG;
+  if (!tokens || !e->has_head) return SL_ERR_ARG;
   r = check_rows(e, m); if (r) return r;
   for (int i = 0; i < m; ++i) if (tokens[i] < 0 || tokens[i] >= e->vocab) return SL_ERR_ARG;
   r = to_device(e, e->tok_in, tokens, (size_t)m * 4); if (r) return r;
@@ -1055,6 +1058,7 @@ int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
 
 int sl_chained_step_argmax(sl_engine* e, int32_t first, int k, int32_t* out) {
   int r = guard(e); if (r) return r;
+  e->normed_rows = 0;
   e->logits_view = e->normed_view = nullptr;
   if (!out || !e->has_head || k < 1 || k > MAX_CHAIN || first < 0 || first >= e->vocab) return SL_ERR_ARG;
   if (e->has_attn && e->pos + k > e->max_seq) return SL_ERR_ARG;
@@ -1087,7 +1091,11 @@ static int forward_common(sl_engine* e, int m, int final_norm, uint16_t* out, co
   hipLaunchKernelGGL(k_final_rows, dim3(m), dim3(64), 0, e->stream, ha);
   advance(e, m);
   SL_TRY(e, hipEventRecord(e->ev1, e->stream));
-  int r = read_back(e, out, final_norm ? e->normed : e->rows_out, (size_t)m * H * 2, what); if (r) return r;
+  // out == nullptr: the rows stay on the device (the reference's forward returns a device array, and a prefill only
+  // ever looks at the last row of the last chunk); sl_hidden_rows / sl_head_argmax_rows read them later
+  int r = out ? read_back(e, out, final_norm ? e->normed : e->rows_out, (size_t)m * H * 2, what) : finish(e, what);
+  if (r) return r;
+  e->normed_rows = final_norm ? m : 0;
   time_end(e);
   return SL_OK;
 }
@@ -1100,7 +1108,7 @@ int sl_forward_rows(sl_engine* e, const uint16_t* x, int m, int final_norm, uint
 }
 int sl_forward_tokens(sl_engine* e, const int32_t* tokens, int m, uint16_t* out) {
   int r = guard(e); if (r) return r;
-  if (!tokens || !out || !e->has_head) return SL_ERR_ARG;
+  if (!tokens || !e->has_head) return SL_ERR_ARG;
   r = check_rows(e, m); if (r) return r;
   for (int i = 0; i < m; ++i) if (tokens[i] < 0 || tokens[i] >= e->vocab) return SL_ERR_ARG;
   r = to_device(e, e->tok_in, tokens, (size_t)m * 4); if (r) return r;
@@ -1132,6 +1140,17 @@ int sl_head_argmax(sl_engine* e, const uint16_t* normed, int m, int32_t* out) {
   HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
   launch_head(e, m, ha, 0, false);
   return read_back(e, out, e->tok_out, (size_t)m * 4, "headArgmax");
+}
+
+// lm_head + arg-max of rows first .. first + m - 1 of the normed rows that the last sl_forward_tokens / sl_forward_rows
+// (with final norm) left on the device: the first token after a prefill without the rows' trip to the host and back.
+int sl_head_argmax_rows(sl_engine* e, int first, int m, int32_t* out) {
+  int r = guard(e); if (r) return r;
+  if (!out || !e->has_head || m < 1 || first < 0 || first + m > e->normed_rows) return SL_ERR_ARG;
+  e->logits_view = e->normed_view = nullptr;
+  HiddenArgs ha{e->normed + (size_t)first * H, nullptr, nullptr, nullptr, nullptr};
+  launch_head(e, m, ha, 0, false);
+  return read_back(e, out, e->tok_out, (size_t)m * 4, "headArgmaxRows");
 }
 
 // lm_head + arg-max for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that
@@ -1414,15 +1433,14 @@ int sl_greedy_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_
   if (!prompt || n_prompt < 1 || n_new < 0 || (n_new > 0 && !out) || !e->has_head) return SL_ERR_ARG;
   if (chain_k < 1) chain_k = 1;
   if (chain_k > MAX_CHAIN) chain_k = MAX_CHAIN;
-  std::vector<uint16_t> nr((size_t)e->max_m * H);
   int done = 0, last_m = 0;
-  while (done < n_prompt) {
+  while (done < n_prompt) {                    // the rows of a chunk stay on the device: only the last row of the last chunk is used
     last_m = n_prompt - done < e->max_m ? n_prompt - done : e->max_m;
-    r = sl_forward_tokens(e, prompt + done, last_m, nr.data()); if (r) return r;
+    r = sl_forward_tokens(e, prompt + done, last_m, nullptr); if (r) return r;
     done += last_m;
   }
   if (n_new == 0) return SL_OK;
-  r = sl_head_argmax(e, nr.data() + (size_t)(last_m - 1) * H, 1, &out[0]); if (r) return r;
+  r = sl_head_argmax_rows(e, last_m - 1, 1, &out[0]); if (r) return r;
   int have = 1;
   while (have < n_new) {
     const int k = n_new - have < chain_k ? n_new - have : chain_k;

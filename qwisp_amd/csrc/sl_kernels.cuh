@@ -521,7 +521,7 @@ __global__ __launch_bounds__(64) void k_gdn_prep_rows(GdnPrepArgs p) {
     const float sc = isk ? f16r(0.08838834764831845f) : f16r(0.0078125f);
 #pragma unroll
     for (int j = 0; j < GDN_PREP_ROWS; ++j) {
-      if (j >= rows) break;
+      if (j >= rows) continue;                  // (uniform; a break would keep the loop from unrolling)
       const int t = t0 + j;
       float a0 = 0.0f, a1 = 0.0f;
 #pragma unroll

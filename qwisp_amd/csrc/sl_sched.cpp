@@ -176,7 +176,6 @@ struct sl_lane_slots {
   std::vector<sl_engine*> lanes;
   std::vector<int> pos;             // resumable prefill: prompt tokens consumed per slot
   std::vector<int> reserved;        // tokens of KV budget a slot holds (0 = free)
-  std::vector<uint16_t> normed;
   std::vector<sl_engine*> group;
   std::vector<int32_t> toks, outs;
   int chunk = 1, max_seq = 0;
@@ -201,12 +200,12 @@ int lane_admit_step(void* ctx, const int32_t* prompt, int n_prompt, int slot, in
   int last_m = 0;
   while (L->pos[slot] < n_prompt && grant > 0) {
     const int m = n_prompt - L->pos[slot] < L->chunk ? n_prompt - L->pos[slot] : L->chunk;
-    if (sl_forward_tokens(e, prompt + L->pos[slot], m, L->normed.data()) != SL_OK) return -1;
+    if (sl_forward_tokens(e, prompt + L->pos[slot], m, nullptr) != SL_OK) return -1;   // the rows stay on the device
     L->pos[slot] += m; *consumed += m; grant -= L->chunk; last_m = m;
   }
   if (L->pos[slot] < n_prompt) return 1;
   if (last_m == 0) return -1;                       // called again after completion
-  return sl_head_argmax(e, L->normed.data() + (size_t)(last_m - 1) * SL_H, 1, first) == SL_OK ? 0 : -1;
+  return sl_head_argmax_rows(e, last_m - 1, 1, first) == SL_OK ? 0 : -1;
 }
 int lane_step(void* ctx, const int32_t* last, int32_t* next) {
   sl_lane_slots* L = (sl_lane_slots*)ctx;
@@ -253,7 +252,6 @@ int sl_lane_slots_create(const sl_engine* base, int n_slots, int chunk_rows, int
   L->pos.assign(n_slots, 0); L->reserved.assign(n_slots, 0);
   L->chunk = chunk_rows; L->max_seq = max_seq_len;
   L->kv_budget_tokens = kv_budget_tokens > 0 ? kv_budget_tokens : (long)n_slots * max_seq_len;
-  L->normed.resize((size_t)rows * SL_H);
   table->ctx = L; table->slot_count = n_slots;
   table->admit_step = lane_admit_step; table->step = lane_step; table->release = lane_release; table->can_admit = lane_can_admit;
   return SL_OK;

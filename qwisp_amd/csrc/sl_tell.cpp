@@ -184,7 +184,6 @@ namespace {
 struct EngineCtx {
   sl_engine* e;
   sl_snap snap;
-  std::vector<uint16_t> normed;   // rows of the last forward
   int last_m;
 };
 int eng_step(void* c, const int32_t* t, int m, int32_t* out) { return sl_step_argmax(((EngineCtx*)c)->e, t, m, out); }
@@ -192,11 +191,11 @@ int eng_chain(void* c, int32_t first, int k, int32_t* out) { return sl_chained_s
 int eng_forward(void* c, const int32_t* t, int m) {
   EngineCtx* x = (EngineCtx*)c;
   x->last_m = m;
-  return sl_forward_tokens(x->e, t, m, x->normed.data());
+  return sl_forward_tokens(x->e, t, m, nullptr);          // the rows stay on the device
 }
 int eng_first(void* c, int32_t* out) {
   EngineCtx* x = (EngineCtx*)c;
-  return sl_head_argmax(x->e, x->normed.data() + (size_t)(x->last_m - 1) * SL_H, 1, out);
+  return sl_head_argmax_rows(x->e, x->last_m - 1, 1, out);
 }
 int eng_snapshot(void* c) { EngineCtx* x = (EngineCtx*)c; return sl_snapshot(x->e, &x->snap); }
 int eng_rollback(void* c) { EngineCtx* x = (EngineCtx*)c; return sl_rollback_one_step(x->e, &x->snap); }
@@ -207,7 +206,7 @@ extern "C" int sl_spec_generate(sl_engine* e, const int32_t* prompt, int n_promp
   if (!e) return SL_ERR_ARG;
   const int max_rows = sl_max_rows(e);
   if (max_rows < 1) return SL_ERR_ARG;
-  EngineCtx x{e, {}, std::vector<uint16_t>((size_t)max_rows * SL_H), 1};
+  EngineCtx x{e, {}, 1};
   sl_spec_backend b;
   b.ctx = &x; b.max_rows = max_rows;
   b.step_argmax = eng_step; b.chained_step_argmax = eng_chain; b.forward_tokens = eng_forward; b.first_token = eng_first;

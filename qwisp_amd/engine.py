@@ -139,8 +139,12 @@ class SeedlessFusedForward:
             return None
         return out
 
-    def forward_tokens(self, tokens):
+    def forward_tokens(self, tokens, on_device=False):
+        """Tell.SpecBackend.forward.  With on_device the rows stay on the GPU (True is returned); hidden_rows and
+        head_argmax_rows read them afterwards."""
         tok = np.ascontiguousarray(tokens, np.int32)
+        if on_device:
+            return True if self.lib.dll.sl_forward_tokens(self.h, _p(tok), len(tok), None) == abi.SL_OK else None
         out = np.empty((len(tok), abi.H), np.float16)
         if self.lib.dll.sl_forward_tokens(self.h, _p(tok), len(tok), _p(out)) != abi.SL_OK:
             return None
@@ -162,6 +166,13 @@ class SeedlessFusedForward:
         x = np.ascontiguousarray(normed, np.float16).reshape(-1, abi.H)
         out = np.empty(x.shape[0], np.int32)
         if self.lib.dll.sl_head_argmax(self.h, _p(x), x.shape[0], _p(out)) != abi.SL_OK:
+            return None
+        return out
+
+    def head_argmax_rows(self, first, m=1):
+        """lm_head + arg-max over rows first .. first+m-1 of the normed rows the last forward left on the device."""
+        out = np.empty(m, np.int32)
+        if self.lib.dll.sl_head_argmax_rows(self.h, first, m, _p(out)) != abi.SL_OK:
             return None
         return out
 

@@ -25,6 +25,7 @@ SIGNATURES = {
     "sl_chained_step_argmax": (_i32, [_vp, _i32, _i32, _vp]),
     "sl_forward_rows": (_i32, [_vp, _vp, _i32, _i32, _vp]),
     "sl_forward_tokens": (_i32, [_vp, _vp, _i32, _vp]),
+    "sl_head_argmax_rows": (_i32, [_vp, _i32, _i32, _vp]),
     "sl_hidden_rows": (_i32, [_vp, _i32, _vp]),
     "sl_logits_row": (_i32, [_vp, _i32, _vp]),
     "sl_head_argmax": (_i32, [_vp, _vp, _i32, _vp]),

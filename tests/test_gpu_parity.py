@@ -516,6 +516,26 @@ def test_greedy_stream_matches_oracle(env, small_model):
             assert same_bits(g, w), (li, first_diff(g, w))
 
 
+def test_forward_rows_kept_on_the_device(env, small_model):
+    """forward with a NULL result buffer leaves the rows on the device (the reference's forward returns a device array):
+    hidden_rows gives the bits of the copying call, head_argmax_rows on the last row the first token that head_argmax
+    gives on the copied row and that the oracle's greedy loop gives; a step invalidates the rows."""
+    cfg, dev, host = small_model
+    a = env["Engine"](cfg, dev, max_m=16, max_seq_len=64)
+    b = env["Engine"](cfg, dev, max_m=16, max_seq_len=64)
+    ora = env["orc"].Oracle(cfg, host, max_m=16, max_seq_len=64)
+    prompt = np.random.default_rng(77).integers(0, cfg.vocab, 13).astype(np.int32)
+    rows = a.forward_tokens(prompt)
+    assert b.forward_tokens(prompt, on_device=True) is True, b.gpu_fault
+    assert same_bits(b.hidden_rows(13), rows)
+    first = b.head_argmax_rows(12)
+    assert first is not None and first.tolist() == a.head_argmax(rows[-1:]).tolist() == ora.greedy_generate(prompt, 1).tolist()
+    assert b.head_argmax_rows(10, 3).tolist() == a.head_argmax(rows[10:13]).tolist()
+    assert b.head_argmax_rows(12, 2) is None and b.head_argmax_rows(-1, 1) is None      # beyond the rows held
+    assert b.step_argmax([int(first[0])]) is not None
+    assert b.head_argmax_rows(0) is None                                                  # a step ran since
+
+
 def test_rows_equal_single_steps_and_chain(env, small_model):
     """SeedlessVerifyTests.swift:613 (rows == loop of M=1) and :2445 (chain == steps)."""
     cfg, dev, host = small_model
