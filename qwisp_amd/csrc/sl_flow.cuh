@@ -482,28 +482,34 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
   // first unit only.
   uint4 w4 = make_uint4(0, 0, 0, 0);
   int prep_kvh = -1;
-  // A thread stages two 16-byte pieces of a unit's key and value tiles: rows srow and srow + 32 (the row of the new
-  // position comes from this step's projection instead).
+  // A thread stages two 16-byte pieces of a unit's key and value tiles: rows srow and srow + 32.  The tiles travel
+  // through registers one unit ahead of their use, so the loads of the next unit are in flight while this one is
+  // scored or summed.  (Rows beyond the context repeat its last row and the row of the new position is fetched like
+  // any other: neither is stored to LDS, the new row comes from this step's projection instead.)
   const int srow = tid >> 5, c8 = (tid & 31) * 8;
-  auto stage = [&](bool keys, bool values, int u) {
+  uint4 kq[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)}, vq[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+  auto fetch = [&](bool keys, bool values, int u) {
     const int j0 = (u >> 1) * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
     const size_t off = ((size_t)(u & 1) * uni(P.max_seq) + j0) * 256 + c8;
-    uint4 kq[2], vq[2];
-    bool on[2];
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
-      const int row = it * 32 + srow;
-      on[it] = row < nk && j0 + row != pos;
-      if (on[it] && keys) kq[it] = ld16(uni(Y.kcache) + off + (size_t)row * 256);
-      if (on[it] && values) vq[it] = ld16(uni(Y.vcache) + off + (size_t)row * 256);
-    }
-#pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int row = it * 32 + srow;
-      if (on[it] && keys) st16(&L.kt[row * KT_STRIDE + c8], kq[it]);
-      if (on[it] && values) st16(&g_vt[row * 256 + c8], vq[it]);
+      const int row = min(it * 32 + srow, nk - 1);
+      if (keys) kq[it] = ld16(uni(Y.kcache) + off + (size_t)row * 256);
+      if (values) vq[it] = ld16(uni(Y.vcache) + off + (size_t)row * 256);
     }
   };
+  auto put = [&](bool keys, bool values, int u) {
+    const int j0 = (u >> 1) * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int row = it * 32 + srow;
+      if (row < nk && j0 + row != pos) {
+        if (keys) st16(&L.kt[row * KT_STRIDE + c8], kq[it]);
+        if (values) st16(&g_vt[row * 256 + c8], vq[it]);
+      }
+    }
+  };
+  if (wg < U) fetch(true, true, wg);
   for (int ub = wg; ub < U; ub += GU * RND) {
     const int nr = min(RND, (U - ub + GU - 1) / GU);       // units of this round
     // pass 1, keys: scores and softmax weights of every unit of the round; maxima and sums published per tile.
@@ -514,7 +520,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
       const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
       lds_barrier();                    // the key tile aliases the activation vector the in-projection just read
-      stage(true, r == 0, u);
+      put(true, r == 0, u);
       // waves 0..7: query heads of the group; wave 8: new key; wave 9: new value -- 4 tagged words per lane
       const int src = wave < 8 ? (kvh * 8 + wave) * 512 : (wave == 8 ? 8192 + kvh * 256 : 8192 + 512 + kvh * 256);
       if (kvh != prep_kvh) {
@@ -568,6 +574,10 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
         st_co_h4(co_rsrc(uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 4 * lane, o);
         *reinterpret_cast<uint2*>(&L.kt[(pos - j0) * KT_STRIDE + 4 * lane]) = make_uint2(pack2(o[0], o[1]), pack2(o[2], o[3]));
       }
+      // next in line (requested behind the poll above, which must not wait for it): the keys of the round's next
+      // unit, or after the last one the values of its second unit (those of the first are staged already)
+      if (r + 1 < nr) fetch(true, false, u + GU);
+      else if (nr > 1) fetch(false, true, ub + GU);
       lds_barrier();
       {
         // scores: wave (head, half) takes the 32 leaves of its half of the 256 dims, lane j is key j.  The 128
@@ -615,7 +625,11 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
       const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
       lds_barrier();                    // the previous unit's value tile has been read; the weights are in place
-      if (r > 0) stage(false, true, u);
+      if (r > 0) {
+        put(false, true, u);
+        if (r + 1 < nr) fetch(false, true, u + GU);
+      }
+      if (r + 1 == nr && ub + GU * RND < U) fetch(true, true, ub + GU * RND);   // the next round's first unit
       if (has_new && wave == 9) {
         const uint32_t a = vn[kvh * 128 + 2 * lane], b = vn[kvh * 128 + 2 * lane + 1];
         stw2(co_rsrc(uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 2 * lane, a, b);
@@ -850,9 +864,10 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     // First round trip: {max, sum} of the first 64 tiles (lane i fetches tile i), the partials of the first MB tiles
     // and the output gate (it sits in the q projection of this step) are polled together, each piece until it has
     // arrived; at contexts of up to MB tiles that is everything the merge needs.  Beyond that a round trip per MB
-    // tiles would dominate (about 3 us each, whatever its size), so all 16 waves fetch: per block of 64 tiles wave w
-    // polls tiles 4w .. 4w+3 and parks their values in LDS (the value tile's space), and wave 0 then adds the block
-    // up from LDS (its {max, sum} words fetched during the poll).  The accumulation always runs in tile order.
+    // tiles would dominate (two to three us each, whatever its size), so the other waves fetch: waves 2..15 poll
+    // blocks of 64 tiles, two blocks ahead, and park their values in LDS, wave 0 adds a block up from LDS while the
+    // next ones are on their way, and wave 1 carries the chain of the tiles' sums.  The accumulation always runs in
+    // tile order.
     constexpr int MPH = FLOW_MERGE_WGS / SL_ATT_HEADS, LPW = 128 / MPH;      // workgroups per head, chunks (lanes) per workgroup
     const int mi = wg - (G - FLOW_MERGE_WGS), h = mi / MPH, slot0 = h * uni(P.max_tiles);
     const bool act = lane < LPW;
@@ -865,6 +880,29 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     uint2 g2 = make_uint2(0u, 0u);
     if (wave == 0) {
       uint4 a[MB];
+      // maxima of the tiles beyond the first 64, eight blocks per round trip: they are published after the first pass
+      // over the keys, well before the first partial sums, so this wait is over when those arrive
+      for (int t0 = 64; t0 < nt && !fail; t0 += 512) {
+        float pm[8];
+        unsigned have = 0, spins = 0;
+        for (;;) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            if (have & (1u << j)) continue;
+            const int t = t0 + 64 * j + lane;
+            bool ok = true;
+            pm[j] = NEG;
+            if (t < nt) { const uint4 m = ldw4(rml, (slot0 + t) * 4); ok = m.z == tcore32 && m.w == tcore32; pm[j] = __uint_as_float(m.x); }
+            if (__all(ok ? 1 : 0)) have |= 1u << j;
+          }
+          if (have == 0xffu) break;
+          if (++spins > uni(F.spin_limit)) { fail = 1; break; }
+        }
+        if (!fail) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) Mx = fmaxf(Mx, tree_max<64>(pm[j]));
+        }
+      }
       {
         const bool mine = lane < nt;
         const int cnt0 = min(MB, nt);
@@ -891,19 +929,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
           if (++spins > uni(F.spin_limit)) { fail = 1; break; }
           __builtin_amdgcn_s_sleep(1);
         }
-        Mx = tree_max<64>(mine ? __uint_as_float(m0.x) : NEG);
-      }
-      for (int t0 = 64; t0 < nt && !fail; t0 += 64) {       // maxima of the tiles beyond the first 64
-        const bool mine = t0 + lane < nt;
-        unsigned spins = 0;
-        for (;;) {
-          bool ok = true;
-          float pm = NEG;
-          if (mine) { const uint4 m = ldw4(rml, (slot0 + t0 + lane) * 4); ok = m.z == tcore32 && m.w == tcore32; pm = __uint_as_float(m.x); }
-          if (__all(ok ? 1 : 0)) { Mx = fmaxf(Mx, tree_max<64>(pm)); break; }
-          if (++spins > uni(F.spin_limit)) { fail = 1; break; }
-          __builtin_amdgcn_s_sleep(1);
-        }
+        Mx = fmaxf(Mx, tree_max<64>(mine ? __uint_as_float(m0.x) : NEG));
       }
       if (!fail) {                                          // the first batch is already here
         float fl = 0.0f, pl = 0.0f;
@@ -919,53 +945,125 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
       }
     }
     if (nt > MB) {                                          // uniform for the grid
-      uint2* park = reinterpret_cast<uint2*>(g_vt);         // [64 tiles][64 lanes] {o0, o1}
-      lds_barrier();                                      // tile units this workgroup may have had are done with the space
-      for (int t0 = 0; t0 < nt; t0 += 64) {
-        uint4 q[4];
-        // wave 0, lane i: {max, sum} of tile t0 + i (its tags were verified above), fetched in the shadow of the poll
-        uint4 ma = m0;
-        if (wave == 0 && t0 > 0 && t0 + lane < nt) ma = ldw4(rml, (slot0 + t0 + lane) * 4);
-        unsigned spins = 0;
-        for (;;) {
-          bool ok = true;
+      // Blocks of 64 tiles in a pipeline: waves 2..15 poll the partial sums of block b (five tiles each) and park
+      // them in LDS, while wave 0 adds up block b-1 from the other parking buffer in tile order and wave 1 carries
+      // the chain of the tiles' sums (the merge is one dependent chain per lane: a wave that also fetches and sums
+      // the weights issues three times the instructions per tile).  One barrier per block; both groups of waves run
+      // nbp + 1 of them, nbp = the block count rounded up to even (a block beyond the context is empty).
+      uint2* const park0 = reinterpret_cast<uint2*>(g_vt);                       // [64 tiles][64 lanes] {o0, o1}
+      uint2* const park1 = reinterpret_cast<uint2*>(g_vt + SDPA_TILE * 256);     // the softmax weights' space (merging workgroups own no units)
+      static_assert(SDPA_ROUND * 8 * 64 * 4 >= 64 * 64 * 8, "second parking buffer");
+      // (the polling waves start at once, while wave 0 is still waiting for the maxima and the first tiles above; tile
+      // units this workgroup may have had ended with a barrier, so the parking space is free)
+      if (wave == 0) {                                      // for wave 1: the maximum, the sum so far, block 0's {max, sum} words
+        if (lane == 0) { g_L.red[0] = Mx; g_L.red[1] = Ls; }
+        *reinterpret_cast<uint2*>(&g_L.part[2 * lane]) = make_uint2(m0.x, m0.y);
+      }
+      const int nb = (nt + 63) / 64, nbp = (nb + 1) & ~1;
+      if (wave >= 2) {
+        // A wave's five tiles of a block are requested two blocks ahead (a round trip to memory takes about two blocks'
+        // additions), so a block costs a round trip only when its tiles have not been published yet.  Two register
+        // sets take turns: a set is parked and at once requested again for the block after the next.  Every request
+        // is unconditional (tile and block indices clamped into the context), so the wait for one set leaves the
+        // other set's loads in flight.
+        uint4 qa[5], qb[5];
+        auto request = [&](uint4 (&dst)[5], int blk) {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int t = t0 + 4 * wave + j;
-            if (t >= MB && t < nt && act) { q[j] = ldw4(rpo, ((slot0 + t) * 128 + chunk) * 4); ok = ok && q[j].z == tcore32 && q[j].w == tcore32; }
+          for (int j = 0; j < 5; ++j) {
+            const int t = min(64 * min(blk, nb - 1) + min(5 * (wave - 2) + j, 63), nt - 1);
+            dst[j] = ldw4(rpo, ((slot0 + t) * 128 + chunk) * 4);
           }
-          if (__all(ok ? 1 : 0)) break;
-          if (++spins > uni(F.spin_limit)) { fail = 1; break; }
-          __builtin_amdgcn_s_sleep(1);
-        }
+        };
+        auto wanted = [&](int blk, int j) {
+          const int i = 5 * (wave - 2) + j, t = 64 * blk + i;
+          return i < 64 && t >= MB && t < nt && act;
+        };
+        auto poll_block = [&](uint4 (&cur)[5], int blk) {
+          uint2* const park = (blk & 1) ? park1 : park0;
+          unsigned spins = 0;
+          for (;;) {
+            bool ok = true;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int t = t0 + 4 * wave + j;
-          if (t >= MB && t < nt && act) park[(4 * wave + j) * 64 + lane] = make_uint2(q[j].x, q[j].y);
+            for (int j = 0; j < 5; ++j) ok = ok && (!wanted(blk, j) || (cur[j].z == tcore32 && cur[j].w == tcore32));
+            if (__all(ok ? 1 : 0)) break;
+            if (++spins > uni(F.spin_limit)) { fail = 1; break; }
+            request(cur, blk);
+          }
+#pragma unroll
+          for (int j = 0; j < 5; ++j) if (wanted(blk, j)) park[(5 * (wave - 2) + j) * 64 + lane] = make_uint2(cur[j].x, cur[j].y);
+          request(cur, blk + 2);
+        };
+        request(qa, 0);
+        request(qb, 1);
+        for (int b = 0; b < nbp; b += 2) {
+          poll_block(qa, b);
+          lds_barrier();
+          poll_block(qb, b + 1);
+          lds_barrier();
         }
         lds_barrier();
-        if (wave == 0 && !fail) {
-          float fl = 0.0f, pl = 0.0f;                       // lane i: scale and sum of tile t0+i
-          if (t0 + lane < nt) { fl = exp_c(__uint_as_float(ma.x) - Mx); pl = __uint_as_float(ma.y); }
+      } else {
+        // waves 0, 1; lane i: {max, sum} of tile i of the block (tags verified above); the words of the next block are
+        // requested before this one is added up
+        uint4 ma = m0, mb = m0;
+        auto add_block = [&](const uint4& cur, uint4& nxt, int blk) {
+          const int t0 = 64 * blk;
+          const uint2* const park = (blk & 1) ? park1 : park0;
+          nxt = ldw4(rml, (slot0 + min(t0 + 64 + lane, nt - 1)) * 4);
+          float fl = 0.0f, pl = 0.0f;                     // lane i: scale and sum of tile t0+i
+          if (t0 + lane < nt) { fl = exp_c(__uint_as_float(cur.x) - Mx); pl = __uint_as_float(cur.y); }
           const int lo = t0 == 0 ? MB : 0, hi = min(64, nt - t0);
-          for (int u0 = lo; u0 < hi; u0 += 8) {             // eight LDS reads and sixteen lane reads at a time, used in tile order
-            uint2 v[8];
-            float f[8], l[8];
+          if (wave == 0 && !fail) {
+            // sixteen LDS reads and sixteen lane reads at a time, used in tile order (one wave issues an instruction
+            // every eight clocks or so and waits tens of clocks for a batch of either kind: few, large batches)
+            int u0 = lo;
+            for (; u0 + 16 <= hi; u0 += 16) {
+              uint2 v[16];
+              float f[16];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = park[min(u0 + i, 63) * 64 + lane];
-            lanes8(fl, u0, f);
-            lanes8(pl, u0, l);
+              for (int i = 0; i < 16; ++i) v[i] = park[(u0 + i) * 64 + lane];
+              lanes8(fl, u0, reinterpret_cast<float(&)[8]>(f[0]));
+              lanes8(fl, u0 + 8, reinterpret_cast<float(&)[8]>(f[8]));
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-              if (u0 + i < hi) {
-                Ls = fmaf(l[i], f[i], Ls);
-                O0 = fmaf(__uint_as_float(v[i].x), f[i], O0); O1 = fmaf(__uint_as_float(v[i].y), f[i], O1);
+              for (int i = 0; i < 16; ++i) { O0 = fmaf(__uint_as_float(v[i].x), f[i], O0); O1 = fmaf(__uint_as_float(v[i].y), f[i], O1); }
+            }
+            for (; u0 < hi; u0 += 8) {
+              uint2 v[8];
+              float f[8];
+#pragma unroll
+              for (int i = 0; i < 8; ++i) v[i] = park[min(u0 + i, 63) * 64 + lane];
+              lanes8(fl, u0, f);
+#pragma unroll
+              for (int i = 0; i < 8; ++i) {
+                if (u0 + i < hi) { O0 = fmaf(__uint_as_float(v[i].x), f[i], O0); O1 = fmaf(__uint_as_float(v[i].y), f[i], O1); }
               }
             }
+          } else if (wave == 1) {
+            for (int u0 = lo; u0 < hi; u0 += 8) {
+              float f[8], l[8];
+              lanes8(fl, u0, f);
+              lanes8(pl, u0, l);
+#pragma unroll
+              for (int i = 0; i < 8; ++i) if (u0 + i < hi) Ls = fmaf(l[i], f[i], Ls);
+            }
           }
+        };
+        lds_barrier();                                    // block 0 is parked; wave 0 has left the maximum and its sum so far
+        if (wave == 1) {
+          Mx = g_L.red[0]; Ls = g_L.red[1];
+          const uint2 w = *reinterpret_cast<const uint2*>(&g_L.part[2 * lane]);
+          ma.x = w.x; ma.y = w.y;
         }
-        lds_barrier();                                    // the block is consumed before the next one is parked
+        for (int b = 0; b < nbp; b += 2) {
+          add_block(ma, mb, b);
+          lds_barrier();
+          add_block(mb, ma, b + 1);
+          lds_barrier();
+        }
+        if (wave == 1 && lane == 0) g_L.red[2] = Ls;
       }
+      lds_barrier();
+      if (wave == 0) Ls = g_L.red[2];
     }
     if (fail) st_co32(uni(P.bar) + 32, 1u);
     if (wave == 0 && !fail && act) {
