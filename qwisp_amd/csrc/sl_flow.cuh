@@ -240,18 +240,36 @@ SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, fl
 // published first; the rows that are only read a stage later (GDN: z; attention: the output gates; 4096 either
 // way, one per wave) follow while the first batch is on its way to its consumers, and their weights are only
 // requested once this stage's own inputs have arrived, so they stream during the arithmetic.
-//   GDN: workgroup wg owns rows 32 wg .. 32 wg + 31 (wave w: two of them) and every fourth workgroup one of the
-//        64 b / a rows (wave 0); deferred row 8192 + 16 wg + w.
+//   GDN: workgroup wg owns the block of 32 rows gdn_row_block(wg) (wave w: two of them) and eight workgroups of
+//        every XCD one of the 64 b / a rows (wave 0); deferred row 8192 + 16 wg + w.
 //   attention: urgent index c = 20 wg + slot, slot = 2w, 2w + 1 on waves 0..3 and 4 + w on the others;
 //        c < 4096 is query element c % 256 of head c / 256, then k and v; deferred: gate element of the same numbering.
+// GDN layers, who computes what: workgroup n runs on XCD n % 8, and an exchange between workgroups of one XCD goes
+// through that XCD's L2 (1.1 against 1.5 us for a few hundred words).  XCD x therefore owns the value heads 4x .. 4x+3
+// with their two key heads 2x, 2x+1 in both stages: its 32 workgroups compute those heads' q, k, v rows and gate rows
+// of the in-projection (8 + 8 + 16 blocks of 32 rows, eight of them one b / a row more) and then their 32 units (value
+// head, 16 of its 128 value dims) of the recurrence.
+SL_DEV int gdn_row_block(int wg) {              // first of the workgroup's 32 urgent in-projection rows, / 32
+  const int x = wg & 7, j = wg >> 3;
+  if (j < 8) return (2 * x + (j >> 2)) * 4 + (j & 3);                    // q rows of key head 2x + j/4
+  if (j < 16) return 64 + (2 * x + ((j - 8) >> 2)) * 4 + (j & 3);        // k rows
+  return 128 + (4 * x + ((j - 16) >> 2)) * 4 + (j & 3);                  // v rows of value head 4x + (j-16)/4
+}
+SL_DEV int gdn_extra_row(int wg) {              // the workgroup's b (j < 4) or a (j < 8) row, -1: none
+  const int x = wg & 7, j = wg >> 3;
+  return j < 4 ? 12288 + 4 * x + j : (j < 8 ? 12320 + 4 * x + (j - 4) : -1);
+}
+SL_DEV int gdn_unit_head(int wg) { return 4 * (wg & 7) + (wg >> 6); }   // value head of the workgroup's recurrence unit
+SL_DEV int gdn_unit_dvb(int wg) { return (wg >> 3) & 7; }               // its block of 16 value dims
 struct InRows { int crit[3]; int ncrit; int def; };
 SL_DEV int attn_urgent_row(int c) { return c < 4096 ? ((c >> 8) * 512 + (c & 255)) : (8192 + (c - 4096)); }
 SL_DEV int attn_gate_row(int zi) { return (zi >> 8) * 512 + 256 + (zi & 255); }
 SL_DEV InRows in_rows(bool lin, int wg, int wave) {
   InRows r;
   if (lin) {
-    const bool extra = wave == 0 && (wg & 3) == 0;
-    r.crit[0] = wg * 32 + wave * 2; r.crit[1] = r.crit[0] + 1; r.crit[2] = extra ? 12288 + (wg >> 2) : 0;
+    const int xr = gdn_extra_row(wg);
+    const bool extra = wave == 0 && xr >= 0;
+    r.crit[0] = gdn_row_block(wg) * 32 + wave * 2; r.crit[1] = r.crit[0] + 1; r.crit[2] = extra ? xr : 0;
     r.ncrit = extra ? 3 : 2;
     r.def = 8192 + wg * 16 + wave;
   } else {
@@ -330,8 +348,8 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   if (wave == PUB_WAVE) {
     const rsrc_t rp = co_rsrc(uni(F.tproj));
     if (lin) {
-      if (lane < 32) stw1(rp, wg * 32 + lane, g_L.pub[lane]);
-      else if (lane == 32 && (wg & 3) == 0) stw1(rp, 12288 + (wg >> 2), g_L.pub[32]);
+      if (lane < 32) stw1(rp, gdn_row_block(wg) * 32 + lane, g_L.pub[lane]);
+      else if (lane == 32 && gdn_extra_row(wg) >= 0) stw1(rp, gdn_extra_row(wg), g_L.pub[32]);
     } else if (lane < 20) {
       stw1(rp, attn_urgent_row(wg * 20 + lane), g_L.pub[lane]);
     }
@@ -363,7 +381,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
   if (wg >= 256) return true;
   const int par = (int)((uni(g_K.parity) >> li) & 1ull);
   const uint16_t* hin = uni(Y.hist[par]);
-  const int hv = wg >> 3, dvb = wg & 7, hk = hv >> 1;
+  const int hv = gdn_unit_head(wg), dvb = gdn_unit_dvb(wg), hk = hv >> 1;
   const int half = lane >> 5, l32 = lane & 31;
   // waves 8..15 hold the recurrent state (they take no part in this stage's or the next stage's poll)
   float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -833,7 +851,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
 SL_DEV void store_hist(const LayerP& Y, int li, const GdnHist& gh) {
   const int tid = fresh_v(threadIdx.x), wg = fresh_s(blockIdx.x);
   if (tid < 272) {
-    const int hv = wg >> 3, dvb = wg & 7, hk = hv >> 1;
+    const int hv = gdn_unit_head(wg), dvb = gdn_unit_dvb(wg), hk = hv >> 1;
     const int ch = tid < 128 ? hk * 128 + tid : (tid < 256 ? 2048 + hk * 128 + (tid - 128) : 4096 + hv * 128 + dvb * 16 + (tid - 256));
     if (tid >= 256 || ((hv & 1) == 0 && dvb == 0)) {
       uint16_t* hout = uni(Y.hist[(int)(((uni(g_K.parity) >> li) & 1ull) ^ 1ull)]);
@@ -869,9 +887,15 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     // next ones are on their way, and wave 1 carries the chain of the tiles' sums.  The accumulation always runs in
     // tile order.
     constexpr int MPH = FLOW_MERGE_WGS / SL_ATT_HEADS, LPW = 128 / MPH;      // workgroups per head, chunks (lanes) per workgroup
-    const int mi = wg - (G - FLOW_MERGE_WGS), h = mi / MPH, slot0 = h * uni(P.max_tiles);
+    // Workgroup n runs on XCD n % 8, and at short contexts the tile units of heads 2x, 2x+1 run on XCD x (flow_sdpa4:
+    // workgroup % 8 = kv head * 4 + head pair): the workgroups that merge those two heads are taken from the same XCD,
+    // so the partial sums change hands through that XCD's L2 (1.1 against 1.5 us for a small exchange).
+    static_assert(FLOW_MERGE_WGS % 8 == 0 && FLOW_MERGE_WGS / 8 == 2 * MPH, "two heads per XCD");
+    const int mi = wg - (G - FLOW_MERGE_WGS);
+    const int xcd = mi & 7, kx = mi >> 3;                 // (G - FLOW_MERGE_WGS is a multiple of 8 on the full machine)
+    const int h = 2 * xcd + kx / MPH, slot0 = h * uni(P.max_tiles);
     const bool act = lane < LPW;
-    const int chunk = LPW * (mi % MPH) + (act ? lane : 0);      // (idle lanes of a narrower workgroup fetch and store nothing)
+    const int chunk = LPW * (kx % MPH) + (act ? lane : 0);      // (idle lanes of a narrower workgroup fetch and store nothing)
     const rsrc_t rml = co_rsrc(uni(F.tml)), rpo = co_rsrc(uni(F.tpo)), rp = co_rsrc(uni(F.tproj));
     constexpr int MB = 12;
     int fail = 0;
