@@ -1461,45 +1461,70 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
   const DecodeP& P = F.d;
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
-  const int nchunks = (uni(P.vocab) + 63) / 64;
   const int nl = uni(P.n_layers);
   float bv = NEG; int bi = 0x7fffffff;
+  // The vocabulary in groups of four rows, dealt out evenly: wave gw takes groups gw, gw + NW, ... and the groups left
+  // over go one each to waves 0, 1, ... of every workgroup in turn, so that the four waves of a SIMD (which share its
+  // issue slot: the stage ends when the last of them is through) differ by at most one group anywhere on the chip.
+  // A wave meets its groups in rising order, so its first maximum is the one of the lowest index.
+  const int NG = (uni(P.vocab) + 3) / 4, per = NG / NW, ex = wave * G + wg;
+  const int mine = per + (ex < NG - per * NW ? 1 : 0);
+  auto group_of = [&](int k) { return k < per ? gw + k * NW : per * NW + ex; };
   WRegs<1, 4> cur, nxt;
-  auto load_group = [&](WRegs<1, 4>& r, int chunk, int g4) {
+  auto load_group = [&](WRegs<1, 4>& r, int k) {
+    const long g = group_of(k);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const long row = (long)chunk * 64 + g4 * 4 + j;
-      const bool v = chunk < nchunks && row < uni(P.vocab);
+      const long row = g * 4 + j;
+      const bool v = k < mine && row < uni(P.vocab);
       wload_row<1>(r.w[j], r.sb[j], uni(P.lm_w), uni(P.lm_sb), (size_t)(v ? row : 0), v, lane);
     }
   };
-  load_group(cur, gw, 0);
+  load_group(cur, 0);
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(P.final_norm) + 2 * tid);
   float r0, r1;
   fstamp<ST>(nl, 0, 0, tid == 0);
   if (!poll_vec2048<ST>(P, uni(F.tmoe), flow_tag(base, nl - 1, FS_C), r0, r1, nl, 0)) return false;
   const uint32_t thd32 = flow_tag32(base, nl, 0);
   flow_prologue(h0, h1, true, r0, r1, lnw, wg == 0 ? uni(P.normed) : nullptr);
-  for (int chunk = gw; chunk < nchunks; chunk += NW) {
-#pragma unroll 1
-    for (int g4 = 0; g4 < 16; ++g4) {
-      int nchunk = chunk, ng = g4 + 1;
-      if (ng == 16) { ng = 0; nchunk = chunk + NW; }
-      load_group(nxt, nchunk, ng);
-      const F4 o = dot_1x4(cur);
-      const long r0w = (long)chunk * 64 + g4 * 4;
-      if (r0w < uni(P.vocab)) {
+  // the activation row stays in registers for all groups; the two weight sets swap roles from group to group (a copy
+  // would cost twenty moves per group in a stage that is bound by its instruction count)
+  uint32_t x[16]; float sx[4];
+  lds_get_x(0, lane, x, sx);
+  // The four row sums of a group are reduced together.  After the first two levels of the reduction tree (lane
+  // pairs, then quads) the four lanes of a quad hold the same value, so one register can carry all four rows, lane l
+  // the row rho(l) = l % 4 in the lower quad of every eight lanes and 3 - l % 4 in the upper one: the partners of the
+  // remaining levels (mirror within 8, mirror within 16, the other row of 16, the other half) then hold the same row,
+  // and every addition has the operands it has in tree_sum.  A lane follows the maximum of its own row class; the
+  // four classes meet when the stage ends (lowest index on ties, as everywhere).
+  const int rho = (lane & 4) ? 3 - (lane & 3) : (lane & 3);
+  auto group_step = [&](const WRegs<1, 4>& a, WRegs<1, 4>& b, int k) {
+    load_group(b, k + 1);
+    float q[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float v = f16r(o.v[j]);
-          if (v > bv) { bv = v; bi = (int)(r0w + j); }
-        }
-        if (lane == 0) *reinterpret_cast<uint2*>(uni(P.logits) + r0w) = make_uint2(pack2(o.v[0], o.v[1]), pack2(o.v[2], o.v[3]));
-      }
-      cur = nxt;
+    for (int j = 0; j < 4; ++j) q[j] = tree_sum<4>(quad_term(a.w[j][0], a.sb[j][0], x, sx));
+    float f = rho == 0 ? q[0] : (rho == 1 ? q[1] : (rho == 2 ? q[2] : q[3]));
+    f = f + dpp_f<DPP_HALF_MIRROR>(f);
+    f = f + dpp_f<DPP_MIRROR>(f);
+    f = swap32_sum(swap16_sum(f));
+    const long row = (long)group_of(k) * 4 + rho;
+    if (row < uni(P.vocab)) {
+      const float v = f16r(f);
+      if (v > bv) { bv = v; bi = (int)row; }
+      if (lane < 4) uni(P.logits)[row] = f2h(f);
     }
+  };
+#pragma unroll 1
+  for (int k = 0; k < mine; k += 2) {
+    group_step(cur, nxt, k);
+    if (k + 1 < mine) group_step(nxt, cur, k + 1);
   }
   fstamp<ST>(nl, 0, 3, tid == 0);
+#pragma unroll
+  for (int msk = 1; msk < 4; msk <<= 1) {               // lanes 0..3: the four row classes
+    const float ov = __shfl_xor(bv, msk, 64); const int oi = __shfl_xor(bi, msk, 64);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
   if (lane == 0) { L.red[wave] = bv; L.ired[wave] = bi; }
   lds_barrier();
   if (wave == PUB_WAVE && lane == 0) {
