@@ -56,12 +56,20 @@ def tie_placements(a, vocab):
     other_wg = (a + 3 * 1024) % vocab
     far = (a + vocab // 2 + 17) % vocab
     low = 3 if a > 3 else vocab - 5
-    return [[same_group], [same_wave], [next_wave], [other_wg], [far], [low, far], [same_group, other_wg, low]]
+    # the single-launch head deals groups of four rows out to its 4096 waves in turn (group g to wave g % 4096, the
+    # groups left over one each to the first waves of every workgroup): a later group of the winner's wave, the wave
+    # after it, and a row of the left-over groups
+    turn = 4 * 4096
+    later_group = (a + turn) % (vocab - vocab % turn) if vocab >= 2 * turn else far
+    wave_after = (a + 4) % vocab
+    left_over = vocab - 7
+    return [[same_group], [same_wave], [next_wave], [other_wg], [far], [low, far], [same_group, other_wg, low],
+            [later_group], [wave_after], [left_over], [later_group, left_over]]
 
 
 def test_argmax_ties_go_to_the_lowest_index_on_every_path(env):
     torch, Engine, orc = env["torch"], env["Engine"], env["orc"]
-    cfg = ModelConfig(n_layers=1, n_experts=8, vocab=16384, layer_types=("gdn",))
+    cfg = ModelConfig(n_layers=1, n_experts=8, vocab=4 * (3 * 4096 + 640), layer_types=("gdn",))   # three turns of the waves + left-over groups
     dev, host = device_and_host_model(cfg)
     eng0 = Engine(cfg, dev, max_m=32, max_seq_len=64)
     tok = 5
