@@ -144,6 +144,25 @@ SL_DEV float tree_sum(float v) {
   return lo + hi;
 #endif
 }
+// Four sums over the 64 lanes reduced together.  After the first two levels of tree_sum (lane pairs, then quads)
+// the four lanes of a quad hold the same value, so one register can carry all four: lane l the value of row
+// rho(l) = l % 4 in the lower quad of every eight lanes and 3 - l % 4 in the upper one.  The partners of the remaining
+// levels (mirror within 8, mirror within 16, the other row of 16, the other half) then hold the same row, and every
+// addition has the operands it has in tree_sum<64>: the same bits with 19 instead of 40 instructions.  Returns the
+// sum of row rho(lane); lanes 0..3 hold rows 0..3.
+SL_DEV int quad_row(int lane) { return (lane & 4) ? 3 - (lane & 3) : (lane & 3); }
+SL_DEV float tree_sum4(float q0, float q1, float q2, float q3, int lane) {
+  q0 = tree_sum<4>(q0); q1 = tree_sum<4>(q1); q2 = tree_sum<4>(q2); q3 = tree_sum<4>(q3);
+  const int rho = quad_row(lane);
+  float f = rho == 0 ? q0 : (rho == 1 ? q1 : (rho == 2 ? q2 : q3));
+  f = f + dpp_f<DPP_HALF_MIRROR>(f);
+  f = f + dpp_f<DPP_MIRROR>(f);
+  return swap32_sum(swap16_sum(f));
+}
+// The value of lane j of the caller's quad, j = 0..3 (after tree_sum4: rows 0..3, in the lower quad of every eight lanes).
+SL_DEV void quad_values(float f, float (&out)[4]) {
+  out[0] = dpp_f<0x00>(f); out[1] = dpp_f<0x55>(f); out[2] = dpp_f<0xAA>(f); out[3] = dpp_f<0xFF>(f);
+}
 template <int WIDTH>
 SL_DEV float tree_max(float v) {
   static_assert(WIDTH == 64, "group sizes used by the kernels");

@@ -269,8 +269,15 @@ __global__ __launch_bounds__(HIDDEN ? 512 : 256, HIDDEN ? 2 : 3) void k_qmv_tile
       }
     }
     float out[R];
+    if constexpr (R == 4) {                              // the four sums in one register, then handed round the quad
+      float o4[4];
+      quad_values(tree_sum4(acc[0], acc[1], acc[2], acc[3], lane), o4);
 #pragma unroll
-    for (int r = 0; r < R; ++r) out[r] = tree_sum<64>(acc[r]);
+      for (int r = 0; r < 4; ++r) out[r] = o4[r];
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; ++r) out[r] = tree_sum<64>(acc[r]);
+    }
     if constexpr (ARGMAX) {
       if (lane == 0) {
         float bv = -__int_as_float(0x7f800000);
@@ -923,8 +930,8 @@ __global__ __launch_bounds__(256, 3) void k_moe_b_grouped(MoeBGroupArgs a) {
       for (int q = 0; q < 4; ++q) { const uint4 v = src[q]; xp[4 * q] = v.x; xp[4 * q + 1] = v.y; xp[4 * q + 2] = v.z; xp[4 * q + 3] = v.w; }
       { const uint4 v = src[4]; sx[0] = __uint_as_float(v.x); sx[1] = __uint_as_float(v.y); sx[2] = __uint_as_float(v.z); sx[3] = __uint_as_float(v.w); }
       float o[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) o[r] = tree_sum<64>(quad_term_masked(mk[r], sb[r], xp, sx));
+      quad_values(tree_sum4(quad_term_masked(mk[0], sb[0], xp, sx), quad_term_masked(mk[1], sb[1], xp, sx),
+                            quad_term_masked(mk[2], sb[2], xp, sx), quad_term_masked(mk[3], sb[3], xp, sx), lane), o);
       if (lane == 0)
         *reinterpret_cast<uint32_t*>(a.act + (size_t)s_pair[j] * 512 + i0) =
             pack2(swiglu16(f16r(o[0]), f16r(o[2])), swiglu16(f16r(o[1]), f16r(o[3])));
@@ -948,15 +955,14 @@ __global__ __launch_bounds__(256) void k_moe_b(MoeBArgs a) {
   word_sums(x, sx);
   uint32_t xp[16];
   pack_x(x, xp);
-  float o[4];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const float g = tree_sum<64>(quad_term(gw[r], gs[r], xp, sx));
-    const float u = tree_sum<64>(quad_term(uw[r], us[r], xp, sx));
-    o[r] = swiglu16(f16r(g), f16r(u));
-  }
-  if (lane == 0)
-    *reinterpret_cast<uint2*>(a.act + ((size_t)m * 8 + k) * 512 + i0) = make_uint2(pack2(o[0], o[1]), pack2(o[2], o[3]));
+  // the four gate sums and the four up sums each reduced in one register: lane r (r < 4) holds row r of both and
+  // forms its SwiGLU
+  const float g = tree_sum4(quad_term(gw[0], gs[0], xp, sx), quad_term(gw[1], gs[1], xp, sx),
+                            quad_term(gw[2], gs[2], xp, sx), quad_term(gw[3], gs[3], xp, sx), lane);
+  const float u = tree_sum4(quad_term(uw[0], us[0], xp, sx), quad_term(uw[1], us[1], xp, sx),
+                            quad_term(uw[2], us[2], xp, sx), quad_term(uw[3], us[3], xp, sx), lane);
+  const float o = swiglu16(f16r(g), f16r(u));
+  if (lane < 4) a.act[((size_t)m * 8 + k) * 512 + i0 + lane] = f2h(o);
 }
 
 // MoE stage C: routed down-proj, half-precision combine in routing order, shared down-proj and the
