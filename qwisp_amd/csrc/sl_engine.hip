@@ -120,6 +120,7 @@ struct sl_engine {
   float *rope_cos = nullptr, *rope_sin = nullptr;
   // scratch
   uint16_t *hA = nullptr, *hB = nullptr, *proj = nullptr, *ycore = nullptr, *qrot = nullptr, *mix = nullptr, *xn = nullptr;
+  float* xsum = nullptr;           // [max_m, 256] word sums of the rows in xn (steps of two or more rows)
   uint16_t *rlogits = nullptr, *sgate = nullptr, *sh_act = nullptr, *act = nullptr, *moe_out = nullptr, *normed = nullptr;
   uint16_t *logits = nullptr, *rows_out = nullptr;
   float *pm = nullptr, *pl = nullptr, *po = nullptr, *cand_v = nullptr;
@@ -320,17 +321,19 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   a.sh_act = e->sh_act; a.rlogits = e->rlogits; a.sgate = e->sgate;
   const int router_blocks = (e->n_experts + 1 + 15) / 16;
   if (M >= 2) {                                         // residual + norm once per row instead of once per wave
-    hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, ha);
+    HiddenArgs hs = ha;
+    hs.xs_out = e->xsum;                                // and the row's word sums for the routed experts' dots
+    hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hs);
     a.xn_in = ha.xn_out;
   }
   hipLaunchKernelGGL(k_moe_a, dim3(MOE_A_SHARED_BLOCKS + router_blocks, M), dim3(256), 0, e->stream, a);
   hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, e->n_experts, L.route_inds, L.route_scores);
   MoeBArgs b{};
   b.xn = e->xn; b.g_w = L.sw_gate.w; b.g_sb = L.sw_gate.sb; b.u_w = L.sw_up.w; b.u_sb = L.sw_up.sb;
-  b.act = e->act; b.inds = L.route_inds;
+  b.act = e->act; b.inds = L.route_inds; b.xsum = M >= 2 ? e->xsum : nullptr;
   if (M >= MOE_GROUP_MIN_ROWS && M <= GROUP_CAP) {      // weights of an expert fetched once for all rows that chose it
     hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, e->n_experts, e->hy_lists, e->hy_counts, (int32_t*)nullptr);
-    MoeBGroupArgs g{e->xn, b.g_w, b.g_sb, b.u_w, b.u_sb, e->act, e->hy_lists, e->hy_counts};
+    MoeBGroupArgs g{e->xn, b.g_w, b.g_sb, b.u_w, b.u_sb, e->act, e->hy_lists, e->hy_counts, e->xsum};
     hipLaunchKernelGGL(k_moe_b_grouped, dim3(64, e->n_experts), dim3(256), 0, e->stream, g);
   } else {
     hipLaunchKernelGGL(k_moe_b, dim3(256, M), dim3(256), 0, e->stream, b);
@@ -346,6 +349,7 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
 void launch_hidden_tile(sl_engine* e, const HiddenArgs& ha, const uint32_t* w, const uint32_t* sb, int N, int M) {
   HiddenArgs hn = ha;
   hn.xn_out = e->xn;
+  hn.xs_out = e->xsum;
   hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
   constexpr int PLACES = 768;
   int G = N / 16;
@@ -353,7 +357,7 @@ void launch_hidden_tile(sl_engine* e, const HiddenArgs& ha, const uint32_t* w, c
   if (G > PLACES && over <= 16) G -= over;
   if (G * 16 + G < N) G = (N + 15) / 16;          // (not with the shapes of this model)
   hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, false>), dim3(G, (M + 7) / 8), dim3(256), 0, e->stream, HiddenArgs{}, e->xn, H,
-                     w, sb, N, e->proj, PROJ_STRIDE, M);
+                     w, sb, N, e->proj, PROJ_STRIDE, M, (float*)nullptr, (int32_t*)nullptr, e->xsum);
 }
 // Hybrid mode: steps of at least 16 rows (prefill chunks, lane batches) take the dense projections to the matrix cores.
 // (Rows of one sequence or one row each of a batch of lanes: the projections and the experts do not care.)
@@ -706,7 +710,7 @@ int alloc_runtime(sl_engine* e) {
   e->hA = dalloc<uint16_t>(e, MH, true); e->hB = dalloc<uint16_t>(e, MH, true);
   e->proj = dalloc<uint16_t>(e, (size_t)max_m * PROJ_STRIDE, true);
   e->ycore = dalloc<uint16_t>(e, (size_t)max_m * 4096, true);
-  e->mix = dalloc<uint16_t>(e, MH, true); e->xn = dalloc<uint16_t>(e, MH, true);
+  e->mix = dalloc<uint16_t>(e, MH, true); e->xn = dalloc<uint16_t>(e, MH, true); e->xsum = dalloc<float>(e, (size_t)max_m * 256, true);
   e->rlogits = dalloc<uint16_t>(e, (size_t)max_m * 256, true); e->sgate = dalloc<uint16_t>(e, max_m, true);
   e->sh_act = dalloc<uint16_t>(e, (size_t)max_m * 512, true); e->act = dalloc<uint16_t>(e, (size_t)max_m * 8 * 512, true);
   e->hy_lists = dalloc<uint16_t>(e, (size_t)SL_MAX_EXPERTS * GROUP_CAP, true);
@@ -719,7 +723,7 @@ int alloc_runtime(sl_engine* e) {
   e->tok_in = dalloc<int32_t>(e, max_m, true);
   e->tok_out = dalloc<int32_t>(e, max_m > MAX_CHAIN ? max_m : MAX_CHAIN, true);
   e->st = dalloc<int32_t>(e, 1 + d->n_layers, true);
-  if (!e->hA || !e->hB || !e->proj || !e->ycore || !e->mix || !e->xn || !e->rlogits || !e->sgate || !e->sh_act || !e->act || !e->hy_lists || !e->hy_counts ||
+  if (!e->hA || !e->hB || !e->proj || !e->ycore || !e->mix || !e->xn || !e->xsum || !e->rlogits || !e->sgate || !e->sh_act || !e->act || !e->hy_lists || !e->hy_counts ||
       !e->moe_out || !e->normed || !e->rows_out || !e->tok_in || !e->tok_out || !e->st) return SL_ERR_DEVICE;
   if (has_head) {
     int ncu = 0;

@@ -45,6 +45,7 @@ struct HiddenArgs {
   const uint16_t* lnw;     // [2048] norm weight, or null for "x is used as given"
   uint16_t* h_out;         // [M, 2048] receives half(h + r) (written once per row), or null
   uint16_t* xn_out;        // [M, 2048] receives the normed row (written once per row), or null
+  float* xs_out;           // [M, 256] receives the left-to-right sums of each run of 8 elements of that row (word_sums), or null
 };
 // Every wave of the grid calls this; `writer` selects the single wave that stores the outputs.
 SL_DEV void hidden_prologue(const HiddenArgs& a, int m, int lane, bool writer, float* x) {
@@ -64,6 +65,11 @@ SL_DEV void hidden_prologue(const HiddenArgs& a, int m, int lane, bool writer, f
     for (int i = 0; i < 32; ++i) x[i] = f16r(w[i] * f16r(x[i] * inv));
   }
   if (writer && a.xn_out) store32(a.xn_out + (size_t)m * H + 32 * lane, x);
+  if (writer && a.xs_out) {                       // the dots of the row's consumers need these sums: formed once here
+    float sx[4];
+    word_sums(x, sx);
+    *reinterpret_cast<float4*>(a.xs_out + (size_t)m * 256 + 4 * lane) = make_float4(sx[0], sx[1], sx[2], sx[3]);
+  }
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -196,7 +202,8 @@ template <int NBLK, int R, int MT, bool HIDDEN, bool ARGMAX = false>
 __global__ __launch_bounds__(HIDDEN ? 512 : 256, HIDDEN ? 2 : 3) void k_qmv_tile(HiddenArgs ha, const uint16_t* __restrict__ xin, int x_stride,
                                                   const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB,
                                                   int N, uint16_t* __restrict__ y, int y_stride, int M,
-                                                  float* __restrict__ cand_v = nullptr, int32_t* __restrict__ cand_i = nullptr) {
+                                                  float* __restrict__ cand_v = nullptr, int32_t* __restrict__ cand_i = nullptr,
+                                                  const float* __restrict__ xsums = nullptr) {
   static_assert(!HIDDEN || NBLK == 1, "the hidden row is one block of 2048");
   static_assert(!ARGMAX || R == 4, "candidates are formed over four rows per wave");
   constexpr int WPR = NBLK * 256, GPR = NBLK * 32;
@@ -224,13 +231,20 @@ __global__ __launch_bounds__(HIDDEN ? 512 : 256, HIDDEN ? 2 : 3) void k_qmv_tile
   for (int m = wave; m < mc; m += waves) {
 #pragma unroll
     for (int b = 0; b < NBLK; ++b) {
+      uint4* dst = xs + ((m * NBLK + b) * 64 + lane) * 5;
+      if (!HIDDEN && NBLK == 1 && xsums) {                 // the stored halves are the packed pairs; their sums came with the row
+        const uint16_t* src = xin + (size_t)(m0 + m) * x_stride + 32 * lane;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[j] = ld16(src + 8 * j);
+        dst[4] = ld16(xsums + (size_t)(m0 + m) * 256 + 4 * lane);
+        continue;
+      }
       float x[32], sx[4];
       if constexpr (HIDDEN) hidden_prologue(ha, m0 + m, lane, blockIdx.x == 0, x);
       else load32(xin + (size_t)(m0 + m) * x_stride + b * 2048 + 32 * lane, x);
       word_sums(x, sx);
       uint32_t xp[16];
       pack_x(x, xp);
-      uint4* dst = xs + ((m * NBLK + b) * 64 + lane) * 5;
 #pragma unroll
       for (int j = 0; j < 4; ++j) dst[j] = make_uint4(xp[4 * j], xp[4 * j + 1], xp[4 * j + 2], xp[4 * j + 3]);
       dst[4] = make_uint4(__float_as_uint(sx[0]), __float_as_uint(sx[1]), __float_as_uint(sx[2]), __float_as_uint(sx[3]));
@@ -829,6 +843,7 @@ struct MoeBArgs {
   const uint32_t *g_w, *g_sb, *u_w, *u_sb;   // [E*512, 2048]
   uint16_t* act;               // [M, 8, 512]
   const int32_t* inds;         // [M, 8]
+  const float* xsum;           // [M, 256] word sums of the rows (HiddenArgs::xs_out), or null: formed here
 };
 constexpr int GROUP_CAP = 2048;         // pairs per expert: an expert is chosen at most once per row, M <= 2048
 // Pairs (row, slot) listed per expert (M * 8 pairs walked by 1024 threads), places handed out by LDS counters.
@@ -880,6 +895,7 @@ struct MoeBGroupArgs {
   uint16_t* act;               // [M, 8, 512]
   const uint16_t* lists;       // [E, GROUP_CAP] pair indices row*8 + slot
   const int32_t* counts;       // [E]
+  const float* xsum;           // [M, 256] word sums of the rows (HiddenArgs::xs_out), or null: formed here
 };
 constexpr int MOEB_MT = 8;
 __global__ __launch_bounds__(256, 3) void k_moe_b_grouped(MoeBGroupArgs a) {
@@ -904,12 +920,19 @@ __global__ __launch_bounds__(256, 3) void k_moe_b_grouped(MoeBGroupArgs a) {
     for (int j = wave; j < mc; j += 4) {
       const int p = a.lists[(size_t)e * GROUP_CAP + t0 + j];
       if (lane == 0) s_pair[j] = p;
+      uint4* dst = xs + (j * 64 + lane) * 5;
+      if (a.xsum) {                                        // the stored halves are the packed pairs; their sums came with the row
+        const uint16_t* src = a.xn + (size_t)(p >> 3) * H + 32 * lane;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dst[q] = ld16(src + 8 * q);
+        dst[4] = ld16(a.xsum + (size_t)(p >> 3) * 256 + 4 * lane);
+        continue;
+      }
       float x[32], sx[4];
       load32(a.xn + (size_t)(p >> 3) * H + 32 * lane, x);
       word_sums(x, sx);
       uint32_t xp[16];
       pack_x(x, xp);
-      uint4* dst = xs + (j * 64 + lane) * 5;
 #pragma unroll
       for (int q = 0; q < 4; ++q) dst[q] = make_uint4(xp[4 * q], xp[4 * q + 1], xp[4 * q + 2], xp[4 * q + 3]);
       dst[4] = make_uint4(__float_as_uint(sx[0]), __float_as_uint(sx[1]), __float_as_uint(sx[2]), __float_as_uint(sx[3]));
@@ -950,11 +973,20 @@ __global__ __launch_bounds__(256) void k_moe_b(MoeBArgs a) {
     gw[r] = ld16(a.g_w + (base + r) * 256 + 4 * lane); gs[r] = a.g_sb[(base + r) * 32 + (lane >> 1)];
     uw[r] = ld16(a.u_w + (base + r) * 256 + 4 * lane); us[r] = a.u_sb[(base + r) * 32 + (lane >> 1)];
   }
-  float x[32], sx[4];
-  load32(a.xn + (size_t)m * H + 32 * lane, x);
-  word_sums(x, sx);
+  float sx[4];
   uint32_t xp[16];
-  pack_x(x, xp);
+  if (a.xsum) {                                          // the stored halves are the packed pairs
+    const uint16_t* src = a.xn + (size_t)m * H + 32 * lane;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { const uint4 v = ld16(src + 8 * j); xp[4 * j] = v.x; xp[4 * j + 1] = v.y; xp[4 * j + 2] = v.z; xp[4 * j + 3] = v.w; }
+    const float4 s4 = *reinterpret_cast<const float4*>(a.xsum + (size_t)m * 256 + 4 * lane);
+    sx[0] = s4.x; sx[1] = s4.y; sx[2] = s4.z; sx[3] = s4.w;
+  } else {
+    float x[32];
+    load32(a.xn + (size_t)m * H + 32 * lane, x);
+    word_sums(x, sx);
+    pack_x(x, xp);
+  }
   // the four gate sums and the four up sums each reduced in one register: lane r (r < 4) holds row r of both and
   // forms its SwiGLU
   const float g = tree_sum4(quad_term(gw[0], gs[0], xp, sx), quad_term(gw[1], gs[1], xp, sx),
