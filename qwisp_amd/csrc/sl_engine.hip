@@ -326,17 +326,27 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
     hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hs);
     a.xn_in = ha.xn_out;
   }
-  hipLaunchKernelGGL(k_moe_a, dim3(MOE_A_SHARED_BLOCKS + router_blocks, M), dim3(256), 0, e->stream, a);
+  const bool grouped = M >= MOE_GROUP_MIN_ROWS && M <= GROUP_CAP;   // the shared expert then rides with the routed ones, by expert
+  a.skip_shared = grouped ? 1 : 0;
+  hipLaunchKernelGGL(k_moe_a, dim3((grouped ? 0 : MOE_A_SHARED_BLOCKS) + router_blocks, M), dim3(256), 0, e->stream, a);
   hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, e->n_experts, L.route_inds, L.route_scores);
   MoeBArgs b{};
   b.xn = e->xn; b.g_w = L.sw_gate.w; b.g_sb = L.sw_gate.sb; b.u_w = L.sw_up.w; b.u_sb = L.sw_up.sb;
   b.act = e->act; b.inds = L.route_inds; b.xsum = M >= 2 ? e->xsum : nullptr;
-  if (M >= MOE_GROUP_MIN_ROWS && M <= GROUP_CAP) {      // weights of an expert fetched once for all rows that chose it
-    hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, e->n_experts, e->hy_lists, e->hy_counts, (int32_t*)nullptr);
-    MoeBGroupArgs g{e->xn, b.g_w, b.g_sb, b.u_w, b.u_sb, e->act, e->hy_lists, e->hy_counts, e->xsum};
-    hipLaunchKernelGGL(k_moe_b_grouped, dim3(64, e->n_experts), dim3(256), 0, e->stream, g);
+  if (grouped) {                                        // weights of an expert fetched once for all rows that chose it
+    hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, e->n_experts, e->hy_lists, e->hy_counts, e->hy_counts + SL_MAX_EXPERTS);
+    MoeBGroupArgs g{e->xn, b.g_w, b.g_sb, b.u_w, b.u_sb, e->act, e->hy_lists, e->hy_counts, e->xsum, e->hy_counts + SL_MAX_EXPERTS,
+                    L.sh_gate.w, L.sh_gate.sb, L.sh_up.w, L.sh_up.sb, e->sh_act, M};
+    hipLaunchKernelGGL(k_moe_b_grouped, dim3(64, (M + 63) / 64 + e->n_experts), dim3(256), 0, e->stream, g);
   } else {
     hipLaunchKernelGGL(k_moe_b, dim3(256, M), dim3(256), 0, e->stream, b);
+  }
+  if (M >= MOE_GROUP_MIN_ROWS && M <= GROUP_CAP && e->hy_d && e->hy_sy) {   // the down stage by expert as well, then the combine
+    MoeCGroupArgs cg{e->act, e->sh_act, L.sw_down.w, L.sw_down.sb, L.sh_down.w, L.sh_down.sb, e->hy_lists, e->hy_counts,
+                     e->hy_counts + SL_MAX_EXPERTS, e->hy_d, e->hy_sy, M, e->n_experts};
+    hipLaunchKernelGGL(k_moe_c_grouped, dim3(64, (M + 63) / 64 + e->n_experts), dim3(256), 0, e->stream, cg);
+    hipLaunchKernelGGL(k_moe_combine_rows, dim3(H / 256, M), dim3(256), 0, e->stream, e->hy_d, L.route_scores, e->sgate, e->hy_sy, e->moe_out);
+    return;
   }
   MoeCArgs c{};
   c.act = e->act; c.sh_act = e->sh_act; c.inds = L.route_inds; c.scores = L.route_scores; c.sgate = e->sgate;
@@ -711,6 +721,11 @@ int alloc_runtime(sl_engine* e) {
   e->proj = dalloc<uint16_t>(e, (size_t)max_m * PROJ_STRIDE, true);
   e->ycore = dalloc<uint16_t>(e, (size_t)max_m * 4096, true);
   e->mix = dalloc<uint16_t>(e, MH, true); e->xn = dalloc<uint16_t>(e, MH, true); e->xsum = dalloc<float>(e, (size_t)max_m * 256, true);
+  if (max_m >= MOE_GROUP_MIN_ROWS) {               // exact steps of many rows run the experts' down stage by expert: results by pair, then the combine
+    const size_t rows = (size_t)(max_m < GROUP_CAP ? max_m : GROUP_CAP);
+    e->hy_d = dalloc<uint16_t>(e, rows * 8 * H); e->hy_sy = dalloc<uint16_t>(e, rows * H);
+    if (!e->hy_d || !e->hy_sy) return SL_ERR_DEVICE;
+  }
   e->rlogits = dalloc<uint16_t>(e, (size_t)max_m * 256, true); e->sgate = dalloc<uint16_t>(e, max_m, true);
   e->sh_act = dalloc<uint16_t>(e, (size_t)max_m * 512, true); e->act = dalloc<uint16_t>(e, (size_t)max_m * 8 * 512, true);
   e->hy_lists = dalloc<uint16_t>(e, (size_t)SL_MAX_EXPERTS * GROUP_CAP, true);
@@ -956,11 +971,11 @@ float sl_last_gpu_ms(const sl_engine* e) { return e ? e->last_ms : 0.0f; }
 void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
 int sl_set_hybrid(sl_engine* e, int enable) {
   int r = guard(e); if (r) return r;
-  if (enable && !e->hy_d) {
+  if (enable && !e->hy_sg) {
     const size_t rows = (size_t)(e->max_m < GROUP_CAP ? e->max_m : GROUP_CAP);
-    e->hy_d = dalloc<uint16_t>(e, rows * 8 * H);
+    if (!e->hy_d) e->hy_d = dalloc<uint16_t>(e, rows * 8 * H);        // (engines of 128 rows or more have these two already)
     e->hy_sg = dalloc<uint16_t>(e, rows * SL_MOE_I); e->hy_su = dalloc<uint16_t>(e, rows * SL_MOE_I);
-    e->hy_sy = dalloc<uint16_t>(e, rows * H);
+    if (!e->hy_sy) e->hy_sy = dalloc<uint16_t>(e, rows * H);
     if (!e->hy_d || !e->hy_sg || !e->hy_su || !e->hy_sy) return SL_ERR_DEVICE;
     if (rows >= GC) {
       e->gc_scratch = dalloc<unsigned char>(e, (rows / GC) * SL_GDN_HV * GC_UNIT_BYTES);

@@ -885,7 +885,7 @@ __global__ __launch_bounds__(1024) void k_group_pairs(const int32_t* __restrict_
     if (part == 0 && e < E) order[rank] = e;
   }
 }
-// Stage B by expert (steps of many rows): grid (64, E).  A workgroup holds eight gate/up row pairs of one expert
+// Stage B by expert (steps of many rows): grid (64, E), or (64, ceil(M / 64) + E) with the shared expert.  A workgroup holds eight gate/up row pairs of one expert
 // (two pairs per wave, unpacked into masks once) and walks the expert's list of (row, slot) pairs in tiles of
 // MOEB_MT activation rows parked in LDS as in k_qmv_tile, so the expert's weights are fetched and unpacked once
 // per step instead of once per row that chose it.  Same arithmetic per (pair, weight row) as k_moe_b.
@@ -896,29 +896,43 @@ struct MoeBGroupArgs {
   const uint16_t* lists;       // [E, GROUP_CAP] pair indices row*8 + slot
   const int32_t* counts;       // [E]
   const float* xsum;           // [M, 256] word sums of the rows (HiddenArgs::xs_out), or null: formed here
+  const int32_t* order;        // [E] experts by falling count: the long lists start first
+  // the shared expert as one more list (every row of the step, in segments of 64 rows that come first in the grid):
+  const uint32_t *shg_w, *shg_sb, *shu_w, *shu_sb;   // its gate_proj / up_proj [512, 2048], or null: grid (64, E) only
+  uint16_t* sh_act;            // [M, 512]
+  int M;
 };
-constexpr int MOEB_MT = 8;
+constexpr int MOEB_MT = 8;          // pairs per tile: one per eight lanes of a wave in the tile's SwiGLU
 __global__ __launch_bounds__(256, 3) void k_moe_b_grouped(MoeBGroupArgs a) {
   __shared__ uint4 xs[MOEB_MT * 64 * 5];
   __shared__ int s_pair[MOEB_MT];
-  const int e = blockIdx.y, cnt = min(a.counts[e], GROUP_CAP);
+  const int S = a.shg_w ? (a.M + 63) / 64 : 0;           // grid (64, S + E): the shared expert's segments, then the experts
+  const bool shared = (int)blockIdx.y < S;
+  const int e = shared ? 0 : a.order[blockIdx.y - S];
+  const int row0 = shared ? 64 * blockIdx.y : 0;
+  const int cnt = shared ? min(64, a.M - row0) : min(a.counts[e], GROUP_CAP);
   if (cnt == 0) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int i0 = (blockIdx.x * 4 + wave) * 2;
   const size_t base = (size_t)e * 512 + i0;
+  const uint32_t* const gw = shared ? a.shg_w : a.g_w;
+  const uint32_t* const gsb = shared ? a.shg_sb : a.g_sb;
+  const uint32_t* const uw = shared ? a.shu_w : a.u_w;
+  const uint32_t* const usb = shared ? a.shu_sb : a.u_sb;
   uint4 wv[4];
   uint32_t sb[4];
 #pragma unroll
   for (int r = 0; r < 2; ++r) {
-    wv[r] = ld16(a.g_w + (base + r) * 256 + 4 * lane); sb[r] = a.g_sb[(base + r) * 32 + (lane >> 1)];
-    wv[2 + r] = ld16(a.u_w + (base + r) * 256 + 4 * lane); sb[2 + r] = a.u_sb[(base + r) * 32 + (lane >> 1)];
+    wv[r] = ld16(gw + (base + r) * 256 + 4 * lane); sb[r] = gsb[(base + r) * 32 + (lane >> 1)];
+    wv[2 + r] = ld16(uw + (base + r) * 256 + 4 * lane); sb[2 + r] = usb[(base + r) * 32 + (lane >> 1)];
   }
   h2_t mk[4][16];
   for (int t0 = 0; t0 < cnt; t0 += MOEB_MT) {
     const int mc = min(MOEB_MT, cnt - t0);
     if (t0) __syncthreads();                             // the previous tile has been read
     for (int j = wave; j < mc; j += 4) {
-      const int p = a.lists[(size_t)e * GROUP_CAP + t0 + j];
+      // a pair index row * 8 + slot; a row of the shared expert counts as its slot 0 here
+      const int p = shared ? (row0 + t0 + j) * 8 : (int)a.lists[(size_t)e * GROUP_CAP + t0 + j];
       if (lane == 0) s_pair[j] = p;
       uint4* dst = xs + (j * 64 + lane) * 5;
       if (a.xsum) {                                        // the stored halves are the packed pairs; their sums came with the row
@@ -945,6 +959,10 @@ __global__ __launch_bounds__(256, 3) void k_moe_b_grouped(MoeBGroupArgs a) {
         word_masks(wv[r].z, mk[r] + 8); word_masks(wv[r].w, mk[r] + 12);
       }
     }
+    // The sums of pair j are parked on lanes 8j and 8j + 1 (gate and up of the wave's two rows), and the SwiGLU of
+    // the whole tile is formed once, sixteen lanes at a time: per pair it would cost every lane of the wave two
+    // evaluations of the exact sigmoid, a quarter of the kernel's instructions.
+    float G = 0.0f, U = 0.0f;
     for (int j = 0; j < mc; ++j) {
       const uint4* src = xs + (j * 64 + lane) * 5;
       uint32_t xp[16];
@@ -952,12 +970,17 @@ __global__ __launch_bounds__(256, 3) void k_moe_b_grouped(MoeBGroupArgs a) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) { const uint4 v = src[q]; xp[4 * q] = v.x; xp[4 * q + 1] = v.y; xp[4 * q + 2] = v.z; xp[4 * q + 3] = v.w; }
       { const uint4 v = src[4]; sx[0] = __uint_as_float(v.x); sx[1] = __uint_as_float(v.y); sx[2] = __uint_as_float(v.z); sx[3] = __uint_as_float(v.w); }
-      float o[4];
+      float o[4];                                          // rows 0..3 in the lower quad of every eight lanes
       quad_values(tree_sum4(quad_term_masked(mk[0], sb[0], xp, sx), quad_term_masked(mk[1], sb[1], xp, sx),
                             quad_term_masked(mk[2], sb[2], xp, sx), quad_term_masked(mk[3], sb[3], xp, sx), lane), o);
-      if (lane == 0)
-        *reinterpret_cast<uint32_t*>(a.act + (size_t)s_pair[j] * 512 + i0) =
-            pack2(swiglu16(f16r(o[0]), f16r(o[2])), swiglu16(f16r(o[1]), f16r(o[3])));
+      const bool mine = (lane >> 3) == j;
+      G = mine ? ((lane & 1) ? o[1] : o[0]) : G;
+      U = mine ? ((lane & 1) ? o[3] : o[2]) : U;
+    }
+    const float y = swiglu16(f16r(G), f16r(U));
+    if ((lane & 7) < 2 && (lane >> 3) < mc) {
+      const int p = s_pair[lane >> 3];
+      (shared ? a.sh_act + (size_t)(p >> 3) * 512 : a.act + (size_t)p * 512)[i0 + (lane & 1)] = f2h(y);
     }
   }
 }
@@ -1061,6 +1084,108 @@ __global__ __launch_bounds__(256) void k_moe_c(MoeCArgs a) {
   }
   const float s = sigmoid16(h2f(a.sgate[m]));
   if (li == 0) a.out[(size_t)m * H + n] = f2h(f16r(acc + f16r(s * sy)));
+}
+
+// Stage C by expert (steps of many rows): the down-projections of the pairs that chose expert e, with e's rows
+// fetched and unpacked into masks once per step instead of once per pair (reference: the grouped family
+// moe_count / moe_csr / gqmm4_grouped, SeedlessMetalForward.swift:3116-3556).  Grid (64, ceil(M / 64) + E): the shared
+// expert's rows in segments of 64, then the experts.  A workgroup holds 32 output rows of its expert, two per group
+// of 16 lanes (K = 512: a lane owns 32 activations), and walks the list in tiles of MOEC_MT pairs whose activation
+// rows are parked in LDS with their word sums.  Same arithmetic per (pair, output row) as k_moe_c:
+// d = half(tree_sum<16>(quad term)).  The results go out by pair (routed) or by row (shared);
+// k_moe_combine_rows adds them up in routing order.
+struct MoeCGroupArgs {
+  const uint16_t* act;         // [M, 8, 512]
+  const uint16_t* sh_act;      // [M, 512]
+  const uint32_t *d_w, *d_sb;  // [E*2048, 512]
+  const uint32_t *shd_w, *shd_sb;   // [2048, 512]
+  const uint16_t* lists;       // [E, GROUP_CAP] pair indices row*8 + slot
+  const int32_t* counts;       // [E]
+  const int32_t* order;        // [E] experts by falling count
+  uint16_t* d;                 // [M*8, 2048] routed down results by pair
+  uint16_t* sy;                // [M, 2048] shared down results by row
+  int M, E;
+};
+constexpr int MOEC_MT = 16;
+__global__ __launch_bounds__(256, 3) void k_moe_c_grouped(MoeCGroupArgs a) {
+  constexpr int XP = 20;                                  // words per lane slot: 16 + 4 pad
+  constexpr int PIECES = MOEC_MT * 64 / 256;              // 16-byte pieces of a tile per thread
+  __shared__ __align__(16) uint32_t s_x[MOEC_MT * 16 * XP];
+  __shared__ __align__(16) float s_sx[MOEC_MT * 16 * 4];
+  __shared__ int s_dst[MOEC_MT];
+  // blockIdx.y < S: segment of 64 rows of the shared expert (first, and cut up: as one list of M rows it would run
+  // thirty times longer than an expert's and end the launch with 64 workgroups); then the experts by falling count
+  const int S = (a.M + 63) / 64;
+  const bool shared = (int)blockIdx.y < S;
+  const int e = shared ? 0 : a.order[blockIdx.y - S];
+  const int row0 = shared ? 64 * blockIdx.y : 0;
+  const int cnt = shared ? min(64, a.M - row0) : min(a.counts[e], GROUP_CAP);
+  if (cnt == 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int sub = lane >> 4, li = lane & 15;
+  const int n0 = blockIdx.x * 32 + (wave * 4 + sub) * 2;  // this 16-lane group's two output rows
+  uint4 wv[2];
+  uint32_t sb[2];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const size_t row = (shared ? 0 : (size_t)e * 2048) + n0 + r;
+    wv[r] = ld16((shared ? a.shd_w : a.d_w) + row * 64 + 4 * li);
+    sb[r] = (shared ? a.shd_sb : a.d_sb)[row * 8 + (li >> 1)];
+  }
+  // a tile's pieces travel through registers one tile ahead (pair j = piece / 64, lane slot l, quarter q; pairs beyond
+  // the list repeat its last one and are not used)
+  uint4 px[PIECES];
+  int pp[PIECES];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int c = tid + 256 * i, j = min(t0 + (c >> 6), cnt - 1), l = (c >> 2) & 15, q = c & 3;
+      pp[i] = shared ? row0 + j : (int)a.lists[(size_t)e * GROUP_CAP + j];
+      px[i] = ld16((shared ? a.sh_act : a.act) + (size_t)pp[i] * 512 + 32 * l + 8 * q);
+    }
+  };
+  fetch(0);
+  h2_t mk[2][16];
+  for (int t0 = 0; t0 < cnt; t0 += MOEC_MT) {
+    const int mc = min(MOEC_MT, cnt - t0);
+    if (t0) __syncthreads();                             // the previous tile has been read
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int c = tid + 256 * i, j = c >> 6, l = (c >> 2) & 15, q = c & 3;
+      if ((c & 63) == 0) s_dst[j] = pp[i];
+      st16(&s_x[(j * 16 + l) * XP + 4 * q], px[i]);
+    }
+    __syncthreads();
+    if (t0 + MOEC_MT < cnt) fetch(t0 + MOEC_MT);
+    if (tid < mc * 16) {
+      float x[32], sx[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) unpack8(ld16(&s_x[tid * XP + 4 * q]), x + 8 * q);
+      word_sums(x, sx);
+      *reinterpret_cast<float4*>(&s_sx[tid * 4]) = make_float4(sx[0], sx[1], sx[2], sx[3]);
+    }
+    if (t0 == 0) {
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        word_masks(wv[r].x, mk[r]); word_masks(wv[r].y, mk[r] + 4);
+        word_masks(wv[r].z, mk[r] + 8); word_masks(wv[r].w, mk[r] + 12);
+      }
+    }
+    __syncthreads();
+    for (int j = 0; j < mc; ++j) {
+      uint32_t xp[16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) { const uint4 v = ld16(&s_x[(j * 16 + li) * XP + 4 * q]); xp[4 * q] = v.x; xp[4 * q + 1] = v.y; xp[4 * q + 2] = v.z; xp[4 * q + 3] = v.w; }
+      const float4 s4 = *reinterpret_cast<const float4*>(&s_sx[(j * 16 + li) * 4]);
+      const float sx[4] = {s4.x, s4.y, s4.z, s4.w};
+      const float d0 = tree_sum<16>(quad_term_masked(mk[0], sb[0], xp, sx));
+      const float d1 = tree_sum<16>(quad_term_masked(mk[1], sb[1], xp, sx));
+      if (li == 0) {
+        uint16_t* dst = (shared ? a.sy : a.d) + (size_t)s_dst[j] * H + n0;
+        *reinterpret_cast<uint32_t*>(dst) = pack2(d0, d1);
+      }
+    }
+  }
 }
 
 // -------------------------------------------------------------------------------------------------
