@@ -856,8 +856,15 @@ __global__ __launch_bounds__(1024) void k_group_pairs(const int32_t* __restrict_
   static_assert(SL_MAX_EXPERTS * 4 == 1024, "four lanes rank one expert");
   if (threadIdx.x < SL_MAX_EXPERTS) s_cnt[threadIdx.x] = 0;
   __syncthreads();
-  for (int p = threadIdx.x; p < M * 8; p += 1024) {
-    const int e = inds[p];
+  // a thread's pairs (M <= GROUP_CAP: at most 16) are all requested before the first of them is counted: the walk
+  // is one round trip to memory instead of one per pair
+  static_assert(GROUP_CAP * 8 == 16 * 1024, "sixteen pairs per thread at most");
+  int ev[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) { const int p = threadIdx.x + 1024 * i; ev[i] = p < M * 8 ? inds[p] : -1; }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int p = threadIdx.x + 1024 * i, e = ev[i];
     if (e >= 0 && e < E) {
       const int pos = atomicAdd(&s_cnt[e], 1);
       if (pos < GROUP_CAP) lists[e * GROUP_CAP + pos] = (uint16_t)p;

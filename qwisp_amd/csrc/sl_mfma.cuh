@@ -280,7 +280,7 @@ struct RouterMmArgs {
   uint16_t* sgate;       // [M]
 };
 __global__ __launch_bounds__(256) void k_router_mfma(RouterMmArgs a) {
-  constexpr int G = 2, XS = 64 * G + 8, K = 2048;
+  constexpr int G = 4, XS = 64 * G + 8, K = 2048;        // 256 k per barrier: the launch is short of workgroups, so a chunk's round trips show
   __shared__ __align__(16) uint16_t xs[2][32 * XS];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, hh = lane >> 5;
