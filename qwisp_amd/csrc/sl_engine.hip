@@ -312,6 +312,7 @@ void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   launch_qmm4_mfma(QmmArgs{e->sh_act, SL_MOE_I, L.sh_down.w, L.sh_down.sb, M, H, SL_MOE_I, e->hy_sy, H}, e->stream);
   hipLaunchKernelGGL(k_moe_combine_rows, dim3(H / 256, M), dim3(256), 0, e->stream, e->hy_d, L.route_scores, e->sgate, e->hy_sy, e->moe_out);
 }
+constexpr int MOE_PROLOGUE_MAX_ROWS = 8;  // up to here stage A's waves do residual + norm themselves
 constexpr int MOE_GROUP_MIN_ROWS = 128;   // below, most experts are chosen by one row and the extra launches cost more
 void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   MoeAArgs a{};
@@ -320,7 +321,10 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   a.router_w = L.router_w; a.sgate_w = L.sgate_w; a.g8_w = L.gate8_w; a.g8_sb = L.gate8_sb; a.E = e->n_experts;
   a.sh_act = e->sh_act; a.rlogits = e->rlogits; a.sgate = e->sgate;
   const int router_blocks = (e->n_experts + 1 + 15) / 16;
-  if (M >= 2) {                                         // residual + norm once per row instead of once per wave
+  // residual + norm once per row (k_final_rows) instead of once per wave of stage A; for a few rows (a verify step)
+  // the waves' own prologue costs less than the launch
+  const bool rows_first = M > MOE_PROLOGUE_MAX_ROWS;
+  if (rows_first) {
     HiddenArgs hs = ha;
     hs.xs_out = e->xsum;                                // and the row's word sums for the routed experts' dots
     hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hs);
@@ -332,7 +336,7 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, e->n_experts, L.route_inds, L.route_scores);
   MoeBArgs b{};
   b.xn = e->xn; b.g_w = L.sw_gate.w; b.g_sb = L.sw_gate.sb; b.u_w = L.sw_up.w; b.u_sb = L.sw_up.sb;
-  b.act = e->act; b.inds = L.route_inds; b.xsum = M >= 2 ? e->xsum : nullptr;
+  b.act = e->act; b.inds = L.route_inds; b.xsum = rows_first ? e->xsum : nullptr;
   if (grouped) {                                        // weights of an expert fetched once for all rows that chose it
     hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, e->n_experts, e->hy_lists, e->hy_counts, e->hy_counts + SL_MAX_EXPERTS);
     MoeBGroupArgs g{e->xn, b.g_w, b.g_sb, b.u_w, b.u_sb, e->act, e->hy_lists, e->hy_counts, e->xsum, e->hy_counts + SL_MAX_EXPERTS,
