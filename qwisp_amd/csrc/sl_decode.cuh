@@ -112,7 +112,7 @@ struct Lds {
   int inds[8];
   float scores[8];
   float dbuf[2 * 9 * 4];
-  int pf[4];                                // poll verdict slots (three in rotation) and the give-up flag
+  int pf[4];                                // poll outcome slots (three in rotation) and the give-up flag
   uint32_t pub[64];                         // a stage's tagged outputs, gathered for the publishing wave
   float sq[8 * 256];                        // attention: scaled queries of one kv group
   float knew[256], vnew[256];

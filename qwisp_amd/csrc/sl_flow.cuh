@@ -120,7 +120,7 @@ SL_DEV void fstamp(int layer, int stage, int kind, bool who) {
     if (who && layer < STAMP_LAYERS) g_stamps[(layer * 8 + stage) * STAMP_KINDS + kind] = (uint32_t)wall_clock64();
   }
 }
-// One polling round's verdict for the whole workgroup: 1 = all tags present, 0 = retry, -1 = give up (spin
+// One polling round's outcome for the whole workgroup: 1 = all tags present, 0 = retry, -1 = give up (spin
 // limit reached here, or another workgroup raised the abort word).  One barrier per round: a wave with a
 // missing tag marks slot (round % 3) in LDS before the barrier, everybody reads it after, and thread 0 then
 // clears the slot of the round before (nobody can still be reading that one), so a successful round leaves
