@@ -184,6 +184,17 @@ SL_DEV float tree_max(float v) {
   return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 #endif
 }
+// Largest of an unsigned value over the 64 lanes, in every lane (the tree of tree_max: no trip through scalar registers).
+SL_DEV uint32_t wave_max_u32(uint32_t v) {
+  v = max(v, dpp_u<DPP_XOR1>(v));
+  v = max(v, dpp_u<DPP_XOR2>(v));
+  v = max(v, dpp_u<DPP_HALF_MIRROR>(v));
+  v = max(v, dpp_u<DPP_MIRROR>(v));
+  const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  v = max(r[0], r[1]);
+  const auto q = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return max(q[0], q[1]);
+}
 // Value of the previous lane (lanes 0, 16, 32, 48 get 0): for left-to-right chains inside a 16-lane row.
 SL_DEV float prev_lane(float v) { return dpp_f<DPP_SHR1>(v); }
 

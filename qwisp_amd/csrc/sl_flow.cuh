@@ -1299,21 +1299,16 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
         }, uni(P.bar) + 32)) return false;
     fstamp<ST>(li, FS_B, 1, tid == 0);
   }
-  // Wave 0 picks the 8 largest keys in order (max, remove, repeat; the wave-wide max is a DPP reduction plus
-  // one lane per row); wave 1 forms the softmax sums meanwhile.
+  // Wave 0 picks the 8 largest keys in order (max, remove, repeat); wave 1 forms the softmax sums meanwhile.
   if (wave == 0) {
     const uint4 k4 = *reinterpret_cast<const uint4*>(&key[4 * lane]);
     uint32_t k[4] = {k4.x, k4.y, k4.z, k4.w};
     const int E = uni(P.E);
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      uint32_t m = max(max(k[0], k[1]), max(k[2], k[3]));
-      m = max(m, dpp_u<DPP_XOR1>(m));
-      m = max(m, dpp_u<DPP_XOR2>(m));
-      m = max(m, dpp_u<DPP_HALF_MIRROR>(m));
-      m = max(m, dpp_u<DPP_MIRROR>(m));
-      const uint32_t M = max(max((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
-                             max((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
+      // (the wave-wide maximum stays in vector registers: a value read out to a scalar register takes tens of clocks
+      // to become usable, eight times in a row)
+      const uint32_t M = wave_max_u32(max(max(k[0], k[1]), max(k[2], k[3])));
 #pragma unroll
       for (int i = 0; i < 4; ++i) k[i] = (k[i] == M) ? 0u : k[i];
       if (lane == 0) L.inds[r] = min(255 - (int)(M & 255u), E - 1);
