@@ -121,6 +121,7 @@ struct sl_engine {
   // scratch
   uint16_t *hA = nullptr, *hB = nullptr, *proj = nullptr, *ycore = nullptr, *qrot = nullptr, *mix = nullptr, *xn = nullptr;
   float* xsum = nullptr;           // [max_m, 256] word sums of the rows in xn (steps of two or more rows)
+  float* ysum = nullptr;           // [max_m, 512] word sums of the rows in ycore (gated mixer outputs) for the exact K = 4096 projection
   uint16_t *rlogits = nullptr, *sgate = nullptr, *sh_act = nullptr, *act = nullptr, *moe_out = nullptr, *normed = nullptr;
   uint16_t *logits = nullptr, *rows_out = nullptr;
   float *pm = nullptr, *pl = nullptr, *po = nullptr, *cand_v = nullptr;
@@ -420,9 +421,9 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
     launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.out_proj.w, L.out_proj.sb, M, H, 4096, e->mix, H}, e->stream);
   } else if (M >= 2) {
     // the gated norm once per row, then the row-tiled projection (same bits as the fused kernel below)
-    hipLaunchKernelGGL(k_gdn_gate_rows, dim3(SL_GDN_HV, M), dim3(64), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32);
+    hipLaunchKernelGGL(k_gdn_gate_rows, dim3(SL_GDN_HV, M), dim3(64), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32, e->ysum);
     hipLaunchKernelGGL((k_qmv_tile<2, 2, 4, false>), dim3(H / 8, (M + 3) / 4), dim3(256), 0, e->stream, HiddenArgs{}, e->ycore, 4096,
-                       L.out_proj.w, L.out_proj.sb, H, e->mix, H, M);
+                       L.out_proj.w, L.out_proj.sb, H, e->mix, H, M, (float*)nullptr, (int32_t*)nullptr, e->ysum);
   } else {
     hipLaunchKernelGGL(k_qmv_gdn_out<2>, dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32,
                        L.out_proj.w, L.out_proj.sb, H, e->mix);
@@ -465,12 +466,13 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
   SdpaMergeArgs g{};
   g.pm = e->pm; g.pl = e->pl; g.po = e->po; g.proj = e->proj; g.st = e->st; g.maxTiles = e->max_tiles; g.gated = e->ycore; g.lanes = lanes;
   g.group = tiles_per_part;
+  g.gsum = mm ? nullptr : e->ysum;                       // the exact merge leaves the gated rows' word sums for the projection
   if (mm && lanes) hipLaunchKernelGGL(k_sdpa_merge_par<16>, dim3(SL_ATT_HEADS, M), dim3(1024), 0, e->stream, g);
   else if (mm) hipLaunchKernelGGL(k_sdpa_merge_par<4>, dim3(SL_ATT_HEADS, M), dim3(256), 0, e->stream, g);
   else hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
   if (mm && !(lanes && M < MM_OUT_ROWS)) launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.o_proj.w, L.o_proj.sb, M, H, 4096, e->mix, H}, e->stream);
   else if (M >= 2) hipLaunchKernelGGL((k_qmv_tile<2, 2, 4, false>), dim3(H / 8, (M + 3) / 4), dim3(256), 0, e->stream, HiddenArgs{}, e->ycore, 4096,
-                                      L.o_proj.w, L.o_proj.sb, H, e->mix, H, M);
+                                      L.o_proj.w, L.o_proj.sb, H, e->mix, H, M, (float*)nullptr, (int32_t*)nullptr, mm ? (float*)nullptr : e->ysum);
   else hipLaunchKernelGGL((k_qmv_plain<2, 2>), dim3(H / 8, M), dim3(256), 0, e->stream, e->ycore, 4096, L.o_proj.w, L.o_proj.sb,
                           H, e->mix, H);
 }
@@ -724,7 +726,7 @@ int alloc_runtime(sl_engine* e) {
   e->hA = dalloc<uint16_t>(e, MH, true); e->hB = dalloc<uint16_t>(e, MH, true);
   e->proj = dalloc<uint16_t>(e, (size_t)max_m * PROJ_STRIDE, true);
   e->ycore = dalloc<uint16_t>(e, (size_t)max_m * 4096, true);
-  e->mix = dalloc<uint16_t>(e, MH, true); e->xn = dalloc<uint16_t>(e, MH, true); e->xsum = dalloc<float>(e, (size_t)max_m * 256, true);
+  e->mix = dalloc<uint16_t>(e, MH, true); e->xn = dalloc<uint16_t>(e, MH, true); e->xsum = dalloc<float>(e, (size_t)max_m * 256, true); e->ysum = dalloc<float>(e, (size_t)max_m * 512, true);
   if (max_m >= MOE_GROUP_MIN_ROWS) {               // exact steps of many rows run the experts' down stage by expert: results by pair, then the combine
     const size_t rows = (size_t)(max_m < GROUP_CAP ? max_m : GROUP_CAP);
     e->hy_d = dalloc<uint16_t>(e, rows * 8 * H); e->hy_sy = dalloc<uint16_t>(e, rows * H);
@@ -742,7 +744,7 @@ int alloc_runtime(sl_engine* e) {
   e->tok_in = dalloc<int32_t>(e, max_m, true);
   e->tok_out = dalloc<int32_t>(e, max_m > MAX_CHAIN ? max_m : MAX_CHAIN, true);
   e->st = dalloc<int32_t>(e, 1 + d->n_layers, true);
-  if (!e->hA || !e->hB || !e->proj || !e->ycore || !e->mix || !e->xn || !e->xsum || !e->rlogits || !e->sgate || !e->sh_act || !e->act || !e->hy_lists || !e->hy_counts ||
+  if (!e->hA || !e->hB || !e->proj || !e->ycore || !e->mix || !e->xn || !e->xsum || !e->ysum || !e->rlogits || !e->sgate || !e->sh_act || !e->act || !e->hy_lists || !e->hy_counts ||
       !e->moe_out || !e->normed || !e->rows_out || !e->tok_in || !e->tok_out || !e->st) return SL_ERR_DEVICE;
   if (has_head) {
     int ncu = 0;

@@ -232,11 +232,11 @@ __global__ __launch_bounds__(HIDDEN ? 512 : 256, HIDDEN ? 2 : 3) void k_qmv_tile
 #pragma unroll
     for (int b = 0; b < NBLK; ++b) {
       uint4* dst = xs + ((m * NBLK + b) * 64 + lane) * 5;
-      if (!HIDDEN && NBLK == 1 && xsums) {                 // the stored halves are the packed pairs; their sums came with the row
-        const uint16_t* src = xin + (size_t)(m0 + m) * x_stride + 32 * lane;
+      if (!HIDDEN && xsums) {                              // the stored halves are the packed pairs; their sums came with the row
+        const uint16_t* src = xin + (size_t)(m0 + m) * x_stride + b * 2048 + 32 * lane;
 #pragma unroll
         for (int j = 0; j < 4; ++j) dst[j] = ld16(src + 8 * j);
-        dst[4] = ld16(xsums + (size_t)(m0 + m) * 256 + 4 * lane);
+        dst[4] = ld16(xsums + (size_t)(m0 + m) * (256 * NBLK) + b * 256 + 4 * lane);
         continue;
       }
       float x[32], sx[4];
@@ -697,8 +697,10 @@ __global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict_
 // gated[m, hv, :] = half(silu(z) * norm(y)) in place of y.  One wave per (value head, row); lane l owns the pair
 // 2l, 2l+1, so the sum of squares is the same balanced tree as in the fused kernel above.
 // -------------------------------------------------------------------------------------------------
+// `ysum` (or null) receives the row's word sums (left-to-right sums of each run of 8 gated values, [M, 512]) for the
+// projection that follows: a run sits on four neighbouring lanes, the sum passes along them.
 __global__ __launch_bounds__(64) void k_gdn_gate_rows(uint16_t* __restrict__ ycore, const uint16_t* __restrict__ proj,
-                                                      const float* __restrict__ norm_w, int norm_f32) {
+                                                      const float* __restrict__ norm_w, int norm_f32, float* __restrict__ ysum = nullptr) {
   const int hv = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;
   uint16_t* yp = ycore + (size_t)m * 4096 + hv * 128 + 2 * lane;
   const uint32_t yw = *reinterpret_cast<const uint32_t*>(yp);
@@ -709,7 +711,18 @@ __global__ __launch_bounds__(64) void k_gdn_gate_rows(uint16_t* __restrict__ yco
   const float w0 = norm_w[2 * lane], w1 = norm_w[2 * lane + 1];
   const float n0 = norm_f32 ? w0 * (y0 * inv) : f16r(w0 * f16r(y0 * inv));
   const float n1 = norm_f32 ? w1 * (y1 * inv) : f16r(w1 * f16r(y1 * inv));
-  *reinterpret_cast<uint32_t*>(yp) = pack2(f16r((z0 * sigmoid32(z0)) * n0), f16r((z1 * sigmoid32(z1)) * n1));
+  const float o0 = f16r((z0 * sigmoid32(z0)) * n0), o1 = f16r((z1 * sigmoid32(z1)) * n1);
+  *reinterpret_cast<uint32_t*>(yp) = pack2(o0, o1);
+  if (ysum) {
+    const int q = lane & 3;
+    float sw = (0.0f + o0) + o1;
+#pragma unroll
+    for (int r = 1; r < 4; ++r) {
+      const float v = prev_lane(sw);
+      if (q == r) sw = (v + o0) + o1;
+    }
+    if (q == 3) ysum[(size_t)m * 512 + hv * 16 + (lane >> 2)] = sw;
+  }
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -1395,6 +1408,7 @@ struct SdpaMergeArgs {
   const int32_t* st;
   int maxTiles;
   uint16_t* gated;             // [M, 4096]
+  float* gsum;                 // [M, 512] word sums of the gated rows for the projection that follows (k_sdpa_merge), or null
   const LaneRef* lanes;
   int group = 0;               // > 1: one partial per `group` key tiles at index tile / group (k_sdpa_merge_par only)
 };
@@ -1432,6 +1446,11 @@ __global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) r[i] = f16r(f16r(O[i] / L) * sigmoid16(gt[i]));
   *reinterpret_cast<uint2*>(a.gated + (size_t)m * 4096 + h * 256 + 4 * lane) = make_uint2(pack2(r[0], r[1]), pack2(r[2], r[3]));
+  if (a.gsum) {                                          // a run of 8 values sits on two neighbouring lanes
+    const float v = prev_lane(((0.0f + r[0]) + r[1]) + r[2] + r[3]);
+    const float sw = (lane & 1) ? (((v + r[0]) + r[1]) + r[2]) + r[3] : 0.0f;
+    if (lane & 1) a.gsum[(size_t)m * 512 + h * 32 + (lane >> 1)] = sw;
+  }
 }
 
 // -------------------------------------------------------------------------------------------------
