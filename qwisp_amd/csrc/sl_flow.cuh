@@ -213,24 +213,22 @@ constexpr int PAIR_WAVE0 = 160 * DEC_WAVES;      // first wave of the shared gat
                  const int wg = fresh_s(blockIdx.x), G = fresh_s(gridDim.x), NW = G * DEC_WAVES, gw = wg * DEC_WAVES + wave; \
                  (void)tid; (void)lane; (void)wave; (void)wg; (void)G; (void)NW; (void)gw
 
-// Waves 0..7 poll a 2048-long tagged vector (4 words per thread); every thread then takes the pair it owns.
+// Every thread polls the two tagged words of the pair it owns of a 2048-long vector.
 template <bool ST>
 SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, float& r0, float& r1, int sl, int ss) {
   const int tid = fresh_v(threadIdx.x);
-  uint32_t* rs = reinterpret_cast<uint32_t*>(g_L.part);       // [1024] packed pairs
   const rsrc_t rr = co_rsrc(vec);
   bool ok = false;
-  if (!flow_poll(tid < 512, [&]() {
+  uint2 b = make_uint2(0u, 0u);
+  if (!flow_poll(true, [&]() {
         if (!ok) {
-          const uint4 b = ldw4(rr, 4 * tid);
-          ok = tag_ok(b.x, tag) && tag_ok(b.y, tag) && tag_ok(b.z, tag) && tag_ok(b.w, tag);
-          *reinterpret_cast<uint2*>(&rs[2 * tid]) = make_uint2((b.x & 0xffffu) | (b.y << 16), (b.z & 0xffffu) | (b.w << 16));
+          b = ldw2(rr, 2 * tid);
+          ok = tag_ok(b.x, tag) && tag_ok(b.y, tag);
         }
         return ok;
       }, uni(P.bar) + 32)) return false;
   fstamp<ST>(sl, ss, 1, tid == 0);
-  const uint32_t w = rs[tid];
-  r0 = lo_h(w); r1 = hi_h(w);
+  r0 = lo_h(b.x); r1 = lo_h(b.y);
   return true;
 }
 
