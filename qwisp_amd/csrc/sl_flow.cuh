@@ -1099,47 +1099,31 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     if (lin) store_hist(Y, li, gh);
     return true;
   }
-  // every thread prepares 4 consecutive elements of the 4096-long activation; waves 0..7 fetch them, for
-  // themselves and for the wave 8 above (handed over through LDS)
+  // every thread prepares 4 consecutive elements of the 4096-long activation and polls them itself
   const int e0 = 256 * wave + 4 * lane;
   float out[4], sz[4] = {0.0f, 0.0f, 0.0f, 0.0f};            // sz: z * sigmoid(z) of the gate values
   {
-    uint4* ystage = reinterpret_cast<uint4*>(g_vt);            // [512] y chunks, [512] silu(z) quads of waves 8..15
     const uint32_t ty = lin ? tcore : tmerge;
     const rsrc_t ry = co_rsrc(uni(F.tycore)), rz = co_rsrc(uni(F.tproj));
-    uint4 a = make_uint4(0, 0, 0, 0), b = make_uint4(0, 0, 0, 0);
-    bool zdone = false, y1done = false, y2done = false;   // what has arrived is not fetched again
-    if (!flow_poll(wave < 8, [&]() {
-          if (!y1done) { a = ldw4(ry, e0); y1done = tag_ok(a.x, ty) && tag_ok(a.y, ty) && tag_ok(a.z, ty) && tag_ok(a.w, ty); }
-          if (!y2done) {
-            const uint4 a2 = ldw4(ry, e0 + 2048);
-            y2done = tag_ok(a2.x, ty) && tag_ok(a2.y, ty) && tag_ok(a2.z, ty) && tag_ok(a2.w, ty);
-            ystage[tid] = a2;
-          }
-          bool ok = y1done && y2done;
+    uint4 a = make_uint4(0, 0, 0, 0);
+    bool zdone = false, ydone = false;                    // what has arrived is not fetched again
+    if (!flow_poll(true, [&]() {
+          if (!ydone) { a = ldw4(ry, e0); ydone = tag_ok(a.x, ty) && tag_ok(a.y, ty) && tag_ok(a.z, ty) && tag_ok(a.w, ty); }
+          bool ok = ydone;
           if (lin && !zdone) {                      // the gate values were published a stage earlier: fetched once
-            b = ldw4(rz, 8192 + e0);
-            const uint4 b2 = ldw4(rz, 8192 + e0 + 2048);
-            zdone = tag_ok(b.x, tin) && tag_ok(b.y, tin) && tag_ok(b.z, tin) && tag_ok(b.w, tin) &&
-                    tag_ok(b2.x, tin) && tag_ok(b2.y, tin) && tag_ok(b2.z, tin) && tag_ok(b2.w, tin);
+            const uint4 b = ldw4(rz, 8192 + e0);
+            zdone = tag_ok(b.x, tin) && tag_ok(b.y, tin) && tag_ok(b.z, tin) && tag_ok(b.w, tin);
             ok = ok && zdone;
             if (zdone) {
               // z * sigmoid(z) does not need the core output: formed while that is still on its way
               const float z1[4] = {lo_h(b.x), lo_h(b.y), lo_h(b.z), lo_h(b.w)};
-              const float z2[4] = {lo_h(b2.x), lo_h(b2.y), lo_h(b2.z), lo_h(b2.w)};
-              float s2[4];
 #pragma unroll
-              for (int i = 0; i < 4; ++i) { sz[i] = z1[i] * sigmoid32(z1[i]); s2[i] = z2[i] * sigmoid32(z2[i]); }
-              ystage[512 + tid] = make_uint4(__float_as_uint(s2[0]), __float_as_uint(s2[1]), __float_as_uint(s2[2]), __float_as_uint(s2[3]));
+              for (int i = 0; i < 4; ++i) sz[i] = z1[i] * sigmoid32(z1[i]);
             }
           }
           return ok;
         }, uni(P.bar) + 32)) return false;
     fstamp<ST>(li, FS_OUT, 1, tid == 0);
-    if (wave >= 8) {
-      a = ystage[tid - 512];
-      if (lin) { b = ystage[tid]; sz[0] = __uint_as_float(b.x); sz[1] = __uint_as_float(b.y); sz[2] = __uint_as_float(b.z); sz[3] = __uint_as_float(b.w); }
-    }
     if (lin) store_hist(Y, li, gh);
     out[0] = lo_h(a.x); out[1] = lo_h(a.y); out[2] = lo_h(a.z); out[3] = lo_h(a.w);
   }
