@@ -949,19 +949,23 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
           }
           if (mdone && gdone && have == (1u << cnt0) - 1u) break;
           if (++spins > uni(F.spin_limit)) { fail = 1; break; }
-          __builtin_amdgcn_s_sleep(1);
         }
         Mx = fmaxf(Mx, tree_max<64>(mine ? __uint_as_float(m0.x) : NEG));
       }
       if (!fail) {                                          // the first batch is already here
         float fl = 0.0f, pl = 0.0f;
         if (lane < nt) { fl = exp_c(__uint_as_float(m0.x) - Mx); pl = __uint_as_float(m0.y); }
+        // the tiles' scales and sums as scalars, read out in batches ahead of their use (a scalar written by the
+        // vector unit takes tens of clocks to become readable)
+        static_assert(MB <= 16, "two batches of eight lane reads");
+        float f[16], l[16];
+        lanes8(fl, 0, reinterpret_cast<float(&)[8]>(f[0])); lanes8(fl, 8, reinterpret_cast<float(&)[8]>(f[8]));
+        lanes8(pl, 0, reinterpret_cast<float(&)[8]>(l[0])); lanes8(pl, 8, reinterpret_cast<float(&)[8]>(l[8]));
 #pragma unroll
         for (int u = 0; u < MB; ++u) {
           if (u < nt) {
-            const float f = row_lane_f(fl, u), l = row_lane_f(pl, u);
-            Ls = fmaf(l, f, Ls);
-            O0 = fmaf(__uint_as_float(a[u].x), f, O0); O1 = fmaf(__uint_as_float(a[u].y), f, O1);
+            Ls = fmaf(l[u], f[u], Ls);
+            O0 = fmaf(__uint_as_float(a[u].x), f[u], O0); O1 = fmaf(__uint_as_float(a[u].y), f[u], O1);
           }
         }
       }
