@@ -900,6 +900,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     float Mx = NEG, Ls = 0.0f, O0 = 0.0f, O1 = 0.0f;
     uint4 m0 = make_uint4(0, 0, 0, 0);
     uint2 g2 = make_uint2(0u, 0u);
+    float sg0 = 0.0f, sg1 = 0.0f;                          // sigmoids of the lane's two gate values
     if (wave == 0) {
       uint4 a[MB];
       // maxima of the tiles beyond the first 64, eight blocks per round trip: they are published after the first pass
@@ -939,6 +940,8 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
           if (!gdone) {
             if (act) g2 = ldw2(rp, h * 512 + 256 + 2 * chunk);
             gdone = __all((!act || (tag_ok(g2.x, tin) && tag_ok(g2.y, tin))) ? 1 : 0) != 0;
+            // the gate was published a stage earlier: its sigmoids are formed while the tiles are still on their way
+            if (gdone) { sg0 = sigmoid16(lo_h(g2.x)); sg1 = sigmoid16(lo_h(g2.y)); }
           }
 #pragma unroll
           for (int u = 0; u < MB; ++u) {
@@ -1093,8 +1096,8 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     }
     if (fail) st_co32(uni(P.bar) + 32, 1u);
     if (wave == 0 && !fail && act) {
-      const uint32_t r0 = tagged(f16r(f16r(O0 / Ls) * sigmoid16(lo_h(g2.x))), tmerge);
-      const uint32_t r1 = tagged(f16r(f16r(O1 / Ls) * sigmoid16(lo_h(g2.y))), tmerge);
+      const uint32_t r0 = tagged(f16r(f16r(O0 / Ls) * sg0), tmerge);
+      const uint32_t r1 = tagged(f16r(f16r(O1 / Ls) * sg1), tmerge);
       stw2(co_rsrc(uni(F.tycore)), h * 256 + 2 * chunk, r0, r1);
     }
     fstamp<ST>(li, FS_MERGE, 4, tid == 0);
