@@ -147,7 +147,7 @@ SL_DEV int flow_round(bool ok, unsigned& spins, unsigned* abort_word) {
 // round trip again and again (all-gather of 8 KB between 256 workgroups: 2.0 against 2.2 us per dependent round).
 // `attempt()` fetches what the lane still misses and returns whether the lane is complete; `polls` is uniform per
 // wave.  Bounded like flow_round: a wave that gives up raises the abort word, and false comes back to everybody.
-template <typename Attempt>
+template <bool MEET = true, typename Attempt>
 SL_DEV bool flow_poll(bool polls, Attempt attempt, unsigned* abort_word) {
   if (polls) {
     for (unsigned spins = 0;; ++spins) {
@@ -159,6 +159,7 @@ SL_DEV bool flow_poll(bool polls, Attempt attempt, unsigned* abort_word) {
       }
     }                                                   // (no back-off between attempts: a sleep of 64 clocks measured 0.3 % slower)
   }
+  if constexpr (!MEET) return true;                     // the caller's next barrier is the meeting point; it looks at the give-up flag there
   lds_barrier();
   return g_L.pf[3] == 0;
 }
@@ -1269,50 +1270,52 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   const DecodeP& P = F.d;
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
-  float* lg = L.part;                                   // [256] logits
   float* ex = L.part + 256;                             // [256] exp(logit - max)
-  uint32_t* key = reinterpret_cast<uint32_t*>(L.part + 512);   // [256] order keys
-  {
+  // Waves 0 and 1 each poll all the logits (four per lane, 1 KB) and go straight on: wave 0 picks the 8 largest keys
+  // in order (max, remove, repeat), wave 1 forms the softmax sums.  The workgroup meets once, when the indices are
+  // known (a hop of the logits through LDS and a barrier ahead of the routing measured 0.1 % slower).
+  if (wave < 2) {
     const uint32_t ta = flow_tag(base, li, FS_A);
     const rsrc_t rl = co_rsrc(uni(F.trlog));
     const int E = uni(P.E);
-    bool got = tid >= E;
-    if (tid < 256) { lg[tid] = NEG; key[tid] = 0; }
-    if (!flow_poll(wave < 4, [&]() {                 // up to 256 experts: threads 0..255
-          if (!got) {
-            const uint32_t w = ldw1(rl, tid);
-            got = tag_ok(w, ta);
-            if (got) { lg[tid] = lo_h(w); key[tid] = route_key(w, tid); }
-          }
-          return got;
-        }, uni(P.bar) + 32)) return false;
+    uint4 w4 = make_uint4(0u, 0u, 0u, 0u);
+    const bool mine = 4 * lane < E;                        // (words of experts beyond E are ignored)
+    flow_poll<false>(true, [&]() {
+      if (mine) w4 = ldw4(rl, 4 * lane);
+      const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ok = ok && (4 * lane + i >= E || tag_ok(w[i], ta));
+      return ok;
+    }, uni(P.bar) + 32);
     fstamp<ST>(li, FS_B, 1, tid == 0);
-  }
-  // Wave 0 picks the 8 largest keys in order (max, remove, repeat); wave 1 forms the softmax sums meanwhile.
-  if (wave == 0) {
-    const uint4 k4 = *reinterpret_cast<const uint4*>(&key[4 * lane]);
-    uint32_t k[4] = {k4.x, k4.y, k4.z, k4.w};
-    const int E = uni(P.E);
+    const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+    if (wave == 0) {
+      uint32_t k[4];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      // (the wave-wide maximum stays in vector registers: a value read out to a scalar register takes tens of clocks
-      // to become usable, eight times in a row)
-      const uint32_t M = wave_max_u32(max(max(k[0], k[1]), max(k[2], k[3])));
+      for (int i = 0; i < 4; ++i) k[i] = 4 * lane + i < E ? route_key(w[i], 4 * lane + i) : 0u;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) k[i] = (k[i] == M) ? 0u : k[i];
-      if (lane == 0) L.inds[r] = min(255 - (int)(M & 255u), E - 1);
+      for (int r = 0; r < 8; ++r) {
+        // (the wave-wide maximum stays in vector registers: a value read out to a scalar register takes tens of clocks
+        // to become usable, eight times in a row)
+        const uint32_t M = wave_max_u32(max(max(k[0], k[1]), max(k[2], k[3])));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) k[i] = (k[i] == M) ? 0u : k[i];
+        if (lane == 0) L.inds[r] = min(255 - (int)(M & 255u), E - 1);
+      }
+    } else {
+      float v[4], x4[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = 4 * lane + i < E ? lo_h(w[i]) : NEG;
+      const float mx = tree_max<64>(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { x4[i] = (4 * lane + i < E) ? exp_c(v[i] - mx) : 0.0f; ex[4 * lane + i] = x4[i]; }
+      const float Z = tree_sum<64>(((x4[0] + x4[1]) + x4[2]) + x4[3]);
+      if (lane == 0) L.gb[0] = Z;
     }
-  } else if (wave == 1) {
-    float v[4], x4[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = lg[4 * lane + i];
-    const float mx = tree_max<64>(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { x4[i] = (4 * lane + i < uni(P.E)) ? exp_c(v[i] - mx) : 0.0f; ex[4 * lane + i] = x4[i]; }
-    const float Z = tree_sum<64>(((x4[0] + x4[1]) + x4[2]) + x4[3]);
-    if (lane == 0) L.gb[0] = Z;
   }
   lds_barrier();
+  if (g_L.pf[3] != 0) return false;
   fstamp<ST>(li, FS_B, 2, tid == 0);
   // (the renormalised scores are only needed by the combine of the next stage and are formed there, off this
   // stage's path: exp values, sum and indices stay in LDS)
