@@ -371,6 +371,7 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
 // New conv-history samples of a thread's channel; written to memory by the next stage once its poll is over
 // (a store issued here would hold up that poll until it is acknowledged).
 struct GdnHist { uint32_t t12; uint32_t tnew; };
+constexpr int BETA_TID = 5 * 64, DECAY_TID = 6 * 64;
 template <bool ST>
 SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, GdnHist& gh) {
   FLOW_IDS;
@@ -393,8 +394,14 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
   if (tid < 128) ch = hk * 128 + tid;
   else if (tid < 256) ch = 2048 + hk * 128 + (tid - 128);
   else if (tid < 272) ch = 4096 + hv * 128 + dvb * 16 + (tid - 256);
-  else if (tid == 272) ch = 12288 + hv;       // beta logit
-  else if (tid == 273) ch = 12320 + hv;       // decay logit
+  // the two gate logits sit on the first lanes of waves 5 and 6, which have nothing else to do here: on wave 4, next
+  // to the value channels, the three branches ran one after the other and the decay's chain of exponentials and a
+  // logarithm (1 us) held the whole workgroup at the barrier
+  else if (tid == BETA_TID) ch = 12288 + hv;  // beta logit
+  else if (tid == DECAY_TID) ch = 12320 + hv; // decay logit
+  // the decay's constants of this head do not depend on the projection: fetched and exponentiated ahead of the wait
+  float decay_rate = 0.0f, dt_bias = 0.0f;
+  if (tid == DECAY_TID) { decay_rate = exp_c(uni(Y.a_log)[hv]); dt_bias = uni(Y.dt_bias)[hv]; }
   // history taps stay raw until the wait is over: converting them here would wait for the loads
   uint16_t traw[3] = {0, 0, 0};
   float cw[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -409,7 +416,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
     const uint32_t tin = flow_tag(base, li, FS_IN);
     const rsrc_t rp = co_rsrc(uni(F.tproj));
     bool got = ch < 0;
-    if (!flow_poll(wave < 5, [&]() {                 // channels sit on threads 0..273
+    if (!flow_poll(wave < 7, [&]() {                 // channels sit on threads 0..271 and on the two gate threads
           if (!got) { const uint32_t w = ldw1(rp, ch); got = tag_ok(w, tin); newest = lo_h(w); }
           return got;
         }, uni(P.bar) + 32)) return false;
@@ -423,10 +430,10 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
     acc = fmaf(newest, cw[3], acc);
     const float c = f16r(acc * sigmoid32(acc));
     if (tid < 128) L.q[tid] = c; else if (tid < 256) L.k[tid - 128] = c; else L.v[tid - 256] = c;
-  } else if (tid == 272) {
+  } else if (tid == BETA_TID) {
     L.gb[1] = sigmoid16(newest);
-  } else if (tid == 273) {
-    L.gb[0] = exp_c(-(exp_c(uni(Y.a_log)[hv]) * softplus_c(newest + uni(Y.dt_bias)[hv])));
+  } else if (tid == DECAY_TID) {
+    L.gb[0] = exp_c(-(decay_rate * softplus_c(newest + dt_bias)));
   }
   lds_barrier();
   if (wave < 2) {
