@@ -1414,6 +1414,9 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
         }, uni(P.bar) + 32)) return false;
     fstamp<ST>(li, FS_C, 1, tid == 0);
   }
+  // the shared expert's gate came with the poll: its sigmoid is formed by the publishing wave while the units run
+  float sgs = 0.0f;
+  if (wave == PUB_WAVE) sgs = sigmoid16(L.gb[1]);
 #pragma unroll
   for (int qq = 0; qq < 2; ++qq) {
     const int un = (wave - 6) * 2 + qq, ql = un / 9, slot = un % 9;
@@ -1442,8 +1445,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     float acc = 0.0f;
 #pragma unroll
     for (int k = 0; k < 8; ++k) acc = f16r(acc + f16r(L.dbuf[(ql * 9 + k) * 4 + sb4] * L.scores[k]));
-    const float s = sigmoid16(L.gb[1]);
-    stw1(co_rsrc(uni(F.tmoe)), quad * 4 + sb4, tagged(f16r(acc + f16r(s * L.dbuf[(ql * 9 + 8) * 4 + sb4])), flow_tag(base, li, FS_C)));
+    stw1(co_rsrc(uni(F.tmoe)), quad * 4 + sb4, tagged(f16r(acc + f16r(sgs * L.dbuf[(ql * 9 + 8) * 4 + sb4])), flow_tag(base, li, FS_C)));
   }
   fstamp<ST>(li, FS_C, 4, tid == PUB_WAVE * 64);
   lds_barrier();
