@@ -430,12 +430,12 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
     acc = fmaf(newest, cw[3], acc);
     const float c = f16r(acc * sigmoid32(acc));
     if (tid < 128) L.q[tid] = c; else if (tid < 256) L.k[tid - 128] = c; else L.v[tid - 256] = c;
-  } else if (tid == BETA_TID) {
-    L.gb[1] = sigmoid16(newest);
-  } else if (tid == DECAY_TID) {
-    L.gb[0] = exp_c(-(decay_rate * softplus_c(newest + dt_bias)));
   }
   lds_barrier();
+  // between the two barriers: waves 0 and 1 norm q and k, and the gate threads form beta and the decay meanwhile
+  // (neither is needed before the recurrence)
+  if (tid == BETA_TID) L.gb[1] = sigmoid16(newest);
+  else if (tid == DECAY_TID) L.gb[0] = exp_c(-(decay_rate * softplus_c(newest + dt_bias)));
   if (wave < 2) {
     float* buf = wave ? L.k : L.q;
     const float x0 = buf[2 * lane], x1 = buf[2 * lane + 1];
