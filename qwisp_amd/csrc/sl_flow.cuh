@@ -205,7 +205,9 @@ SL_DEV void flow_prologue(float& h0, float& h1, bool has_r, float r0, float r1, 
 
 // Stores of a wave are acknowledged in order with its loads, so a wave that has just published results cannot
 // finish a poll before the write has travelled to memory and back.  All tagged results of a stage are therefore
-// gathered in LDS and written by wave 15 (full 64-byte lines), and wave 15 never takes part in a poll.
+// gathered in LDS and written by one wave, wave 15 (full 64-byte lines), so that only that wave's polls of the next
+// stage return behind a store.  (It does poll where every thread fetches its own share of a vector: handing its
+// share to another wave through LDS measured slower than the late return.)
 constexpr int PUB_WAVE = DEC_WAVES - 1;
 constexpr int DENSE_WAVE0 = 128 * DEC_WAVES;     // first wave of the router rows (workgroup 128)
 constexpr int PAIR_WAVE0 = 160 * DEC_WAVES;      // first wave of the shared gate/up pairs (workgroups 160..191)
