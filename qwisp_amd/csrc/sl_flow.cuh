@@ -385,7 +385,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
   const uint16_t* hin = uni(Y.hist[par]);
   const int hv = gdn_unit_head(wg), dvb = gdn_unit_dvb(wg), hk = hv >> 1;
   const int half = lane >> 5, l32 = lane & 31;
-  // waves 8..15 hold the recurrent state (they take no part in this stage's or the next stage's poll)
+  // waves 8..15 hold the recurrent state (they take no part in this stage's poll)
   float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   if (wave >= 8) {
     const int dv = dvb * 16 + (wave - 8) * 2 + half;
