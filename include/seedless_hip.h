@@ -267,14 +267,19 @@ typedef struct {
   int32_t min_match;     /* QWISP_SUFFIX_MINMATCH, default 4 */
   int32_t gate;          /* 1 = speculation gate on (QWISP_SPEC_GATE) */
   int32_t gate_reprobe;  /* emitted tokens before drafting is tried again (QWISP_SPEC_REPROBE, default 256, >= 8) */
+  int32_t pending_prefix; /* 1 = the reference's opt-in "A3" mode (QWISP_RAW_A3, TellRuntime.swift:792-845): after a reject
+                           * the accepted tokens are not run again at once but kept pending and verified as leading rows of
+                           * the next step: rows = [pending] + [u] + drafts <= max_m; the list is flushed with
+                           * sl_forward_tokens at min(24, max_m - 1 - max_draft) tokens; no gate; needs max_m >= 3 */
 } sl_spec_options;
 typedef struct {
-  int32_t steps, drafted, accepted, draftless, rejects, chain_calls, gate_suspensions, reserved;
+  int32_t steps, drafted, accepted, draftless, rejects, chain_calls, gate_suspensions, pending_flushes;
 } sl_spec_stats;
-/* Tell.runSpecLoop without its A3 mode (TellRuntime.swift:716-886): prefill, then per step a suffix draft,
- * one sl_step_argmax over [pending token] + drafts, acceptance of the matching prefix; a reject is undone with
- * sl_rollback_one_step and the accepted rows are run again with sl_forward_tokens.  The n_new tokens written to
- * `out` are those of sl_greedy_generate.  max_seq_len must cover n_prompt + n_new + max_draft + chain_k. */
+/* Tell.runSpecLoop (TellRuntime.swift:716-886): prefill, then per step a suffix draft, one sl_step_argmax over
+ * [next token] + drafts, acceptance of the matching prefix; a reject is undone with sl_rollback_one_step and the
+ * accepted rows are run again with sl_forward_tokens (or kept pending, see pending_prefix; the caches then end
+ * before any tokens still pending when the loop returns).  The n_new tokens written to `out` are those of
+ * sl_greedy_generate.  max_seq_len must cover n_prompt + n_new + max_draft + chain_k. */
 int sl_spec_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_new, const sl_spec_options* opt,
                      int32_t* out, sl_spec_stats* stats);
 /* The same loop on a table of callbacks shaped like Tell.SpecBackend (TellRuntime.swift:83-111); every

@@ -57,12 +57,12 @@ class Snap(C.Structure):
 
 class SpecOptions(C.Structure):
     _fields_ = [("max_draft", C.c_int32), ("chain_k", C.c_int32), ("min_match", C.c_int32), ("gate", C.c_int32),
-                ("gate_reprobe", C.c_int32)]
+                ("gate_reprobe", C.c_int32), ("pending_prefix", C.c_int32)]
 
 
 class SpecStats(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("steps", "drafted", "accepted", "draftless", "rejects", "chain_calls",
-                                         "gate_suspensions", "reserved")]
+                                         "gate_suspensions", "pending_flushes")]
 
 
 STEP_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int32), C.c_int, C.POINTER(C.c_int32))

@@ -4,9 +4,11 @@
 //   * sl_suffix_draft      - Tell.suffixDraft (Tell.swift:104-175): training-free draft from the longest suffix
 //                            of the sequence that occurred before, continued by majority vote.
 //   * sl_spec_gate_*       - the mechanical speculation gate (Tell.swift:45-57).
-//   * sl_spec_generate     - Tell.runSpecLoop without the A3 research mode (TellRuntime.swift:716-886):
+//   * sl_spec_generate     - Tell.runSpecLoop (TellRuntime.swift:716-886):
 //                            draft -> verify [u] + drafts as rows of one step -> accept the matching prefix;
-//                            on a reject roll the step back and rebuild with the accepted rows.  The loop
+//                            on a reject roll the step back and rebuild with the accepted rows - or, in the
+//                            pending-prefix mode (the reference's opt-in "A3", TellRuntime.swift:792-845), keep
+//                            the accepted tokens pending and run them as leading rows of the next step.  The loop
 //                            itself (sl_spec_generate_backend) runs on a table of callbacks shaped like
 //                            Tell.SpecBackend (TellRuntime.swift:83-111), so it is testable without a device.
 //
@@ -23,6 +25,7 @@ namespace {
 
 constexpr int SUFFIX_ALPHA = 4;     // draft length cap = alpha * match length (Tell.swift:19)
 constexpr int GATE_WINDOW = 8;      // Tell.swift:45
+constexpr int PENDING_CAP = 24;     // TellRuntime.swift:734
 
 int gate_threshold(int hist_len) { return 4 + hist_len / 3000; }
 int gate_window_needed(int hist_len) { const int w = GATE_WINDOW - hist_len / 6000; return w > 1 ? w : 1; }
@@ -98,6 +101,17 @@ int sl_spec_generate_backend(const sl_spec_backend* b, const int32_t* prompt, in
   const int chain_k = !b->chained_step_argmax || opt->chain_k < 0 ? 0 : (opt->chain_k > 256 ? 256 : opt->chain_k);
   const int min_match = opt->min_match < 1 ? 4 : opt->min_match;
   const int reprobe = opt->gate_reprobe < 8 ? 8 : opt->gate_reprobe;
+  // Pending-prefix mode: a verify step is [pending] + [u] + drafts, so the pending list is flushed once it has
+  // pending_cap tokens (24 in the reference, TellRuntime.swift:734; less where max_rows is small).  The gate is
+  // off in this mode (TellRuntime.swift:759).
+  const bool pending_mode = opt->pending_prefix != 0;
+  int pending_cap = 0;
+  if (pending_mode) {
+    if (max_rows < 3) return SL_ERR_ARG;
+    if (max_k > max_rows - 2) max_k = max_rows - 2;
+    pending_cap = max_rows - 1 - max_k < PENDING_CAP ? max_rows - 1 - max_k : PENDING_CAP;
+  }
+  const bool gate = opt->gate && !pending_mode;
   sl_spec_stats st;
   std::memset(&st, 0, sizeof(st));
   if (stats) *stats = st;
@@ -118,20 +132,20 @@ int sl_spec_generate_backend(const sl_spec_backend* b, const int32_t* prompt, in
   std::vector<int32_t> emitted;
   emitted.reserve((size_t)n_new + 300);
   std::vector<int32_t> drafts(max_k > 0 ? max_k : 1), rows((size_t)max_rows), evals((size_t)(max_rows > 256 ? max_rows : 256));
-  std::vector<int32_t> window;
+  std::vector<int32_t> window, pending;
   long suspended_until = -1;
   auto emit = [&](int32_t t) { emitted.push_back(t); hist.push_back(t); };
 
   while ((int)emitted.size() < n_new) {
     int D = 0;
-    if (max_k > 0 && !(opt->gate && (long)emitted.size() < suspended_until)) {
+    if (max_k > 0 && !(gate && (long)emitted.size() < suspended_until)) {
       hist.push_back(u);
       D = suffix_draft(hist.data(), (int)hist.size(), 32, max_k, min_match, drafts.data());
       hist.pop_back();
     }
     st.steps++; st.drafted += D; if (D == 0) st.draftless++;
     if (D == 0) {
-      if (chain_k > 0) {
+      if (chain_k > 0 && pending.empty()) {
         // K greedy steps in one submission; the last result is the next pending token
         r = b->chained_step_argmax(b->ctx, u, chain_k, evals.data()); if (r) return r;
         st.chain_calls++;
@@ -140,6 +154,15 @@ int sl_spec_generate_backend(const sl_spec_backend* b, const int32_t* prompt, in
         if (add > n_new - (int)emitted.size()) add = n_new - (int)emitted.size();
         for (int i = 0; i < add; ++i) emit(evals[i]);
         u = evals[chain_k - 1];
+      } else if (!pending.empty()) {
+        // one step over [pending] + [u] realises the pending rows; the last row's result follows u
+        const int pk = (int)pending.size();
+        std::memcpy(rows.data(), pending.data(), (size_t)pk * sizeof(int32_t));
+        rows[pk] = u;
+        r = b->step_argmax(b->ctx, rows.data(), pk + 1, evals.data()); if (r) return r;
+        emit(u);
+        u = evals[pk];
+        pending.clear();
       } else {
         r = b->step_argmax(b->ctx, &u, 1, evals.data()); if (r) return r;
         emit(u);
@@ -148,13 +171,42 @@ int sl_spec_generate_backend(const sl_spec_backend* b, const int32_t* prompt, in
       continue;
     }
     r = b->snapshot(b->ctx); if (r) return r;
+    if (pending_mode) {
+      // [pending] + [u] + drafts as one step; row pk is u's, so draft p is checked against the result of row pk + p
+      const int pk = (int)pending.size();
+      std::memcpy(rows.data(), pending.data(), (size_t)pk * sizeof(int32_t));
+      rows[pk] = u;
+      for (int i = 0; i < D; ++i) rows[pk + 1 + i] = drafts[i];
+      r = b->step_argmax(b->ctx, rows.data(), pk + 1 + D, evals.data()); if (r) return r;
+      int p = 0;
+      while (p < D && drafts[p] == evals[pk + p]) ++p;
+      st.accepted += p;
+      if (p == D) {
+        pending.clear();                               // the step has advanced the caches over every row
+      } else {
+        // reject: back to before the pending rows; u and the accepted drafts join them and wait for the next step
+        st.rejects++;
+        r = b->rollback(b->ctx); if (r) return r;
+        pending.push_back(u);
+        for (int i = 0; i < p; ++i) pending.push_back(drafts[i]);
+        if ((int)pending.size() >= pending_cap) {
+          r = b->forward_tokens(b->ctx, pending.data(), (int)pending.size()); if (r) return r;
+          st.pending_flushes++;
+          pending.clear();
+        }
+      }
+      emit(u);
+      for (int i = 0; i < p; ++i) emit(drafts[i]);
+      u = evals[pk + p];
+      continue;
+    }
     rows[0] = u;
     for (int i = 0; i < D; ++i) rows[1 + i] = drafts[i];
     r = b->step_argmax(b->ctx, rows.data(), 1 + D, evals.data()); if (r) return r;
     int p = 0;
     while (p < D && drafts[p] == evals[p]) ++p;
     st.accepted += p;
-    if (opt->gate) {
+    if (gate) {
       window.push_back(p);
       if ((int)window.size() > GATE_WINDOW) window.erase(window.begin());
       if (gate_should_suspend(window.data(), (int)window.size(), (int)hist.size())) {

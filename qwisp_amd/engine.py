@@ -183,16 +183,18 @@ class SeedlessFusedForward:
             return None
         return out[:n_new]
 
-    def spec_generate(self, prompt, n_new, max_draft=16, chain_k=8, min_match=4, gate=True, gate_reprobe=256):
-        """Tell.runSpecLoop (TellRuntime.swift:716): suffix drafts verified as rows of one step.  Returns
+    def spec_generate(self, prompt, n_new, max_draft=16, chain_k=8, min_match=4, gate=True, gate_reprobe=256,
+                      pending_prefix=False):
+        """Tell.runSpecLoop (TellRuntime.swift:716): suffix drafts verified as rows of one step; pending_prefix = its
+        opt-in A3 mode (accepted tokens of a rejected step wait as leading rows of the next).  Returns
         (tokens, stats dict) or None."""
         pr = np.ascontiguousarray(prompt, np.int32)
         out = np.empty(max(n_new, 1), np.int32)
-        opt = abi.SpecOptions(max_draft, chain_k, min_match, 1 if gate else 0, gate_reprobe)
+        opt = abi.SpecOptions(max_draft, chain_k, min_match, 1 if gate else 0, gate_reprobe, 1 if pending_prefix else 0)
         st = abi.SpecStats()
         if self.lib.dll.sl_spec_generate(self.h, _p(pr), len(pr), n_new, C.byref(opt), _p(out), C.byref(st)) != abi.SL_OK:
             return None
-        return out[:n_new], {n: getattr(st, n) for n, _ in abi.SpecStats._fields_ if n != "reserved"}
+        return out[:n_new], {n: getattr(st, n) for n, _ in abi.SpecStats._fields_}
 
     # -- snapshots ------------------------------------------------------------------------------------
     def snapshot(self):

@@ -720,16 +720,19 @@ def test_spec_loop_stream_equals_greedy_stream(env):
     ref = env["Engine"](cfg, dev, max_m=8, max_seq_len=256)
     want = ref.greedy_generate(prompt, n_new, chain_k=8)
     assert want is not None, ref.gpu_fault
-    for max_draft, chain_k, gate in [(7, 8, False), (3, 0, False), (7, 4, True)]:
+    # the last two: the pending-prefix mode (accepted tokens of a rejected step run as leading rows of the next step)
+    for max_draft, chain_k, gate, pending in [(7, 8, False, False), (3, 0, False, False), (7, 4, True, False),
+                                              (3, 4, False, True), (5, 0, False, True)]:
         eng = env["Engine"](cfg, dev, max_m=8, max_seq_len=256)
-        res = eng.spec_generate(prompt, n_new, max_draft=max_draft, chain_k=chain_k, min_match=1, gate=gate, gate_reprobe=8)
+        res = eng.spec_generate(prompt, n_new, max_draft=max_draft, chain_k=chain_k, min_match=1, gate=gate, gate_reprobe=8,
+                                pending_prefix=pending)
         assert res is not None, eng.gpu_fault
         got, st = res
-        assert got.tolist() == want.tolist(), (max_draft, chain_k, gate, st)
-        print("spec loop", (max_draft, chain_k, gate), st)
+        assert got.tolist() == want.tolist(), (max_draft, chain_k, gate, pending, st)
+        print("spec loop", (max_draft, chain_k, gate, pending), st)
         assert st["drafted"] > 0 and st["accepted"] <= st["drafted"] and st["steps"] > 0
         assert st["rejects"] > 0 or st["accepted"] == st["drafted"]
-        assert eng.position >= len(prompt) + n_new - 1
+        assert eng.position >= len(prompt) + n_new - 1 - (8 if pending else 0)
         eng.close()
     ref.close()
 

@@ -182,7 +182,7 @@ def test_spec_loop_stream_equals_greedy_on_a_fake_backend(dll, chain_k, gate, ma
     n_new = 300
     want = fm.greedy(prompt.tolist(), n_new + 40)
     out = np.zeros(n_new, np.int32)
-    opt = abi.SpecOptions(max_draft, chain_k, 4, gate, 16)
+    opt = abi.SpecOptions(max_draft, chain_k, 4, gate, 16, 0)
     st = abi.SpecStats()
     r = dll.sl_spec_generate_backend(C.byref(fm.b), prompt.ctypes.data_as(C.c_void_p), len(prompt), n_new, C.byref(opt),
                                      out.ctypes.data_as(C.c_void_p), C.byref(st))
@@ -200,3 +200,47 @@ def test_spec_loop_stream_equals_greedy_on_a_fake_backend(dll, chain_k, gate, ma
         assert st.gate_suspensions >= 0
     # every reject was followed by a rebuild of the accepted rows
     assert sum(1 for k, _ in fm.calls if k == "forward") == -(-len(prompt) // fm.b.max_rows) + st.rejects
+
+
+@pytest.mark.parametrize("chain_k,max_draft,max_rows,with_chain", [(8, 8, 40, True), (0, 8, 40, True), (4, 5, 9, True), (8, 16, 12, False)])
+def test_pending_prefix_mode_stream_equals_greedy_on_a_fake_backend(dll, chain_k, max_draft, max_rows, with_chain):
+    """The reference's opt-in A3 mode (TellRuntime.swift:792-845): after a reject nothing is rebuilt; the token and
+    its accepted drafts wait and run as leading rows of the next step (draft p is checked against row pk + p of
+    [pending] + [u] + drafts).  Same lossless contract; the backend's cache is a prefix of prompt + stream, behind
+    it by at most the pending list; no step exceeds max_rows; a rebuild (forward after the prefill) only happens
+    when the pending list reaches its cap."""
+    fm = FakeModel(max_rows=max_rows, with_chain=with_chain)
+    prompt = np.array([1, 2, 3, 4, 5, 6, 1, 2, 3], np.int32)
+    n_new = 300
+    want = fm.greedy(prompt.tolist(), n_new + 60)
+    out = np.zeros(n_new, np.int32)
+    opt = abi.SpecOptions(max_draft, chain_k, 4, 1, 16, 1)         # the gate flag is ignored in this mode
+    st = abi.SpecStats()
+    r = dll.sl_spec_generate_backend(C.byref(fm.b), prompt.ctypes.data_as(C.c_void_p), len(prompt), n_new, C.byref(opt),
+                                     out.ctypes.data_as(C.c_void_p), C.byref(st))
+    assert r == abi.SL_OK
+    assert out.tolist() == want[:n_new]
+    full = prompt.tolist() + want
+    max_k = min(max_draft, max_rows - 2)
+    cap = min(24, max_rows - 1 - max_k)
+    assert fm.cache == full[:len(fm.cache)] and len(fm.cache) >= len(prompt) + n_new - 1 - (cap + max_k)
+    assert st.drafted > 0 and st.accepted > 0 and st.rejects > 0 and st.gate_suspensions == 0
+    assert max(m for kind, m in fm.calls if kind == "step") <= max_rows
+    if cap > 1:
+        assert st.rejects > st.pending_flushes            # rejects were not rebuilt at once: their tokens rode along later
+    else:
+        assert st.rejects == st.pending_flushes           # a list of one is flushed as soon as it exists
+    forwards = [m for kind, m in fm.calls if kind == "forward"]
+    assert len(forwards) == -(-len(prompt) // max_rows) + st.pending_flushes
+    assert all(cap <= m <= max_rows for m in forwards[-st.pending_flushes:]) if st.pending_flushes else True
+    if not (chain_k and with_chain):
+        assert st.chain_calls == 0
+
+
+def test_pending_prefix_mode_needs_three_rows(dll):
+    fm = FakeModel(max_rows=2)
+    prompt = np.array([1, 2, 3], np.int32)
+    out = np.zeros(4, np.int32)
+    opt = abi.SpecOptions(4, 0, 4, 0, 16, 1)
+    assert dll.sl_spec_generate_backend(C.byref(fm.b), prompt.ctypes.data_as(C.c_void_p), 3, 4, C.byref(opt),
+                                        out.ctypes.data_as(C.c_void_p), None) == abi.SL_ERR_ARG
