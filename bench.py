@@ -27,6 +27,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_FP16_PEAK_TFLOPS = 2500.0
 PROMPT_LEN = 512
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "k_decode_flow_decode_b1_40layer_hbm_traffic_pmc.txt")
 
@@ -57,6 +58,41 @@ def step_bytes(cfg, ctx):
     head = q4(cfg.vocab, H)
     norms = (2 * cfg.n_layers + 1) * H * 2
     return cfg.n_layers * moe + n_gdn * gdn + n_attn * attn + head + norms, head
+
+
+def lane_step_bytes(cfg, ctxs):
+    """Algorithmic HBM bytes of one step of len(ctxs) lanes (row b = lane b's next token): what the lanes share is
+    counted once (dense projections, router, shared expert, norms, head), every routed expert the batch touches once
+    (expected count per layer under the uniform routing of random weights: E (1 - (1 - 8/E)^B)), and per lane its
+    recurrent state and conv history read + written and its KV prefix read."""
+    q4 = lambda n, k: n * k // 2 + n * k // 16
+    H, I, E, B = 2048, 512, cfg.n_experts, len(ctxs)
+    expert = 2 * q4(I, H) + q4(H, I)
+    touched = E * (1.0 - (1.0 - 8.0 / E) ** B)
+    moe = E * H * 2 + expert + H * 2 + touched * expert
+    gdn_w = q4(12352, H) + q4(H, 4096) + 8192 * 4 * 4
+    gdn_lane = 2 * 3 * 8192 * 2 + 2 * 32 * 128 * 128 * 4
+    attn_w = q4(9216, H) + q4(H, 4096)
+    kv = sum(2 * 2 * c * 256 * 2 for c in ctxs)
+    n_attn = sum(0 if cfg.is_linear(i) else 1 for i in range(cfg.n_layers))
+    n_gdn = cfg.n_layers - n_attn
+    shared = cfg.n_layers * moe + n_gdn * gdn_w + n_attn * attn_w + q4(cfg.vocab, H) + (2 * cfg.n_layers + 1) * H * 2
+    return int(shared + n_gdn * B * gdn_lane + n_attn * kv)
+
+
+def prefill_flops(cfg, n):
+    """Multiply-adds x 2 of a prompt of n tokens: every projection row a token uses (router, shared expert and 8 routed
+    experts, the mixers' projections), causal attention scores and weighted sums (16 heads x 256 dims, key j <= row),
+    the gated delta rule per row (state [32 heads][128][128]: decay, k S, rank-1 update, S q) and the head on the last row."""
+    H, I, E = 2048, 512, cfg.n_experts
+    moe = (E + 1) * H + 9 * 3 * I * H
+    gdn = 12352 * H + H * 4096 + 4 * 32 * 128 * 128
+    attn = 9216 * H + H * 4096
+    n_attn = sum(0 if cfg.is_linear(i) else 1 for i in range(cfg.n_layers))
+    n_gdn = cfg.n_layers - n_attn
+    per_token = cfg.n_layers * moe + n_gdn * gdn + n_attn * attn
+    scores = n_attn * 16 * 256 * 2 * (n * (n + 1) // 2)
+    return 2 * (n * per_token + scores + cfg.vocab * H)
 
 
 def block_benchmarks(eng, cfg, np, torch):
@@ -257,6 +293,9 @@ def main():
         dt = time.perf_counter() - t0
         lanes_report = {"lanes": B, "ms_per_step": dt * 1e3 / n_lane_steps, "tok_s_aggregate": B * n_lane_steps / dt,
                         "contexts": f"{min(ctxs)}-{max(ctxs)} tokens, mean {sum(ctxs) // B}", "fill_s": t_fill, "path": "rows of the kernel-per-stage path, one launch sequence for all lanes"}
+        lane_b = lane_step_bytes(cfg, ctxs)             # the step's own byte roofline (shared weights once, touched experts once)
+        lanes_report["bytes_per_step"] = lane_b
+        lanes_report["frac_of_peak"] = lane_b / (dt / n_lane_steps) / 1e9 / HBM_PEAK_GBS
         if B >= 16:                                     # the same batch with projections, experts and lm_head on the matrix cores
             lanes[0].set_hybrid(True)
             for _ in range(2):
@@ -267,7 +306,8 @@ def main():
                 toks = step(lanes, toks).tolist()
             torch.cuda.synchronize()
             dt = time.perf_counter() - t0
-            lanes_report["hybrid_matrix_cores"] = {"ms_per_step": dt * 1e3 / n_lane_steps, "tok_s_aggregate": B * n_lane_steps / dt}
+            lanes_report["hybrid_matrix_cores"] = {"ms_per_step": dt * 1e3 / n_lane_steps, "tok_s_aggregate": B * n_lane_steps / dt,
+                                                   "frac_of_peak": lane_b / (dt / n_lane_steps) / 1e9 / HBM_PEAK_GBS}
             lanes[0].set_hybrid(False)
         for lane in lanes:
             lane.close()
@@ -309,6 +349,9 @@ def main():
                 assert o is not None, lane.gpu_fault
                 lane.close()
             prefill_report[name] = {"ms": times[-1] * 1e3, "tok_s": PF / times[-1]}
+            if hyb:                                        # against the dense fp16 rate of the matrix cores
+                prefill_report[name]["tflops"] = prefill_flops(cfg, PF) / times[-1] / 1e12
+                prefill_report[name]["frac_of_fp16_peak"] = prefill_report[name]["tflops"] / MFMA_FP16_PEAK_TFLOPS
         for m in [int(x) for x in args.prefill_also.split(",") if x]:
             times = []
             for rep in range(2):

@@ -334,17 +334,20 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   const bool grouped = M >= MOE_GROUP_MIN_ROWS && M <= GROUP_CAP;   // the shared expert then rides with the routed ones, by expert
   a.skip_shared = grouped ? 1 : 0;
   hipLaunchKernelGGL(k_moe_a, dim3((grouped ? 0 : MOE_A_SHARED_BLOCKS) + router_blocks, M), dim3(256), 0, e->stream, a);
-  hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, e->n_experts, L.route_inds, L.route_scores);
+  const bool route_in_b = !rows_first;                  // a few rows: stage B's waves route for themselves, one launch less
+  if (!route_in_b) hipLaunchKernelGGL(k_route_rows, dim3(M), dim3(64), 0, e->stream, e->rlogits, e->n_experts, L.route_inds, L.route_scores);
   MoeBArgs b{};
   b.xn = e->xn; b.g_w = L.sw_gate.w; b.g_sb = L.sw_gate.sb; b.u_w = L.sw_up.w; b.u_sb = L.sw_up.sb;
   b.act = e->act; b.inds = L.route_inds; b.xsum = rows_first ? e->xsum : nullptr;
+  if (route_in_b) { b.rlogits = e->rlogits; b.E = e->n_experts; b.inds_out = L.route_inds; b.scores_out = L.route_scores; }
   if (grouped) {                                        // weights of an expert fetched once for all rows that chose it
     hipLaunchKernelGGL(k_group_pairs, dim3(1), dim3(1024), 0, e->stream, L.route_inds, M, e->n_experts, e->hy_lists, e->hy_counts, e->hy_counts + SL_MAX_EXPERTS);
     MoeBGroupArgs g{e->xn, b.g_w, b.g_sb, b.u_w, b.u_sb, e->act, e->hy_lists, e->hy_counts, e->xsum, e->hy_counts + SL_MAX_EXPERTS,
                     L.sh_gate.w, L.sh_gate.sb, L.sh_up.w, L.sh_up.sb, e->sh_act, M};
     hipLaunchKernelGGL(k_moe_b_grouped, dim3(64, (M + 63) / 64 + e->n_experts), dim3(256), 0, e->stream, g);
   } else {
-    hipLaunchKernelGGL(k_moe_b, dim3(256, M), dim3(256), 0, e->stream, b);
+    if (route_in_b) hipLaunchKernelGGL(k_moe_b<true>, dim3(256, M), dim3(256), 0, e->stream, b);
+    else hipLaunchKernelGGL(k_moe_b<false>, dim3(256, M), dim3(256), 0, e->stream, b);
   }
   if (M >= MOE_GROUP_MIN_ROWS && M <= GROUP_CAP && e->hy_d && e->hy_sy) {   // the down stage by expert as well, then the combine
     MoeCGroupArgs cg{e->act, e->sh_act, L.sw_down.w, L.sw_down.sb, L.sh_down.w, L.sh_down.sb, e->hy_lists, e->hy_counts,

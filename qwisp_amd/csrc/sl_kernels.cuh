@@ -857,6 +857,12 @@ struct MoeBArgs {
   uint16_t* act;               // [M, 8, 512]
   const int32_t* inds;         // [M, 8]
   const float* xsum;           // [M, 256] word sums of the rows (HiddenArgs::xs_out), or null: formed here
+  // a few rows (a verify step): no routing launch before this one; every wave routes its row itself from the logits
+  // and workgroup 0 of the row leaves indices and scores for stage C
+  const uint16_t* rlogits;     // [M, 256] (k_moe_b<true>; otherwise `inds` holds the routing)
+  int E;
+  int32_t* inds_out;           // [M, 8]
+  uint16_t* scores_out;        // [M, 8]
 };
 constexpr int GROUP_CAP = 2048;         // pairs per expert: an expert is chosen at most once per row, M <= 2048
 // Pairs (row, slot) listed per expert (M * 8 pairs walked by 1024 threads), places handed out by LDS counters.
@@ -1004,11 +1010,23 @@ __global__ __launch_bounds__(256, 3) void k_moe_b_grouped(MoeBGroupArgs a) {
     }
   }
 }
+template <bool ROUTE>
 __global__ __launch_bounds__(256) void k_moe_b(MoeBArgs a) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int p0 = (blockIdx.x * 4 + wave) * 4;          // row index in [0, 8*512)
   const int k = p0 >> 9, i0 = p0 & 511;
-  const size_t base = (size_t)a.inds[m * 8 + k] * 512 + i0;
+  __shared__ int s_inds[ROUTE ? 4 : 1][8];
+  __shared__ float s_sc[ROUTE ? 4 : 1][8];
+  int expert;
+  if constexpr (ROUTE) {
+    route_wave(a.rlogits + (size_t)m * 256, a.E, lane, s_inds[wave], s_sc[wave]);
+    __syncthreads();
+    expert = s_inds[wave][k];
+    if (blockIdx.x == 0 && wave == 0 && lane < 8) { a.inds_out[m * 8 + lane] = s_inds[0][lane]; a.scores_out[m * 8 + lane] = f2h(s_sc[0][lane]); }
+  } else {
+    expert = a.inds[m * 8 + k];
+  }
+  const size_t base = (size_t)expert * 512 + i0;
   uint4 gw[4], uw[4];
   uint32_t gs[4], us[4];
 #pragma unroll
