@@ -313,6 +313,7 @@ void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   launch_qmm4_mfma(QmmArgs{e->sh_act, SL_MOE_I, L.sh_down.w, L.sh_down.sb, M, H, SL_MOE_I, e->hy_sy, H}, e->stream);
   hipLaunchKernelGGL(k_moe_combine_rows, dim3(H / 256, M), dim3(256), 0, e->stream, e->hy_d, L.route_scores, e->sgate, e->hy_sy, e->moe_out);
 }
+constexpr int HIDDEN_TILE_MAX_ROWS = 4;  // up to here the in-projection's waves do residual + norm of a row each
 constexpr int MOE_PROLOGUE_MAX_ROWS = 8;  // up to here stage A's waves do residual + norm themselves
 constexpr int MOE_GROUP_MIN_ROWS = 128;   // below, most experts are chosen by one row and the extra launches cost more
 void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
@@ -361,19 +362,25 @@ void launch_moe(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   c.d_w = L.sw_down.w; c.d_sb = L.sw_down.sb; c.shd_w = L.sh_down.w; c.shd_sb = L.sh_down.sb; c.out = e->moe_out;
   hipLaunchKernelGGL(k_moe_c, dim3(128, M), dim3(256), 0, e->stream, c);
 }
-// In-projection of M >= 2 rows: residual + norm once per row, then the row-tiled projection into e->proj.  Workgroups
+// In-projection of M >= 2 rows: residual + norm once per row (beyond four rows), then the row-tiled projection into e->proj.  Workgroups
 // of 16 weight rows, three to a compute unit: when the count is just over a multiple of the machine's 768 places the
 // surplus rows go one each to the first workgroups instead of opening another round.
 void launch_hidden_tile(sl_engine* e, const HiddenArgs& ha, const uint32_t* w, const uint32_t* sb, int N, int M) {
-  HiddenArgs hn = ha;
-  hn.xn_out = e->xn;
-  hn.xs_out = e->xsum;
-  hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
   constexpr int PLACES = 768;
   int G = N / 16;
   const int over = G % PLACES;
   if (G > PLACES && over <= 16) G -= over;
   if (G * 16 + G < N) G = (N + 15) / 16;          // (not with the shapes of this model)
+  if (M <= HIDDEN_TILE_MAX_ROWS) {
+    // a few rows (a verify step): the waves of every workgroup do residual + norm of a row each, one launch less
+    hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, true>), dim3(G, (M + 7) / 8), dim3(256), 0, e->stream, ha, (const uint16_t*)nullptr, 0,
+                       w, sb, N, e->proj, PROJ_STRIDE, M);
+    return;
+  }
+  HiddenArgs hn = ha;
+  hn.xn_out = e->xn;
+  hn.xs_out = e->xsum;
+  hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, hn);
   hipLaunchKernelGGL((k_qmv_tile<1, 4, 8, false>), dim3(G, (M + 7) / 8), dim3(256), 0, e->stream, HiddenArgs{}, e->xn, H,
                      w, sb, N, e->proj, PROJ_STRIDE, M, (float*)nullptr, (int32_t*)nullptr, e->xsum);
 }
@@ -402,7 +409,11 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
   g.hist[0] = L.hist[0]; g.hist[1] = L.hist[1]; g.state[0] = L.state[0]; g.state[1] = L.state[1];
   g.st = e->st + li;       // st[1] of this view = parity of layer li
   g.ycore = e->ycore; g.M = M; g.lanes = lanes; g.layer = li;
-  if (!lanes && M >= 2) {
+  const bool few = !lanes && !mm && M >= 2 && M <= GDN_FEW_ROWS;
+  if (few) {
+    // a verify step: conv, norms, recurrence and gated norm of a value head in one workgroup, one launch instead of three
+    hipLaunchKernelGGL(k_gdn_few_rows, dim3(SL_GDN_HV), dim3(1024), 0, e->stream, g, L.gdn_norm_w, L.norm_f32, e->ysum);
+  } else if (!lanes && M >= 2) {
     // rows of one sequence: the state-independent part for all rows at once, then the scan without barriers
     GdnPrepArgs pa{g, e->gdn_qn, e->gdn_kn, e->gdn_vc, e->gdn_gb};
     hipLaunchKernelGGL(k_gdn_prep_rows, dim3(65, (M + GDN_PREP_ROWS - 1) / GDN_PREP_ROWS), dim3(64), 0, e->stream, pa);
@@ -424,7 +435,7 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
     launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.out_proj.w, L.out_proj.sb, M, H, 4096, e->mix, H}, e->stream);
   } else if (M >= 2) {
     // the gated norm once per row, then the row-tiled projection (same bits as the fused kernel below)
-    hipLaunchKernelGGL(k_gdn_gate_rows, dim3(SL_GDN_HV, M), dim3(64), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32, e->ysum);
+    if (!few) hipLaunchKernelGGL(k_gdn_gate_rows, dim3(SL_GDN_HV, M), dim3(64), 0, e->stream, e->ycore, e->proj, L.gdn_norm_w, L.norm_f32, e->ysum);
     hipLaunchKernelGGL((k_qmv_tile<2, 2, 4, false>), dim3(H / 8, (M + 3) / 4), dim3(256), 0, e->stream, HiddenArgs{}, e->ycore, 4096,
                        L.out_proj.w, L.out_proj.sb, H, e->mix, H, M, (float*)nullptr, (int32_t*)nullptr, e->ysum);
   } else {

@@ -190,16 +190,16 @@ __global__ __launch_bounds__(256) void k_qmv_plain(const uint16_t* __restrict__ 
 // k_qmv_hidden / k_qmv_plain.  The tile's activation rows are prepared once per workgroup (residual, norm,
 // packing: wave w takes rows w, w + waves, ...) and parked in LDS, 20 words per lane (16 packed pairs, 4 sums)
 // so that a lane reads back its own 80 bytes with five 16-byte reads free of bank conflicts.
-// HIDDEN: x comes from the hidden prologue (K = 2048); otherwise from the fp16 buffer xin (K = 2048*NBLK).
-// Grid (G, ceil(M / MT)); up to 8 waves with the hidden prologue, 4 without (three workgroups share a compute
-// unit).  G workgroups cover G*waves*R rows; rows beyond that (fewer than G) are taken one each by wave 0 of the
+// HIDDEN: x comes from the hidden prologue (K = 2048; steps of up to four rows, where a wave preparing one row in
+// every workgroup costs less than a launch that prepares the rows once); otherwise from the fp16 buffer xin
+// (K = 2048*NBLK).  Grid (G, ceil(M / MT)), four waves (three workgroups share a compute unit).  G workgroups cover G*waves*R rows; rows beyond that (fewer than G) are taken one each by wave 0 of the
 // first workgroups, so that G can be chosen to fill the machine exactly once (12352 rows: 768 workgroups of 16
 // rows + 64 single rows, instead of 772 workgroups on 768 places).
 // -------------------------------------------------------------------------------------------------
 // ARGMAX (lm_head, R = 4, 4 waves): y is the logits matrix and every workgroup also leaves one (value, index)
 // candidate per activation row, the first maximum of its 16 rounded logits, for k_argmax_final.
 template <int NBLK, int R, int MT, bool HIDDEN, bool ARGMAX = false>
-__global__ __launch_bounds__(HIDDEN ? 512 : 256, HIDDEN ? 2 : 3) void k_qmv_tile(HiddenArgs ha, const uint16_t* __restrict__ xin, int x_stride,
+__global__ __launch_bounds__(256, 3) void k_qmv_tile(HiddenArgs ha, const uint16_t* __restrict__ xin, int x_stride,
                                                   const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB,
                                                   int N, uint16_t* __restrict__ y, int y_stride, int M,
                                                   float* __restrict__ cand_v = nullptr, int32_t* __restrict__ cand_i = nullptr,
@@ -714,6 +714,138 @@ __global__ __launch_bounds__(64) void k_gdn_gate_rows(uint16_t* __restrict__ yco
   const float o0 = f16r((z0 * sigmoid32(z0)) * n0), o1 = f16r((z1 * sigmoid32(z1)) * n1);
   *reinterpret_cast<uint32_t*>(yp) = pack2(o0, o1);
   if (ysum) {
+    const int q = lane & 3;
+    float sw = (0.0f + o0) + o1;
+#pragma unroll
+    for (int r = 1; r < 4; ++r) {
+      const float v = prev_lane(sw);
+      if (q == r) sw = (v + o0) + o1;
+    }
+    if (q == 3) ysum[(size_t)m * 512 + hv * 16 + (lane >> 2)] = sw;
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// A GDN layer's core for a few rows of one sequence (a verify step, M <= GDN_FEW_ROWS) in one launch: what
+// k_gdn_prep_rows, k_gdn_scan_rows and k_gdn_gate_rows do in three, with the same arithmetic per row.  Grid 32: a
+// workgroup of 16 waves owns one value head, so the gated norm over the head's 128 outputs stays inside it.  Every
+// load from the projection rows is requested up front (a thread holds the conv window of its channel, M + 3 taps);
+// conv outputs, normed queries / keys, decays and betas of all rows wait in LDS, and the recurrence then runs
+// through the rows without a barrier.  Wave w holds state rows 8 w .. 8 w + 7 of the head, one per half-wave and pass.
+// -------------------------------------------------------------------------------------------------
+constexpr int GDN_FEW_ROWS = 8;
+__global__ __launch_bounds__(1024) void k_gdn_few_rows(GdnArgs a, const float* __restrict__ norm_w, int norm_f32, float* __restrict__ ysum) {
+  __shared__ float s_q[GDN_FEW_ROWS][128], s_k[GDN_FEW_ROWS][128], s_v[GDN_FEW_ROWS][128], s_y[GDN_FEW_ROWS][128];
+  __shared__ float s_g[GDN_FEW_ROWS], s_b[GDN_FEW_ROWS];
+  const int hv = blockIdx.x, hk = hv >> 1, M = a.M;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+  const bool par = a.st[1] != 0;
+  const uint16_t* hin = par ? a.hist[1] : a.hist[0];
+  uint16_t* hout = par ? a.hist[0] : a.hist[1];
+  const float* sin_ = par ? a.state[1] : a.state[0];
+  float* sout = par ? a.state[0] : a.state[1];
+  float s[4][4];
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int dv = wave * 8 + it * 2 + half;
+    const float4 v = *reinterpret_cast<const float4*>(sin_ + ((size_t)hv * 128 + dv) * 128 + 4 * l32);
+    s[it][0] = v.x; s[it][1] = v.y; s[it][2] = v.z; s[it][3] = v.w;
+  }
+  // waves 0-1: query channels of the key head, 2-3: its key channels, 4-5: the value channels of this head;
+  // wave 6, lane t: decay of row t; wave 7, lane t: beta of row t; waves 8..8+M-1: the z row of the gated norm
+  const int ch = tid < 128 ? hk * 128 + tid : (tid < 256 ? 2048 + hk * 128 + (tid - 128) : 4096 + hv * 128 + (tid - 256));
+  uint16_t win[GDN_FEW_ROWS + 3];
+  float cw[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (tid < 384) {
+#pragma unroll
+    for (int j = 0; j < GDN_FEW_ROWS + 3; ++j) {
+      const int row = min(j, M + 2);                     // rows of the concatenation [hist(3) | qkv(M)]
+      win[j] = (row < 3) ? hin[row * SL_CONV_DIM + ch] : a.proj[(size_t)(row - 3) * PROJ_STRIDE + ch];
+    }
+    const float4 c4 = *reinterpret_cast<const float4*>(a.conv_w + ch * 4);
+    cw[0] = c4.x; cw[1] = c4.y; cw[2] = c4.z; cw[3] = c4.w;
+  }
+  uint32_t zw = 0;
+  float nw0 = 0.0f, nw1 = 0.0f;
+  if (wave >= 8 && wave - 8 < M) {
+    zw = *reinterpret_cast<const uint32_t*>(a.proj + (size_t)(wave - 8) * PROJ_STRIDE + 8192 + hv * 128 + 2 * lane);
+    nw0 = norm_w[2 * lane]; nw1 = norm_w[2 * lane + 1];
+  }
+  if (tid < 384) {
+    float* dst = tid < 128 ? &s_q[0][tid] : (tid < 256 ? &s_k[0][tid - 128] : &s_v[0][tid - 256]);
+#pragma unroll
+    for (int t = 0; t < GDN_FEW_ROWS; ++t) {
+      if (t >= M) continue;
+      float acc = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) acc = fmaf(h2f(win[t + k]), cw[k], acc);
+      dst[t * 128] = f16r(acc * sigmoid32(acc));
+    }
+  } else if (wave == 6 && lane < M) {
+    const float aP = h2f(a.proj[(size_t)lane * PROJ_STRIDE + 12320 + hv]);
+    s_g[lane] = exp_c(-(exp_c(a.a_log[hv]) * softplus_c(aP + a.dt_bias[hv])));
+  } else if (wave == 7 && lane < M) {
+    s_b[lane] = sigmoid16(h2f(a.proj[(size_t)lane * PROJ_STRIDE + 12288 + hv]));
+  }
+  __syncthreads();
+  if (wave < 2 * M) {
+    // weightless rmsnorm over 128, then the key / query scale, both rounded to half: wave = (row, query | key)
+    float* buf = (wave & 1) ? s_k[wave >> 1] : s_q[wave >> 1];
+    const float x0 = buf[2 * lane], x1 = buf[2 * lane + 1];
+    float ss = fmaf(x1, x1, fmaf(x0, x0, 0.0f));
+    ss = tree_sum<64>(ss);
+    const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
+    const float sc = (wave & 1) ? f16r(0.08838834764831845f) : f16r(0.0078125f);
+    buf[2 * lane] = f16r(sc * f16r(x0 * inv)); buf[2 * lane + 1] = f16r(sc * f16r(x1 * inv));
+  }
+  __syncthreads();
+  for (int t = 0; t < M; ++t) {
+    const float g = s_g[t], beta = s_b[t];
+    const float4 k4 = *reinterpret_cast<const float4*>(&s_k[t][4 * l32]);
+    const float4 q4 = *reinterpret_cast<const float4*>(&s_q[t][4 * l32]);
+    const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, qq[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int dvl = wave * 8 + it * 2 + half;
+      float acc = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { s[it][i] = s[it][i] * g; acc = fmaf(s[it][i], kk[i], acc); }
+      const float kv = tree_sum<32>(acc);
+      const float delta = (s_v[t][dvl] - kv) * beta;
+      acc = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { s[it][i] = fmaf(kk[i], delta, s[it][i]); acc = fmaf(s[it][i], qq[i], acc); }
+      const float y = tree_sum<32>(acc);
+      if (l32 == 0) s_y[t][dvl] = f16r(y);
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int dv = wave * 8 + it * 2 + half;
+    *reinterpret_cast<float4*>(sout + ((size_t)hv * 128 + dv) * 128 + 4 * l32) = make_float4(s[it][0], s[it][1], s[it][2], s[it][3]);
+  }
+  // history shift: rows M .. M + 2 of [hist | qkv]; query and key channels by the even heads, value channels by every head
+  if (tid < 384 && (tid >= 256 || (hv & 1) == 0)) {
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+      uint16_t tap = win[3];                             // (a run-time index into the window would move it to scratch memory)
+#pragma unroll
+      for (int r = 1; r <= GDN_FEW_ROWS; ++r) if (M == r) tap = win[r + j];
+      hout[j * SL_CONV_DIM + ch] = tap;
+    }
+  }
+  __syncthreads();
+  if (wave >= 8 && wave - 8 < M) {
+    // gated norm of row wave - 8 over the head's 128 outputs (the arithmetic of k_gdn_gate_rows), and the sums of
+    // each run of 8 gated values for the out-projection's dots
+    const int m = wave - 8;
+    const float y0 = s_y[m][2 * lane], y1 = s_y[m][2 * lane + 1], z0 = lo_h(zw), z1 = hi_h(zw);
+    const float ss = tree_sum<64>(fmaf(y1, y1, fmaf(y0, y0, 0.0f)));
+    const float inv = 1.0f / sqrtf(ss / 128.0f + EPS);
+    const float n0 = norm_f32 ? nw0 * (y0 * inv) : f16r(nw0 * f16r(y0 * inv));
+    const float n1 = norm_f32 ? nw1 * (y1 * inv) : f16r(nw1 * f16r(y1 * inv));
+    const float o0 = f16r((z0 * sigmoid32(z0)) * n0), o1 = f16r((z1 * sigmoid32(z1)) * n1);
+    *reinterpret_cast<uint32_t*>(a.ycore + (size_t)m * 4096 + hv * 128 + 2 * lane) = pack2(o0, o1);
     const int q = lane & 3;
     float sw = (0.0f + o0) + o1;
 #pragma unroll
