@@ -390,6 +390,7 @@ void launch_hidden_tile(sl_engine* e, const HiddenArgs& ha, const uint32_t* w, c
 // fewer than 64 rows keeps the row-tiled exact kernel for them (256 workgroups per 4 rows; 32 rows: 21 against 28 us).
 // Prefill chunks do not switch, so that a row's result does not depend on the chunking.
 constexpr int MM_OUT_ROWS = 64;
+constexpr int GDN_PREP_LONG = 512;    // from here on a wave of the GDN preparation walks 16 rows, below 4
 bool use_matrix_cores(const sl_engine* e, int M, const LaneRef* lanes) { (void)lanes; return e->hybrid && M >= 16 && M <= GROUP_CAP; }
 // `lanes` (null for rows of one sequence) = this layer's row of the lane table: row b of the batch is lane b's next token.
 void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs& ha, const LaneRef* lanes) {
@@ -416,7 +417,8 @@ void launch_gdn_mixer(sl_engine* e, LayerDev& L, int li, int M, const HiddenArgs
   } else if (!lanes && M >= 2) {
     // rows of one sequence: the state-independent part for all rows at once, then the scan without barriers
     GdnPrepArgs pa{g, e->gdn_qn, e->gdn_kn, e->gdn_vc, e->gdn_gb};
-    hipLaunchKernelGGL(k_gdn_prep_rows, dim3(65, (M + GDN_PREP_ROWS - 1) / GDN_PREP_ROWS), dim3(64), 0, e->stream, pa);
+    if (M >= GDN_PREP_LONG) hipLaunchKernelGGL(k_gdn_prep_rows<16>, dim3(65, (M + 15) / 16), dim3(64), 0, e->stream, pa);
+    else hipLaunchKernelGGL(k_gdn_prep_rows<4>, dim3(65, (M + 3) / 4), dim3(64), 0, e->stream, pa);
     if (mm && e->gc_scratch && M % GC == 0 && e->pos % GC == 0) {
       // hybrid chunks cut at multiples of 64 rows: the delta rule in its chunked form on the matrix cores
       GdnChunkArgs ca{e->gdn_qn, e->gdn_kn, e->gdn_vc, e->gdn_gb, e->gc_scratch, {L.state[0], L.state[1]}, {L.hist[0], L.hist[1]},

@@ -514,24 +514,26 @@ struct GdnPrepArgs {
   uint16_t* vc;              // [M, 4096] conv + silu of the value channels
   float* gb;                 // [M, 64]: decay g of the 32 value heads, then beta
 };
-// One wave per (unit, block of GDN_PREP_ROWS rows): units 0..15 query heads, 16..31 key heads, 32..63 value heads,
+// One wave per (unit, block of PR rows): units 0..15 query heads, 16..31 key heads, 32..63 value heads,
 // 64 decay / beta.  A wave walks its rows with the conv window in registers (a row's four taps are the three rows
 // before it and itself: every row of the projection is loaded once, all loads of the block up front), which also
 // keeps the number of waves of a 2048-row chunk at 8320 instead of one per row and unit.  The arithmetic per row is
 // that of conv_silu.
-constexpr int GDN_PREP_ROWS = 16;
+// PR = 16 for long chunks; steps of fewer rows take PR = 4, so that a step of 17 rows is 325 waves and not 130 waves
+// of up to 16 rows in sequence.
+template <int PR>
 __global__ __launch_bounds__(64) void k_gdn_prep_rows(GdnPrepArgs p) {
   const GdnArgs& a = p.g;
-  const int u = blockIdx.x, t0 = blockIdx.y * GDN_PREP_ROWS, lane = threadIdx.x;
-  const int rows = min(GDN_PREP_ROWS, a.M - t0);
+  const int u = blockIdx.x, t0 = blockIdx.y * PR, lane = threadIdx.x;
+  const int rows = min(PR, a.M - t0);
   const uint16_t* hin = a.st[1] ? a.hist[1] : a.hist[0];
   if (u < 64) {
     const bool isq = u < 16, isk = u >= 16 && u < 32;
     const int ch = u < 32 ? (isk ? 2048 : 0) + (u & 15) * 128 + 2 * lane : 4096 + (u - 32) * 128 + 2 * lane;
     // rows t0 .. t0 + rows + 2 of the concatenation [hist(3) | qkv(M)], two neighbouring channels per lane
-    uint32_t win[GDN_PREP_ROWS + 3];
+    uint32_t win[PR + 3];
 #pragma unroll
-    for (int j = 0; j < GDN_PREP_ROWS + 3; ++j) {
+    for (int j = 0; j < PR + 3; ++j) {
       const int row = min(t0 + j, t0 + rows + 2);
       win[j] = (row < 3) ? *reinterpret_cast<const uint32_t*>(hin + row * SL_CONV_DIM + ch)
                          : *reinterpret_cast<const uint32_t*>(a.proj + (size_t)(row - 3) * PROJ_STRIDE + ch);
@@ -541,7 +543,7 @@ __global__ __launch_bounds__(64) void k_gdn_prep_rows(GdnPrepArgs p) {
     for (int k = 0; k < 4; ++k) { w0[k] = a.conv_w[ch * 4 + k]; w1[k] = a.conv_w[(ch + 1) * 4 + k]; }
     const float sc = isk ? f16r(0.08838834764831845f) : f16r(0.0078125f);
 #pragma unroll
-    for (int j = 0; j < GDN_PREP_ROWS; ++j) {
+    for (int j = 0; j < PR; ++j) {
       if (j >= rows) continue;                  // (uniform; a break would keep the loop from unrolling)
       const int t = t0 + j;
       float a0 = 0.0f, a1 = 0.0f;

@@ -72,10 +72,12 @@ def test_generator_device_equals_host(env):
 # ---- matrix-core GEMM of the hybrid prefill ---------------------------------------------------------
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("m", [2, 5, 8, 9, 13, 17, 32])
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 8, 9, 13, 17, 32])
 def test_row_tiles_of_any_count_equal_single_steps(env, small_model, m):
     """The row kernels take activation rows in tiles of 8 (in-projection, lm_head) and 4 (out-projection): full
-    tiles, ragged last tiles and several tiles give, row by row, the bits of single steps (SeedlessVerifyTests.swift:613)."""
+    tiles, ragged last tiles and several tiles give, row by row, the bits of single steps (SeedlessVerifyTests.swift:613).
+    Steps of up to 4 and up to 8 rows take the launch-saving variants (in-projection waves that prepare their rows, the
+    GDN core of a value head in one workgroup, stage B routing for itself); 9 rows and more the general row kernels."""
     cfg, dev, host = small_model
     a = env["Engine"](cfg, dev, max_m=32, max_seq_len=96)
     b = env["Engine"](cfg, dev, max_m=32, max_seq_len=96)
