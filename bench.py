@@ -208,7 +208,7 @@ def main():
     dev = synth.generate_device(cfg, lib.get())
     t_gen = time.time() - t0
     max_seq = PROMPT_LEN + args.warmup + args.steps + 16 + 24 * max(args.verify_rows, 0)
-    eng = SeedlessFusedForward(cfg, dev, max_m=64, max_seq_len=max_seq)
+    eng = SeedlessFusedForward(cfg, dev, max_m=max(64, args.verify_rows), max_seq_len=max_seq)
     host = None
     if args.cpu_tokens > 0:
         host = {k: (v.cpu().numpy().view(np.uint32) if v.dtype == torch.int32 else v.cpu().numpy()) for k, v in dev.items()}
