@@ -982,7 +982,8 @@ __global__ __launch_bounds__(64) void k_route_rows(const uint16_t* __restrict__ 
   if (lane < 8) { inds[m * 8 + lane] = s_inds[lane]; scores[m * 8 + lane] = f2h(s_sc[lane]); }
 }
 
-// MoE stage B: the 8 routed experts' gate/up with SwiGLU, after k_route_rows.  A wave owns four consecutive rows of
+// MoE stage B: the 8 routed experts' gate/up with SwiGLU, after k_route_rows (ROUTE: every wave routes its row itself
+// first, for steps of a few rows, and workgroup 0 of the row leaves the routing for stage C).  A wave owns four consecutive rows of
 // one expert (gate and up); all eight weight loads are in flight before the first dot.  Grid (256, M).
 // Reference: gqmm4_swiglu_rows SeedlessMetalForward.swift:1419-1460.
 struct MoeBArgs {
