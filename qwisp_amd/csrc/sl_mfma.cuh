@@ -83,10 +83,13 @@ inline unsigned xcd_tile_grid(int col_blocks, int row_blocks) {   // workgroups 
 // row (B) -- word st of the 64-k group on the lower half-wave, word 4+st on the upper, so that a lane fetches its four
 // words of a group with one 16-byte load; the order within the eight is {0,4,1,5,2,6,3,7} on both sides.
 // -------------------------------------------------------------------------------------------------
-// Dequantisation of a packed word (8 weights) in packed half arithmetic: masking with 0x000F000F leaves the nibbles
-// j and j+4; or-ing a nibble into the mantissa of 1024.0 gives 1024 + q exactly, subtracting 1024 gives q exactly,
-// and half(q * s + b) is one fused multiply-add per pair.  `k1024` is the pattern 0x64006400 held in a vector
-// register, so that mask and or are one instruction (v_and_or_b32 takes one literal).
+// Dequantisation of a packed word (8 weights) in packed half arithmetic.  Masking with 0x000F000F leaves the nibbles
+// j and j+4 at the bottom of the two halves; or-ing a nibble into the mantissa of 1024.0 gives 1024 + q exactly and
+// subtracting 1024 gives q exactly.  Masking with 0x00F000F0 instead takes the nibbles one place up without a shift:
+// or-ed into 1024.0 they read 1024 + 16 q, and (1024 + 16 q) / 16 - 64 = q, again exact, is one fused multiply-add.
+// So a word costs one shift (by 8, for its upper two pairs) instead of three.  half(q * s + b) is one more fused
+// multiply-add per pair.  `k1024` is the pattern 0x64006400 held in a vector register, so that mask and or are one
+// instruction (v_and_or_b32 takes one literal).
 typedef _Float16 mf_h8 __attribute__((ext_vector_type(8)));
 SL_DEV uint32_t dequant_k1024() {
   uint32_t k = 0x64006400u;
@@ -95,16 +98,18 @@ SL_DEV uint32_t dequant_k1024() {
 }
 SL_DEV mf_h2 dequant_pair(uint32_t w, int j, mf_h2 s2, mf_h2 b2, uint32_t k1024) {   // nibbles j and j+4
   const mf_h2 f1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
-  const mf_h2 q = __builtin_bit_cast(mf_h2, ((w >> (4 * j)) & 0x000F000Fu) | k1024) - f1024;
+  const mf_h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f}, m64 = {(_Float16)-64.0f, (_Float16)-64.0f};
+  const uint32_t src = (j & 2) ? (w >> 8) : w;
+  mf_h2 q;
+  if (j & 1) q = __builtin_elementwise_fma(__builtin_bit_cast(mf_h2, (src & 0x00F000F0u) | k1024), sixteenth, m64);
+  else q = __builtin_bit_cast(mf_h2, (src & 0x000F000Fu) | k1024) - f1024;
   return __builtin_elementwise_fma(q, s2, b2);
 }
 SL_DEV mf_h8 dequant8(uint32_t w, mf_h2 s2, mf_h2 b2, uint32_t k1024) {
-  const mf_h2 f1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
   mf_h8 r;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const mf_h2 q = __builtin_bit_cast(mf_h2, ((w >> (4 * j)) & 0x000F000Fu) | k1024) - f1024;
-    const mf_h2 v = __builtin_elementwise_fma(q, s2, b2);
+    const mf_h2 v = dequant_pair(w, j, s2, b2, k1024);
     r[2 * j] = v[0]; r[2 * j + 1] = v[1];
   }
   return r;
