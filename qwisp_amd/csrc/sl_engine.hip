@@ -558,15 +558,6 @@ void launch_decode(sl_engine* e, int out_off, bool feed, int steps) {
   e->pos += steps;
   if (steps & 1) for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
 }
-// After a persistent step: a workgroup that gave up waiting leaves the abort word set.
-int check_decode_abort(sl_engine* e) {
-  unsigned flag = 0;
-  SL_TRY(e, hipMemcpyAsync(e->pinned, e->dec_bar + 32, 4, hipMemcpyDeviceToHost, e->stream));
-  SL_TRY(e, hipStreamSynchronize(e->stream));
-  std::memcpy(&flag, e->pinned, 4);
-  if (flag) { if (e->fault.empty()) e->fault = "persistent decode kernel: grid barrier timed out"; return SL_ERR_DEVICE; }
-  return SL_OK;
-}
 int to_device(sl_engine* e, void* dst, const void* src, size_t bytes) {
   if (bytes > e->pinned_bytes) return SL_ERR_ARG;
   std::memcpy(e->pinned, src, bytes);
@@ -608,7 +599,7 @@ int alloc_layer_state(sl_engine* e, LayerDev& L) {
 }
 int alloc_runtime(sl_engine* e);
 }  // namespace
-static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, const char* what);
+static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, const char* what, bool abort_word = false);
 static void time_end(sl_engine* e);
 
 int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** out) {
@@ -833,7 +824,7 @@ int alloc_runtime(sl_engine* e) {
       if (per_cu >= 1) e->dec_grid = 256;
     }
   }
-  e->pinned_bytes = MH * 2 + 4096 + (size_t)d->n_layers * 4 + (size_t)MAX_CHAIN * 4;
+  e->pinned_bytes = MH * 2 + 4096 + (size_t)d->n_layers * 4 + (size_t)MAX_CHAIN * 4 + 64;
   SL_TRY(e, hipHostMalloc(&e->pinned, e->pinned_bytes, hipHostMallocDefault));
   SL_TRY(e, hipStreamSynchronize(e->stream));
   return SL_OK;
@@ -1053,11 +1044,20 @@ int sl_profile_head_read(sl_engine* e, double* ms_sum, int64_t* launches) {
   return SL_OK;
 }
 
-static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, const char* what) {
-  if (bytes > e->pinned_bytes) return SL_ERR_ARG;
+// abort_word: after a persistent step, the word a workgroup that gave up waiting leaves set comes back with the same
+// synchronisation (the last 64 bytes of the pinned buffer are kept for it).
+static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, const char* what, bool abort_word) {
+  if (bytes > e->pinned_bytes - 64) return SL_ERR_ARG;
+  unsigned char* flag_at = (unsigned char*)e->pinned + e->pinned_bytes - 64;
   SL_TRY(e, hipMemcpyAsync(e->pinned, dev, bytes, hipMemcpyDeviceToHost, e->stream));
+  if (abort_word) SL_TRY(e, hipMemcpyAsync(flag_at, e->dec_bar + 32, 4, hipMemcpyDeviceToHost, e->stream));
   int r = finish(e, what);
   if (r) return r;
+  if (abort_word) {
+    unsigned flag = 0;
+    std::memcpy(&flag, flag_at, 4);
+    if (flag) { if (e->fault.empty()) e->fault = "persistent decode kernel: grid barrier timed out"; return SL_ERR_DEVICE; }
+  }
   std::memcpy(dst, e->pinned, bytes);
   return SL_OK;
 }
@@ -1091,8 +1091,7 @@ int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
     advance(e, m);
   }
   SL_TRY(e, hipEventRecord(e->ev1, e->stream));
-  r = read_back(e, out, e->tok_out, (size_t)m * 4, "stepArgmax"); if (r) return r;
-  if (persistent) { r = check_decode_abort(e); if (r) return r; }
+  r = read_back(e, out, e->tok_out, (size_t)m * 4, "stepArgmax", persistent); if (r) return r;
   time_end(e);
   return SL_OK;
 }
@@ -1117,8 +1116,7 @@ int sl_chained_step_argmax(sl_engine* e, int32_t first, int k, int32_t* out) {
     advance(e, 1);
   }
   SL_TRY(e, hipEventRecord(e->ev1, e->stream));
-  r = read_back(e, out, e->tok_out, (size_t)k * 4, "chainedStepArgmax"); if (r) return r;
-  if (persistent) { r = check_decode_abort(e); if (r) return r; }
+  r = read_back(e, out, e->tok_out, (size_t)k * 4, "chainedStepArgmax", persistent); if (r) return r;
   time_end(e);
   return SL_OK;
 }
