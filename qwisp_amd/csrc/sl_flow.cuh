@@ -1303,13 +1303,17 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
       uint32_t k[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) k[i] = 4 * lane + i < E ? route_key(w[i], 4 * lane + i) : 0u;
+      // a lane's four keys in falling order first (keys are distinct: the index rides in the low byte), so that a round
+      // is the wave-wide maximum of the lanes' first keys and a shift of the winner's list
+      auto order = [](uint32_t& a, uint32_t& b) { const uint32_t hi = max(a, b), lo = min(a, b); a = hi; b = lo; };
+      order(k[0], k[1]); order(k[2], k[3]); order(k[0], k[2]); order(k[1], k[3]); order(k[1], k[2]);
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
         // (the wave-wide maximum stays in vector registers: a value read out to a scalar register takes tens of clocks
         // to become usable, eight times in a row)
-        const uint32_t M = wave_max_u32(max(max(k[0], k[1]), max(k[2], k[3])));
-#pragma unroll
-        for (int i = 0; i < 4; ++i) k[i] = (k[i] == M) ? 0u : k[i];
+        const uint32_t M = wave_max_u32(k[0]);
+        const bool won = k[0] == M;
+        k[0] = won ? k[1] : k[0]; k[1] = won ? k[2] : k[1]; k[2] = won ? k[3] : k[2]; k[3] = won ? 0u : k[3];
         if (lane == 0) L.inds[r] = min(255 - (int)(M & 255u), E - 1);
       }
     } else {
