@@ -12,10 +12,14 @@
  *  - All functions returning int return SL_OK (0) or a negative sl_status.  The first failure
  *    of an engine is sticky: sl_fault() returns its message and every later call on that engine
  *    returns SL_ERR_POISONED without touching its outputs (SFV:388-401, TellRuntime.swift:193).
- *  - One thread inside one engine at a time (the reference serialises callers with a semaphore,
- *    LLMBackend.swift:129).  Different engines and lanes may be driven from different threads: batch-1 steps, which
- *    occupy the whole GPU with one launch, are serialised inside the library (the reference treats the GPU as
- *    exclusive, AGENTS.md:95).
+ *  - One process per GPU, and one call at work on it at a time (the reference serialises callers with a semaphore,
+ *    LLMBackend.swift:129, and treats the GPU as exclusive, AGENTS.md:95).  Engines and lanes may be created, driven
+ *    and destroyed from different threads: every entry point that submits work holds one process-wide lock until its
+ *    results are back, because a batch-1 step occupies every compute unit with one launch and must not share them.
+ *    sl_head_argmax_noalloc only enqueues on the caller's stream and is outside that lock: its caller keeps it from
+ *    overlapping other calls on the same GPU.  A second process on the same GPU is not supported.
+ *  - After sl_destroy(e) returns, e is invalid for every call, sl_fault included, also when lanes created from e
+ *    keep its weights alive for a while; no lane can be created from an engine that has been destroyed.
  *  - Weights are MLX-affine 4-bit, group 64 along K: w = scale*q + bias, q packed 8 per
  *    little-endian uint32, nibble j of a word is (word >> 4*j) & 15 (SeedlessMetalForward.swift
  *    :171-174); scales/biases are fp16 [N, K/64].
@@ -356,7 +360,10 @@ int sl_set_persistent(sl_engine* e, int enable);
 /* forwardRowsHybrid (SeedlessFusedVerify.swift:4240-4247): while enabled, calls with 16 <= m <= 2048 rows of one
  * sequence (prefill chunks) compute the dense mixer projections (GDN in/out, attention q|k|v and o) on the matrix
  * cores, the routed experts grouped by expert (steelMoEGather, SeedlessFusedVerify.swift:4174) with weights
- * dequantised to half, and the attention tile pass (scores, probabilities in half, values).  Like the reference's matrix-unit prefill this is not bit-identical to
+ * dequantised to half, the attention tile pass (scores, probabilities in half, values) and, when the router and
+ * shared-gate rows are fp16, their logits as one fp16 GEMM (with 8-bit gates they stay on the exact rows): an expert
+ * whose logit is within fp16 noise of the eighth largest may then be chosen differently from the exact path.
+ * Like the reference's matrix-unit prefill this is not bit-identical to
  * the GEMV order (tolerance-level agreement) but deterministic.  Calls whose row count and start position are multiples
  * of 64 also run the recurrence of the GDN layers block-wise on the matrix cores (the chunked form of the delta rule);
  * a prompt's rows do not depend on how it is cut into such calls, nor on how it is cut into other calls, but the two
@@ -381,6 +388,14 @@ int sl_stage_clock_words(void);
  * the kernel ends normally and the step returns SL_ERR_DEVICE (sticky).  The engine's default is 2^19 rounds, about
  * half a second; 0 makes the first unanswered poll give up.  No kernel is made to fault or hang. */
 int sl_debug_set_spin_limit(sl_engine* e, unsigned rounds);
+/* Test hooks for the tags of the single-launch step (no counterpart in the reference, whose stages are separated by
+ * command-buffer order).  Values exchanged between workgroups carry a counter of stage instances, 8 * (layers + 1) per
+ * step; before a launch that would take it past 0x7ff00000 the library clears its exchange buffers and restarts the
+ * counter, so an engine can step indefinitely.  sl_debug_set_flow_counter moves the counter (to step an engine across
+ * that point in a test); sl_debug_flow_tags evaluates, without a device, the 16-bit and 32-bit tags of (layer, stage)
+ * at counter value `base` and returns 1 if a launch of `steps` steps from `base` is preceded by a restart, else 0. */
+int sl_debug_set_flow_counter(sl_engine* e, uint32_t value);
+int sl_debug_flow_tags(uint32_t base, int layer, int stage, int steps, int n_layers, uint32_t* tag16, uint32_t* tag32);
 
 /* Per-kernel timing in the manner of forwardRowsProfiled (SFV:4352): while enabled, every launch of
  * the dominant kernel (the persistent step kernel, or lm_head in the kernel-per-stage sequence) is bracketed by HIP events on the engine's stream; the read call returns the

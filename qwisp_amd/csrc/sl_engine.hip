@@ -57,10 +57,13 @@ constexpr int MAX_CHAIN = 256;
 constexpr int ROUTER_PAD_ROWS = 288;
 
 // The single-launch step is a grid of workgroups that wait for each other's results without a grid barrier: it
-// only makes progress when all of them are resident at once.  One such launch fills the machine, so two of them
-// (two engines or lanes driven from two host threads) must never overlap: from launch to read-back a step holds
-// this process-wide lock.
-std::mutex g_flow_mutex;
+// only makes progress when all of them are resident at once, so nothing else of this process may occupy compute
+// units while it runs (another engine's step, a lane batch, a prefill chunk).  Every entry point that submits work
+// and waits for it holds this process-wide lock from its first launch to its read-back; it is recursive because the
+// lane entry points fall back to the single-engine ones.  (sl_head_argmax_noalloc, which only enqueues on the
+// caller's stream, is outside it: its caller keeps it apart from single-launch steps.)
+std::recursive_mutex g_gpu_mutex;
+#define SL_ENTER(e) std::lock_guard<std::recursive_mutex> gpu_lock_(g_gpu_mutex); int r = guard(e); if (r) return r
 std::atomic<uint64_t> g_engine_uid{1};
 
 // ---- scratch of the entry point that allocates nothing (sl_head_argmax_noalloc) --------------------------------
@@ -103,7 +106,7 @@ struct sl_engine {
   uint64_t uid = g_engine_uid.fetch_add(1);   // never reused: identifies an engine in another engine's lane table
   // lanes keep their base alive: a base destroyed while lanes exist is only marked, and goes with its last lane
   sl_engine* base_of = nullptr;
-  int lane_refs = 0;
+  std::atomic<int> lane_refs{0};
   bool destroy_pending = false;
   int n_layers = 0, n_experts = 0, vocab = 0, max_m = 0, max_seq = 0, max_tiles = 0;
   int normed_rows = 0;             // final-normed rows of the last forward still held in `normed` (0 after a step)
@@ -136,6 +139,8 @@ struct sl_engine {
   int dec_grid = 0;                // 0 = not available (fewer than 256 compute units)
   FlowP* flow_params = nullptr;    // device copy of the single-launch step's parameters
   FlowP flow_host;
+  uint32_t flow_base = 0;                                   // host mirror of the device's stage-instance counter
+  std::vector<std::pair<void*, size_t>> flow_tagged;        // the tagged exchange buffers (cleared when the counter is rebased)
   void* pinned = nullptr;        // host staging
   size_t pinned_bytes = 0;
   // host mirrors of the device step state
@@ -284,8 +289,10 @@ int finish(sl_engine* e, const char* what) {
 }
 
 // ---- launch sequences -------------------------------------------------------------------------------
-// Hybrid prefill: router and shared-gate logits stay on the exact GEMV rows (routing decides which experts run);
-// the shared expert and the routed experts, grouped by expert, go to the matrix cores.
+// Hybrid prefill: the shared expert and the routed experts, grouped by expert, go to the matrix cores.  So do the
+// router and shared-gate logits when the gates are fp16 rows (one fp16 GEMM, k_router_mfma: another accumulation
+// order than the exact rows, so an expert whose logit is within fp16 noise of the eighth may be chosen differently);
+// 8-bit gates keep the exact rows of k_moe_a.
 void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   const int E = e->n_experts;
   MoeAArgs a{};
@@ -548,7 +555,22 @@ void launch_head(sl_engine* e, int M, const HiddenArgs& ha, int out_off, bool fe
 }
 // `steps` batch-1 steps in a single persistent launch (each token fed back on the device); host mirrors advance
 // as the kernel's own update does.
+// The step kernel tags what it exchanges with a counter of stage instances that it advances by 8 * (layers + 1) per
+// step (sl_flow.cuh).  Attention partials carry 31 bits of it and their slots are not rewritten every step, so the
+// counter must never wrap while a stale slot could still hold the equal tag of 2^31 instances earlier.  It does not
+// get there: before a launch that would take the counter past FLOW_BASE_LIMIT the host clears every tagged buffer
+// (tag 0 is never expected: expected tags have their top bit set) and starts the counter again at 0.
+constexpr uint32_t FLOW_BASE_LIMIT = 0x7ff00000u;
+bool flow_rebase_needed(uint32_t base, int steps, int n_layers) {
+  return (uint64_t)base + (uint64_t)(steps + 1) * (uint64_t)(n_layers + 1) * 8u > (uint64_t)FLOW_BASE_LIMIT;
+}
 void launch_decode(sl_engine* e, int out_off, bool feed, int steps) {
+  if (flow_rebase_needed(e->flow_base, steps, e->n_layers)) {
+    for (const auto& b : e->flow_tagged) (void)hipMemsetAsync(b.first, 0, b.second, e->stream);
+    (void)hipMemsetAsync(e->dec_bar + 16, 0, 4, e->stream);
+    e->flow_base = 0;
+  }
+  e->flow_base += (uint32_t)steps * (uint32_t)(e->n_layers + 1) * 8u;
   const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
   auto kern = e->gate8 ? (e->stage_clock ? k_decode_flow<true, true> : k_decode_flow<true, false>)
@@ -795,13 +817,19 @@ int alloc_runtime(sl_engine* e) {
         FlowP F;
         std::memset(&F, 0, sizeof(F));
         F.d = P;
-        F.tproj = dalloc<uint32_t>(e, PROJ_STRIDE, true); F.tycore = dalloc<uint32_t>(e, 4096, true);
-        F.tmix = dalloc<uint32_t>(e, H, true); F.trlog = dalloc<uint32_t>(e, 256, true); F.tsg = dalloc<uint32_t>(e, 4, true);
-        F.tsh = dalloc<uint32_t>(e, 512, true); F.tact = dalloc<uint32_t>(e, 8 * 512, true); F.tmoe = dalloc<uint32_t>(e, H, true);
-        F.tml = dalloc<uint4>(e, (size_t)SL_ATT_HEADS * e->max_tiles, true);
-        F.tpo = dalloc<uint4>(e, (size_t)SL_ATT_HEADS * e->max_tiles * 128, true);
-        F.tcand = dalloc<uint4>(e, 256, true);
-        F.ttok = dalloc<uint4>(e, 4, true);
+        auto tagged_words = [&](size_t n) {
+          uint32_t* p = dalloc<uint32_t>(e, n, true);
+          e->flow_tagged.emplace_back(p, n * sizeof(uint32_t));
+          return p;
+        };
+        auto tagged_chunks = [&](size_t n) { return reinterpret_cast<uint4*>(tagged_words(4 * n)); };
+        F.tproj = tagged_words(PROJ_STRIDE); F.tycore = tagged_words(4096);
+        F.tmix = tagged_words(H); F.trlog = tagged_words(256); F.tsg = tagged_words(4);
+        F.tsh = tagged_words(512); F.tact = tagged_words(8 * 512); F.tmoe = tagged_words(H);
+        F.tml = tagged_chunks((size_t)SL_ATT_HEADS * e->max_tiles);
+        F.tpo = tagged_chunks((size_t)SL_ATT_HEADS * e->max_tiles * 128);
+        F.tcand = tagged_chunks(256);
+        F.ttok = tagged_chunks(4);
         F.sdpa_round = SDPA_ROUND;
         F.spin_limit = FLOW_SPIN_LIMIT;
         if (const char* s = std::getenv("QWISP_SDPA_ROUND")) {      // smaller rounds, for tests of the round loop
@@ -836,6 +864,11 @@ int alloc_runtime(sl_engine* e) {
 int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine** out) {
   if (!base || !out || max_m < 1 || max_seq_len < 1) return SL_ERR_ARG;
   if (!base->fault.empty()) return SL_ERR_POISONED;
+  {
+    const sl_engine* root = base->base_of ? base->base_of : base;       // (a lane of a lane hangs on the root's weights)
+    if (root->destroy_pending || !root->fault.empty()) return SL_ERR_POISONED;
+  }
+  std::lock_guard<std::recursive_mutex> gpu_lock_(g_gpu_mutex);
   sl_engine* e = new sl_engine();
   *out = e;
   e->n_layers = base->n_layers; e->n_experts = base->n_experts; e->vocab = base->vocab;
@@ -904,6 +937,7 @@ int bind_lanes(sl_engine* d, sl_engine** lanes, int b) {
 // steps are queued back to back.
 int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t* out) {
   if (!lanes || b < 1 || !tokens || !out) return SL_ERR_ARG;
+  std::lock_guard<std::recursive_mutex> gpu_lock_(g_gpu_mutex);
   for (int i = 0; i < b; ++i) {
     if (!lanes[i]) return SL_ERR_ARG;
     for (int j = 0; j < i; ++j) if (lanes[j] == lanes[i]) return SL_ERR_ARG;
@@ -952,12 +986,13 @@ int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t
 // Sampling is outside this build (greedy only); Tell falls back to its own sampler on "unsupported".
 int sl_step_sample_rows(sl_engine* e, const int32_t* tokens, int m, float temperature, float top_p, uint64_t seed, int32_t* out) {
   (void)tokens; (void)m; (void)temperature; (void)top_p; (void)seed; (void)out;
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   return SL_ERR_UNSUPPORTED;
 }
 
 void sl_destroy(sl_engine* e) {
   if (!e) return;
+  std::lock_guard<std::recursive_mutex> gpu_lock_(g_gpu_mutex);
   if (e->lane_refs > 0) {            // lanes still read these weights: the memory goes with the last of them
     if (e->stream) (void)hipStreamSynchronize(e->stream);
     e->destroy_pending = true;
@@ -983,7 +1018,7 @@ int sl_max_rows(const sl_engine* e) { return e ? e->max_m : -1; }
 float sl_last_gpu_ms(const sl_engine* e) { return e ? e->last_ms : 0.0f; }
 void* sl_stream(sl_engine* e) { return e ? (void*)e->stream : nullptr; }
 int sl_set_hybrid(sl_engine* e, int enable) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (enable && !e->hy_sg) {
     const size_t rows = (size_t)(e->max_m < GROUP_CAP ? e->max_m : GROUP_CAP);
     if (!e->hy_d) e->hy_d = dalloc<uint16_t>(e, rows * 8 * H);        // (engines of 128 rows or more have these two already)
@@ -1001,7 +1036,7 @@ int sl_set_hybrid(sl_engine* e, int enable) {
   return SL_OK;
 }
 int sl_set_persistent(sl_engine* e, int enable) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   e->use_persistent = enable != 0;
   return SL_OK;
 }
@@ -1009,7 +1044,7 @@ int sl_set_persistent(sl_engine* e, int enable) {
 // workgroup records 100 MHz clock stamps of the last step of a launch; the call copies them out,
 // out[wg * sl_stage_clock_words() + (layer * 8 + stage) * 8 + kind] (0 = not reached).
 int sl_debug_stage_clock(sl_engine* e, int enable, uint32_t* out, int cap_words) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!e->flow_params) return SL_ERR_UNSUPPORTED;
   if (out && cap_words > 0) {
     const size_t n = std::min<size_t>((size_t)cap_words, (size_t)e->dec_grid * STAMP_WORDS);
@@ -1023,13 +1058,28 @@ int sl_stage_clock_words(void) { return STAMP_WORDS; }
 // single-launch step stops waiting, raises the abort word and leaves (every workgroup then does the same at its next
 // wait, so the kernel ends normally).  0 makes the first unanswered poll give up.
 int sl_debug_set_spin_limit(sl_engine* e, unsigned rounds) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!e->flow_params) return SL_ERR_UNSUPPORTED;
   e->flow_host.spin_limit = rounds;
   return copy_sync(e, e->flow_params, &e->flow_host, sizeof(FlowP), hipMemcpyHostToDevice);
 }
+// Test hook: moves the stage-instance counter (device word and host mirror) so that a test can step an engine across
+// the point where the counter is rebased without running millions of steps first.
+int sl_debug_set_flow_counter(sl_engine* e, uint32_t value) {
+  SL_ENTER(e);
+  if (!e->flow_params) return SL_ERR_UNSUPPORTED;
+  e->flow_base = value;
+  return copy_sync(e, e->dec_bar + 16, &value, 4, hipMemcpyHostToDevice);
+}
+// The tags of stage instance (layer, stage) at counter value `base`, and whether a launch of `steps` steps from there
+// is preceded by a rebase: pure functions of their arguments (no device needed).
+int sl_debug_flow_tags(uint32_t base, int layer, int stage, int steps, int n_layers, uint32_t* tag16, uint32_t* tag32) {
+  if (tag16) *tag16 = flow_tag(base, layer, stage);
+  if (tag32) *tag32 = flow_tag32(base, layer, stage);
+  return flow_rebase_needed(base, steps, n_layers) ? 1 : 0;
+}
 int sl_profile_head(sl_engine* e, int enable) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (enable && e->head_ev.empty()) {
     e->head_ev.resize(2 * MAX_CHAIN, nullptr);
     for (auto& ev : e->head_ev) SL_TRY(e, hipEventCreate(&ev));
@@ -1070,16 +1120,14 @@ static void time_end(sl_engine* e) {
 }
 
 int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   e->normed_rows = 0;
   e->logits_view = e->normed_view = nullptr;
-  if (!tokens || !e->has_head) return SL_ERR_ARG;
+  if (!tokens || !out || !e->has_head) return SL_ERR_ARG;
   r = check_rows(e, m); if (r) return r;
   for (int i = 0; i < m; ++i) if (tokens[i] < 0 || tokens[i] >= e->vocab) return SL_ERR_ARG;
   r = to_device(e, e->tok_in, tokens, (size_t)m * 4); if (r) return r;
   const bool persistent = (m == 1 && e->dec_grid > 0 && e->use_persistent);
-  std::unique_lock<std::mutex> flow_lock(g_flow_mutex, std::defer_lock);
-  if (persistent) flow_lock.lock();
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   if (persistent) {
     launch_decode(e, 0, false, 1);
@@ -1097,15 +1145,13 @@ int sl_step_argmax(sl_engine* e, const int32_t* tokens, int m, int32_t* out) {
 }
 
 int sl_chained_step_argmax(sl_engine* e, int32_t first, int k, int32_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   e->normed_rows = 0;
   e->logits_view = e->normed_view = nullptr;
   if (!out || !e->has_head || k < 1 || k > MAX_CHAIN || first < 0 || first >= e->vocab) return SL_ERR_ARG;
   if (e->has_attn && e->pos + k > e->max_seq) return SL_ERR_ARG;
   r = to_device(e, e->tok_in, &first, 4); if (r) return r;
   const bool persistent = (e->dec_grid > 0 && e->use_persistent);
-  std::unique_lock<std::mutex> flow_lock(g_flow_mutex, std::defer_lock);
-  if (persistent) flow_lock.lock();
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
   if (persistent) launch_decode(e, 0, true, k);        // the whole chain in one launch
   for (int s = 0; s < k && !persistent; ++s) {
@@ -1139,14 +1185,14 @@ static int forward_common(sl_engine* e, int m, int final_norm, uint16_t* out, co
   return SL_OK;
 }
 int sl_forward_rows(sl_engine* e, const uint16_t* x, int m, int final_norm, uint16_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!x || !out || (final_norm && !e->final_norm)) return SL_ERR_ARG;
   r = check_rows(e, m); if (r) return r;
   r = to_device(e, e->hA, x, (size_t)m * H * 2); if (r) return r;
   return forward_common(e, m, final_norm, out, "forwardRows");
 }
 int sl_forward_tokens(sl_engine* e, const int32_t* tokens, int m, uint16_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!tokens || !e->has_head) return SL_ERR_ARG;
   r = check_rows(e, m); if (r) return r;
   for (int i = 0; i < m; ++i) if (tokens[i] < 0 || tokens[i] >= e->vocab) return SL_ERR_ARG;
@@ -1155,7 +1201,7 @@ int sl_forward_tokens(sl_engine* e, const int32_t* tokens, int m, uint16_t* out)
   return forward_common(e, m, 1, out, "forward");
 }
 int sl_hidden_rows(sl_engine* e, int m, uint16_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!out || m < 1 || m > e->max_m) return SL_ERR_ARG;
   if (e->normed_view) {   // after a lane-batched step: this lane's one row, held by the driver
     if (m != 1) return SL_ERR_ARG;
@@ -1164,7 +1210,7 @@ int sl_hidden_rows(sl_engine* e, int m, uint16_t* out) {
   return read_back(e, out, e->normed, (size_t)m * H * 2, "hiddenRows");
 }
 int sl_logits_row(sl_engine* e, int m, uint16_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!out || !e->has_head || m < 0 || m >= e->max_m) return SL_ERR_ARG;
   if (e->logits_view && m != 0) return SL_ERR_ARG;   // after a lane-batched step a lane has one row
   const uint16_t* src = e->logits_view ? e->logits_view : e->logits + (size_t)m * e->vocab;
@@ -1172,7 +1218,7 @@ int sl_logits_row(sl_engine* e, int m, uint16_t* out) {
   return r;
 }
 int sl_head_argmax(sl_engine* e, const uint16_t* normed, int m, int32_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!normed || !out || !e->has_head || m < 1 || m > e->max_m) return SL_ERR_ARG;
   e->logits_view = e->normed_view = nullptr;      // the logits this call leaves are the engine's own rows
   r = to_device(e, e->xn, normed, (size_t)m * H * 2); if (r) return r;
@@ -1184,7 +1230,7 @@ int sl_head_argmax(sl_engine* e, const uint16_t* normed, int m, int32_t* out) {
 // lm_head + arg-max of rows first .. first + m - 1 of the normed rows that the last sl_forward_tokens / sl_forward_rows
 // (with final norm) left on the device: the first token after a prefill without the rows' trip to the host and back.
 int sl_head_argmax_rows(sl_engine* e, int first, int m, int32_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!out || !e->has_head || m < 1 || first < 0 || first + m > e->normed_rows) return SL_ERR_ARG;
   e->logits_view = e->normed_view = nullptr;
   HiddenArgs ha{e->normed + (size_t)first * H, nullptr, nullptr, nullptr, nullptr};
@@ -1203,6 +1249,7 @@ int sl_head_argmax_noalloc(sl_engine* e, const uint16_t* normed_dev, int m, int3
   if (m > NA_MAX_ROWS || e->vocab > NA_MAX_VOCAB) return SL_ERR_TOO_LARGE;
   if (!e->na_scratch) return SL_ERR_DEVICE;
   hipStream_t st = (hipStream_t)stream;
+  (void)hipGetLastError();            // an error an unrelated earlier call of this thread left behind is not this call's
   uint16_t* logits = reinterpret_cast<uint16_t*>(e->na_scratch);
   float* cand_v = reinterpret_cast<float*>(static_cast<unsigned char*>(e->na_scratch) + NA_LOGITS_BYTES);
   int32_t* cand_i = reinterpret_cast<int32_t*>(cand_v + NA_CAND);
@@ -1219,20 +1266,20 @@ int sl_head_argmax_noalloc(sl_engine* e, const uint16_t* normed_dev, int m, int3
 }
 
 int sl_snapshot(sl_engine* e, sl_snap* s) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!s) return SL_ERR_ARG;
   s->kv_len = e->pos; s->reserved = 0;
   return SL_OK;
 }
 int sl_rollback_one_step(sl_engine* e, const sl_snap* s) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!s || s->kv_len < 0 || s->kv_len > e->pos) return SL_ERR_ARG;
   e->pos = s->kv_len;
   for (int i = 0; i < e->n_layers; ++i) if (e->layers[i].is_linear) e->parity[i] ^= 1;
   return push_state(e);
 }
 int sl_reset(sl_engine* e) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   for (LayerDev& L : e->layers) {
     if (!L.is_linear) continue;
     for (int p = 0; p < 2; ++p) {
@@ -1246,7 +1293,7 @@ int sl_reset(sl_engine* e) {
   return push_state(e);
 }
 int sl_full_snapshot(sl_engine* e, sl_full_snap** out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!out) return SL_ERR_ARG;
   sl_full_snap* s = new sl_full_snap();
   s->pos = e->pos;
@@ -1264,7 +1311,7 @@ int sl_full_snapshot(sl_engine* e, sl_full_snap** out) {
   return SL_OK;
 }
 int sl_full_restore(sl_engine* e, const sl_full_snap* s) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!s || (int)s->hist.size() != e->n_layers) return SL_ERR_ARG;
   for (int i = 0; i < e->n_layers; ++i) {
     LayerDev& L = e->layers[i];
@@ -1298,7 +1345,7 @@ size_t sl_persist_size(sl_engine* e) {
   return n;
 }
 int sl_persist_write(sl_engine* e, void* dst, size_t cap) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!dst || cap < sl_persist_size(e)) return SL_ERR_ARG;
   uint8_t* p = (uint8_t*)dst;
   auto u32 = [&](uint32_t v) { std::memcpy(p, &v, 4); p += 4; };
@@ -1325,7 +1372,7 @@ int sl_persist_write(sl_engine* e, void* dst, size_t cap) {
   return SL_OK;
 }
 int sl_persist_restore(sl_engine* e, const void* src, size_t len) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!src) return SL_ERR_ARG;
   const uint8_t* p = (const uint8_t*)src;
   const uint8_t* end = p + len;
@@ -1364,7 +1411,7 @@ int sl_persist_restore(sl_engine* e, const void* src, size_t len) {
 }
 
 int sl_read_layer_cache(sl_engine* e, int layer, void* a, void* b) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (layer < 0 || layer >= e->n_layers) return SL_ERR_ARG;
   LayerDev& L = e->layers[layer];
   if (L.is_linear) {
@@ -1380,7 +1427,7 @@ int sl_read_layer_cache(sl_engine* e, int layer, void* a, void* b) {
   return SL_OK;
 }
 int sl_load_layer_cache(sl_engine* e, int layer, const void* a, const void* b, int len) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (layer < 0 || layer >= e->n_layers) return SL_ERR_ARG;
   LayerDev& L = e->layers[layer];
   if (L.is_linear) {
@@ -1399,7 +1446,7 @@ int sl_load_layer_cache(sl_engine* e, int layer, const void* a, const void* b, i
 }
 
 int sl_read_route(sl_engine* e, int layer, int m, int32_t* inds, uint16_t* scores) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (layer < 0 || layer >= e->n_layers || m < 1 || m > e->max_m) return SL_ERR_ARG;
   if (inds) { r = copy_sync(e, inds, e->layers[layer].route_inds, (size_t)m * 32, hipMemcpyDeviceToHost); if (r) return r; }
   if (scores) { r = copy_sync(e, scores, e->layers[layer].route_scores, (size_t)m * 16, hipMemcpyDeviceToHost); if (r) return r; }
@@ -1408,7 +1455,7 @@ int sl_read_route(sl_engine* e, int layer, int m, int32_t* inds, uint16_t* score
 
 // ---- per-block entry points -----------------------------------------------------------------------
 int sl_moe_block_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!x || !out || layer < 0 || layer >= e->n_layers || m < 1 || m > e->max_m) return SL_ERR_ARG;
   r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
@@ -1420,7 +1467,7 @@ int sl_moe_block_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_
   return SL_OK;
 }
 int sl_gdn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!x || !out || layer < 0 || layer >= e->n_layers || m < 1 || m > e->max_m || !e->layers[layer].is_linear) return SL_ERR_ARG;
   r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
@@ -1433,7 +1480,7 @@ int sl_gdn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_
   return push_state(e);
 }
 int sl_attn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!x || !out || layer < 0 || layer >= e->n_layers || e->layers[layer].is_linear) return SL_ERR_ARG;
   r = check_rows(e, m); if (r) return r;
   r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
@@ -1449,7 +1496,7 @@ int sl_attn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16
 
 // Test hook: copy `count` fp16 elements of one internal scratch buffer of the last launch sequence.
 int sl_debug_scratch(sl_engine* e, int which, uint16_t* out, size_t count) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   const uint16_t* src = nullptr;
   switch (which) {
     case 0: src = e->proj; break;
@@ -1468,7 +1515,7 @@ int sl_debug_scratch(sl_engine* e, int which, uint16_t* out, size_t count) {
 }
 
 int sl_greedy_generate(sl_engine* e, const int32_t* prompt, int n_prompt, int n_new, int chain_k, int32_t* out) {
-  int r = guard(e); if (r) return r;
+  SL_ENTER(e);
   if (!prompt || n_prompt < 1 || n_new < 0 || (n_new > 0 && !out) || !e->has_head) return SL_ERR_ARG;
   if (chain_k < 1) chain_k = 1;
   if (chain_k > MAX_CHAIN) chain_k = MAX_CHAIN;

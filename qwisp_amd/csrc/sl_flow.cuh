@@ -84,11 +84,17 @@ SL_DEV int fresh_s(int x) { asm volatile("" : "+s"(x)); return x; }
 enum { FS_IN = 0, FS_CORE = 1, FS_MERGE = 2, FS_OUT = 3, FS_A = 4, FS_B = 5, FS_C = 6 };
 constexpr unsigned FLOW_SPIN_LIMIT = 1u << 19;
 
-// `base` counts stage instances over all launches (32 bits, advanced by 8*(layers+1) per launch).
-SL_DEV uint32_t flow_tag(uint32_t base, int layer, int stage) { return 0x8000u | ((base + (uint32_t)(layer * 8 + stage)) & 0x7fffu); }
+// `base` counts stage instances over all launches (advanced by 8*(layers+1) per step).  The 16-bit tags keep 15 bits
+// of it: every slot that carries one is rewritten by the stage instance that a consumer expects before that consumer
+// polls it, at most one step (8*(layers+1) < 2^15 instances) after its previous writer, so an equal tag always means
+// the expected writer.  The 32-bit tags keep 31 bits, and their slots may stay untouched for any number of steps; the
+// host therefore never lets the counter reach 2^31: before the launch that would, it clears every exchange buffer and
+// restarts the counter at 0 (launch_decode in sl_engine.hip).
+#define SL_HD __host__ __device__ __forceinline__
+SL_HD uint32_t flow_tag(uint32_t base, int layer, int stage) { return 0x8000u | ((base + (uint32_t)(layer * 8 + stage)) & 0x7fffu); }
 // 16-byte chunks carry the whole counter: their slots are not rewritten every layer (a key tile beyond
 // the current position keeps what an earlier, longer sequence left there).
-SL_DEV uint32_t flow_tag32(uint32_t base, int layer, int stage) { return 0x80000000u | (base + (uint32_t)(layer * 8 + stage)); }
+SL_HD uint32_t flow_tag32(uint32_t base, int layer, int stage) { return 0x80000000u | (base + (uint32_t)(layer * 8 + stage)); }
 SL_DEV uint32_t tagged(float v, uint32_t tag) { return (uint32_t)f2h(v) | (tag << 16); }
 SL_DEV bool tag_ok(uint32_t w, uint32_t tag) { return (w >> 16) == tag; }
 

@@ -126,3 +126,52 @@ def test_engine_needs_the_gpu():
     from qwisp_amd.engine import SeedlessFusedForward
     with pytest.raises(lib.SeedlessError):
         SeedlessFusedForward(cfg, t, max_m=1, max_seq_len=8)
+
+
+def test_step_kernel_tags_never_meet_across_the_counter_restart():
+    """The single-launch step tags what it exchanges with a counter of stage instances.  The 32-bit tags keep 31 bits
+    of it, so the host restarts the counter before it gets near 2^31.  Checked here without a device: for any counter
+    value from which a launch is NOT preceded by a restart, every tag of that launch is below the wrap (top bit set,
+    strictly increasing with the instance, no carry into the top bit), and from the restart limit on a restart is
+    always announced; 16-bit tags of the instances of one step (the farthest a slot's writer can be from its reader)
+    are pairwise distinct."""
+    L = lib.get()
+    t16, t32 = C.c_uint32(), C.c_uint32()
+
+    def tags(base, layer, stage, steps=1, n_layers=40):
+        r = L.dll.sl_debug_flow_tags(base, layer, stage, steps, n_layers, C.byref(t16), C.byref(t32))
+        return r, t16.value, t32.value
+
+    n_layers, per_step = 40, 8 * 41
+    rng = np.random.default_rng(5)
+    limit = 0x7FF00000
+    bases = [0, 1, per_step, 0x7FFF, 0x8000, 0x12345678] + [int(b) for b in rng.integers(0, limit, 200)]
+    # the last counter values from which launches of 1 and of 256 steps still run without a restart
+    for steps in (1, 8, 256):
+        last = limit - (steps + 1) * per_step
+        bases += [last - 1, last]
+        assert tags(last, 0, 0, steps)[0] == 0 and tags(last + 1, 0, 0, steps)[0] == 1
+        assert tags(0xFFFFFFFF, 0, 0, steps)[0] == 1 and tags(0x80000000, 0, 0, steps)[0] == 1
+    for base in bases:
+        for steps in (1, 256):
+            restart, _, _ = tags(base, 0, 0, steps)
+            if restart:
+                continue
+            # first and last stage instance the launch touches (the token hand-over of the step after the last uses
+            # stage 7 of layer 0 at the next step's base)
+            first = tags(base, 0, 0, steps)[2]
+            end_base = base + steps * per_step
+            last = tags(end_base, 0, 7, steps)[2]
+            assert first == (0x80000000 | base) and last == (0x80000000 | (end_base + 7))
+            assert end_base + per_step < 2 ** 31, "no carry into the tag's top bit"
+            assert last > first
+    # 16-bit tags: the instances of two consecutive steps never share a tag, and the top bit is always set
+    for base in (0, 0x7FF0, 0x7FFF, 0x8000, limit - 3 * per_step):
+        seen = {}
+        for step in range(2):
+            for layer in range(n_layers + 1):
+                for stage in range(8):
+                    t = tags(base + step * per_step, layer, stage)[1]
+                    assert t & 0x8000 and t < 0x10000
+                    assert t not in seen, (base, step, layer, stage, seen[t])
+                    seen[t] = (step, layer, stage)

@@ -827,6 +827,24 @@ def test_argument_errors_and_fault_firewall(env, small_model):
     assert eng.step_argmax([cfg.vocab]) is None and eng.gpu_fault is None      # token out of range
     assert eng.step_argmax([1, 2]) is not None
     assert eng.chained_step_argmax(3, 7) is None and eng.gpu_fault is None     # would overflow the arena
+    # a NULL result pointer is refused before anything is launched: position and caches stay where they were
+    import ctypes as C
+    dll, pos0 = env["lib"].dll, eng.position
+    tok = np.array([1, 2], np.int32)
+    tp = tok.ctypes.data_as(C.c_void_p)
+    xp = xrows(1, 3).ctypes.data_as(C.c_void_p)
+    for m in (1, 2):                                                           # the single-launch step and the row path
+        assert dll.sl_step_argmax(eng.h, tp, m, None) == abi.SL_ERR_ARG
+    assert dll.sl_step_argmax(eng.h, None, 1, tp) == abi.SL_ERR_ARG
+    assert dll.sl_chained_step_argmax(eng.h, 1, 2, None) == abi.SL_ERR_ARG
+    assert dll.sl_head_argmax(eng.h, xp, 1, None) == abi.SL_ERR_ARG
+    assert dll.sl_head_argmax_rows(eng.h, 0, 1, None) == abi.SL_ERR_ARG
+    assert dll.sl_forward_rows(eng.h, xp, 1, 0, None) == abi.SL_ERR_ARG
+    assert dll.sl_hidden_rows(eng.h, 1, None) == abi.SL_ERR_ARG
+    assert dll.sl_logits_row(eng.h, 0, None) == abi.SL_ERR_ARG
+    arr = (C.c_void_p * 1)(eng.h)
+    assert dll.sl_lane_step_argmax(arr, 1, tp, None) == abi.SL_ERR_ARG
+    assert eng.position == pos0 and eng.gpu_fault is None
     ok = eng.step_argmax([5])
     assert ok is not None
     eng.inject_failure()
@@ -888,6 +906,34 @@ def test_single_launch_step_gives_up_reports_and_poisons(env, small_model):
     eng.close(); other.close()
 
 
+def test_single_launch_steps_across_the_tag_counter_restart(env, small_model):
+    """The counter of stage instances that tags the step kernel's exchanges is restarted (exchange buffers cleared)
+    before it can reach 2^31: an engine moved to just below that point gives the stream of a fresh engine, through the
+    restart and after it, with attention partials of an earlier, longer sequence still sitting in their slots."""
+    cfg, dev, host = small_model
+    ref, eng = env["Engine"](cfg, dev, max_m=1, max_seq_len=400), env["Engine"](cfg, dev, max_m=1, max_seq_len=400)
+    dll = env["lib"].dll
+    per_step = 8 * (cfg.n_layers + 1)
+
+    def stream(e, n_chains, first=17):
+        toks, cur = [], first
+        for _ in range(n_chains):
+            o = e.chained_step_argmax(cur, 8)
+            assert o is not None, e.gpu_fault
+            toks += o.tolist(); cur = int(o[-1])
+        return toks
+    want = stream(ref, 40)                                   # 320 steps: five key tiles
+    long_first = stream(eng, 40)                             # leaves tagged partials of five tiles behind
+    assert long_first == want
+    for e in (ref, eng):
+        assert dll.sl_reset(e.h) == abi.SL_OK
+    want = stream(ref, 12)
+    # 29 steps below the limit: the restart comes before the fourth chain
+    assert dll.sl_debug_set_flow_counter(eng.h, 0x7FF00000 - 29 * per_step) == abi.SL_OK
+    assert stream(eng, 12) == want
+    ref.close(); eng.close()
+
+
 def test_lanes_outlive_their_base_and_two_threads_drive_two_engines(env, small_model):
     import threading
     cfg, dev, host = small_model
@@ -895,7 +941,13 @@ def test_lanes_outlive_their_base_and_two_threads_drive_two_engines(env, small_m
     lane = base.new_lane(max_m=4, max_seq_len=96)
     solo = env["Engine"](cfg, dev, max_m=4, max_seq_len=96)
     assert lane.max_m == 4 and lane.max_seq_len == 96
+    import ctypes as C
+    base_h = base.h
     base.close()                                  # the weights stay until the last lane is gone
+    # ... but no further lane can be attached, neither to the destroyed engine nor through one of its lanes
+    late = C.c_void_p()
+    assert env["lib"].dll.sl_lane_create(lane.h, 1, 32, C.byref(late)) == abi.SL_ERR_POISONED
+    del base_h
     prompt = [3, 1415, 926, 535]
     a, b = lane.greedy_generate(prompt, 6), solo.greedy_generate(prompt, 6)
     assert a is not None and a.tolist() == b.tolist()
@@ -923,5 +975,26 @@ def test_lanes_outlive_their_base_and_two_threads_drive_two_engines(env, small_m
         o = ref.chained_step_argmax(cur, 8); want += o.tolist(); cur = int(o[-1])
     assert out["a"] == want, out["a"]
     assert isinstance(out["b"], list) and len(out["b"]) == 96
-    for e in (lane, solo, e1, e2, ref):
+    # a single-launch step needs every compute unit: steps of several rows on another engine (kernel-per-stage launches)
+    # driven from a second thread take turns with it as well
+    e3, e4 = env["Engine"](cfg, dev, max_m=1, max_seq_len=160), env["Engine"](cfg, dev, max_m=4, max_seq_len=160)
+    out.clear()
+
+    def run_rows(name, e):
+        toks = []
+        for i in range(24):
+            o = e.step_argmax([5 + i, 6, 7, 8])
+            if o is None:
+                out[name] = e.gpu_fault
+                return
+            toks += o.tolist()
+        out[name] = toks
+    th = [threading.Thread(target=run, args=("a", e3, 11)), threading.Thread(target=run_rows, args=("rows", e4))]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    assert out["a"] == want, out["a"]
+    assert isinstance(out["rows"], list) and len(out["rows"]) == 96, out["rows"]
+    for e in (lane, solo, e1, e2, e3, e4, ref):
         e.close()

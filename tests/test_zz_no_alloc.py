@@ -50,4 +50,37 @@ def test_head_argmax_without_allocation_equals_head_argmax():
     assert L.dll.sl_head_argmax_noalloc(eng.h, C.c_void_p(xd.data_ptr()), 9, C.c_void_p(od.data_ptr()), C.c_void_p(stream)) == abi.SL_ERR_TOO_LARGE
     assert L.dll.sl_head_argmax_noalloc(eng.h, None, 1, C.c_void_p(od.data_ptr()), C.c_void_p(stream)) == abi.SL_ERR_ARG
     assert eng.gpu_fault is None and eng.head_argmax(np.zeros((1, abi.H), np.float16)) is not None
+
+    # It allocates nothing: the device's free memory is the same before and after a series of calls ...
+    x = np.random.default_rng(7).normal(0, 1, (6, abi.H)).astype(np.float16)
+    want = eng.head_argmax(x)
+    xd = torch.from_numpy(x).cuda()
+    od = torch.full((8,), -1, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for m in (6, 2, 1, 6):
+        assert L.dll.sl_head_argmax_noalloc(eng.h, C.c_void_p(xd.data_ptr()), m, C.c_void_p(od.data_ptr()), C.c_void_p(stream)) == abi.SL_OK
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    assert od.cpu().numpy()[:6].tolist() == want.tolist()
+    # ... and it neither allocates, copies nor synchronises: a stream capture, which fails on any of those, records it,
+    # and every replay of the graph (with eager work and synchronisations between the replays) gives the eager result
+    g = torch.cuda.CUDAGraph()
+    od.fill_(-1)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g):
+        cap = torch.cuda.current_stream().cuda_stream
+        st = L.dll.sl_head_argmax_noalloc(eng.h, C.c_void_p(xd.data_ptr()), 6, C.c_void_p(od.data_ptr()), C.c_void_p(cap))
+    assert st == abi.SL_OK
+    for rep in range(3):
+        xr = np.random.default_rng(100 + rep).normal(0, 1, (6, abi.H)).astype(np.float16)
+        want = eng.head_argmax(xr)                         # eager work of the library between the replays
+        xd.copy_(torch.from_numpy(xr))
+        od.fill_(-1)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert od.cpu().numpy()[:6].tolist() == want.tolist(), rep
+    assert eng.gpu_fault is None
     eng.close()
