@@ -146,6 +146,41 @@ def block_benchmarks(eng, cfg, np, torch):
     return rep
 
 
+def microbench(L):
+    """The three machine limits the design notes quote, measured by the library's own micro-benchmark kernels
+    (qwisp_amd/csrc/sl_ubench.hip); every figure is the best of three runs."""
+    import ctypes as C
+    f, g = C.c_float(), C.c_float()
+
+    def best(call, pick=min):
+        vals = []
+        for _ in range(3):
+            r = call()
+            assert r == 0, f"micro-benchmark failed with status {r}"
+            vals.append((f.value, g.value))
+        return pick(vals)
+    ex = {}
+    for mode, name in ((0, "allgather_2048_words_barrier_per_round"), (1, "allgather_2048_words_one_barrier"),
+                       (2, "allgather_2048_words_every_thread_its_pair"), (3, "256_words_among_32_workgroups_of_one_xcd"),
+                       (4, "256_words_among_32_workgroups_across_xcds")):
+        ex[name] = round(best(lambda: L.dll.sl_ubench_exchange(mode, 2008, C.byref(f)))[0], 3)
+    gm = {}
+    for mode, name in ((0, "loads_only"), (1, "with_dot"), (2, "with_dot_and_row_reduction")):
+        for grid in (256, 512):
+            gm[f"{name}_grid{grid}"] = round(best(lambda: L.dll.sl_ubench_gemv_stream(mode, grid, C.byref(f)), max)[0], 3)
+    mf = {}
+    for wps in (1, 2):
+        for lds in (0, 1):
+            for valu in (0, 1, 2, 4, 8):
+                if lds and valu > 2:
+                    continue
+                t = best(lambda: L.dll.sl_ubench_mfma_issue(valu, lds, wps, C.byref(f), C.byref(g)), max)
+                mf[f"valu_steps{valu}_lds{lds}_waves{wps}"] = {"tflops": round(t[0], 1), "ns_per_mfma_per_simd": round(t[1], 2)}
+    return {"microbench": {"exchange_us_per_dependent_round": ex, "gemv_stream_tb_per_s": gm, "mfma_issue": mf,
+                           "notes": "exchange: 256 workgroups x 1024 threads, 2000 dependent rounds; gemv: 2.4 GB of K = 2048 "
+                                    "4-bit rows; mfma: v_mfma_f32_32x32x16_f16, a valu step = 3 vector instructions on a half pair"}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -182,6 +217,10 @@ def main():
                          "object in the JSON line; empty = skip)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run a plain device copy of this many MiB (reference for rocprofv3 FETCH_SIZE/WRITE_SIZE) and exit")
+    ap.add_argument("--microbench", type=int, default=0,
+                    help="only run the library's micro-benchmarks of the machine limits that bound the kernels (dependent "
+                         "hand-over between 256 resident workgroups, 4-bit row streaming through the dot, issue cost of vector "
+                         "instructions beside matrix instructions), print their figures as one JSON line and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
@@ -202,6 +241,9 @@ def main():
         return
     from qwisp_amd import lib, synth
     from qwisp_amd.engine import SeedlessFusedForward
+    if args.microbench:
+        print(json.dumps(microbench(lib.get())))
+        return
 
     cfg = synth.ModelConfig(n_layers=args.layers)
     t0 = time.time()

@@ -397,6 +397,22 @@ int sl_debug_set_spin_limit(sl_engine* e, unsigned rounds);
 int sl_debug_set_flow_counter(sl_engine* e, uint32_t value);
 int sl_debug_flow_tags(uint32_t base, int layer, int stage, int steps, int n_layers, uint32_t* tag16, uint32_t* tag32);
 
+/* Micro-benchmarks of the machine limits that bound the kernels (measurement hooks; no counterpart in the reference).
+ * Each runs on the current device's default stream, allocates and frees its own buffers and returns one figure.
+ *  sl_ubench_exchange: a chain of `rounds` dependent hand-overs between the 256 resident workgroups of a persistent
+ *    launch (every wait bounded), microseconds per round.  mode 0: all-gather of 2048 tagged words, eight waves poll,
+ *    one barrier per polling round; 1: the same with one barrier per hand-over; 2: every thread polls the two words it
+ *    owns, one barrier per hand-over (the step kernel's form); 3: 256 words among the 32 workgroups of one XCD;
+ *    4: 256 words among 32 workgroups spread over the XCDs.  SL_ERR_UNSUPPORTED on a part with fewer than 256 CUs.
+ *  sl_ubench_gemv_stream: 2.4 GB of 4-bit rows (K = 2048) streamed through `grid` workgroups of 16 waves, TB/s.
+ *    mode 0: loads only; 1: with the step kernel's dot; 2: with the dot and the 64-lane reduction per row.
+ *  sl_ubench_mfma_issue: v_mfma_f32_32x32x16_f16 with `valu_steps` (0..8) unpacking steps of three vector instructions
+ *    and optionally one 16-byte LDS operand read per matrix instruction, 1 or 2 waves per SIMD: TFLOP/s of the whole
+ *    chip and nanoseconds per matrix instruction and SIMD. */
+int sl_ubench_exchange(int mode, int rounds, float* us_per_round);
+int sl_ubench_gemv_stream(int mode, int grid, float* tb_per_s);
+int sl_ubench_mfma_issue(int valu_steps, int lds_read, int waves_per_simd, float* tflops, float* ns_per_mfma);
+
 /* Per-kernel timing in the manner of forwardRowsProfiled (SFV:4352): while enabled, every launch of
  * the dominant kernel (the persistent step kernel, or lm_head in the kernel-per-stage sequence) is bracketed by HIP events on the engine's stream; the read call returns the
  * summed duration and the number of launches since it was enabled. */

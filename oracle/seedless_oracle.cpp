@@ -8,9 +8,9 @@
 // exp/log/sin/cos — is fixed here ("canonical order"); the HIP kernels implement the same order,
 // so indices, tokens, hidden states and caches compare bit-for-bit.
 //
-// Canonical reductions (one rule everywhere): a reduction over n values is a balanced binary
-// tree over 64 (or fewer) "lane" partials, adjacent lanes paired first; a lane partial is a
-// left-to-right fmaf chain over the contiguous elements the lane owns.
+// Canonical reductions: a reduction over n values is a balanced binary tree over 64 (or fewer)
+// "lane" partials, adjacent lanes paired first; what a lane partial is (fmaf chains over the
+// elements the lane owns, or a sub-tree) is stated per function below.
 //
 // PARITY PINNING: the reference ships no golden vectors for this path (its tests derive inputs
 // from MLXRandom at run time) and none of its code can be built here (Swift + MLX + Metal), so
@@ -37,49 +37,74 @@ constexpr int SDPA_TILE = 64;
 
 // ------------------------------------------------------------------------------------------------
 // 4-bit GEMV.  Reference: qmm4 (SeedlessMetalForward.swift:238-310): y[n] = sum_k x[k]*(s*q+b),
-// evaluated per word of 8 nibbles as s*sum(x*q) + b*sum(x), fp32 accumulate, fp16 result.
-// Canonical order: word term t = fmaf(s, dq, b*sx), dq = fmaf chain over the word's 8 nibbles,
-// sx = left-to-right sum of the 8 x; lane l of L = min(64, K/32) owns words 4l..4l+3 of every
-// block of 4L words and accumulates ((t0+t1)+(t2+t3)) block after block; lanes are tree-summed.
+// evaluated as s*sum(x*q) + b*sum(x) per run of weights that share one (s, b), fp32 accumulate,
+// fp16 result.
+// Canonical order: a "share" is 32 consecutive elements (4 packed words, half a quantisation
+// group, so one scale and one bias).  Its term is T = fmaf(s, dq, b*sx) with
+//   dq = A + B, A = fmaf chain over the share's even-indexed elements in order, B = the same over
+//        the odd-indexed ones (two chains: on the device the even and odd nibbles of a word are
+//        isolated by different masks and meet only here),
+//   sx = balanced binary tree over the 16 pair sums x[2i] + x[2i+1], adjacent pairs first.
+// Lane l of L = min(64, K/32) owns share l of every block of L shares and adds its terms block
+// after block; the lanes are tree-summed.
 // ------------------------------------------------------------------------------------------------
 struct XPrep {
-  int K = 0, W = 0;
-  std::vector<float> xt;   // xt[i*W + w] = x[8w+i]
-  std::vector<float> sx;   // per word
+  int K = 0, S = 0;
+  std::vector<float> xe, xo;   // even / odd elements, xe[i*S + sh] = x[32 sh + 2i], xo[...] = x[32 sh + 2i + 1]
+  std::vector<float> sx;       // per share
   void set(const float* x, int k) {
-    K = k; W = k / 8;
-    xt.resize((size_t)8 * W); sx.resize(W);
-    for (int w = 0; w < W; ++w) {
-      float s = 0.0f;
-      for (int i = 0; i < 8; ++i) { float v = x[8 * w + i]; xt[(size_t)i * W + w] = v; s = s + v; }
-      sx[w] = s;
+    K = k; S = k / 32;
+    xe.resize((size_t)16 * S); xo.resize((size_t)16 * S); sx.resize(S);
+    for (int sh = 0; sh < S; ++sh) {
+      float ps[16];
+      for (int i = 0; i < 16; ++i) {
+        const float a = x[32 * sh + 2 * i], b = x[32 * sh + 2 * i + 1];
+        xe[(size_t)i * S + sh] = a; xo[(size_t)i * S + sh] = b; ps[i] = a + b;
+      }
+      sx[sh] = tree_sum(ps, 16);
     }
   }
 };
 
 static float qdot(const XPrep& xp, const uint32_t* wrow, const uint16_t* srow, const uint16_t* brow) {
-  const int W = xp.W;
-  float t[512];
-  for (int w0 = 0; w0 < W; w0 += 8) {
-    float dq[8];
-    for (int j = 0; j < 8; ++j) dq[j] = 0.0f;
-    for (int i = 0; i < 8; ++i) {
-      const float* xr = &xp.xt[(size_t)i * W + w0];
-      for (int j = 0; j < 8; ++j)
-        dq[j] = std::fmaf(xr[j], (float)((wrow[w0 + j] >> (4 * i)) & 15u), dq[j]);
+  const int S = xp.S;
+  float t[128];
+  for (int s0 = 0; s0 < S; s0 += 8) {          // eight shares at a time (the loops over j vectorise)
+    const int nb = std::min(8, S - s0);
+    float A[8], B[8];
+    uint32_t wt[4][8];                         // word wd of share j
+    for (int j = 0; j < 8; ++j) {
+      A[j] = 0.0f; B[j] = 0.0f;
+      for (int wd = 0; wd < 4; ++wd) wt[wd][j] = j < nb ? wrow[4 * (s0 + j) + wd] : 0u;
     }
-    const float s = h2f(srow[w0 / 8]), b = h2f(brow[w0 / 8]);
-    for (int j = 0; j < 8; ++j) t[w0 + j] = std::fmaf(s, dq[j], b * xp.sx[w0 + j]);
+    if (nb == 8) {
+      for (int i = 0; i < 16; ++i) {           // pair i of a share: nibbles 2(i%4), 2(i%4)+1 of its word i/4
+        const float* xe = &xp.xe[(size_t)i * S + s0];
+        const float* xo = &xp.xo[(size_t)i * S + s0];
+        const uint32_t* wv = wt[i >> 2];
+        const int sh = 8 * (i & 3);
+        for (int j = 0; j < 8; ++j) {
+          A[j] = std::fmaf(xe[j], (float)((wv[j] >> sh) & 15u), A[j]);
+          B[j] = std::fmaf(xo[j], (float)((wv[j] >> (sh + 4)) & 15u), B[j]);
+        }
+      }
+    } else {
+      for (int i = 0; i < 16; ++i)
+        for (int j = 0; j < nb; ++j) {
+          A[j] = std::fmaf(xp.xe[(size_t)i * S + s0 + j], (float)((wt[i >> 2][j] >> (8 * (i & 3))) & 15u), A[j]);
+          B[j] = std::fmaf(xp.xo[(size_t)i * S + s0 + j], (float)((wt[i >> 2][j] >> (8 * (i & 3) + 4)) & 15u), B[j]);
+        }
+    }
+    for (int j = 0; j < nb; ++j) {
+      const float sc = h2f(srow[(s0 + j) / 2]), bi = h2f(brow[(s0 + j) / 2]);
+      t[s0 + j] = std::fmaf(sc, A[j] + B[j], bi * xp.sx[s0 + j]);
+    }
   }
-  const int L = std::min(64, W / 4), nblk = W / (4 * L);
+  const int L = std::min(64, S), nblk = S / L;
   float p[64];
   for (int l = 0; l < L; ++l) {
-    float acc = 0.0f;
-    for (int blk = 0; blk < nblk; ++blk) {
-      const float* tw = &t[blk * 4 * L + 4 * l];
-      float v = (tw[0] + tw[1]) + (tw[2] + tw[3]);
-      acc = (blk == 0) ? v : (acc + v);
-    }
+    float acc = t[l];
+    for (int blk = 1; blk < nblk; ++blk) acc = acc + t[blk * L + l];
     p[l] = acc;
   }
   return tree_sum(p, L);
@@ -89,6 +114,7 @@ static float qdot(const XPrep& xp, const uint32_t* wrow, const uint16_t* srow, c
 static void qmv(const float* x, const sl_q4& q, int row0, int nrows, float* y) {
   XPrep xp; xp.set(x, q.k);
   const int W = q.k / 8, G = q.k / 64;
+  if (q.k % 64 != 0 || q.k > 4096) { std::fprintf(stderr, "oracle qmv: K = %d is not a multiple of 64 up to 4096\n", q.k); std::abort(); }
 #pragma omp parallel for schedule(static)
   for (int n = 0; n < nrows; ++n) {
     size_t r = (size_t)row0 + n;
@@ -130,16 +156,13 @@ static float q8_dot(const float* x, const uint32_t* wrow, const uint16_t* srow, 
   return tree_sum(p, 64);
 }
 
-// Sum of squares over D (a multiple of 64) values.
+// Sum of squares over D values (D/2 a power of two): pair terms fmaf(x1, x1, x0*x0), then a balanced binary tree
+// over the D/2 pair terms, adjacent ones first.  (Any split of the vector into aligned power-of-two blocks reduces
+// in this order: a lane that owns 32 elements, a wave of 64 pairs, 16 waves.)
 static float sumsq(const float* x, int D) {
-  const int per = D / 64;
-  float p[64];
-  for (int l = 0; l < 64; ++l) {
-    float acc = 0.0f;
-    for (int i = 0; i < per; ++i) acc = std::fmaf(x[l * per + i], x[l * per + i], acc);
-    p[l] = acc;
-  }
-  return tree_sum(p, 64);
+  std::vector<float> p((size_t)D / 2);
+  for (int i = 0; i < D / 2; ++i) p[i] = std::fmaf(x[2 * i + 1], x[2 * i + 1], x[2 * i] * x[2 * i]);
+  return tree_sum(p.data(), D / 2);
 }
 static inline float inv_rms(const float* x, int D) { return 1.0f / std::sqrt(sumsq(x, D) / (float)D + EPS); }
 
@@ -346,8 +369,9 @@ static void gdn_layer_rows(Engine& e, int li, const float* x, int M, float* out)
 //     SeedlessMetalForward.swift:4922-4989 (q pre-scaled by 1/16, fp32 softmax, fp16 out);
 //     output gate: SeedlessMetalForward.swift:1012-1022.
 // Canonical softmax order: keys in tiles of 64 aligned at absolute positions; per tile exact max,
-// p = exp(s - max), l = tree over the 64 p, o = fmaf chain over keys; tiles merged in order with
-// the global max: L = sum l_t*f_t, O = sum o_t*f_t as fmaf chains, out = half(O/L).
+// p = exp(s - max), l = tree over the 64 p, o = (fmaf chain over keys 0..31) + (fmaf chain over keys
+// 32..63); tiles merged in order with the global max: L = sum l_t*f_t, O = sum o_t*f_t as fmaf
+// chains, out = half(O/L).
 static void build_rope(Engine& e) {
   e.ropeCos.resize((size_t)e.maxSeq * 32); e.ropeSin.resize((size_t)e.maxSeq * 32);
   for (int i = 0; i < 32; ++i) {
@@ -371,14 +395,16 @@ static void norm_rope(const Engine& e, const float* x, const uint16_t* w, int po
     out[d] = (d < 32) ? f16r(std::fmaf(-x1, s[i], x0 * c[i])) : f16r(std::fmaf(x1, c[i], x0 * s[i]));
   }
 }
+// Score of one key: eight fmaf chains over 32 consecutive dims each, combined by a balanced tree (on the device a
+// lane owns a key and a chain is the unit of work a wave can take).
 static float dot256(const float* q, const uint16_t* k) {
-  float p[64];
-  for (int l = 0; l < 64; ++l) {
+  float c[8];
+  for (int j = 0; j < 8; ++j) {
     float acc = 0.0f;
-    for (int i = 0; i < 4; ++i) acc = std::fmaf(q[4 * l + i], h2f(k[4 * l + i]), acc);
-    p[l] = acc;
+    for (int i = 0; i < 32; ++i) acc = std::fmaf(q[32 * j + i], h2f(k[32 * j + i]), acc);
+    c[j] = acc;
   }
-  return tree_sum(p, 64);
+  return tree_sum(c, 8);
 }
 static void sdpa_row(const float* qrot /*[HD]*/, const uint16_t* kc, const uint16_t* vc, int N, float* out /*[HD]*/) {
   float q[HD];
@@ -391,12 +417,16 @@ static void sdpa_row(const float* qrot /*[HD]*/, const uint16_t* kc, const uint1
     float mx = -INFINITY;
     for (int j = 0; j < nk; ++j) { s[j] = dot256(q, kc + (size_t)(j0 + j) * HD); mx = std::fmax(mx, s[j]); }
     for (int j = 0; j < SDPA_TILE; ++j) p[j] = (j < nk) ? exp_c(s[j] - mx) : 0.0f;
+    // weighted value sum of the tile: one fmaf chain over its first 32 keys, one over the other 32, added
     float* o = &to[(size_t)t * HD];
-    for (int d = 0; d < HD; ++d) o[d] = 0.0f;
+    float ob[HD];
+    for (int d = 0; d < HD; ++d) { o[d] = 0.0f; ob[d] = 0.0f; }
     for (int j = 0; j < nk; ++j) {
       const uint16_t* vr = vc + (size_t)(j0 + j) * HD;
-      for (int d = 0; d < HD; ++d) o[d] = std::fmaf(p[j], h2f(vr[d]), o[d]);
+      float* dst = j < SDPA_TILE / 2 ? o : ob;
+      for (int d = 0; d < HD; ++d) dst[d] = std::fmaf(p[j], h2f(vr[d]), dst[d]);
     }
+    for (int d = 0; d < HD; ++d) o[d] = o[d] + ob[d];
     tm[t] = mx; tl[t] = tree_sum(p, SDPA_TILE);
   }
   float Mx = -INFINITY;

@@ -99,11 +99,11 @@ SL_DEV void st_co_h4(rsrc_t r, int idx, const float* x) {
 }
 
 // ---- activation vector in LDS ------------------------------------------------------------------------
-// Packed pair i (elements 2i, 2i+1) of lane l of block b lives at xs[(16*b + i)*64 + l]; word sums at
-// sxs[(4*b + j)*64 + l].
+// Packed pair i (elements 2i, 2i+1) of lane l of block b lives at xs[(16*b + i)*64 + l]; the sum of the lane's share
+// of 32 elements at sxs[64*b + l].
 struct Lds {
   union {                                    // the staged key tile is only live while xs is not
-    struct { uint32_t xs[2048]; float sxs[512]; };
+    struct { uint32_t xs[2048]; float sxs[128]; };
     uint16_t kt[SDPA_TILE * KT_STRIDE];
   };
   float red[64];
@@ -114,10 +114,10 @@ struct Lds {
   float dbuf[2 * 9 * 4];
   int pf[4];                                // poll outcome slots (three in rotation) and the give-up flag
   uint32_t pub[64];                         // a stage's tagged outputs, gathered for the publishing wave
-  float sq[8 * 256];                        // attention: scaled queries of one kv group
+  alignas(16) float sq[8 * 256];            // attention: scaled queries of one kv group (read back 16 bytes at a time)
   float knew[256], vnew[256];
-  float sm[8 * 64];                         // attention: per head softmax weights of the tile
-  float part[16 * 64];                      // attention: half-tree score partials; router: logits and exps
+  alignas(16) float sm[8 * 64];             // attention: per head softmax weights of the tile (read back 16 bytes at a time)
+  float part[16 * 64];                      // attention: score partials of the waves; router: logits and exps
 };
 __shared__ Lds g_L;
 extern __shared__ __align__(16) uint16_t g_vt[];   // dynamic: staged value tile [64][256] halves, then the softmax
@@ -125,19 +125,10 @@ extern __shared__ __align__(16) uint16_t g_vt[];   // dynamic: staged value tile
 constexpr int SDPA_ROUND = 20;
 constexpr int DEC_DYN_LDS = SDPA_TILE * 256 * 2 + SDPA_ROUND * 8 * 64 * 4;
 
-SL_DEV void lds_put_x(int b, int lane, const float* x) {
-#pragma unroll
-  for (int i = 0; i < 16; ++i) g_L.xs[(16 * b + i) * 64 + lane] = pack2(x[2 * i], x[2 * i + 1]);
-  float sx[4];
-  word_sums(x, sx);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) g_L.sxs[(4 * b + j) * 64 + lane] = sx[j];
-}
-SL_DEV void lds_get_x(int b, int lane, uint32_t* xp, float* sx) {
+SL_DEV void lds_get_x(int b, int lane, uint32_t* xp, float& sx) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) xp[i] = g_L.xs[(16 * b + i) * 64 + lane];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) sx[j] = g_L.sxs[(4 * b + j) * 64 + lane];
+  sx = g_L.sxs[64 * b + lane];
 }
 
 // ---- weight prefetch: R rows of K = 2048*NBLK held in registers ----------------------------------------
@@ -162,53 +153,26 @@ SL_DEV void wload_row(uint4* w, uint32_t* sb, const uint32_t* __restrict__ W, co
 }
 struct F4 { float v[4]; };
 struct F2 { float v[2]; };
-// The three dot shapes of a step, each compiled once (arguments travel in registers):
-// 4 rows x 2048, 2 rows x 2048, 1 row x 4096.
-SL_DEV F4 dot_1x4_(uint4 w0, uint4 w1, uint4 w2, uint4 w3, uint32_t s0, uint32_t s1, uint32_t s2, uint32_t s3) {
-  const int lane = threadIdx.x & 63;
-  uint32_t x[16]; float sx[4];
-  lds_get_x(0, lane, x, sx);
-  F4 o;
-  o.v[0] = tree_sum<64>(quad_term(w0, s0, x, sx));
-  o.v[1] = tree_sum<64>(quad_term(w1, s1, x, sx));
-  o.v[2] = tree_sum<64>(quad_term(w2, s2, x, sx));
-  o.v[3] = tree_sum<64>(quad_term(w3, s3, x, sx));
-  return o;
-}
+// Dot shapes of a step (arguments travel in registers): 2 rows x 2048, 1 row x 4096.
 SL_DEV F2 dot_1x2_(uint4 w0, uint4 w1, uint32_t s0, uint32_t s1) {
   const int lane = threadIdx.x & 63;
-  uint32_t x[16]; float sx[4];
+  uint32_t x[16]; float sx;
   lds_get_x(0, lane, x, sx);
   F2 o;
-  o.v[0] = tree_sum<64>(quad_term(w0, s0, x, sx));
-  o.v[1] = tree_sum<64>(quad_term(w1, s1, x, sx));
+  o.v[0] = tree_sum<64>(share_term(w0, s0, x, sx));
+  o.v[1] = tree_sum<64>(share_term(w1, s1, x, sx));
   return o;
 }
 SL_DEV float dot_2x1_(uint4 w0, uint4 w1, uint32_t s0, uint32_t s1) {
   const int lane = threadIdx.x & 63;
-  uint32_t x[16]; float sx[4];
+  uint32_t x[16]; float sx;
   lds_get_x(0, lane, x, sx);
-  float acc = quad_term(w0, s0, x, sx);
+  float acc = share_term(w0, s0, x, sx);
   lds_get_x(1, lane, x, sx);
-  acc = acc + quad_term(w1, s1, x, sx);
+  acc = acc + share_term(w1, s1, x, sx);
   return tree_sum<64>(acc);
 }
-SL_DEV F4 dot_1x4(const WRegs<1, 4>& r) { return dot_1x4_(r.w[0][0], r.w[1][0], r.w[2][0], r.w[3][0], r.sb[0][0], r.sb[1][0], r.sb[2][0], r.sb[3][0]); }
 SL_DEV F2 dot_1x2(const WRegs<1, 2>& r) { return dot_1x2_(r.w[0][0], r.w[1][0], r.sb[0][0], r.sb[1][0]); }
 SL_DEV float dot_2x1(const WRegs<2, 1>& r) { return dot_2x1_(r.w[0][0], r.w[0][1], r.sb[0][0], r.sb[0][1]); }
-
-// 8 leaves (32 dims) of the score tree of one key against one query head: balanced sub-tree.
-SL_DEV float score_leaf8(const uint16_t* kr, const float* qh) {
-  float n[8];
-#pragma unroll
-  for (int l = 0; l < 8; ++l) {
-    const uint2 kraw = *reinterpret_cast<const uint2*>(kr + 4 * l);
-    float node = fmaf(qh[4 * l], lo_h(kraw.x), 0.0f);
-    node = fmaf(qh[4 * l + 1], hi_h(kraw.x), node);
-    node = fmaf(qh[4 * l + 2], lo_h(kraw.y), node);
-    n[l] = fmaf(qh[4 * l + 3], hi_h(kraw.y), node);
-  }
-  return ((n[0] + n[1]) + (n[2] + n[3])) + ((n[4] + n[5]) + (n[6] + n[7]));
-}
 
 }  // namespace sl

@@ -2,9 +2,9 @@
 //
 // Every function here is built from IEEE binary32 +,-,*,/,sqrt, fmaf and integer operations only
 // and the translation unit is compiled with -ffp-contract=off, so results do not depend on how
-// a kernel is tiled.  Reductions follow one rule: lane partials are left-to-right fmaf chains
-// over contiguous elements, lanes are combined by an xor-butterfly (adjacent lanes first), which
-// is a balanced binary tree whose value is the same on every lane.
+// a kernel is tiled.  Reductions: lanes are combined by an xor-butterfly (adjacent lanes first), which
+// is a balanced binary tree whose value is the same on every lane; a lane partial is an fmaf chain over
+// elements the lane owns or a sub-tree of the same balanced tree, as stated where it is formed.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
@@ -222,59 +222,58 @@ SL_DEV uint4 pack8(const float* f) {
 template <class T>
 SL_DEV T* as_global(T* p) { return (T*)(T __attribute__((address_space(1)))*)(unsigned long long)p; }
 
-// ---- one packed word against 8 activations ---------------------------------------------------------
-// The 8 activations arrive as 4 packed half pairs.  Masking the word with 0x000F000F leaves two
-// halves whose bit patterns are the nibbles j and j+4: as (subnormal) half values they equal
-// q * 2^-24 exactly, so the products x*q*2^-24 and their fp32 fmaf chain are the chain of x*q scaled
-// by a power of two -- same rounding, no integer-to-float conversion.  The compiler folds the half
-// operands into v_fma_mix_f32.  The 2^24 is returned to the scale: t = fmaf(s*2^24, dq', b*sx).
+// ---- 4-bit dot: a share of 32 activations against 4 packed words ------------------------------------------
+// A share is 32 consecutive elements of a row: 4 packed words (one 16-byte load), half a quantisation group, so one
+// scale s and one bias b.  Its term is T = fmaf(s, A + B, b * sx), A the fmaf chain over the share's even-indexed
+// elements in order, B the chain over the odd-indexed ones, sx the balanced tree over the 16 pair sums.
+//
+// The activations arrive as 16 packed half pairs {x[2i], x[2i+1]}.  Masking a word with 0x000F000F leaves two halves
+// whose bit patterns are the nibbles 0 and 4: as (subnormal) half values they equal q * 2^-24 exactly; masking with
+// 0x00F000F0 leaves the nibbles 1 and 5 four bits up, q * 2^-20.  After one shift by 8 the same two masks give the
+// nibbles 2 | 6 and 3 | 7: five integer operations per word, no integer-to-float conversion, and the masked halves go
+// straight into v_fma_mix_f32.  Every product and partial sum of chain A is thereby the true one times 2^-24, of
+// chain B times 2^-20 (powers of two: same roundings), so A + B is formed as fmaf(B', 2^-4, A') and the 2^24 is
+// returned with the scale.
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 SL_DEV h2_t as_h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
-// The four masked forms of a word: mk[j] holds the nibbles j (low half) and j+4 (high half).
-// Nibbles 3 and 7 of a packed word, each at the bottom of its 16-bit half: (w >> 12) & 0x000F000F.  A packed 16-bit
-// shift needs no mask behind it (one instruction instead of two; the compiler does not find it by itself).  Used in
-// the dots of single rows; in the row-tiled kernels, which form the masks once per tile, it measured slower.
-typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
-SL_DEV uint32_t top_nibbles(uint32_t w) {
-  u16x2_t v = __builtin_bit_cast(u16x2_t, w);
-  v = v >> (u16x2_t)(12);
-  return __builtin_bit_cast(uint32_t, v);
-}
+// The four masked forms of a word: mk[0] nibbles 0 | 4, mk[1] nibbles 1 | 5 (x16), mk[2] nibbles 2 | 6, mk[3] nibbles 3 | 7 (x16).
 SL_DEV void word_masks(uint32_t w, h2_t* mk /*4*/) {
-  mk[0] = as_h2(w & 0x000F000Fu); mk[1] = as_h2((w >> 4) & 0x000F000Fu);
-  mk[2] = as_h2((w >> 8) & 0x000F000Fu); mk[3] = as_h2((w >> 12) & 0x000F000Fu);
+  const uint32_t w8 = w >> 8;
+  mk[0] = as_h2(w & 0x000F000Fu); mk[1] = as_h2(w & 0x00F000F0u);
+  mk[2] = as_h2(w8 & 0x000F000Fu); mk[3] = as_h2(w8 & 0x00F000F0u);
 }
-// word_dot with the masked forms prepared by the caller: the same chain
-SL_DEV float word_dot_masked(const h2_t* mk /*4*/, const uint32_t* xp /*4 packed pairs*/) {
+// One word's eight multiply-adds: elements 0, 2, 4, 6 onto chain A, elements 1, 3, 5, 7 onto chain B.
+SL_DEV void word_chains(const h2_t* mk /*4*/, const uint32_t* xp /*4 packed pairs*/, float& A, float& B) {
   const h2_t x0 = as_h2(xp[0]), x1 = as_h2(xp[1]), x2 = as_h2(xp[2]), x3 = as_h2(xp[3]);
-  float dq = 0.0f;
-  dq = fmaf((float)x0.x, (float)mk[0].x, dq);
-  dq = fmaf((float)x0.y, (float)mk[1].x, dq);
-  dq = fmaf((float)x1.x, (float)mk[2].x, dq);
-  dq = fmaf((float)x1.y, (float)mk[3].x, dq);
-  dq = fmaf((float)x2.x, (float)mk[0].y, dq);
-  dq = fmaf((float)x2.y, (float)mk[1].y, dq);
-  dq = fmaf((float)x3.x, (float)mk[2].y, dq);
-  dq = fmaf((float)x3.y, (float)mk[3].y, dq);
-  return dq;
+  A = fmaf((float)x0.x, (float)mk[0].x, A);
+  B = fmaf((float)x0.y, (float)mk[1].x, B);
+  A = fmaf((float)x1.x, (float)mk[2].x, A);
+  B = fmaf((float)x1.y, (float)mk[3].x, B);
+  A = fmaf((float)x2.x, (float)mk[0].y, A);
+  B = fmaf((float)x2.y, (float)mk[1].y, B);
+  A = fmaf((float)x3.x, (float)mk[2].y, A);
+  B = fmaf((float)x3.y, (float)mk[3].y, B);
 }
-// dq' = 2^-24 * (fmaf chain over the 8 nibbles, least significant first)
-SL_DEV float word_dot(uint32_t w, const uint32_t* xp /*4 packed pairs*/) {
-  const h2_t m0 = as_h2(w & 0x000F000Fu), m1 = as_h2((w >> 4) & 0x000F000Fu);
-  const h2_t m2 = as_h2((w >> 8) & 0x000F000Fu), m3 = as_h2(top_nibbles(w));
-  const h2_t x0 = as_h2(xp[0]), x1 = as_h2(xp[1]), x2 = as_h2(xp[2]), x3 = as_h2(xp[3]);
-  float dq = 0.0f;
-  dq = fmaf((float)x0.x, (float)m0.x, dq);
-  dq = fmaf((float)x0.y, (float)m1.x, dq);
-  dq = fmaf((float)x1.x, (float)m2.x, dq);
-  dq = fmaf((float)x1.y, (float)m3.x, dq);
-  dq = fmaf((float)x2.x, (float)m0.y, dq);
-  dq = fmaf((float)x2.y, (float)m1.y, dq);
-  dq = fmaf((float)x3.x, (float)m2.y, dq);
-  dq = fmaf((float)x3.y, (float)m3.y, dq);
-  return dq;
+// T of a share whose 16 masked forms the caller prepared (reused over several activation rows).
+SL_DEV float share_term_masked(const h2_t* mk /*16*/, uint32_t sb, const uint32_t* xp /*16 packed pairs*/, float sx) {
+  float A = 0.0f, B = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) word_chains(mk + 4 * j, xp + 4 * j, A, B);
+  const float s = lo_h(sb) * 16777216.0f, b = hi_h(sb);
+  return fmaf(s, fmaf(B, 0.0625f, A), b * sx);
 }
-// Four consecutive words of one group-half: t_j = fmaf(s, dq_j, b*sx_j); returns (t0+t1)+(t2+t3).
+SL_DEV float share_term(uint4 w, uint32_t sb, const uint32_t* xp /*16 packed pairs*/, float sx) {
+  const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+  float A = 0.0f, B = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    h2_t mk[4];
+    word_masks(ws[j], mk);
+    word_chains(mk, xp + 4 * j, A, B);
+  }
+  const float s = lo_h(sb) * 16777216.0f, b = hi_h(sb);
+  return fmaf(s, fmaf(B, 0.0625f, A), b * sx);
+}
 // 8-bit affine row dot, group 64 (the router gate and shared-expert gate of the released checkpoint; reference
 // kernel qmm8, SeedlessMetalForward.swift:372-428).  Lane l owns the 32 contiguous values 32l..32l+31 = 8 words,
 // half a group.  Per 8 values: t = fmaf(s, chain of fmaf(x, q), b * sx) with sx the sequential fp32 sum of the
@@ -295,37 +294,45 @@ SL_DEV float q8_lane(const uint32_t* w8 /*8 words*/, uint32_t sb, const float* x
   }
   return (t[0] + t[1]) + (t[2] + t[3]);
 }
-SL_DEV float quad_term(uint4 w, uint32_t sb, const uint32_t* xp /*16 packed pairs*/, const float* sx /*4*/) {
-  const float s = lo_h(sb) * 16777216.0f, b = hi_h(sb);
-  float t0 = fmaf(s, word_dot(w.x, xp), b * sx[0]);
-  float t1 = fmaf(s, word_dot(w.y, xp + 4), b * sx[1]);
-  float t2 = fmaf(s, word_dot(w.z, xp + 8), b * sx[2]);
-  float t3 = fmaf(s, word_dot(w.w, xp + 12), b * sx[3]);
-  return (t0 + t1) + (t2 + t3);
-}
-// quad_term with the 16 masked forms of the four words prepared by the caller (reused over several activation rows)
-SL_DEV float quad_term_masked(const h2_t* mk /*16*/, uint32_t sb, const uint32_t* xp, const float* sx) {
-  const float s = lo_h(sb) * 16777216.0f, b = hi_h(sb);
-  float t0 = fmaf(s, word_dot_masked(mk, xp), b * sx[0]);
-  float t1 = fmaf(s, word_dot_masked(mk + 4, xp + 4), b * sx[1]);
-  float t2 = fmaf(s, word_dot_masked(mk + 8, xp + 8), b * sx[2]);
-  float t3 = fmaf(s, word_dot_masked(mk + 12, xp + 12), b * sx[3]);
-  return (t0 + t1) + (t2 + t3);
-}
 // 32 half-valued floats -> 16 packed pairs (exact)
 SL_DEV void pack_x(const float* x, uint32_t* xp) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) xp[i] = pack2(x[2 * i], x[2 * i + 1]);
 }
-// Left-to-right sums of each run of 8 activations.
-SL_DEV void word_sums(const float* x /*32*/, float* sx /*4*/) {
+// Sum of a share's 32 activations: balanced tree over the 16 pair sums x[2i] + x[2i+1], adjacent pairs first.
+SL_DEV float share_sum(const float* x /*32*/) {
+  float p[16];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    float s = 0.0f;
+  for (int i = 0; i < 16; ++i) p[i] = x[2 * i] + x[2 * i + 1];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) s = s + x[8 * j + i];
-    sx[j] = s;
-  }
+  for (int st = 1; st < 16; st <<= 1)
+#pragma unroll
+    for (int i = 0; i < 16; i += 2 * st) p[i] = p[i] + p[i + st];
+  return p[0];
+}
+// The same from the packed pairs.
+SL_DEV float share_sum_packed(const uint32_t* xp /*16*/) {
+  float p[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) p[i] = lo_h(xp[i]) + hi_h(xp[i]);
+#pragma unroll
+  for (int st = 1; st < 16; st <<= 1)
+#pragma unroll
+    for (int i = 0; i < 16; i += 2 * st) p[i] = p[i] + p[i + st];
+  return p[0];
+}
+// Sum of squares of 32 consecutive elements as the sub-tree of the canonical order: pair terms fmaf(x1, x1, x0*x0),
+// then a balanced tree over the 16 of them.  (A sum of squares over D elements is the balanced binary tree over its
+// D/2 pair terms, adjacent ones first; lanes that own aligned runs of 32 elements continue it with tree_sum.)
+SL_DEV float share_sumsq(const float* x /*32*/) {
+  float p[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) p[i] = fmaf(x[2 * i + 1], x[2 * i + 1], x[2 * i] * x[2 * i]);
+#pragma unroll
+  for (int st = 1; st < 16; st <<= 1)
+#pragma unroll
+    for (int i = 0; i < 16; i += 2 * st) p[i] = p[i] + p[i + st];
+  return p[0];
 }
 
 // ---- counter-based generator (the same rule a host implementation can state) -----------------------

@@ -123,8 +123,8 @@ struct sl_engine {
   float *rope_cos = nullptr, *rope_sin = nullptr;
   // scratch
   uint16_t *hA = nullptr, *hB = nullptr, *proj = nullptr, *ycore = nullptr, *qrot = nullptr, *mix = nullptr, *xn = nullptr;
-  float* xsum = nullptr;           // [max_m, 256] word sums of the rows in xn (steps of two or more rows)
-  float* ysum = nullptr;           // [max_m, 512] word sums of the rows in ycore (gated mixer outputs) for the exact K = 4096 projection
+  float* xsum = nullptr;           // [max_m, 64] share sums of the rows in xn (steps of two or more rows)
+  float* ysum = nullptr;           // [max_m, 128] share sums of the rows in ycore (gated mixer outputs) for the exact K = 4096 projection
   uint16_t *rlogits = nullptr, *sgate = nullptr, *sh_act = nullptr, *act = nullptr, *moe_out = nullptr, *normed = nullptr;
   uint16_t *logits = nullptr, *rows_out = nullptr;
   float *pm = nullptr, *pl = nullptr, *po = nullptr, *cand_v = nullptr;
@@ -755,7 +755,7 @@ int alloc_runtime(sl_engine* e) {
   e->hA = dalloc<uint16_t>(e, MH, true); e->hB = dalloc<uint16_t>(e, MH, true);
   e->proj = dalloc<uint16_t>(e, (size_t)max_m * PROJ_STRIDE, true);
   e->ycore = dalloc<uint16_t>(e, (size_t)max_m * 4096, true);
-  e->mix = dalloc<uint16_t>(e, MH, true); e->xn = dalloc<uint16_t>(e, MH, true); e->xsum = dalloc<float>(e, (size_t)max_m * 256, true); e->ysum = dalloc<float>(e, (size_t)max_m * 512, true);
+  e->mix = dalloc<uint16_t>(e, MH, true); e->xn = dalloc<uint16_t>(e, MH, true); e->xsum = dalloc<float>(e, (size_t)max_m * 64, true); e->ysum = dalloc<float>(e, (size_t)max_m * 128, true);
   if (max_m >= MOE_GROUP_MIN_ROWS) {               // exact steps of many rows run the experts' down stage by expert: results by pair, then the combine
     const size_t rows = (size_t)(max_m < GROUP_CAP ? max_m : GROUP_CAP);
     e->hy_d = dalloc<uint16_t>(e, rows * 8 * H); e->hy_sy = dalloc<uint16_t>(e, rows * H);

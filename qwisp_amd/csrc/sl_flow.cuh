@@ -172,39 +172,22 @@ SL_DEV bool flow_poll(bool polls, Attempt attempt, unsigned* abort_word) {
 
 // Prologue on the whole workgroup: thread t owns elements 2t, 2t+1 of the hidden row and keeps them in
 // registers from stage to stage (every workgroup follows the whole residual stream, so it is never exchanged).
-//   h' = half(h + r) (returned in h0, h1); x = w * half(h' * inv_rms(h')) -> packed into LDS with the word sums.
-// Sum of squares keeps the canonical order: wave 0, lane l chains its 32 contiguous elements.
+//   h' = half(h + r) (returned in h0, h1); x = w * half(h' * inv_rms(h')) -> packed into LDS with the share sums.
+// Sum of squares in the canonical order (a balanced tree over the 1024 pair terms): every wave reduces its 64 pair
+// terms, the 16 wave sums meet in LDS, and every wave adds them up for itself, so one barrier is enough.
 SL_DEV void flow_prologue(float& h0, float& h1, bool has_r, float r0, float r1, uint32_t lnw_pair, uint16_t* xn_plain) {
   const int tid = fresh_v(threadIdx.x), lane = tid & 63, wave = tid >> 6;
-  uint32_t* hs = reinterpret_cast<uint32_t*>(g_L.sq);          // 1024 words of scratch (attention's query area)
   if (has_r) { h0 = f16r(h0 + r0); h1 = f16r(h1 + r1); }
-  hs[tid + (tid >> 4)] = pack2(h0, h1);       // 17-word lane stride: conflict-free for the chain below
+  const float ws = tree_sum<64>(fmaf(h1, h1, h0 * h0));
+  if (lane == 0) g_L.red[wave] = ws;
   lds_barrier();
-  if (wave == 0) {
-    float ss = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const uint32_t w = hs[17 * lane + i];
-      const float a = lo_h(w), b = hi_h(w);
-      ss = fmaf(a, a, ss);
-      ss = fmaf(b, b, ss);
-    }
-    ss = tree_sum<64>(ss);
-    if (lane == 0) g_L.gb[0] = 1.0f / sqrtf(ss / 2048.0f + EPS);
-  }
-  lds_barrier();
-  const float inv = g_L.gb[0];
+  const float ss = tree_sum<16>(g_L.red[lane & 15]);
+  const float inv = 1.0f / sqrtf(ss / 2048.0f + EPS);
   const float y0 = f16r(lo_h(lnw_pair) * f16r(h0 * inv)), y1 = f16r(hi_h(lnw_pair) * f16r(h1 * inv));
   g_L.xs[(tid & 15) * 64 + (tid >> 4)] = pack2(y0, y1);
-  // left-to-right sum over each word of 8 elements = 4 consecutive threads
-  const int q = tid & 3;
-  float s = (0.0f + y0) + y1;
-#pragma unroll
-  for (int r = 1; r < 4; ++r) {
-    const float v = prev_lane(s);
-    if (q == r) s = (v + y0) + y1;
-  }
-  if (q == 3) g_L.sxs[((tid & 15) >> 2) * 64 + (tid >> 4)] = s;
+  // a share of 32 elements = the pairs of 16 consecutive threads: balanced tree over the pair sums
+  const float s = tree_sum<16>(y0 + y1);
+  if ((tid & 15) == 0) g_L.sxs[tid >> 4] = s;
   if (xn_plain) *reinterpret_cast<uint32_t*>(xn_plain + 2 * tid) = pack2(y0, y1);
   lds_barrier();
 }
@@ -217,6 +200,33 @@ SL_DEV void flow_prologue(float& h0, float& h1, bool has_r, float r0, float r1, 
 constexpr int PUB_WAVE = DEC_WAVES - 1;
 constexpr int DENSE_WAVE0 = 128 * DEC_WAVES;     // first wave of the router rows (workgroup 128)
 constexpr int PAIR_WAVE0 = 160 * DEC_WAVES;      // first wave of the shared gate/up pairs (workgroups 160..191)
+
+// ---- weight rows parked in LDS ahead of their stage ------------------------------------------------------------
+// A stage that requests its weight rows when it starts has them in flight while it polls for its inputs: the polls
+// of a wave return behind its own loads, and a burst of 14 MB from all workgroups at once takes 2.5 us to arrive, so
+// the hand-over ends with the burst however early the inputs were published.  The rows that do not depend on the
+// routing and whose stage starts with a long hand-over therefore travel one to three stages ahead, straight into LDS
+// (global_load_lds_dwordx4: no registers are held meanwhile): the in-projection rows of layer l+1 are requested when
+// a workgroup is through with the K = 4096 projection of layer l (the upper half of the grid has no rows there and
+// starts at once), a GDN layer's out-projection rows when its in-projection is done.  The ring lies in the dynamic
+// LDS behind stage C's activation rows; only attention's tile stage uses that space otherwise, and no row is parked
+// across it.  A wave reads back only rows it requested itself, after waiting for its own loads (vmcnt).
+#ifndef SL_WRING
+#define SL_WRING 1
+#endif
+constexpr int WR_OFF = 12288;                    // bytes into g_vt (stage C's rows take 9 * 16 * XC_STRIDE words = 11520 bytes)
+constexpr int WR_SLOTS = DEC_WAVES * 3 + 1;      // three rows of 1 KB per wave, and the b / a row of a GDN in-projection
+static_assert(WR_OFF + WR_SLOTS * 1024 <= DEC_DYN_LDS, "the ring fits the dynamic LDS");
+SL_DEV void wr_request(int slot, const uint32_t* row_words, int lane) {
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  typedef const __attribute__((address_space(1))) void* glb_ptr;
+  __builtin_amdgcn_global_load_lds((glb_ptr)(row_words + 4 * lane), (lds_ptr)(reinterpret_cast<unsigned char*>(g_vt) + WR_OFF + slot * 1024), 16, 0, 0);
+}
+SL_DEV uint4 wr_read(int slot, int lane) {
+  return *reinterpret_cast<const uint4*>(reinterpret_cast<const unsigned char*>(g_vt) + WR_OFF + slot * 1024 + 16 * lane);
+}
+// Before a wave reads rows it requested: its loads have landed (the compiler does not know that they write LDS).
+SL_DEV void wr_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 #define FLOW_IDS const int tid = fresh_v(threadIdx.x), lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); \
                  const int wg = fresh_s(blockIdx.x), G = fresh_s(gridDim.x), NW = G * DEC_WAVES, gw = wg * DEC_WAVES + wave; \
@@ -296,7 +306,15 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   const InRows rows = in_rows(lin, wg, wave);
   WRegs<1, 3> wr;
 #pragma unroll
-  for (int j = 0; j < 3; ++j) wload_row<1>(wr.w[j], wr.sb[j], uni(Y.in_w), uni(Y.in_sb), (size_t)rows.crit[j], j < rows.ncrit, lane);
+  for (int j = 0; j < 3; ++j) {
+#if SL_WRING
+    // the rows themselves were requested into LDS stages ago (flow_request_in); only their scales and biases come now
+    wr.w[j][0] = make_uint4(0, 0, 0, 0);
+    wr.sb[j][0] = j < rows.ncrit ? uni(Y.in_sb)[(size_t)rows.crit[j] * 32 + (lane >> 1)] : 0u;
+#else
+    wload_row<1>(wr.w[j], wr.sb[j], uni(Y.in_w), uni(Y.in_sb), (size_t)rows.crit[j], j < rows.ncrit, lane);
+#endif
+  }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.input_ln) + 2 * tid);
   float r0 = 0.0f, r1 = 0.0f;
   if (li == 0) {
@@ -330,23 +348,35 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   }
   // the deferred row (no branch around the load: the waits that follow stay exact)
   uint4 wd; uint32_t sbd;
+#if SL_WRING
+  wd = make_uint4(0, 0, 0, 0);
+  sbd = uni(Y.in_sb)[(size_t)rows.def * 32 + (lane >> 1)];
+#else
   wload_row<1>(&wd, &sbd, uni(Y.in_w), uni(Y.in_sb), (size_t)rows.def, true, lane);
+#endif
   const uint32_t tin = flow_tag(base, li, FS_IN);
   flow_prologue(h0, h1, li > 0, r0, r1, lnw, nullptr);
   fstamp<ST>(li, FS_IN, 2, tid == 0);
-  uint32_t x[16]; float sx[4];
+  uint32_t x[16]; float sx;
   lds_get_x(0, lane, x, sx);
+#if SL_WRING
+  wr_wait();
+  wr.w[0][0] = wr_read(wave * 3, lane);
+  if (rows.ncrit >= 2) wr.w[1][0] = wr_read(wave * 3 + 1, lane);
+  if (rows.ncrit >= 3) wr.w[2][0] = wr_read(DEC_WAVES * 3, lane);
+  wd = wr_read(wave * 3 + 2, lane);
+#endif
   {
     // urgent rows: slot of row j = first slot of the wave + j (the extra b / a row: slot 32)
     const int slot0 = lin ? 2 * wave : (wave < 4 ? 2 * wave : 4 + wave);
-    const float o0 = tree_sum<64>(quad_term(wr.w[0][0], wr.sb[0][0], x, sx));
+    const float o0 = tree_sum<64>(share_term(wr.w[0][0], wr.sb[0][0], x, sx));
     if (lane == 0) g_L.pub[slot0] = tagged(o0, tin);
     if (rows.ncrit >= 2) {                // wave-uniform
-      const float o1 = tree_sum<64>(quad_term(wr.w[1][0], wr.sb[1][0], x, sx));
+      const float o1 = tree_sum<64>(share_term(wr.w[1][0], wr.sb[1][0], x, sx));
       if (lane == 0) g_L.pub[slot0 + 1] = tagged(o1, tin);
     }
     if (rows.ncrit >= 3) {
-      const float o2 = tree_sum<64>(quad_term(wr.w[2][0], wr.sb[2][0], x, sx));
+      const float o2 = tree_sum<64>(share_term(wr.w[2][0], wr.sb[2][0], x, sx));
       if (lane == 0) g_L.pub[32] = tagged(o2, tin);
     }
   }
@@ -363,7 +393,7 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   }
   fstamp<ST>(li, FS_IN, 4, tid == PUB_WAVE * 64);
   {
-    const float od = tree_sum<64>(quad_term(wd, sbd, x, sx));
+    const float od = tree_sum<64>(share_term(wd, sbd, x, sx));
     if (lane == 0) g_L.pub[40 + wave] = tagged(od, tin);
   }
   lds_barrier();
@@ -372,7 +402,30 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
     stw1(co_rsrc(uni(F.tproj)), lin ? 8192 + zi : attn_gate_row(zi), g_L.pub[40 + lane]);
   }
   fstamp<ST>(li, FS_IN, 5, tid == PUB_WAVE * 64);
+#if SL_WRING
+  // a GDN layer's K = 4096 projection row of this wave (2 KB) takes the places of the rows just used
+  if (lin && gw < H) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // (the rows just read are in registers)
+    wr_request(wave * 3, uni(Y.out_w) + (size_t)gw * 512, lane);
+    wr_request(wave * 3 + 1, uni(Y.out_w) + (size_t)gw * 512 + 256, lane);
+  }
+#endif
   return true;
+}
+// Requests the in-projection rows of layer Y for this wave into the ring (the rows in_rows() deals out).
+SL_DEV void flow_request_in(const LayerP& Y) {
+#if SL_WRING
+  FLOW_IDS;
+  const InRows rows = in_rows(uni(Y.is_linear) != 0, wg, wave);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // whatever this wave last read from its places is in registers
+  const uint32_t* W = uni(Y.in_w);
+  wr_request(wave * 3, W + (size_t)rows.crit[0] * 256, lane);
+  if (rows.ncrit >= 2) wr_request(wave * 3 + 1, W + (size_t)rows.crit[1] * 256, lane);
+  if (rows.ncrit >= 3) wr_request(DEC_WAVES * 3, W + (size_t)rows.crit[2] * 256, lane);
+  wr_request(wave * 3 + 2, W + (size_t)rows.def * 256, lane);
+#else
+  (void)Y;
+#endif
 }
 
 // ---- GDN stage 2: conv + prep + gated delta rule ------------------------------------------------------
@@ -538,6 +591,8 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       if (row < nk && j0 + row != pos) {
         if (keys) st16(&L.kt[row * KT_STRIDE + c8], kq[it]);
         if (values) st16(&g_vt[row * 256 + c8], vq[it]);
+      } else if (row >= nk && values) {
+        st16(&g_vt[row * 256 + c8], make_uint4(0, 0, 0, 0));       // weight 0 times value 0 leaves a sum as it is
       }
     }
   };
@@ -572,10 +627,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
           float wv[4];
           const uint2 wraw = *reinterpret_cast<const uint2*>(nwp + 4 * lane);
           wv[0] = lo_h(wraw.x); wv[1] = hi_h(wraw.x); wv[2] = lo_h(wraw.y); wv[3] = hi_h(wraw.y);
-          float ss = 0.0f;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) ss = fmaf(xv[i], xv[i], ss);
-          ss = tree_sum<64>(ss);
+          const float ss = tree_sum<64>(fmaf(xv[1], xv[1], xv[0] * xv[0]) + fmaf(xv[3], xv[3], xv[2] * xv[2]));
           const float inv = 1.0f / sqrtf(ss / 256.0f + EPS);
           float* dst = isq ? &L.sq[wave * 256] : L.knew;
 #pragma unroll
@@ -612,30 +664,28 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       else if (nr > 1) fetch(false, true, ub + GU);
       lds_barrier();
       {
-        // scores: wave (head, half) takes the 32 leaves of its half of the 256 dims, lane j is key j.  The 128
-        // query values sit two per lane and reach the multiply as scalar operands (readlane), so LDS only
-        // serves the key rows.
+        // scores: wave (head, half) takes four of the eight chains of 32 dims, lane j is key j; the queries come as
+        // LDS broadcasts (one 16-byte read per four multiply-adds), the key row from the staged tile
         const int h = wave >> 1, half = wave & 1;
         const uint16_t* kr = &L.kt[(lane < nk ? lane : 0) * KT_STRIDE + 128 * half];
-        const float qa = L.sq[h * 256 + 128 * half + lane], qb = L.sq[h * 256 + 128 * half + 64 + lane];
-        float g[4];
+        const float* qh = &L.sq[h * 256 + 128 * half];
+        // (the four chains advance side by side, four dims at a time)
+        float c[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int gi = 0; gi < 4; ++gi) {
-          float n[8];
+        for (int l = 0; l < 8; ++l) {
 #pragma unroll
-          for (int l = 0; l < 8; ++l) {
-            const int d = 32 * gi + 4 * l;                 // first dim of the leaf within the half
-            const float qv = d < 64 ? qa : qb;
+          for (int gi = 0; gi < 4; ++gi) {
+            const int d = 32 * gi + 4 * l;
             const uint2 kraw = *reinterpret_cast<const uint2*>(kr + d);
             const h2_t k01 = as_h2(kraw.x), k23 = as_h2(kraw.y);      // half operands go straight into the FMA
-            float node = fmaf(row_lane_f(qv, (d & 63)), (float)k01.x, 0.0f);
-            node = fmaf(row_lane_f(qv, (d & 63) + 1), (float)k01.y, node);
-            node = fmaf(row_lane_f(qv, (d & 63) + 2), (float)k23.x, node);
-            n[l] = fmaf(row_lane_f(qv, (d & 63) + 3), (float)k23.y, node);
+            const float4 q4 = *reinterpret_cast<const float4*>(qh + d);
+            c[gi] = fmaf(q4.x, (float)k01.x, c[gi]);
+            c[gi] = fmaf(q4.y, (float)k01.y, c[gi]);
+            c[gi] = fmaf(q4.z, (float)k23.x, c[gi]);
+            c[gi] = fmaf(q4.w, (float)k23.y, c[gi]);
           }
-          g[gi] = ((n[0] + n[1]) + (n[2] + n[3])) + ((n[4] + n[5]) + (n[6] + n[7]));
         }
-        L.part[wave * 64 + lane] = (g[0] + g[1]) + (g[2] + g[3]);
+        L.part[wave * 64 + lane] = (c[0] + c[1]) + (c[2] + c[3]);
       }
       lds_barrier();
       if ((wave & 1) == 0) {
@@ -654,7 +704,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
     for (int r = 0; r < nr; ++r) {
       const int u = ub + r * GU;
       const int tile = u >> 1, kvh = u & 1;
-      const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
+      const int j0 = tile * SDPA_TILE;
       const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
       lds_barrier();                    // the previous unit's value tile has been read; the weights are in place
       if (r > 0) {
@@ -669,29 +719,29 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       }
       lds_barrier();
       const int h = wave >> 1, half = wave & 1;
-      float o0 = 0.0f, o1 = 0.0f;
+      // two chains over the keys, 0..31 and 32..63, added at the end; all 64 keys are walked (beyond the context the
+      // weight and the staged value are zero).  The weights come as LDS broadcasts, four keys per read.
+      float oa0 = 0.0f, oa1 = 0.0f, ob0 = 0.0f, ob1 = 0.0f;
       const uint16_t* vt = &g_vt[128 * half + 2 * lane];
-      const float pmine = ps[(r * 8 + h) * 64 + lane];     // weight of key `lane`; handed out by readlane below
-      int j = 0;
-      for (; j + 8 <= nk; j += 8) {            // the eight LDS reads are issued together, then used in key order
-        uint32_t v8[8];
+      const float* pw = &ps[(r * 8 + h) * 64];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v8[i] = *reinterpret_cast<const uint32_t*>(vt + (j + i) * 256);
+      for (int j = 0; j < 32; j += 4) {
+        uint32_t va[4], vb[4];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float pj = row_lane_f(pmine, j + i);
-          const h2_t v01 = as_h2(v8[i]);
-          o0 = fmaf(pj, (float)v01.x, o0);
-          o1 = fmaf(pj, (float)v01.y, o1);
+        for (int i = 0; i < 4; ++i) {
+          va[i] = *reinterpret_cast<const uint32_t*>(vt + (j + i) * 256);
+          vb[i] = *reinterpret_cast<const uint32_t*>(vt + (32 + j + i) * 256);
+        }
+        const float4 pa = *reinterpret_cast<const float4*>(pw + j), pb = *reinterpret_cast<const float4*>(pw + 32 + j);
+        const float pav[4] = {pa.x, pa.y, pa.z, pa.w}, pbv[4] = {pb.x, pb.y, pb.z, pb.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const h2_t a01 = as_h2(va[i]), b01 = as_h2(vb[i]);
+          oa0 = fmaf(pav[i], (float)a01.x, oa0); oa1 = fmaf(pav[i], (float)a01.y, oa1);
+          ob0 = fmaf(pbv[i], (float)b01.x, ob0); ob1 = fmaf(pbv[i], (float)b01.y, ob1);
         }
       }
-      for (; j < nk; ++j) {
-        const uint32_t vv = *reinterpret_cast<const uint32_t*>(vt + j * 256);
-        const float pj = row_lane_f(pmine, j);
-        const h2_t v01 = as_h2(vv);
-        o0 = fmaf(pj, (float)v01.x, o0);
-        o1 = fmaf(pj, (float)v01.y, o1);
-      }
+      const float o0 = oa0 + ob0, o1 = oa1 + ob1;
       const int head = kvh * 8 + h;
       stw4(co_rsrc(uni(F.tpo)), ((head * uni(P.max_tiles) + tile) * 128 + 64 * half + lane) * 4, __float_as_uint(o0), __float_as_uint(o1), tcore, tcore);
     }
@@ -728,6 +778,8 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
     if (row < nk && j0 + row != pos) {
       st16(&L.kt[row * KT_STRIDE + c8], ld16(kbase + (size_t)row * 256 + c8));
       st16(&g_vt[row * 256 + c8], ld16(vbase + (size_t)row * 256 + c8));
+    } else if (row >= nk) {
+      st16(&g_vt[row * 256 + c8], make_uint4(0, 0, 0, 0));         // weight 0 times value 0 leaves a sum as it is
     }
   }
   // waves 0,1: the unit's two query heads; wave 8: new key; wave 9: new value -- 4 tagged words per lane
@@ -760,10 +812,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
     const float xv[4] = {lo_h(w4.x), lo_h(w4.y), lo_h(w4.z), lo_h(w4.w)};
     float wv[4];
     wv[0] = lo_h(wraw.x); wv[1] = hi_h(wraw.x); wv[2] = lo_h(wraw.y); wv[3] = hi_h(wraw.y);
-    float ss = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) ss = fmaf(xv[i], xv[i], ss);
-    ss = tree_sum<64>(ss);
+    const float ss = tree_sum<64>(fmaf(xv[1], xv[1], xv[0] * xv[0]) + fmaf(xv[3], xv[3], xv[2] * xv[2]));
     const float inv = 1.0f / sqrtf(ss / 256.0f + EPS);
     float* dst = isq ? &L.sq[wave * 256] : L.knew;
 #pragma unroll
@@ -793,22 +842,23 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
   }
   lds_barrier();
   {
-    // scores: wave (head, slice) takes the 8 leaves of its 32 dims, lane j is key j; the 32 query values sit one
-    // per lane (lanes 0..31) and reach the multiply as scalar operands
+    // scores: wave (head, slice) takes one of the eight chains of 32 dims, lane j is key j; the queries come as LDS
+    // broadcasts
     const int hh = wave >> 3, sl = wave & 7;
     const uint16_t* kr = &L.kt[(lane < nk ? lane : 0) * KT_STRIDE + 32 * sl];
-    const float qv = L.sq[hh * 256 + 32 * sl + (lane & 31)];
-    float n[8];
+    const float* qs = &L.sq[hh * 256 + 32 * sl];
+    float ch = 0.0f;
 #pragma unroll
     for (int l = 0; l < 8; ++l) {
       const uint2 kraw = *reinterpret_cast<const uint2*>(kr + 4 * l);
       const h2_t k01 = as_h2(kraw.x), k23 = as_h2(kraw.y);
-      float node = fmaf(row_lane_f(qv, 4 * l), (float)k01.x, 0.0f);
-      node = fmaf(row_lane_f(qv, 4 * l + 1), (float)k01.y, node);
-      node = fmaf(row_lane_f(qv, 4 * l + 2), (float)k23.x, node);
-      n[l] = fmaf(row_lane_f(qv, 4 * l + 3), (float)k23.y, node);
+      const float4 q4 = *reinterpret_cast<const float4*>(qs + 4 * l);
+      ch = fmaf(q4.x, (float)k01.x, ch);
+      ch = fmaf(q4.y, (float)k01.y, ch);
+      ch = fmaf(q4.z, (float)k23.x, ch);
+      ch = fmaf(q4.w, (float)k23.y, ch);
     }
-    L.part[wave * 64 + lane] = ((n[0] + n[1]) + (n[2] + n[3])) + ((n[4] + n[5]) + (n[6] + n[7]));
+    L.part[wave * 64 + lane] = ch;
   }
   lds_barrier();
   if ((wave & 7) == 0) {
@@ -825,32 +875,31 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
   }
   lds_barrier();
   if (wave < 4) {
-    // values: wave (head, half of the dims), two dims per lane (one LDS word per key); the weight of key j is
-    // handed out by readlane.  Eight LDS reads are issued together, then used in key order.
+    // values: wave (head, half of the dims), two dims per lane (one LDS word per key); two chains over the keys,
+    // 0..31 and 32..63, added at the end; all 64 keys are walked (beyond the context the weight and the staged value are
+    // zero).  The weights come as LDS broadcasts, four keys per read.
     const int hh = wave >> 1, half = wave & 1;
-    float o0 = 0.0f, o1 = 0.0f;
+    float oa0 = 0.0f, oa1 = 0.0f, ob0 = 0.0f, ob1 = 0.0f;
     const uint16_t* vt = &g_vt[128 * half + 2 * lane];
-    const float pmine = L.sm[hh * 64 + lane];
-    int j = 0;
-    for (; j + 8 <= nk; j += 8) {              // eight LDS reads and eight weights at a time, used in key order
-      uint32_t v8[8];
-      float p8[8];
+    const float* pw = &L.sm[hh * 64];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v8[i] = *reinterpret_cast<const uint32_t*>(vt + (j + i) * 256);
-      lanes8(pmine, j, p8);
+    for (int j = 0; j < 32; j += 4) {
+      uint32_t va[4], vb[4];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const h2_t v01 = as_h2(v8[i]);
-        o0 = fmaf(p8[i], (float)v01.x, o0);
-        o1 = fmaf(p8[i], (float)v01.y, o1);
+      for (int i = 0; i < 4; ++i) {
+        va[i] = *reinterpret_cast<const uint32_t*>(vt + (j + i) * 256);
+        vb[i] = *reinterpret_cast<const uint32_t*>(vt + (32 + j + i) * 256);
+      }
+      const float4 pa = *reinterpret_cast<const float4*>(pw + j), pb = *reinterpret_cast<const float4*>(pw + 32 + j);
+      const float pav[4] = {pa.x, pa.y, pa.z, pa.w}, pbv[4] = {pb.x, pb.y, pb.z, pb.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const h2_t a01 = as_h2(va[i]), b01 = as_h2(vb[i]);
+        oa0 = fmaf(pav[i], (float)a01.x, oa0); oa1 = fmaf(pav[i], (float)a01.y, oa1);
+        ob0 = fmaf(pbv[i], (float)b01.x, ob0); ob1 = fmaf(pbv[i], (float)b01.y, ob1);
       }
     }
-    for (; j < nk; ++j) {
-      const h2_t v01 = as_h2(*reinterpret_cast<const uint32_t*>(vt + j * 256));
-      const float pj = row_lane_f(pmine, j);
-      o0 = fmaf(pj, (float)v01.x, o0);
-      o1 = fmaf(pj, (float)v01.y, o1);
-    }
+    const float o0 = oa0 + ob0, o1 = oa1 + ob1;
     const int head = kvh * 8 + hq * 2 + hh;
     stw4(co_rsrc(uni(F.tpo)), ((head * uni(P.max_tiles) + tile) * 128 + 64 * half + lane) * 4, __float_as_uint(o0), __float_as_uint(o1),
          tcore, tcore);
@@ -886,6 +935,13 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   const float NEG = -__int_as_float(0x7f800000);
   WRegs<2, 1> wr;
   const bool valid = gw < H;
+#if SL_WRING
+  if (lin) {           // the row was requested into LDS when the in-projection ended; its scales and biases come now
+    wr.w[0][0] = wr.w[0][1] = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) wr.sb[0][b] = valid ? uni(Y.out_sb)[(size_t)gw * 64 + b * 32 + (lane >> 1)] : 0u;
+  } else
+#endif
   wload_row<2>(wr.w[0], wr.sb[0], uni(Y.out_w), uni(Y.out_sb), (size_t)(valid ? gw : 0), valid, lane);
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
@@ -1168,16 +1224,15 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     const int b = e0 >> 11, r = e0 & 2047, lo = r >> 5, i0 = r & 31;
     g_L.xs[(16 * b + (i0 >> 1)) * 64 + lo] = pack2(out[0], out[1]);
     g_L.xs[(16 * b + (i0 >> 1) + 1) * 64 + lo] = pack2(out[2], out[3]);
-    float sfirst = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) sfirst = sfirst + out[i];
-    float srest = prev_lane(sfirst);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) srest = srest + out[i];
-    if (lane & 1) g_L.sxs[(4 * b + (i0 >> 3)) * 64 + lo] = srest;
+    // a share of 32 elements sits on eight neighbouring lanes: balanced tree over its 16 pair sums
+    const float ssum = tree_sum<8>((out[0] + out[1]) + (out[2] + out[3]));
+    if ((lane & 7) == 0) g_L.sxs[64 * b + lo] = ssum;
   }
   lds_barrier();
   fstamp<ST>(li, FS_OUT, 2, tid == 0);
+#if SL_WRING
+  if (lin) { wr_wait(); wr.w[0][0] = wr_read(wave * 3, lane); wr.w[0][1] = wr_read(wave * 3 + 1, lane); }
+#endif
   const float o = dot_2x1(wr);
   fstamp<ST>(li, FS_OUT, 3, tid == 0);
   if (wg * DEC_WAVES < H) {                       // uniform per workgroup
@@ -1226,7 +1281,7 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
   flow_prologue(h0, h1, true, r0, r1, lnw, nullptr);
   fstamp<ST>(li, FS_A, 2, tid == 0);
   if (is_dense) {
-    uint32_t xp[16]; float sx[4];
+    uint32_t xp[16]; float sx;
     lds_get_x(0, lane, xp, sx);
     const uint32_t dww[16] = {dwr[0].x, dwr[0].y, dwr[0].z, dwr[0].w, dwr[1].x, dwr[1].y, dwr[1].z, dwr[1].w,
                               dwr[2].x, dwr[2].y, dwr[2].z, dwr[2].w, dwr[3].x, dwr[3].y, dwr[3].z, dwr[3].w};
@@ -1362,7 +1417,8 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
 
 // ---- MoE stage C: down-projections, half combine, gated shared add ---------------------------------------
 // Units (quad of 4 outputs, slot): slots 0..7 routed experts, slot 8 shared; 2 quads per workgroup.  The nine
-// activation rows are fetched once per workgroup into LDS (packed pairs, 20-word stride per 32 elements).
+// activation rows are fetched once per workgroup into LDS (packed pairs, 20-word stride per 32 elements, the
+// share's sum in word 16 of its slot).
 constexpr int XC_STRIDE = 20;
 template <bool ST>
 SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
@@ -1407,23 +1463,36 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     // the first 128
     const rsrc_t ra = co_rsrc(uni(F.tact)), rs = co_rsrc(uni(F.tsh)), rg = co_rsrc(uni(F.tsg));
     bool have[2] = {false, tid >= 128};           // a chunk that has arrived is not fetched again
-    if (!flow_poll(true, [&]() {
-          bool ok = true;
+    float psum[2] = {0.0f, 0.0f};                 // sum of the chunk's two pair sums
+    flow_poll<false>(true, [&]() {
+      bool ok = true;
 #pragma unroll
-          for (int c = 0; c < 2; ++c) {
-            if (have[c]) continue;
-            // chunk t holds elements 4(t%128).. of slot t/128 (slot 8 = shared): packed pairs 2(t%128), 2(t%128)+1
-            const int t = tid + 1024 * c, slot = t >> 7, pi = 2 * (t & 127);
-            const uint4 a4 = (slot < 8) ? ldw4(ra, 4 * t) : ldw4(rs, 4 * (t & 127));
-            const uint32_t tx = (slot < 8) ? tb : ta;
-            have[c] = tag_ok(a4.x, tx) && tag_ok(a4.y, tx) && tag_ok(a4.z, tx) && tag_ok(a4.w, tx);
-            ok = ok && have[c];
-            *reinterpret_cast<uint2*>(&xc[(slot * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
-                make_uint2((a4.x & 0xffffu) | (a4.y << 16), (a4.z & 0xffffu) | (a4.w << 16));
-          }
-          if (tid == 0) { const uint32_t w = ldw1(rg, 0); ok = ok && tag_ok(w, ta); L.gb[1] = lo_h(w); }
-          return ok;
-        }, uni(P.bar) + 32)) return false;
+      for (int c = 0; c < 2; ++c) {
+        if (have[c]) continue;
+        // chunk t holds elements 4(t%128).. of slot t/128 (slot 8 = shared): packed pairs 2(t%128), 2(t%128)+1
+        const int t = tid + 1024 * c, slot = t >> 7, pi = 2 * (t & 127);
+        const uint4 a4 = (slot < 8) ? ldw4(ra, 4 * t) : ldw4(rs, 4 * (t & 127));
+        const uint32_t tx = (slot < 8) ? tb : ta;
+        have[c] = tag_ok(a4.x, tx) && tag_ok(a4.y, tx) && tag_ok(a4.z, tx) && tag_ok(a4.w, tx);
+        ok = ok && have[c];
+        psum[c] = (lo_h(a4.x) + lo_h(a4.y)) + (lo_h(a4.z) + lo_h(a4.w));
+        *reinterpret_cast<uint2*>(&xc[(slot * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
+            make_uint2((a4.x & 0xffffu) | (a4.y << 16), (a4.z & 0xffffu) | (a4.w << 16));
+      }
+      if (tid == 0) { const uint32_t w = ldw1(rg, 0); ok = ok && tag_ok(w, ta); L.gb[1] = lo_h(w); }
+      return ok;
+    }, uni(P.bar) + 32);
+    // a share of 32 activations = the chunks of eight neighbouring threads: its sum (the balanced tree over the 16 pair
+    // sums) goes into the padding word behind the share's packed pairs
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      if (c == 1 && wave >= 2) break;               // second chunks sit on threads 0..127 (wave-uniform)
+      const int t = tid + 1024 * c;
+      const float ssum = tree_sum<8>(psum[c]);
+      if ((tid & 7) == 0) xc[((t >> 7) * 16 + ((t & 127) >> 3)) * XC_STRIDE + 16] = __float_as_uint(ssum);
+    }
+    lds_barrier();
+    if (g_L.pf[3] != 0) return false;
     fstamp<ST>(li, FS_C, 1, tid == 0);
   }
   // the shared expert's gate came with the poll: its sigmoid is formed by the publishing wave while the units run
@@ -1437,15 +1506,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
       const uint4* src = reinterpret_cast<const uint4*>(&xc[(slot * 16 + li16) * XC_STRIDE]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) { const uint4 q = src[j]; xp[4 * j] = q.x; xp[4 * j + 1] = q.y; xp[4 * j + 2] = q.z; xp[4 * j + 3] = q.w; }
-      float sx[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float sacc = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { sacc = sacc + lo_h(xp[4 * j + i]); sacc = sacc + hi_h(xp[4 * j + i]); }
-        sx[j] = sacc;
-      }
-      const float d = tree_sum<16>(quad_term(wv[qq], sbv[qq], xp, sx));
+      const float d = tree_sum<16>(share_term(wv[qq], sbv[qq], xp, __uint_as_float(xc[(slot * 16 + li16) * XC_STRIDE + 16])));
       if (li16 == 0) L.dbuf[(ql * 9 + slot) * 4 + sub] = f16r(d);
     }
   }
@@ -1499,7 +1560,7 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
   flow_prologue(h0, h1, true, r0, r1, lnw, wg == 0 ? uni(P.normed) : nullptr);
   // the activation row stays in registers for all groups; the two weight sets swap roles from group to group (a copy
   // would cost twenty moves per group in a stage that is bound by its instruction count)
-  uint32_t x[16]; float sx[4];
+  uint32_t x[16]; float sx;
   lds_get_x(0, lane, x, sx);
   // The four row sums of a group are reduced together.  After the first two levels of the reduction tree (lane
   // pairs, then quads) the four lanes of a quad hold the same value, so one register can carry all four rows, lane l
@@ -1512,7 +1573,7 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
     load_group(b, k + 1);
     float q[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) q[j] = tree_sum<4>(quad_term(a.w[j][0], a.sb[j][0], x, sx));
+    for (int j = 0; j < 4; ++j) q[j] = tree_sum<4>(share_term(a.w[j][0], a.sb[j][0], x, sx));
     float f = rho == 0 ? q[0] : (rho == 1 ? q[1] : (rho == 2 ? q[2] : q[3]));
     f = f + dpp_f<DPP_HALF_MIRROR>(f);
     f = f + dpp_f<DPP_MIRROR>(f);
@@ -1607,6 +1668,10 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
   const FlowP& F = g_K.F;
   const DecodeP& P = F.d;
   const int nl = uni(P.n_layers);
+  // A workgroup that leaves (a wait gave up, or the launch is over) first lets its outstanding loads land: rows on
+  // their way into LDS must not arrive after the LDS has passed to another workgroup.
+#define FLOW_TRY(call) do { if (!(call)) { wr_wait(); return; } } while (0)
+  flow_request_in(g_K.layers[0]);
   for (int step = 0; step < steps; ++step) {
     const uint32_t base = uni(g_K.base);
     const int pos = uni(g_K.pos);
@@ -1614,26 +1679,33 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
     for (int li = 0; li < nl; ++li) {
       const LayerP& Y = g_K.layers[li];
       const int is_linear = uni(Y.is_linear);
-      if (!flow_in<ST>(F, Y, li, pos, base, h0, h1, step)) return;
+      FLOW_TRY(flow_in<ST>(F, Y, li, pos, base, h0, h1, step));
       GdnHist gh = {0u, 0u};
       if (is_linear) {
-        if (!flow_gdn<ST>(F, Y, li, base, gh)) return;
-        if (!flow_out<ST>(F, Y, li, 0, base, gh)) return;
+        FLOW_TRY(flow_gdn<ST>(F, Y, li, base, gh));
+        FLOW_TRY(flow_out<ST>(F, Y, li, 0, base, gh));
       } else {
-        if (((pos + SDPA_TILE) / SDPA_TILE) * SL_ATT_KV * 4 <= (int)gridDim.x ? !flow_sdpa4<ST>(F, Y, li, pos, base) : !flow_sdpa<ST>(F, Y, li, pos, base)) return;
-        if (!flow_out<ST>(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh)) return;
+        if (((pos + SDPA_TILE) / SDPA_TILE) * SL_ATT_KV * 4 <= (int)gridDim.x) FLOW_TRY(flow_sdpa4<ST>(F, Y, li, pos, base));
+        else FLOW_TRY(flow_sdpa<ST>(F, Y, li, pos, base));
+        FLOW_TRY(flow_out<ST>(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh));
       }
-      if (!flow_moe_a<GATE8, ST>(F, Y, li, base, h0, h1)) return;
-      if (!flow_moe_b<ST>(F, Y, li, base)) return;
-      if (!flow_moe_c<ST>(F, Y, li, base)) return;
+      // through with the K = 4096 projection (the upper half of the grid has no rows there and is here at once): the
+      // in-projection rows of the next layer, or of the next step's first layer, set out for LDS
+      if (li + 1 < nl) flow_request_in(g_K.layers[li + 1]);
+      else if (step + 1 < steps) flow_request_in(g_K.layers[0]);
+      FLOW_TRY((flow_moe_a<GATE8, ST>(F, Y, li, base, h0, h1)));
+      FLOW_TRY(flow_moe_b<ST>(F, Y, li, base));
+      FLOW_TRY(flow_moe_c<ST>(F, Y, li, base));
     }
-    if (!flow_head<ST>(F, pos, out_off + step, feed, base, h0, h1, step + 1 < steps)) return;
+    FLOW_TRY(flow_head<ST>(F, pos, out_off + step, feed, base, h0, h1, step + 1 < steps));
     if (step + 1 < steps) {
       lds_barrier();                     // everybody has read this step's position, tag base and parities
       if (threadIdx.x == 0) { g_K.pos = pos + 1; g_K.base = base + (uint32_t)(nl + 1) * 8u; g_K.parity ^= g_K.linmask; }
       lds_barrier();
     }
   }
+#undef FLOW_TRY
+  wr_wait();
   if constexpr (ST) {
     __syncthreads();
     uint32_t* dst = uni(P.tstamp) + (size_t)blockIdx.x * STAMP_WORDS;

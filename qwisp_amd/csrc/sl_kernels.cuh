@@ -3,11 +3,11 @@
 // M-row verify step equal M single-row steps bit for bit.
 //
 // Reduction order shared by all kernels (and by the CPU checker used in the tests):
-//  * 4-bit dot, K = 2048*NBLK: lane l owns words 4l..4l+3 of each 2048-element block (one 16-byte
-//    load), word term t = fmaf(s, dq, b*sx), lane partial = sum over blocks of (t0+t1)+(t2+t3),
-//    then a 64-lane butterfly.  K = 512: the same with 16 lanes per row, four rows per wave.
-//  * dense fp16 dot / sum of squares over 2048: lane l owns elements 32l..32l+31, fmaf chain, butterfly.
-//  * sum of squares over 128 or 256: 64 leaves of 2 or 4 contiguous elements, balanced tree.
+//  * 4-bit dot, K = 2048*NBLK: lane l owns the share of 32 elements (words 4l..4l+3, one 16-byte load) of each
+//    2048-element block, share term T = fmaf(s, A + B, b*sx) (share_term in sl_device.cuh), lane partial = sum of
+//    its terms block after block, then a 64-lane butterfly.  K = 512: the same with 16 lanes per row, four rows per wave.
+//  * dense fp16 dot over 2048: lane l owns elements 32l..32l+31, fmaf chain, butterfly.
+//  * sum of squares over D = 128, 256 or 2048: pair terms fmaf(x1, x1, x0*x0), balanced tree over the D/2 of them.
 #pragma once
 #include "sl_device.cuh"
 #include "../../include/seedless_hip.h"
@@ -33,10 +33,7 @@ SL_DEV void store32(uint16_t* p, const float* x) {
   for (int j = 0; j < 4; ++j) st16(p + 8 * j, pack8(x + 8 * j));
 }
 SL_DEV float inv_rms_2048(const float* x) {
-  float ss = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 32; ++i) ss = fmaf(x[i], x[i], ss);
-  ss = tree_sum<64>(ss);
+  const float ss = tree_sum<64>(share_sumsq(x));
   return 1.0f / sqrtf(ss / 2048.0f + EPS);
 }
 struct HiddenArgs {
@@ -45,7 +42,7 @@ struct HiddenArgs {
   const uint16_t* lnw;     // [2048] norm weight, or null for "x is used as given"
   uint16_t* h_out;         // [M, 2048] receives half(h + r) (written once per row), or null
   uint16_t* xn_out;        // [M, 2048] receives the normed row (written once per row), or null
-  float* xs_out;           // [M, 256] receives the left-to-right sums of each run of 8 elements of that row (word_sums), or null
+  float* xs_out;           // [M, 64] receives the sums of the row's 64 shares of 32 elements (share_sum), or null
 };
 // Every wave of the grid calls this; `writer` selects the single wave that stores the outputs.
 SL_DEV void hidden_prologue(const HiddenArgs& a, int m, int lane, bool writer, float* x) {
@@ -65,11 +62,7 @@ SL_DEV void hidden_prologue(const HiddenArgs& a, int m, int lane, bool writer, f
     for (int i = 0; i < 32; ++i) x[i] = f16r(w[i] * f16r(x[i] * inv));
   }
   if (writer && a.xn_out) store32(a.xn_out + (size_t)m * H + 32 * lane, x);
-  if (writer && a.xs_out) {                       // the dots of the row's consumers need these sums: formed once here
-    float sx[4];
-    word_sums(x, sx);
-    *reinterpret_cast<float4*>(a.xs_out + (size_t)m * 256 + 4 * lane) = make_float4(sx[0], sx[1], sx[2], sx[3]);
-  }
+  if (writer && a.xs_out) a.xs_out[(size_t)m * 64 + lane] = share_sum(x);   // the dots of the row's consumers need these sums: formed once here
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -91,18 +84,18 @@ SL_DEV void qdot_rows(const uint32_t* __restrict__ W, const uint32_t* __restrict
     }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    float acc = quad_term(wv[r][0], sb[r][0], xp, sx);
+    float acc = share_term(wv[r][0], sb[r][0], xp, sx[0]);
 #pragma unroll
-    for (int b = 1; b < NBLK; ++b) acc = acc + quad_term(wv[r][b], sb[r][b], xp + 16 * b, sx + 4 * b);
+    for (int b = 1; b < NBLK; ++b) acc = acc + share_term(wv[r][b], sb[r][b], xp + 16 * b, sx[b]);
     out[r] = tree_sum<64>(acc);
   }
 }
 // K = 512: 16 lanes per row; li = lane & 15 owns words 4li..4li+3.  Result valid on all 16 lanes.
 SL_DEV float qdot512(const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB, size_t row, int li,
-                     const uint32_t* xp, const float* sx) {
+                     const uint32_t* xp, float sx) {
   const uint4 wv = ld16(W + row * 64 + 4 * li);
   const uint32_t sb = SB[row * 8 + (li >> 1)];
-  return tree_sum<16>(quad_term(wv, sb, xp, sx));
+  return tree_sum<16>(share_term(wv, sb, xp, sx));
 }
 // Dense fp16 row against the lane's 32 activations (router gate, shared-expert gate).
 SL_DEV float dense_dot(const uint16_t* __restrict__ wrow, int lane, const float* x) {
@@ -137,9 +130,9 @@ __global__ __launch_bounds__(256) void k_qmv_hidden(HiddenArgs ha, const uint32_
                                                     const uint32_t* __restrict__ SB, int N, uint16_t* __restrict__ y,
                                                     int y_stride) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float x[32], sx[4];
+  float x[32], sx[1];
   hidden_prologue(ha, m, lane, blockIdx.x == 0 && wave == 0, x);
-  word_sums(x, sx);
+  sx[0] = share_sum(x);
   uint32_t xp[16];
   pack_x(x, xp);
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * R;
@@ -161,13 +154,13 @@ __global__ __launch_bounds__(256) void k_qmv_plain(const uint16_t* __restrict__ 
                                                    const uint32_t* __restrict__ W, const uint32_t* __restrict__ SB,
                                                    int N, uint16_t* __restrict__ y, int y_stride) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float sx[4 * NBLK];
+  float sx[NBLK];
   uint32_t xp[16 * NBLK];
 #pragma unroll
   for (int b = 0; b < NBLK; ++b) {
     float x[32];
     load32(xin + (size_t)m * x_stride + b * 2048 + 32 * lane, x);
-    word_sums(x, sx + 4 * b);
+    sx[b] = share_sum(x);
     pack_x(x, xp + 16 * b);
   }
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * R;
@@ -188,8 +181,9 @@ __global__ __launch_bounds__(256) void k_qmv_plain(const uint16_t* __restrict__ 
 // chunks): a wave fetches and masks its R weight rows once and runs every activation row of the tile against
 // them, so the weight stream and the nibble unpacking are shared; per activation row the arithmetic is that of
 // k_qmv_hidden / k_qmv_plain.  The tile's activation rows are prepared once per workgroup (residual, norm,
-// packing: wave w takes rows w, w + waves, ...) and parked in LDS, 20 words per lane (16 packed pairs, 4 sums)
-// so that a lane reads back its own 80 bytes with five 16-byte reads free of bank conflicts.
+// packing: wave w takes rows w, w + waves, ...) and parked in LDS, 20 words per lane (16 packed pairs, the share's
+// sum and three words of padding) so that a lane reads back its own 80 bytes with five 16-byte reads free of bank
+// conflicts.
 // HIDDEN: x comes from the hidden prologue (K = 2048; steps of up to four rows, where a wave preparing one row in
 // every workgroup costs less than a launch that prepares the rows once); otherwise from the fp16 buffer xin
 // (K = 2048*NBLK).  Grid (G, ceil(M / MT)), four waves (three workgroups share a compute unit).  G workgroups cover G*waves*R rows; rows beyond that (fewer than G) are taken one each by wave 0 of the
@@ -236,18 +230,18 @@ __global__ __launch_bounds__(256, 3) void k_qmv_tile(HiddenArgs ha, const uint16
         const uint16_t* src = xin + (size_t)(m0 + m) * x_stride + b * 2048 + 32 * lane;
 #pragma unroll
         for (int j = 0; j < 4; ++j) dst[j] = ld16(src + 8 * j);
-        dst[4] = ld16(xsums + (size_t)(m0 + m) * (256 * NBLK) + b * 256 + 4 * lane);
+        dst[4] = make_uint4(__float_as_uint(xsums[(size_t)(m0 + m) * (64 * NBLK) + b * 64 + lane]), 0u, 0u, 0u);
         continue;
       }
-      float x[32], sx[4];
+      float x[32];
       if constexpr (HIDDEN) hidden_prologue(ha, m0 + m, lane, blockIdx.x == 0, x);
       else load32(xin + (size_t)(m0 + m) * x_stride + b * 2048 + 32 * lane, x);
-      word_sums(x, sx);
+      const float sx = share_sum(x);
       uint32_t xp[16];
       pack_x(x, xp);
 #pragma unroll
       for (int j = 0; j < 4; ++j) dst[j] = make_uint4(xp[4 * j], xp[4 * j + 1], xp[4 * j + 2], xp[4 * j + 3]);
-      dst[4] = make_uint4(__float_as_uint(sx[0]), __float_as_uint(sx[1]), __float_as_uint(sx[2]), __float_as_uint(sx[3]));
+      dst[4] = make_uint4(__float_as_uint(sx), 0u, 0u, 0u);
     }
   }
   __syncthreads();
@@ -272,13 +266,12 @@ __global__ __launch_bounds__(256, 3) void k_qmv_tile(HiddenArgs ha, const uint16
     for (int b = 0; b < NBLK; ++b) {
       const uint4* src = xs + ((m * NBLK + b) * 64 + lane) * 5;
       uint32_t xp[16];
-      float sx[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) { const uint4 v = src[j]; xp[4 * j] = v.x; xp[4 * j + 1] = v.y; xp[4 * j + 2] = v.z; xp[4 * j + 3] = v.w; }
-      { const uint4 v = src[4]; sx[0] = __uint_as_float(v.x); sx[1] = __uint_as_float(v.y); sx[2] = __uint_as_float(v.z); sx[3] = __uint_as_float(v.w); }
+      const float sx = __uint_as_float(reinterpret_cast<const uint32_t*>(src + 4)[0]);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const float t = quad_term_masked(mk[r][b], sb[r][b], xp, sx);
+        const float t = share_term_masked(mk[r][b], sb[r][b], xp, sx);
         acc[r] = (b == 0) ? t : acc[r] + t;
       }
     }
@@ -325,11 +318,10 @@ __global__ __launch_bounds__(256, 3) void k_qmv_tile(HiddenArgs ha, const uint16
       for (int b = 0; b < NBLK; ++b) {
         const uint4* src = xs + ((m * NBLK + b) * 64 + lane) * 5;
         uint32_t xp[16];
-        float sx[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) { const uint4 v = src[j]; xp[4 * j] = v.x; xp[4 * j + 1] = v.y; xp[4 * j + 2] = v.z; xp[4 * j + 3] = v.w; }
-        { const uint4 v = src[4]; sx[0] = __uint_as_float(v.x); sx[1] = __uint_as_float(v.y); sx[2] = __uint_as_float(v.z); sx[3] = __uint_as_float(v.w); }
-        const float t = quad_term_masked(mx[b], sbx[b], xp, sx);
+        const float sx = __uint_as_float(reinterpret_cast<const uint32_t*>(src + 4)[0]);
+        const float t = share_term_masked(mx[b], sbx[b], xp, sx);
         acc = (b == 0) ? t : acc + t;
       }
       const float o = tree_sum<64>(acc);
@@ -650,7 +642,7 @@ __global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict_
                                                      const float* __restrict__ norm_w, int norm_f32, const uint32_t* __restrict__ W,
                                                      const uint32_t* __restrict__ SB, int N, uint16_t* __restrict__ y) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float sx[8];
+  float sx[2];
   uint32_t xp[32];
   float nw[32];                                  // norm weight as fp32 (exact for an fp16 checkpoint weight)
 #pragma unroll
@@ -678,7 +670,7 @@ __global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict_
       const float nrm = norm_f32 ? nw[i] * (xb[i] * inv) : f16r(nw[i] * f16r(xb[i] * inv));
       xb[i] = f16r((z[i] * sigmoid32(z[i])) * nrm);
     }
-    word_sums(xb, sx + 4 * b);
+    sx[b] = share_sum(xb);
     pack_x(xb, xp + 16 * b);
   }
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * R;
@@ -699,8 +691,8 @@ __global__ __launch_bounds__(256) void k_qmv_gdn_out(const uint16_t* __restrict_
 // gated[m, hv, :] = half(silu(z) * norm(y)) in place of y.  One wave per (value head, row); lane l owns the pair
 // 2l, 2l+1, so the sum of squares is the same balanced tree as in the fused kernel above.
 // -------------------------------------------------------------------------------------------------
-// `ysum` (or null) receives the row's word sums (left-to-right sums of each run of 8 gated values, [M, 512]) for the
-// projection that follows: a run sits on four neighbouring lanes, the sum passes along them.
+// `ysum` (or null) receives the sums of the row's shares of 32 gated values ([M, 128], share_sum's tree) for the
+// projection that follows: a share sits on sixteen neighbouring lanes.
 __global__ __launch_bounds__(64) void k_gdn_gate_rows(uint16_t* __restrict__ ycore, const uint16_t* __restrict__ proj,
                                                       const float* __restrict__ norm_w, int norm_f32, float* __restrict__ ysum = nullptr) {
   const int hv = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;
@@ -716,14 +708,8 @@ __global__ __launch_bounds__(64) void k_gdn_gate_rows(uint16_t* __restrict__ yco
   const float o0 = f16r((z0 * sigmoid32(z0)) * n0), o1 = f16r((z1 * sigmoid32(z1)) * n1);
   *reinterpret_cast<uint32_t*>(yp) = pack2(o0, o1);
   if (ysum) {
-    const int q = lane & 3;
-    float sw = (0.0f + o0) + o1;
-#pragma unroll
-    for (int r = 1; r < 4; ++r) {
-      const float v = prev_lane(sw);
-      if (q == r) sw = (v + o0) + o1;
-    }
-    if (q == 3) ysum[(size_t)m * 512 + hv * 16 + (lane >> 2)] = sw;
+    const float sw = tree_sum<16>(o0 + o1);
+    if ((lane & 15) == 0) ysum[(size_t)m * 128 + hv * 4 + (lane >> 4)] = sw;
   }
 }
 
@@ -839,7 +825,7 @@ __global__ __launch_bounds__(1024) void k_gdn_few_rows(GdnArgs a, const float* _
   __syncthreads();
   if (wave >= 8 && wave - 8 < M) {
     // gated norm of row wave - 8 over the head's 128 outputs (the arithmetic of k_gdn_gate_rows), and the sums of
-    // each run of 8 gated values for the out-projection's dots
+    // each share of 32 gated values for the out-projection's dots
     const int m = wave - 8;
     const float y0 = s_y[m][2 * lane], y1 = s_y[m][2 * lane + 1], z0 = lo_h(zw), z1 = hi_h(zw);
     const float ss = tree_sum<64>(fmaf(y1, y1, fmaf(y0, y0, 0.0f)));
@@ -848,14 +834,8 @@ __global__ __launch_bounds__(1024) void k_gdn_few_rows(GdnArgs a, const float* _
     const float n1 = norm_f32 ? nw1 * (y1 * inv) : f16r(nw1 * f16r(y1 * inv));
     const float o0 = f16r((z0 * sigmoid32(z0)) * n0), o1 = f16r((z1 * sigmoid32(z1)) * n1);
     *reinterpret_cast<uint32_t*>(a.ycore + (size_t)m * 4096 + hv * 128 + 2 * lane) = pack2(o0, o1);
-    const int q = lane & 3;
-    float sw = (0.0f + o0) + o1;
-#pragma unroll
-    for (int r = 1; r < 4; ++r) {
-      const float v = prev_lane(sw);
-      if (q == r) sw = (v + o0) + o1;
-    }
-    if (q == 3) ysum[(size_t)m * 512 + hv * 16 + (lane >> 2)] = sw;
+    const float sw = tree_sum<16>(o0 + o1);
+    if ((lane & 15) == 0) ysum[(size_t)m * 128 + hv * 4 + (lane >> 4)] = sw;
   }
 }
 
@@ -880,13 +860,13 @@ struct MoeAArgs {
 constexpr int MOE_A_SHARED_BLOCKS = 64;
 __global__ __launch_bounds__(256) void k_moe_a(MoeAArgs a) {
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float x[32], sx[4];
+  float x[32], sx[1];
   if (a.xn_in) load32(a.xn_in + (size_t)m * H + 32 * lane, x);
   else hidden_prologue(a.ha, m, lane, blockIdx.x == 0 && wave == 0, x);
   // skip_shared: the grid holds the router blocks only
   const int bx = a.skip_shared ? (int)blockIdx.x + MOE_A_SHARED_BLOCKS : (int)blockIdx.x;
   if (bx < MOE_A_SHARED_BLOCKS) {
-    word_sums(x, sx);
+    sx[0] = share_sum(x);
     uint32_t xp[16];
     pack_x(x, xp);
     const size_t i0 = ((size_t)bx * 4 + wave) * 2;
@@ -991,7 +971,7 @@ struct MoeBArgs {
   const uint32_t *g_w, *g_sb, *u_w, *u_sb;   // [E*512, 2048]
   uint16_t* act;               // [M, 8, 512]
   const int32_t* inds;         // [M, 8]
-  const float* xsum;           // [M, 256] word sums of the rows (HiddenArgs::xs_out), or null: formed here
+  const float* xsum;           // [M, 64] share sums of the rows (HiddenArgs::xs_out), or null: formed here
   // a few rows (a verify step): no routing launch before this one; every wave routes its row itself from the logits
   // and workgroup 0 of the row leaves indices and scores for stage C
   const uint16_t* rlogits;     // [M, 256] (k_moe_b<true>; otherwise `inds` holds the routing)
@@ -1056,7 +1036,7 @@ struct MoeBGroupArgs {
   uint16_t* act;               // [M, 8, 512]
   const uint16_t* lists;       // [E, GROUP_CAP] pair indices row*8 + slot
   const int32_t* counts;       // [E]
-  const float* xsum;           // [M, 256] word sums of the rows (HiddenArgs::xs_out), or null: formed here
+  const float* xsum;           // [M, 64] share sums of the rows (HiddenArgs::xs_out), or null: formed here
   const int32_t* order;        // [E] experts by falling count: the long lists start first
   // the shared expert as one more list (every row of the step, in segments of 64 rows that come first in the grid):
   const uint32_t *shg_w, *shg_sb, *shu_w, *shu_sb;   // its gate_proj / up_proj [512, 2048], or null: grid (64, E) only
@@ -1100,17 +1080,17 @@ __global__ __launch_bounds__(256, 3) void k_moe_b_grouped(MoeBGroupArgs a) {
         const uint16_t* src = a.xn + (size_t)(p >> 3) * H + 32 * lane;
 #pragma unroll
         for (int q = 0; q < 4; ++q) dst[q] = ld16(src + 8 * q);
-        dst[4] = ld16(a.xsum + (size_t)(p >> 3) * 256 + 4 * lane);
+        dst[4] = make_uint4(__float_as_uint(a.xsum[(size_t)(p >> 3) * 64 + lane]), 0u, 0u, 0u);
         continue;
       }
-      float x[32], sx[4];
+      float x[32];
       load32(a.xn + (size_t)(p >> 3) * H + 32 * lane, x);
-      word_sums(x, sx);
+      const float sx = share_sum(x);
       uint32_t xp[16];
       pack_x(x, xp);
 #pragma unroll
       for (int q = 0; q < 4; ++q) dst[q] = make_uint4(xp[4 * q], xp[4 * q + 1], xp[4 * q + 2], xp[4 * q + 3]);
-      dst[4] = make_uint4(__float_as_uint(sx[0]), __float_as_uint(sx[1]), __float_as_uint(sx[2]), __float_as_uint(sx[3]));
+      dst[4] = make_uint4(__float_as_uint(sx), 0u, 0u, 0u);
     }
     __syncthreads();
     if (t0 == 0) {
@@ -1127,13 +1107,12 @@ __global__ __launch_bounds__(256, 3) void k_moe_b_grouped(MoeBGroupArgs a) {
     for (int j = 0; j < mc; ++j) {
       const uint4* src = xs + (j * 64 + lane) * 5;
       uint32_t xp[16];
-      float sx[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) { const uint4 v = src[q]; xp[4 * q] = v.x; xp[4 * q + 1] = v.y; xp[4 * q + 2] = v.z; xp[4 * q + 3] = v.w; }
-      { const uint4 v = src[4]; sx[0] = __uint_as_float(v.x); sx[1] = __uint_as_float(v.y); sx[2] = __uint_as_float(v.z); sx[3] = __uint_as_float(v.w); }
+      const float sx = __uint_as_float(reinterpret_cast<const uint32_t*>(src + 4)[0]);
       float o[4];                                          // rows 0..3 in the lower quad of every eight lanes
-      quad_values(tree_sum4(quad_term_masked(mk[0], sb[0], xp, sx), quad_term_masked(mk[1], sb[1], xp, sx),
-                            quad_term_masked(mk[2], sb[2], xp, sx), quad_term_masked(mk[3], sb[3], xp, sx), lane), o);
+      quad_values(tree_sum4(share_term_masked(mk[0], sb[0], xp, sx), share_term_masked(mk[1], sb[1], xp, sx),
+                            share_term_masked(mk[2], sb[2], xp, sx), share_term_masked(mk[3], sb[3], xp, sx), lane), o);
       const bool mine = (lane >> 3) == j;
       G = mine ? ((lane & 1) ? o[1] : o[0]) : G;
       U = mine ? ((lane & 1) ? o[3] : o[2]) : U;
@@ -1169,26 +1148,25 @@ __global__ __launch_bounds__(256) void k_moe_b(MoeBArgs a) {
     gw[r] = ld16(a.g_w + (base + r) * 256 + 4 * lane); gs[r] = a.g_sb[(base + r) * 32 + (lane >> 1)];
     uw[r] = ld16(a.u_w + (base + r) * 256 + 4 * lane); us[r] = a.u_sb[(base + r) * 32 + (lane >> 1)];
   }
-  float sx[4];
+  float sx;
   uint32_t xp[16];
   if (a.xsum) {                                          // the stored halves are the packed pairs
     const uint16_t* src = a.xn + (size_t)m * H + 32 * lane;
 #pragma unroll
     for (int j = 0; j < 4; ++j) { const uint4 v = ld16(src + 8 * j); xp[4 * j] = v.x; xp[4 * j + 1] = v.y; xp[4 * j + 2] = v.z; xp[4 * j + 3] = v.w; }
-    const float4 s4 = *reinterpret_cast<const float4*>(a.xsum + (size_t)m * 256 + 4 * lane);
-    sx[0] = s4.x; sx[1] = s4.y; sx[2] = s4.z; sx[3] = s4.w;
+    sx = a.xsum[(size_t)m * 64 + lane];
   } else {
     float x[32];
     load32(a.xn + (size_t)m * H + 32 * lane, x);
-    word_sums(x, sx);
+    sx = share_sum(x);
     pack_x(x, xp);
   }
   // the four gate sums and the four up sums each reduced in one register: lane r (r < 4) holds row r of both and
   // forms its SwiGLU
-  const float g = tree_sum4(quad_term(gw[0], gs[0], xp, sx), quad_term(gw[1], gs[1], xp, sx),
-                            quad_term(gw[2], gs[2], xp, sx), quad_term(gw[3], gs[3], xp, sx), lane);
-  const float u = tree_sum4(quad_term(uw[0], us[0], xp, sx), quad_term(uw[1], us[1], xp, sx),
-                            quad_term(uw[2], us[2], xp, sx), quad_term(uw[3], us[3], xp, sx), lane);
+  const float g = tree_sum4(share_term(gw[0], gs[0], xp, sx), share_term(gw[1], gs[1], xp, sx),
+                            share_term(gw[2], gs[2], xp, sx), share_term(gw[3], gs[3], xp, sx), lane);
+  const float u = tree_sum4(share_term(uw[0], us[0], xp, sx), share_term(uw[1], us[1], xp, sx),
+                            share_term(uw[2], us[2], xp, sx), share_term(uw[3], us[3], xp, sx), lane);
   const float o = swiglu16(f16r(g), f16r(u));
   if (lane < 4) a.act[((size_t)m * 8 + k) * 512 + i0 + lane] = f2h(o);
 }
@@ -1208,10 +1186,10 @@ struct MoeCArgs {
 };
 // Grid (128, M), four waves: 16 lanes per output row, 16 rows per workgroup.  The nine activation rows (the stored
 // halves as they are) are parked in LDS once per workgroup, 64 bytes per lane at an 80-byte pitch so that the 16 lanes
-// of a row read them without bank conflicts, and their word sums are formed once per workgroup.
+// of a row read them without bank conflicts, and their share sums are formed once per workgroup.
 __global__ __launch_bounds__(256) void k_moe_c(MoeCArgs a) {
   constexpr int XP = 20;                                  // words per lane slot: 16 + 4 pad
-  __shared__ __align__(16) float s_sx[9 * 16 * 4];
+  __shared__ float s_sx[9 * 16];
   __shared__ __align__(16) uint32_t s_x[9 * 16 * XP];
   const int m = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int sub = lane >> 4, li = lane & 15;
@@ -1236,11 +1214,10 @@ __global__ __launch_bounds__(256) void k_moe_c(MoeCArgs a) {
   }
   __syncthreads();
   if (tid < 9 * 16) {
-    float x[32], sx[4];
+    float x[32];
 #pragma unroll
     for (int j = 0; j < 4; ++j) unpack8(ld16(&s_x[tid * XP + 4 * j]), x + 8 * j);
-    word_sums(x, sx);
-    *reinterpret_cast<float4*>(&s_sx[tid * 4]) = make_float4(sx[0], sx[1], sx[2], sx[3]);
+    s_sx[tid] = share_sum(x);
   }
   __syncthreads();
   float acc = 0.0f, sy = 0.0f;
@@ -1249,9 +1226,7 @@ __global__ __launch_bounds__(256) void k_moe_c(MoeCArgs a) {
     uint32_t xp[16];
 #pragma unroll
     for (int j = 0; j < 4; ++j) { const uint4 v = ld16(&s_x[(k * 16 + li) * XP + 4 * j]); xp[4 * j] = v.x; xp[4 * j + 1] = v.y; xp[4 * j + 2] = v.z; xp[4 * j + 3] = v.w; }
-    const float4 s4 = *reinterpret_cast<const float4*>(&s_sx[(k * 16 + li) * 4]);
-    const float sx[4] = {s4.x, s4.y, s4.z, s4.w};
-    const float d = f16r(tree_sum<16>(quad_term(wv[k], sb[k], xp, sx)));
+    const float d = f16r(tree_sum<16>(share_term(wv[k], sb[k], xp, s_sx[k * 16 + li])));
     if (k < 8) acc = f16r(acc + f16r(d * sc[k]));
     else sy = d;
   }
@@ -1264,8 +1239,8 @@ __global__ __launch_bounds__(256) void k_moe_c(MoeCArgs a) {
 // moe_count / moe_csr / gqmm4_grouped, SeedlessMetalForward.swift:3116-3556).  Grid (64, ceil(M / 64) + E): the shared
 // expert's rows in segments of 64, then the experts.  A workgroup holds 32 output rows of its expert, two per group
 // of 16 lanes (K = 512: a lane owns 32 activations), and walks the list in tiles of MOEC_MT pairs whose activation
-// rows are parked in LDS with their word sums.  Same arithmetic per (pair, output row) as k_moe_c:
-// d = half(tree_sum<16>(quad term)).  The results go out by pair (routed) or by row (shared);
+// rows are parked in LDS with their share sums.  Same arithmetic per (pair, output row) as k_moe_c:
+// d = half(tree_sum<16>(share term)).  The results go out by pair (routed) or by row (shared);
 // k_moe_combine_rows adds them up in routing order.
 struct MoeCGroupArgs {
   const uint16_t* act;         // [M, 8, 512]
@@ -1284,7 +1259,7 @@ __global__ __launch_bounds__(256, 3) void k_moe_c_grouped(MoeCGroupArgs a) {
   constexpr int XP = 20;                                  // words per lane slot: 16 + 4 pad
   constexpr int PIECES = MOEC_MT * 64 / 256;              // 16-byte pieces of a tile per thread
   __shared__ __align__(16) uint32_t s_x[MOEC_MT * 16 * XP];
-  __shared__ __align__(16) float s_sx[MOEC_MT * 16 * 4];
+  __shared__ float s_sx[MOEC_MT * 16];
   __shared__ int s_dst[MOEC_MT];
   // blockIdx.y < S: segment of 64 rows of the shared expert (first, and cut up: as one list of M rows it would run
   // thirty times longer than an expert's and end the launch with 64 workgroups); then the experts by falling count
@@ -1331,11 +1306,10 @@ __global__ __launch_bounds__(256, 3) void k_moe_c_grouped(MoeCGroupArgs a) {
     __syncthreads();
     if (t0 + MOEC_MT < cnt) fetch(t0 + MOEC_MT);
     if (tid < mc * 16) {
-      float x[32], sx[4];
+      float x[32];
 #pragma unroll
       for (int q = 0; q < 4; ++q) unpack8(ld16(&s_x[tid * XP + 4 * q]), x + 8 * q);
-      word_sums(x, sx);
-      *reinterpret_cast<float4*>(&s_sx[tid * 4]) = make_float4(sx[0], sx[1], sx[2], sx[3]);
+      s_sx[tid] = share_sum(x);
     }
     if (t0 == 0) {
 #pragma unroll
@@ -1349,10 +1323,9 @@ __global__ __launch_bounds__(256, 3) void k_moe_c_grouped(MoeCGroupArgs a) {
       uint32_t xp[16];
 #pragma unroll
       for (int q = 0; q < 4; ++q) { const uint4 v = ld16(&s_x[(j * 16 + li) * XP + 4 * q]); xp[4 * q] = v.x; xp[4 * q + 1] = v.y; xp[4 * q + 2] = v.z; xp[4 * q + 3] = v.w; }
-      const float4 s4 = *reinterpret_cast<const float4*>(&s_sx[(j * 16 + li) * 4]);
-      const float sx[4] = {s4.x, s4.y, s4.z, s4.w};
-      const float d0 = tree_sum<16>(quad_term_masked(mk[0], sb[0], xp, sx));
-      const float d1 = tree_sum<16>(quad_term_masked(mk[1], sb[1], xp, sx));
+      const float sx = s_sx[j * 16 + li];
+      const float d0 = tree_sum<16>(share_term_masked(mk[0], sb[0], xp, sx));
+      const float d1 = tree_sum<16>(share_term_masked(mk[1], sb[1], xp, sx));
       if (li == 0) {
         uint16_t* dst = (shared ? a.sy : a.d) + (size_t)s_dst[j] * H + n0;
         *reinterpret_cast<uint32_t*>(dst) = pack2(d0, d1);
@@ -1391,10 +1364,7 @@ __global__ __launch_bounds__(64) void k_attn_prep(AttnPrepArgs a) {
   const uint2 wraw = *reinterpret_cast<const uint2*>(nw + 4 * lane);
   const float xv[4] = {lo_h(raw.x), hi_h(raw.x), lo_h(raw.y), hi_h(raw.y)};
   const float wv[4] = {lo_h(wraw.x), hi_h(wraw.x), lo_h(wraw.y), hi_h(wraw.y)};
-  float ss = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) ss = fmaf(xv[i], xv[i], ss);
-  ss = tree_sum<64>(ss);
+  const float ss = tree_sum<64>(fmaf(xv[1], xv[1], xv[0] * xv[0]) + fmaf(xv[3], xv[3], xv[2] * xv[2]));
   const float inv = 1.0f / sqrtf(ss / 256.0f + EPS);
 #pragma unroll
   for (int i = 0; i < 4; ++i) s_n[4 * lane + i] = f16r(wv[i] * f16r(xv[i] * inv));
@@ -1424,9 +1394,9 @@ __global__ __launch_bounds__(64) void k_attn_prep(AttnPrepArgs a) {
 // -------------------------------------------------------------------------------------------------
 // Decode attention, tile pass: one workgroup of four waves per (key tile of 64, kv head, row), a wave per pair of
 // query heads.  The tile's keys are
-// staged in LDS; lane j scores key j against the query heads of its wave (a balanced tree over
-// 64 leaves of 4 dims), then p = exp(s - tile max), l = butterfly sum of p, o = fmaf chain over
-// the tile's keys with the value tile parked in LDS (fetched once per workgroup).  Reference semantics: sdpa_rows
+// staged in LDS; lane j scores key j against the query heads of its wave (eight fmaf chains over 32 dims
+// each, combined by a balanced tree), then p = exp(s - tile max), l = butterfly sum of p, o = two fmaf chains over
+// the halves of the tile's keys with the value tile parked in LDS (fetched once per workgroup).  Reference semantics: sdpa_rows
 // SeedlessMetalForward.swift:4922-4989 (q scaled by 1/16, fp32 softmax).
 // -------------------------------------------------------------------------------------------------
 struct SdpaArgs {
@@ -1472,36 +1442,36 @@ __global__ __launch_bounds__(256) void k_sdpa_tile(SdpaArgs a) {
   __syncthreads();
   const float NEG = -__int_as_float(0x7f800000);
   const int h0 = 2 * wave;
-  // scores: a balanced tree over 64 leaves of 4 dims, eight leaves (one sub-tree) at a time so that the staged
-  // key row is read in step with its use
+  // scores: eight fmaf chains over 32 dims each (the staged key row is read in step with its use, the queries come
+  // as LDS broadcasts), combined by a balanced tree
   float sc[2];
   {
-    float grp[2][8];
+    // (the sixteen chains of a lane advance side by side, four dims at a time: a chain on its own would wait for
+    // every multiply-add before it)
+    float c[2][8];
+#pragma unroll
+    for (int g = 0; g < 8; ++g) { c[0][g] = 0.0f; c[1][g] = 0.0f; }
     const uint16_t* kr = &s_k[(lane < nk ? lane : 0) * KT_STRIDE];
 #pragma unroll
-    for (int g = 0; g < 8; ++g) {
-      float n[2][8];
+    for (int l = 0; l < 8; ++l) {
 #pragma unroll
-      for (int l = 0; l < 8; ++l) {
-        const int leaf = 8 * g + l;
-        const uint2 kraw = *reinterpret_cast<const uint2*>(kr + 4 * leaf);
-        const float kf[4] = {lo_h(kraw.x), hi_h(kraw.x), lo_h(kraw.y), hi_h(kraw.y)};
+      for (int g = 0; g < 8; ++g) {
+        const int d = 32 * g + 4 * l;
+        const uint2 kraw = *reinterpret_cast<const uint2*>(kr + d);
+        const h2_t k01 = as_h2(kraw.x), k23 = as_h2(kraw.y);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          const float4 q4 = *reinterpret_cast<const float4*>(&s_q[(h0 + h) * 256 + 4 * leaf]);
-          float node = fmaf(q4.x, kf[0], 0.0f);
-          node = fmaf(q4.y, kf[1], node);
-          node = fmaf(q4.z, kf[2], node);
-          n[h][l] = fmaf(q4.w, kf[3], node);
+          const float4 q4 = *reinterpret_cast<const float4*>(&s_q[(h0 + h) * 256 + d]);
+          c[h][g] = fmaf(q4.x, (float)k01.x, c[h][g]);
+          c[h][g] = fmaf(q4.y, (float)k01.y, c[h][g]);
+          c[h][g] = fmaf(q4.z, (float)k23.x, c[h][g]);
+          c[h][g] = fmaf(q4.w, (float)k23.y, c[h][g]);
         }
       }
-#pragma unroll
-      for (int h = 0; h < 2; ++h) grp[h][g] = ((n[h][0] + n[h][1]) + (n[h][2] + n[h][3])) + ((n[h][4] + n[h][5]) + (n[h][6] + n[h][7]));
-      asm volatile("" : "+v"(grp[0][g]), "+v"(grp[1][g]) : : "memory");   // both heads' sub-trees end here: nothing is carried along
     }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const float t = ((grp[h][0] + grp[h][1]) + (grp[h][2] + grp[h][3])) + ((grp[h][4] + grp[h][5]) + (grp[h][6] + grp[h][7]));
+      const float t = ((c[h][0] + c[h][1]) + (c[h][2] + c[h][3])) + ((c[h][4] + c[h][5]) + (c[h][6] + c[h][7]));
       sc[h] = (lane < nk) ? t : NEG;
     }
   }
@@ -1518,16 +1488,23 @@ __global__ __launch_bounds__(256) void k_sdpa_tile(SdpaArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) o[h][i] = 0.0f;
   }
-  // Weighted value sums: the chain of fmaf over the tile's keys in order.  All 64 keys are walked: beyond nk the weight
-  // and the parked value are zero, and fmaf(0, 0, o) returns o as it is.  Eight keys at a time: their weights come
-  // over as scalars (lane reads), their value pieces from LDS.
+  // Weighted value sums: one chain of fmaf over the tile's first 32 keys in order, one over its other 32, added at
+  // the end.  All 64 keys are walked: beyond nk the weight and the parked value are zero, and fmaf(0, 0, o) returns o
+  // as it is.  Eight keys at a time: their weights come over as scalars (lane reads), their value pieces from LDS.
   __syncthreads();                                   // every wave is done with the keys
   uint16_t* s_v = s_k;                               // [64][256] halves
 #pragma unroll
   for (int it = 0; it < 8; ++it) st16(&s_v[(it * 8 + (tid >> 5)) * 256 + (tid & 31) * 8], vr[it]);
   __syncthreads();
+  float oa[2][4];
 #pragma unroll
   for (int j0v = 0; j0v < SDPA_TILE; j0v += 8) {
+    if (j0v == SDPA_TILE / 2) {                        // the first half's chain is complete: the second starts from zero
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { oa[h][i] = o[h][i]; o[h][i] = 0.0f; }
+    }
     uint2 vraw[8];
     float pj[2][8];
 #pragma unroll
@@ -1548,7 +1525,8 @@ __global__ __launch_bounds__(256) void k_sdpa_tile(SdpaArgs a) {
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const size_t pi = ((size_t)m * 16 + kvh * 8 + h0 + h) * a.maxTiles + tile;
-    *reinterpret_cast<float4*>(a.po + pi * 256 + 4 * lane) = make_float4(o[h][0], o[h][1], o[h][2], o[h][3]);
+    *reinterpret_cast<float4*>(a.po + pi * 256 + 4 * lane) =
+        make_float4(oa[h][0] + o[h][0], oa[h][1] + o[h][1], oa[h][2] + o[h][2], oa[h][3] + o[h][3]);
   }
 }
 
@@ -1561,7 +1539,7 @@ struct SdpaMergeArgs {
   const int32_t* st;
   int maxTiles;
   uint16_t* gated;             // [M, 4096]
-  float* gsum;                 // [M, 512] word sums of the gated rows for the projection that follows (k_sdpa_merge), or null
+  float* gsum;                 // [M, 128] share sums of the gated rows for the projection that follows (k_sdpa_merge), or null
   const LaneRef* lanes;
   int group = 0;               // > 1: one partial per `group` key tiles at index tile / group (k_sdpa_merge_par only)
 };
@@ -1599,10 +1577,9 @@ __global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) r[i] = f16r(f16r(O[i] / L) * sigmoid16(gt[i]));
   *reinterpret_cast<uint2*>(a.gated + (size_t)m * 4096 + h * 256 + 4 * lane) = make_uint2(pack2(r[0], r[1]), pack2(r[2], r[3]));
-  if (a.gsum) {                                          // a run of 8 values sits on two neighbouring lanes
-    const float v = prev_lane(((0.0f + r[0]) + r[1]) + r[2] + r[3]);
-    const float sw = (lane & 1) ? (((v + r[0]) + r[1]) + r[2]) + r[3] : 0.0f;
-    if (lane & 1) a.gsum[(size_t)m * 512 + h * 32 + (lane >> 1)] = sw;
+  if (a.gsum) {                                          // a share of 32 values sits on eight neighbouring lanes
+    const float sw = tree_sum<8>((r[0] + r[1]) + (r[2] + r[3]));
+    if ((lane & 7) == 0) a.gsum[(size_t)m * 128 + h * 8 + (lane >> 3)] = sw;
   }
 }
 
@@ -1617,9 +1594,9 @@ __global__ __launch_bounds__(256) void k_head(HiddenArgs ha, const uint32_t* __r
   __shared__ float s_v[4];
   __shared__ int s_i[4];
   const int m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float x[32], sx[4];
+  float x[32], sx[1];
   hidden_prologue(ha, m, lane, blockIdx.x == 0 && wave == 0, x);
-  word_sums(x, sx);
+  sx[0] = share_sum(x);
   uint32_t xp[16];
   pack_x(x, xp);
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * 4;

@@ -71,6 +71,9 @@ SIGNATURES = {
     "sl_debug_set_spin_limit": (_i32, [_vp, C.c_uint32]),
     "sl_debug_set_flow_counter": (_i32, [_vp, C.c_uint32]),
     "sl_debug_flow_tags": (_i32, [C.c_uint32, _i32, _i32, _i32, _i32, _vp, _vp]),
+    "sl_ubench_exchange": (_i32, [_i32, _i32, C.POINTER(_f32)]),
+    "sl_ubench_gemv_stream": (_i32, [_i32, _i32, C.POINTER(_f32)]),
+    "sl_ubench_mfma_issue": (_i32, [_i32, _i32, _i32, C.POINTER(_f32), C.POINTER(_f32)]),
     "sl_profile_head": (_i32, [_vp, _i32]),
     "sl_profile_head_read": (_i32, [_vp, C.POINTER(C.c_double), C.POINTER(_i64)]),
     "sl_selftest_math": (_i32, [_i32, _vp, _vp, _i64]),
