@@ -123,7 +123,7 @@ __shared__ Lds g_L;
 extern __shared__ __align__(16) uint16_t g_vt[];   // dynamic: staged value tile [64][256] halves, then the softmax
                                                    // weights of up to SDPA_ROUND (tile, kv head) units [8 heads][64 keys]
 constexpr int SDPA_ROUND = 20;
-constexpr int DEC_DYN_LDS = SDPA_TILE * 256 * 2 + SDPA_ROUND * 8 * 64 * 4;
+constexpr int DEC_DYN_LDS = SDPA_TILE * 256 * 2 + SDPA_ROUND * 8 * 64 * 4 + 4096;   // (+ room for the rows parked ahead of their stage)
 
 SL_DEV void lds_get_x(int b, int lane, uint32_t* xp, float& sx) {
 #pragma unroll

@@ -54,6 +54,7 @@ struct LayerDev {
 constexpr size_t HIST_ELEMS = (size_t)(SL_CONV_K - 1) * SL_CONV_DIM;
 constexpr size_t STATE_ELEMS = (size_t)SL_GDN_HV * SL_GDN_D * SL_GDN_D;
 constexpr int MAX_CHAIN = 256;
+constexpr int MERGE_LONG_ROWS = 64;      // steps of up to this many rows merge their attention tiles with the 16-wave kernel
 constexpr int ROUTER_PAD_ROWS = 288;
 
 // The single-launch step is a grid of workgroups that wait for each other's results without a grid barrier: it
@@ -492,6 +493,7 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
   g.gsum = mm ? nullptr : e->ysum;                       // the exact merge leaves the gated rows' word sums for the projection
   if (mm && lanes) hipLaunchKernelGGL(k_sdpa_merge_par<16>, dim3(SL_ATT_HEADS, M), dim3(1024), 0, e->stream, g);
   else if (mm) hipLaunchKernelGGL(k_sdpa_merge_par<4>, dim3(SL_ATT_HEADS, M), dim3(256), 0, e->stream, g);
+  else if (M <= MERGE_LONG_ROWS) hipLaunchKernelGGL(k_sdpa_merge_long, dim3(SL_ATT_HEADS, M), dim3(1024), MERGE_DYN_LDS, e->stream, g);
   else hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
   if (mm && !(lanes && M < MM_OUT_ROWS)) launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.o_proj.w, L.o_proj.sb, M, H, 4096, e->mix, H}, e->stream);
   else if (M >= 2) hipLaunchKernelGGL((k_qmv_tile<2, 2, 4, false>), dim3(H / 8, (M + 3) / 4), dim3(256), 0, e->stream, HiddenArgs{}, e->ycore, 4096,
@@ -733,6 +735,7 @@ int alloc_runtime(sl_engine* e) {
   const bool has_head = e->has_head;
   struct { int n_layers, vocab; } dd = {e->n_layers, e->vocab};
   const auto* d = &dd;
+  SL_TRY(e, hipFuncSetAttribute((const void*)k_sdpa_merge_long, hipFuncAttributeMaxDynamicSharedMemorySize, MERGE_DYN_LDS));
   if (has_head) {
     e->n_cand = d->vocab / 16;
     e->logits = dalloc<uint16_t>(e, (size_t)max_m * d->vocab);

@@ -208,15 +208,13 @@ constexpr int PAIR_WAVE0 = 160 * DEC_WAVES;      // first wave of the shared gat
 // routing and whose stage starts with a long hand-over therefore travel one to three stages ahead, straight into LDS
 // (global_load_lds_dwordx4: no registers are held meanwhile): the in-projection rows of layer l+1 are requested when
 // a workgroup is through with the K = 4096 projection of layer l (the upper half of the grid has no rows there and
-// starts at once), a GDN layer's out-projection rows when its in-projection is done.  The ring lies in the dynamic
+// starts at once), a GDN layer's out-projection rows when its recurrence stage begins (by the waves that do not poll
+// there).  The ring lies in the dynamic
 // LDS behind stage C's activation rows; only attention's tile stage uses that space otherwise, and no row is parked
-// across it.  A wave reads back only rows it requested itself, after waiting for its own loads (vmcnt).
-#ifndef SL_WRING
-#define SL_WRING 1
-#endif
+// across it.  A wave reads back rows it requested itself after waiting for its own loads (vmcnt); rows requested by
+// another wave after that wave's wait and a barrier.
 constexpr int WR_OFF = 12288;                    // bytes into g_vt (stage C's rows take 9 * 16 * XC_STRIDE words = 11520 bytes)
 constexpr int WR_SLOTS = DEC_WAVES * 3 + 1;      // three rows of 1 KB per wave, and the b / a row of a GDN in-projection
-static_assert(WR_OFF + WR_SLOTS * 1024 <= DEC_DYN_LDS, "the ring fits the dynamic LDS");
 SL_DEV void wr_request(int slot, const uint32_t* row_words, int lane) {
   typedef __attribute__((address_space(3))) void* lds_ptr;
   typedef const __attribute__((address_space(1))) void* glb_ptr;
@@ -225,6 +223,22 @@ SL_DEV void wr_request(int slot, const uint32_t* row_words, int lane) {
 SL_DEV uint4 wr_read(int slot, int lane) {
   return *reinterpret_cast<const uint4*>(reinterpret_cast<const unsigned char*>(g_vt) + WR_OFF + slot * 1024 + 16 * lane);
 }
+// The rows' {scale, bias} words travel with them: 32 words per row of 2048 weights, lane l < 32 fetches word l.
+constexpr int SBR_OFF = WR_OFF + WR_SLOTS * 1024;
+SL_DEV void sbr_request(int slot, const uint32_t* sb_words, int lane) {
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  typedef const __attribute__((address_space(1))) void* glb_ptr;
+  if (lane < 32)
+    __builtin_amdgcn_global_load_lds((glb_ptr)(sb_words + lane), (lds_ptr)(reinterpret_cast<unsigned char*>(g_vt) + SBR_OFF + slot * 128), 4, 0, 0);
+}
+SL_DEV uint32_t sbr_read(int slot, int lane) {
+  return *reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned char*>(g_vt) + SBR_OFF + slot * 128 + 4 * (lane >> 1));
+}
+// A GDN layer's conv taps and the history rows of the channels a workgroup's recurrence unit needs (threads 0..271:
+// five waves) are parked the same way while the in-projection runs: [wave][64 lanes] conv weights (16 bytes), then
+// three rows of [wave][64 lanes] history words (the word that holds the channel's half).
+constexpr int CVW_OFF = SBR_OFF + WR_SLOTS * 128, CVH_OFF = CVW_OFF + 5 * 1024, CV_END = CVH_OFF + 3 * 5 * 256;
+static_assert(CV_END <= DEC_DYN_LDS, "the parked rows fit the dynamic LDS");
 // Before a wave reads rows it requested: its loads have landed (the compiler does not know that they write LDS).
 SL_DEV void wr_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
@@ -297,6 +311,25 @@ SL_DEV InRows in_rows(bool lin, int wg, int wave) {
   }
   return r;
 }
+// The channel a thread of a GDN recurrence unit looks after (threads 0..271: 128 query, 128 key, 16 value channels).
+SL_DEV int gdn_unit_channel(int wg, int tid) {
+  const int hv = gdn_unit_head(wg), dvb = gdn_unit_dvb(wg), hk = hv >> 1;
+  return tid < 128 ? hk * 128 + tid : (tid < 256 ? 2048 + hk * 128 + (tid - 128) : 4096 + hv * 128 + dvb * 16 + (tid - 256));
+}
+SL_DEV void flow_request_conv(const LayerP& Y, int li) {
+  FLOW_IDS;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  typedef const __attribute__((address_space(1))) void* glb_ptr;
+  if (wave < 5) {
+    const int ch = gdn_unit_channel(wg, min(tid, 271));
+    unsigned char* const lds = reinterpret_cast<unsigned char*>(g_vt);
+    const uint16_t* hin = uni(Y.hist[(int)((uni(g_K.parity) >> li) & 1ull)]);
+    __builtin_amdgcn_global_load_lds((glb_ptr)(uni(Y.conv_w) + ch * 4), (lds_ptr)(lds + CVW_OFF + wave * 1024), 16, 0, 0);
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+      __builtin_amdgcn_global_load_lds((glb_ptr)(hin + k * SL_CONV_DIM + (ch & ~1)), (lds_ptr)(lds + CVH_OFF + (k * 5 + wave) * 256), 4, 0, 0);
+  }
+}
 template <bool ST>
 SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base, float& h0, float& h1, int step) {
   FLOW_IDS;
@@ -307,13 +340,9 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   WRegs<1, 3> wr;
 #pragma unroll
   for (int j = 0; j < 3; ++j) {
-#if SL_WRING
-    // the rows themselves were requested into LDS stages ago (flow_request_in); only their scales and biases come now
+    // (the rows and their scales were requested into LDS stages ago, flow_request_in: read back after the prologue)
     wr.w[j][0] = make_uint4(0, 0, 0, 0);
-    wr.sb[j][0] = j < rows.ncrit ? uni(Y.in_sb)[(size_t)rows.crit[j] * 32 + (lane >> 1)] : 0u;
-#else
-    wload_row<1>(wr.w[j], wr.sb[j], uni(Y.in_w), uni(Y.in_sb), (size_t)rows.crit[j], j < rows.ncrit, lane);
-#endif
+    wr.sb[j][0] = 0u;
   }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.input_ln) + 2 * tid);
   float r0 = 0.0f, r1 = 0.0f;
@@ -348,24 +377,19 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   }
   // the deferred row (no branch around the load: the waits that follow stay exact)
   uint4 wd; uint32_t sbd;
-#if SL_WRING
   wd = make_uint4(0, 0, 0, 0);
-  sbd = uni(Y.in_sb)[(size_t)rows.def * 32 + (lane >> 1)];
-#else
-  wload_row<1>(&wd, &sbd, uni(Y.in_w), uni(Y.in_sb), (size_t)rows.def, true, lane);
-#endif
+  sbd = 0u;
+  if (lin) flow_request_conv(Y, li);             // behind the poll, to arrive while this stage computes
   const uint32_t tin = flow_tag(base, li, FS_IN);
   flow_prologue(h0, h1, li > 0, r0, r1, lnw, nullptr);
   fstamp<ST>(li, FS_IN, 2, tid == 0);
   uint32_t x[16]; float sx;
   lds_get_x(0, lane, x, sx);
-#if SL_WRING
   wr_wait();
-  wr.w[0][0] = wr_read(wave * 3, lane);
-  if (rows.ncrit >= 2) wr.w[1][0] = wr_read(wave * 3 + 1, lane);
-  if (rows.ncrit >= 3) wr.w[2][0] = wr_read(DEC_WAVES * 3, lane);
-  wd = wr_read(wave * 3 + 2, lane);
-#endif
+  wr.w[0][0] = wr_read(wave * 3, lane); wr.sb[0][0] = sbr_read(wave * 3, lane);
+  if (rows.ncrit >= 2) { wr.w[1][0] = wr_read(wave * 3 + 1, lane); wr.sb[1][0] = sbr_read(wave * 3 + 1, lane); }
+  if (rows.ncrit >= 3) { wr.w[2][0] = wr_read(DEC_WAVES * 3, lane); wr.sb[2][0] = sbr_read(DEC_WAVES * 3, lane); }
+  wd = wr_read(wave * 3 + 2, lane); sbd = sbr_read(wave * 3 + 2, lane);
   {
     // urgent rows: slot of row j = first slot of the wave + j (the extra b / a row: slot 32)
     const int slot0 = lin ? 2 * wave : (wave < 4 ? 2 * wave : 4 + wave);
@@ -402,30 +426,19 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
     stw1(co_rsrc(uni(F.tproj)), lin ? 8192 + zi : attn_gate_row(zi), g_L.pub[40 + lane]);
   }
   fstamp<ST>(li, FS_IN, 5, tid == PUB_WAVE * 64);
-#if SL_WRING
-  // a GDN layer's K = 4096 projection row of this wave (2 KB) takes the places of the rows just used
-  if (lin && gw < H) {
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // (the rows just read are in registers)
-    wr_request(wave * 3, uni(Y.out_w) + (size_t)gw * 512, lane);
-    wr_request(wave * 3 + 1, uni(Y.out_w) + (size_t)gw * 512 + 256, lane);
-  }
-#endif
   return true;
 }
 // Requests the in-projection rows of layer Y for this wave into the ring (the rows in_rows() deals out).
 SL_DEV void flow_request_in(const LayerP& Y) {
-#if SL_WRING
   FLOW_IDS;
   const InRows rows = in_rows(uni(Y.is_linear) != 0, wg, wave);
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // whatever this wave last read from its places is in registers
   const uint32_t* W = uni(Y.in_w);
-  wr_request(wave * 3, W + (size_t)rows.crit[0] * 256, lane);
-  if (rows.ncrit >= 2) wr_request(wave * 3 + 1, W + (size_t)rows.crit[1] * 256, lane);
-  if (rows.ncrit >= 3) wr_request(DEC_WAVES * 3, W + (size_t)rows.crit[2] * 256, lane);
-  wr_request(wave * 3 + 2, W + (size_t)rows.def * 256, lane);
-#else
-  (void)Y;
-#endif
+  const uint32_t* SB = uni(Y.in_sb);
+  wr_request(wave * 3, W + (size_t)rows.crit[0] * 256, lane); sbr_request(wave * 3, SB + (size_t)rows.crit[0] * 32, lane);
+  if (rows.ncrit >= 2) { wr_request(wave * 3 + 1, W + (size_t)rows.crit[1] * 256, lane); sbr_request(wave * 3 + 1, SB + (size_t)rows.crit[1] * 32, lane); }
+  if (rows.ncrit >= 3) { wr_request(DEC_WAVES * 3, W + (size_t)rows.crit[2] * 256, lane); sbr_request(DEC_WAVES * 3, SB + (size_t)rows.crit[2] * 32, lane); }
+  wr_request(wave * 3 + 2, W + (size_t)rows.def * 256, lane); sbr_request(wave * 3 + 2, SB + (size_t)rows.def * 32, lane);
 }
 
 // ---- GDN stage 2: conv + prep + gated delta rule ------------------------------------------------------
@@ -441,7 +454,6 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
   Lds& L = g_L;
   if (wg >= 256) return true;
   const int par = (int)((uni(g_K.parity) >> li) & 1ull);
-  const uint16_t* hin = uni(Y.hist[par]);
   const int hv = gdn_unit_head(wg), dvb = gdn_unit_dvb(wg), hk = hv >> 1;
   const int half = lane >> 5, l32 = lane & 31;
   // waves 8..15 hold the recurrent state (they take no part in this stage's poll)
@@ -450,6 +462,20 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
     const int dv = dvb * 16 + (wave - 8) * 2 + half;
     const float4 v4 = *reinterpret_cast<const float4*>(uni(Y.state[par]) + ((size_t)hv * 128 + dv) * 128 + 4 * l32);
     s[0] = v4.x; s[1] = v4.y; s[2] = v4.z; s[3] = v4.w;
+    // The workgroup's rows of the K = 4096 projection (2 KB per wave) set out for LDS now, into the places of the
+    // in-projection rows.  The state waves request them, their own and those of the wave eight below: they take no
+    // part in this stage's poll, which would otherwise return behind the rows.
+    if (wg * DEC_WAVES < H) {
+#pragma unroll
+      for (int o = 0; o < 2; ++o) {
+        const int w = wave - 8 * o;
+        const size_t row = (size_t)(wg * DEC_WAVES + w);
+        wr_request(w * 3, uni(Y.out_w) + row * 512, lane);
+        wr_request(w * 3 + 1, uni(Y.out_w) + row * 512 + 256, lane);
+        sbr_request(w * 3, uni(Y.out_sb) + row * 64, lane);
+        sbr_request(w * 3 + 1, uni(Y.out_sb) + row * 64 + 32, lane);
+      }
+    }
   }
   int ch = -1;
   if (tid < 128) ch = hk * 128 + tid;
@@ -463,15 +489,9 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
   // the decay's constants of this head do not depend on the projection: fetched and exponentiated ahead of the wait
   float decay_rate = 0.0f, dt_bias = 0.0f;
   if (tid == DECAY_TID) { decay_rate = exp_c(uni(Y.a_log)[hv]); dt_bias = uni(Y.dt_bias)[hv]; }
-  // history taps stay raw until the wait is over: converting them here would wait for the loads
+  // history taps and conv weights were parked in LDS while the in-projection ran (flow_request_conv): read after the poll
   uint16_t traw[3] = {0, 0, 0};
   float cw[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (tid < 272) {
-#pragma unroll
-    for (int k = 0; k < 3; ++k) traw[k] = hin[k * SL_CONV_DIM + ch];
-    const float4 c4 = *reinterpret_cast<const float4*>(uni(Y.conv_w) + ch * 4);
-    cw[0] = c4.x; cw[1] = c4.y; cw[2] = c4.z; cw[3] = c4.w;
-  }
   float newest = 0.0f;
   {
     const uint32_t tin = flow_tag(base, li, FS_IN);
@@ -482,6 +502,17 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
           return got;
         }, uni(P.bar) + 32)) return false;
     fstamp<ST>(li, FS_CORE, 1, tid == 0);
+  }
+  if (tid < 272) {
+    wr_wait();
+    const unsigned char* const lds = reinterpret_cast<const unsigned char*>(g_vt);
+    const float4 c4 = *reinterpret_cast<const float4*>(lds + CVW_OFF + wave * 1024 + 16 * lane);
+    cw[0] = c4.x; cw[1] = c4.y; cw[2] = c4.z; cw[3] = c4.w;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const uint32_t hw = *reinterpret_cast<const uint32_t*>(lds + CVH_OFF + (k * 5 + wave) * 256 + 4 * lane);
+      traw[k] = (uint16_t)((ch & 1) ? (hw >> 16) : (hw & 0xffffu));
+    }
   }
   const float tap[3] = {h2f(traw[0]), h2f(traw[1]), h2f(traw[2])};
   if (tid < 272) {
@@ -607,7 +638,8 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       const int j0 = tile * SDPA_TILE, nk = min(SDPA_TILE, N - j0);
       const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
       lds_barrier();                    // the key tile aliases the activation vector the in-projection just read
-      put(true, r == 0, u);
+      // (the tile travelling in registers is parked behind the poll below: parked first, the poll would only start
+      // once the tile has arrived)
       // waves 0..7: query heads of the group; wave 8: new key; wave 9: new value -- 4 tagged words per lane
       const int src = wave < 8 ? (kvh * 8 + wave) * 512 : (wave == 8 ? 8192 + kvh * 256 : 8192 + 512 + kvh * 256);
       if (kvh != prep_kvh) {
@@ -651,6 +683,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
           vn[kvh * 128 + 2 * lane + 1] = (w4.z & 0xffffu) | (w4.w << 16);
         }
       }
+      put(true, r == 0, u);
       if (has_new && wave == 8) {         // the unit whose tile holds the new position: its key row
         float o[4];
 #pragma unroll
@@ -771,16 +804,14 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
   const bool has_new = (pos >= j0) && (pos < j0 + SDPA_TILE);
   const uint16_t* kbase = uni(Y.kcache) + ((size_t)kvh * uni(P.max_seq) + j0) * 256;
   const uint16_t* vbase = uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + j0) * 256;
-  lds_barrier();                    // the key tile aliases the activation vector the in-projection just read
+  // The unit's key and value tile: requested now, parked in LDS once the poll below is over.  (Parked first, the
+  // poll would only start when the tile has arrived, and the stage would pay the tile's latency and then the poll's.)
+  uint4 kq[2], vq[2];
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
-    const int row = it * 32 + (tid >> 5), c8 = (tid & 31) * 8;
-    if (row < nk && j0 + row != pos) {
-      st16(&L.kt[row * KT_STRIDE + c8], ld16(kbase + (size_t)row * 256 + c8));
-      st16(&g_vt[row * 256 + c8], ld16(vbase + (size_t)row * 256 + c8));
-    } else if (row >= nk) {
-      st16(&g_vt[row * 256 + c8], make_uint4(0, 0, 0, 0));         // weight 0 times value 0 leaves a sum as it is
-    }
+    const int row = min(it * 32 + (tid >> 5), nk - 1), c8 = (tid & 31) * 8;       // (rows beyond the context repeat its last row: not stored)
+    kq[it] = ld16(kbase + (size_t)row * 256 + c8);
+    vq[it] = ld16(vbase + (size_t)row * 256 + c8);
   }
   // waves 0,1: the unit's two query heads; wave 8: new key; wave 9: new value -- 4 tagged words per lane
   const bool fetches = wave < 2 || wave == 8 || wave == 9;
@@ -806,6 +837,17 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
           return tag_ok(w4.x, tin) && tag_ok(w4.y, tin) && tag_ok(w4.z, tin) && tag_ok(w4.w, tin);
         }, uni(P.bar) + 32)) return false;
     fstamp<ST>(li, FS_CORE, 1, tid == 0);
+  }
+  // (the poll's barrier is behind us: the key tile aliases the activation vector the in-projection read)
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int row = it * 32 + (tid >> 5), c8 = (tid & 31) * 8;
+    if (row < nk && j0 + row != pos) {
+      st16(&L.kt[row * KT_STRIDE + c8], kq[it]);
+      st16(&g_vt[row * 256 + c8], vq[it]);
+    } else if (row >= nk) {
+      st16(&g_vt[row * 256 + c8], make_uint4(0, 0, 0, 0));         // weight 0 times value 0 leaves a sum as it is
+    }
   }
   if (wave < 2 || wave == 8) {
     const bool isq = wave < 2;
@@ -935,13 +977,10 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   const float NEG = -__int_as_float(0x7f800000);
   WRegs<2, 1> wr;
   const bool valid = gw < H;
-#if SL_WRING
   if (lin) {           // the row was requested into LDS when the in-projection ended; its scales and biases come now
     wr.w[0][0] = wr.w[0][1] = make_uint4(0, 0, 0, 0);
-#pragma unroll
-    for (int b = 0; b < 2; ++b) wr.sb[0][b] = valid ? uni(Y.out_sb)[(size_t)gw * 64 + b * 32 + (lane >> 1)] : 0u;
+    wr.sb[0][0] = wr.sb[0][1] = 0u;
   } else
-#endif
   wload_row<2>(wr.w[0], wr.sb[0], uni(Y.out_w), uni(Y.out_sb), (size_t)(valid ? gw : 0), valid, lane);
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
@@ -981,14 +1020,20 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
         float pm[8];
         unsigned have = 0, spins = 0;
         for (;;) {
+          uint4 mq[8];
+          const unsigned missing = ~have;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {                    // all requests of an attempt first, then the looks at them
+            const int t = t0 + 64 * j + lane;
+            mq[j] = make_uint4(0u, 0u, tcore32, tcore32);
+            if ((missing & (1u << j)) && t < nt) mq[j] = ldw4(rml, (slot0 + t) * 4);
+          }
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
-            if (have & (1u << j)) continue;
+            if (!(missing & (1u << j))) continue;
             const int t = t0 + 64 * j + lane;
-            bool ok = true;
-            pm[j] = NEG;
-            if (t < nt) { const uint4 m = ldw4(rml, (slot0 + t) * 4); ok = m.z == tcore32 && m.w == tcore32; pm[j] = __uint_as_float(m.x); }
-            if (__all(ok ? 1 : 0)) have |= 1u << j;
+            pm[j] = t < nt ? __uint_as_float(mq[j].x) : NEG;
+            if (__all((mq[j].z == tcore32 && mq[j].w == tcore32) ? 1 : 0)) have |= 1u << j;
           }
           if (have == 0xffu) break;
           if (++spins > uni(F.spin_limit)) { fail = 1; break; }
@@ -1004,28 +1049,29 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
         bool mdone = false, gdone = false;
         unsigned have = 0, spins = 0;
         for (;;) {
-          if (!mdone) {
-            bool ok = true;
-            if (mine) { m0 = ldw4(rml, (slot0 + lane) * 4); ok = m0.z == tcore32 && m0.w == tcore32; }
-            mdone = __all(ok ? 1 : 0) != 0;
-          }
-          if (!gdone) {
-            if (act) g2 = ldw2(rp, h * 512 + 256 + 2 * chunk);
+          // every piece still missing is requested first and looked at afterwards: with a look behind each request the
+          // round trips of an attempt would follow one another (up to fourteen of them)
+          const bool want_m = !mdone, want_g = !gdone;
+          const unsigned missing = ~have;
+          if (want_m && mine) m0 = ldw4(rml, (slot0 + lane) * 4);
+          if (want_g && act) g2 = ldw2(rp, h * 512 + 256 + 2 * chunk);
+#pragma unroll
+          for (int u = 0; u < MB; ++u)
+            if (u < cnt0 && (missing & (1u << u)) && act) a[u] = ldw4(rpo, ((slot0 + u) * 128 + chunk) * 4);
+          if (want_m) mdone = __all((!mine || (m0.z == tcore32 && m0.w == tcore32)) ? 1 : 0) != 0;
+          if (want_g) {
             gdone = __all((!act || (tag_ok(g2.x, tin) && tag_ok(g2.y, tin))) ? 1 : 0) != 0;
             // the gate was published a stage earlier: its sigmoids are formed while the tiles are still on their way
             if (gdone) { sg0 = sigmoid16(lo_h(g2.x)); sg1 = sigmoid16(lo_h(g2.y)); }
           }
 #pragma unroll
-          for (int u = 0; u < MB; ++u) {
-            if (u < cnt0 && !(have & (1u << u))) {
-              if (act) a[u] = ldw4(rpo, ((slot0 + u) * 128 + chunk) * 4);
-              if (__all((!act || (a[u].z == tcore32 && a[u].w == tcore32)) ? 1 : 0)) have |= 1u << u;
-            }
-          }
+          for (int u = 0; u < MB; ++u)
+            if (u < cnt0 && (missing & (1u << u)) && __all((!act || (a[u].z == tcore32 && a[u].w == tcore32)) ? 1 : 0)) have |= 1u << u;
           if (mdone && gdone && have == (1u << cnt0) - 1u) break;
           if (++spins > uni(F.spin_limit)) { fail = 1; break; }
         }
         Mx = fmaxf(Mx, tree_max<64>(mine ? __uint_as_float(m0.x) : NEG));
+        fstamp<ST>(li, FS_MERGE, 1, lane == 0);
       }
       if (!fail) {                                          // the first batch is already here
         float fl = 0.0f, pl = 0.0f;
@@ -1043,6 +1089,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
             O0 = fmaf(__uint_as_float(a[u].x), f[u], O0); O1 = fmaf(__uint_as_float(a[u].y), f[u], O1);
           }
         }
+        fstamp<ST>(li, FS_MERGE, 3, lane == 0);
       }
     }
     if (nt > MB) {                                          // uniform for the grid
@@ -1181,16 +1228,23 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   // every thread prepares 4 consecutive elements of the 4096-long activation and polls them itself
   const int e0 = 256 * wave + 4 * lane;
   float out[4], sz[4] = {0.0f, 0.0f, 0.0f, 0.0f};            // sz: z * sigmoid(z) of the gate values
+  // the gated norm's weights do not depend on the hand-over: requested ahead of the poll, which outlasts them
+  float4 wraw = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  if (lin) wraw = *reinterpret_cast<const float4*>(uni(Y.gdn_norm_w) + (e0 & 127));
   {
     const uint32_t ty = lin ? tcore : tmerge;
     const rsrc_t ry = co_rsrc(uni(F.tycore)), rz = co_rsrc(uni(F.tproj));
     uint4 a = make_uint4(0, 0, 0, 0);
     bool zdone = false, ydone = false;                    // what has arrived is not fetched again
     if (!flow_poll(true, [&]() {
-          if (!ydone) { a = ldw4(ry, e0); ydone = tag_ok(a.x, ty) && tag_ok(a.y, ty) && tag_ok(a.z, ty) && tag_ok(a.w, ty); }
+          // (both requests first, then the looks at them: one round trip per attempt)
+          const bool want_y = !ydone, want_z = lin && !zdone;
+          uint4 b = make_uint4(0, 0, 0, 0);
+          if (want_y) a = ldw4(ry, e0);
+          if (want_z) b = ldw4(rz, 8192 + e0);
+          if (want_y) ydone = tag_ok(a.x, ty) && tag_ok(a.y, ty) && tag_ok(a.z, ty) && tag_ok(a.w, ty);
           bool ok = ydone;
-          if (lin && !zdone) {                      // the gate values were published a stage earlier: fetched once
-            const uint4 b = ldw4(rz, 8192 + e0);
+          if (want_z) {                             // the gate values were published a stage earlier: fetched once
             zdone = tag_ok(b.x, tin) && tag_ok(b.y, tin) && tag_ok(b.z, tin) && tag_ok(b.w, tin);
             ok = ok && zdone;
             if (zdone) {
@@ -1207,7 +1261,6 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     out[0] = lo_h(a.x); out[1] = lo_h(a.y); out[2] = lo_h(a.z); out[3] = lo_h(a.w);
   }
   if (lin) {
-    const float4 wraw = *reinterpret_cast<const float4*>(uni(Y.gdn_norm_w) + (e0 & 127));
     const float nw[4] = {wraw.x, wraw.y, wraw.z, wraw.w};
     const bool nf32 = uni(Y.gdn_norm_f32) != 0;
     const float la = fmaf(out[1], out[1], fmaf(out[0], out[0], 0.0f));
@@ -1228,11 +1281,13 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     const float ssum = tree_sum<8>((out[0] + out[1]) + (out[2] + out[3]));
     if ((lane & 7) == 0) g_L.sxs[64 * b + lo] = ssum;
   }
+  if (lin) wr_wait();          // the rows this wave requested for the workgroup have landed (the barrier hands them on)
   lds_barrier();
   fstamp<ST>(li, FS_OUT, 2, tid == 0);
-#if SL_WRING
-  if (lin) { wr_wait(); wr.w[0][0] = wr_read(wave * 3, lane); wr.w[0][1] = wr_read(wave * 3 + 1, lane); }
-#endif
+  if (lin) {
+    wr.w[0][0] = wr_read(wave * 3, lane); wr.w[0][1] = wr_read(wave * 3 + 1, lane);
+    wr.sb[0][0] = sbr_read(wave * 3, lane); wr.sb[0][1] = sbr_read(wave * 3 + 1, lane);
+  }
   const float o = dot_2x1(wr);
   fstamp<ST>(li, FS_OUT, 3, tid == 0);
   if (wg * DEC_WAVES < H) {                       // uniform per workgroup
@@ -1466,12 +1521,22 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     float psum[2] = {0.0f, 0.0f};                 // sum of the chunk's two pair sums
     flow_poll<false>(true, [&]() {
       bool ok = true;
+      // (the requests of an attempt first, then the looks at them: one round trip per attempt)
+      const bool want[2] = {!have[0], !have[1]};
+      uint4 q4[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+      uint32_t gw1 = 0;
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
-        if (have[c]) continue;
+        const int t = tid + 1024 * c, slot = t >> 7;
+        if (want[c]) q4[c] = (slot < 8) ? ldw4(ra, 4 * t) : ldw4(rs, 4 * (t & 127));
+      }
+      if (tid == 0) gw1 = ldw1(rg, 0);
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        if (!want[c]) continue;
         // chunk t holds elements 4(t%128).. of slot t/128 (slot 8 = shared): packed pairs 2(t%128), 2(t%128)+1
         const int t = tid + 1024 * c, slot = t >> 7, pi = 2 * (t & 127);
-        const uint4 a4 = (slot < 8) ? ldw4(ra, 4 * t) : ldw4(rs, 4 * (t & 127));
+        const uint4 a4 = q4[c];
         const uint32_t tx = (slot < 8) ? tb : ta;
         have[c] = tag_ok(a4.x, tx) && tag_ok(a4.y, tx) && tag_ok(a4.z, tx) && tag_ok(a4.w, tx);
         ok = ok && have[c];
@@ -1479,7 +1544,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
         *reinterpret_cast<uint2*>(&xc[(slot * 16 + (pi >> 4)) * XC_STRIDE + (pi & 15)]) =
             make_uint2((a4.x & 0xffffu) | (a4.y << 16), (a4.z & 0xffffu) | (a4.w << 16));
       }
-      if (tid == 0) { const uint32_t w = ldw1(rg, 0); ok = ok && tag_ok(w, ta); L.gb[1] = lo_h(w); }
+      if (tid == 0) { ok = ok && tag_ok(gw1, ta); L.gb[1] = lo_h(gw1); }
       return ok;
     }, uni(P.bar) + 32);
     // a share of 32 activations = the chunks of eight neighbouring threads: its sum (the balanced tree over the 16 pair
@@ -1691,8 +1756,8 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
       }
       // through with the K = 4096 projection (the upper half of the grid has no rows there and is here at once): the
       // in-projection rows of the next layer, or of the next step's first layer, set out for LDS
-      if (li + 1 < nl) flow_request_in(g_K.layers[li + 1]);
-      else if (step + 1 < steps) flow_request_in(g_K.layers[0]);
+      const LayerP* const Ynext = li + 1 < nl ? &g_K.layers[li + 1] : (step + 1 < steps ? &g_K.layers[0] : nullptr);
+      if (Ynext) flow_request_in(*Ynext);
       FLOW_TRY((flow_moe_a<GATE8, ST>(F, Y, li, base, h0, h1)));
       FLOW_TRY(flow_moe_b<ST>(F, Y, li, base));
       FLOW_TRY(flow_moe_c<ST>(F, Y, li, base));

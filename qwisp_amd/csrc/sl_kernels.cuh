@@ -1453,20 +1453,27 @@ __global__ __launch_bounds__(256) void k_sdpa_tile(SdpaArgs a) {
     for (int g = 0; g < 8; ++g) { c[0][g] = 0.0f; c[1][g] = 0.0f; }
     const uint16_t* kr = &s_k[(lane < nk ? lane : 0) * KT_STRIDE];
 #pragma unroll
-    for (int l = 0; l < 8; ++l) {
+    for (int gh = 0; gh < 8; gh += 4) {                // four chains (times two heads) at a time
 #pragma unroll
-      for (int g = 0; g < 8; ++g) {
-        const int d = 32 * g + 4 * l;
-        const uint2 kraw = *reinterpret_cast<const uint2*>(kr + d);
-        const h2_t k01 = as_h2(kraw.x), k23 = as_h2(kraw.y);
+      for (int l = 0; l < 8; ++l) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const float4 q4 = *reinterpret_cast<const float4*>(&s_q[(h0 + h) * 256 + d]);
-          c[h][g] = fmaf(q4.x, (float)k01.x, c[h][g]);
-          c[h][g] = fmaf(q4.y, (float)k01.y, c[h][g]);
-          c[h][g] = fmaf(q4.z, (float)k23.x, c[h][g]);
-          c[h][g] = fmaf(q4.w, (float)k23.y, c[h][g]);
+        for (int g = gh; g < gh + 4; ++g) {
+          const int d = 32 * g + 4 * l;
+          const uint2 kraw = *reinterpret_cast<const uint2*>(kr + d);
+          const h2_t k01 = as_h2(kraw.x), k23 = as_h2(kraw.y);
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const float4 q4 = *reinterpret_cast<const float4*>(&s_q[(h0 + h) * 256 + d]);
+            c[h][g] = fmaf(q4.x, (float)k01.x, c[h][g]);
+            c[h][g] = fmaf(q4.y, (float)k01.y, c[h][g]);
+            c[h][g] = fmaf(q4.z, (float)k23.x, c[h][g]);
+            c[h][g] = fmaf(q4.w, (float)k23.y, c[h][g]);
+          }
         }
+        // (the chains' values are pinned here and the LDS reads of later steps stay behind: left to itself the
+        //  scheduler hoists every read of the unrolled loops and spills)
+        asm volatile("" : "+v"(c[0][gh]), "+v"(c[0][gh + 1]), "+v"(c[0][gh + 2]), "+v"(c[0][gh + 3]),
+                          "+v"(c[1][gh]), "+v"(c[1][gh + 1]), "+v"(c[1][gh + 2]), "+v"(c[1][gh + 3]) : : "memory");
       }
     }
 #pragma unroll
@@ -1543,6 +1550,92 @@ struct SdpaMergeArgs {
   const LaneRef* lanes;
   int group = 0;               // > 1: one partial per `group` key tiles at index tile / group (k_sdpa_merge_par only)
 };
+// The same merge for few rows and long contexts (decode steps, lane batches, verify rows): one workgroup of 16 waves
+// per (head, row).  The chains over the tiles stay what they are -- in tile order, one fmaf per tile and element --
+// but the work around them is spread: twelve waves fetch the tiles' partial sums a block of 64 tiles ahead and park
+// them in LDS, the scale of a tile, exp(max_t - max), is formed once per tile (lane = tile) instead of once per lane
+// and tile, and four waves carry the chains, 64 of the head's 256 dims each (every one of them also carries the chain
+// of the sums, so that none has to wait for another).  One barrier per block (of the kind that leaves loads in flight).
+constexpr int MERGE_BLOCK = 64;
+constexpr int MERGE_DYN_LDS = 2 * MERGE_BLOCK * 256 * (int)sizeof(float);
+__global__ __launch_bounds__(1024) void k_sdpa_merge_long(SdpaMergeArgs a) {
+  extern __shared__ __align__(16) float s_park[];          // [2][MERGE_BLOCK tiles][256 dims]
+  const int h = blockIdx.x, m = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int N = a.lanes ? a.lanes[m].st[0] + 1 : a.st[0] + m + 1;
+  const int nt = (N + SDPA_TILE - 1) / SDPA_TILE, nb = (nt + MERGE_BLOCK - 1) / MERGE_BLOCK;
+  const size_t base = ((size_t)m * 16 + h) * a.maxTiles;
+  const float NEG = -__int_as_float(0x7f800000);
+  if (wave >= 4) {
+    // tiles i = (wave - 4) + 12 j of a block, j = 0..5; two register sets take turns, a set is parked and at once
+    // requested again for the block after the next (indices clamped into the context: every load is unconditional)
+    constexpr int PER = 6;
+    float4 qa[PER], qb[PER];
+    auto request = [&](float4 (&dst)[PER], int blk) {
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        const int t = min(MERGE_BLOCK * min(blk, nb - 1) + min((wave - 4) + 12 * j, MERGE_BLOCK - 1), nt - 1);
+        dst[j] = *reinterpret_cast<const float4*>(a.po + (base + t) * 256 + 4 * lane);
+      }
+    };
+    auto park = [&](const float4 (&src)[PER], int blk) {
+      float* const dst = s_park + (size_t)(blk & 1) * MERGE_BLOCK * 256;
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        const int i = (wave - 4) + 12 * j;
+        if (i < MERGE_BLOCK) *reinterpret_cast<float4*>(dst + i * 256 + 4 * lane) = src[j];
+      }
+    };
+    request(qa, 0);
+    request(qb, 1);
+    for (int k = 0; k <= nb; k += 2) {
+      if (k < nb) { park(qa, k); request(qa, k + 2); }
+      lds_barrier();
+      if (k + 1 <= nb) {
+        if (k + 1 < nb) { park(qb, k + 1); request(qb, k + 3); }
+        lds_barrier();
+      }
+    }
+    return;
+  }
+  // waves 0..3: the chains.  Lane i of a block holds tile i's maximum and sum; the global maximum first.
+  float Mx = NEG;
+  for (int t = lane; t < nt; t += 64) Mx = fmaxf(Mx, a.pm[base + t]);
+  Mx = tree_max<64>(Mx);
+  const int d = 64 * wave + lane;
+  const uint16_t graw = a.proj[(size_t)m * PROJ_STRIDE + h * 512 + 256 + d];
+  float L = 0.0f, O = 0.0f;
+  float pmv = a.pm[base + min(lane, nt - 1)], plv = a.pl[base + min(lane, nt - 1)];
+  for (int k = 0; k <= nb; ++k) {
+    if (k >= 1) {
+      const int kb = k - 1, t0 = MERGE_BLOCK * kb, cnt = min(MERGE_BLOCK, nt - t0);
+      const float fl = (lane < cnt) ? exp_c(pmv - Mx) : 0.0f, pl = (lane < cnt) ? plv : 0.0f;
+      if (k < nb) { pmv = a.pm[base + min(t0 + MERGE_BLOCK + lane, nt - 1)]; plv = a.pl[base + min(t0 + MERGE_BLOCK + lane, nt - 1)]; }
+      const float* const src = s_park + (size_t)(kb & 1) * MERGE_BLOCK * 256 + d;
+      int u0 = 0;
+      for (; u0 + 8 <= cnt; u0 += 8) {                 // eight tiles at a time: their scales and sums as scalars, their values from LDS
+        float f[8], l[8], o[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = src[(u0 + i) * 256];
+        lanes8(fl, u0, f);
+        lanes8(pl, u0, l);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { L = fmaf(l[i], f[i], L); O = fmaf(o[i], f[i], O); }
+      }
+      for (; u0 < cnt; ++u0) {
+        const float f = row_lane_f(fl, u0), l = row_lane_f(pl, u0);
+        L = fmaf(l, f, L); O = fmaf(src[u0 * 256], f, O);
+      }
+    }
+    lds_barrier();
+  }
+  const float r = f16r(f16r(O / L) * sigmoid16(h2f(graw)));
+  a.gated[(size_t)m * 4096 + h * 256 + d] = f2h(r);
+  if (a.gsum) {                                          // a share of 32 values sits on 32 neighbouring lanes
+    const float sw = tree_sum<32>(r);
+    if ((lane & 31) == 0) a.gsum[(size_t)m * 128 + h * 8 + (d >> 5)] = sw;
+  }
+}
 __global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
   const int h = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;
   const int N = a.lanes ? a.lanes[m].st[0] + 1 : a.st[0] + m + 1;

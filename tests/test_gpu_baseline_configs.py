@@ -257,6 +257,11 @@ def test_32_lanes_each_equal_to_its_own_oracle(env, small_model):
 # final-normed rows (rms about 1) is stated per row: median relative rms error 2 %, worst row 10 %.
 HYBRID_REL_RMS_MEDIAN = 0.02
 HYBRID_REL_RMS_WORST = 0.10
+# The same after the 40 layers of the full-size model (first 64 rows of a 2048-row chunk): the random-init stack keeps
+# amplifying what the first layers differ by (and with 256 experts more rows sit near a routing tie), measured 15 %
+# median and 32 % worst relative rms; the bound leaves half as much again.
+FULL_HYBRID_REL_RMS_MEDIAN = 0.23
+FULL_HYBRID_REL_RMS_WORST = 0.50
 
 
 def test_hybrid_rows_and_hybrid_lane_step_against_the_oracle(env, small_model):
@@ -274,9 +279,9 @@ def test_hybrid_rows_and_hybrid_lane_step_against_the_oracle(env, small_model):
     hyb.close()
     # 16 lanes stepped together with the driver in hybrid mode, each against its own oracle's logits
     B = 16
-    base = env["Engine"](cfg, dev, max_m=B, max_seq_len=96)
-    lanes = [base.new_lane(max_m=B, max_seq_len=96) for _ in range(B)]
-    oras = [env["orc"].Oracle(cfg, host, max_m=B, max_seq_len=96) for _ in range(B)]
+    base = env["Engine"](cfg, dev, max_m=B, max_seq_len=320)
+    lanes = [base.new_lane(max_m=B, max_seq_len=320) for _ in range(B)]
+    oras = [env["orc"].Oracle(cfg, host, max_m=B, max_seq_len=320) for _ in range(B)]
     rng = np.random.default_rng(4001)
     cur = []
     for i, (lane, o) in enumerate(zip(lanes, oras)):
@@ -296,6 +301,33 @@ def test_hybrid_rows_and_hybrid_lane_step_against_the_oracle(env, small_model):
         assert np.linalg.norm(lg - lw) / np.linalg.norm(lw) < 0.05, i
         agree += int(got[i]) == w
     assert agree >= B - 2, agree          # greedy tokens may differ only at near-ties
+    # the matrix-core attention of a lane batch over several key tiles (k_sdpa_lane_mfma walks four tiles per workgroup
+    # and the partial sums of the workgroups are merged): three of the lanes go on to contexts of 150, 220 and 300
+    # tokens, their oracles with them, and the next batched step is held against the oracles' logits again
+    # (the lanes' caches hold one token written by the matrix-core step above, so from here on they follow their oracles
+    # to tolerance, not bit for bit: the same tokens are fed to both, the predictions may part at near-ties)
+    long_ctx = {3: 150, 8: 220, 13: 300}
+    for i, n in long_ctx.items():
+        more = rng.integers(0, cfg.vocab, n - lanes[i].position - 1).astype(np.int32)
+        same = 0
+        for j in range(0, len(more), B):
+            tl, tw = lanes[i].step_argmax(more[j:j + B]), oras[i].step_argmax(more[j:j + B])
+            assert tl is not None, lanes[i].gpu_fault
+            same += int((tl == tw).sum())
+        assert same >= 0.9 * len(more), (i, same, len(more))
+    cur = [int(t) for t in got]
+    for i in long_ctx:
+        cur[i] = 7 + i
+    assert [lanes[i].position for i in sorted(long_ctx)] == [149, 219, 299]
+    got = type(base).lane_step_argmax(lanes, cur)
+    assert got is not None, [l.gpu_fault for l in lanes]
+    agree = 0
+    for i, (lane, o) in enumerate(zip(lanes, oras)):
+        w = int(o.step_argmax([cur[i]])[0])
+        lg, lw = lane.logits_row(0).astype(np.float64), o.logits_row(0).astype(np.float64)
+        assert np.linalg.norm(lg - lw) / np.linalg.norm(lw) < 0.05, (i, lane.position)
+        agree += int(got[i]) == w
+    assert agree >= B - 2, agree
     for lane in lanes:
         lane.close()
     base.close()
@@ -362,6 +394,13 @@ def test_full_size_32_lanes_at_1k_to_16k_contexts_equal_solo_steps(env):
     r2 = np.concatenate([two.forward_tokens(pr[:1024]), two.forward_tokens(pr[1024:])])
     assert r1 is not None, one.gpu_fault
     assert same_bits(r1, r2) and np.isfinite(r1.astype(np.float32)).all()
+    # and the chunk's first 64 rows against the oracle's exact rows of the same 64 tokens (a row only sees the rows
+    # before it, so the oracle need not follow the other 1984): 40 layers compound what 8 layers do in the bound above
+    ora64 = env["orc"].Oracle(cfg, host, max_m=64, max_seq_len=64)
+    w64 = ora64.forward_tokens(pr[:64]).astype(np.float64)
+    rel = np.linalg.norm(r1[:64].astype(np.float64) - w64, axis=1) / np.linalg.norm(w64, axis=1)
+    print("full-size hybrid chunk, first 64 rows against the oracle: median rel rms %.4f worst %.4f" % (np.median(rel), rel.max()))
+    assert np.median(rel) < FULL_HYBRID_REL_RMS_MEDIAN and rel.max() < FULL_HYBRID_REL_RMS_WORST, (np.median(rel), rel.max())
     t1, t2 = one.head_argmax(r1[-1:]), two.head_argmax(r2[-1:])
     assert t1.tolist() == t2.tolist()
     assert one.chained_step_argmax(int(t1[0]), 4).tolist() == two.chained_step_argmax(int(t2[0]), 4).tolist()
