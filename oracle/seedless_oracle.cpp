@@ -34,6 +34,7 @@ constexpr int HK = SL_GDN_HK, HV = SL_GDN_HV, GD = SL_GDN_D, CK = SL_CONV_K, CD 
 constexpr int KEYDIM = HK * GD, VALDIM = HV * GD;
 constexpr float EPS = 1e-6f;
 constexpr int SDPA_TILE = 64;
+constexpr int MERGE_BLOCK = 64;     // key tiles whose partial sums form one chain in the merge
 
 // ------------------------------------------------------------------------------------------------
 // 4-bit GEMV.  Reference: qmm4 (SeedlessMetalForward.swift:238-310): y[n] = sum_k x[k]*(s*q+b),
@@ -431,12 +432,20 @@ static void sdpa_row(const float* qrot /*[HD]*/, const uint16_t* kc, const uint1
   }
   float Mx = -INFINITY;
   for (int t = 0; t < nt; ++t) Mx = std::fmax(Mx, tm[t]);
+  // Tiles are added up in blocks of 64: within a block one fmaf chain in tile order (from zero), the blocks' chains
+  // added in block order.  (Up to 4096 keys that is a single chain over the tiles.)
   float Lsum = 0.0f, O[HD];
   for (int d = 0; d < HD; ++d) O[d] = 0.0f;
-  for (int t = 0; t < nt; ++t) {
-    const float f = exp_c(tm[t] - Mx);
-    Lsum = std::fmaf(tl[t], f, Lsum);
-    for (int d = 0; d < HD; ++d) O[d] = std::fmaf(to[(size_t)t * HD + d], f, O[d]);
+  for (int t0 = 0; t0 < nt; t0 += MERGE_BLOCK) {
+    float Lb = 0.0f, Ob[HD];
+    for (int d = 0; d < HD; ++d) Ob[d] = 0.0f;
+    for (int t = t0; t < std::min(nt, t0 + MERGE_BLOCK); ++t) {
+      const float f = exp_c(tm[t] - Mx);
+      Lb = std::fmaf(tl[t], f, Lb);
+      for (int d = 0; d < HD; ++d) Ob[d] = std::fmaf(to[(size_t)t * HD + d], f, Ob[d]);
+    }
+    Lsum = t0 == 0 ? Lb : Lsum + Lb;
+    for (int d = 0; d < HD; ++d) O[d] = t0 == 0 ? Ob[d] : O[d] + Ob[d];
   }
   for (int d = 0; d < HD; ++d) out[d] = f16r(O[d] / Lsum);
 }

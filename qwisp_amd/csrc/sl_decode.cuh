@@ -117,13 +117,17 @@ struct Lds {
   alignas(16) float sq[8 * 256];            // attention: scaled queries of one kv group (read back 16 bytes at a time)
   float knew[256], vnew[256];
   alignas(16) float sm[8 * 64];             // attention: per head softmax weights of the tile (read back 16 bytes at a time)
-  float part[16 * 64];                      // attention: score partials of the waves; router: logits and exps
+  alignas(16) float part[16 * 64];          // router: logits and exps; attention merge: hand-over words
 };
 __shared__ Lds g_L;
 extern __shared__ __align__(16) uint16_t g_vt[];   // dynamic: staged value tile [64][256] halves, then the softmax
                                                    // weights of up to SDPA_ROUND (tile, kv head) units [8 heads][64 keys]
-constexpr int SDPA_ROUND = 20;
-constexpr int DEC_DYN_LDS = SDPA_TILE * 256 * 2 + SDPA_ROUND * 8 * 64 * 4 + 4096;   // (+ room for the rows parked ahead of their stage)
+constexpr int SDPA_ROUND = 12;
+// Attention tile units use the dynamic LDS as: value tile 32 KB | softmax weights of a round's units | score partials
+// [8 heads][8 chains of 32 dims][64 keys] fp32 (also the value sums of the keys' second half on their way to the first).
+constexpr int SPART_OFF = SDPA_TILE * 256 * 2 + SDPA_ROUND * 8 * 64 * 4;            // bytes into g_vt
+constexpr int DEC_DYN_LDS = 77824;               // what the rows parked ahead of their stage need (the larger of the two uses)
+static_assert(SPART_OFF + 64 * 64 * 4 <= DEC_DYN_LDS, "score partials fit");
 
 SL_DEV void lds_get_x(int b, int lane, uint32_t* xp, float& sx) {
 #pragma unroll

@@ -852,7 +852,9 @@ int alloc_runtime(sl_engine* e) {
       // every workgroup of the grid must be resident at once: one per compute unit
       int per_cu = 0;
       SL_TRY(e, hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k_decode_flow<false, false>, DEC_THREADS, DEC_DYN_LDS));
-      if (per_cu >= 1) e->dec_grid = 256;
+      // (the merging workgroups keep every tile's {max, sum} in the key tile's LDS space: 4224 tiles = 270336 tokens;
+      // beyond that the kernel-per-stage sequence runs)
+      if (per_cu >= 1 && e->max_tiles <= SDPA_TILE * KT_STRIDE * 2 / 8) e->dec_grid = 256;
     }
   }
   e->pinned_bytes = MH * 2 + 4096 + (size_t)d->n_layers * 4 + (size_t)MAX_CHAIN * 4 + 64;
@@ -1047,7 +1049,11 @@ int sl_set_persistent(sl_engine* e, int enable) {
 // workgroup records 100 MHz clock stamps of the last step of a launch; the call copies them out,
 // out[wg * sl_stage_clock_words() + (layer * 8 + stage) * 8 + kind] (0 = not reached).
 int sl_debug_stage_clock(sl_engine* e, int enable, uint32_t* out, int cap_words) {
-  SL_ENTER(e);
+  // (reading the stamps is allowed on an engine whose last launch gave up: they show where every workgroup stood)
+  std::lock_guard<std::recursive_mutex> gpu_lock_(g_gpu_mutex);
+  if (!e) return SL_ERR_ARG;
+  if (!e->fault.empty() && (enable || !out)) return SL_ERR_POISONED;
+  int r = SL_OK;
   if (!e->flow_params) return SL_ERR_UNSUPPORTED;
   if (out && cap_words > 0) {
     const size_t n = std::min<size_t>((size_t)cap_words, (size_t)e->dec_grid * STAMP_WORDS);
@@ -1109,7 +1115,10 @@ static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, con
   if (abort_word) {
     unsigned flag = 0;
     std::memcpy(&flag, flag_at, 4);
-    if (flag) { if (e->fault.empty()) e->fault = "persistent decode kernel: grid barrier timed out"; return SL_ERR_DEVICE; }
+    if (flag) {      // (the word names the wait that gave up first: 1 = a stage's hand-over, 16 + n = wait n of the attention merge)
+      if (e->fault.empty()) e->fault = "persistent decode kernel: grid barrier timed out (wait " + std::to_string(flag) + ")";
+      return SL_ERR_DEVICE;
+    }
   }
   std::memcpy(dst, e->pinned, bytes);
   return SL_OK;

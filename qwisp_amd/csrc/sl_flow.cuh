@@ -98,9 +98,20 @@ SL_HD uint32_t flow_tag32(uint32_t base, int layer, int stage) { return 0x800000
 SL_DEV uint32_t tagged(float v, uint32_t tag) { return (uint32_t)f2h(v) | (tag << 16); }
 SL_DEV bool tag_ok(uint32_t w, uint32_t tag) { return (w >> 16) == tag; }
 
+// Loads of words that other workgroups publish.  To the optimiser a buffer-load intrinsic only reads memory, so in a
+// loop that polls with it and stores nothing the load is loop-invariant: it gets hoisted, and the loop spins on its
+// first look until its bound (the volatile bit of the intrinsic only acts at instruction selection).  Every loop that
+// polls therefore starts its trips with SL_FRESH_LOOK(), an empty asm with a memory clobber that no load moves across.
+// (One per trip: in front of every load it cost 0.45 % of the step, and an opaque offset operand per load 2 %.)
+#define SL_FRESH_LOOK() asm volatile("" ::: "memory")
 SL_DEV uint32_t ldw1(rsrc_t r, int idx) { return __builtin_amdgcn_raw_buffer_load_b32(r, idx * 4, 0, CO_SC1); }
 SL_DEV uint2 ldw2(rsrc_t r, int idx) { const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, idx * 4, 0, CO_SC1); return make_uint2(v.x, v.y); }
 SL_DEV uint4 ldw4(rsrc_t r, int idx) { const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, idx * 4, 0, CO_SC1); return make_uint4(v.x, v.y, v.z, v.w); }
+// (the same with a wave-uniform part of the index in the instruction's scalar offset: no vector register per address)
+SL_DEV uint4 ldw4s(rsrc_t r, int idx, int uniform_idx) {
+  const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, idx * 4, uniform_idx * 4, CO_SC1);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
 SL_DEV void stw1(rsrc_t r, int idx, uint32_t w) { __builtin_amdgcn_raw_buffer_store_b32(w, r, idx * 4, 0, CO_SC1); }
 SL_DEV void stw2(rsrc_t r, int idx, uint32_t a, uint32_t b) {
   u32x2_t v; v.x = a; v.y = b;
@@ -131,11 +142,11 @@ SL_DEV void fstamp(int layer, int stage, int kind, bool who) {
 // missing tag marks slot (round % 3) in LDS before the barrier, everybody reads it after, and thread 0 then
 // clears the slot of the round before (nobody can still be reading that one), so a successful round leaves
 // all three slots clear for the next stage.
-SL_DEV int flow_round(bool ok, unsigned& spins, unsigned* abort_word) {
+SL_DEV int flow_round(bool ok, unsigned& spins, unsigned* abort_word, unsigned code = 1u) {
   const unsigned slot = spins % 3u;
   if (!__all(ok ? 1 : 0) && (threadIdx.x & 63) == 0) g_L.pf[slot] = 1;
   if (threadIdx.x == 0 && (spins > g_K.F.spin_limit || ((spins & 63u) == 63u && ld_co32(abort_word) != 0))) {
-    st_co32(abort_word, 1u);
+    if (ld_co32(abort_word) == 0u) st_co32(abort_word, code);        // (the first to give up names its wait)
     g_L.pf[3] = 1;
   }
   lds_barrier();
@@ -154,13 +165,14 @@ SL_DEV int flow_round(bool ok, unsigned& spins, unsigned* abort_word) {
 // `attempt()` fetches what the lane still misses and returns whether the lane is complete; `polls` is uniform per
 // wave.  Bounded like flow_round: a wave that gives up raises the abort word, and false comes back to everybody.
 template <bool MEET = true, typename Attempt>
-SL_DEV bool flow_poll(bool polls, Attempt attempt, unsigned* abort_word) {
+SL_DEV bool flow_poll(bool polls, Attempt attempt, unsigned* abort_word, unsigned code = 1u) {
   if (polls) {
     for (unsigned spins = 0;; ++spins) {
+      SL_FRESH_LOOK();
       const bool ok = attempt();
       if (__all(ok ? 1 : 0)) break;
       if (spins > g_K.F.spin_limit || ((spins & 63u) == 63u && ld_co32(abort_word) != 0)) {
-        if ((threadIdx.x & 63) == 0) { st_co32(abort_word, 1u); g_L.pf[3] = 1; }
+        if ((threadIdx.x & 63) == 0) { if (ld_co32(abort_word) == 0u) st_co32(abort_word, code); g_L.pf[3] = 1; }
         break;
       }
     }                                                   // (no back-off between attempts: a sleep of 64 clocks measured 0.3 % slower)
@@ -259,7 +271,7 @@ SL_DEV bool poll_vec2048(const DecodeP& P, const uint32_t* vec, uint32_t tag, fl
           ok = tag_ok(b.x, tag) && tag_ok(b.y, tag);
         }
         return ok;
-      }, uni(P.bar) + 32)) return false;
+      }, uni(P.bar) + 32, 2u)) return false;
   fstamp<ST>(sl, ss, 1, tid == 0);
   r0 = lo_h(b.x); r1 = lo_h(b.y);
   return true;
@@ -361,7 +373,7 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
           ok = c.z == ttag && c.w == ttag;
           if (ok && lane == 0) g_K.tok = (int)c.x;
         }
-        const int v = flow_round(ok, spins, uni(P.bar) + 32);
+        const int v = flow_round(ok, spins, uni(P.bar) + 32, 3u);
         if (v > 0) break;
         if (v < 0) return false;
       }
@@ -500,7 +512,7 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
     if (!flow_poll(wave < 7, [&]() {                 // channels sit on threads 0..271 and on the two gate threads
           if (!got) { const uint32_t w = ldw1(rp, ch); got = tag_ok(w, tin); newest = lo_h(w); }
           return got;
-        }, uni(P.bar) + 32)) return false;
+        }, uni(P.bar) + 32, 4u)) return false;
     fstamp<ST>(li, FS_CORE, 1, tid == 0);
   }
   if (tid < 272) {
@@ -592,12 +604,16 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
   if (wg >= GU) return true;
   const int U = nt * SL_ATT_KV, RND = uni(F.sdpa_round);
   float* const ps = reinterpret_cast<float*>(g_vt + SDPA_TILE * 256);      // [SDPA_ROUND][8 heads][64 keys]
+  float* const sp = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(g_vt) + SPART_OFF);   // [8 heads][8 chains][64 keys]
   uint32_t* const vn = reinterpret_cast<uint32_t*>(L.vnew);                // [kv head][128 words]: the new value row
   // The queries of the kv head's group and the new key and value row are the same for every unit of a workgroup
   // (with an even count of unit workgroups a workgroup stays with one kv head): polled, normed and rotated for its
   // first unit only.
   uint4 w4 = make_uint4(0, 0, 0, 0);
   int prep_kvh = -1;
+  const int hp = wave >> 2, kh = (wave >> 1) & 1, dh = wave & 1;        // second pass: pair of heads, half of the keys, of the dims
+  float pend_m = 0.0f, pend_l = 0.0f, po[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};     // results waiting to be published
+  int pend_slot = -1;
   // A thread stages two 16-byte pieces of a unit's key and value tiles: rows srow and srow + 32.  The tiles travel
   // through registers one unit ahead of their use, so the loads of the next unit are in flight while this one is
   // scored or summed.  (Rows beyond the context repeat its last row and the row of the new position is fetched like
@@ -649,7 +665,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
           if (!flow_poll(wave < 10, [&]() {
                 w4 = ldw4(rp, src + 4 * lane);
                 return tag_ok(w4.x, tin) && tag_ok(w4.y, tin) && tag_ok(w4.z, tin) && tag_ok(w4.w, tin);
-              }, uni(P.bar) + 32)) return false;
+              }, uni(P.bar) + 32, 5u)) return false;
           fstamp<ST>(li, FS_CORE, 1, tid == 0);
         }
         if (wave < 9) {
@@ -695,44 +711,56 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       // unit, or after the last one the values of its second unit (those of the first are staged already)
       if (r + 1 < nr) fetch(true, false, u + GU);
       else if (nr > 1) fetch(false, true, ub + GU);
+      // the previous unit's {max, sum} go out here: a store right before the wait for a tile would make that wait last
+      // until the store is acknowledged (loads and stores share one counter and may finish in either order)
+      if (pend_slot >= 0 && wave < 8 && lane == 0) stw4(co_rsrc(uni(F.tml)), pend_slot * 4, __float_as_uint(pend_m), __float_as_uint(pend_l), tcore, tcore);
+      pend_slot = -1;
       lds_barrier();
       {
-        // scores: wave (head, half) takes four of the eight chains of 32 dims, lane j is key j; the queries come as
-        // LDS broadcasts (one 16-byte read per four multiply-adds), the key row from the staged tile
-        const int h = wave >> 1, half = wave & 1;
-        const uint16_t* kr = &L.kt[(lane < nk ? lane : 0) * KT_STRIDE + 128 * half];
-        const float* qh = &L.sq[h * 256 + 128 * half];
-        // (the four chains advance side by side, four dims at a time)
+        // scores: wave (chain ch of 32 dims, four of the eight heads), lane j is key j: a key's 32 dims are read once
+        // for four heads; the queries come as LDS broadcasts (one 16-byte read per four multiply-adds)
+        const int ch = wave & 7, hg = wave >> 3;
+        const uint16_t* kr = &L.kt[(lane < nk ? lane : 0) * KT_STRIDE + 32 * ch];
+        uint32_t kw[16];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint4 t = *reinterpret_cast<const uint4*>(kr + 8 * i);
+          kw[4 * i] = t.x; kw[4 * i + 1] = t.y; kw[4 * i + 2] = t.z; kw[4 * i + 3] = t.w;
+        }
         float c[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int l = 0; l < 8; ++l) {
+        for (int d4 = 0; d4 < 8; ++d4) {
+          const h2_t k01 = as_h2(kw[2 * d4]), k23 = as_h2(kw[2 * d4 + 1]);
 #pragma unroll
-          for (int gi = 0; gi < 4; ++gi) {
-            const int d = 32 * gi + 4 * l;
-            const uint2 kraw = *reinterpret_cast<const uint2*>(kr + d);
-            const h2_t k01 = as_h2(kraw.x), k23 = as_h2(kraw.y);      // half operands go straight into the FMA
-            const float4 q4 = *reinterpret_cast<const float4*>(qh + d);
-            c[gi] = fmaf(q4.x, (float)k01.x, c[gi]);
-            c[gi] = fmaf(q4.y, (float)k01.y, c[gi]);
-            c[gi] = fmaf(q4.z, (float)k23.x, c[gi]);
-            c[gi] = fmaf(q4.w, (float)k23.y, c[gi]);
+          for (int hh = 0; hh < 4; ++hh) {
+            const float4 q4 = *reinterpret_cast<const float4*>(&L.sq[(4 * hg + hh) * 256 + 32 * ch + 4 * d4]);
+            c[hh] = fmaf(q4.x, (float)k01.x, c[hh]);
+            c[hh] = fmaf(q4.y, (float)k01.y, c[hh]);
+            c[hh] = fmaf(q4.z, (float)k23.x, c[hh]);
+            c[hh] = fmaf(q4.w, (float)k23.y, c[hh]);
           }
         }
-        L.part[wave * 64 + lane] = (c[0] + c[1]) + (c[2] + c[3]);
+#pragma unroll
+        for (int hh = 0; hh < 4; ++hh) sp[((4 * hg + hh) * 8 + ch) * 64 + lane] = c[hh];
       }
       lds_barrier();
-      if ((wave & 1) == 0) {
-        const int h = wave >> 1;
-        const float dotv = L.part[wave * 64 + lane] + L.part[(wave + 1) * 64 + lane];
+      if (wave < 8) {
+        const int h = wave;
+        float pr[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pr[i] = sp[(h * 8 + i) * 64 + lane];
+        const float dotv = ((pr[0] + pr[1]) + (pr[2] + pr[3])) + ((pr[4] + pr[5]) + (pr[6] + pr[7]));
         const float sc = (lane < nk) ? dotv : NEG;
         const float mx = tree_max<64>(sc);
         const float p = (lane < nk) ? exp_c(sc - mx) : 0.0f;
         const float l = tree_sum<64>(p);
         ps[(r * 8 + h) * 64 + lane] = p;
-        const int head = kvh * 8 + h;
-        if (lane == 0) stw4(co_rsrc(uni(F.tml)), (head * uni(P.max_tiles) + tile) * 4, __float_as_uint(mx), __float_as_uint(l), tcore, tcore);
+        pend_m = mx; pend_l = l;
+        pend_slot = (kvh * 8 + h) * uni(P.max_tiles) + tile;
       }
     }
+    if (pend_slot >= 0 && wave < 8 && lane == 0) stw4(co_rsrc(uni(F.tml)), pend_slot * 4, __float_as_uint(pend_m), __float_as_uint(pend_l), tcore, tcore);
+    pend_slot = -1;
     // pass 2, values: the weighted value sums of the same units, in the same order
     for (int r = 0; r < nr; ++r) {
       const int u = ub + r * GU;
@@ -745,39 +773,54 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
         if (r + 1 < nr) fetch(false, true, u + GU);
       }
       if (r + 1 == nr && ub + GU * RND < U) fetch(true, true, ub + GU * RND);   // the next round's first unit
+      if (pend_slot >= 0 && kh == 0) {                     // the previous unit's sums (behind the wait for this unit's tile)
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+          stw4(co_rsrc(uni(F.tpo)), ((pend_slot + e * uni(P.max_tiles)) * 128 + 64 * dh + lane) * 4, __float_as_uint(po[e][0]), __float_as_uint(po[e][1]), tcore, tcore);
+      }
+      pend_slot = -1;
       if (has_new && wave == 9) {
         const uint32_t a = vn[kvh * 128 + 2 * lane], b = vn[kvh * 128 + 2 * lane + 1];
         stw2(co_rsrc(uni(Y.vcache) + ((size_t)kvh * uni(P.max_seq) + pos) * 256), 2 * lane, a, b);
         *reinterpret_cast<uint2*>(&g_vt[(pos - j0) * 256 + 4 * lane]) = make_uint2(a, b);
       }
       lds_barrier();
-      const int h = wave >> 1, half = wave & 1;
-      // two chains over the keys, 0..31 and 32..63, added at the end; all 64 keys are walked (beyond the context the
-      // weight and the staged value are zero).  The weights come as LDS broadcasts, four keys per read.
-      float oa0 = 0.0f, oa1 = 0.0f, ob0 = 0.0f, ob1 = 0.0f;
-      const uint16_t* vt = &g_vt[128 * half + 2 * lane];
-      const float* pw = &ps[(r * 8 + h) * 64];
+      // wave (pair of heads, half of the keys, half of the dims), two dims per lane: a value is read once for two heads.
+      // The two chains over the keys, 0..31 and 32..63, run on different waves and meet through LDS; all 64 keys are
+      // walked (beyond the context the weight and the staged value are zero).  The weights come as LDS broadcasts,
+      // four keys per read.
+      float o[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
+      const uint16_t* vt = &g_vt[(32 * kh) * 256 + 128 * dh + 2 * lane];
+      const float* pw = &ps[(r * 8 + 2 * hp) * 64 + 32 * kh];
 #pragma unroll
       for (int j = 0; j < 32; j += 4) {
-        uint32_t va[4], vb[4];
+        uint32_t va[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          va[i] = *reinterpret_cast<const uint32_t*>(vt + (j + i) * 256);
-          vb[i] = *reinterpret_cast<const uint32_t*>(vt + (32 + j + i) * 256);
-        }
-        const float4 pa = *reinterpret_cast<const float4*>(pw + j), pb = *reinterpret_cast<const float4*>(pw + 32 + j);
+        for (int i = 0; i < 4; ++i) va[i] = *reinterpret_cast<const uint32_t*>(vt + (j + i) * 256);
+        const float4 pa = *reinterpret_cast<const float4*>(pw + j), pb = *reinterpret_cast<const float4*>(pw + 64 + j);
         const float pav[4] = {pa.x, pa.y, pa.z, pa.w}, pbv[4] = {pb.x, pb.y, pb.z, pb.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const h2_t a01 = as_h2(va[i]), b01 = as_h2(vb[i]);
-          oa0 = fmaf(pav[i], (float)a01.x, oa0); oa1 = fmaf(pav[i], (float)a01.y, oa1);
-          ob0 = fmaf(pbv[i], (float)b01.x, ob0); ob1 = fmaf(pbv[i], (float)b01.y, ob1);
+          const h2_t a01 = as_h2(va[i]);
+          o[0][0] = fmaf(pav[i], (float)a01.x, o[0][0]); o[0][1] = fmaf(pav[i], (float)a01.y, o[0][1]);
+          o[1][0] = fmaf(pbv[i], (float)a01.x, o[1][0]); o[1][1] = fmaf(pbv[i], (float)a01.y, o[1][1]);
         }
       }
-      const float o0 = oa0 + ob0, o1 = oa1 + ob1;
-      const int head = kvh * 8 + h;
-      stw4(co_rsrc(uni(F.tpo)), ((head * uni(P.max_tiles) + tile) * 128 + 64 * half + lane) * 4, __float_as_uint(o0), __float_as_uint(o1), tcore, tcore);
+      float4* const xo = reinterpret_cast<float4*>(sp) + (hp * 2 + dh) * 64 + lane;
+      if (kh == 1) *xo = make_float4(o[0][0], o[0][1], o[1][0], o[1][1]);
+      lds_barrier();
+      if (kh == 0) {
+        const float4 ob = *xo;
+        po[0][0] = o[0][0] + ob.x; po[0][1] = o[0][1] + ob.y; po[1][0] = o[1][0] + ob.z; po[1][1] = o[1][1] + ob.w;
+        pend_slot = (kvh * 8 + 2 * hp) * uni(P.max_tiles) + tile;
+      }
     }
+    if (pend_slot >= 0 && kh == 0) {
+#pragma unroll
+      for (int e = 0; e < 2; ++e)
+        stw4(co_rsrc(uni(F.tpo)), ((pend_slot + e * uni(P.max_tiles)) * 128 + 64 * dh + lane) * 4, __float_as_uint(po[e][0]), __float_as_uint(po[e][1]), tcore, tcore);
+    }
+    pend_slot = -1;
     lds_barrier();
   }
   fstamp<ST>(li, FS_CORE, 4, tid == 0);
@@ -835,7 +878,7 @@ SL_DEV bool flow_sdpa4(const FlowP& F, const LayerP& Y, int li, int pos, uint32_
     if (!flow_poll(fetches, [&]() {
           w4 = ldw4(rp, src + 4 * lane);
           return tag_ok(w4.x, tin) && tag_ok(w4.y, tin) && tag_ok(w4.z, tin) && tag_ok(w4.w, tin);
-        }, uni(P.bar) + 32)) return false;
+        }, uni(P.bar) + 32, 6u)) return false;
     fstamp<ST>(li, FS_CORE, 1, tid == 0);
   }
   // (the poll's barrier is behind us: the key tile aliases the activation vector the in-projection read)
@@ -1006,11 +1049,17 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     const bool act = lane < LPW;
     const int chunk = LPW * (kx % MPH) + (act ? lane : 0);      // (idle lanes of a narrower workgroup fetch and store nothing)
     const rsrc_t rml = co_rsrc(uni(F.tml)), rpo = co_rsrc(uni(F.tpo)), rp = co_rsrc(uni(F.tproj));
-    constexpr int MB = 12;
     int fail = 0;
     float Mx = NEG, Ls = 0.0f, O0 = 0.0f, O1 = 0.0f;
     uint4 m0 = make_uint4(0, 0, 0, 0);
     uint2 g2 = make_uint2(0u, 0u);
+    // {max, sum} of every tile, kept in LDS once they have been seen (the key tile's space: merging workgroups stage none)
+    uint2* const mls = reinterpret_cast<uint2*>(g_L.kt);
+    constexpr int MB = 12;                                  // tiles of the first round trip
+    if (nt > MB) {                                          // the hand-over words of the long merge (below), before any wave uses them
+      if (tid < 128) reinterpret_cast<volatile uint32_t*>(reinterpret_cast<unsigned char*>(g_vt) + (DEC_WAVES - 2) * 8 * 64 * 8)[tid] = 0u;
+      lds_barrier();
+    }
     float sg0 = 0.0f, sg1 = 0.0f;                          // sigmoids of the lane's two gate values
     if (wave == 0) {
       uint4 a[MB];
@@ -1020,6 +1069,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
         float pm[8];
         unsigned have = 0, spins = 0;
         for (;;) {
+          SL_FRESH_LOOK();
           uint4 mq[8];
           const unsigned missing = ~have;
 #pragma unroll
@@ -1033,10 +1083,13 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
             if (!(missing & (1u << j))) continue;
             const int t = t0 + 64 * j + lane;
             pm[j] = t < nt ? __uint_as_float(mq[j].x) : NEG;
-            if (__all((mq[j].z == tcore32 && mq[j].w == tcore32) ? 1 : 0)) have |= 1u << j;
+            if (__all((mq[j].z == tcore32 && mq[j].w == tcore32) ? 1 : 0)) {
+              have |= 1u << j;
+              if (t < nt) mls[t] = make_uint2(mq[j].x, mq[j].y);      // kept for the blocks' additions below
+            }
           }
           if (have == 0xffu) break;
-          if (++spins > uni(F.spin_limit)) { fail = 1; break; }
+          if (++spins > uni(F.spin_limit)) { fail = 17; break; }
         }
         if (!fail) {
 #pragma unroll
@@ -1049,6 +1102,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
         bool mdone = false, gdone = false;
         unsigned have = 0, spins = 0;
         for (;;) {
+          SL_FRESH_LOOK();
           // every piece still missing is requested first and looked at afterwards: with a look behind each request the
           // round trips of an attempt would follow one another (up to fourteen of them)
           const bool want_m = !mdone, want_g = !gdone;
@@ -1068,9 +1122,10 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
           for (int u = 0; u < MB; ++u)
             if (u < cnt0 && (missing & (1u << u)) && __all((!act || (a[u].z == tcore32 && a[u].w == tcore32)) ? 1 : 0)) have |= 1u << u;
           if (mdone && gdone && have == (1u << cnt0) - 1u) break;
-          if (++spins > uni(F.spin_limit)) { fail = 1; break; }
+          if (++spins > uni(F.spin_limit)) { fail = 18; break; }
         }
         Mx = fmaxf(Mx, tree_max<64>(mine ? __uint_as_float(m0.x) : NEG));
+        if (mine) mls[lane] = make_uint2(m0.x, m0.y);
         fstamp<ST>(li, FS_MERGE, 1, lane == 0);
       }
       if (!fail) {                                          // the first batch is already here
@@ -1092,7 +1147,8 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
         fstamp<ST>(li, FS_MERGE, 3, lane == 0);
       }
     }
-    if (nt > MB) {                                          // uniform for the grid
+    const int nb = (nt + 63) / 64;                          // blocks of 64 tiles: a chain each, the chains added in block order
+    if (nt > MB && nb <= 2) {                               // uniform for the grid
       // Blocks of 64 tiles in a pipeline: waves 2..15 poll the partial sums of block b (five tiles each) and park
       // them in LDS, while wave 0 adds up block b-1 from the other parking buffer in tile order and wave 1 carries
       // the chain of the tiles' sums (the merge is one dependent chain per lane: a wave that also fetches and sums
@@ -1100,14 +1156,14 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
       // nbp + 1 of them, nbp = the block count rounded up to even (a block beyond the context is empty).
       uint2* const park0 = reinterpret_cast<uint2*>(g_vt);                       // [64 tiles][64 lanes] {o0, o1}
       uint2* const park1 = reinterpret_cast<uint2*>(g_vt + SDPA_TILE * 256);     // the softmax weights' space (merging workgroups own no units)
-      static_assert(SDPA_ROUND * 8 * 64 * 4 >= 64 * 64 * 8, "second parking buffer");
+      
       // (the polling waves start at once, while wave 0 is still waiting for the maxima and the first tiles above; tile
       // units this workgroup may have had ended with a barrier, so the parking space is free)
       if (wave == 0) {                                      // for wave 1: the maximum, the sum so far, block 0's {max, sum} words
         if (lane == 0) { g_L.red[0] = Mx; g_L.red[1] = Ls; }
         *reinterpret_cast<uint2*>(&g_L.part[2 * lane]) = make_uint2(m0.x, m0.y);
       }
-      const int nb = (nt + 63) / 64, nbp = (nb + 1) & ~1;
+      const int nbp = 2;
       if (wave >= 2) {
         // A wave's five tiles of a block are requested two blocks ahead (a round trip to memory takes about two blocks'
         // additions), so a block costs a round trip only when its tiles have not been published yet.  Two register
@@ -1134,7 +1190,8 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
 #pragma unroll
             for (int j = 0; j < 5; ++j) ok = ok && (!wanted(blk, j) || (cur[j].z == tcore32 && cur[j].w == tcore32));
             if (__all(ok ? 1 : 0)) break;
-            if (++spins > uni(F.spin_limit)) { fail = 1; break; }
+            if (++spins > uni(F.spin_limit)) { fail = 19; break; }
+            SL_FRESH_LOOK();
             request(cur, blk);
           }
 #pragma unroll
@@ -1161,6 +1218,8 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
           float fl = 0.0f, pl = 0.0f;                     // lane i: scale and sum of tile t0+i
           if (t0 + lane < nt) { fl = exp_c(__uint_as_float(cur.x) - Mx); pl = __uint_as_float(cur.y); }
           const int lo = t0 == 0 ? MB : 0, hi = min(64, nt - t0);
+          float S0 = 0.0f, S1 = 0.0f, SL = 0.0f;
+          if (blk == 1 && blk < nb) { S0 = O0; S1 = O1; SL = Ls; O0 = 0.0f; O1 = 0.0f; Ls = 0.0f; }
           if (wave == 0 && !fail) {
             // sixteen LDS reads and sixteen lane reads at a time, used in tile order (one wave issues an instruction
             // every eight clocks or so and waits tens of clocks for a batch of either kind: few, large batches)
@@ -1195,6 +1254,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
               for (int i = 0; i < 8; ++i) if (u0 + i < hi) Ls = fmaf(l[i], f[i], Ls);
             }
           }
+          if (blk == 1 && blk < nb) { O0 = S0 + O0; O1 = S1 + O1; Ls = SL + Ls; }
         };
         lds_barrier();                                    // block 0 is parked; wave 0 has left the maximum and its sum so far
         if (wave == 1) {
@@ -1212,8 +1272,124 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
       }
       lds_barrier();
       if (wave == 0) Ls = g_L.red[2];
+    } else if (nt > MB) {
+      // More than 128 tiles: the blocks' chains run side by side.  Wave 2 + w takes blocks w, w + 14, ...: it polls
+      // sixteen tiles at a time (one 16-byte chunk per lane and tile; the tile index sits in the load's scalar offset,
+      // so sixteen requests in flight cost no address registers) -- from the start of the stage, while the maxima are
+      // still on their way -- and, once wave 0 has left the global maximum, adds them up in tile order (block 0 goes
+      // on from wave 0's chain over the first tiles) and leaves the block's chain in LDS.  Wave 1 carries the chains
+      // of the tiles' sums, which need no partial sums.  After one barrier wave 0 adds the blocks' chains in block
+      // order.  The waves meet through LDS words only; every wait is bounded, and a wave that gives up raises the
+      // abort word, which ends the others' waits.  (What bounds this stage is the rate at which 32 workgroups pull
+      // 16 MB of published chunks past their caches, about 1 TB/s at 32K tokens: a block's quarters dealt out to four
+      // waves with the chain handed on through LDS only added polls, 46.9 against 41.0 us.)
+      uint2* const blk_o = reinterpret_cast<uint2*>(g_vt);                        // [block][64 lanes] {o0, o1}
+      constexpr int RW_OFF = (DEC_WAVES - 2) * 8 * 64 * 8, MAX_BLOCKS = (SDPA_TILE * KT_STRIDE * 2 / 8 + 63) / 64;
+      static_assert(MAX_BLOCKS * 512 <= RW_OFF && MAX_BLOCKS + 2 <= 128, "a chain and a word per block of the longest context");
+      volatile uint32_t* const rw = reinterpret_cast<volatile uint32_t*>(reinterpret_cast<unsigned char*>(g_vt) + RW_OFF);
+      // rw[0]: wave 0 has left the maximum, its sum and its chains; rw[1]: abort.
+      // (Cleared at the top of the stage.)
+      const unsigned limit = uni(F.spin_limit);
+      if (wave == 0) {
+        if (lane == 0) { g_L.red[0] = Mx; g_L.red[1] = Ls; }
+        blk_o[lane] = make_uint2(__float_as_uint(O0), __float_as_uint(O1));
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if (lane == 0) rw[0] = 1u;
+      } else if (wave == 1) {
+        unsigned spins = 0;
+        while (rw[0] == 0u) {
+          if (++spins > limit || rw[1] != 0u) { fail = 20; break; }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        if (!fail) {
+          Mx = g_L.red[0];
+          float Lb = g_L.red[1], La = 0.0f;               // the block's chain (block 0: from wave 0's), the blocks before
+          for (int b = 0; b < nb; ++b) {
+            const int t0 = 64 * b;
+            const uint2 cur = mls[min(t0 + lane, nt - 1)];
+            float fl = 0.0f, pl = 0.0f;
+            if (t0 + lane < nt) { fl = exp_c(__uint_as_float(cur.x) - Mx); pl = __uint_as_float(cur.y); }
+            const int lo = b == 0 ? MB : 0, hi = min(64, nt - t0);
+            for (int u0 = lo & ~7; u0 < hi; u0 += 8) {
+              float f[8], l[8];
+              lanes8(fl, u0, f);
+              lanes8(pl, u0, l);
+#pragma unroll
+              for (int i = 0; i < 8; ++i) if (u0 + i >= lo && u0 + i < hi) Lb = fmaf(l[i], f[i], Lb);
+            }
+            La = b == 0 ? Lb : La + Lb;
+            Lb = 0.0f;
+          }
+          if (lane == 0) g_L.red[2] = La;
+        } else if (lane == 0) rw[1] = 1u;
+      } else {
+        constexpr int WB = 16;                            // tiles per round trip (a multiple of 8)
+        unsigned spins = 0;
+        bool have_max = false;
+        for (int b = wave - 2; b < nb && !fail; b += DEC_WAVES - 2) {
+          const int tlo = b == 0 ? MB : 64 * b, thi = min(64 * b + 64, nt);
+          float B0 = 0.0f, B1 = 0.0f, fl = 0.0f;
+          for (int tb = tlo; tb < thi && !fail; tb += WB) {
+            uint4 v[WB];
+            auto request = [&]() {
+#pragma unroll
+              for (int j = 0; j < WB; ++j) v[j] = ldw4s(rpo, chunk * 4, (slot0 + min(tb + j, nt - 1)) * 512);
+            };
+            request();
+            for (;;) {
+              bool ok = true;
+#pragma unroll
+              for (int j = 0; j < WB; ++j) ok = ok && (tb + j >= thi || !act || (v[j].z == tcore32 && v[j].w == tcore32));
+              if (__all(ok ? 1 : 0)) break;
+              if (++spins > limit || rw[1] != 0u) { fail = 21; break; }
+              SL_FRESH_LOOK();
+              request();
+            }
+            if (fail) break;
+            if (!have_max) {
+              while (rw[0] == 0u) {
+                if (++spins > limit || rw[1] != 0u) { fail = 22; break; }
+              }
+              if (fail) break;
+              __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+              Mx = g_L.red[0];
+              have_max = true;
+            }
+            if (tb == tlo) {                               // lane i: the scale of tile i of the block
+              const int t = 64 * b + lane;
+              fl = t < nt ? exp_c(__uint_as_float(mls[min(t, nt - 1)].x) - Mx) : 0.0f;
+              if (b == 0) { const uint2 c0 = blk_o[lane]; B0 = __uint_as_float(c0.x); B1 = __uint_as_float(c0.y); }
+            }
+            float f[WB];
+#pragma unroll
+            for (int k = 0; k < WB; k += 8) lanes8(fl, tb - 64 * b + k, reinterpret_cast<float(&)[8]>(f[k]));   // (lanes beyond 63 belong to tiles beyond the block: unused)
+            if (tb + WB <= thi) {
+#pragma unroll
+              for (int i = 0; i < WB; ++i) { B0 = fmaf(__uint_as_float(v[i].x), f[i], B0); B1 = fmaf(__uint_as_float(v[i].y), f[i], B1); }
+            } else {
+#pragma unroll
+              for (int i = 0; i < WB; ++i) {
+                if (tb + i < thi) { B0 = fmaf(__uint_as_float(v[i].x), f[i], B0); B1 = fmaf(__uint_as_float(v[i].y), f[i], B1); }
+              }
+            }
+          }
+          if (!fail) blk_o[b * 64 + lane] = make_uint2(__float_as_uint(B0), __float_as_uint(B1));
+        }
+        if (fail && lane == 0) rw[1] = 1u;
+      }
+      lds_barrier();
+      if (rw[1] != 0u) fail = 24;
+      if (wave == 0 && !fail) {
+        Ls = g_L.red[2];
+        const uint2 c0 = blk_o[lane];
+        O0 = __uint_as_float(c0.x); O1 = __uint_as_float(c0.y);
+        for (int b = 1; b < nb; ++b) {
+          const uint2 c = blk_o[b * 64 + lane];
+          O0 = O0 + __uint_as_float(c.x); O1 = O1 + __uint_as_float(c.y);
+        }
+      }
     }
-    if (fail) st_co32(uni(P.bar) + 32, 1u);
+    if (fail && ld_co32(uni(P.bar) + 32) == 0u) st_co32(uni(P.bar) + 32, (uint32_t)fail);
     if (wave == 0 && !fail && act) {
       const uint32_t r0 = tagged(f16r(f16r(O0 / Ls) * sg0), tmerge);
       const uint32_t r1 = tagged(f16r(f16r(O1 / Ls) * sg1), tmerge);
@@ -1255,7 +1431,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
             }
           }
           return ok;
-        }, uni(P.bar) + 32)) return false;
+        }, uni(P.bar) + 32, 7u)) return false;
     fstamp<ST>(li, FS_OUT, 1, tid == 0);
     if (lin) store_hist(Y, li, gh);
     out[0] = lo_h(a.x); out[1] = lo_h(a.y); out[2] = lo_h(a.z); out[3] = lo_h(a.w);
@@ -1412,7 +1588,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) ok = ok && (4 * lane + i >= E || tag_ok(w[i], ta));
       return ok;
-    }, uni(P.bar) + 32);
+    }, uni(P.bar) + 32, 8u);
     fstamp<ST>(li, FS_B, 1, tid == 0);
     const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
     if (wave == 0) {
@@ -1546,7 +1722,7 @@ SL_DEV bool flow_moe_c(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
       }
       if (tid == 0) { ok = ok && tag_ok(gw1, ta); L.gb[1] = lo_h(gw1); }
       return ok;
-    }, uni(P.bar) + 32);
+    }, uni(P.bar) + 32, 9u);
     // a share of 32 activations = the chunks of eight neighbouring threads: its sum (the balanced tree over the 16 pair
     // sums) goes into the padding word behind the share's packed pairs
 #pragma unroll
@@ -1677,7 +1853,7 @@ SL_DEV bool flow_head(const FlowP& F, int pos, int out_off, int feed, uint32_t b
     for (;;) {
       bool ok = true;
       if (tid < G) { const uint4 c = ldw4(rc, tid * 4); ok = c.z == thd32 && c.w == thd32; v = __uint_as_float(c.x); i = (int)c.y; }
-      const int r = flow_round(ok, spins, uni(P.bar) + 32);
+      const int r = flow_round(ok, spins, uni(P.bar) + 32, 10u);
       if (r > 0) break;
       if (r < 0) return false;
     }
@@ -1735,7 +1911,7 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
   const int nl = uni(P.n_layers);
   // A workgroup that leaves (a wait gave up, or the launch is over) first lets its outstanding loads land: rows on
   // their way into LDS must not arrive after the LDS has passed to another workgroup.
-#define FLOW_TRY(call) do { if (!(call)) { wr_wait(); return; } } while (0)
+#define FLOW_TRY(call) do { if (!(call)) goto flow_exit; } while (0)
   flow_request_in(g_K.layers[0]);
   for (int step = 0; step < steps; ++step) {
     const uint32_t base = uni(g_K.base);
@@ -1770,8 +1946,9 @@ __global__ __launch_bounds__(DEC_THREADS) void k_decode_flow(const FlowP* __rest
     }
   }
 #undef FLOW_TRY
+flow_exit:
   wr_wait();
-  if constexpr (ST) {
+  if constexpr (ST) {                                  // (also after a wait that gave up: the stamps show where every workgroup stood)
     __syncthreads();
     uint32_t* dst = uni(P.tstamp) + (size_t)blockIdx.x * STAMP_WORDS;
     for (int i = threadIdx.x; i < STAMP_WORDS; i += DEC_THREADS) dst[i] = g_stamps[i];

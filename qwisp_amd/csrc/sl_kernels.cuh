@@ -1604,11 +1604,13 @@ __global__ __launch_bounds__(1024) void k_sdpa_merge_long(SdpaMergeArgs a) {
   Mx = tree_max<64>(Mx);
   const int d = 64 * wave + lane;
   const uint16_t graw = a.proj[(size_t)m * PROJ_STRIDE + h * 512 + 256 + d];
-  float L = 0.0f, O = 0.0f;
+  float L = 0.0f, O = 0.0f, La = 0.0f, Oa = 0.0f;         // the block's chains (from zero), the sum of the blocks before
   float pmv = a.pm[base + min(lane, nt - 1)], plv = a.pl[base + min(lane, nt - 1)];
   for (int k = 0; k <= nb; ++k) {
     if (k >= 1) {
       const int kb = k - 1, t0 = MERGE_BLOCK * kb, cnt = min(MERGE_BLOCK, nt - t0);
+      if (kb == 1) { La = L; Oa = O; } else if (kb > 1) { La = La + L; Oa = Oa + O; }
+      if (kb >= 1) { L = 0.0f; O = 0.0f; }
       const float fl = (lane < cnt) ? exp_c(pmv - Mx) : 0.0f, pl = (lane < cnt) ? plv : 0.0f;
       if (k < nb) { pmv = a.pm[base + min(t0 + MERGE_BLOCK + lane, nt - 1)]; plv = a.pl[base + min(t0 + MERGE_BLOCK + lane, nt - 1)]; }
       const float* const src = s_park + (size_t)(kb & 1) * MERGE_BLOCK * 256 + d;
@@ -1629,6 +1631,7 @@ __global__ __launch_bounds__(1024) void k_sdpa_merge_long(SdpaMergeArgs a) {
     }
     lds_barrier();
   }
+  if (nb > 1) { L = La + L; O = Oa + O; }
   const float r = f16r(f16r(O / L) * sigmoid16(h2f(graw)));
   a.gated[(size_t)m * 4096 + h * 256 + d] = f2h(r);
   if (a.gsum) {                                          // a share of 32 values sits on 32 neighbouring lanes
@@ -1645,8 +1648,15 @@ __global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
   for (int t = lane; t < nt; t += 64) Mx = fmaxf(Mx, a.pm[base + t]);
   Mx = tree_max<64>(Mx);
   // tiles are added up in order; sixteen tiles' partials are requested together (one memory round trip per sixteen tiles)
-  float L = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  // (a chain per block of 64 tiles, the blocks' chains added in block order)
+  float L = 0.0f, O[4] = {0.0f, 0.0f, 0.0f, 0.0f}, La = 0.0f, Oa[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   for (int t0 = 0; t0 < nt; t0 += 16) {
+    if (t0 >= MERGE_BLOCK && t0 % MERGE_BLOCK == 0) {
+      const bool first = t0 == MERGE_BLOCK;
+      La = first ? L : La + L; L = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { Oa[i] = first ? O[i] : Oa[i] + O[i]; O[i] = 0.0f; }
+    }
     float4 o[16];
     float pmv[16], plv[16];
 #pragma unroll
@@ -1663,6 +1673,11 @@ __global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
         O[0] = fmaf(o[u].x, f, O[0]); O[1] = fmaf(o[u].y, f, O[1]); O[2] = fmaf(o[u].z, f, O[2]); O[3] = fmaf(o[u].w, f, O[3]);
       }
     }
+  }
+  if (nt > MERGE_BLOCK) {
+    L = La + L;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) O[i] = Oa[i] + O[i];
   }
   const uint2 graw = *reinterpret_cast<const uint2*>(a.proj + (size_t)m * PROJ_STRIDE + h * 512 + 256 + 4 * lane);
   const float gt[4] = {lo_h(graw.x), hi_h(graw.x), lo_h(graw.y), hi_h(graw.y)};

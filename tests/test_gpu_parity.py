@@ -610,6 +610,28 @@ def test_persistent_step_long_context(env, small_model):
             assert same_bits(x, y), (li, first_diff(x, y))
 
 
+@pytest.mark.parametrize("ctx", [900, 3000])
+def test_persistent_step_merge_waits_for_late_tiles(env, small_model, ctx):
+    """13 to 128 key tiles per head: fourteen waves of a merging workgroup fetch the tiles' partial sums, and the
+    tile that holds the new position is published last.  A wave whose first look comes too early has to look again:
+    its loop must issue new loads (the optimiser once hoisted them out of the loop, and the step gave up waiting).
+    Same tokens and logits as the kernel-per-stage sequence."""
+    cfg, dev, host = small_model
+    a = env["Engine"](cfg, dev, max_m=64, max_seq_len=ctx + 64)
+    b = env["Engine"](cfg, dev, max_m=64, max_seq_len=ctx + 64)
+    assert b.set_persistent(False)
+    toks = np.random.default_rng(77).integers(0, cfg.vocab, ctx).astype(np.int32)
+    for eng in (a, b):
+        for i in range(0, len(toks), 64):
+            assert eng.step_argmax(toks[i:i + 64]) is not None, eng.gpu_fault
+    ta = a.chained_step_argmax(11, 6)
+    tb = b.chained_step_argmax(11, 6)
+    assert ta is not None and tb is not None, (a.gpu_fault, b.gpu_fault)
+    assert ta.tolist() == tb.tolist()
+    assert same_bits(a.logits_row(0), b.logits_row(0))
+    a.close(); b.close()
+
+
 @pytest.mark.parametrize("round_units", [None, 1])
 def test_persistent_step_with_several_tile_units_per_workgroup(env, small_model, monkeypatch, round_units):
     """Beyond 7168 tokens of context there are more (key tile, kv head) units than the workgroups that take them
