@@ -380,7 +380,9 @@ int sl_set_hybrid(sl_engine* e, int enable);
  * out[wg * sl_stage_clock_words() + (layer * 8 + stage) * 8 + kind], 0 = not reached; stage 0 in-projection, 1 recurrence
  * or attention tiles, 2 attention merge, 3 K = 4096 projection, 4 router and shared gate/up, 5 routed gate/up, 6 down and
  * combine; layer n_layers = head (stage 0 lm_head, 1 final arg-max); kind 0 stage entered, 1 inputs arrived,
- * 2 preparation done, 3 arithmetic done, 4 results stored. */
+ * 2 preparation done, 3 arithmetic done, 4 results stored.  A launch whose waits gave up copies its stamps out as
+ * well, and reading them (enable = 0, out != NULL) is the one call a poisoned engine still answers: the stamps show
+ * where every workgroup stood; the fault text names the wait that gave up first. */
 int sl_debug_stage_clock(sl_engine* e, int enable, uint32_t* out, int cap_words);
 int sl_stage_clock_words(void);
 /* Test hook beside injectCBFailure (SFV:404) for the single-launch step's own failure path: after `rounds` unanswered

@@ -1570,20 +1570,21 @@ __global__ __launch_bounds__(1024) void k_sdpa_merge_long(SdpaMergeArgs a) {
     // tiles i = (wave - 4) + 12 j of a block, j = 0..5; two register sets take turns, a set is parked and at once
     // requested again for the block after the next (indices clamped into the context: every load is unconditional)
     constexpr int PER = 6;
-    float4 qa[PER], qb[PER];
-    auto request = [&](float4 (&dst)[PER], int blk) {
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));       // (a native vector: arrays of HIP's float4 ended up in scratch memory here)
+    f32x4_t qa[PER], qb[PER];
+    auto request = [&](f32x4_t (&dst)[PER], int blk) __attribute__((always_inline)) {
 #pragma unroll
       for (int j = 0; j < PER; ++j) {
         const int t = min(MERGE_BLOCK * min(blk, nb - 1) + min((wave - 4) + 12 * j, MERGE_BLOCK - 1), nt - 1);
-        dst[j] = *reinterpret_cast<const float4*>(a.po + (base + t) * 256 + 4 * lane);
+        dst[j] = *reinterpret_cast<const f32x4_t*>(a.po + (base + t) * 256 + 4 * lane);
       }
     };
-    auto park = [&](const float4 (&src)[PER], int blk) {
+    auto park = [&](const f32x4_t (&src)[PER], int blk) __attribute__((always_inline)) {
       float* const dst = s_park + (size_t)(blk & 1) * MERGE_BLOCK * 256;
 #pragma unroll
       for (int j = 0; j < PER; ++j) {
         const int i = (wave - 4) + 12 * j;
-        if (i < MERGE_BLOCK) *reinterpret_cast<float4*>(dst + i * 256 + 4 * lane) = src[j];
+        if (i < MERGE_BLOCK) *reinterpret_cast<f32x4_t*>(dst + i * 256 + 4 * lane) = src[j];
       }
     };
     request(qa, 0);
