@@ -72,15 +72,16 @@ def test_generator_device_equals_host(env):
 # ---- matrix-core GEMM of the hybrid prefill ---------------------------------------------------------
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("m", [2, 3, 4, 5, 8, 9, 13, 17, 32])
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 8, 9, 13, 16, 17, 32, 49, 127])
 def test_row_tiles_of_any_count_equal_single_steps(env, small_model, m):
     """The row kernels take activation rows in tiles of 8 (in-projection, lm_head) and 4 (out-projection): full
     tiles, ragged last tiles and several tiles give, row by row, the bits of single steps (SeedlessVerifyTests.swift:613).
     Steps of up to 4 and up to 8 rows take the launch-saving variants (in-projection waves that prepare their rows, the
-    GDN core of a value head in one workgroup, stage B routing for itself); 9 rows and more the general row kernels."""
+    GDN core of a value head in one workgroup, stage B routing for itself); 9 rows and more the general row kernels, up to
+    the 127 rows below the steps whose experts are grouped."""
     cfg, dev, host = small_model
-    a = env["Engine"](cfg, dev, max_m=32, max_seq_len=96)
-    b = env["Engine"](cfg, dev, max_m=32, max_seq_len=96)
+    a = env["Engine"](cfg, dev, max_m=max(32, m), max_seq_len=160)
+    b = env["Engine"](cfg, dev, max_m=max(32, m), max_seq_len=160)
     rng = np.random.default_rng(500 + m)
     pre = rng.integers(0, cfg.vocab, 7).tolist()
     assert a.step_argmax(pre).tolist() == b.step_argmax(pre).tolist()
@@ -328,6 +329,26 @@ def test_moe_block_rows(moe_model, m, seed):
     assert same_bits(gs, ws), first_diff(gs, ws)
     assert same_bits(got, want), first_diff(got, want)
     assert np.isfinite(got.astype(np.float32)).all() and np.abs(got.astype(np.float32)).max() > 0
+
+
+@pytest.mark.parametrize("m,seed", [(16, 1200), (49, 1201), (127, 1202)])
+def test_moe_block_of_a_lane_sized_step_against_the_oracle(env, m, seed):
+    """16 to 127 rows (a batch of lanes, a small prefill chunk) with all 256 experts: many experts are chosen by
+    several rows of the step, each (row, expert) pair is still computed on its own.  Routing and output carry the
+    oracle's bits, on a second call over other rows as well."""
+    cfg = ModelConfig(n_layers=1, n_experts=256, vocab=0, layer_types=("gdn",))
+    dev, host = device_and_host_model(cfg)
+    eng = env["Engine"](cfg, dev, max_m=m, max_seq_len=16)
+    ora = env["orc"].Oracle(cfg, host, max_m=m, max_seq_len=16)
+    for call in range(2):
+        x = xrows(m, seed + 50 * call)
+        got, want = eng.moe_block_rows(0, x), ora.moe_block_rows(0, x)
+        assert got is not None, eng.gpu_fault
+        gi, gs = eng.read_route(0, m)
+        wi, ws = ora.read_route(0, m)
+        assert np.array_equal(gi, wi) and same_bits(gs, ws)
+        assert same_bits(got, want), (call, first_diff(got, want))
+    eng.close()
 
 
 def test_moe_block_rows_with_8bit_gates(env):

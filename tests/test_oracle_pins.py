@@ -312,7 +312,9 @@ def test_swiglu_against_float64():
 
 
 # ---- attention -------------------------------------------------------------------------------------
-@pytest.mark.parametrize("N", [1, 2, 63, 64, 65, 129, 300])
+# (4096 keys = one block of 64 tiles; 4097, 8200 and 12345 keys = two, three and four blocks: the blocks' chains start
+# from zero and are added in block order, so a block dropped, counted twice or scaled by another block's maximum fails)
+@pytest.mark.parametrize("N", [1, 2, 63, 64, 65, 129, 300, 4096, 4097, 8200, 12345])
 def test_sdpa_against_float64(N):
     q = rng.normal(0, 1, 256).astype(np.float16)
     k = rng.normal(0, 1, (N, 256)).astype(np.float16)
@@ -344,6 +346,20 @@ def test_sdpa_equal_keys_average_values_and_ignore_the_tail():
     out2 = np.empty(256, np.float16)
     dll.orc_sdpa(orc.p(q), orc.p(k2), orc.p(v2), N, orc.p(out2))
     assert np.array_equal(out, out2)
+
+
+def test_sdpa_blocks_of_tiles_weigh_every_key_once():
+    """Equal keys over three blocks of 64 tiles: every key has the same weight, so the output is the mean of all values;
+    with the values of one block set apart (100 in block 1, 0 elsewhere) the output is that block's share of the keys."""
+    N = 64 * 64 * 2 + 777
+    q = rng.normal(0, 1, 256).astype(np.float16)
+    k = np.tile(rng.normal(0, 1, (1, 256)).astype(np.float16), (N, 1))
+    v = np.zeros((N, 256), np.float16)
+    v[4096:8192] = 100.0
+    out = np.empty(256, np.float16)
+    dll.orc_sdpa(orc.p(q), orc.p(k), orc.p(v), N, orc.p(out))
+    ref = 100.0 * 4096 / N
+    assert np.all(np.abs(out.astype(np.float64) - ref) <= 2.0 ** -10 * ref), (out[:4], ref)
 
 
 def test_rope_table_and_rotation():
