@@ -257,7 +257,33 @@ __global__ __launch_bounds__(64 * WPB) void k_qmm4_mfma16(QmmArgs a) {
       }
     }
   }
-  // D layout of a 32x32 tile: register r of lane (col, hh) holds row 8*(r/4) + 4*hh + r%4, column col
+  // D layout of a 32x32 tile: register r of lane (col, hh) holds row 8*(r/4) + 4*hh + r%4, column col.  Stored from
+  // there a value is a two-byte store with an address of its own; where the workgroup's tile fits the staging space
+  // (and rows of Y start on 16-byte boundaries) it is laid down in LDS [row][column] and goes out in 16-byte pieces.
+  constexpr int TC = WPB * NS * 32, YS = TC + 8;         // columns of the workgroup's tile, halves per row in LDS
+  if constexpr (RT * 32 * YS <= 2 * RT * 32 * XS) {
+    if ((a.y_stride & 7) == 0 && (reinterpret_cast<uintptr_t>(yout) & 15) == 0) {     // uniform
+      uint16_t* const ys = &xs[0][0];
+      __syncthreads();                                   // the last chunk has been read
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            ys[(t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3)) * YS + (wave * NS + s) * 32 + col] = f2h(acc[t][s][r]);
+      __syncthreads();
+      const int nwg = tile.col_block * TC;
+      constexpr int PPR = TC / 8, PIECES = RT * 32 * PPR;  // 16-byte pieces per row, per tile
+#pragma unroll
+      for (int p = 0; p < (PIECES + NT - 1) / NT; ++p) {
+        const int idx = p * NT + tid, row = idx / PPR, piece = idx % PPR;
+        if (idx < PIECES && m0 + row < a.M && nwg + piece * 8 < a.N)
+          st16(yout + (size_t)(m0 + row) * a.y_stride + nwg + piece * 8, *reinterpret_cast<const uint4*>(&ys[row * YS + piece * 8]));
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int s = 0; s < NS; ++s) {
     if (n0 + 32 * s >= a.N) continue;
@@ -488,18 +514,30 @@ SL_DEV void grouped_pass(const QmmGroupArgs& a, uint16_t* xsb, const uint16_t* l
       }
     }
   }
-  if (live) {
+  // The results leave through LDS: a lane holds sixteen rows of one column, and stored from there every value would
+  // be a two-byte store with a row look-up and an address of its own (a third of the instructions of a short
+  // K = 512 pass).  The tile is laid down [row][128 columns of the workgroup] in the staging space instead and goes
+  // out in 16-byte pieces, two per thread and 32-row tile.
+  constexpr int YS = 128 + 8;                            // halves per row of the result tile
+  static_assert(RT * 32 * YS <= 2 * BUF, "the result tile fits the staging buffers");
+  __syncthreads();                                       // the last chunk has been read
+  const int wcol = (tid >> 6) * 32 + col;
 #pragma unroll
-    for (int t = 0; t < RT; ++t)
+  for (int t = 0; t < RT; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-        if (row < cnt) {
-          float v = f16r(acc[t][0][r]);
-          if constexpr (DUAL) v = swiglu_mm(v, f16r(acc[t][1][r]));
-          a.y[(size_t)list[row] * a.y_stride + n0 + col] = f2h(v);
-        }
-      }
+    for (int r = 0; r < 16; ++r) {
+      const int row = t * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+      float v = acc[t][0][r];
+      if constexpr (DUAL) v = swiglu_mm(f16r(v), f16r(acc[t][1][r]));
+      xsb[row * YS + wcol] = f2h(v);
+    }
+  __syncthreads();
+  const int nwg = n0 - (tid >> 6) * 32;                  // first column of the workgroup
+#pragma unroll
+  for (int p = 0; p < RT * 2; ++p) {
+    const int idx = p * 256 + tid, row = idx >> 4, piece = idx & 15;
+    if (row < cnt && nwg + piece * 8 < a.NE)
+      st16(a.y + (size_t)list[row] * a.y_stride + nwg + piece * 8, *reinterpret_cast<const uint4*>(&xsb[row * YS + piece * 8]));
   }
 }
 template <bool DUAL>
