@@ -54,6 +54,10 @@ struct LayerDev {
 constexpr size_t HIST_ELEMS = (size_t)(SL_CONV_K - 1) * SL_CONV_DIM;
 constexpr size_t STATE_ELEMS = (size_t)SL_GDN_HV * SL_GDN_D * SL_GDN_D;
 constexpr int MAX_CHAIN = 256;
+#ifndef SL_MERGE_BLOCKS_ROWS
+#define SL_MERGE_BLOCKS_ROWS 8
+#endif
+constexpr int MERGE_BLOCKS_ROWS = SL_MERGE_BLOCKS_ROWS;   // steps of up to this many rows: the blocks' chains side by side, a workgroup per quarter head
 constexpr int MERGE_LONG_ROWS = 64;      // steps of up to this many rows merge their attention tiles with the 16-wave kernel
 constexpr int ROUTER_PAD_ROWS = 288;
 
@@ -493,6 +497,7 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
   g.gsum = mm ? nullptr : e->ysum;                       // the exact merge leaves the gated rows' word sums for the projection
   if (mm && lanes) hipLaunchKernelGGL(k_sdpa_merge_par<16>, dim3(SL_ATT_HEADS, M), dim3(1024), 0, e->stream, g);
   else if (mm) hipLaunchKernelGGL(k_sdpa_merge_par<4>, dim3(SL_ATT_HEADS, M), dim3(256), 0, e->stream, g);
+  else if (M <= MERGE_BLOCKS_ROWS) hipLaunchKernelGGL(k_sdpa_merge_blocks, dim3(SL_ATT_HEADS, M, 4), dim3(64 * MERGE_BLOCKS_WAVES), 0, e->stream, g);
   else if (M <= MERGE_LONG_ROWS) hipLaunchKernelGGL(k_sdpa_merge_long, dim3(SL_ATT_HEADS, M), dim3(1024), MERGE_DYN_LDS, e->stream, g);
   else hipLaunchKernelGGL(k_sdpa_merge, dim3(SL_ATT_HEADS, M), dim3(64), 0, e->stream, g);
   if (mm && !(lanes && M < MM_OUT_ROWS)) launch_qmm4_mfma(QmmArgs{e->ycore, 4096, L.o_proj.w, L.o_proj.sb, M, H, 4096, e->mix, H}, e->stream);

@@ -1640,6 +1640,84 @@ __global__ __launch_bounds__(1024) void k_sdpa_merge_long(SdpaMergeArgs a) {
     if ((lane & 31) == 0) a.gsum[(size_t)m * 128 + h * 8 + (d >> 5)] = sw;
   }
 }
+// The same merge with the blocks' chains side by side: the chain of a block of 64 tiles starts from zero and the
+// blocks' chains are added in block order, so the blocks are independent until that last addition.  One workgroup of
+// four waves per (head, row, quarter of the head's dims): lane = dim, wave w takes blocks w, w + 4, ... -- the 64
+// partial sums of a block are 64 loads per lane in flight at once (one round trip per block instead of one per
+// sixteen tiles), the next block of the wave already requested while this one is added up -- and after every group
+// of four blocks wave 0 adds their chains in block order.  For steps of a few rows at long contexts, where the
+// 16 x M workgroups of the other kernels leave most of the machine idle and walk the tiles one round trip after another.
+constexpr int MERGE_BLOCKS_WAVES = 4;
+__global__ __launch_bounds__(64 * MERGE_BLOCKS_WAVES) void k_sdpa_merge_blocks(SdpaMergeArgs a) {
+  constexpr int W = MERGE_BLOCKS_WAVES;
+  __shared__ float s_o[2][W][64];
+  __shared__ float s_l[2][W];
+  const int h = blockIdx.x, m = blockIdx.y, q = blockIdx.z, tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int N = a.lanes ? a.lanes[m].st[0] + 1 : a.st[0] + m + 1;
+  const int nt = (N + SDPA_TILE - 1) / SDPA_TILE, nb = (nt + MERGE_BLOCK - 1) / MERGE_BLOCK;
+  const size_t base = ((size_t)m * 16 + h) * a.maxTiles;
+  const int d = 64 * q + lane;
+  const float* const po = a.po + base * 256 + d;
+  float v[MERGE_BLOCK], vn[MERGE_BLOCK];
+  auto request = [&](float (&dst)[MERGE_BLOCK], int b) __attribute__((always_inline)) {
+    const int t0 = MERGE_BLOCK * b;                        // (tiles beyond the context repeat its last tile and are not used)
+#pragma unroll
+    for (int i = 0; i < MERGE_BLOCK; ++i) dst[i] = po[(size_t)min(t0 + i, nt - 1) * 256];
+  };
+  if (wave < nb) request(v, wave);
+  // lane i: {max, sum} of tile i of the wave's block (requested with the block, ahead of the maximum over all tiles)
+  auto tile_ml = [&](int b, float& pm, float& pl) __attribute__((always_inline)) {
+    const size_t i = base + min(MERGE_BLOCK * min(b, nb - 1) + lane, nt - 1);
+    pm = a.pm[i]; pl = a.pl[i];
+  };
+  float pmv, plv, pmn = 0.0f, pln = 0.0f;
+  tile_ml(wave, pmv, plv);
+  float Mx = -__int_as_float(0x7f800000);
+  for (int t = lane; t < nt; t += 64) Mx = fmaxf(Mx, a.pm[base + t]);
+  Mx = tree_max<64>(Mx);
+  const uint16_t graw = a.proj[(size_t)m * PROJ_STRIDE + h * 512 + 256 + d];
+  float L = 0.0f, O = 0.0f;                                // wave 0: the blocks' chains added up so far
+  for (int g0 = 0, k = 0; g0 < nb; g0 += W, k ^= 1) {
+    const int b = g0 + wave;
+    if (b < nb) {
+      const int t0 = MERGE_BLOCK * b, cnt = min(MERGE_BLOCK, nt - t0);
+      if (b + W < nb) { request(vn, b + W); tile_ml(b + W, pmn, pln); }
+      const float fl = (lane < cnt) ? exp_c(pmv - Mx) : 0.0f, pl = (lane < cnt) ? plv : 0.0f;
+      float Lb = 0.0f, Ob = 0.0f;
+#pragma unroll
+      for (int u0 = 0; u0 < MERGE_BLOCK; u0 += 8) {
+        if (u0 < cnt) {                                    // uniform for the wave
+          float f[8], l[8];
+          lanes8(fl, u0, f);
+          lanes8(pl, u0, l);
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (u0 + i < cnt) { Lb = fmaf(l[i], f[i], Lb); Ob = fmaf(v[u0 + i], f[i], Ob); }
+        }
+      }
+      s_o[k][wave][lane] = Ob;
+      if (lane == 0) s_l[k][wave] = Lb;
+#pragma unroll
+      for (int i = 0; i < MERGE_BLOCK; ++i) v[i] = vn[i];
+      pmv = pmn; plv = pln;
+    }
+    __syncthreads();                                       // (the other buffer is written next: one barrier per group)
+    if (wave == 0) {
+      for (int w = 0; w < W && g0 + w < nb; ++w) {
+        const float ob = s_o[k][w][lane], lb = s_l[k][w];
+        if (g0 + w == 0) { O = ob; L = lb; } else { O = O + ob; L = L + lb; }
+      }
+    }
+  }
+  if (wave != 0) return;
+  const float r = f16r(f16r(O / L) * sigmoid16(h2f(graw)));
+  a.gated[(size_t)m * 4096 + h * 256 + d] = f2h(r);
+  if (a.gsum) {                                            // a share of 32 values sits on 32 neighbouring lanes
+    const float sw = tree_sum<32>(r);
+    if ((lane & 31) == 0) a.gsum[(size_t)m * 128 + h * 8 + (d >> 5)] = sw;
+  }
+}
 __global__ __launch_bounds__(64) void k_sdpa_merge(SdpaMergeArgs a) {
   const int h = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;
   const int N = a.lanes ? a.lanes[m].st[0] + 1 : a.st[0] + m + 1;
