@@ -13,6 +13,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "sl_flow.cuh"
@@ -509,20 +510,21 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
 // All layers over M rows held in hA.  On return the hidden state is hA + moe_out (residual pending).
 // With `lane_tab` the M rows are one token each of M lanes (caches and positions from the table, the longest
 // lane needing `lane_tiles` key tiles); without, M consecutive rows of this engine's own sequence.
+void launch_layer(sl_engine* e, int li, int M, const LaneRef* lane_tab = nullptr, int lane_tiles = 0) {
+  LayerDev& L = e->layers[li];
+  const LaneRef* lanes = lane_tab ? lane_tab + (size_t)li * e->max_m : nullptr;
+  HiddenArgs ha{e->hA, li > 0 ? e->moe_out : nullptr, L.input_ln, e->hB, nullptr};
+  if (L.is_linear) launch_gdn_mixer(e, L, li, M, ha, lanes);
+  else launch_attn_mixer(e, L, M, ha, lanes, lane_tiles);
+  HiddenArgs hb{e->hB, e->mix, L.post_ln, e->hA, e->xn};
+  // grouping by expert pays once an expert sees several rows; a batch of fewer than 64 lanes leaves most experts
+  // with one row or none, and the per-row expert kernels stream the same weights with less overhead (rows of one
+  // sequence always take the grouped path, so that a row's result does not depend on the size of its chunk)
+  if (use_matrix_cores(e, M, lanes) && (!lanes || M >= 64)) launch_moe_hybrid(e, L, M, hb);
+  else launch_moe(e, L, M, hb);
+}
 void launch_layers(sl_engine* e, int M, const LaneRef* lane_tab = nullptr, int lane_tiles = 0) {
-  for (int li = 0; li < e->n_layers; ++li) {
-    LayerDev& L = e->layers[li];
-    const LaneRef* lanes = lane_tab ? lane_tab + (size_t)li * e->max_m : nullptr;
-    HiddenArgs ha{e->hA, li > 0 ? e->moe_out : nullptr, L.input_ln, e->hB, nullptr};
-    if (L.is_linear) launch_gdn_mixer(e, L, li, M, ha, lanes);
-    else launch_attn_mixer(e, L, M, ha, lanes, lane_tiles);
-    HiddenArgs hb{e->hB, e->mix, L.post_ln, e->hA, e->xn};
-    // grouping by expert pays once an expert sees several rows; a batch of fewer than 64 lanes leaves most experts
-    // with one row or none, and the per-row expert kernels stream the same weights with less overhead (rows of one
-    // sequence always take the grouped path, so that a row's result does not depend on the size of its chunk)
-    if (use_matrix_cores(e, M, lanes) && (!lanes || M >= 64)) launch_moe_hybrid(e, L, M, hb);
-    else launch_moe(e, L, M, hb);
-  }
+  for (int li = 0; li < e->n_layers; ++li) launch_layer(e, li, M, lane_tab, lane_tiles);
 }
 void advance(sl_engine* e, int M) {
   hipLaunchKernelGGL(k_advance, dim3(1), dim3(64), 0, e->stream, e->st, M, e->n_layers);
@@ -915,6 +917,22 @@ bool lanes_batchable(sl_engine** lanes, int b) {
   }
   return true;
 }
+// How a batch of lanes is split into groups that are stepped side by side (sl_lane_step_argmax): [off[g], off[g+1]) are
+// the lanes of group g, its first lane lends scratch rows and stream.  Two groups from 32 lanes on, so that a group
+// keeps the 16 rows that the matrix-core kernels of hybrid mode want.  (Measured at 32 lanes of 1K-16K tokens: one group
+// 9.83 ms per step of exact rows and 8.0 ms hybrid, two groups 9.14 and 7.9, four groups of 8 rows 14.9: the device
+// then spends its time on 2000 launches.)
+constexpr int LANE_GROUPS_MAX = 2, LANE_GROUP_ROWS = 16;
+int lane_groups(sl_engine** lanes, int b, int* off) {
+  int ng = b >= 2 * LANE_GROUP_ROWS ? 2 : 1;
+  for (int g = 0; g <= ng; ++g) off[g] = (int)((long long)b * g / ng);
+  for (int g = 1; g < ng; ++g) {                    // every group's first lane must be able to drive it
+    sl_engine* dg = lanes[off[g]];
+    const int n = off[g + 1] - off[g];
+    if (n > dg->max_m || !dg->has_head || dg->max_seq != lanes[0]->max_seq) { ng = 1; off[1] = b; break; }
+  }
+  return ng;
+}
 // Device table of the lanes' caches, [n_layers][max_m] in the driver; rebuilt when the set of lanes changes.
 int bind_lanes(sl_engine* d, sl_engine** lanes, int b) {
   if ((int)d->lane_set.size() == b &&
@@ -958,37 +976,91 @@ int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t
     return SL_OK;
   }
   sl_engine* d = lanes[0];
-  int max_pos = 0;
   for (int i = 0; i < b; ++i) {
     int r = guard(lanes[i]); if (r) return r;
     if (tokens[i] < 0 || tokens[i] >= d->vocab) return SL_ERR_ARG;
     if (lanes[i]->has_attn && lanes[i]->pos + 1 > lanes[i]->max_seq) return SL_ERR_ARG;
-    if (lanes[i]->pos > max_pos) max_pos = lanes[i]->pos;
   }
-  int r = bind_lanes(d, lanes, b); if (r) return r;
+  // Two groups of lanes, each on the scratch rows and the stream of its first lane, queued layer by layer in turn:
+  // the two launch sequences run side by side on the device, so the short kernels of one group (norms, routing,
+  // gates: a third of a step's launches, a few microseconds each and bound by nothing but their start and end) and the
+  // ends of its large ones are covered by the other group's kernels.  The dense weights are streamed once per group
+  // instead of once per step (5 % of a 32-lane step's bytes); what a lane computes does not change.
+  int off[LANE_GROUPS_MAX + 1];
+  const int ng = lane_groups(lanes, b, off);
+  int tiles[LANE_GROUPS_MAX];
+  for (int g = 0; g < ng; ++g) {
+    sl_engine* dg = lanes[off[g]];
+    const int n = off[g + 1] - off[g];
+    if (g > 0 && d->hybrid != dg->hybrid) { const int r = sl_set_hybrid(dg, d->hybrid ? 1 : 0); if (r) return r; }
+    int max_pos = 0;
+    for (int i = off[g]; i < off[g + 1]; ++i) if (lanes[i]->pos > max_pos) max_pos = lanes[i]->pos;
+    tiles[g] = (max_pos + 1 + SDPA_TILE - 1) / SDPA_TILE;
+    const int r = bind_lanes(dg, lanes + off[g], n); if (r) return r;
+  }
   // work queued on the other lanes' own streams (none after a completed call) must not overlap this step
   for (int i = 1; i < b; ++i) SL_TRY(lanes[i], hipStreamSynchronize(lanes[i]->stream));
-  r = to_device(d, d->tok_in, tokens, (size_t)b * 4); if (r) return r;
   SL_TRY(d, hipEventRecord(d->ev0, d->stream));
-  hipLaunchKernelGGL(k_embed, dim3(H / 256, b), dim3(256), 0, d->stream, d->tok_in, d->embed.w, d->embed.sb, d->hA);
-  launch_layers(d, b, d->lane_tab, (max_pos + 1 + SDPA_TILE - 1) / SDPA_TILE);
-  HiddenArgs ha{d->hA, d->moe_out, d->final_norm, d->hB, d->normed};
-  launch_head(d, b, ha, 0, false);
-  hipLaunchKernelGGL(k_lane_advance, dim3(b), dim3(64), 0, d->stream, d->lane_tab, d->n_layers);
+  for (int g = 0; g < ng; ++g) {
+    sl_engine* dg = lanes[off[g]];
+    const int n = off[g + 1] - off[g];
+    const int r = to_device(dg, dg->tok_in, tokens + off[g], (size_t)n * 4); if (r) return r;
+    if (g > 0) SL_TRY(dg, hipStreamWaitEvent(dg->stream, d->ev0, 0));      // (the step's time is measured on the first group's stream)
+    hipLaunchKernelGGL(k_embed, dim3(H / 256, n), dim3(256), 0, dg->stream, dg->tok_in, dg->embed.w, dg->embed.sb, dg->hA);
+  }
+  // (a host thread per further group: one thread queues some 500 launches of a step in about 3.5 ms, which would bound
+  // a step of two groups from below)
+  hipError_t queued[LANE_GROUPS_MAX];
+  auto queue_group = [&](int g) {
+    sl_engine* dg = lanes[off[g]];
+    const int n = off[g + 1] - off[g];
+    if (g > 0) { (void)hipSetDevice(dg->device); (void)hipGetLastError(); }
+    launch_layers(dg, n, dg->lane_tab, tiles[g]);
+    HiddenArgs ha{dg->hA, dg->moe_out, dg->final_norm, dg->hB, dg->normed};
+    launch_head(dg, n, ha, 0, false);
+    hipLaunchKernelGGL(k_lane_advance, dim3(n), dim3(64), 0, dg->stream, dg->lane_tab, dg->n_layers);
+    queued[g] = g > 0 ? hipGetLastError() : hipSuccess;   // (a helper's launch errors are its thread's: handed back here)
+  };
+  {
+    std::vector<std::thread> helpers;
+    for (int g = 1; g < ng; ++g) helpers.emplace_back(queue_group, g);
+    queue_group(0);
+    for (auto& t : helpers) t.join();
+  }
+  for (int g = 1; g < ng; ++g)
+    if (!ok(d, queued[g], "stepArgmaxBatch (second group)")) {
+      for (int h = 0; h < ng; ++h) (void)hipStreamSynchronize(lanes[off[h]]->stream);
+      for (int i = 1; i < b; ++i) if (lanes[i]->fault.empty()) lanes[i]->fault = d->fault;
+      return SL_ERR_DEVICE;
+    }
+  for (int g = 1; g < ng; ++g) {                         // the first group's stream ends the step: it waits for the others
+    sl_engine* dg = lanes[off[g]];
+    SL_TRY(dg, hipEventRecord(dg->ev1, dg->stream));
+    SL_TRY(d, hipStreamWaitEvent(d->stream, dg->ev1, 0));
+  }
   SL_TRY(d, hipEventRecord(d->ev1, d->stream));
-  r = read_back(d, out, d->tok_out, (size_t)b * 4, "stepArgmaxBatch");
+  int r = SL_OK;
+  for (int g = 0; g < ng && !r; ++g) {
+    sl_engine* dg = lanes[off[g]];
+    r = read_back(dg, out + off[g], dg->tok_out, (size_t)(off[g + 1] - off[g]) * 4, "stepArgmaxBatch");
+    if (r && d->fault.empty()) d->fault = dg->fault;
+  }
   if (r) {   // the lanes' caches were written by the failed step: all of them are unusable
+    for (int g = 1; g < ng; ++g) (void)hipStreamSynchronize(lanes[off[g]]->stream);
     for (int i = 1; i < b; ++i) if (lanes[i]->fault.empty()) lanes[i]->fault = d->fault;
     return r;
   }
   time_end(d);
-  for (int i = 0; i < b; ++i) {
-    sl_engine* l = lanes[i];
-    l->pos += 1;
-    for (int j = 0; j < l->n_layers; ++j) if (l->layers[j].is_linear) l->parity[j] ^= 1;
-    l->logits_view = d->logits + (size_t)i * d->vocab;
-    l->normed_view = d->normed + (size_t)i * H;
-    l->last_ms = d->last_ms;
+  for (int g = 0; g < ng; ++g) {
+    sl_engine* dg = lanes[off[g]];
+    for (int i = off[g]; i < off[g + 1]; ++i) {
+      sl_engine* l = lanes[i];
+      l->pos += 1;
+      for (int j = 0; j < l->n_layers; ++j) if (l->layers[j].is_linear) l->parity[j] ^= 1;
+      l->logits_view = dg->logits + (size_t)(i - off[g]) * dg->vocab;
+      l->normed_view = dg->normed + (size_t)(i - off[g]) * H;
+      l->last_ms = d->last_ms;
+    }
   }
   return SL_OK;
 }
