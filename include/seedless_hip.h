@@ -176,8 +176,8 @@ int sl_lane_create(const sl_engine* base, int max_m, int max_seq_len, sl_engine*
  * lanes of one base and one max_seq_len, the lanes go through the layers together as b rows in the scratch of
  * lanes[0]: every projection, expert and lm_head kernel is launched once for all lanes, the recurrence and
  * attention kernels take each row to its lane's caches and position.  From 32 lanes on the batch is stepped as two
- * halves side by side, the second in the scratch and on the stream of its own first lane (lanes[b / 2], which must
- * have max_m >= its half; otherwise one group), queued by a helper thread of the call.  Otherwise the lanes'
+ * halves side by side (lanes of even index, lanes of odd index), the second in the scratch and on the stream of its
+ * own first lane (lanes[1], which must have max_m >= b / 2; otherwise one group), queued by a helper thread of the call.  Otherwise the lanes'
  * single-launch steps run back to back.  After a batched step sl_logits_row(lane, 0) and sl_hidden_rows(lane, 1) give that
  * lane's row.  A device failure poisons every lane of the call. */
 int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t* out);

@@ -917,21 +917,18 @@ bool lanes_batchable(sl_engine** lanes, int b) {
   }
   return true;
 }
-// How a batch of lanes is split into groups that are stepped side by side (sl_lane_step_argmax): [off[g], off[g+1]) are
-// the lanes of group g, its first lane lends scratch rows and stream.  Two groups from 32 lanes on, so that a group
+// Into how many groups a batch of lanes is dealt (lane i to group i % groups) that are stepped side by side
+// (sl_lane_step_argmax); a group's first lane lends scratch rows and stream.  Two groups from 32 lanes on, so that a group
 // keeps the 16 rows that the matrix-core kernels of hybrid mode want.  (Measured at 32 lanes of 1K-16K tokens: one group
 // 9.83 ms per step of exact rows and 8.0 ms hybrid, two groups 9.14 and 7.9, four groups of 8 rows 14.9: the device
 // then spends its time on 2000 launches.)
 constexpr int LANE_GROUPS_MAX = 2, LANE_GROUP_ROWS = 16;
-int lane_groups(sl_engine** lanes, int b, int* off) {
-  int ng = b >= 2 * LANE_GROUP_ROWS ? 2 : 1;
-  for (int g = 0; g <= ng; ++g) off[g] = (int)((long long)b * g / ng);
-  for (int g = 1; g < ng; ++g) {                    // every group's first lane must be able to drive it
-    sl_engine* dg = lanes[off[g]];
-    const int n = off[g + 1] - off[g];
-    if (n > dg->max_m || !dg->has_head || dg->max_seq != lanes[0]->max_seq) { ng = 1; off[1] = b; break; }
-  }
-  return ng;
+int lane_groups(sl_engine** lanes, int b) {
+  if (b < 2 * LANE_GROUP_ROWS) return 1;
+  // the second group's first lane (lanes[1]) must be able to drive its half
+  const sl_engine* d1 = lanes[1];
+  if (b / 2 > d1->max_m || !d1->has_head || d1->max_seq != lanes[0]->max_seq) return 1;
+  return 2;
 }
 // Device table of the lanes' caches, [n_layers][max_m] in the driver; rebuilt when the set of lanes changes.
 int bind_lanes(sl_engine* d, sl_engine** lanes, int b) {
@@ -986,34 +983,37 @@ int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t
   // gates: a third of a step's launches, a few microseconds each and bound by nothing but their start and end) and the
   // ends of its large ones are covered by the other group's kernels.  The dense weights are streamed once per group
   // instead of once per step (5 % of a 32-lane step's bytes); what a lane computes does not change.
-  int off[LANE_GROUPS_MAX + 1];
-  const int ng = lane_groups(lanes, b, off);
+  // (Lane i goes to group i % 2: whatever order the caller keeps its lanes in, neighbours are dealt to both groups,
+  // so a batch sorted by context length does not end up as a short group and a long one.)
+  const int ng = lane_groups(lanes, b);
+  std::vector<sl_engine*> grp[LANE_GROUPS_MAX];
+  std::vector<int32_t> gtok[LANE_GROUPS_MAX];
+  for (int i = 0; i < b; ++i) { grp[i % ng].push_back(lanes[i]); gtok[i % ng].push_back(tokens[i]); }
   int tiles[LANE_GROUPS_MAX];
   for (int g = 0; g < ng; ++g) {
-    sl_engine* dg = lanes[off[g]];
-    const int n = off[g + 1] - off[g];
+    sl_engine* dg = grp[g][0];
     if (g > 0 && d->hybrid != dg->hybrid) { const int r = sl_set_hybrid(dg, d->hybrid ? 1 : 0); if (r) return r; }
     int max_pos = 0;
-    for (int i = off[g]; i < off[g + 1]; ++i) if (lanes[i]->pos > max_pos) max_pos = lanes[i]->pos;
+    for (const sl_engine* l : grp[g]) if (l->pos > max_pos) max_pos = l->pos;
     tiles[g] = (max_pos + 1 + SDPA_TILE - 1) / SDPA_TILE;
-    const int r = bind_lanes(dg, lanes + off[g], n); if (r) return r;
+    const int r = bind_lanes(dg, grp[g].data(), (int)grp[g].size()); if (r) return r;
   }
   // work queued on the other lanes' own streams (none after a completed call) must not overlap this step
   for (int i = 1; i < b; ++i) SL_TRY(lanes[i], hipStreamSynchronize(lanes[i]->stream));
   SL_TRY(d, hipEventRecord(d->ev0, d->stream));
   for (int g = 0; g < ng; ++g) {
-    sl_engine* dg = lanes[off[g]];
-    const int n = off[g + 1] - off[g];
-    const int r = to_device(dg, dg->tok_in, tokens + off[g], (size_t)n * 4); if (r) return r;
+    sl_engine* dg = grp[g][0];
+    const int n = (int)grp[g].size();
+    const int r = to_device(dg, dg->tok_in, gtok[g].data(), (size_t)n * 4); if (r) return r;
     if (g > 0) SL_TRY(dg, hipStreamWaitEvent(dg->stream, d->ev0, 0));      // (the step's time is measured on the first group's stream)
     hipLaunchKernelGGL(k_embed, dim3(H / 256, n), dim3(256), 0, dg->stream, dg->tok_in, dg->embed.w, dg->embed.sb, dg->hA);
   }
-  // (a host thread per further group: one thread queues some 500 launches of a step in about 3.5 ms, which would bound
-  // a step of two groups from below)
+  // (a host thread per further group: queueing a group's 500 launches takes 1.4 ms of host time, so both sequences
+  // are on the device early in the step)
   hipError_t queued[LANE_GROUPS_MAX];
   auto queue_group = [&](int g) {
-    sl_engine* dg = lanes[off[g]];
-    const int n = off[g + 1] - off[g];
+    sl_engine* dg = grp[g][0];
+    const int n = (int)grp[g].size();
     if (g > 0) { (void)hipSetDevice(dg->device); (void)hipGetLastError(); }
     launch_layers(dg, n, dg->lane_tab, tiles[g]);
     HiddenArgs ha{dg->hA, dg->moe_out, dg->final_norm, dg->hB, dg->normed};
@@ -1029,38 +1029,38 @@ int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t
   }
   for (int g = 1; g < ng; ++g)
     if (!ok(d, queued[g], "stepArgmaxBatch (second group)")) {
-      for (int h = 0; h < ng; ++h) (void)hipStreamSynchronize(lanes[off[h]]->stream);
+      for (int h = 0; h < ng; ++h) (void)hipStreamSynchronize(grp[h][0]->stream);
       for (int i = 1; i < b; ++i) if (lanes[i]->fault.empty()) lanes[i]->fault = d->fault;
       return SL_ERR_DEVICE;
     }
   for (int g = 1; g < ng; ++g) {                         // the first group's stream ends the step: it waits for the others
-    sl_engine* dg = lanes[off[g]];
+    sl_engine* dg = grp[g][0];
     SL_TRY(dg, hipEventRecord(dg->ev1, dg->stream));
     SL_TRY(d, hipStreamWaitEvent(d->stream, dg->ev1, 0));
   }
   SL_TRY(d, hipEventRecord(d->ev1, d->stream));
   int r = SL_OK;
   for (int g = 0; g < ng && !r; ++g) {
-    sl_engine* dg = lanes[off[g]];
-    r = read_back(dg, out + off[g], dg->tok_out, (size_t)(off[g + 1] - off[g]) * 4, "stepArgmaxBatch");
+    sl_engine* dg = grp[g][0];
+    r = read_back(dg, gtok[g].data(), dg->tok_out, grp[g].size() * 4, "stepArgmaxBatch");
     if (r && d->fault.empty()) d->fault = dg->fault;
   }
   if (r) {   // the lanes' caches were written by the failed step: all of them are unusable
-    for (int g = 1; g < ng; ++g) (void)hipStreamSynchronize(lanes[off[g]]->stream);
+    for (int g = 1; g < ng; ++g) (void)hipStreamSynchronize(grp[g][0]->stream);
     for (int i = 1; i < b; ++i) if (lanes[i]->fault.empty()) lanes[i]->fault = d->fault;
     return r;
   }
   time_end(d);
-  for (int g = 0; g < ng; ++g) {
-    sl_engine* dg = lanes[off[g]];
-    for (int i = off[g]; i < off[g + 1]; ++i) {
-      sl_engine* l = lanes[i];
-      l->pos += 1;
-      for (int j = 0; j < l->n_layers; ++j) if (l->layers[j].is_linear) l->parity[j] ^= 1;
-      l->logits_view = dg->logits + (size_t)(i - off[g]) * dg->vocab;
-      l->normed_view = dg->normed + (size_t)(i - off[g]) * H;
-      l->last_ms = d->last_ms;
-    }
+  for (int i = 0; i < b; ++i) {
+    sl_engine* l = lanes[i];
+    sl_engine* dg = grp[i % ng][0];
+    const int row = i / ng;
+    out[i] = gtok[i % ng][row];
+    l->pos += 1;
+    for (int j = 0; j < l->n_layers; ++j) if (l->layers[j].is_linear) l->parity[j] ^= 1;
+    l->logits_view = dg->logits + (size_t)row * dg->vocab;
+    l->normed_view = dg->normed + (size_t)row * H;
+    l->last_ms = d->last_ms;
   }
   return SL_OK;
 }
