@@ -131,7 +131,7 @@ def block_benchmarks(eng, cfg, np, torch):
         out["roofline_us"] = nbytes / HBM_PEAK_GBS / 1e3
         return out
 
-    rep = {"method": f"block entry points, kernel-per-stage sequence, batch 1, HIP events, median of {REPS - DROP} calls"}
+    rep = {"method": f"block entry points (one launch per block: the step kernel's stages for that block), batch 1, HIP events, median of {REPS - DROP} calls"}
     lane = eng.new_lane(max_m=1, max_seq_len=64)
     rep["moe_block"] = timed(lane, lambda e, li, x: e.moe_block_rows(li, x), list(range(cfg.n_layers)), moe_b)
     if lin:

@@ -237,7 +237,9 @@ int sl_read_route(sl_engine* e, int layer, int m, int32_t* inds, uint16_t* score
  * workloads: fusedMoEBlockRows (SFV:1986), fusedGdnLayerRows (SFV:3065), fusedAttnLayerRows
  * (SFV:2460).  x is the already-normed input [m, 2048]; out is the block output before the
  * residual add.  They run on layer `layer` of the engine and advance only that layer's caches
- * (an attention block call advances the engine position by m). */
+ * (an attention block call advances the engine position by m).  A single row (m = 1) takes one launch: the
+ * stages of the single-launch step for that block alone (unless sl_set_persistent(e, 0)); more rows take the
+ * kernel-per-stage sequence.  Same bits either way. */
 int sl_moe_block_rows(sl_engine* e, int layer, const uint16_t* x_f16, int m, uint16_t* out_f16);
 int sl_gdn_layer_rows(sl_engine* e, int layer, const uint16_t* x_f16, int m, uint16_t* out_f16);
 int sl_attn_layer_rows(sl_engine* e, int layer, const uint16_t* x_f16, int m, uint16_t* out_f16);

@@ -160,6 +160,7 @@ struct sl_engine {
   double head_ms_sum = 0.0;
   long head_launches = 0;
   bool use_persistent = true;
+  bool last_block_flow = false;    // the last block entry point ran as a single launch: its intermediate rows are in the exchange buffers
   bool hybrid = false;             // prefill chunks: dense projections and grouped experts on the matrix cores (not bit-identical to the GEMV order)
   // scratch of the hybrid MoE (allocated when hybrid is first enabled): routed gate / up / down results per pair,
   // shared gate / up / down rows, pairs listed per expert
@@ -511,6 +512,7 @@ void launch_attn_mixer(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha, c
 // With `lane_tab` the M rows are one token each of M lanes (caches and positions from the table, the longest
 // lane needing `lane_tiles` key tiles); without, M consecutive rows of this engine's own sequence.
 void launch_layer(sl_engine* e, int li, int M, const LaneRef* lane_tab = nullptr, int lane_tiles = 0) {
+  e->last_block_flow = false;
   LayerDev& L = e->layers[li];
   const LaneRef* lanes = lane_tab ? lane_tab + (size_t)li * e->max_m : nullptr;
   HiddenArgs ha{e->hA, li > 0 ? e->moe_out : nullptr, L.input_ln, e->hB, nullptr};
@@ -573,13 +575,26 @@ constexpr uint32_t FLOW_BASE_LIMIT = 0x7ff00000u;
 bool flow_rebase_needed(uint32_t base, int steps, int n_layers) {
   return (uint64_t)base + (uint64_t)(steps + 1) * (uint64_t)(n_layers + 1) * 8u > (uint64_t)FLOW_BASE_LIMIT;
 }
-void launch_decode(sl_engine* e, int out_off, bool feed, int steps) {
+// Moves the host's mirror of the tag counter on by `steps` step-sized strides, restarting it first where it would wrap.
+void flow_advance_base(sl_engine* e, int steps) {
   if (flow_rebase_needed(e->flow_base, steps, e->n_layers)) {
     for (const auto& b : e->flow_tagged) (void)hipMemsetAsync(b.first, 0, b.second, e->stream);
     (void)hipMemsetAsync(e->dec_bar + 16, 0, 4, e->stream);
     e->flow_base = 0;
   }
   e->flow_base += (uint32_t)steps * (uint32_t)(e->n_layers + 1) * 8u;
+}
+// One block of one layer (mode 0: the mixer, 1: the MoE block) on the row in e->xn, in a single launch of the step
+// kernel's stages; the result is left in the exchange buffer `tagged_out` with the tags of (layer, stage).
+bool block_flow_ready(const sl_engine* e, int m) { return m == 1 && e->dec_grid > 0 && e->use_persistent && e->flow_params; }
+void launch_block_flow(sl_engine* e, int layer, int mode) {
+  e->last_block_flow = true;
+  flow_advance_base(e, 1);
+  auto kern = e->gate8 ? k_block_flow<true> : k_block_flow<false>;
+  hipLaunchKernelGGL(kern, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, layer, mode);
+}
+void launch_decode(sl_engine* e, int out_off, bool feed, int steps) {
+  flow_advance_base(e, steps);
   const bool prof = e->profile_head && e->head_pending < MAX_CHAIN;
   if (prof) (void)hipEventRecord(e->head_ev[2 * e->head_pending], e->stream);
   auto kern = e->gate8 ? (e->stage_clock ? k_decode_flow<true, true> : k_decode_flow<true, false>)
@@ -632,6 +647,7 @@ int alloc_runtime(sl_engine* e);
 }  // namespace
 static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, const char* what, bool abort_word = false);
 static void time_end(sl_engine* e);
+static int read_back_tagged(sl_engine* e, uint16_t* out, const uint32_t* words, uint32_t tag, const char* what);
 
 int sl_create(const sl_model_desc* d, int max_m, int max_seq_len, sl_engine** out) {
   if (!d || !out || max_m < 1 || max_seq_len < 1 || d->n_layers < 1 || !d->layers) return SL_ERR_ARG;
@@ -785,7 +801,7 @@ int alloc_runtime(sl_engine* e) {
   e->st = dalloc<int32_t>(e, 1 + d->n_layers, true);
   if (!e->hA || !e->hB || !e->proj || !e->ycore || !e->mix || !e->xn || !e->xsum || !e->ysum || !e->rlogits || !e->sgate || !e->sh_act || !e->act || !e->hy_lists || !e->hy_counts ||
       !e->moe_out || !e->normed || !e->rows_out || !e->tok_in || !e->tok_out || !e->st) return SL_ERR_DEVICE;
-  if (has_head) {
+  {                                // (also for engines without a head: their block entry points use the single-launch stages)
     int ncu = 0;
     SL_TRY(e, hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, 0));
     if (ncu >= 256 && d->n_layers <= FLOW_MAX_LAYERS) {
@@ -842,6 +858,7 @@ int alloc_runtime(sl_engine* e) {
         F.ttok = tagged_chunks(4);
         F.sdpa_round = SDPA_ROUND;
         F.spin_limit = FLOW_SPIN_LIMIT;
+        F.xin = e->xn;
         if (const char* s = std::getenv("QWISP_SDPA_ROUND")) {      // smaller rounds, for tests of the round loop
           const int v = std::atoi(s);
           if (v >= 1 && v <= SDPA_ROUND) F.sdpa_round = v;
@@ -855,6 +872,8 @@ int alloc_runtime(sl_engine* e) {
         SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
         SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
         SL_TRY(e, hipFuncSetAttribute((const void*)k_decode_flow<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
+        SL_TRY(e, hipFuncSetAttribute((const void*)k_block_flow<false>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
+        SL_TRY(e, hipFuncSetAttribute((const void*)k_block_flow<true>, hipFuncAttributeMaxDynamicSharedMemorySize, DEC_DYN_LDS));
       }
       // every workgroup of the grid must be resident at once: one per compute unit
       int per_cu = 0;
@@ -1198,6 +1217,20 @@ static int read_back(sl_engine* e, void* dst, const void* dev, size_t bytes, con
     }
   }
   std::memcpy(dst, e->pinned, bytes);
+  return SL_OK;
+}
+// The 2048-long result of a single-block launch: halves with their 16-bit tags, checked and stripped here.
+static int read_back_tagged(sl_engine* e, uint16_t* out, const uint32_t* words, uint32_t tag, const char* what) {
+  std::vector<uint32_t> w(H);
+  const int r = read_back(e, w.data(), words, (size_t)H * 4, what, true);
+  if (r) return r;
+  for (int i = 0; i < H; ++i) {
+    if ((w[i] >> 16) != tag) {
+      if (e->fault.empty()) e->fault = std::string(what) + ": single-block launch left an incomplete result";
+      return SL_ERR_DEVICE;
+    }
+    out[i] = (uint16_t)(w[i] & 0xffffu);
+  }
   return SL_OK;
 }
 static void time_end(sl_engine* e) {
@@ -1548,7 +1581,16 @@ int sl_moe_block_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_
   if (!x || !out || layer < 0 || layer >= e->n_layers || m < 1 || m > e->max_m) return SL_ERR_ARG;
   r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
+  if (block_flow_ready(e, m)) {                  // a single row: the stages of the step kernel in one launch, same bits
+    launch_block_flow(e, layer, 1);
+    SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+    const uint32_t tag = flow_tag(e->flow_base - (uint32_t)(e->n_layers + 1) * 8u, layer, FS_C);
+    r = read_back_tagged(e, out, e->flow_host.tmoe, tag, "moeBlockRows"); if (r) return r;
+    time_end(e);
+    return SL_OK;
+  }
   HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
+  e->last_block_flow = false;
   launch_moe(e, e->layers[layer], m, ha);
   SL_TRY(e, hipEventRecord(e->ev1, e->stream));
   r = read_back(e, out, e->moe_out, (size_t)m * H * 2, "moeBlockRows"); if (r) return r;
@@ -1560,10 +1602,18 @@ int sl_gdn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16_
   if (!x || !out || layer < 0 || layer >= e->n_layers || m < 1 || m > e->max_m || !e->layers[layer].is_linear) return SL_ERR_ARG;
   r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
-  HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
-  launch_gdn_mixer(e, e->layers[layer], layer, m, ha, nullptr);
-  SL_TRY(e, hipEventRecord(e->ev1, e->stream));
-  r = read_back(e, out, e->mix, (size_t)m * H * 2, "gdnLayerRows"); if (r) return r;
+  if (block_flow_ready(e, m)) {
+    launch_block_flow(e, layer, 0);
+    SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+    const uint32_t tag = flow_tag(e->flow_base - (uint32_t)(e->n_layers + 1) * 8u, layer, FS_OUT);
+    r = read_back_tagged(e, out, e->flow_host.tmix, tag, "gdnLayerRows"); if (r) return r;
+  } else {
+    HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
+    e->last_block_flow = false;
+    launch_gdn_mixer(e, e->layers[layer], layer, m, ha, nullptr);
+    SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+    r = read_back(e, out, e->mix, (size_t)m * H * 2, "gdnLayerRows"); if (r) return r;
+  }
   time_end(e);
   e->parity[layer] ^= 1;
   return push_state(e);
@@ -1574,10 +1624,18 @@ int sl_attn_layer_rows(sl_engine* e, int layer, const uint16_t* x, int m, uint16
   r = check_rows(e, m); if (r) return r;
   r = to_device(e, e->xn, x, (size_t)m * H * 2); if (r) return r;
   SL_TRY(e, hipEventRecord(e->ev0, e->stream));
-  HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
-  launch_attn_mixer(e, e->layers[layer], m, ha, nullptr, 0);
-  SL_TRY(e, hipEventRecord(e->ev1, e->stream));
-  r = read_back(e, out, e->mix, (size_t)m * H * 2, "attnLayerRows"); if (r) return r;
+  if (block_flow_ready(e, m)) {
+    launch_block_flow(e, layer, 0);
+    SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+    const uint32_t tag = flow_tag(e->flow_base - (uint32_t)(e->n_layers + 1) * 8u, layer, FS_OUT);
+    r = read_back_tagged(e, out, e->flow_host.tmix, tag, "attnLayerRows"); if (r) return r;
+  } else {
+    HiddenArgs ha{e->xn, nullptr, nullptr, nullptr, nullptr};
+    e->last_block_flow = false;
+    launch_attn_mixer(e, e->layers[layer], m, ha, nullptr, 0);
+    SL_TRY(e, hipEventRecord(e->ev1, e->stream));
+    r = read_back(e, out, e->mix, (size_t)m * H * 2, "attnLayerRows"); if (r) return r;
+  }
   time_end(e);
   e->pos += m;
   return push_state(e);
@@ -1600,6 +1658,17 @@ int sl_debug_scratch(sl_engine* e, int which, uint16_t* out, size_t count) {
     default: return SL_ERR_ARG;
   }
   if (!src || !out) return SL_ERR_ARG;
+  if (e->last_block_flow) {
+    // a single-launch block keeps its rows in the step kernel's exchange buffers (halves with tags): router logits,
+    // mixer output and MoE output can be read from there, the other scratch rows were not written
+    const uint32_t* words = which == 7 ? e->flow_host.trlog : (which == 3 ? e->flow_host.tmix : (which == 8 ? e->flow_host.tmoe : nullptr));
+    const size_t cap = which == 7 ? 256 : (size_t)H;
+    if (!words || count > cap) return SL_ERR_UNSUPPORTED;
+    std::vector<uint32_t> w(count);
+    r = copy_sync(e, w.data(), words, count * 4, hipMemcpyDeviceToHost); if (r) return r;
+    for (size_t i = 0; i < count; ++i) out[i] = (uint16_t)(w[i] & 0xffffu);
+    return SL_OK;
+  }
   return copy_sync(e, out, src, count * 2, hipMemcpyDeviceToHost);
 }
 

@@ -35,6 +35,7 @@ struct FlowP {
   uint4 *ttok;          // {token, token, tag, tag}: the token a step of a multi-step launch hands to the next [1]
   int sdpa_round;       // long contexts: (tile, kv head) units a workgroup scores before it turns to their values
   unsigned spin_limit;  // polling rounds after which a workgroup gives up and raises the abort word (FLOW_SPIN_LIMIT; tests: 0)
+  const uint16_t* xin;  // single-block launches (k_block_flow): the block's input row, plain halves [2048]
 };
 
 // Parameters live in LDS for the whole launch.  Reading them there (ds_read + readfirstlane) does not
@@ -204,6 +205,17 @@ SL_DEV void flow_prologue(float& h0, float& h1, bool has_r, float r0, float r1, 
   lds_barrier();
 }
 
+// The same hand-over to the dot products for a row that is used as it is (the input of a single block: no residual,
+// no norm): packed pairs and share sums into LDS.
+SL_DEV void flow_plain_x(const uint16_t* x) {
+  const int tid = fresh_v(threadIdx.x);
+  const uint32_t w = *reinterpret_cast<const uint32_t*>(x + 2 * tid);
+  g_L.xs[(tid & 15) * 64 + (tid >> 4)] = w;
+  const float s = tree_sum<16>(lo_h(w) + hi_h(w));
+  if ((tid & 15) == 0) g_L.sxs[tid >> 4] = s;
+  lds_barrier();
+}
+
 // Stores of a wave are acknowledged in order with its loads, so a wave that has just published results cannot
 // finish a poll before the write has travelled to memory and back.  All tagged results of a stage are therefore
 // gathered in LDS and written by one wave, wave 15 (full 64-byte lines), so that only that wave's polls of the next
@@ -342,7 +354,7 @@ SL_DEV void flow_request_conv(const LayerP& Y, int li) {
       __builtin_amdgcn_global_load_lds((glb_ptr)(hin + k * SL_CONV_DIM + (ch & ~1)), (lds_ptr)(lds + CVH_OFF + (k * 5 + wave) * 256), 4, 0, 0);
   }
 }
-template <bool ST>
+template <bool ST, bool PLAIN = false>
 SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base, float& h0, float& h1, int step) {
   FLOW_IDS;
   fstamp<ST>(li, FS_IN, 0, tid == 0);
@@ -358,7 +370,9 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.input_ln) + 2 * tid);
   float r0 = 0.0f, r1 = 0.0f;
-  if (li == 0) {
+  if constexpr (PLAIN) {
+    // (a single block: its input row is given)
+  } else if (li == 0) {
     // the token's embedding row, dequantised in half arithmetic: half(half(s * q) + b) (embed_rows_q4,
     // SeedlessFusedVerify.swift:556-569); thread t owns elements 2t, 2t+1
     if (step > 0) {
@@ -393,7 +407,8 @@ SL_DEV bool flow_in(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t b
   sbd = 0u;
   if (lin) flow_request_conv(Y, li);             // behind the poll, to arrive while this stage computes
   const uint32_t tin = flow_tag(base, li, FS_IN);
-  flow_prologue(h0, h1, li > 0, r0, r1, lnw, nullptr);
+  if constexpr (PLAIN) { (void)lnw; flow_plain_x(uni(F.xin)); }
+  else flow_prologue(h0, h1, li > 0, r0, r1, lnw, nullptr);
   fstamp<ST>(li, FS_IN, 2, tid == 0);
   uint32_t x[16]; float sx;
   lds_get_x(0, lane, x, sx);
@@ -1478,7 +1493,7 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
 // ---- MoE stage A -------------------------------------------------------------------------------------
 // GATE8: the router and shared-gate rows are 8-bit affine rows instead of fp16 (a compile-time variant, so that
 // the fp16 configuration carries none of its registers or branches).
-template <bool GATE8, bool ST>
+template <bool GATE8, bool ST, bool PLAIN = false>
 SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, float& h0, float& h1) {
   FLOW_IDS;
   fstamp<ST>(li, FS_A, 0, tid == 0);
@@ -1506,10 +1521,15 @@ SL_DEV bool flow_moe_a(const FlowP& F, const LayerP& Y, int li, uint32_t base, f
     dsb = reinterpret_cast<const uint32_t*>(uni(Y.sgate_w))[(size_t)gd * 32 + (lane >> 1)];
   }
   const uint32_t lnw = *reinterpret_cast<const uint32_t*>(uni(Y.post_ln) + 2 * tid);
-  float r0, r1;
-  if (!poll_vec2048<ST>(P, uni(F.tmix), flow_tag(base, li, FS_OUT), r0, r1, li, FS_A)) return false;
   const uint32_t ta = flow_tag(base, li, FS_A);
-  flow_prologue(h0, h1, true, r0, r1, lnw, nullptr);
+  if constexpr (PLAIN) {
+    (void)lnw;
+    flow_plain_x(uni(F.xin));
+  } else {
+    float r0, r1;
+    if (!poll_vec2048<ST>(P, uni(F.tmix), flow_tag(base, li, FS_OUT), r0, r1, li, FS_A)) return false;
+    flow_prologue(h0, h1, true, r0, r1, lnw, nullptr);
+  }
   fstamp<ST>(li, FS_A, 2, tid == 0);
   if (is_dense) {
     uint32_t xp[16]; float sx;
@@ -1953,6 +1973,64 @@ flow_exit:
     uint32_t* dst = uni(P.tstamp) + (size_t)blockIdx.x * STAMP_WORDS;
     for (int i = threadIdx.x; i < STAMP_WORDS; i += DEC_THREADS) dst[i] = g_stamps[i];
   }
+}
+
+// ---- a single block in one launch ---------------------------------------------------------------------------------
+// One layer's mixer (mode 0: in-projection, recurrence or attention, out-projection) or its MoE block (mode 1: router,
+// shared and routed experts, combine) on the row F.xin, taken as it is (no residual, no norm): the stages of the step
+// kernel, handed over the same way, so the arithmetic is that of a decode step.  The result stays in its exchange
+// buffer (tmix / tmoe: halves with the tags of this launch), from where the host takes it; position, parities and caches
+// are read as they stand and the host moves them on.
+template <bool GATE8>
+__global__ __launch_bounds__(DEC_THREADS) void k_block_flow(const FlowP* __restrict__ Fp, int li, int mode) {
+  {
+    const int tid = threadIdx.x;
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(Fp);
+    uint32_t* dst = reinterpret_cast<uint32_t*>(&g_K.F);
+    for (int i = tid; i < (int)(sizeof(FlowP) / 4); i += DEC_THREADS) dst[i] = src[i];
+    const int nl = Fp->d.n_layers;
+    const uint32_t* lsrc = reinterpret_cast<const uint32_t*>(Fp->d.layers);
+    uint32_t* ldst = reinterpret_cast<uint32_t*>(g_K.layers);
+    for (int i = tid; i < nl * (int)(sizeof(LayerP) / 4); i += DEC_THREADS) ldst[i] = lsrc[i];
+    if (tid < 64) {
+      const int bit = (tid < nl) ? (Fp->d.st[1 + tid] & 1) : 0;
+      const unsigned long long m = __ballot(bit);
+      const unsigned long long lm = __ballot((tid < nl) ? (Fp->d.layers[tid].is_linear != 0) : 0);
+      if (tid == 0) { g_K.parity = m; g_K.linmask = lm; g_K.pos = Fp->d.st[0]; g_K.base = ld_co32(Fp->d.bar + 16); g_K.tok = 0; }
+      if (tid < 4) g_L.pf[tid] = 0;
+    }
+    __syncthreads();
+  }
+  const FlowP& F = g_K.F;
+  const DecodeP& P = F.d;
+  const LayerP& Y = g_K.layers[li];
+  const uint32_t base = uni(g_K.base);
+  const int pos = uni(g_K.pos);
+  float h0 = 0.0f, h1 = 0.0f;
+  bool ok = true;
+  if (mode == 0) {
+    flow_request_in(Y);
+    ok = flow_in<false, true>(F, Y, li, pos, base, h0, h1, 0);
+    GdnHist gh = {0u, 0u};
+    if (ok) {
+      if (uni(Y.is_linear)) {
+        ok = flow_gdn<false>(F, Y, li, base, gh);
+        if (ok) ok = flow_out<false>(F, Y, li, 0, base, gh);
+      } else {
+        if (((pos + SDPA_TILE) / SDPA_TILE) * SL_ATT_KV * 4 <= (int)gridDim.x) ok = flow_sdpa4<false>(F, Y, li, pos, base);
+        else ok = flow_sdpa<false>(F, Y, li, pos, base);
+        if (ok) ok = flow_out<false>(F, Y, li, (pos + SDPA_TILE) / SDPA_TILE, base, gh);
+      }
+    }
+  } else {
+    ok = flow_moe_a<GATE8, false, true>(F, Y, li, base, h0, h1);
+    if (ok) ok = flow_moe_b<false>(F, Y, li, base);
+    if (ok) ok = flow_moe_c<false>(F, Y, li, base);
+  }
+  wr_wait();
+  // the next launch's tags.  (Every workgroup has read `base` by now: workgroup 0's last stage consumed results to
+  // which, directly or through the stages before, every workgroup of the grid contributed.)
+  if (blockIdx.x == 0 && threadIdx.x == 0) st_co32(uni(P.bar) + 16, base + (uint32_t)(uni(P.n_layers) + 1) * 8u);
 }
 
 }  // namespace sl
