@@ -591,7 +591,8 @@ void launch_block_flow(sl_engine* e, int layer, int mode) {
   e->last_block_flow = true;
   flow_advance_base(e, 1);
   auto kern = e->gate8 ? k_block_flow<true> : k_block_flow<false>;
-  hipLaunchKernelGGL(kern, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, layer, mode);
+  hipLaunchKernelGGL(kern, dim3(e->dec_grid), dim3(DEC_THREADS), DEC_DYN_LDS, e->stream, e->flow_params, e->flow_host.d.layers,
+                     (const int32_t*)e->st, (const unsigned*)e->dec_bar, e->n_layers, layer, mode);
 }
 void launch_decode(sl_engine* e, int out_off, bool feed, int steps) {
   flow_advance_base(e, steps);

@@ -1982,21 +1982,22 @@ flow_exit:
 // buffer (tmix / tmoe: halves with the tags of this launch), from where the host takes it; position, parities and caches
 // are read as they stand and the host moves them on.
 template <bool GATE8>
-__global__ __launch_bounds__(DEC_THREADS) void k_block_flow(const FlowP* __restrict__ Fp, int li, int mode) {
+__global__ __launch_bounds__(DEC_THREADS) void k_block_flow(const FlowP* __restrict__ Fp, const LayerP* __restrict__ layers,
+                                                            const int32_t* __restrict__ st, const unsigned* bar, int nl, int li, int mode) {
   {
+    // (the layer's parameters, the position and the tag counter come through pointers passed as arguments, so their
+    // loads leave together with those of the parameter block instead of after it; only layer li is copied)
     const int tid = threadIdx.x;
     const uint32_t* src = reinterpret_cast<const uint32_t*>(Fp);
     uint32_t* dst = reinterpret_cast<uint32_t*>(&g_K.F);
     for (int i = tid; i < (int)(sizeof(FlowP) / 4); i += DEC_THREADS) dst[i] = src[i];
-    const int nl = Fp->d.n_layers;
-    const uint32_t* lsrc = reinterpret_cast<const uint32_t*>(Fp->d.layers);
-    uint32_t* ldst = reinterpret_cast<uint32_t*>(g_K.layers);
-    for (int i = tid; i < nl * (int)(sizeof(LayerP) / 4); i += DEC_THREADS) ldst[i] = lsrc[i];
+    const uint32_t* lsrc = reinterpret_cast<const uint32_t*>(layers + li);
+    uint32_t* ldst = reinterpret_cast<uint32_t*>(g_K.layers + li);
+    for (int i = tid; i < (int)(sizeof(LayerP) / 4); i += DEC_THREADS) ldst[i] = lsrc[i];
     if (tid < 64) {
-      const int bit = (tid < nl) ? (Fp->d.st[1 + tid] & 1) : 0;
+      const int bit = (tid < nl) ? (st[1 + tid] & 1) : 0;
       const unsigned long long m = __ballot(bit);
-      const unsigned long long lm = __ballot((tid < nl) ? (Fp->d.layers[tid].is_linear != 0) : 0);
-      if (tid == 0) { g_K.parity = m; g_K.linmask = lm; g_K.pos = Fp->d.st[0]; g_K.base = ld_co32(Fp->d.bar + 16); g_K.tok = 0; }
+      if (tid == 0) { g_K.parity = m; g_K.linmask = 0ull; g_K.pos = st[0]; g_K.base = ld_co32(bar + 16); g_K.tok = 0; }
       if (tid < 4) g_L.pf[tid] = 0;
     }
     __syncthreads();
