@@ -457,6 +457,61 @@ def test_gdn_layer_sequence(env):
     assert np.abs(gs).max() > 0
 
 
+def test_single_row_blocks_in_one_launch_equal_the_kernel_per_stage_sequence(env):
+    """A single row through a block entry point takes one launch of the step kernel's stages for that block; with
+    sl_set_persistent(0) the same call takes the kernel-per-stage sequence.  Outputs, routing and caches carry the same
+    bits: a MoE block with all 256 experts, a GDN layer over a run of steps, an attention layer at contexts on both sides
+    of the step kernel's change of tile units (2048 tokens)."""
+    Engine, orc = env["Engine"], env["orc"]
+    # MoE block
+    cfg = ModelConfig(n_layers=1, n_experts=256, vocab=0, layer_types=("gdn",))
+    dev, _ = device_and_host_model(cfg)
+    one, seq = Engine(cfg, dev, max_m=2, max_seq_len=16), Engine(cfg, dev, max_m=2, max_seq_len=16)
+    assert seq.set_persistent(False)
+    for call in range(3):
+        x = xrows(1, 5100 + call)
+        a, b = one.moe_block_rows(0, x), seq.moe_block_rows(0, x)
+        assert a is not None and b is not None, (one.gpu_fault, seq.gpu_fault)
+        assert same_bits(a, b), (call, first_diff(a, b))
+        (ai, as_), (bi, bs) = one.read_route(0, 1), seq.read_route(0, 1)
+        assert np.array_equal(ai, bi) and same_bits(as_, bs)
+    one.close(); seq.close()
+    # GDN layer: the recurrent state and the conv history move on from call to call
+    cfg = ModelConfig(n_layers=1, n_experts=8, vocab=0, layer_types=("gdn",))
+    dev, _ = device_and_host_model(cfg)
+    one, seq = Engine(cfg, dev, max_m=2, max_seq_len=16), Engine(cfg, dev, max_m=2, max_seq_len=16)
+    assert seq.set_persistent(False)
+    state0 = orc.synth_f32((abi.GDN_HV, abi.GDN_D, abi.GDN_D), 5110, 0.0, 0.1)
+    hist0 = np.zeros((abi.CONV_K - 1, abi.CONV_DIM), np.float16)
+    assert one.load_layer_cache(0, hist0, state0) and seq.load_layer_cache(0, hist0, state0)
+    for call, m in enumerate([1, 1, 1, 2, 1, 1]):            # (the two-row call takes the sequence on both engines)
+        x = xrows(m, 5120 + call)
+        a, b = one.gdn_layer_rows(0, x), seq.gdn_layer_rows(0, x)
+        assert a is not None and b is not None, (one.gpu_fault, seq.gpu_fault)
+        assert same_bits(a, b), (call, first_diff(a, b))
+    for u, v in zip(one.read_layer_cache(0), seq.read_layer_cache(0)):
+        assert same_bits(u, v), first_diff(u, v)
+    one.close(); seq.close()
+    # attention layer
+    cfg = ModelConfig(n_layers=1, n_experts=8, vocab=0, layer_types=("attn",))
+    dev, _ = device_and_host_model(cfg)
+    for S in (130, 2300):
+        one, seq = Engine(cfg, dev, max_m=2, max_seq_len=S + 8), Engine(cfg, dev, max_m=2, max_seq_len=S + 8)
+        assert seq.set_persistent(False)
+        k = orc.synth_f16((abi.ATT_KV, S, abi.ATT_D), 5130, 0.0, 1.0)
+        v = orc.synth_f16((abi.ATT_KV, S, abi.ATT_D), 5131, 0.0, 1.0)
+        assert one.load_layer_cache(0, k, v) and seq.load_layer_cache(0, k, v)
+        for call in range(3):
+            x = xrows(1, 5140 + call)
+            a, b = one.attn_layer_rows(0, x), seq.attn_layer_rows(0, x)
+            assert a is not None and b is not None, (one.gpu_fault, seq.gpu_fault)
+            assert same_bits(a, b), (S, call, first_diff(a, b))
+        assert one.position == seq.position == S + 3
+        for u, w in zip(one.read_layer_cache(0), seq.read_layer_cache(0)):
+            assert same_bits(u, w)
+        one.close(); seq.close()
+
+
 # ---- benchmark configuration 2: one attention layer over a pre-filled KV arena ------------------------------
 @pytest.mark.parametrize("S", [0, 1, 63, 64, 200, 4096])
 def test_attention_layer_decode(env, S):
@@ -748,6 +803,41 @@ def test_lanes_share_weights_and_equal_solo(env, small_model):
     assert type(base).lane_step_argmax([lanes[0], lanes[0]], [1, 2]) is None      # the same lane twice
     for lane in lanes:
         lane.close()
+
+
+def test_lane_batch_in_two_groups_equals_one_group(env, small_model):
+    """From 32 lanes on a batch is stepped as two groups side by side (lanes of even and of odd index), the second in
+    the scratch rows of lanes[1]; when that lane has too few scratch rows the batch stays one group.  Tokens, logits
+    and caches are the same either way (and the same as solo steps, which the other lane tests hold them to)."""
+    cfg, dev, host = small_model
+    B = 32
+    base = env["Engine"](cfg, dev, max_m=B, max_seq_len=96)
+    def make(second_rows):
+        return [base.new_lane(max_m=(second_rows if i == 1 else B), max_seq_len=96) for i in range(B)]
+    two, one = make(B), make(8)                              # 8 scratch rows < 16: one group
+    rng = np.random.default_rng(5200)
+    cur = []
+    for i in range(B):
+        pr = rng.integers(0, cfg.vocab, 1 + (23 * i) % 70).astype(np.int32)
+        ta = tb = None
+        for j in range(0, len(pr), 8):
+            ta, tb = two[i].step_argmax(pr[j:j + 8]), one[i].step_argmax(pr[j:j + 8])
+        assert ta.tolist() == tb.tolist()
+        cur.append(int(ta[-1]))
+    for step in range(3):
+        a, b = type(base).lane_step_argmax(two, cur), type(base).lane_step_argmax(one, cur)
+        assert a is not None and b is not None, ([l.gpu_fault for l in two], [l.gpu_fault for l in one])
+        assert a.tolist() == b.tolist(), step
+        cur = a.tolist()
+    for i in range(B):
+        assert same_bits(two[i].logits_row(0), one[i].logits_row(0)), i
+        assert two[i].position == one[i].position
+        for li in range(cfg.n_layers):
+            for x, y in zip(two[i].read_layer_cache(li), one[i].read_layer_cache(li)):
+                assert same_bits(x, y), (i, li)
+    for lane in two + one:
+        lane.close()
+    base.close()
 
 
 def test_spec_loop_stream_equals_greedy_stream(env):
