@@ -337,7 +337,7 @@ def main():
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         lanes_report = {"lanes": B, "ms_per_step": dt * 1e3 / n_lane_steps, "tok_s_aggregate": B * n_lane_steps / dt,
-                        "contexts": f"{min(ctxs)}-{max(ctxs)} tokens, mean {sum(ctxs) // B}", "fill_s": t_fill, "path": "rows of the kernel-per-stage path, one launch sequence for all lanes"}
+                        "contexts": f"{min(ctxs)}-{max(ctxs)} tokens, mean {sum(ctxs) // B}", "fill_s": t_fill, "path": "rows of the kernel-per-stage path; from 32 lanes on two launch sequences side by side, 16 lanes each"}
         lane_b = lane_step_bytes(cfg, ctxs)             # the step's own byte roofline (shared weights once, touched experts once)
         lanes_report["bytes_per_step"] = lane_b
         lanes_report["frac_of_peak"] = lane_b / (dt / n_lane_steps) / 1e9 / HBM_PEAK_GBS

@@ -13,6 +13,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <system_error>
 #include <thread>
 #include <vector>
 
@@ -1043,8 +1044,14 @@ int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t
   };
   {
     std::vector<std::thread> helpers;
-    for (int g = 1; g < ng; ++g) helpers.emplace_back(queue_group, g);
+    int started = 1;
+    try {
+      for (int g = 1; g < ng; ++g) { helpers.emplace_back(queue_group, g); started = g + 1; }
+    } catch (const std::system_error&) {
+      // no thread to be had: the groups not handed to one are queued from this thread, after its own
+    }
     queue_group(0);
+    for (int g = started; g < ng; ++g) queue_group(g);
     for (auto& t : helpers) t.join();
   }
   for (int g = 1; g < ng; ++g)
