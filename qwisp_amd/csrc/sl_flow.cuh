@@ -604,6 +604,11 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
 #define SL_MERGE_WGS 32
 #endif
 constexpr int FLOW_MERGE_WGS = SL_MERGE_WGS;     // workgroups that merge the attention tiles: two or four per query head
+// Contexts of 33 to 1024 key tiles (2K to 64K tokens): every workgroup takes tile units, and afterwards every workgroup
+// merges a sixteenth of a query head (flow_merge_wide).  Below, the tile units are split over the query heads and the
+// merging workgroups poll everything in one round trip; above, the parked partial sums no longer fit the LDS.
+constexpr int WIDE_MERGE_MAX_TILES = 1024;
+SL_DEV bool sdpa_wide_merge(int nt) { return nt > 32 && nt <= WIDE_MERGE_MAX_TILES; }
 template <bool ST>
 SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base) {
   FLOW_IDS;
@@ -615,7 +620,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag32(base, li, FS_CORE);
   // The workgroups that merge the tiles take no units: they start polling at once, see every tile's maximum after
   // the first pass below and add up the tiles' value sums while the second pass is still producing them.
-  const int GU = G > 2 * FLOW_MERGE_WGS ? G - FLOW_MERGE_WGS : G;
+  const int GU = (G > 2 * FLOW_MERGE_WGS && !sdpa_wide_merge(nt)) ? G - FLOW_MERGE_WGS : G;
   if (wg >= GU) return true;
   const int U = nt * SL_ATT_KV, RND = uni(F.sdpa_round);
   float* const ps = reinterpret_cast<float*>(g_vt + SDPA_TILE * 256);      // [SDPA_ROUND][8 heads][64 keys]
@@ -1025,6 +1030,110 @@ SL_DEV void store_hist(const LayerP& Y, int li, const GdnHist& gh) {
   }
 }
 
+// ---- attention merge on all workgroups ------------------------------------------------------------------------
+// Workgroup n merges dims 16 (n % 16) .. + 15 of query head n / 16: eight 16-byte chunks per key tile.  What bounds a
+// merge on few workgroups is how fast those can pull the published chunks (16 MB per layer at 32K tokens through 32
+// compute units); spread over the whole grid every thread fetches at most eight chunks, all in one round trip, parks
+// them in LDS, and the sums are formed from LDS.  The order is the canonical one: per block of 64 tiles a chain from
+// zero in tile order (one lane per (block, chunk); the tiles' sums likewise, one lane per block), the blocks' chains
+// added in block order.
+template <bool ST>
+SL_DEV bool flow_merge_wide(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t base) {
+  FLOW_IDS;
+  const DecodeP& P = F.d;
+  const float NEG = -__int_as_float(0x7f800000);
+  const uint32_t tin = flow_tag(base, li, FS_IN), tmerge = flow_tag(base, li, FS_MERGE), tcore32 = flow_tag32(base, li, FS_CORE);
+  const int h = wg >> 4, c0 = 8 * (wg & 15), slot0 = h * uni(P.max_tiles);
+  const rsrc_t rml = co_rsrc(uni(F.tml)), rpo = co_rsrc(uni(F.tpo)), rp = co_rsrc(uni(F.tproj));
+  unsigned char* const dyn = reinterpret_cast<unsigned char*>(g_vt);
+  float* const ll = reinterpret_cast<float*>(dyn);                       // [1024] tile sums
+  float* const fl = reinterpret_cast<float*>(dyn + 4096);                // [1024] tile scales exp(max - global max)
+  uint2* const park = reinterpret_cast<uint2*>(dyn + 12288);             // [tile][8 chunks] {o0, o1}
+  static_assert(12288 + WIDE_MERGE_MAX_TILES * 8 * 8 <= DEC_DYN_LDS && WIDE_MERGE_MAX_TILES <= DEC_THREADS, "parked sums fit; a thread per tile");
+  lds_barrier();                                                         // the tile units are through with the dynamic LDS
+  // every tile's {max, sum} (thread t: tile t) and, on lanes 0..15 of wave 0, the slice's output gate
+  float m = NEG;
+  uint32_t gatew = 0;
+  {
+    const bool mine = tid < nt, gmine = tid < 16;
+    bool mdone = !mine, gdone = !gmine;
+    uint4 q = make_uint4(0u, 0u, 0u, 0u);
+    if (!flow_poll(wave * 64 < nt, [&]() {
+          const bool want_m = !mdone, want_g = !gdone;
+          uint32_t g = 0;
+          if (want_m) q = ldw4(rml, (slot0 + tid) * 4);
+          if (want_g) g = ldw1(rp, h * 512 + 256 + 2 * c0 + tid);
+          if (want_m) mdone = q.z == tcore32 && q.w == tcore32;
+          if (want_g) { gdone = tag_ok(g, tin); gatew = g; }
+          return mdone && gdone;
+        }, uni(P.bar) + 32, 25u)) return false;
+    if (mine) { m = __uint_as_float(q.x); ll[tid] = __uint_as_float(q.y); }
+    const float wm = tree_max<64>(m);
+    if (lane == 0) g_L.red[wave] = wm;
+    if (gmine) g_L.red[32 + tid] = sigmoid16(lo_h(gatew));
+  }
+  lds_barrier();
+  fstamp<ST>(li, FS_MERGE, 1, tid == 0);
+  {
+    const float Mx = tree_max<64>(g_L.red[lane & 15]);
+    if (tid < nt) fl[tid] = exp_c(m - Mx);
+  }
+  // the partial sums: item i = tid + 1024 j is chunk i % 8 of tile i / 8; all requests of an attempt first, then the looks
+  {
+    const int items = 8 * nt;
+    uint4 v[8];
+    unsigned have = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) if (tid + DEC_THREADS * j >= items) have |= 1u << j;
+    if (!flow_poll(true, [&]() {
+          const unsigned missing = ~have;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int i = tid + DEC_THREADS * j;
+            if (missing & (1u << j)) v[j] = ldw4(rpo, ((slot0 + (i >> 3)) * 128 + c0 + (i & 7)) * 4);
+          }
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if ((missing & (1u << j)) && v[j].z == tcore32 && v[j].w == tcore32) {
+              have |= 1u << j;
+              park[tid + DEC_THREADS * j] = make_uint2(v[j].x, v[j].y);
+            }
+          return (have & 0xffu) == 0xffu;
+        }, uni(P.bar) + 32, 26u)) return false;              // (its barrier also hands the scales and the parked sums on)
+  }
+  fstamp<ST>(li, FS_MERGE, 2, tid == 0);
+  const int nb = (nt + 63) / 64;                               // at most 16
+  float* const blk = g_L.part;                                 // [block][8 chunks][2], then [block] sums at 256
+  if (tid < 8 * nb) {
+    const int b = tid >> 3, c = tid & 7;
+    const int t1 = min(64 * b + 64, nt);
+    float B0 = 0.0f, B1 = 0.0f;
+    for (int t = 64 * b; t < t1; ++t) {
+      const uint2 pv = park[t * 8 + c];
+      const float f = fl[t];
+      B0 = fmaf(__uint_as_float(pv.x), f, B0); B1 = fmaf(__uint_as_float(pv.y), f, B1);
+    }
+    blk[2 * tid] = B0; blk[2 * tid + 1] = B1;
+  } else if (wave == 2 && lane < nb) {
+    const int t1 = min(64 * lane + 64, nt);
+    float Lb = 0.0f;
+    for (int t = 64 * lane; t < t1; ++t) Lb = fmaf(ll[t], fl[t], Lb);
+    blk[256 + lane] = Lb;
+  }
+  lds_barrier();
+  fstamp<ST>(li, FS_MERGE, 3, tid == 0);
+  if (wave == PUB_WAVE && lane < 8) {
+    float O0 = blk[2 * lane], O1 = blk[2 * lane + 1], Ls = blk[256];
+    for (int b = 1; b < nb; ++b) { O0 = O0 + blk[2 * (8 * b + lane)]; O1 = O1 + blk[2 * (8 * b + lane) + 1]; Ls = Ls + blk[256 + b]; }
+    const uint32_t r0 = tagged(f16r(f16r(O0 / Ls) * g_L.red[32 + 2 * lane]), tmerge);
+    const uint32_t r1 = tagged(f16r(f16r(O1 / Ls) * g_L.red[32 + 2 * lane + 1]), tmerge);
+    stw2(co_rsrc(uni(F.tycore)), h * 256 + 2 * (c0 + lane), r0, r1);
+  }
+  fstamp<ST>(li, FS_MERGE, 4, tid == PUB_WAVE * 64);
+  (void)Y;
+  return true;
+}
+
 // ---- K = 4096 projection (GDN out_proj with gated rmsnorm prologue / attention merge + o_proj) ---------
 template <bool ST>
 SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t base, const GdnHist& gh) {
@@ -1042,7 +1151,9 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
   wload_row<2>(wr.w[0], wr.sb[0], uni(Y.out_w), uni(Y.out_sb), (size_t)(valid ? gw : 0), valid, lane);
   const uint32_t tin = flow_tag(base, li, FS_IN), tcore = flow_tag(base, li, FS_CORE), tmerge = flow_tag(base, li, FS_MERGE);
   const uint32_t tcore32 = flow_tag32(base, li, FS_CORE);
-  if (!lin && wg >= G - FLOW_MERGE_WGS) {
+  if (!lin && sdpa_wide_merge(nt)) {
+    if (!flow_merge_wide<ST>(F, Y, li, nt, base)) return false;
+  } else if (!lin && wg >= G - FLOW_MERGE_WGS) {
     // Merge the attention tiles in order with the global max: the last 32 workgroups take half a head each (they own
     // no tile units, so their waves have no stores of their own to wait for and poll from the start of the
     // stage).  Wave 0 is the merging wave: a lane owns one 16-byte chunk (2 dims) of its 128 dims.
