@@ -123,6 +123,8 @@ struct sl_engine {
   bool gate8 = false;              // router / shared gate are 8-bit rows (all layers alike)
   hipStream_t stream = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  hipStream_t side = nullptr;      // hybrid MoE: the shared expert's kernels run here, beside routing and the routed experts
+  hipEvent_t side_fork = nullptr, side_join = nullptr;
   std::vector<void*> allocs;
   std::vector<LayerDev> layers;
   DevQ4 embed, lm_head;
@@ -310,6 +312,18 @@ void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   const int router_blocks = (E + 1 + 15) / 16;
   hipLaunchKernelGGL(k_final_rows, dim3(M), dim3(64), 0, e->stream, ha);     // residual + norm once per row
   a.xn_in = ha.xn_out;
+  // The shared expert needs nothing of the routing: its three kernels go to a second stream and run beside the router,
+  // the routing and the grouping (a small GEMM, a kernel of one wave per row and one of a single workgroup, which
+  // leave the device nearly idle for 40 us per layer) and the routed experts; the combine waits for both.
+  hipStream_t shs = e->side ? e->side : e->stream;
+  if (e->side) {
+    (void)hipEventRecord(e->side_fork, e->stream);
+    (void)hipStreamWaitEvent(e->side, e->side_fork, 0);
+  }
+  launch_qmm4_mfma(QmmArgs{e->xn, H, L.sh_gate.w, L.sh_gate.sb, M, SL_MOE_I, H, e->hy_sg, SL_MOE_I, L.sh_up.w, L.sh_up.sb, e->hy_su}, shs);
+  hipLaunchKernelGGL(k_swiglu_rows, dim3((M * SL_MOE_I + 255) / 256), dim3(256), 0, shs, e->hy_sg, e->hy_su, e->sh_act, M * SL_MOE_I);
+  launch_qmm4_mfma(QmmArgs{e->sh_act, SL_MOE_I, L.sh_down.w, L.sh_down.sb, M, H, SL_MOE_I, e->hy_sy, H}, shs);
+  if (e->side) (void)hipEventRecord(e->side_join, e->side);
   if (L.router_pad)      // fp16 gates: router and shared-gate logits of all rows as one small GEMM on the matrix cores
     hipLaunchKernelGGL(k_router_mfma, dim3((ROUTER_PAD_ROWS / 32 + 3) / 4, (M + 31) / 32), dim3(256), 0, e->stream,
                        RouterMmArgs{ha.xn_out, L.router_pad, M, ROUTER_PAD_ROWS, e->rlogits, e->sgate});
@@ -322,10 +336,7 @@ void launch_moe_hybrid(sl_engine* e, LayerDev& L, int M, const HiddenArgs& ha) {
   hipLaunchKernelGGL(k_qmm4_mfma_grouped<true>, dim3(SL_MOE_I / 128, E), dim3(256), 0, e->stream, g);
   QmmGroupArgs d{e->act, SL_MOE_I, 1, L.sw_down.w, L.sw_down.sb, nullptr, nullptr, H, SL_MOE_I, e->hy_lists, e->hy_counts, e->hy_counts + SL_MAX_EXPERTS, e->hy_d, H};
   hipLaunchKernelGGL(k_qmm4_mfma_grouped<false>, dim3(H / 128, E), dim3(256), 0, e->stream, d);
-  // shared expert
-  launch_qmm4_mfma(QmmArgs{e->xn, H, L.sh_gate.w, L.sh_gate.sb, M, SL_MOE_I, H, e->hy_sg, SL_MOE_I, L.sh_up.w, L.sh_up.sb, e->hy_su}, e->stream);
-  hipLaunchKernelGGL(k_swiglu_rows, dim3((M * SL_MOE_I + 255) / 256), dim3(256), 0, e->stream, e->hy_sg, e->hy_su, e->sh_act, M * SL_MOE_I);
-  launch_qmm4_mfma(QmmArgs{e->sh_act, SL_MOE_I, L.sh_down.w, L.sh_down.sb, M, H, SL_MOE_I, e->hy_sy, H}, e->stream);
+  if (e->side) (void)hipStreamWaitEvent(e->stream, e->side_join, 0);
   hipLaunchKernelGGL(k_moe_combine_rows, dim3(H / 256, M), dim3(256), 0, e->stream, e->hy_d, L.route_scores, e->sgate, e->hy_sy, e->moe_out);
 }
 constexpr int HIDDEN_TILE_MAX_ROWS = 4;  // up to here the in-projection's waves do residual + norm of a row each
@@ -1113,6 +1124,9 @@ void sl_destroy(sl_engine* e) {
   for (void* p : e->allocs) (void)hipFree(p);
   if (e->pinned) (void)hipHostFree(e->pinned);
   for (hipEvent_t ev : e->head_ev) (void)hipEventDestroy(ev);
+  if (e->side_fork) (void)hipEventDestroy(e->side_fork);
+  if (e->side_join) (void)hipEventDestroy(e->side_join);
+  if (e->side) { (void)hipStreamSynchronize(e->side); (void)hipStreamDestroy(e->side); }
   if (e->ev0) (void)hipEventDestroy(e->ev0);
   if (e->ev1) (void)hipEventDestroy(e->ev1);
   if (e->stream) (void)hipStreamDestroy(e->stream);
@@ -1140,6 +1154,11 @@ int sl_set_hybrid(sl_engine* e, int enable) {
       SL_TRY(e, hipFuncSetAttribute((const void*)k_gdn_chunk_scan, hipFuncAttributeMaxDynamicSharedMemorySize, GC_SCAN_LDS));
     }
     SL_TRY(e, hipStreamSynchronize(e->stream));
+  }
+  if (enable && !e->side) {
+    SL_TRY(e, hipStreamCreateWithFlags(&e->side, hipStreamNonBlocking));
+    SL_TRY(e, hipEventCreateWithFlags(&e->side_fork, hipEventDisableTiming));
+    SL_TRY(e, hipEventCreateWithFlags(&e->side_join, hipEventDisableTiming));
   }
   e->hybrid = enable != 0;
   return SL_OK;
