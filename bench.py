@@ -433,8 +433,22 @@ def main():
             dt = time.perf_counter() - t0
             assert o is not None, lane.gpu_fault
             b_tok, _ = step_bytes(cfg, S + args.chain + n_tok // 2)
-            sweep_report.append({"context": S, "ms_per_token": dt * 1e3 / n_tok, "tok_s": n_tok / dt, "bytes_per_token": b_tok,
-                                 "frac_of_peak": b_tok / (dt / n_tok) / 1e9 / HBM_PEAK_GBS})
+            entry = {"context": S, "ms_per_token": dt * 1e3 / n_tok, "tok_s": n_tok / dt, "bytes_per_token": b_tok,
+                     "frac_of_peak": b_tok / (dt / n_tok) / 1e9 / HBM_PEAK_GBS}
+            if args.stage_timeline:
+                # where an attention layer's time goes at this context: one more chain on the stamping variant of the kernel
+                from qwisp_amd import stage_timeline
+                lib.get().dll.sl_debug_stage_clock(lane.h, 1, None, 0)
+                o = lane.chained_step_argmax(t, args.chain)
+                o = lane.chained_step_argmax(int(o[-1]), args.chain)
+                assert o is not None, lane.gpu_fault
+                att = stage_timeline.collect(lane).summary().get("attention_layer")
+                lib.get().dll.sl_debug_stage_clock(lane.h, 0, None, 0)
+                if att:
+                    entry["attention_layer_us"] = {"layer": att["us"], "mixer": att["mixer_us"], "moe_block": att["moe_block_us"],
+                                                   "in-proj": att["in-proj"]["total_us"], "tile units": att["core"]["total_us"],
+                                                   "merge + out-proj": att["out-proj"]["total_us"]}
+            sweep_report.append(entry)
             lane.close()
 
     blocks_report = None

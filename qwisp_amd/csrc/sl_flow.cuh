@@ -736,6 +736,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
       if (pend_slot >= 0 && wave < 8 && lane == 0) stw4(co_rsrc(uni(F.tml)), pend_slot * 4, __float_as_uint(pend_m), __float_as_uint(pend_l), tcore, tcore);
       pend_slot = -1;
       lds_barrier();
+      if (ub == wg && r == 0) fstamp<ST>(li, FS_CORE, 2, tid == 0);     // first unit: queries prepared, key tile parked
       {
         // scores: wave (chain ch of 32 dims, four of the eight heads), lane j is key j: a key's 32 dims are read once
         // for four heads; the queries come as LDS broadcasts (one 16-byte read per four multiply-adds)
@@ -781,6 +782,7 @@ SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t
     }
     if (pend_slot >= 0 && wave < 8 && lane == 0) stw4(co_rsrc(uni(F.tml)), pend_slot * 4, __float_as_uint(pend_m), __float_as_uint(pend_l), tcore, tcore);
     pend_slot = -1;
+    if (ub == wg) fstamp<ST>(li, FS_CORE, 3, tid == 0);                 // first round: scores and softmax weights of its units done
     // pass 2, values: the weighted value sums of the same units, in the same order
     for (int r = 0; r < nr; ++r) {
       const int u = ub + r * GU;
@@ -1051,26 +1053,42 @@ SL_DEV bool flow_merge_wide(const FlowP& F, const LayerP& Y, int li, int nt, uin
   uint2* const park = reinterpret_cast<uint2*>(dyn + 12288);             // [tile][8 chunks] {o0, o1}
   static_assert(12288 + WIDE_MERGE_MAX_TILES * 8 * 8 <= DEC_DYN_LDS && WIDE_MERGE_MAX_TILES <= DEC_THREADS, "parked sums fit; a thread per tile");
   lds_barrier();                                                         // the tile units are through with the dynamic LDS
-  // every tile's {max, sum} (thread t: tile t) and, on lanes 0..15 of wave 0, the slice's output gate
+  // One round trip for everything: every tile's {max, sum} (thread t: tile t), the slice's output gate (lanes 0..15 of
+  // wave 0) and the partial sums -- item i = tid + 1024 j is chunk i % 8 of tile i / 8.  All requests of an attempt
+  // first, then the looks at them; what has arrived is parked and not asked for again.
   float m = NEG;
-  uint32_t gatew = 0;
   {
     const bool mine = tid < nt, gmine = tid < 16;
     bool mdone = !mine, gdone = !gmine;
-    uint4 q = make_uint4(0u, 0u, 0u, 0u);
-    if (!flow_poll(wave * 64 < nt, [&]() {
+    const int items = 8 * nt;
+    uint4 v[8];
+    unsigned have = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) if (tid + DEC_THREADS * j >= items) have |= 1u << j;
+    if (!flow_poll(true, [&]() {
           const bool want_m = !mdone, want_g = !gdone;
+          const unsigned missing = ~have;
+          uint4 q = make_uint4(0u, 0u, 0u, 0u);
           uint32_t g = 0;
           if (want_m) q = ldw4(rml, (slot0 + tid) * 4);
           if (want_g) g = ldw1(rp, h * 512 + 256 + 2 * c0 + tid);
-          if (want_m) mdone = q.z == tcore32 && q.w == tcore32;
-          if (want_g) { gdone = tag_ok(g, tin); gatew = g; }
-          return mdone && gdone;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int i = tid + DEC_THREADS * j;
+            if (missing & (1u << j)) v[j] = ldw4(rpo, ((slot0 + (i >> 3)) * 128 + c0 + (i & 7)) * 4);
+          }
+          if (want_m && q.z == tcore32 && q.w == tcore32) { mdone = true; m = __uint_as_float(q.x); ll[tid] = __uint_as_float(q.y); }
+          if (want_g && tag_ok(g, tin)) { gdone = true; g_L.red[32 + tid] = sigmoid16(lo_h(g)); }
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if ((missing & (1u << j)) && v[j].z == tcore32 && v[j].w == tcore32) {
+              have |= 1u << j;
+              park[tid + DEC_THREADS * j] = make_uint2(v[j].x, v[j].y);
+            }
+          return mdone && gdone && (have & 0xffu) == 0xffu;
         }, uni(P.bar) + 32, 25u)) return false;
-    if (mine) { m = __uint_as_float(q.x); ll[tid] = __uint_as_float(q.y); }
     const float wm = tree_max<64>(m);
     if (lane == 0) g_L.red[wave] = wm;
-    if (gmine) g_L.red[32 + tid] = sigmoid16(lo_h(gatew));
   }
   lds_barrier();
   fstamp<ST>(li, FS_MERGE, 1, tid == 0);
@@ -1078,46 +1096,39 @@ SL_DEV bool flow_merge_wide(const FlowP& F, const LayerP& Y, int li, int nt, uin
     const float Mx = tree_max<64>(g_L.red[lane & 15]);
     if (tid < nt) fl[tid] = exp_c(m - Mx);
   }
-  // the partial sums: item i = tid + 1024 j is chunk i % 8 of tile i / 8; all requests of an attempt first, then the looks
-  {
-    const int items = 8 * nt;
-    uint4 v[8];
-    unsigned have = 0;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) if (tid + DEC_THREADS * j >= items) have |= 1u << j;
-    if (!flow_poll(true, [&]() {
-          const unsigned missing = ~have;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const int i = tid + DEC_THREADS * j;
-            if (missing & (1u << j)) v[j] = ldw4(rpo, ((slot0 + (i >> 3)) * 128 + c0 + (i & 7)) * 4);
-          }
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            if ((missing & (1u << j)) && v[j].z == tcore32 && v[j].w == tcore32) {
-              have |= 1u << j;
-              park[tid + DEC_THREADS * j] = make_uint2(v[j].x, v[j].y);
-            }
-          return (have & 0xffu) == 0xffu;
-        }, uni(P.bar) + 32, 26u)) return false;              // (its barrier also hands the scales and the parked sums on)
-  }
+  lds_barrier();
   fstamp<ST>(li, FS_MERGE, 2, tid == 0);
   const int nb = (nt + 63) / 64;                               // at most 16
   float* const blk = g_L.part;                                 // [block][8 chunks][2], then [block] sums at 256
+  // (sixteen LDS reads at a time ahead of their multiply-adds: read one by one, every step of a chain would wait for
+  // its read)
   if (tid < 8 * nb) {
     const int b = tid >> 3, c = tid & 7;
     const int t1 = min(64 * b + 64, nt);
     float B0 = 0.0f, B1 = 0.0f;
-    for (int t = 64 * b; t < t1; ++t) {
-      const uint2 pv = park[t * 8 + c];
-      const float f = fl[t];
-      B0 = fmaf(__uint_as_float(pv.x), f, B0); B1 = fmaf(__uint_as_float(pv.y), f, B1);
+    for (int t0 = 64 * b; t0 < t1; t0 += 16) {
+      uint2 pv[16];
+      float f[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { const int t = min(t0 + i, t1 - 1); pv[i] = park[t * 8 + c]; f[i] = fl[t]; }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const bool in = t0 + i < t1;
+        const float n0 = fmaf(__uint_as_float(pv[i].x), f[i], B0), n1 = fmaf(__uint_as_float(pv[i].y), f[i], B1);
+        B0 = in ? n0 : B0; B1 = in ? n1 : B1;
+      }
     }
     blk[2 * tid] = B0; blk[2 * tid + 1] = B1;
   } else if (wave == 2 && lane < nb) {
     const int t1 = min(64 * lane + 64, nt);
     float Lb = 0.0f;
-    for (int t = 64 * lane; t < t1; ++t) Lb = fmaf(ll[t], fl[t], Lb);
+    for (int t0 = 64 * lane; t0 < t1; t0 += 16) {
+      float l[16], f[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { const int t = min(t0 + i, t1 - 1); l[i] = ll[t]; f[i] = fl[t]; }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { const float n = fmaf(l[i], f[i], Lb); Lb = (t0 + i < t1) ? n : Lb; }
+    }
     blk[256 + lane] = Lb;
   }
   lds_barrier();
