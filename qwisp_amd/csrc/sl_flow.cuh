@@ -1092,42 +1092,57 @@ SL_DEV bool flow_merge_wide(const FlowP& F, const LayerP& Y, int li, int nt, uin
   }
   lds_barrier();
   fstamp<ST>(li, FS_MERGE, 1, tid == 0);
+  // (tiles up to the next multiple of 16 count as tiles of scale 0 and sums 0, so the chains below walk whole batches
+  // without a test per tile: a multiply-add of zeros leaves a sum as it is)
+  const int nt16 = (nt + 15) & ~15;
   {
     const float Mx = tree_max<64>(g_L.red[lane & 15]);
     if (tid < nt) fl[tid] = exp_c(m - Mx);
+    else if (tid < nt16) { fl[tid] = 0.0f; ll[tid] = 0.0f; }
+    for (int i = 8 * nt + tid; i < 8 * nt16; i += DEC_THREADS) park[i] = make_uint2(0u, 0u);
   }
   lds_barrier();
   fstamp<ST>(li, FS_MERGE, 2, tid == 0);
   const int nb = (nt + 63) / 64;                               // at most 16
   float* const blk = g_L.part;                                 // [block][8 chunks][2], then [block] sums at 256
-  // (sixteen LDS reads at a time ahead of their multiply-adds: read one by one, every step of a chain would wait for
-  // its read)
-  if (tid < 8 * nb) {
-    const int b = tid >> 3, c = tid & 7;
-    const int t1 = min(64 * b + 64, nt);
-    float B0 = 0.0f, B1 = 0.0f;
+  // One lane per (block, one of the 16 dims): a single wave issues an instruction every eight clocks or so, so what a
+  // chain costs is its instruction count -- sixteen tiles per batch, their values and scales read with constant
+  // offsets ahead of the sixteen multiply-adds.
+  if (tid < 16 * nb) {
+    const int b = tid >> 4, c2 = tid & 15;
+    const int t1 = min(64 * b + 64, nt16);
+    const float* const parkf = reinterpret_cast<const float*>(park);
+    float B = 0.0f;
     for (int t0 = 64 * b; t0 < t1; t0 += 16) {
-      uint2 pv[16];
-      float f[16];
+      const float* const pp = parkf + t0 * 16 + c2;
+      const float4* const fp = reinterpret_cast<const float4*>(fl + t0);
+      float pv[16];
+      float4 f4[4];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) { const int t = min(t0 + i, t1 - 1); pv[i] = park[t * 8 + c]; f[i] = fl[t]; }
+      for (int i = 0; i < 16; ++i) pv[i] = pp[16 * i];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const bool in = t0 + i < t1;
-        const float n0 = fmaf(__uint_as_float(pv[i].x), f[i], B0), n1 = fmaf(__uint_as_float(pv[i].y), f[i], B1);
-        B0 = in ? n0 : B0; B1 = in ? n1 : B1;
+      for (int j = 0; j < 4; ++j) f4[j] = fp[j];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        B = fmaf(pv[4 * j], f4[j].x, B); B = fmaf(pv[4 * j + 1], f4[j].y, B);
+        B = fmaf(pv[4 * j + 2], f4[j].z, B); B = fmaf(pv[4 * j + 3], f4[j].w, B);
       }
     }
-    blk[2 * tid] = B0; blk[2 * tid + 1] = B1;
-  } else if (wave == 2 && lane < nb) {
-    const int t1 = min(64 * lane + 64, nt);
+    blk[tid] = B;
+  } else if (wave == 4 && lane < nb) {
+    const int t1 = min(64 * lane + 64, nt16);
     float Lb = 0.0f;
     for (int t0 = 64 * lane; t0 < t1; t0 += 16) {
-      float l[16], f[16];
+      const float4* const lp = reinterpret_cast<const float4*>(ll + t0);
+      const float4* const fp = reinterpret_cast<const float4*>(fl + t0);
+      float4 l4[4], f4[4];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) { const int t = min(t0 + i, t1 - 1); l[i] = ll[t]; f[i] = fl[t]; }
+      for (int j = 0; j < 4; ++j) { l4[j] = lp[j]; f4[j] = fp[j]; }
 #pragma unroll
-      for (int i = 0; i < 16; ++i) { const float n = fmaf(l[i], f[i], Lb); Lb = (t0 + i < t1) ? n : Lb; }
+      for (int j = 0; j < 4; ++j) {
+        Lb = fmaf(l4[j].x, f4[j].x, Lb); Lb = fmaf(l4[j].y, f4[j].y, Lb);
+        Lb = fmaf(l4[j].z, f4[j].z, Lb); Lb = fmaf(l4[j].w, f4[j].w, Lb);
+      }
     }
     blk[256 + lane] = Lb;
   }
