@@ -248,7 +248,9 @@ int sl_attn_layer_rows(sl_engine* e, int layer, const uint16_t* x_f16, int m, ui
  * `count` fp16 elements of an internal scratch buffer left by the last launch sequence.
  * which: 0 projection rows (stride 12352), 1 GDN core output / gated attention output (stride 4096),
  * 2 rotated queries, 3 mixer output, 4 post-normed rows, 5 routed activations, 6 shared activations,
- * 7 router logits (stride 256), 8 MoE output. */
+ * 7 router logits (stride 256), 8 MoE output.  After a block entry point that ran as a single launch (one
+ * row) only 3, 7 and 8 exist (one row each, taken from the launch's exchange buffers); the others answer
+ * SL_ERR_UNSUPPORTED. */
 int sl_debug_scratch(sl_engine* e, int which, uint16_t* out_f16, size_t count);
 
 /* Greedy loop standing in for Tell.runSpecLoop without drafts (TellRuntime.swift:716-802):
