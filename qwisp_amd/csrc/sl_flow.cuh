@@ -1721,6 +1721,19 @@ SL_DEV uint32_t route_key(uint32_t hbits, int e) {
   u = (u & 0x8000u) ? (~u & 0xffffu) : (u | 0x8000u);
   return (u << 8) | (uint32_t)(255 - e);
 }
+// Rounds [r0, r1) of the top-8 selection on one wave: k holds the lane's keys not yet chosen, in falling order.
+SL_DEV void route_rounds(uint32_t (&k)[4], int r0, int r1, int E, int lane) {
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    if (r < r0 || r >= r1) continue;                      // (uniform)
+    // (the wave-wide maximum stays in vector registers: a value read out to a scalar register takes tens of clocks
+    // to become usable, eight times in a row)
+    const uint32_t M = wave_max_u32(k[0]);
+    const bool won = k[0] == M;
+    k[0] = won ? k[1] : k[0]; k[1] = won ? k[2] : k[1]; k[2] = won ? k[3] : k[2]; k[3] = won ? 0u : k[3];
+    if (lane == 0) g_L.inds[r] = min(255 - (int)(M & 255u), E - 1);
+  }
+}
 template <bool ST>
 SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   FLOW_IDS;
@@ -1729,6 +1742,11 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
   Lds& L = g_L;
   const float NEG = -__int_as_float(0x7f800000);
   float* ex = L.part + 256;                             // [256] exp(logit - max)
+  // A workgroup's routed gate/up rows belong to one of the eight chosen experts (slot = workgroup / 32): wave 0 runs the
+  // max-and-remove rounds only up to that slot, the workgroup meets and requests its rows, and wave 0 finds the
+  // remaining indices (needed from the next stage on) while the rows are on their way.
+  const int myslot = (wg >> 5) & 7;
+  uint32_t rk[4] = {0u, 0u, 0u, 0u};
   // Waves 0 and 1 each poll all the logits (four per lane, 1 KB) and go straight on: wave 0 picks the 8 largest keys
   // in order (max, remove, repeat), wave 1 forms the softmax sums.  The workgroup meets once, when the indices are
   // known (a hop of the logits through LDS and a barrier ahead of the routing measured 0.1 % slower).
@@ -1756,15 +1774,8 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
       // is the wave-wide maximum of the lanes' first keys and a shift of the winner's list
       auto order = [](uint32_t& a, uint32_t& b) { const uint32_t hi = max(a, b), lo = min(a, b); a = hi; b = lo; };
       order(k[0], k[1]); order(k[2], k[3]); order(k[0], k[2]); order(k[1], k[3]); order(k[1], k[2]);
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        // (the wave-wide maximum stays in vector registers: a value read out to a scalar register takes tens of clocks
-        // to become usable, eight times in a row)
-        const uint32_t M = wave_max_u32(k[0]);
-        const bool won = k[0] == M;
-        k[0] = won ? k[1] : k[0]; k[1] = won ? k[2] : k[1]; k[2] = won ? k[3] : k[2]; k[3] = won ? 0u : k[3];
-        if (lane == 0) L.inds[r] = min(255 - (int)(M & 255u), E - 1);
-      }
+      rk[0] = k[0]; rk[1] = k[1]; rk[2] = k[2]; rk[3] = k[3];
+      route_rounds(rk, 0, myslot + 1, E, lane);
     } else {
       float v[4], x4[4];
 #pragma unroll
@@ -1792,6 +1803,7 @@ SL_DEV bool flow_moe_b(const FlowP& F, const LayerP& Y, int li, uint32_t base) {
     wload_row<1>(wr.w[0], wr.sb[0], uni(Y.swg_w), uni(Y.swg_sb), row, true, lane);
     wload_row<1>(wr.w[1], wr.sb[1], uni(Y.swu_w), uni(Y.swu_sb), row, true, lane);
   }
+  if (wave == 0) route_rounds(rk, myslot + 1, 8, uni(P.E), lane);
   if (active) {
     const F2 gu = dot_1x2(wr);
     fstamp<ST>(li, FS_B, 3, tid == 0);
