@@ -597,7 +597,7 @@ void flow_advance_base(sl_engine* e, int steps) {
   e->flow_base += (uint32_t)steps * (uint32_t)(e->n_layers + 1) * 8u;
 }
 // One block of one layer (mode 0: the mixer, 1: the MoE block) on the row in e->xn, in a single launch of the step
-// kernel's stages; the result is left in the exchange buffer `tagged_out` with the tags of (layer, stage).
+// kernel's stages; the result is left in the stage's exchange buffer (tmix / tmoe: halves with the tags of this launch).
 bool block_flow_ready(const sl_engine* e, int m) { return m == 1 && e->dec_grid > 0 && e->use_persistent && e->flow_params; }
 void launch_block_flow(sl_engine* e, int layer, int mode) {
   e->last_block_flow = true;
@@ -952,8 +952,8 @@ bool lanes_batchable(sl_engine** lanes, int b) {
 // Into how many groups a batch of lanes is dealt (lane i to group i % groups) that are stepped side by side
 // (sl_lane_step_argmax); a group's first lane lends scratch rows and stream.  Two groups from 32 lanes on, so that a group
 // keeps the 16 rows that the matrix-core kernels of hybrid mode want.  (Measured at 32 lanes of 1K-16K tokens: one group
-// 9.83 ms per step of exact rows and 8.0 ms hybrid, two groups 9.14 and 7.9, four groups of 8 rows 14.9: the device
-// then spends its time on 2000 launches.)
+// 9.83 ms per step of exact rows and 8.0 ms hybrid, two groups 9.1 and 7.8, four groups of 8 rows 14.9: kernels of
+// 8 rows are too small to share the device, and there are 2000 of them.)
 constexpr int LANE_GROUPS_MAX = 2, LANE_GROUP_ROWS = 16;
 int lane_groups(sl_engine** lanes, int b) {
   if (b < 2 * LANE_GROUP_ROWS) return 1;
@@ -1010,8 +1010,8 @@ int sl_lane_step_argmax(sl_engine** lanes, int b, const int32_t* tokens, int32_t
     if (tokens[i] < 0 || tokens[i] >= d->vocab) return SL_ERR_ARG;
     if (lanes[i]->has_attn && lanes[i]->pos + 1 > lanes[i]->max_seq) return SL_ERR_ARG;
   }
-  // Two groups of lanes, each on the scratch rows and the stream of its first lane, queued layer by layer in turn:
-  // the two launch sequences run side by side on the device, so the short kernels of one group (norms, routing,
+  // Two groups of lanes, each on the scratch rows and the stream of its first lane: the two launch sequences run
+  // side by side on the device, so the short kernels of one group (norms, routing,
   // gates: a third of a step's launches, a few microseconds each and bound by nothing but their start and end) and the
   // ends of its large ones are covered by the other group's kernels.  The dense weights are streamed once per group
   // instead of once per step (5 % of a 32-lane step's bytes); what a lane computes does not change.
