@@ -1037,7 +1037,7 @@ SL_DEV void store_hist(const LayerP& Y, int li, const GdnHist& gh) {
 // merge on few workgroups is how fast those can pull the published chunks (16 MB per layer at 32K tokens through 32
 // compute units); spread over the whole grid every thread fetches at most eight chunks, all in one round trip, parks
 // them in LDS, and the sums are formed from LDS.  The order is the canonical one: per block of 64 tiles a chain from
-// zero in tile order (one lane per (block, chunk); the tiles' sums likewise, one lane per block), the blocks' chains
+// zero in tile order (one lane per (block, dim); the tiles' sums likewise, one lane per block), the blocks' chains
 // added in block order.
 template <bool ST>
 SL_DEV bool flow_merge_wide(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t base) {
