@@ -14,7 +14,8 @@ sample of the same workload).  After the timed decode region the same engine als
 paths on the same weights and reports them as extra objects of the line: `lane_batch` (32 sequences at mixed contexts of 1K-16K tokens
 stepped together), `verify` (4-row verify steps) and `prefill` (a 2048-token prompt in chunks of 1024
 rows, exact rows and hybrid on the matrix cores), `context_sweep` (decode after prompts of 4096, 8192 and 32768
-tokens), `blocks` (the single blocks of the reference's configurations 0-2) and `stage_timeline`;
+tokens, with the stage times of an attention layer at each context), `blocks` (the single blocks of the reference's
+configurations 0-2, one launch each) and `stage_timeline`;
 `--lanes 0 --verify-rows 0 --prefill-chunk 0 --context-sweep= --blocks 0 --stage-timeline 0` skips them.
 `--microbench 1` prints the machine-limit micro-benchmarks instead (dependent exchanges between workgroups, the
 4-bit GEMV streaming rate, matrix-instruction issue), the figures the design notes price the step against.
