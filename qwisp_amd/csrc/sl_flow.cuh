@@ -604,11 +604,12 @@ SL_DEV bool flow_gdn(const FlowP& F, const LayerP& Y, int li, uint32_t base, Gdn
 #define SL_MERGE_WGS 32
 #endif
 constexpr int FLOW_MERGE_WGS = SL_MERGE_WGS;     // workgroups that merge the attention tiles: two or four per query head
-// Contexts of 33 to 1024 key tiles (2K to 64K tokens): every workgroup takes tile units, and afterwards every workgroup
-// merges a sixteenth of a query head (flow_merge_wide).  Below, the tile units are split over the query heads and the
-// merging workgroups poll everything in one round trip; above, the parked partial sums no longer fit the LDS.
+// Contexts of 13 to 1024 key tiles (from 800 tokens to 64K): every workgroup merges a sixteenth of a query head after
+// the tile units (flow_merge_wide), and beyond 32 tiles every workgroup takes tile units as well.  Up to 12 tiles the 32
+// merging workgroups get everything in one round trip, from workgroups of their own XCD (0.2 % faster there than the
+// wide merge); above 1024 tiles the parked partial sums no longer fit the LDS.
 constexpr int WIDE_MERGE_MAX_TILES = 1024;
-SL_DEV bool sdpa_wide_merge(int nt) { return nt > 32 && nt <= WIDE_MERGE_MAX_TILES; }
+SL_DEV bool sdpa_wide_merge(int nt) { return nt > 12 && nt <= WIDE_MERGE_MAX_TILES; }
 template <bool ST>
 SL_DEV bool flow_sdpa(const FlowP& F, const LayerP& Y, int li, int pos, uint32_t base) {
   FLOW_IDS;
@@ -1185,11 +1186,9 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
     // stage).  Wave 0 is the merging wave: a lane owns one 16-byte chunk (2 dims) of its 128 dims.
     // First round trip: {max, sum} of the first 64 tiles (lane i fetches tile i), the partials of the first MB tiles
     // and the output gate (it sits in the q projection of this step) are polled together, each piece until it has
-    // arrived; at contexts of up to MB tiles that is everything the merge needs.  Beyond that a round trip per MB
-    // tiles would dominate (two to three us each, whatever its size), so the other waves fetch: waves 2..15 poll
-    // blocks of 64 tiles, two blocks ahead, and park their values in LDS, wave 0 adds a block up from LDS while the
-    // next ones are on their way, and wave 1 carries the chain of the tiles' sums.  The accumulation always runs in
-    // tile order.
+    // arrived; at contexts of up to MB tiles that is everything the merge needs.  (From there to 1024 tiles every
+    // workgroup merges a slice, flow_merge_wide; beyond, the waves of these workgroups share the blocks of 64 tiles,
+    // below.)  The accumulation always runs in tile order.
     constexpr int MPH = FLOW_MERGE_WGS / SL_ATT_HEADS, LPW = 128 / MPH;      // workgroups per head, chunks (lanes) per workgroup
     // Workgroup n runs on XCD n % 8, and at short contexts the tile units of heads 2x, 2x+1 run on XCD x (flow_sdpa4:
     // workgroup % 8 = kv head * 4 + head pair): the workgroups that merge those two heads are taken from the same XCD,
@@ -1300,132 +1299,8 @@ SL_DEV bool flow_out(const FlowP& F, const LayerP& Y, int li, int nt, uint32_t b
       }
     }
     const int nb = (nt + 63) / 64;                          // blocks of 64 tiles: a chain each, the chains added in block order
-    if (nt > MB && nb <= 2) {                               // uniform for the grid
-      // Blocks of 64 tiles in a pipeline: waves 2..15 poll the partial sums of block b (five tiles each) and park
-      // them in LDS, while wave 0 adds up block b-1 from the other parking buffer in tile order and wave 1 carries
-      // the chain of the tiles' sums (the merge is one dependent chain per lane: a wave that also fetches and sums
-      // the weights issues three times the instructions per tile).  One barrier per block; both groups of waves run
-      // nbp + 1 of them, nbp = the block count rounded up to even (a block beyond the context is empty).
-      uint2* const park0 = reinterpret_cast<uint2*>(g_vt);                       // [64 tiles][64 lanes] {o0, o1}
-      uint2* const park1 = reinterpret_cast<uint2*>(g_vt + SDPA_TILE * 256);     // the softmax weights' space (merging workgroups own no units)
-      
-      // (the polling waves start at once, while wave 0 is still waiting for the maxima and the first tiles above; tile
-      // units this workgroup may have had ended with a barrier, so the parking space is free)
-      if (wave == 0) {                                      // for wave 1: the maximum, the sum so far, block 0's {max, sum} words
-        if (lane == 0) { g_L.red[0] = Mx; g_L.red[1] = Ls; }
-        *reinterpret_cast<uint2*>(&g_L.part[2 * lane]) = make_uint2(m0.x, m0.y);
-      }
-      const int nbp = 2;
-      if (wave >= 2) {
-        // A wave's five tiles of a block are requested two blocks ahead (a round trip to memory takes about two blocks'
-        // additions), so a block costs a round trip only when its tiles have not been published yet.  Two register
-        // sets take turns: a set is parked and at once requested again for the block after the next.  Every request
-        // is unconditional (tile and block indices clamped into the context), so the wait for one set leaves the
-        // other set's loads in flight.
-        uint4 qa[5], qb[5];
-        auto request = [&](uint4 (&dst)[5], int blk) {
-#pragma unroll
-          for (int j = 0; j < 5; ++j) {
-            const int t = min(64 * min(blk, nb - 1) + min(5 * (wave - 2) + j, 63), nt - 1);
-            dst[j] = ldw4(rpo, ((slot0 + t) * 128 + chunk) * 4);
-          }
-        };
-        auto wanted = [&](int blk, int j) {
-          const int i = 5 * (wave - 2) + j, t = 64 * blk + i;
-          return i < 64 && t >= MB && t < nt && act;
-        };
-        auto poll_block = [&](uint4 (&cur)[5], int blk) {
-          uint2* const park = (blk & 1) ? park1 : park0;
-          unsigned spins = 0;
-          for (;;) {
-            bool ok = true;
-#pragma unroll
-            for (int j = 0; j < 5; ++j) ok = ok && (!wanted(blk, j) || (cur[j].z == tcore32 && cur[j].w == tcore32));
-            if (__all(ok ? 1 : 0)) break;
-            if (++spins > uni(F.spin_limit)) { fail = 19; break; }
-            SL_FRESH_LOOK();
-            request(cur, blk);
-          }
-#pragma unroll
-          for (int j = 0; j < 5; ++j) if (wanted(blk, j)) park[(5 * (wave - 2) + j) * 64 + lane] = make_uint2(cur[j].x, cur[j].y);
-          request(cur, blk + 2);
-        };
-        request(qa, 0);
-        request(qb, 1);
-        for (int b = 0; b < nbp; b += 2) {
-          poll_block(qa, b);
-          lds_barrier();
-          poll_block(qb, b + 1);
-          lds_barrier();
-        }
-        lds_barrier();
-      } else {
-        // waves 0, 1; lane i: {max, sum} of tile i of the block (tags verified above); the words of the next block are
-        // requested before this one is added up
-        uint4 ma = m0, mb = m0;
-        auto add_block = [&](const uint4& cur, uint4& nxt, int blk) {
-          const int t0 = 64 * blk;
-          const uint2* const park = (blk & 1) ? park1 : park0;
-          nxt = ldw4(rml, (slot0 + min(t0 + 64 + lane, nt - 1)) * 4);
-          float fl = 0.0f, pl = 0.0f;                     // lane i: scale and sum of tile t0+i
-          if (t0 + lane < nt) { fl = exp_c(__uint_as_float(cur.x) - Mx); pl = __uint_as_float(cur.y); }
-          const int lo = t0 == 0 ? MB : 0, hi = min(64, nt - t0);
-          float S0 = 0.0f, S1 = 0.0f, SL = 0.0f;
-          if (blk == 1 && blk < nb) { S0 = O0; S1 = O1; SL = Ls; O0 = 0.0f; O1 = 0.0f; Ls = 0.0f; }
-          if (wave == 0 && !fail) {
-            // sixteen LDS reads and sixteen lane reads at a time, used in tile order (one wave issues an instruction
-            // every eight clocks or so and waits tens of clocks for a batch of either kind: few, large batches)
-            int u0 = lo;
-            for (; u0 + 16 <= hi; u0 += 16) {
-              uint2 v[16];
-              float f[16];
-#pragma unroll
-              for (int i = 0; i < 16; ++i) v[i] = park[(u0 + i) * 64 + lane];
-              lanes8(fl, u0, reinterpret_cast<float(&)[8]>(f[0]));
-              lanes8(fl, u0 + 8, reinterpret_cast<float(&)[8]>(f[8]));
-#pragma unroll
-              for (int i = 0; i < 16; ++i) { O0 = fmaf(__uint_as_float(v[i].x), f[i], O0); O1 = fmaf(__uint_as_float(v[i].y), f[i], O1); }
-            }
-            for (; u0 < hi; u0 += 8) {
-              uint2 v[8];
-              float f[8];
-#pragma unroll
-              for (int i = 0; i < 8; ++i) v[i] = park[min(u0 + i, 63) * 64 + lane];
-              lanes8(fl, u0, f);
-#pragma unroll
-              for (int i = 0; i < 8; ++i) {
-                if (u0 + i < hi) { O0 = fmaf(__uint_as_float(v[i].x), f[i], O0); O1 = fmaf(__uint_as_float(v[i].y), f[i], O1); }
-              }
-            }
-          } else if (wave == 1) {
-            for (int u0 = lo; u0 < hi; u0 += 8) {
-              float f[8], l[8];
-              lanes8(fl, u0, f);
-              lanes8(pl, u0, l);
-#pragma unroll
-              for (int i = 0; i < 8; ++i) if (u0 + i < hi) Ls = fmaf(l[i], f[i], Ls);
-            }
-          }
-          if (blk == 1 && blk < nb) { O0 = S0 + O0; O1 = S1 + O1; Ls = SL + Ls; }
-        };
-        lds_barrier();                                    // block 0 is parked; wave 0 has left the maximum and its sum so far
-        if (wave == 1) {
-          Mx = g_L.red[0]; Ls = g_L.red[1];
-          const uint2 w = *reinterpret_cast<const uint2*>(&g_L.part[2 * lane]);
-          ma.x = w.x; ma.y = w.y;
-        }
-        for (int b = 0; b < nbp; b += 2) {
-          add_block(ma, mb, b);
-          lds_barrier();
-          add_block(mb, ma, b + 1);
-          lds_barrier();
-        }
-        if (wave == 1 && lane == 0) g_L.red[2] = Ls;
-      }
-      lds_barrier();
-      if (wave == 0) Ls = g_L.red[2];
-    } else if (nt > MB) {
-      // More than 128 tiles: the blocks' chains run side by side.  Wave 2 + w takes blocks w, w + 14, ...: it polls
+    if (nt > MB) {
+      // (More than 1024 tiles -- up to there every workgroup merges, flow_merge_wide.)  The blocks' chains run side by side.  Wave 2 + w takes blocks w, w + 14, ...: it polls
       // sixteen tiles at a time (one 16-byte chunk per lane and tile; the tile index sits in the load's scalar offset,
       // so sixteen requests in flight cost no address registers) -- from the start of the stage, while the maxima are
       // still on their way -- and, once wave 0 has left the global maximum, adds them up in tile order (block 0 goes

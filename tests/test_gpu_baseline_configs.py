@@ -128,7 +128,9 @@ def test_gdn_layer_1024_sequential_steps(env):
 
 
 # ---- configuration 2: attention over 8K and 32K tokens of pre-filled keys and values --------------------------
-@pytest.mark.parametrize("S", [8192, 32768])
+# (66000 tokens, beyond the benchmark's contexts: more than 1024 key tiles, where the single-launch path merges the
+# tiles on 32 workgroups again instead of on all of them)
+@pytest.mark.parametrize("S", [8192, 32768, 66000])
 def test_attention_layer_decode_long_arena(env, S):
     cfg = ModelConfig(n_layers=1, n_experts=8, vocab=0, layer_types=("attn",))
     dev, host = device_and_host_model(cfg)
